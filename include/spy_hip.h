@@ -1,0 +1,134 @@
+/*
+ * spy_hip.h -- C ABI of the MI355X (gfx950) backend for Spy's LLaMA-2 token loop.
+ *
+ * This is the drop-in boundary.  Spy has no C ABI of its own: its backends are C++ classes
+ * derived from spy::Backend (backend/interface/include/backend/backend.h:31-95) whose
+ * submit(OperatorNode*, callback) dispatches on OperatorType to one OperatorImpl<Op>::execute
+ * per operator (backend/host/include/operator_impl.h:17-89, backend/host/backend/cpu_backend.cpp:71-94).
+ * Each spy_hip_op_* entry point below replaces one of those execute() bodies and takes the same
+ * operands: the operator's input/output `Tensor`s (orchestration/include/number/tensor.h:209-222)
+ * flattened to POD, and the operator's Param struct flattened to scalars.
+ *
+ * Conventions
+ *   - every function returns 0 on success, a positive hipError_t, or a negative SPY_HIP_E* code;
+ *     nothing throws and nothing aborts (the reference asserts/aborts instead,
+ *     backend/host/include/default_backend.h:72-78);
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); launches are
+ *     asynchronous, the caller synchronises;
+ *   - all tensor memory is device memory owned by the caller; kernels never allocate;
+ *   - shapes use Spy's order: ne[0] is the contiguous dimension, nb[] are BYTE strides and nb[0]
+ *     is the size of one block (tensor.h:50-57).
+ */
+#ifndef SPY_HIP_H
+#define SPY_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SPY_HIP_EUNSUPPORTED (-1) /* OperatorStatus::Unsupport (backend.h:22-29) */
+#define SPY_HIP_EINVAL       (-2) /* shape / argument check failed (spy_assert in the reference) */
+#define SPY_HIP_ENOSPACE     (-3) /* caller-provided scratch too small */
+
+/* NumberType ids (orchestration/include/number/number_impl/type.h:12-45) */
+enum spy_hip_type {
+    SPY_HIP_F32 = 0, SPY_HIP_F16 = 1, SPY_HIP_Q4_0 = 2, SPY_HIP_Q8_0 = 8,
+    SPY_HIP_Q4_K = 12, SPY_HIP_Q6_K = 14, SPY_HIP_I32 = 26
+};
+
+/* spy::Tensor flattened (tensor.h:23-36, 209-222) */
+typedef struct spy_hip_tensor {
+    int32_t type;
+    int32_t dim;
+    int64_t ne[4];
+    int64_t nb[4];
+    void   *data;
+} spy_hip_tensor;
+
+/* ---- runtime: replaces DefaultCPUBackend's constructor / alloc_memory / dealloc_memory
+ *      (backend/host/include/default_backend.h:121-156) and the capacity queries of
+ *      spy::Backend (backend.h:44-51) ------------------------------------------------------- */
+int spy_hip_init(int device_id);
+int spy_hip_device_info(char *name, int name_len, int *num_cu, size_t *total_mem, size_t *free_mem);
+int spy_hip_alloc(void **ptr, size_t bytes);
+int spy_hip_free(void *ptr);
+int spy_hip_upload(void *dst_dev, const void *src_host, size_t bytes, void *stream);
+int spy_hip_download(void *dst_host, const void *src_dev, size_t bytes, void *stream);
+int spy_hip_fill_u8(void *dst_dev, int value, size_t bytes, void *stream);   /* fill kernel, graph-safe */
+int spy_hip_sync(void *stream);                      /* NULL: whole device */
+int spy_hip_stream_create(void **stream);
+int spy_hip_stream_destroy(void *stream);
+int spy_hip_event_create(void **event);
+int spy_hip_event_record(void *event, void *stream);
+int spy_hip_event_elapsed_ms(void *start, void *stop, float *ms);   /* synchronises on `stop` */
+int spy_hip_event_destroy(void *event);
+const char *spy_hip_error_string(int code);
+
+/* ---- operators: one per OperatorImpl<Op>::execute of the host backend ---------------------- */
+
+/* MatMul -- OperatorMatMulImpl::execute (backend/host/operator/mat.cpp:71-146).
+ * dst[i01,i11,i2,i3] = dot(w[:,i01,i2,i3], x[:,i11,i2,i3]).  Type routing as
+ * target_buffer_type (mat.cpp:32-42): (Q4_0|Q8_0, F32) quantizes x to Q8_0, (F16, F32) rounds x
+ * to fp16; additionally (Q4_K|Q6_K, F32) -> Q8_0 activations, which the reference lacks.
+ * `scratch` holds the converted activations (the reference allocates it in get_control_header,
+ * mat.cpp:61-68); query its size with spy_hip_op_matmul_scratch_size. */
+size_t spy_hip_op_matmul_scratch_size(const spy_hip_tensor *w, const spy_hip_tensor *x);
+int spy_hip_op_matmul(void *stream, const spy_hip_tensor *w, const spy_hip_tensor *x, const spy_hip_tensor *dst,
+                      void *scratch, size_t scratch_bytes);
+/* NormRMS -- OperatorNormRMSImpl::execute (non-linear.cpp:194-223); eps = NormRMSParam::eps */
+int spy_hip_op_norm_rms(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *dst, float eps);
+/* Add/Sub/Mul/Div -- binary_execution<Op> (basic.cpp:15-50); op: 0 add, 1 sub, 2 mul, 3 div */
+int spy_hip_op_binary(void *stream, int op, const spy_hip_tensor *a, const spy_hip_tensor *b, const spy_hip_tensor *dst);
+/* Silu -- OperatorSiluImpl::execute (non-linear.cpp:57-77) */
+int spy_hip_op_silu(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *dst);
+/* Softmax -- OperatorSoftmaxImpl::execute (non-linear.cpp:86-185); mask may be NULL;
+ * scale = SoftmaxParam::scale */
+int spy_hip_op_softmax(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *mask, const spy_hip_tensor *dst, float scale);
+/* Rope -- OperatorRopeImpl::execute (non-linear.cpp:270-371); fields of RopeParam
+ * (orchestration/include/operator/non-linear.h:191-207).  Supported: mode None/Norm (-1/0) with
+ * extend_factor == 0 and xpos_base == 0 (the LLaMA defaults); anything else -> EUNSUPPORTED. */
+typedef struct spy_hip_rope_param {
+    int32_t mode, num_past, num_dim, num_context, num_origin_context;
+    float   freq_base, freq_scale, extend_factor, attention_factor, beta_fast, beta_slow, xpos_base;
+    int32_t xpos_down;
+} spy_hip_rope_param;
+int spy_hip_op_rope(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *pos, const spy_hip_tensor *dst, const spy_hip_rope_param *p);
+/* Dup / Copy -- dup_execute (view.cpp:83-195): F32->F32, F32->F16, F16->F32 through strides */
+int spy_hip_op_dup(void *stream, const spy_hip_tensor *src, const spy_hip_tensor *dst);
+/* Contiguous -- OperatorContiguousImpl::execute (view.cpp:285-321) */
+int spy_hip_op_contiguous(void *stream, const spy_hip_tensor *src, const spy_hip_tensor *dst);
+/* GetRow -- OperatorGetRowImpl::execute (view.cpp:33-81): F32 or Q8_0 table -> F32 rows.
+ * Row ids outside the table leave the output row untouched and raise the device-side error flag
+ * returned by spy_hip_take_error (the reference asserts, view.cpp:61). */
+int spy_hip_op_get_row(void *stream, const spy_hip_tensor *table, const spy_hip_tensor *ids, const spy_hip_tensor *dst);
+int spy_hip_take_error(int *flag);   /* reads and clears the device error flag (synchronises) */
+/* Greedy sampling -- SamplerImpl<Greedy>::sample (model/include/llm/sampler/greedy.h:20-25):
+ * index of the FIRST maximum of n logits, written to *out_index (device int32) */
+int spy_hip_argmax(void *stream, const float *logits, int64_t n, int32_t *out_index);
+
+/* ---- kernel families used by the operators above and by the fused token loop --------------- */
+
+/* Quantizator<FP32,Q8_0>::transform (backend/host/include/simd/vec_convert.h:178-261):
+ * nrow rows of K floats (row stride x_stride BYTES) -> nrow rows of K/32 native Q8_0 blocks */
+int spy_hip_quantize_q8_0(void *stream, const float *x, int64_t x_stride, void *y, int64_t nrow, int64_t K);
+/* Quantizator<FP32,FP16>::transform (vec_convert.h:39-65) */
+int spy_hip_quantize_f16(void *stream, const float *x, int64_t x_stride, void *y, int64_t nrow, int64_t K);
+/* Dot<W,Q8_0>::exec over every weight row (vec_dot.h:42-115): dst[t*dst_stride + m] =
+ * dot(w row m, xq row t) (+ residual[t*dst_stride + m] when residual != NULL).
+ * w: M rows of K elements in native block layout, contiguous; xq: T rows of K/32 native Q8_0
+ * blocks, contiguous; strides in ELEMENTS. */
+int spy_hip_gemv_q8_0act(void *stream, int wtype, const void *w, const void *xq, float *dst, const float *residual,
+                         int64_t M, int64_t K, int64_t T, int64_t dst_stride);
+/* the int32 dot of every 32-element block (Q4_0, Q8_0, Q4_K sub-blocks) or 16-element
+ * sub-block (Q6_K) of every weight row with activation row 0: out[m*nsub + b], written by the
+ * GEMV kernels themselves (same code path, dump switch on).  `out` must hold M*nsub + M int32:
+ * the last M slots receive the float results and are scratch. */
+int spy_hip_block_dots(void *stream, int wtype, const void *w, const void *xq, int32_t *out, int64_t M, int64_t K);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,457 @@
+// One entry point per operator of Spy's host backend (backend/host/operator/*.cpp in the Spy
+// tree), taking the operator's tensors with their byte strides.  These are the general,
+// stride-honouring forms that a per-operator submit() uses; the fused token loop has its own
+// specialised kernels.
+#include "common.cuh"
+
+#include <math.h>
+
+int *spy_hip_err_flag_ptr();
+
+struct tdesc {              // a tensor as the kernels see it
+    uint8_t *p;
+    int64_t ne[4], nb[4];
+};
+static tdesc mk(const spy_hip_tensor *t) {
+    tdesc d;
+    d.p = (uint8_t *)t->data;
+    for (int i = 0; i < 4; i++) { d.ne[i] = t->ne[i]; d.nb[i] = t->nb[i]; }
+    return d;
+}
+static __device__ __forceinline__ uint8_t *at(const tdesc &t, int64_t i0, int64_t i1, int64_t i2, int64_t i3) {
+    return t.p + i0 * t.nb[0] + i1 * t.nb[1] + i2 * t.nb[2] + i3 * t.nb[3];
+}
+static bool same_ne(const spy_hip_tensor *a, const spy_hip_tensor *b) {
+    for (int i = 0; i < 4; i++) if (a->ne[i] != b->ne[i]) return false;
+    return true;
+}
+static bool same_shape(const spy_hip_tensor *a, const spy_hip_tensor *b) {      // Shape::operator== (tensor.h:106-109)
+    if (a->type != b->type || a->dim != b->dim) return false;
+    for (int i = 0; i < 4; i++) if (a->ne[i] != b->ne[i] || a->nb[i] != b->nb[i]) return false;
+    return true;
+}
+static unsigned grid_for(int64_t n, int per) { return (unsigned)((n + per - 1) / per); }
+#define CHECK_GRID(n, per) SPY_CHECK_ARG((n) > 0 && ((n) + (per) - 1) / (per) < (1ll << 31))
+
+// ---------------------------------------------------------------------------------------------
+// NormRMS (non-linear.cpp:194-223): y = x * (1 / sqrt(sum(x^2)/n + eps)); one workgroup per row.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void norm_rms_kernel(tdesc x, tdesc y, float eps) {
+    __shared__ float s_part[4];
+    const int64_t r = blockIdx.x;
+    const int64_t ne0 = y.ne[0], ne1 = y.ne[1], ne2 = y.ne[2];
+    const int64_t i3 = r / (ne1 * ne2), i2 = r % (ne1 * ne2) / ne1, i1 = r % ne1;
+    const float *s = (const float *)at(x, 0, i1, i2, i3);
+    float *d = (float *)at(y, 0, i1, i2, i3);
+    float acc = 0.0f;
+    for (int64_t i = threadIdx.x; i < ne0; i += 256) { const float v = s[i]; acc = fmaf(v, v, acc); }
+    acc = wave_sum(acc);
+    if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = acc;
+    __syncthreads();
+    const float sum = (s_part[0] + s_part[1]) + (s_part[2] + s_part[3]);
+    const float mean = sum / (float)ne0;
+    const float scale = 1.0f / sqrtf(mean + eps);
+    for (int64_t i = threadIdx.x; i < ne0; i += 256) d[i] = s[i] * scale;
+}
+
+extern "C" int spy_hip_op_norm_rms(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *dst, float eps) {
+    SPY_CHECK_ARG(x && dst && x->data && dst->data);
+    if (x->type != SPY_HIP_F32 || dst->type != SPY_HIP_F32) return SPY_HIP_EUNSUPPORTED;   // spy_assert (non-linear.cpp:199-200)
+    SPY_CHECK_ARG(same_ne(x, dst) && x->nb[0] == 4 && dst->nb[0] == 4);
+    const int64_t nrow = spy_t_nrow(dst);
+    CHECK_GRID(nrow, 1);
+    norm_rms_kernel<<<dim3((unsigned)nrow), dim3(256), 0, (hipStream_t)stream>>>(mk(x), mk(dst), eps);
+    return SPY_LAUNCH_RC();
+}
+
+// ---------------------------------------------------------------------------------------------
+// Add / Sub / Mul / Div (basic.cpp:15-50): dst = a (op) b, b broadcast over rows by i % ne1x and
+// repeated along dim 0 when ne00 is a multiple of ne10.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void binary_kernel(int op, tdesc a, tdesc b, tdesc d, int64_t total) {
+    const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (g >= total) return;
+    const int64_t i0 = g % a.ne[0], r = g / a.ne[0];
+    const int64_t i1 = r % a.ne[1], i2 = r / a.ne[1] % a.ne[2], i3 = r / (a.ne[1] * a.ne[2]);
+    const float va = *(const float *)at(a, i0, i1, i2, i3);
+    const float vb = *(const float *)at(b, i0 % b.ne[0], i1 % b.ne[1], i2 % b.ne[2], i3 % b.ne[3]);
+    float v;
+    switch (op) {
+    case 0: v = va + vb; break;
+    case 1: v = va - vb; break;
+    case 2: v = va * vb; break;
+    default: v = va / vb; break;
+    }
+    *(float *)at(d, i0, i1, i2, i3) = v;
+}
+
+extern "C" int spy_hip_op_binary(void *stream, int op, const spy_hip_tensor *a, const spy_hip_tensor *b, const spy_hip_tensor *dst) {
+    SPY_CHECK_ARG(a && b && dst && a->data && b->data && dst->data && op >= 0 && op <= 3);
+    if (a->type != SPY_HIP_F32 || b->type != SPY_HIP_F32 || dst->type != SPY_HIP_F32) return SPY_HIP_EUNSUPPORTED;
+    SPY_CHECK_ARG(same_ne(a, dst));
+    for (int i = 0; i < 4; i++) SPY_CHECK_ARG(b->ne[i] > 0 && a->ne[i] % b->ne[i] == 0);   // Shape::can_repeat (tensor.h:186-190)
+    const int64_t total = spy_t_nelem(a);
+    CHECK_GRID(total, 256);
+    binary_kernel<<<dim3(grid_for(total, 256)), dim3(256), 0, (hipStream_t)stream>>>(op, mk(a), mk(b), mk(dst), total);
+    return SPY_LAUNCH_RC();
+}
+
+// ---------------------------------------------------------------------------------------------
+// Silu (non-linear.cpp:11-14,57-77): the reference looks silu up in a table indexed by fp16(x),
+// whose entries are v / (1 + expf(-v)) evaluated in fp32 on v = float(fp16(x)).
+// ---------------------------------------------------------------------------------------------
+static __device__ __forceinline__ float silu_ref(float x) {
+    const float v = h2f(f2h(x));
+    return v / (1.0f + expf(-v));
+}
+
+__global__ __launch_bounds__(256) void silu_kernel(tdesc x, tdesc d, int64_t total) {
+    const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (g >= total) return;
+    const int64_t i0 = g % x.ne[0], r = g / x.ne[0];
+    const int64_t i1 = r % x.ne[1], i2 = r / x.ne[1] % x.ne[2], i3 = r / (x.ne[1] * x.ne[2]);
+    *(float *)at(d, i0, i1, i2, i3) = silu_ref(*(const float *)at(x, i0, i1, i2, i3));
+}
+
+extern "C" int spy_hip_op_silu(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *dst) {
+    SPY_CHECK_ARG(x && dst && x->data && dst->data);
+    if (x->type != SPY_HIP_F32 || dst->type != SPY_HIP_F32) return SPY_HIP_EUNSUPPORTED;
+    SPY_CHECK_ARG(same_ne(x, dst));
+    const int64_t total = spy_t_nelem(x);
+    CHECK_GRID(total, 256);
+    silu_kernel<<<dim3(grid_for(total, 256)), dim3(256), 0, (hipStream_t)stream>>>(mk(x), mk(dst), total);
+    return SPY_LAUNCH_RC();
+}
+
+// ---------------------------------------------------------------------------------------------
+// Softmax (non-linear.cpp:86-180): t = (s + mask) * scale; m = max t; e = mask == -inf ? 0 :
+// expf(float(fp16(t - m))); p = e * (1 / sum e).  One workgroup per row; dst doubles as the
+// row scratch exactly as in the reference.
+// ---------------------------------------------------------------------------------------------
+static __device__ __forceinline__ float block_reduce_256(float v, bool is_max, float *s_part) {
+    v = is_max ? wave_max(v) : wave_sum(v);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return is_max ? fmaxf(fmaxf(s_part[0], s_part[1]), fmaxf(s_part[2], s_part[3])) : (s_part[0] + s_part[1]) + (s_part[2] + s_part[3]);
+}
+
+__global__ __launch_bounds__(256) void softmax_kernel(tdesc x, tdesc mask, bool has_mask, tdesc y, float scale) {
+    __shared__ float s_part[4];
+    const int64_t r = blockIdx.x;
+    const int64_t ne0 = y.ne[0], ne1 = y.ne[1], ne2 = y.ne[2];
+    const int64_t i3 = r / (ne1 * ne2), i2 = r % (ne1 * ne2) / ne1, i1 = r % ne1;
+    const float *s = (const float *)at(x, 0, i1, i2, i3);
+    const float *mk_ = has_mask ? (const float *)at(mask, 0, i1, 0, 0) : nullptr;
+    float *d = (float *)at(y, 0, i1, i2, i3);
+    float mx = -INFINITY;
+    for (int64_t i = threadIdx.x; i < ne0; i += 256) {
+        const float t = has_mask ? (s[i] + mk_[i]) * scale : s[i] * scale;
+        d[i] = t;
+        mx = fmaxf(mx, t);
+    }
+    mx = block_reduce_256(mx, true, s_part);
+    float sum = 0.0f;
+    for (int64_t i = threadIdx.x; i < ne0; i += 256) {
+        float e;
+        if (has_mask && mk_[i] == -INFINITY) e = 0.0f;
+        else e = expf(h2f(f2h(d[i] - mx)));
+        d[i] = e;
+        sum += e;
+    }
+    sum = block_reduce_256(sum, false, s_part);
+    const float inv = 1.0f / sum;
+    for (int64_t i = threadIdx.x; i < ne0; i += 256) d[i] *= inv;
+}
+
+extern "C" int spy_hip_op_softmax(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *mask, const spy_hip_tensor *dst, float scale) {
+    SPY_CHECK_ARG(x && dst && x->data && dst->data);
+    if (x->type != SPY_HIP_F32 || dst->type != SPY_HIP_F32) return SPY_HIP_EUNSUPPORTED;
+    SPY_CHECK_ARG(same_ne(x, dst) && x->nb[0] == 4 && dst->nb[0] == 4);
+    tdesc m = mk(x);
+    if (mask) {
+        // the mask is typed INT32 by the graph (inout.cpp:43-47) but read as float (non-linear.cpp:147)
+        SPY_CHECK_ARG(mask->data && mask->nb[0] == 4 && mask->ne[0] >= dst->ne[0] && mask->ne[1] >= dst->ne[1]);
+        m = mk(mask);
+    }
+    const int64_t nrow = spy_t_nrow(dst);
+    CHECK_GRID(nrow, 1);
+    softmax_kernel<<<dim3((unsigned)nrow), dim3(256), 0, (hipStream_t)stream>>>(mk(x), m, mask != nullptr, mk(dst), scale);
+    return SPY_LAUNCH_RC();
+}
+
+// ---------------------------------------------------------------------------------------------
+// Rope (non-linear.cpp:270-371), default branch: pair k of token i2 is rotated by
+// theta_k = pos[i2] * theta_scale^k where the power is built by k successive fp32
+// multiplications (:304-309); cos/sin of theta*freq_scale, times attention_factor.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(64) void rope_kernel(tdesc x, const int32_t *pos, int64_t pos_stride, tdesc y, float theta_scale,
+                                                  float freq_scale, float mscale) {
+    const int64_t i1 = blockIdx.x, i2 = blockIdx.y, i3 = blockIdx.z;
+    const float p = (float)*(const int32_t *)((const uint8_t *)pos + i2 * pos_stride);
+    const int64_t npair = y.ne[0] / 2;
+    for (int64_t k = threadIdx.x; k < npair; k += 64) {
+        float theta = p;
+        for (int64_t j = 0; j < k; j++) theta *= theta_scale;
+        const float ang = freq_scale * theta;
+        const float c = cosf(ang) * mscale, s = sinf(ang) * mscale;
+        const float *sp = (const float *)at(x, 2 * k, i1, i2, i3);
+        float *dp = (float *)at(y, 2 * k, i1, i2, i3);
+        const float x0 = sp[0], x1 = sp[1];
+        dp[0] = x0 * c - x1 * s;
+        dp[1] = x0 * s + x1 * c;
+    }
+}
+
+extern "C" int spy_hip_op_rope(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *pos, const spy_hip_tensor *dst, const spy_hip_rope_param *p) {
+    SPY_CHECK_ARG(x && pos && dst && p && x->data && pos->data && dst->data);
+    if (x->type != SPY_HIP_F32 || dst->type != SPY_HIP_F32 || pos->type != SPY_HIP_I32) return SPY_HIP_EUNSUPPORTED;
+    if (p->mode != 0 && p->mode != -1) return SPY_HIP_EUNSUPPORTED;          // GLM / Neox (Neox aborts in the reference too)
+    if (p->extend_factor != 0.0f || p->xpos_base != 0.0f) return SPY_HIP_EUNSUPPORTED;
+    SPY_CHECK_ARG(same_ne(x, dst) && x->nb[0] == 4 && dst->nb[0] == 4 && dst->ne[0] % 2 == 0 && p->num_dim > 0);
+    SPY_CHECK_ARG(pos->ne[0] >= dst->ne[2] && dst->ne[1] < 65536 && dst->ne[2] < (1ll << 31) && dst->ne[3] < 65536);
+    SPY_CHECK_ARG(dst->ne[1] > 0 && dst->ne[2] > 0 && dst->ne[3] > 0);
+    const float theta_scale = powf(p->freq_base, -2.0f / (float)p->num_dim);   // host libm, as the reference (:282)
+    // CUDA-style grids cap y/z at 65535: put the token index on x when it is the large one
+    const dim3 grid((unsigned)dst->ne[1], (unsigned)dst->ne[2], (unsigned)dst->ne[3]);
+    SPY_CHECK_ARG(dst->ne[2] < 65536);
+    rope_kernel<<<grid, dim3(64), 0, (hipStream_t)stream>>>(mk(x), (const int32_t *)pos->data, pos->nb[0], mk(dst), theta_scale,
+                                                           p->freq_scale, p->attention_factor);
+    return SPY_LAUNCH_RC();
+}
+
+// ---------------------------------------------------------------------------------------------
+// Dup / Copy (view.cpp:83-195).  mode 0: same shape, element (i0..i3) -> element (i0..i3);
+// mode 1: contiguous src -> contiguous dst of another shape = flat copy; mode 2: strided src,
+// flat source counter unravelled in the destination's dimensions (:164-171).
+// conv: 0 raw 4-byte copy, 1 f32 -> f16, 2 f16 -> f32, 3 raw 2-byte copy.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void dup_kernel(tdesc s, tdesc d, int mode, int conv, int64_t total) {
+    const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (g >= total) return;
+    const int64_t i00 = g % s.ne[0], r = g / s.ne[0];
+    const int64_t i01 = r % s.ne[1], i02 = r / s.ne[1] % s.ne[2], i03 = r / (s.ne[1] * s.ne[2]);
+    const uint8_t *sp = at(s, i00, i01, i02, i03);
+    uint8_t *dp;
+    if (mode == 0) dp = at(d, i00, i01, i02, i03);
+    else if (mode == 1) dp = d.p + g * d.nb[0];
+    else {
+        const int64_t i0 = g % d.ne[0], i1 = g / d.ne[0] % d.ne[1];
+        const int64_t i2 = g % (d.ne[2] * d.ne[1] * d.ne[0]) / (d.ne[1] * d.ne[0]), i3 = g / (d.ne[2] * d.ne[1] * d.ne[0]);
+        dp = at(d, i0, i1, i2, i3);
+    }
+    switch (conv) {
+    case 0: *(uint32_t *)dp = *(const uint32_t *)sp; break;
+    case 1: *(uint16_t *)dp = f2h(*(const float *)sp); break;
+    case 2: *(float *)dp = h2f(*(const uint16_t *)sp); break;
+    default: *(uint16_t *)dp = *(const uint16_t *)sp; break;
+    }
+}
+
+static int conv_code(int ts, int td) {
+    if (ts == td && (ts == SPY_HIP_F32 || ts == SPY_HIP_I32)) return 0;
+    if (ts == SPY_HIP_F32 && td == SPY_HIP_F16) return 1;
+    if (ts == SPY_HIP_F16 && td == SPY_HIP_F32) return 2;
+    if (ts == SPY_HIP_F16 && td == SPY_HIP_F16) return 3;
+    return -1;
+}
+
+extern "C" int spy_hip_op_dup(void *stream, const spy_hip_tensor *src, const spy_hip_tensor *dst) {
+    SPY_CHECK_ARG(src && dst && src->data && dst->data);
+    const int conv = conv_code(src->type, dst->type);
+    if (conv < 0) return SPY_HIP_EUNSUPPORTED;
+    SPY_CHECK_ARG(spy_t_nelem(src) == spy_t_nelem(dst));                     // operator/view.h Copy::propagate
+    int mode;
+    if (spy_t_contiguous(src)) {
+        if (same_shape(src, dst)) mode = 0;                                  // row-by-row memcpy (view.cpp:106-109)
+        else if (spy_t_contiguous(dst)) mode = 1;                            // rows appended to a contiguous destination (:132-159)
+        else return SPY_HIP_EUNSUPPORTED;                                    // spy_assert(false) (:160-162)
+    } else {
+        if (conv == 2 || conv == 3) return SPY_HIP_EUNSUPPORTED;             // only F32 sources (:173-188)
+        mode = 2;
+    }
+    const int64_t total = spy_t_nelem(src);
+    CHECK_GRID(total, 256);
+    dup_kernel<<<dim3(grid_for(total, 256)), dim3(256), 0, (hipStream_t)stream>>>(mk(src), mk(dst), mode, conv, total);
+    return SPY_LAUNCH_RC();
+}
+
+// Contiguous (view.cpp:285-321): dst (contiguous, src's dims) [i0..i3] = src[i0..i3]
+__global__ __launch_bounds__(256) void contiguous_kernel(tdesc s, float *d, int64_t total) {
+    const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (g >= total) return;
+    const int64_t i0 = g % s.ne[0], r = g / s.ne[0];
+    const int64_t i1 = r % s.ne[1], i2 = r / s.ne[1] % s.ne[2], i3 = r / (s.ne[1] * s.ne[2]);
+    d[g] = *(const float *)at(s, i0, i1, i2, i3);
+}
+
+extern "C" int spy_hip_op_contiguous(void *stream, const spy_hip_tensor *src, const spy_hip_tensor *dst) {
+    SPY_CHECK_ARG(src && dst && src->data && dst->data);
+    if (src->type != SPY_HIP_F32 || dst->type != SPY_HIP_F32) return SPY_HIP_EUNSUPPORTED;
+    SPY_CHECK_ARG(same_ne(src, dst) && spy_t_contiguous(dst));
+    const int64_t total = spy_t_nelem(src);
+    CHECK_GRID(total, 256);
+    contiguous_kernel<<<dim3(grid_for(total, 256)), dim3(256), 0, (hipStream_t)stream>>>(mk(src), (float *)dst->data, total);
+    return SPY_LAUNCH_RC();
+}
+
+// ---------------------------------------------------------------------------------------------
+// GetRow (view.cpp:33-81): one workgroup per requested row; F32 copy or Q8_0 -> F32
+// (q * fp16 scale, vec_convert.h:436-442).
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void get_row_kernel(tdesc table, bool q8, const int32_t *ids, int64_t ne10, int64_t ne11,
+                                                      float *dst, int64_t dst_row_elems, int64_t nrow_table, int *err) {
+    const int64_t r = blockIdx.x;
+    const int64_t i12 = r / (ne10 * ne11), i11 = r % (ne10 * ne11) / ne10;
+    const int64_t row = ids[r];
+    if (row < 0 || row >= nrow_table) { if (threadIdx.x == 0 && err) atomicExch(err, 1); return; }
+    const uint8_t *sp = table.p + row * table.nb[1] + i11 * table.nb[2] + i12 * table.nb[3];
+    float *dp = dst + r * dst_row_elems;
+    const int64_t ne00 = table.ne[0];
+    if (!q8) { for (int64_t i = threadIdx.x; i < ne00; i += 256) dp[i] = ((const float *)sp)[i]; }
+    else {
+        for (int64_t i = threadIdx.x; i < ne00; i += 256) {
+            const blk_q8_0 *b = (const blk_q8_0 *)sp + (i >> 5);
+            dp[i] = (float)b->qs[i & 31] * h2f(b->d);
+        }
+    }
+}
+
+extern "C" int spy_hip_op_get_row(void *stream, const spy_hip_tensor *table, const spy_hip_tensor *ids, const spy_hip_tensor *dst) {
+    SPY_CHECK_ARG(table && ids && dst && table->data && ids->data && dst->data);
+    if (ids->type != SPY_HIP_I32 || dst->type != SPY_HIP_F32) return SPY_HIP_EUNSUPPORTED;
+    if (table->type != SPY_HIP_F32 && table->type != SPY_HIP_Q8_0) return SPY_HIP_EUNSUPPORTED;   // spy_abort (view.cpp:74-75)
+    SPY_CHECK_ARG(spy_t_contiguous(ids) && spy_t_contiguous(dst) && dst->ne[0] == table->ne[0]);
+    SPY_CHECK_ARG(table->nb[0] == spy_type_size(table->type));
+    const int64_t n = ids->ne[0] * ids->ne[1] * ids->ne[2];
+    SPY_CHECK_ARG(spy_t_nrow(dst) >= n);
+    CHECK_GRID(n, 1);
+    get_row_kernel<<<dim3((unsigned)n), dim3(256), 0, (hipStream_t)stream>>>(mk(table), table->type == SPY_HIP_Q8_0, (const int32_t *)ids->data,
+                                                                             ids->ne[0], ids->ne[1], (float *)dst->data, dst->ne[0],
+                                                                             spy_t_nrow(table), spy_hip_err_flag_ptr());
+    return SPY_LAUNCH_RC();
+}
+
+// ---------------------------------------------------------------------------------------------
+// Greedy argmax (greedy.h:20-25): std::max_element keeps the FIRST maximum.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(1024) void argmax_kernel(const float *__restrict__ x, int64_t n, int32_t *out) {
+    __shared__ float s_v[16];
+    __shared__ int s_i[16];
+    float best = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int64_t i = threadIdx.x; i < n; i += 1024) {
+        const float v = x[i];
+        if (v > best || (bi == 0x7fffffff && !(v < best))) { best = v; bi = (int)i; }   // strided scan keeps the lowest index per thread
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(best, o, SPY_WAVE);
+        const int oi = __shfl_xor(bi, o, SPY_WAVE);
+        if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
+    }
+    if ((threadIdx.x & 63) == 0) { s_v[threadIdx.x >> 6] = best; s_i[threadIdx.x >> 6] = bi; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 16; w++) if (s_v[w] > best || (s_v[w] == best && s_i[w] < bi)) { best = s_v[w]; bi = s_i[w]; }
+        *out = bi == 0x7fffffff ? 0 : bi;
+    }
+}
+
+extern "C" int spy_hip_argmax(void *stream, const float *logits, int64_t n, int32_t *out_index) {
+    SPY_CHECK_ARG(logits && out_index && n > 0 && n < (1ll << 31));
+    argmax_kernel<<<dim3(1), dim3(1024), 0, (hipStream_t)stream>>>(logits, n, out_index);
+    return SPY_LAUNCH_RC();
+}
+
+// ---------------------------------------------------------------------------------------------
+// MatMul (mat.cpp:32-146)
+// ---------------------------------------------------------------------------------------------
+// fp16 weight rows x fp16 activation rows (Dot<FP16,FP16>, vec_dot.h:117-146): one wave per
+// output element, lanes stride along the contraction.  w and dst strided, xh contiguous.
+__global__ __launch_bounds__(256) void matmul_f16_kernel(tdesc w, const uint16_t *__restrict__ xh, tdesc d, int64_t ne11, int64_t total) {
+    const int64_t o = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (o >= total) return;
+    const int lane = threadIdx.x & 63;
+    const int64_t ne00 = w.ne[0], ne01 = w.ne[1], ne02 = w.ne[2];
+    const int64_t i01 = o % ne01, i11 = o / ne01 % ne11, i02 = o / (ne01 * ne11) % ne02, i03 = o / (ne01 * ne11 * ne02);
+    const uint16_t *wr = (const uint16_t *)at(w, 0, i01, i02, i03);
+    const uint16_t *xr = xh + ((i03 * ne02 + i02) * ne11 + i11) * ne00;
+    float acc = 0.0f;
+    for (int64_t k = lane; k < ne00; k += 64) acc = fmaf(h2f(wr[k]), h2f(xr[k]), acc);
+    acc = wave_sum(acc);
+    if (lane == 0) *(float *)at(d, i01, i11, i02, i03) = acc;
+}
+
+static int mid_type(int t0, int t1) {                                        // target_buffer_type (mat.cpp:32-42) + K-quants
+    if (t0 == t1) return t0;
+    if (t0 == SPY_HIP_F16 && t1 == SPY_HIP_F32) return SPY_HIP_F16;
+    if ((t0 == SPY_HIP_Q4_0 || t0 == SPY_HIP_Q8_0 || t0 == SPY_HIP_Q4_K || t0 == SPY_HIP_Q6_K) && t1 == SPY_HIP_F32) return SPY_HIP_Q8_0;
+    return t0;
+}
+
+extern "C" size_t spy_hip_op_matmul_scratch_size(const spy_hip_tensor *w, const spy_hip_tensor *x) {
+    if (!w || !x) return 0;
+    const int tm = mid_type(w->type, x->type);
+    if (tm == x->type) return 0;
+    if (tm != SPY_HIP_Q8_0 && tm != SPY_HIP_F16) return 0;
+    if (x->ne[0] % spy_block_size(tm) != 0) return 0;
+    return (size_t)(spy_t_nrow(x) * spy_row_size(tm, x->ne[0]));
+}
+
+extern "C" int spy_hip_op_matmul(void *stream, const spy_hip_tensor *w, const spy_hip_tensor *x, const spy_hip_tensor *dst,
+                                 void *scratch, size_t scratch_bytes) {
+    SPY_CHECK_ARG(w && x && dst && w->data && x->data && dst->data);
+    const int t0 = w->type, t1 = x->type, tm = mid_type(t0, t1);
+    if (dst->type != SPY_HIP_F32) return SPY_HIP_EUNSUPPORTED;
+    const bool quant = (t0 == SPY_HIP_Q4_0 || t0 == SPY_HIP_Q8_0 || t0 == SPY_HIP_Q4_K || t0 == SPY_HIP_Q6_K) && tm == SPY_HIP_Q8_0;
+    const bool half = (t0 == SPY_HIP_F16 && tm == SPY_HIP_F16);
+    if (!quant && !half) return SPY_HIP_EUNSUPPORTED;                        // generic Dot<> aborts (vec_dot.h:29-40)
+    if (t1 != SPY_HIP_F32 && t1 != tm) return SPY_HIP_EUNSUPPORTED;
+    const int64_t ne00 = w->ne[0], ne01 = w->ne[1], ne02 = w->ne[2], ne03 = w->ne[3];
+    const int64_t ne10 = x->ne[0], ne11 = x->ne[1], ne12 = x->ne[2], ne13 = x->ne[3];
+    SPY_CHECK_ARG(ne00 == ne10 && ne02 == ne12 && ne03 == ne13);             // operator/mat.h:56-59
+    SPY_CHECK_ARG(dst->ne[0] == ne01 && dst->ne[1] == ne11 && dst->ne[2] == ne12 && dst->ne[3] == ne13 && dst->nb[0] == 4);
+    SPY_CHECK_ARG(ne00 % spy_block_size(t0) == 0 && ne00 % spy_block_size(tm) == 0);
+    hipStream_t st = (hipStream_t)stream;
+
+    // 1. activations -> mid type, contiguous [ne10, ne11, ne12, ne13] in scratch (mat.cpp:95-128)
+    const uint8_t *xm = (const uint8_t *)x->data;
+    const int64_t mid_row = spy_row_size(tm, ne10);
+    if (t1 != tm) {
+        const size_t need = (size_t)(spy_t_nrow(x) * mid_row);
+        if (!scratch || scratch_bytes < need) return SPY_HIP_ENOSPACE;
+        SPY_CHECK_ARG(x->nb[0] == 4);
+        for (int64_t i13 = 0; i13 < ne13; i13++)
+            for (int64_t i12 = 0; i12 < ne12; i12++) {
+                const float *src = (const float *)((const uint8_t *)x->data + i12 * x->nb[2] + i13 * x->nb[3]);
+                uint8_t *out = (uint8_t *)scratch + ((i13 * ne12 + i12) * ne11) * mid_row;
+                int rc = (tm == SPY_HIP_Q8_0) ? spy_hip_quantize_q8_0(stream, src, x->nb[1], out, ne11, ne10)
+                                              : spy_hip_quantize_f16(stream, src, x->nb[1], out, ne11, ne10);
+                if (rc) return rc;
+            }
+        xm = (const uint8_t *)scratch;
+    } else {
+        SPY_CHECK_ARG(spy_t_contiguous(x));
+    }
+
+    // 2. dots
+    if (quant) {
+        SPY_CHECK_ARG(w->nb[0] == spy_type_size(t0) && w->nb[1] == spy_row_size(t0, ne00));   // whole contiguous rows
+        SPY_CHECK_ARG(dst->nb[1] % 4 == 0);
+        for (int64_t i3 = 0; i3 < ne03; i3++)
+            for (int64_t i2 = 0; i2 < ne02; i2++) {
+                const uint8_t *wp = (const uint8_t *)w->data + i2 * w->nb[2] + i3 * w->nb[3];
+                const uint8_t *xp = xm + ((i3 * ne12 + i2) * ne11) * mid_row;
+                float *dp = (float *)((uint8_t *)dst->data + i2 * dst->nb[2] + i3 * dst->nb[3]);
+                int rc = spy_hip_gemv_q8_0act(stream, t0, wp, xp, dp, nullptr, ne01, ne00, ne11, dst->nb[1] / 4);
+                if (rc) return rc;
+            }
+        return 0;
+    }
+    SPY_CHECK_ARG(w->nb[0] == 2);
+    const int64_t total = ne01 * ne11 * ne02 * ne03;
+    CHECK_GRID(total, 4);
+    matmul_f16_kernel<<<dim3(grid_for(total, 4)), dim3(256), 0, st>>>(mk(w), (const uint16_t *)xm, mk(dst), ne11, total);
+    return SPY_LAUNCH_RC();
+}

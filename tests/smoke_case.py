@@ -1,0 +1,24 @@
+"""The smoke check: a small pass of the hot path on the GPU compared with the CPU oracle."""
+import ctypes as C
+
+
+def run_smoke(H, O, np):
+    H.init(0)
+    L, oracle = H.load(), O.load()
+    rng = np.random.default_rng(0)
+    M, K, T = 256, 4096, 2
+    w = O.quantize(oracle, (rng.standard_normal((M, K)) * 0.02).astype(np.float32), O.Q4_0)
+    x = rng.standard_normal((T, K)).astype(np.float32)
+    want = O.matmul(oracle, w, O.Q4_0, M, K, x, nthread=2)
+    dw, dx = H.DeviceBuffer.from_numpy(w), H.DeviceBuffer.from_numpy(x)
+    dd = H.DeviceBuffer(T * M * 4)
+    tw, tx, td = H.tensor(dw, H.Q4_0, [K, M]), H.tensor(dx, H.F32, [K, T]), H.tensor(dd, H.F32, [M, T])
+    need = L.spy_hip_op_matmul_scratch_size(C.byref(tw), C.byref(tx))
+    sc = H.DeviceBuffer(need)
+    H.check(L.spy_hip_op_matmul(None, C.byref(tw), C.byref(tx), C.byref(td), sc.ptr, need), "spy_hip_op_matmul")
+    H.sync()
+    got = dd.download(np.float32).reshape(T, M)
+    err = float(np.abs(got - want).max() / np.abs(want).max())
+    assert np.array_equal(sc.download(np.uint8), O.quantize(oracle, x, O.Q8_0)), "Q8_0 activations differ from the oracle"
+    assert err < 1e-3, err
+    print("smoke ok: Q4_0 matmul %dx%d T=%d, max relative error %.2e on %s" % (M, K, T, err, H.device_info()["name"]))

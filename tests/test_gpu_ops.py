@@ -1,0 +1,227 @@
+"""GPU parity of the per-operator entry points (spy_hip_op_*) against the CPU oracle, through the
+same strided tensor views the LLaMA graph hands to a backend."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from tests import oracle_lib as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def hip():
+    from spy_amd import _lib as H
+    H.init(0)
+    return H
+
+
+def B(t):
+    return C.byref(t)
+
+
+def test_norm_rms(hip, oracle):
+    from tests.gpu_util import dev, dev_empty, call, assert_close
+    rng = np.random.default_rng(1)
+    for T, d in [(1, 4096), (7, 4096), (2, 100)]:
+        x = (rng.standard_normal((T, d)) * 2.5).astype(np.float32)
+        want = np.zeros_like(x)
+        assert oracle.spy_o_norm_rms(B(O.tensor(x, O.F32, [d, T])), B(O.tensor(want, O.F32, [d, T])), 1e-5) == 0
+        dx, dy = dev(x), dev_empty(x.nbytes, 0xFF)
+        call(hip.load().spy_hip_op_norm_rms, None, B(hip.tensor(dx, hip.F32, [d, T])), B(hip.tensor(dy, hip.F32, [d, T])), 1e-5)
+        assert_close(dy.download(np.float32).reshape(T, d), want, "norm_rms %dx%d" % (T, d), tol=1e-5)
+
+
+def test_binary_ops_exact(hip, oracle):
+    from tests.gpu_util import dev, dev_empty, call
+    rng = np.random.default_rng(2)
+    a = rng.standard_normal((6, 4096)).astype(np.float32)
+    w = rng.standard_normal(4096).astype(np.float32)
+    b = rng.standard_normal((6, 4096)).astype(np.float32)
+    da, dw, db = dev(a), dev(w), dev(b)
+    for op in range(4):
+        for (hb, ob, ne_b) in [(dw, w, [4096]), (db, b, [4096, 6])]:
+            want = np.zeros_like(a)
+            assert oracle.spy_o_binary(op, B(O.tensor(a, O.F32, [4096, 6])), B(O.tensor(ob, O.F32, ne_b)), B(O.tensor(want, O.F32, [4096, 6]))) == 0
+            dd = dev_empty(a.nbytes, 0xFF)
+            call(hip.load().spy_hip_op_binary, None, op, B(hip.tensor(da, hip.F32, [4096, 6])), B(hip.tensor(hb, hip.F32, ne_b)),
+                 B(hip.tensor(dd, hip.F32, [4096, 6])))
+            assert np.array_equal(dd.download(np.float32).reshape(6, 4096).view(np.uint32), want.view(np.uint32))   # IEEE single ops: exact
+
+
+def test_silu_all_fp16_inputs(hip, oracle):
+    from tests.gpu_util import dev, dev_empty, call
+    bits = np.arange(0, 0x10000, dtype=np.uint16)
+    finite = (bits & 0x7C00) != 0x7C00
+    x = np.concatenate([bits[finite].view(np.float16).astype(np.float32),
+                        np.random.default_rng(3).standard_normal(4096).astype(np.float32) * 4])
+    want = np.zeros_like(x)
+    assert oracle.spy_o_silu(B(O.tensor(x, O.F32, [x.size])), B(O.tensor(want, O.F32, [x.size]))) == 0
+    dx, dy = dev(x), dev_empty(x.nbytes, 0xFF)
+    call(hip.load().spy_hip_op_silu, None, B(hip.tensor(dx, hip.F32, [x.size])), B(hip.tensor(dy, hip.F32, [x.size])))
+    got = dy.download(np.float32)
+    big = np.abs(want) > 1e-30
+    rel = np.abs(got[big] - want[big]) / np.abs(want[big])
+    print("silu: max elementwise relative error %.3e over %d fp16 inputs" % (rel.max(), big.sum()), flush=True)
+    assert rel.max() < 1e-5 and np.abs(got[~big] - want[~big]).max() < 1e-30
+
+
+def test_masked_softmax(hip, oracle):
+    from tests.gpu_util import dev, dev_empty, call, assert_close
+    rng = np.random.default_rng(4)
+    for (H_, T, n_kv, Cx, P) in [(32, 1, 300, 512, 299), (4, 5, 9, 16, 4), (2, 3, 1030, 1100, 1027)]:
+        s = (rng.standard_normal((H_, T, n_kv)) * 12).astype(np.float32)
+        mask = np.full((T, Cx), -np.inf, dtype=np.float32)
+        for i in range(T):
+            mask[i, :i + P + 1] = 0.0
+        scale = float(1.0 / np.sqrt(128.0))
+        want = np.zeros_like(s)
+        assert oracle.spy_o_softmax(B(O.tensor(s, O.F32, [n_kv, T, H_])), B(O.tensor(mask, O.I32, [Cx, T])), B(O.tensor(want, O.F32, [n_kv, T, H_])), scale) == 0
+        ds, dm, dd = dev(s), dev(mask), dev_empty(s.nbytes, 0xFF)
+        call(hip.load().spy_hip_op_softmax, None, B(hip.tensor(ds, hip.F32, [n_kv, T, H_])), B(hip.tensor(dm, hip.I32, [Cx, T])),
+             B(hip.tensor(dd, hip.F32, [n_kv, T, H_])), scale)
+        got = dd.download(np.float32).reshape(s.shape)
+        assert_close(got, want, "softmax H%d T%d n_kv%d" % (H_, T, n_kv), tol=1e-5)
+        assert np.array_equal(got == 0, want == 0)                          # masked entries exactly zero
+    # unmasked form
+    want = np.zeros_like(s)
+    assert oracle.spy_o_softmax(B(O.tensor(s, O.F32, [n_kv, T, H_])), None, B(O.tensor(want, O.F32, [n_kv, T, H_])), scale) == 0
+    call(hip.load().spy_hip_op_softmax, None, B(hip.tensor(ds, hip.F32, [n_kv, T, H_])), None, B(hip.tensor(dd, hip.F32, [n_kv, T, H_])), scale)
+    assert_close(dd.download(np.float32).reshape(s.shape), want, "softmax unmasked", tol=1e-5)
+
+
+def test_rope(hip, oracle):
+    from tests.gpu_util import dev, dev_empty, call, assert_close
+    rng = np.random.default_rng(5)
+    hd, H_, T = 128, 32, 6
+    pos = np.array([0, 1, 7, 100, 2047, 4351], dtype=np.int32)
+    x = rng.standard_normal((T, H_, hd)).astype(np.float32)
+    want = np.zeros_like(x)
+    rp = O.default_rope(hd, 4352)
+    assert oracle.spy_o_rope(B(O.tensor(x, O.F32, [hd, H_, T])), B(O.tensor(pos, O.I32, [T])), B(O.tensor(want, O.F32, [hd, H_, T])), B(rp)) == 0
+    dx, dp, dy = dev(x), dev(pos), dev_empty(x.nbytes, 0xFF)
+    hp = hip.RopeParam(0, 0, hd, 4352, 4352, 10000.0, 1.0, 0.0, 1.0, 32.0, 1.0, 0.0, 0)
+    call(hip.load().spy_hip_op_rope, None, B(hip.tensor(dx, hip.F32, [hd, H_, T])), B(hip.tensor(dp, hip.I32, [T])),
+         B(hip.tensor(dy, hip.F32, [hd, H_, T])), B(hp))
+    got = dy.download(np.float32).reshape(x.shape)
+    assert_close(got, want, "rope", tol=1e-5)
+    assert np.array_equal(got[0], x[0])                                     # position 0 = identity
+    hp.mode = 2
+    assert hip.load().spy_hip_op_rope(None, B(hip.tensor(dx, hip.F32, [hd, H_, T])), B(hip.tensor(dp, hip.I32, [T])),
+                                      B(hip.tensor(dy, hip.F32, [hd, H_, T])), B(hp)) == hip.EUNSUPPORTED
+
+
+def test_kv_cache_copy_bit_exact(hip, oracle):
+    """KCache_cpy / VCache_cpy (attention.cpp:188-246 in the Spy tree) through the Copy operator."""
+    from tests.gpu_util import dev, call
+    rng = np.random.default_rng(6)
+    hd, H_, T, Cx, P = 128, 32, 3, 40, 17
+    d = hd * H_
+    k = rng.standard_normal((T, H_, hd)).astype(np.float32)
+    v = rng.standard_normal((T, d)).astype(np.float32)
+    kc = np.full((Cx, H_, hd), 0x7777, dtype=np.uint16)
+    vc = np.full((d, Cx), 0x7777, dtype=np.uint16)
+    want_k, want_v = kc.copy(), vc.copy()
+    assert oracle.spy_o_dup(B(O.tensor(k, O.F32, [hd, H_, T])), B(O.tensor(want_k, O.F16, [T * d], offset=2 * d * P))) == 0
+    assert oracle.spy_o_dup(B(O.tensor(v, O.F32, [T, d], nb=[4 * d, 4])), B(O.tensor(want_v, O.F16, [T, d], nb=[2, 2 * Cx], offset=2 * P))) == 0
+    dk, dv, dkc, dvc = dev(k), dev(v), dev(kc), dev(vc)
+    L = hip.load()
+    call(L.spy_hip_op_dup, None, B(hip.tensor(dk, hip.F32, [hd, H_, T])), B(hip.tensor(dkc, hip.F16, [T * d], offset=2 * d * P)))
+    call(L.spy_hip_op_dup, None, B(hip.tensor(dv, hip.F32, [T, d], nb=[4 * d, 4])), B(hip.tensor(dvc, hip.F16, [T, d], nb=[2, 2 * Cx], offset=2 * P)))
+    assert np.array_equal(dkc.download(np.uint16).reshape(kc.shape), want_k)
+    assert np.array_equal(dvc.download(np.uint16).reshape(vc.shape), want_v)
+
+
+def test_contiguous_and_get_row_and_argmax(hip, oracle):
+    from tests.gpu_util import dev, dev_empty, call
+    rng = np.random.default_rng(7)
+    hd, T, H_ = 128, 3, 32
+    o = rng.standard_normal((H_, T, hd)).astype(np.float32)
+    do, dd = dev(o), dev_empty(o.nbytes, 0xFF)
+    L = hip.load()
+    call(L.spy_hip_op_contiguous, None, B(hip.tensor(do, hip.F32, [hd, H_, T], nb=[4, 4 * hd * T, 4 * hd, 4 * hd * T * H_])), B(hip.tensor(dd, hip.F32, [hd, H_, T])))
+    assert np.array_equal(dd.download(np.float32).reshape(T, H_, hd), o.transpose(1, 0, 2))
+    # GetRow: F32 and Q8_0 tables
+    V, d = 1000, 4096
+    emb = rng.standard_normal((V, d)).astype(np.float32)
+    ids = np.array([3, 999, 0, 3, 512], dtype=np.int32)
+    q = O.quantize(oracle, emb, O.Q8_0)
+    for tab, tt in [(emb, O.F32), (q, O.Q8_0)]:
+        want = np.zeros((5, d), np.float32)
+        assert oracle.spy_o_get_row(B(O.tensor(tab, tt, [d, V])), B(O.tensor(ids, O.I32, [5])), B(O.tensor(want, O.F32, [d, 5]))) == 0
+        dt, di, dout = dev(tab), dev(ids), dev_empty(want.nbytes, 0xFF)
+        call(L.spy_hip_op_get_row, None, B(hip.tensor(dt, tt, [d, V])), B(hip.tensor(di, hip.I32, [5])), B(hip.tensor(dout, hip.F32, [d, 5])))
+        assert np.array_equal(dout.download(np.float32).reshape(5, d).view(np.uint32), want.view(np.uint32))
+    flag = C.c_int32(-1)
+    call(L.spy_hip_take_error, C.byref(flag)); assert flag.value == 0
+    bad = np.array([1000], dtype=np.int32)
+    call(L.spy_hip_op_get_row, None, B(hip.tensor(dt, tt, [d, V])), B(hip.tensor(dev(bad), hip.I32, [1])), B(hip.tensor(dout, hip.F32, [d, 1])))
+    call(L.spy_hip_take_error, C.byref(flag)); assert flag.value == 1       # the reference asserts here (view.cpp:61)
+    q4 = O.quantize(oracle, emb[:4], O.Q4_0)
+    assert L.spy_hip_op_get_row(None, B(hip.tensor(dev(q4), hip.Q4_0, [d, 4])), B(hip.tensor(di, hip.I32, [5])), B(hip.tensor(dout, hip.F32, [d, 5]))) == hip.EUNSUPPORTED
+    # argmax: first maximum
+    lg = rng.standard_normal(32000).astype(np.float32)
+    lg[[77, 31999, 4000]] = lg.max() + 1.0
+    dl, di32 = dev(lg), dev_empty(4, 0)
+    call(L.spy_hip_argmax, None, dl.ptr, 32000, di32.ptr)
+    assert di32.download(np.int32)[0] == oracle.spy_o_argmax(O.ptr(lg), 32000) == 77
+
+
+@pytest.mark.parametrize("wtype", [O.Q4_0, O.Q8_0, O.Q4_K, O.Q6_K])
+def test_op_matmul_quantized(hip, oracle, wtype):
+    from tests.gpu_util import dev, dev_empty, call, assert_close
+    rng = np.random.default_rng(8 + wtype)
+    M, K, T = 96, 4096, 5
+    w = O.quantize(oracle, (rng.standard_normal((M, K)) * 0.02).astype(np.float32), wtype)
+    x = rng.standard_normal((T, K)).astype(np.float32)
+    want = O.matmul(oracle, w, wtype, M, K, x, nthread=4)
+    dw, dx, dd = dev(w), dev(x), dev_empty(T * M * 4, 0xFF)
+    tw, tx, td = hip.tensor(dw, wtype, [K, M]), hip.tensor(dx, hip.F32, [K, T]), hip.tensor(dd, hip.F32, [M, T])
+    L = hip.load()
+    need = L.spy_hip_op_matmul_scratch_size(B(tw), B(tx))
+    assert need == T * (K // 32) * 34
+    assert L.spy_hip_op_matmul(None, B(tw), B(tx), B(td), None, 0) == hip.ENOSPACE
+    scratch = dev_empty(need, 0)
+    call(L.spy_hip_op_matmul, None, B(tw), B(tx), B(td), scratch.ptr, need)
+    assert_close(dd.download(np.float32).reshape(T, M), want, "op_matmul type %d" % wtype)
+    # activations: identical Q8_0 bytes to the oracle's
+    assert np.array_equal(scratch.download(np.uint8), O.quantize(oracle, x, O.Q8_0))
+
+
+def test_op_matmul_attention_views(hip, oracle):
+    """attn_score and KQV through the strided K / V^T cache views and the permuted Q."""
+    from tests.gpu_util import dev, dev_empty, call, assert_close
+    rng = np.random.default_rng(9)
+    hd, H_, T, n_kv, Cx = 128, 32, 2, 37, 64
+    d = hd * H_
+    kc = rng.standard_normal((Cx, H_, hd)).astype(np.float16)
+    vc = rng.standard_normal((d, Cx)).astype(np.float16)
+    q = rng.standard_normal((T, H_, hd)).astype(np.float32)
+    P = rng.random((H_, T, n_kv)).astype(np.float32)
+    S_want = np.zeros((H_, T, n_kv), np.float32)
+    O_want = np.zeros((H_, T, hd), np.float32)
+    assert oracle.spy_o_matmul(B(O.tensor(kc.view(np.uint16), O.F16, [hd, n_kv, H_], nb=[2, 2 * d, 2 * hd])),
+                               B(O.tensor(q, O.F32, [hd, T, H_], nb=[4, 4 * d, 4 * hd])), B(O.tensor(S_want, O.F32, [n_kv, T, H_])), 2) == 0
+    assert oracle.spy_o_matmul(B(O.tensor(vc.view(np.uint16), O.F16, [n_kv, hd, H_], nb=[2, 2 * Cx, 2 * Cx * hd])),
+                               B(O.tensor(P, O.F32, [n_kv, T, H_])), B(O.tensor(O_want, O.F32, [hd, T, H_])), 2) == 0
+    L = hip.load()
+    dkc, dvc, dq, dP = dev(kc.view(np.uint16)), dev(vc.view(np.uint16)), dev(q), dev(P)
+    dS, dO = dev_empty(S_want.nbytes, 0xFF), dev_empty(O_want.nbytes, 0xFF)
+    tk = hip.tensor(dkc, hip.F16, [hd, n_kv, H_], nb=[2, 2 * d, 2 * hd])
+    tq = hip.tensor(dq, hip.F32, [hd, T, H_], nb=[4, 4 * d, 4 * hd])
+    tS = hip.tensor(dS, hip.F32, [n_kv, T, H_])
+    need = L.spy_hip_op_matmul_scratch_size(B(tk), B(tq))
+    assert need == hd * T * H_ * 2
+    sc = dev_empty(need, 0)
+    call(L.spy_hip_op_matmul, None, B(tk), B(tq), B(tS), sc.ptr, need)
+    assert_close(dS.download(np.float32).reshape(S_want.shape), S_want, "attn_score", tol=1e-5)
+    tv = hip.tensor(dvc, hip.F16, [n_kv, hd, H_], nb=[2, 2 * Cx, 2 * Cx * hd])
+    tP = hip.tensor(dP, hip.F32, [n_kv, T, H_])
+    tO = hip.tensor(dO, hip.F32, [hd, T, H_])
+    need = L.spy_hip_op_matmul_scratch_size(B(tv), B(tP))
+    sc = dev_empty(need, 0)
+    call(L.spy_hip_op_matmul, None, B(tv), B(tP), B(tO), sc.ptr, need)
+    assert_close(dO.download(np.float32).reshape(O_want.shape), O_want, "KQV", tol=1e-5)
+    # F32 x F32 has no hip implementation: reported, not aborted
+    assert L.spy_hip_op_matmul(None, B(tq), B(tq), B(tS), None, 0) == hip.EUNSUPPORTED
