@@ -102,8 +102,8 @@ def test_gemv_zero_scale_and_single_block(hip, oracle):
     from tests.gpu_util import dev, dev_empty, call
     w = np.zeros((4, 18), np.uint8); w[:, 2:] = 0x5A                      # d = 0: every dot is exactly 0
     xq = O.quantize(oracle, np.linspace(-1, 1, 32).astype(np.float32), O.Q8_0)
-    dout = dev_empty(16, 0xFF)
-    call(hip.load().spy_hip_gemv_q8_0act, None, O.Q4_0, dev(w).ptr, dev(xq).ptr, dout.ptr, None, 4, 32, 1, 4)
+    dw, dxq, dout = dev(w), dev(xq), dev_empty(16, 0xFF)          # keep the buffers alive across the launch
+    call(hip.load().spy_hip_gemv_q8_0act, None, O.Q4_0, dw.ptr, dxq.ptr, dout.ptr, None, 4, 32, 1, 4)
     assert np.array_equal(dout.download(np.float32), np.zeros(4, np.float32))
 
 
@@ -117,8 +117,8 @@ def test_gemv_full_shapes_linearity(hip, oracle):
         w[:, :, :2] = (rng.uniform(0.5, 2, (M, K // 32)) * 0.0025).astype(np.float16).view(np.uint8).reshape(M, K // 32, 2)
         x = rng.standard_normal((1, K)).astype(np.float32)
         xq = O.quantize(oracle, x, O.Q8_0)
-        dout = dev_empty(M * 4, 0xFF)
-        call(hip.load().spy_hip_gemv_q8_0act, None, O.Q4_0, dev(w).ptr, dev(xq).ptr, dout.ptr, None, M, K, 1, M)
+        dw, dxq, dout = dev(w), dev(xq), dev_empty(M * 4, 0xFF)
+        call(hip.load().spy_hip_gemv_q8_0act, None, O.Q4_0, dw.ptr, dxq.ptr, dout.ptr, None, M, K, 1, M)
         got = dout.download(np.float32)
         rows = rng.choice(M, 64, replace=False)
         want = np.array([oracle.spy_o_dot_q4_0_q8_0(w[r].ctypes.data, O.ptr(xq), K) for r in rows], np.float32)

@@ -156,10 +156,12 @@ def test_contiguous_and_get_row_and_argmax(hip, oracle):
     flag = C.c_int32(-1)
     call(L.spy_hip_take_error, C.byref(flag)); assert flag.value == 0
     bad = np.array([1000], dtype=np.int32)
-    call(L.spy_hip_op_get_row, None, B(hip.tensor(dt, tt, [d, V])), B(hip.tensor(dev(bad), hip.I32, [1])), B(hip.tensor(dout, hip.F32, [d, 1])))
+    dbad = dev(bad)
+    call(L.spy_hip_op_get_row, None, B(hip.tensor(dt, tt, [d, V])), B(hip.tensor(dbad, hip.I32, [1])), B(hip.tensor(dout, hip.F32, [d, 1])))
     call(L.spy_hip_take_error, C.byref(flag)); assert flag.value == 1       # the reference asserts here (view.cpp:61)
     q4 = O.quantize(oracle, emb[:4], O.Q4_0)
-    assert L.spy_hip_op_get_row(None, B(hip.tensor(dev(q4), hip.Q4_0, [d, 4])), B(hip.tensor(di, hip.I32, [5])), B(hip.tensor(dout, hip.F32, [d, 5]))) == hip.EUNSUPPORTED
+    dq4 = dev(q4)
+    assert L.spy_hip_op_get_row(None, B(hip.tensor(dq4, hip.Q4_0, [d, 4])), B(hip.tensor(di, hip.I32, [5])), B(hip.tensor(dout, hip.F32, [d, 5]))) == hip.EUNSUPPORTED
     # argmax: first maximum
     lg = rng.standard_normal(32000).astype(np.float32)
     lg[[77, 31999, 4000]] = lg.max() + 1.0
