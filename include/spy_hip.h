@@ -128,6 +128,51 @@ int spy_hip_gemv_q8_0act(void *stream, int wtype, const void *w, const void *xq,
  * the last M slots receive the float results and are scratch. */
 int spy_hip_block_dots(void *stream, int wtype, const void *w, const void *xq, int32_t *out, int64_t M, int64_t K);
 
+/* ---- the token loop: replaces the per-operator dispatch of one forward pass
+ *      (DefaultGraphScheduler::execute, backend/distributor/include/scheduler/default_scheduler.h:46-111,
+ *      over the graph LLAMAModel::build_graph wires, model/src/llm/model/llama.cpp:86-264) and the
+ *      greedy loop of AutoModelGenerator::generate (app/cli/include/cli.h:88-128) for single-token
+ *      passes.  Same operators, same rounding points, same KV-cache layouts
+ *      (K: f16 [n_ctx][n_head][hd], V: f16 [n_embd][n_ctx]; model/src/llm/plugin/attention.cpp:188-262);
+ *      fused into six kernels per layer and replayed as a HIP graph. ----------------------------- */
+typedef struct spy_hip_llama_layer {
+    const float *attn_norm, *ffn_norm;                         /* f32[n_embd], device          */
+    const void  *wq, *wk, *wv, *wo, *w_gate, *w_up, *w_down;   /* native GGUF blocks, device   */
+} spy_hip_llama_layer;
+
+typedef struct spy_hip_llama_desc {
+    int32_t n_layer, n_embd, n_head, n_ff, n_vocab, n_ctx;     /* n_ctx % 8 == 0               */
+    float   eps, rope_freq_base;
+    int32_t wtype;                                             /* type of the 7 layer matrices: Q4_0 or Q8_0 */
+    const void  *tok_embd;  int32_t t_tok_embd;                /* F32 or Q8_0 (GetRow, view.cpp:65-77) */
+    const float *out_norm;
+    const void  *w_out;     int32_t t_out;                     /* Q4_0, Q8_0, Q4_K or Q6_K     */
+    const spy_hip_llama_layer *layers;                         /* host array of n_layer entries */
+} spy_hip_llama_desc;
+
+typedef struct spy_hip_llama spy_hip_llama;
+
+/* Allocates the KV caches (zero-filled) and the activation scratch on the current device --
+ * the Cache / Dynamic tensors the scheduler would request through alloc_memory
+ * (default_scheduler.h:157-175).  Weights stay where the caller uploaded them. */
+int spy_hip_llama_create(const spy_hip_llama_desc *desc, spy_hip_llama **out);
+int spy_hip_llama_destroy(spy_hip_llama *m);
+/* One forward pass over n_token tokens at positions n_past.. (any n_token >= 1; passes of more
+ * than one token run operator by operator).  logits_host: NULL or n_vocab*n_token floats. */
+int spy_hip_llama_forward(spy_hip_llama *m, void *stream, const int32_t *tokens_host, int32_t n_token, int32_t n_past,
+                          float *logits_host);
+/* n_steps single-token passes with greedy sampling on the device: step i consumes the token
+ * sampled by step i-1 (the first consumes first_token at position n_past) and tokens_host[i]
+ * receives the token sampled by step i.  use_graph: replay a captured HIP graph. */
+int spy_hip_llama_decode_greedy(spy_hip_llama *m, void *stream, int32_t first_token, int32_t n_past, int32_t n_steps,
+                                int32_t *tokens_host, int32_t use_graph);
+/* device pointers of the engine's buffers, for tests and profiling: name one of "k_cache",
+ * "v_cache" (layer 0..n_layer-1), "x", "logits", "scores", "attn_out" (layer ignored) */
+int spy_hip_llama_buffer(spy_hip_llama *m, const char *name, int32_t layer, void **ptr, size_t *bytes);
+/* average duration (ms) of the HIP-event-timed single-token passes since the last call, and their
+ * count; timing is recorded around every pass of spy_hip_llama_decode_greedy */
+int spy_hip_llama_timing(spy_hip_llama *m, float *ms_per_pass, int32_t *n_pass);
+
 #ifdef __cplusplus
 }
 #endif

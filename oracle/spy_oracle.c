@@ -1011,12 +1011,12 @@ int32_t spy_o_argmax(const float *logits, int64_t n) {
  * topological order with the host operators above.
  * ========================================================================================== */
 
-static struct { const char *name; int layer; float *out; } g_tap[16];
+static struct { char name[24]; int layer; float *out; } g_tap[16];
 static int g_ntap = 0;
 
 void spy_o_llama_tap(const char *name, int layer, float *out) {
     if (!name) { g_ntap = 0; return; }
-    if (g_ntap < 16) { g_tap[g_ntap].name = name; g_tap[g_ntap].layer = layer; g_tap[g_ntap].out = out; g_ntap++; }
+    if (g_ntap < 16) { strncpy(g_tap[g_ntap].name, name, 23); g_tap[g_ntap].name[23] = 0; g_tap[g_ntap].layer = layer; g_tap[g_ntap].out = out; g_ntap++; }
 }
 
 static void tap(const char *name, int layer, const float *src, int64_t n) {

@@ -35,6 +35,19 @@ class RopeParam(C.Structure):
                 ("beta_slow", C.c_float), ("xpos_base", C.c_float), ("xpos_down", C.c_int32)]
 
 
+class LlamaLayer(C.Structure):
+    """spy_hip_llama_layer"""
+    _fields_ = [(n, C.c_void_p) for n in ("attn_norm", "ffn_norm", "wq", "wk", "wv", "wo", "w_gate", "w_up", "w_down")]
+
+
+class LlamaDesc(C.Structure):
+    """spy_hip_llama_desc"""
+    _fields_ = [("n_layer", C.c_int32), ("n_embd", C.c_int32), ("n_head", C.c_int32), ("n_ff", C.c_int32),
+                ("n_vocab", C.c_int32), ("n_ctx", C.c_int32), ("eps", C.c_float), ("rope_freq_base", C.c_float),
+                ("wtype", C.c_int32), ("tok_embd", C.c_void_p), ("t_tok_embd", C.c_int32), ("out_norm", C.c_void_p),
+                ("w_out", C.c_void_p), ("t_out", C.c_int32), ("layers", C.POINTER(LlamaLayer))]
+
+
 class SpyHipError(RuntimeError):
     def __init__(self, code, what):
         self.code = code
@@ -78,6 +91,12 @@ SIGNATURES = {
     "spy_hip_quantize_f16": (_i32, [_vp, _vp, _i64, _vp, _i64, _i64]),
     "spy_hip_gemv_q8_0act": (_i32, [_vp, _i32, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64]),
     "spy_hip_block_dots": (_i32, [_vp, _i32, _vp, _vp, _vp, _i64, _i64]),
+    "spy_hip_llama_create": (_i32, [C.POINTER(LlamaDesc), C.POINTER(_vp)]),
+    "spy_hip_llama_destroy": (_i32, [_vp]),
+    "spy_hip_llama_forward": (_i32, [_vp, _vp, _vp, _i32, _i32, _vp]),
+    "spy_hip_llama_decode_greedy": (_i32, [_vp, _vp, _i32, _i32, _i32, _vp, _i32]),
+    "spy_hip_llama_buffer": (_i32, [_vp, C.c_char_p, _i32, C.POINTER(_vp), C.POINTER(_sz)]),
+    "spy_hip_llama_timing": (_i32, [_vp, C.POINTER(_f32), C.POINTER(_i32)]),
 }
 
 

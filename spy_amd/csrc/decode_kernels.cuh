@@ -1,0 +1,281 @@
+// Kernels of the fused single-token pass (decode).  Six launches per layer:
+//   qkv      : RMSNorm*w -> Q8_0 (in LDS) -> wq|wk|wv GEMV -> RoPE -> q (fp16), K cache, V^T cache
+//   scores   : s[h][j] = (K[j,h] . fp16(q[h])) * scale            (split over tokens)
+//   pv       : softmax with the reference's fp16 rounding points, then P.V (split over head dims)
+//   wo       : Q8_0(attn) -> wo GEMV -> + residual
+//   gate_up  : RMSNorm*w -> Q8_0 -> gate|up GEMV -> up * silu(gate)
+//   down     : Q8_0(h) -> down GEMV -> + residual
+// Every rounding point of the operator-by-operator graph is kept (see the comments at each step);
+// only fp32 summation orders differ.
+#pragma once
+
+#include "gemv_core.cuh"
+
+struct dev_state {           // lives in device memory so that a captured graph can be replayed
+    int32_t token;           // token consumed by this pass
+    int32_t pos;             // its position = number of tokens already in the KV cache
+    int32_t step;            // passes done since the loop was armed
+    int32_t err;
+};
+
+// ---- persistent GEMV over row tiles with double-buffered weight registers ----------------------
+template <int WT, int LPR> struct gemv_stream {
+    static constexpr int RPW = SPY_WAVE / LPR, RPT = GEMV_WAVES * RPW;
+    wtile<WT> A, B;
+    int tile, ntiles, G, npair, nit, l, g, rofs, M;
+    size_t RB;
+
+    template <class RowPtr> __device__ __forceinline__ void begin(int M_, int K, RowPtr rowptr) {
+        M = M_;
+        const int nblk = K / 32;
+        npair = K / 64; nit = (npair + LPR - 1) / LPR;
+        RB = (size_t)nblk * wt_traits<WT>::BLK;
+        const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+        l = lane % LPR; g = lane / LPR; rofs = wave * RPW + g;
+        ntiles = (M + RPT - 1) / RPT; G = gridDim.x; tile = blockIdx.x;
+        if (tile < ntiles && tile * RPT + rofs < M) load_tile<WT, LPR>(A, rowptr(tile * RPT + rofs), npair, nit, l);
+    }
+
+    // epi(r, total, valid): called by every lane; `total` is the row's dot, present in all LPR lanes
+    template <class RowPtr, class Epi> __device__ __forceinline__ void run(const staged_act &act, RowPtr rowptr, Epi epi) {
+        auto finish = [&](const wtile<WT> &t, int tl) {
+            const int r = tl * RPT + rofs;
+            float acc[1] = {0.0f};
+            if (r < M) dot_tile<WT, LPR, 1>(t, &act, npair, nit, l, acc, nullptr);
+            epi(r, group_sum<LPR>(acc[0]), r < M);
+        };
+        while (tile < ntiles) {
+            int tn = tile + G;
+            if (tn < ntiles && tn * RPT + rofs < M) load_tile<WT, LPR>(B, rowptr(tn * RPT + rofs), npair, nit, l);
+            finish(A, tile);
+            tile = tn;
+            if (tile >= ntiles) break;
+            tn = tile + G;
+            if (tn < ntiles && tn * RPT + rofs < M) load_tile<WT, LPR>(A, rowptr(tn * RPT + rofs), npair, nit, l);
+            finish(B, tile);
+            tile = tn;
+        }
+    }
+};
+
+// silu as the reference's table: v = float(fp16(x)); v / (1 + expf(-v))  (non-linear.cpp:11-14)
+static __device__ __forceinline__ float silu_lut(float x) {
+    const float v = h2f(f2h(x));
+    return v / (1.0f + expf(-v));
+}
+
+// ---- token embedding + RoPE table ---------------------------------------------------------------
+// GetRow (view.cpp:33-81): F32 copy or Q8_0 dequant.  The cos/sin table of this position follows
+// the reference's recurrence: theta_0 = pos, theta_{k+1} = theta_k * theta_scale in fp32
+// (non-linear.cpp:304-309), cosf / sinf of it.
+__global__ __launch_bounds__(256) void embed_kernel(dev_state *st, const uint8_t *__restrict__ table, int q8, int d, int n_vocab,
+                                                    float *__restrict__ x, float *__restrict__ rope_cs, float theta_scale, int hd) {
+    int tok = st->token;
+    if (tok < 0 || tok >= n_vocab) { if (threadIdx.x == 0) st->err = 1; tok = 0; }
+    if (!q8) {
+        const float *row = (const float *)table + (size_t)tok * d;
+        for (int i = threadIdx.x; i < d; i += 256) x[i] = row[i];
+    } else {
+        const blk_q8_0 *row = (const blk_q8_0 *)(table + (size_t)tok * (d / 32) * 34);
+        for (int i = threadIdx.x; i < d; i += 256) x[i] = (float)row[i >> 5].qs[i & 31] * h2f(row[i >> 5].d);
+    }
+    for (int k = threadIdx.x; k < hd / 2; k += 256) {
+        float theta = (float)st->pos;
+        for (int j = 0; j < k; j++) theta *= theta_scale;
+        rope_cs[2 * k] = cosf(theta);
+        rope_cs[2 * k + 1] = sinf(theta);
+    }
+}
+
+// ---- fused GEMVs ----------------------------------------------------------------------------------
+struct fused_args {
+    const uint8_t *W0, *W1, *W2;
+    int M, K;                      // total rows over all matrices, contraction length
+    const float *x_in;             // f32[K] prologue input
+    const float *normw; float eps; // RMSNorm weight (NORM prologue)
+    const float *resid; float *out;
+    const dev_state *st; const float *rope_cs; uint16_t *q16; uint16_t *kc; uint16_t *vc;
+    int n_ctx, d, hd;
+};
+
+enum { EPI_QKV = 0, EPI_RESID = 1, EPI_GATEUP = 2, EPI_STORE = 3 };
+
+template <int WT, int LPR, bool NORM, int EPI>
+__global__ __launch_bounds__(GEMV_THREADS) void fused_gemv_kernel(fused_args a) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    __shared__ float s_red[4];
+    const size_t RB = (size_t)(a.K / 32) * wt_traits<WT>::BLK;
+    auto rowptr = [&](int r) -> const uint8_t * {
+        if constexpr (EPI == EPI_QKV) { const int m = r / a.d, row = r - m * a.d; return (m == 0 ? a.W0 : (m == 1 ? a.W1 : a.W2)) + (size_t)row * RB; }
+        else if constexpr (EPI == EPI_GATEUP) return ((r & 1) ? a.W1 : a.W0) + (size_t)(r >> 1) * RB;
+        else return a.W0 + (size_t)r * RB;
+    };
+    gemv_stream<WT, LPR> gs;
+    gs.begin(a.M, a.K, rowptr);                      // first tile's weights are in flight from here on
+
+    int8_t *s_q = (int8_t *)smem;
+    int2 *s_meta = (int2 *)(smem + a.K);
+    stage_f32<NORM>(a.x_in, a.normw, a.eps, s_q, s_meta, a.K, s_red);
+    staged_act act; act.q = s_q; act.meta = s_meta;
+
+    const int l = gs.l;
+    auto epi = [&](int r, float s, bool valid) {
+        if constexpr (EPI == EPI_RESID) { if (valid && l == 0) a.out[r] = s + a.resid[r]; }
+        else if constexpr (EPI == EPI_STORE) { if (valid && l == 0) a.out[r] = s; }
+        else if constexpr (EPI == EPI_GATEUP) {
+            // rows 2i (gate) and 2i+1 (up) sit in neighbouring lane groups
+            const float other = __shfl_xor(s, LPR, SPY_WAVE);
+            if (valid && l == 0 && (r & 1) == 0) a.out[r >> 1] = other * silu_lut(s);   // Mul(ffn_up, silu(ffn_gate)) (ffn.cpp:24-35)
+        } else {
+            const float other = __shfl_xor(s, LPR, SPY_WAVE);
+            if (valid && l == 0) {
+                const int m = r / a.d, row = r - m * a.d, pos = a.st->pos;
+                if (m == 2) a.vc[(size_t)row * a.n_ctx + pos] = f2h(s);                    // VCache_cpy: [d][C] column pos
+                else {
+                    const int k = (row % a.hd) >> 1;
+                    const float c = a.rope_cs[2 * k], sn = a.rope_cs[2 * k + 1];
+                    // (x0, x1) -> (x0*c - x1*s, x0*s + x1*c) on adjacent rows (non-linear.cpp:359-363)
+                    const float v = (row & 1) ? (other * sn + s * c) : (s * c - other * sn);
+                    if (m == 0) a.q16[row] = f2h(v);                                       // attn_score rounds Q to fp16 (mat.cpp:37)
+                    else a.kc[(size_t)pos * a.d + row] = f2h(v);                           // KCache_cpy: [token][head][hd]
+                }
+            }
+        }
+    };
+    gs.run(act, rowptr, epi);
+}
+
+// ---- attention scores ---------------------------------------------------------------------------
+// One workgroup per chunk of ATT_TCH cached tokens, all heads: a (token, head) key is 256 bytes
+// = 16 lanes x 128-bit.  t = (K.q + mask) * scale with mask = 0 for every cached token of a
+// single-token pass (llama.cpp:248-257), i.e. t = dot * scale.
+#define ATT_TCH 8
+__global__ __launch_bounds__(256) void attn_scores_kernel(const dev_state *st, const uint16_t *__restrict__ q16, const uint16_t *__restrict__ kc,
+                                                          float *__restrict__ scores, int n_head, int n_ctx, float scale) {
+    const int n_kv = st->pos + 1;
+    const int t0 = blockIdx.x * ATT_TCH;
+    if (t0 >= n_kv) return;
+    const int d = n_head * 128;
+    const int piece = threadIdx.x & 15, hsel = threadIdx.x >> 4;     // 16 heads per pass over the workgroup
+    for (int h0 = 0; h0 < n_head; h0 += 16) {
+        const int head = h0 + hsel;
+        const bool hok = head < n_head;
+        float qf[8];
+        {
+            const uint4 qv = hok ? *(const uint4 *)(q16 + head * 128 + piece * 8) : make_uint4(0, 0, 0, 0);
+            const uint32_t qw[4] = {qv.x, qv.y, qv.z, qv.w};
+#pragma unroll
+            for (int j = 0; j < 4; j++) { qf[2 * j] = h2f((uint16_t)(qw[j] & 0xFFFFu)); qf[2 * j + 1] = h2f((uint16_t)(qw[j] >> 16)); }
+        }
+        uint4 kv[ATT_TCH];
+#pragma unroll
+        for (int tt = 0; tt < ATT_TCH; tt++)
+            if (hok && t0 + tt < n_kv) kv[tt] = *(const uint4 *)(kc + (size_t)(t0 + tt) * d + head * 128 + piece * 8);
+#pragma unroll
+        for (int tt = 0; tt < ATT_TCH; tt++) {
+            float s = 0.0f;
+            if (hok && t0 + tt < n_kv) {
+                const uint32_t kw[4] = {kv[tt].x, kv[tt].y, kv[tt].z, kv[tt].w};
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    s = fmaf(h2f((uint16_t)(kw[j] & 0xFFFFu)), qf[2 * j], s);
+                    s = fmaf(h2f((uint16_t)(kw[j] >> 16)), qf[2 * j + 1], s);
+                }
+            }
+            s = group_sum<16>(s);
+            if (hok && piece == 0 && t0 + tt < n_kv) scores[(size_t)head * n_ctx + t0 + tt] = s * scale;
+        }
+    }
+}
+
+// ---- softmax + P.V ------------------------------------------------------------------------------
+// One workgroup per (head, 16 head dims).  The softmax of the head's row is recomputed by each of
+// the 8 workgroups of a head (n_kv expf per workgroup): m = max t; e = expf(float(fp16(t - m)));
+// p = e * (1/sum e) (non-linear.cpp:158-176); P is rounded to fp16 for the KQV product
+// (mat.cpp:37, vec_dot.h:117-146).  V^T rows are contiguous along tokens: 16 lanes x 128-bit.
+__global__ __launch_bounds__(256) void attn_pv_kernel(const dev_state *st, const float *__restrict__ scores, const uint16_t *__restrict__ vc,
+                                                      float *__restrict__ attn_out, int n_ctx) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    __shared__ float s_part[4];
+    const int n_kv = st->pos + 1;
+    const int head = blockIdx.x >> 3, dgrp = blockIdx.x & 7;
+    float *s_t = (float *)smem;                               // n_ctx floats
+    uint16_t *s_p = (uint16_t *)(smem + (size_t)n_ctx * 4);    // n_ctx halfs (+ pad)
+    const float *srow = scores + (size_t)head * n_ctx;
+    float mx = -INFINITY;
+    for (int j = threadIdx.x; j < n_kv; j += 256) { const float t = srow[j]; s_t[j] = t; mx = fmaxf(mx, t); }
+    mx = wave_max(mx);
+    if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(s_part[0], s_part[1]), fmaxf(s_part[2], s_part[3]));
+    __syncthreads();
+    float sum = 0.0f;
+    for (int j = threadIdx.x; j < n_kv; j += 256) { const float e = expf(h2f(f2h(s_t[j] - mx))); s_t[j] = e; sum += e; }
+    sum = wave_sum(sum);
+    if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = sum;
+    __syncthreads();
+    sum = (s_part[0] + s_part[1]) + (s_part[2] + s_part[3]);
+    const float inv = 1.0f / sum;
+    const int n_pad = (n_kv + 7) & ~7;
+    for (int j = threadIdx.x; j < n_pad; j += 256) s_p[j] = j < n_kv ? f2h(s_t[j] * inv) : (uint16_t)0;
+    __syncthreads();
+
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l = lane & 15, g = lane >> 4;
+    const int row = head * 128 + dgrp * 16 + wave * 4 + g;
+    const uint16_t *vrow = vc + (size_t)row * n_ctx;
+    const int npiece = n_pad >> 3;
+    float acc = 0.0f;
+    for (int pc0 = 0; pc0 < npiece; pc0 += 64) {
+        uint4 vv[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) { const int pc = pc0 + u * 16 + l; if (pc < npiece) vv[u] = *(const uint4 *)(vrow + pc * 8); }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int pc = pc0 + u * 16 + l;
+            if (pc < npiece) {
+                const uint4 pp = *(const uint4 *)(s_p + pc * 8);
+                const uint32_t vw[4] = {vv[u].x, vv[u].y, vv[u].z, vv[u].w}, pw[4] = {pp.x, pp.y, pp.z, pp.w};
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    // cache slots past n_kv hold whatever was there before: never multiply them in
+                    if (pc * 8 + 2 * j < n_kv) acc = fmaf(h2f((uint16_t)(vw[j] & 0xFFFFu)), h2f((uint16_t)(pw[j] & 0xFFFFu)), acc);
+                    if (pc * 8 + 2 * j + 1 < n_kv) acc = fmaf(h2f((uint16_t)(vw[j] >> 16)), h2f((uint16_t)(pw[j] >> 16)), acc);
+                }
+            }
+        }
+    }
+    acc = group_sum<16>(acc);
+    if (l == 0) attn_out[row] = acc;
+}
+
+// ---- greedy sampling + loop advance -------------------------------------------------------------
+// argmax with std::max_element's first-maximum rule (greedy.h:20-25), then the loop step of
+// AutoModelGenerator::generate (cli.h:121-123): the sampled token becomes the next input at pos+1.
+__global__ __launch_bounds__(1024) void sample_advance_kernel(dev_state *st, const float *__restrict__ logits, int n, int32_t *__restrict__ tokens_out,
+                                                              int max_out) {
+    __shared__ float s_v[16];
+    __shared__ int s_i[16];
+    float best = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int i = threadIdx.x; i < n; i += 1024) {
+        const float v = logits[i];
+        if (v > best || (bi == 0x7fffffff && !(v < best))) { best = v; bi = i; }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(best, o, SPY_WAVE);
+        const int oi = __shfl_xor(bi, o, SPY_WAVE);
+        if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
+    }
+    if ((threadIdx.x & 63) == 0) { s_v[threadIdx.x >> 6] = best; s_i[threadIdx.x >> 6] = bi; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 16; w++) if (s_v[w] > best || (s_v[w] == best && s_i[w] < bi)) { best = s_v[w]; bi = s_i[w]; }
+        if (bi == 0x7fffffff) bi = 0;
+        const int step = st->step;
+        if (step < max_out) tokens_out[step] = bi;
+        st->token = bi;
+        st->pos = st->pos + 1;
+        st->step = step + 1;
+    }
+}

@@ -1,0 +1,418 @@
+// The token loop on the device: one forward pass of the LLaMA graph
+// (model/src/llm/model/llama.cpp:86-264 and plugins in the Spy tree) for a single new token as
+// six fused kernels per layer, greedy sampling on the device (greedy.h:20-25, cli.h:88-128), the
+// whole pass captured once as a HIP graph and replayed per token.  Passes over several tokens
+// (prompts) run operator by operator through the spy_hip_op_* entry points, exactly as the graph
+// lists them.
+#include "decode_kernels.cuh"
+
+#include <math.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#include <vector>
+
+#define HIP_TRY(x) do { hipError_t e_ = (x); if (e_ != hipSuccess) return (int)e_; } while (0)
+#define RC_TRY(x) do { int rc_ = (x); if (rc_) return rc_; } while (0)
+
+struct spy_hip_llama {
+    spy_hip_llama_desc desc;
+    std::vector<spy_hip_llama_layer> layers;
+    int hd = 0, lpr_d = 0, lpr_ff = 0;
+    std::vector<uint16_t *> k_cache, v_cache;
+    float *x = nullptr, *x1 = nullptr, *attn_out = nullptr, *hbuf = nullptr, *scores = nullptr, *logits = nullptr, *rope_cs = nullptr;
+    uint16_t *q16 = nullptr;
+    uint8_t *xq_head = nullptr;          // native Q8_0 activations for a K-quant output head
+    dev_state *st = nullptr;
+    int32_t *tokens_out = nullptr;
+    int max_out = 0;
+    int num_cu = 256;
+    float theta_scale = 0.0f;
+    // op-by-op path scratch (sized lazily for the largest chunk seen)
+    uint8_t *ops_buf = nullptr; size_t ops_bytes = 0;
+    // graph of one single-token pass
+    hipGraph_t graph = nullptr; hipGraphExec_t graph_exec = nullptr; hipStream_t graph_stream = nullptr;
+    hipStream_t own_stream = nullptr;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    double timed_ms = 0.0; int timed_pass = 0;
+    std::vector<void *> owned;
+};
+
+static int dalloc(spy_hip_llama *m, void **p, size_t bytes, bool zero) {
+    HIP_TRY(hipMalloc(p, bytes));
+    m->owned.push_back(*p);
+    if (zero) HIP_TRY(hipMemset(*p, 0, bytes));
+    return 0;
+}
+
+extern "C" int spy_hip_llama_destroy(spy_hip_llama *m) {
+    if (!m) return 0;
+    (void)hipDeviceSynchronize();
+    if (m->graph_exec) (void)hipGraphExecDestroy(m->graph_exec);
+    if (m->graph) (void)hipGraphDestroy(m->graph);
+    if (m->own_stream) (void)hipStreamDestroy(m->own_stream);
+    if (m->ev0) (void)hipEventDestroy(m->ev0);
+    if (m->ev1) (void)hipEventDestroy(m->ev1);
+    for (void *p : m->owned) (void)hipFree(p);
+    if (m->ops_buf) (void)hipFree(m->ops_buf);
+    delete m;
+    return 0;
+}
+
+extern "C" int spy_hip_llama_create(const spy_hip_llama_desc *desc, spy_hip_llama **out) {
+    SPY_CHECK_ARG(desc && out && desc->layers);
+    *out = nullptr;
+    const spy_hip_llama_desc &c = *desc;
+    SPY_CHECK_ARG(c.n_layer > 0 && c.n_embd > 0 && c.n_head > 0 && c.n_ff > 0 && c.n_vocab > 0 && c.n_ctx > 0);
+    SPY_CHECK_ARG(c.n_embd % c.n_head == 0 && c.n_ctx % 8 == 0 && c.n_embd % 64 == 0 && c.n_ff % 64 == 0);
+    SPY_CHECK_ARG(c.tok_embd && c.out_norm && c.w_out);
+    if (c.wtype != SPY_HIP_Q4_0 && c.wtype != SPY_HIP_Q8_0) return SPY_HIP_EUNSUPPORTED;
+    if (c.t_tok_embd != SPY_HIP_F32 && c.t_tok_embd != SPY_HIP_Q8_0) return SPY_HIP_EUNSUPPORTED;     // GetRow (view.cpp:65-77)
+    if (c.t_out != SPY_HIP_Q4_0 && c.t_out != SPY_HIP_Q8_0 && c.t_out != SPY_HIP_Q4_K && c.t_out != SPY_HIP_Q6_K) return SPY_HIP_EUNSUPPORTED;
+    if ((c.t_out == SPY_HIP_Q4_K || c.t_out == SPY_HIP_Q6_K) && c.n_embd % 256 != 0) return SPY_HIP_EINVAL;
+    spy_hip_llama *m = new spy_hip_llama();
+    m->desc = c;
+    m->layers.assign(c.layers, c.layers + c.n_layer);
+    m->desc.layers = m->layers.data();
+    m->hd = c.n_embd / c.n_head;
+    for (int i = 0; i < c.n_layer; i++) {
+        const spy_hip_llama_layer &L = m->layers[i];
+        if (!L.attn_norm || !L.ffn_norm || !L.wq || !L.wk || !L.wv || !L.wo || !L.w_gate || !L.w_up || !L.w_down) { delete m; return SPY_HIP_EINVAL; }
+    }
+    m->lpr_d  = c.wtype == SPY_HIP_Q4_0 ? pick_lpr<SPY_HIP_Q4_0>(c.n_embd) : pick_lpr<SPY_HIP_Q8_0>(c.n_embd);
+    m->lpr_ff = c.wtype == SPY_HIP_Q4_0 ? pick_lpr<SPY_HIP_Q4_0>(c.n_ff) : pick_lpr<SPY_HIP_Q8_0>(c.n_ff);
+    {
+        int dev = 0; hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0) m->num_cu = prop.multiProcessorCount;
+    }
+    m->theta_scale = powf(c.rope_freq_base, -2.0f / (float)m->hd);      // non-linear.cpp:282, host libm like the reference
+    const size_t d = c.n_embd, C = c.n_ctx;
+    int rc = 0;
+    m->k_cache.resize(c.n_layer); m->v_cache.resize(c.n_layer);
+    for (int i = 0; i < c.n_layer && !rc; i++) {
+        rc = dalloc(m, (void **)&m->k_cache[i], C * d * 2, true);
+        if (!rc) rc = dalloc(m, (void **)&m->v_cache[i], C * d * 2, true);
+    }
+    if (!rc) rc = dalloc(m, (void **)&m->x, d * 4, true);
+    if (!rc) rc = dalloc(m, (void **)&m->x1, d * 4, true);
+    if (!rc) rc = dalloc(m, (void **)&m->attn_out, d * 4, true);
+    if (!rc) rc = dalloc(m, (void **)&m->hbuf, (size_t)c.n_ff * 4, true);
+    if (!rc) rc = dalloc(m, (void **)&m->scores, (size_t)c.n_head * C * 4, true);
+    if (!rc) rc = dalloc(m, (void **)&m->logits, (size_t)c.n_vocab * 4, true);
+    if (!rc) rc = dalloc(m, (void **)&m->rope_cs, (size_t)m->hd * 4, true);
+    if (!rc) rc = dalloc(m, (void **)&m->q16, d * 2, true);
+    if (!rc) rc = dalloc(m, (void **)&m->xq_head, (d / 32) * 34, true);
+    if (!rc) rc = dalloc(m, (void **)&m->st, sizeof(dev_state), true);
+    m->max_out = 1 << 16;
+    if (!rc) rc = dalloc(m, (void **)&m->tokens_out, (size_t)m->max_out * 4, true);
+    if (!rc) rc = (int)hipEventCreate(&m->ev0);
+    if (!rc) rc = (int)hipEventCreate(&m->ev1);
+    if (!rc) rc = (int)hipStreamCreateWithFlags(&m->own_stream, hipStreamNonBlocking);
+    {   // softmax + P.V keeps one head's scores (f32) and probabilities (f16) in LDS
+        const size_t pv_lds = C * 4 + C * 2 + 16;
+        if (!rc && pv_lds > 160 * 1024) rc = SPY_HIP_EUNSUPPORTED;
+        if (!rc && pv_lds > 48 * 1024) rc = (int)hipFuncSetAttribute((const void *)attn_pv_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)pv_lds);
+    }
+    if (rc) { spy_hip_llama_destroy(m); return rc; }
+    *out = m;
+    return 0;
+}
+
+extern "C" int spy_hip_llama_buffer(spy_hip_llama *m, const char *name, int32_t layer, void **ptr, size_t *bytes) {
+    SPY_CHECK_ARG(m && name && ptr);
+    const size_t d = m->desc.n_embd, C = m->desc.n_ctx;
+    void *p = nullptr; size_t n = 0;
+    if (!strcmp(name, "k_cache") || !strcmp(name, "v_cache")) {
+        SPY_CHECK_ARG(layer >= 0 && layer < m->desc.n_layer);
+        p = name[0] == 'k' ? (void *)m->k_cache[layer] : (void *)m->v_cache[layer]; n = C * d * 2;
+    } else if (!strcmp(name, "x")) { p = m->x; n = d * 4; }
+    else if (!strcmp(name, "logits")) { p = m->logits; n = (size_t)m->desc.n_vocab * 4; }
+    else if (!strcmp(name, "scores")) { p = m->scores; n = (size_t)m->desc.n_head * C * 4; }
+    else if (!strcmp(name, "attn_out")) { p = m->attn_out; n = d * 4; }
+    else return SPY_HIP_EINVAL;
+    *ptr = p;
+    if (bytes) *bytes = n;
+    return 0;
+}
+
+extern "C" int spy_hip_llama_timing(spy_hip_llama *m, float *ms_per_pass, int32_t *n_pass) {
+    SPY_CHECK_ARG(m);
+    if (ms_per_pass) *ms_per_pass = m->timed_pass ? (float)(m->timed_ms / m->timed_pass) : 0.0f;
+    if (n_pass) *n_pass = m->timed_pass;
+    m->timed_ms = 0.0; m->timed_pass = 0;
+    return 0;
+}
+
+// ---- the fused single-token pass -----------------------------------------------------------------
+template <int WT, int LPR, bool NORM, int EPI>
+static int launch_fused(spy_hip_llama *m, hipStream_t st, const fused_args &a) {
+    constexpr int RPT = GEMV_WAVES * (SPY_WAVE / LPR);
+    const size_t lds = staged_bytes(a.K);
+    auto kern = fused_gemv_kernel<WT, LPR, NORM, EPI>;
+    if (lds > 48 * 1024) HIP_TRY(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    const int ntiles = (a.M + RPT - 1) / RPT;
+    const int cap = 4 * m->num_cu;
+    kern<<<dim3((unsigned)(ntiles < cap ? ntiles : cap)), dim3(GEMV_THREADS), lds, st>>>(a);
+    return SPY_LAUNCH_RC();
+}
+
+template <int WT, bool NORM, int EPI>
+static int launch_fused_lpr(spy_hip_llama *m, hipStream_t st, int lpr, const fused_args &a) {
+    switch (lpr) {
+    case 16: return launch_fused<WT, 16, NORM, EPI>(m, st, a);
+    case 32: return launch_fused<WT, 32, NORM, EPI>(m, st, a);
+    case 64: if constexpr (EPI == EPI_RESID || EPI == EPI_STORE) return launch_fused<WT, 64, NORM, EPI>(m, st, a); else break;
+    }
+    return SPY_HIP_EUNSUPPORTED;
+}
+
+static bool fused_ok(const spy_hip_llama *m) {
+    // the fused kernels assume 128-wide heads (one key = 16 lanes x 128 bit) and row pairs that
+    // share a wave in the qkv / gate-up epilogues
+    return m->hd == 128 && (m->lpr_d == 16 || m->lpr_d == 32) && m->lpr_ff != 0 && m->desc.n_embd % 4 == 0;
+}
+
+template <int WT>
+static int enqueue_pass(spy_hip_llama *m, hipStream_t st, bool sample) {
+    const spy_hip_llama_desc &c = m->desc;
+    const int d = c.n_embd, F = c.n_ff, C = c.n_ctx, H = c.n_head;
+    embed_kernel<<<dim3(1), dim3(256), 0, st>>>(m->st, (const uint8_t *)c.tok_embd, c.t_tok_embd == SPY_HIP_Q8_0, d, c.n_vocab, m->x,
+                                                m->rope_cs, m->theta_scale, m->hd);
+    RC_TRY(SPY_LAUNCH_RC());
+    const float scale = 1.0f / sqrtf((float)m->hd);                     // SoftmaxParam::scale (attention.cpp:113)
+    const size_t pv_lds = (size_t)C * 4 + (size_t)C * 2 + 16;
+    for (int il = 0; il < c.n_layer; il++) {
+        const spy_hip_llama_layer &L = m->layers[il];
+        fused_args a;
+        memset(&a, 0, sizeof(a));
+        a.st = m->st; a.rope_cs = m->rope_cs; a.q16 = m->q16; a.kc = m->k_cache[il]; a.vc = m->v_cache[il];
+        a.n_ctx = C; a.d = d; a.hd = m->hd; a.eps = c.eps;
+        // attn_norm, attn_norm_linear, Q/K/V_project, rope, KV-cache copies
+        a.W0 = (const uint8_t *)L.wq; a.W1 = (const uint8_t *)L.wk; a.W2 = (const uint8_t *)L.wv;
+        a.M = 3 * d; a.K = d; a.x_in = m->x; a.normw = L.attn_norm;
+        RC_TRY((launch_fused_lpr<WT, true, EPI_QKV>(m, st, m->lpr_d, a)));
+        // attn_score
+        attn_scores_kernel<<<dim3((unsigned)((C + ATT_TCH - 1) / ATT_TCH)), dim3(256), 0, st>>>(m->st, m->q16, m->k_cache[il], m->scores, H, C, scale);
+        RC_TRY(SPY_LAUNCH_RC());
+        // softmax, KQV (+ permute/contiguous: attn_out is already [hd, H] contiguous)
+        attn_pv_kernel<<<dim3((unsigned)(H * 8)), dim3(256), pv_lds, st>>>(m->st, m->scores, m->v_cache[il], m->attn_out, C);
+        RC_TRY(SPY_LAUNCH_RC());
+        // KQV_linear + ffn_input
+        a.W0 = (const uint8_t *)L.wo; a.M = d; a.K = d; a.x_in = m->attn_out; a.resid = m->x; a.out = m->x1;
+        RC_TRY((launch_fused_lpr<WT, false, EPI_RESID>(m, st, m->lpr_d, a)));
+        // ffn_norm, ffn_up, ffn_gate, silu, ffn_par
+        a.W0 = (const uint8_t *)L.w_gate; a.W1 = (const uint8_t *)L.w_up; a.M = 2 * F; a.K = d; a.x_in = m->x1; a.normw = L.ffn_norm; a.out = m->hbuf;
+        RC_TRY((launch_fused_lpr<WT, true, EPI_GATEUP>(m, st, m->lpr_d, a)));
+        // ffn_down + logit_output (the next layer's input)
+        a.W0 = (const uint8_t *)L.w_down; a.M = d; a.K = F; a.x_in = m->hbuf; a.resid = m->x1; a.out = m->x;
+        RC_TRY((launch_fused_lpr<WT, false, EPI_RESID>(m, st, m->lpr_ff, a)));
+    }
+    // result_norm, result_linear, output
+    if (c.t_out == c.wtype) {
+        fused_args a;
+        memset(&a, 0, sizeof(a));
+        a.W0 = (const uint8_t *)c.w_out; a.M = c.n_vocab; a.K = d; a.x_in = m->x; a.normw = c.out_norm; a.eps = c.eps; a.out = m->logits;
+        RC_TRY((launch_fused_lpr<WT, true, EPI_STORE>(m, st, m->lpr_d, a)));
+    } else {
+        // head in another type (e.g. Q6_K): norm + weight + Q8_0 through the operator kernels
+        spy_hip_tensor tx, tw, txn;
+        memset(&tx, 0, sizeof(tx));
+        tx.type = SPY_HIP_F32; tx.dim = 1; tx.ne[0] = d; tx.ne[1] = tx.ne[2] = tx.ne[3] = 1; tx.nb[0] = 4; tx.nb[1] = tx.nb[2] = tx.nb[3] = 4 * d;
+        tw = tx; txn = tx;
+        tx.data = m->x; tw.data = (void *)c.out_norm; txn.data = m->x1;
+        RC_TRY(spy_hip_op_norm_rms(st, &tx, &txn, c.eps));
+        RC_TRY(spy_hip_op_binary(st, 2, &txn, &tw, &txn));
+        RC_TRY(spy_hip_quantize_q8_0(st, m->x1, 4 * d, m->xq_head, 1, d));
+        RC_TRY(spy_hip_gemv_q8_0act(st, c.t_out, c.w_out, m->xq_head, m->logits, nullptr, c.n_vocab, d, 1, c.n_vocab));
+    }
+    if (sample) {
+        sample_advance_kernel<<<dim3(1), dim3(1024), 0, st>>>(m->st, m->logits, c.n_vocab, m->tokens_out, m->max_out);
+        RC_TRY(SPY_LAUNCH_RC());
+    }
+    return 0;
+}
+
+static int enqueue_pass_any(spy_hip_llama *m, hipStream_t st, bool sample) {
+    return m->desc.wtype == SPY_HIP_Q4_0 ? enqueue_pass<SPY_HIP_Q4_0>(m, st, sample) : enqueue_pass<SPY_HIP_Q8_0>(m, st, sample);
+}
+
+// ---- passes over several tokens: operator by operator --------------------------------------------
+static spy_hip_tensor T2(int type, void *p, int64_t e0, int64_t e1) {
+    spy_hip_tensor t;
+    t.type = type; t.dim = 2; t.data = p;
+    t.ne[0] = e0; t.ne[1] = e1; t.ne[2] = 1; t.ne[3] = 1;
+    t.nb[0] = spy_type_size(type); t.nb[1] = spy_row_size(type, e0); t.nb[2] = t.nb[1] * e1; t.nb[3] = t.nb[2];
+    return t;
+}
+static spy_hip_tensor T3s(int type, void *p, int64_t e0, int64_t e1, int64_t e2, int64_t b0, int64_t b1, int64_t b2) {
+    spy_hip_tensor t;
+    t.type = type; t.dim = 3; t.data = p;
+    t.ne[0] = e0; t.ne[1] = e1; t.ne[2] = e2; t.ne[3] = 1;
+    t.nb[0] = b0; t.nb[1] = b1; t.nb[2] = b2; t.nb[3] = e2 * b2;
+    return t;
+}
+
+static int forward_ops(spy_hip_llama *m, hipStream_t st, const int32_t *tokens_host, int T, int P, float *logits_host) {
+    const spy_hip_llama_desc &c = m->desc;
+    const int64_t d = c.n_embd, F = c.n_ff, C = c.n_ctx, H = c.n_head, hd = m->hd, V = c.n_vocab, n_kv = (int64_t)P + T;
+    // scratch layout (bytes)
+    size_t off = 0;
+    auto take = [&](size_t bytes) { size_t o = off; off += (bytes + 255) & ~(size_t)255; return o; };
+    const size_t o_x = take(d * T * 4), o_xn = take(d * T * 4), o_q = take(d * T * 4), o_k = take(d * T * 4), o_v = take(d * T * 4),
+                 o_o = take(d * T * 4), o_o2 = take(d * T * 4), o_t1 = take(d * T * 4), o_up = take(F * T * 4), o_gate = take(F * T * 4),
+                 o_par = take(F * T * 4), o_S = take(n_kv * T * H * 4), o_P = take(n_kv * T * H * 4), o_mask = take(C * T * 4),
+                 o_ids = take(T * 4), o_pos = take(T * 4), o_logits = take(V * T * 4);
+    const size_t act_q8 = (size_t)T * ((F > d ? F : d) / 32) * 34;
+    const size_t act_f16 = (size_t)n_kv * T * H * 2 > (size_t)d * T * 2 ? (size_t)n_kv * T * H * 2 : (size_t)d * T * 2;
+    const size_t o_scr = take(act_q8 > act_f16 ? act_q8 : act_f16);
+    const size_t scr_bytes = off - o_scr;
+    if (off > m->ops_bytes) {
+        if (m->ops_buf) { HIP_TRY(hipStreamSynchronize(st)); HIP_TRY(hipFree(m->ops_buf)); m->ops_buf = nullptr; m->ops_bytes = 0; }
+        HIP_TRY(hipMalloc((void **)&m->ops_buf, off));
+        m->ops_bytes = off;
+    }
+    uint8_t *B = m->ops_buf;
+    float *x = (float *)(B + o_x), *xn = (float *)(B + o_xn), *q = (float *)(B + o_q), *k = (float *)(B + o_k), *v = (float *)(B + o_v),
+          *o = (float *)(B + o_o), *o2 = (float *)(B + o_o2), *t1 = (float *)(B + o_t1), *up = (float *)(B + o_up), *gate = (float *)(B + o_gate),
+          *par = (float *)(B + o_par), *S = (float *)(B + o_S), *Pm = (float *)(B + o_P), *mask = (float *)(B + o_mask), *lg = (float *)(B + o_logits);
+    int32_t *ids = (int32_t *)(B + o_ids), *pos = (int32_t *)(B + o_pos);
+    void *scr = B + o_scr;
+
+    // IO tensors: ids, positions, KQ mask (llama.cpp:248-263)
+    {
+        std::vector<int32_t> hp(T);
+        for (int i = 0; i < T; i++) hp[i] = P + i;
+        std::vector<float> hm((size_t)C * T);
+        for (int64_t i = 0; i < T; i++) for (int64_t j = 0; j < C; j++) hm[C * i + j] = (j <= i + P) ? 0.0f : -INFINITY;
+        HIP_TRY(hipMemcpyAsync(ids, tokens_host, (size_t)T * 4, hipMemcpyHostToDevice, st));
+        HIP_TRY(hipMemcpyAsync(pos, hp.data(), (size_t)T * 4, hipMemcpyHostToDevice, st));
+        HIP_TRY(hipMemcpyAsync(mask, hm.data(), (size_t)C * T * 4, hipMemcpyHostToDevice, st));
+        HIP_TRY(hipStreamSynchronize(st));
+    }
+    spy_hip_tensor t_ids = T2(SPY_HIP_I32, ids, T, 1), t_pos = t_ids, t_mask = T2(SPY_HIP_I32, mask, C, T);
+    t_ids.dim = 1; t_pos.dim = 1; t_pos.data = pos;
+    spy_hip_tensor t_x = T2(SPY_HIP_F32, x, d, T), t_xn = T2(SPY_HIP_F32, xn, d, T), t_q = T2(SPY_HIP_F32, q, d, T), t_k = T2(SPY_HIP_F32, k, d, T),
+                   t_v = T2(SPY_HIP_F32, v, d, T), t_o2 = T2(SPY_HIP_F32, o2, d, T), t_t1 = T2(SPY_HIP_F32, t1, d, T), t_od = T2(SPY_HIP_F32, o, d, T);
+    spy_hip_tensor t_up = T2(SPY_HIP_F32, up, F, T), t_gate = T2(SPY_HIP_F32, gate, F, T), t_par = T2(SPY_HIP_F32, par, F, T);
+    { spy_hip_tensor te = T2(c.t_tok_embd, (void *)c.tok_embd, d, V); RC_TRY(spy_hip_op_get_row(st, &te, &t_ids, &t_x)); }
+    spy_hip_rope_param rp;
+    memset(&rp, 0, sizeof(rp));
+    rp.mode = 0; rp.num_past = P; rp.num_dim = (int32_t)hd; rp.num_context = (int32_t)C; rp.num_origin_context = (int32_t)C;
+    rp.freq_base = c.rope_freq_base; rp.freq_scale = 1.0f; rp.attention_factor = 1.0f; rp.beta_fast = 32.0f; rp.beta_slow = 1.0f;
+    const float scale = 1.0f / sqrtf((float)hd);
+    auto mm = [&](const void *w, int wt, int64_t K, int64_t M, spy_hip_tensor *xin, spy_hip_tensor *out) {
+        spy_hip_tensor tw = T2(wt, (void *)w, K, M);
+        return spy_hip_op_matmul(st, &tw, xin, out, scr, scr_bytes);
+    };
+    for (int il = 0; il < c.n_layer; il++) {
+        const spy_hip_llama_layer &L = m->layers[il];
+        spy_hip_tensor t_nw = T2(SPY_HIP_F32, (void *)L.attn_norm, d, 1); t_nw.dim = 1;
+        RC_TRY(spy_hip_op_norm_rms(st, &t_x, &t_xn, c.eps));
+        RC_TRY(spy_hip_op_binary(st, 2, &t_xn, &t_nw, &t_xn));
+        RC_TRY(mm(L.wq, c.wtype, d, d, &t_xn, &t_q));
+        RC_TRY(mm(L.wk, c.wtype, d, d, &t_xn, &t_k));
+        RC_TRY(mm(L.wv, c.wtype, d, d, &t_xn, &t_v));
+        spy_hip_tensor t_q3 = T3s(SPY_HIP_F32, q, hd, H, T, 4, 4 * hd, 4 * d), t_k3 = T3s(SPY_HIP_F32, k, hd, H, T, 4, 4 * hd, 4 * d);
+        RC_TRY(spy_hip_op_rope(st, &t_q3, &t_pos, &t_q3, &rp));
+        RC_TRY(spy_hip_op_rope(st, &t_k3, &t_pos, &t_k3, &rp));
+        spy_hip_tensor t_qp = T3s(SPY_HIP_F32, q, hd, T, H, 4, 4 * d, 4 * hd);                         // Permute {0,2,1,3}
+        spy_hip_tensor t_vt = T2(SPY_HIP_F32, v, T, d); t_vt.nb[0] = 4 * d; t_vt.nb[1] = 4; t_vt.nb[2] = t_vt.nb[3] = 4 * d * T;   // Transpose
+        spy_hip_tensor t_kc = T2(SPY_HIP_F16, (uint8_t *)m->k_cache[il] + 2 * d * P, (int64_t)T * d, 1); t_kc.dim = 1;
+        RC_TRY(spy_hip_op_dup(st, &t_k3, &t_kc));
+        spy_hip_tensor t_vc = T2(SPY_HIP_F16, (uint8_t *)m->v_cache[il] + 2 * (int64_t)P, T, d);
+        t_vc.nb[0] = 2; t_vc.nb[1] = 2 * C; t_vc.nb[2] = t_vc.nb[3] = d * 2 * C;
+        RC_TRY(spy_hip_op_dup(st, &t_vt, &t_vc));
+        spy_hip_tensor t_kall = T3s(SPY_HIP_F16, m->k_cache[il], hd, n_kv, H, 2, 2 * d, 2 * hd);
+        spy_hip_tensor t_vall = T3s(SPY_HIP_F16, m->v_cache[il], n_kv, hd, H, 2, 2 * C, 2 * C * hd);
+        spy_hip_tensor t_S = T3s(SPY_HIP_F32, S, n_kv, T, H, 4, 4 * n_kv, 4 * n_kv * T), t_P = T3s(SPY_HIP_F32, Pm, n_kv, T, H, 4, 4 * n_kv, 4 * n_kv * T);
+        RC_TRY(spy_hip_op_matmul(st, &t_kall, &t_qp, &t_S, scr, scr_bytes));
+        RC_TRY(spy_hip_op_softmax(st, &t_S, &t_mask, &t_P, scale));
+        spy_hip_tensor t_O = T3s(SPY_HIP_F32, o, hd, T, H, 4, 4 * hd, 4 * hd * T);
+        RC_TRY(spy_hip_op_matmul(st, &t_vall, &t_P, &t_O, scr, scr_bytes));
+        spy_hip_tensor t_Op = T3s(SPY_HIP_F32, o, hd, H, T, 4, 4 * hd * T, 4 * hd);                    // Permute {0,2,1,3}
+        spy_hip_tensor t_o2c = T3s(SPY_HIP_F32, o2, hd, H, T, 4, 4 * hd, 4 * d);
+        RC_TRY(spy_hip_op_contiguous(st, &t_Op, &t_o2c));
+        RC_TRY(mm(L.wo, c.wtype, d, d, &t_o2, &t_t1));
+        RC_TRY(spy_hip_op_binary(st, 0, &t_t1, &t_x, &t_t1));
+        t_nw.data = (void *)L.ffn_norm;
+        RC_TRY(spy_hip_op_norm_rms(st, &t_t1, &t_xn, c.eps));
+        RC_TRY(spy_hip_op_binary(st, 2, &t_xn, &t_nw, &t_xn));
+        RC_TRY(mm(L.w_up, c.wtype, d, F, &t_xn, &t_up));
+        RC_TRY(mm(L.w_gate, c.wtype, d, F, &t_xn, &t_gate));
+        RC_TRY(spy_hip_op_silu(st, &t_gate, &t_gate));
+        RC_TRY(spy_hip_op_binary(st, 2, &t_up, &t_gate, &t_par));
+        RC_TRY(mm(L.w_down, c.wtype, F, d, &t_par, &t_od));
+        RC_TRY(spy_hip_op_binary(st, 0, &t_t1, &t_od, &t_x));
+    }
+    {
+        spy_hip_tensor t_nw = T2(SPY_HIP_F32, (void *)c.out_norm, d, 1); t_nw.dim = 1;
+        RC_TRY(spy_hip_op_norm_rms(st, &t_x, &t_xn, c.eps));
+        RC_TRY(spy_hip_op_binary(st, 2, &t_xn, &t_nw, &t_xn));
+        spy_hip_tensor t_l = T2(SPY_HIP_F32, lg, V, T);
+        RC_TRY(mm(c.w_out, c.t_out, d, V, &t_xn, &t_l));
+    }
+    if (logits_host) HIP_TRY(hipMemcpyAsync(logits_host, lg, (size_t)V * T * 4, hipMemcpyDeviceToHost, st));
+    HIP_TRY(hipStreamSynchronize(st));
+    return 0;
+}
+
+extern "C" int spy_hip_llama_forward(spy_hip_llama *m, void *stream, const int32_t *tokens_host, int32_t n_token, int32_t n_past,
+                                     float *logits_host) {
+    SPY_CHECK_ARG(m && tokens_host && n_token > 0 && n_past >= 0);
+    SPY_CHECK_ARG((int64_t)n_past + n_token <= m->desc.n_ctx);                  // llama.cpp:249
+    hipStream_t st = stream ? (hipStream_t)stream : m->own_stream;
+    for (int i = 0; i < n_token; i++) SPY_CHECK_ARG(tokens_host[i] >= 0 && tokens_host[i] < m->desc.n_vocab);   // view.cpp:61
+    if (n_token == 1 && fused_ok(m) && !getenv("SPY_HIP_FORCE_OPS")) {
+        dev_state h = {tokens_host[0], n_past, 0, 0};
+        HIP_TRY(hipMemcpyAsync(m->st, &h, sizeof(h), hipMemcpyHostToDevice, st));
+        RC_TRY(enqueue_pass_any(m, st, false));
+        if (logits_host) HIP_TRY(hipMemcpyAsync(logits_host, m->logits, (size_t)m->desc.n_vocab * 4, hipMemcpyDeviceToHost, st));
+        HIP_TRY(hipStreamSynchronize(st));
+        return 0;
+    }
+    // longer passes in chunks: each chunk attends to everything before it, so the result per token
+    // is that of one pass over the whole prompt
+    const int CH = 256;
+    for (int t0 = 0; t0 < n_token; t0 += CH) {
+        const int tc = n_token - t0 < CH ? n_token - t0 : CH;
+        RC_TRY(forward_ops(m, st, tokens_host + t0, tc, n_past + t0, logits_host ? logits_host + (size_t)t0 * m->desc.n_vocab : nullptr));
+    }
+    return 0;
+}
+
+extern "C" int spy_hip_llama_decode_greedy(spy_hip_llama *m, void *stream, int32_t first_token, int32_t n_past, int32_t n_steps,
+                                           int32_t *tokens_host, int32_t use_graph) {
+    SPY_CHECK_ARG(m && n_steps > 0 && n_past >= 0 && first_token >= 0 && first_token < m->desc.n_vocab);
+    SPY_CHECK_ARG((int64_t)n_past + n_steps <= m->desc.n_ctx && n_steps <= m->max_out);
+    if (!fused_ok(m)) return SPY_HIP_EUNSUPPORTED;
+    hipStream_t st = stream ? (hipStream_t)stream : m->own_stream;
+    dev_state h = {first_token, n_past, 0, 0};
+    HIP_TRY(hipMemcpyAsync(m->st, &h, sizeof(h), hipMemcpyHostToDevice, st));
+    HIP_TRY(hipStreamSynchronize(st));
+    if (use_graph && (!m->graph_exec || m->graph_stream != st)) {
+        if (m->graph_exec) { (void)hipGraphExecDestroy(m->graph_exec); m->graph_exec = nullptr; }
+        if (m->graph) { (void)hipGraphDestroy(m->graph); m->graph = nullptr; }
+        HIP_TRY(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
+        const int rc = enqueue_pass_any(m, st, true);
+        hipError_t e = hipStreamEndCapture(st, &m->graph);
+        if (rc) return rc;
+        if (e != hipSuccess) return (int)e;
+        HIP_TRY(hipGraphInstantiate(&m->graph_exec, m->graph, nullptr, nullptr, 0));
+        m->graph_stream = st;
+    }
+    HIP_TRY(hipEventRecord(m->ev0, st));
+    for (int i = 0; i < n_steps; i++) {
+        if (use_graph) HIP_TRY(hipGraphLaunch(m->graph_exec, st));
+        else RC_TRY(enqueue_pass_any(m, st, true));
+    }
+    HIP_TRY(hipEventRecord(m->ev1, st));
+    HIP_TRY(hipEventSynchronize(m->ev1));
+    float ms = 0.0f;
+    HIP_TRY(hipEventElapsedTime(&ms, m->ev0, m->ev1));
+    m->timed_ms += ms; m->timed_pass += n_steps;
+    dev_state back;
+    HIP_TRY(hipMemcpy(&back, m->st, sizeof(back), hipMemcpyDeviceToHost));
+    if (back.err) return SPY_HIP_EINVAL;
+    if (tokens_host) HIP_TRY(hipMemcpy(tokens_host, m->tokens_out, (size_t)n_steps * 4, hipMemcpyDeviceToHost));
+    return 0;
+}

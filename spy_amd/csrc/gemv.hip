@@ -3,160 +3,72 @@
 // (backend/host/include/simd/vec_dot.h:42-115, backend/host/operator/mat.cpp:130-143 in the Spy
 // tree) and adds Q4_K / Q6_K weights, which the reference only declares.
 //
-// HBM-bound: each weight byte is read once.  Weights stay in their native GGUF block layout
-// (18-byte Q4_0 / 34-byte Q8_0 blocks, 2-byte aligned), so a workgroup streams a contiguous
-// span of whole rows with 128-bit coalesced loads into LDS and the lanes then pick their
-// 4-byte-aligned block PAIRS (36 / 68 bytes, an odd number of dwords -> conflict-free LDS
-// reads) out of LDS.  Activations are staged once per workgroup as aligned int8 plus
-// {scale, sum(q)} per block; sum(q) turns sum((n-8)*q) into sum(n*q) - 8*sum(q), so the nibbles
-// feed v_dot4_i32_i8 without a per-byte subtract.  The int32 block dot is exact; only the
-// fp32 accumulation order differs from the reference's 8-lane AVX accumulators.
-#include "common.cuh"
+// HBM-bound: each weight byte is read once, straight from the native GGUF block layout.  The
+// int32 block dot is exact; only the fp32 accumulation order differs from the reference's 8-lane
+// AVX accumulators.  See gemv_core.cuh for the work split.
+#include "gemv_core.cuh"
 
-#define GEMV_THREADS 256
-#define GEMV_WAVES 4
-#define GEMV_MAX_ROUNDS 12                 // 128-bit loads per thread per tile (<= 48 KiB tile)
-#define GEMV_TILE_TARGET 28672
+struct gemv_args {
+    const uint8_t *W;        // M rows of K elements, native blocks, contiguous
+    const uint8_t *xq;       // NT rows of native Q8_0 blocks, contiguous
+    float *dst;              // dst[c*dst_stride + m]
+    const float *residual;   // optional, same indexing as dst
+    int32_t *dump;           // optional: int32 block dots of column 0, [M][K/32]
+    int M, K;
+    int64_t dst_stride;
+};
 
-template <int WT> struct wt_traits;
-template <> struct wt_traits<SPY_HIP_Q4_0> { static constexpr int BLK = 18; };
-template <> struct wt_traits<SPY_HIP_Q8_0> { static constexpr int BLK = 34; };
-
-// Stage T rows of native Q8_0 activations into LDS: qs -> s_q[(t*nblk+b)*32 ..], and
-// s_meta[t*nblk+b] = {bits(float scale), sum of the 32 quants}.
-static __device__ __forceinline__ void stage_activations(const uint8_t *__restrict__ xq, int8_t *s_q, int2 *s_meta, int total_blk) {
-    const uint16_t *src = (const uint16_t *)xq;
-    const int total_h = total_blk * 17;
-    for (int h = threadIdx.x; h < total_h; h += GEMV_THREADS) {
-        const int b = h / 17, w = h - b * 17;
-        const uint16_t v = src[h];
-        if (w == 0) s_meta[b].x = __float_as_int(h2f(v));
-        else ((uint16_t *)s_q)[b * 16 + (w - 1)] = v;
-    }
-    __syncthreads();
-    for (int b = threadIdx.x; b < total_blk; b += GEMV_THREADS) {
-        const int4 *q = (const int4 *)(s_q + b * 32);
-        const int4 q0 = q[0], q1 = q[1];
-        int s = 0;
-        s = __builtin_amdgcn_sdot4(q0.x, 0x01010101, s, false); s = __builtin_amdgcn_sdot4(q0.y, 0x01010101, s, false);
-        s = __builtin_amdgcn_sdot4(q0.z, 0x01010101, s, false); s = __builtin_amdgcn_sdot4(q0.w, 0x01010101, s, false);
-        s = __builtin_amdgcn_sdot4(q1.x, 0x01010101, s, false); s = __builtin_amdgcn_sdot4(q1.y, 0x01010101, s, false);
-        s = __builtin_amdgcn_sdot4(q1.z, 0x01010101, s, false); s = __builtin_amdgcn_sdot4(q1.w, 0x01010101, s, false);
-        s_meta[b].y = s;
-    }
-}
-
-// int32 dot of one Q4_0 block (4 dwords of packed nibbles) with 32 int8 activations
-static __device__ __forceinline__ int dot_q4_block(const uint32_t n[4], const int4 x0, const int4 x1, int sumq) {
-    const int xl[4] = {x0.x, x0.y, x0.z, x0.w}, xh[4] = {x1.x, x1.y, x1.z, x1.w};
-    int s = 0;
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        s = __builtin_amdgcn_sdot4((int)(n[i] & 0x0F0F0F0Fu), xl[i], s, false);          // elements 4i..4i+3
-        s = __builtin_amdgcn_sdot4((int)((n[i] >> 4) & 0x0F0F0F0Fu), xh[i], s, false);   // elements 16+4i..
-    }
-    return s - 8 * sumq;
-}
-
-static __device__ __forceinline__ int dot_q8_block(const uint32_t n[8], const int4 x0, const int4 x1) {
-    int s = 0;
-    s = __builtin_amdgcn_sdot4((int)n[0], x0.x, s, false); s = __builtin_amdgcn_sdot4((int)n[1], x0.y, s, false);
-    s = __builtin_amdgcn_sdot4((int)n[2], x0.z, s, false); s = __builtin_amdgcn_sdot4((int)n[3], x0.w, s, false);
-    s = __builtin_amdgcn_sdot4((int)n[4], x1.x, s, false); s = __builtin_amdgcn_sdot4((int)n[5], x1.y, s, false);
-    s = __builtin_amdgcn_sdot4((int)n[6], x1.z, s, false); s = __builtin_amdgcn_sdot4((int)n[7], x1.w, s, false);
-    return s;
-}
-
-// grid.x = number of row tiles; R rows per tile; requires K % 256 == 0 (rows 16-byte aligned,
-// even block count).  LDS: [tile R*RB][s_q T*K][s_meta T*nblk*8].
-template <int WT, int NT, bool DUMP>
-__global__ __launch_bounds__(GEMV_THREADS) void gemv_tile_kernel(const uint8_t *__restrict__ W, const uint8_t *__restrict__ xq,
-                                                                 float *__restrict__ dst, const float *__restrict__ residual,
-                                                                 int32_t *__restrict__ dump, int M, int K, int R, int64_t dst_stride) {
+// Persistent workgroups: each strides over row tiles with the next tile's weights already in
+// flight (two register buffers) while the current one is reduced.
+template <int WT, int LPR, int NT, bool DUMP>
+__global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(gemv_args a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    constexpr int BLK = wt_traits<WT>::BLK;
-    const int nblk = K / 32, npair = nblk / 2;
-    const int RB = nblk * BLK;
-    const int r0 = blockIdx.x * R;
-    const int nrow = min(R, M - r0);
-    const int tile_bytes = nrow * RB;
-    uint8_t *s_tile = smem;
-    int8_t *s_q = (int8_t *)(smem + (((size_t)R * RB + 15) & ~(size_t)15));
-    int2 *s_meta = (int2 *)(s_q + (size_t)NT * K);
+    constexpr int RPW = SPY_WAVE / LPR, RPT = GEMV_WAVES * RPW;
+    const int K = a.K, nblk = K / 32, npair = K / 64, nit = (npair + LPR - 1) / LPR;
+    const size_t RB = (size_t)nblk * wt_traits<WT>::BLK;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l = lane % LPR, g = lane / LPR;
+    const int ntiles = (a.M + RPT - 1) / RPT, G = gridDim.x;
+    const int rofs = wave * RPW + g;
 
-    // 1. put the whole weight tile in flight (registers), 2. stage activations, 3. tile -> LDS
-    const uint8_t *src = W + (size_t)r0 * RB;
-    uint4 regs[GEMV_MAX_ROUNDS];
-#pragma unroll
-    for (int i = 0; i < GEMV_MAX_ROUNDS; i++) {
-        const int off = (i * GEMV_THREADS + threadIdx.x) * 16;
-        if (off < tile_bytes) regs[i] = *(const uint4 *)(src + off);
-    }
-    stage_activations(xq, s_q, s_meta, NT * nblk);
-#pragma unroll
-    for (int i = 0; i < GEMV_MAX_ROUNDS; i++) {
-        const int off = (i * GEMV_THREADS + threadIdx.x) * 16;
-        if (off < tile_bytes) *(uint4 *)(s_tile + off) = regs[i];
-    }
-    __syncthreads();
+    wtile<WT> A, B;
+    int tile = blockIdx.x;
+    if (tile < ntiles && tile * RPT + rofs < a.M) load_tile<WT, LPR>(A, a.W + (size_t)(tile * RPT + rofs) * RB, npair, nit, l);
 
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    for (int r = wave; r < nrow; r += GEMV_WAVES) {
-        const uint32_t *rowp = (const uint32_t *)(s_tile + (size_t)r * RB);
+    staged_act act[NT];
+#pragma unroll
+    for (int c = 0; c < NT; c++) {
+        int8_t *q = (int8_t *)(smem + (size_t)c * staged_bytes(K));
+        int2 *meta = (int2 *)(q + K);
+        stage_native_q8(a.xq + (size_t)c * nblk * 34, q, meta, nblk);
+        act[c].q = q; act[c].meta = meta;
+    }
+
+    auto finish = [&](const wtile<WT> &t, int tl) {
+        const int r = tl * RPT + rofs;
         float acc[NT];
 #pragma unroll
-        for (int t = 0; t < NT; t++) acc[t] = 0.0f;
-        for (int p = lane; p < npair; p += SPY_WAVE) {
-            if constexpr (WT == SPY_HIP_Q4_0) {
-                const uint32_t *wp = rowp + p * 9;
-                uint32_t w[9];
+        for (int c = 0; c < NT; c++) acc[c] = 0.0f;
+        if (r < a.M) dot_tile<WT, LPR, NT>(t, act, npair, nit, l, acc, DUMP ? a.dump + (size_t)r * nblk : nullptr);
 #pragma unroll
-                for (int i = 0; i < 9; i++) w[i] = wp[i];
-                const float dA = h2f((uint16_t)(w[0] & 0xFFFFu)), dB = h2f((uint16_t)(w[4] >> 16));
-                uint32_t a[4];
-#pragma unroll
-                for (int i = 0; i < 4; i++) a[i] = __builtin_amdgcn_alignbit(w[i + 1], w[i], 16);
-#pragma unroll
-                for (int t = 0; t < NT; t++) {
-                    const int bA = t * nblk + 2 * p;
-                    const int4 *xa = (const int4 *)(s_q + (size_t)bA * 32);
-                    const int2 mA = s_meta[bA], mB = s_meta[bA + 1];
-                    const int iA = dot_q4_block(a, xa[0], xa[1], mA.y);
-                    const int iB = dot_q4_block(&w[5], xa[2], xa[3], mB.y);
-                    if constexpr (DUMP) { dump[(size_t)(r0 + r) * nblk + 2 * p] = iA; dump[(size_t)(r0 + r) * nblk + 2 * p + 1] = iB; }
-                    acc[t] = fmaf(dA * __int_as_float(mA.x), (float)iA, acc[t]);
-                    acc[t] = fmaf(dB * __int_as_float(mB.x), (float)iB, acc[t]);
-                }
-            } else {
-                const uint32_t *wp = rowp + p * 17;
-                uint32_t w[17];
-#pragma unroll
-                for (int i = 0; i < 17; i++) w[i] = wp[i];
-                const float dA = h2f((uint16_t)(w[0] & 0xFFFFu)), dB = h2f((uint16_t)(w[8] >> 16));
-                uint32_t a[8];
-#pragma unroll
-                for (int i = 0; i < 8; i++) a[i] = __builtin_amdgcn_alignbit(w[i + 1], w[i], 16);
-#pragma unroll
-                for (int t = 0; t < NT; t++) {
-                    const int bA = t * nblk + 2 * p;
-                    const int4 *xa = (const int4 *)(s_q + (size_t)bA * 32);
-                    const int2 mA = s_meta[bA], mB = s_meta[bA + 1];
-                    const int iA = dot_q8_block(a, xa[0], xa[1]);
-                    const int iB = dot_q8_block(&w[9], xa[2], xa[3]);
-                    if constexpr (DUMP) { dump[(size_t)(r0 + r) * nblk + 2 * p] = iA; dump[(size_t)(r0 + r) * nblk + 2 * p + 1] = iB; }
-                    acc[t] = fmaf(dA * __int_as_float(mA.x), (float)iA, acc[t]);
-                    acc[t] = fmaf(dB * __int_as_float(mB.x), (float)iB, acc[t]);
-                }
+        for (int c = 0; c < NT; c++) {
+            const float s = group_sum<LPR>(acc[c]);
+            if (l == 0 && r < a.M) {
+                const size_t o = (size_t)c * a.dst_stride + r;
+                a.dst[o] = a.residual ? s + a.residual[o] : s;
             }
         }
-#pragma unroll
-        for (int t = 0; t < NT; t++) {
-            const float s = wave_sum(acc[t]);
-            if (lane == 0) {
-                const size_t o = (size_t)t * dst_stride + (r0 + r);
-                dst[o] = residual ? s + residual[o] : s;
-            }
-        }
+    };
+
+    while (tile < ntiles) {
+        int tn = tile + G;
+        if (tn < ntiles && tn * RPT + rofs < a.M) load_tile<WT, LPR>(B, a.W + (size_t)(tn * RPT + rofs) * RB, npair, nit, l);
+        finish(A, tile);
+        tile = tn;
+        if (tile >= ntiles) break;
+        tn = tile + G;
+        if (tn < ntiles && tn * RPT + rofs < a.M) load_tile<WT, LPR>(A, a.W + (size_t)(tn * RPT + rofs) * RB, npair, nit, l);
+        finish(B, tile);
+        tile = tn;
     }
 }
 
@@ -232,29 +144,42 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_generic_kernel(const uint8_
     }
 }
 
-static int tile_rows(int wtype, int64_t K) {
-    const int64_t RB = spy_row_size(wtype, K);
-    int64_t g = GEMV_TILE_TARGET / (GEMV_WAVES * RB);
-    if (g < 1) g = 1;
-    return (int)(GEMV_WAVES * g);
+
+static int g_num_cu = 0;
+static int num_cu() {
+    if (!g_num_cu) {
+        int dev = 0; hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) g_num_cu = prop.multiProcessorCount;
+        if (g_num_cu <= 0) g_num_cu = 256;
+    }
+    return g_num_cu;
 }
 
-template <int WT, int NT, bool DUMP>
-static int launch_tile(hipStream_t st, const void *w, const void *xq, float *dst, const float *residual, int32_t *dump,
-                       int64_t M, int64_t K, int64_t dst_stride) {
-    const int R = tile_rows(WT, K);
-    const int64_t RB = spy_row_size(WT, K);
-    if (R * RB > (int64_t)GEMV_MAX_ROUNDS * GEMV_THREADS * 16) return SPY_HIP_EUNSUPPORTED;
-    const size_t lds = (((size_t)R * RB + 15) & ~(size_t)15) + (size_t)NT * K + (size_t)NT * (K / 32) * 8;
+template <int WT, int LPR, int NT, bool DUMP>
+static int launch_fast(hipStream_t st, const gemv_args &a) {
+    constexpr int RPT = GEMV_WAVES * (SPY_WAVE / LPR);
+    const size_t lds = (size_t)NT * staged_bytes(a.K);
     if (lds > 160 * 1024) return SPY_HIP_EUNSUPPORTED;
-    auto kern = gemv_tile_kernel<WT, NT, DUMP>;
+    auto kern = gemv_kernel<WT, LPR, NT, DUMP>;
     if (lds > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return (int)e;
     }
-    const unsigned grid = (unsigned)((M + R - 1) / R);
-    kern<<<dim3(grid), dim3(GEMV_THREADS), lds, st>>>((const uint8_t *)w, (const uint8_t *)xq, dst, residual, dump, (int)M, (int)K, R, dst_stride);
+    const int ntiles = (a.M + RPT - 1) / RPT;
+    const int cap = 4 * num_cu();
+    const unsigned grid = (unsigned)(ntiles < cap ? ntiles : cap);
+    kern<<<dim3(grid), dim3(GEMV_THREADS), lds, st>>>(a);
     return SPY_LAUNCH_RC();
+}
+
+template <int WT, int NT, bool DUMP>
+static int launch_fast_lpr(hipStream_t st, const gemv_args &a) {
+    switch (pick_lpr<WT>(a.K)) {
+    case 16: return launch_fast<WT, 16, NT, DUMP>(st, a);
+    case 32: return launch_fast<WT, 32, NT, DUMP>(st, a);
+    case 64: return launch_fast<WT, 64, NT, DUMP>(st, a);
+    }
+    return SPY_HIP_EUNSUPPORTED;
 }
 
 template <int WT, bool DUMP>
@@ -267,21 +192,22 @@ static int launch_generic(hipStream_t st, const void *w, const void *xq, float *
 }
 
 template <int WT>
-static int gemv_tiled_cols(hipStream_t st, const void *w, const uint8_t *xq, float *dst, const float *residual,
-                           int64_t M, int64_t K, int64_t T, int64_t dst_stride) {
+static int gemv_fast_cols(hipStream_t st, const void *w, const uint8_t *xq, float *dst, const float *residual,
+                          int64_t M, int64_t K, int64_t T, int64_t dst_stride) {
     // weights are re-read once per group of up to 8 activation rows
     const int64_t xrow = (K / 32) * 34;
     int64_t t = 0;
     while (t < T) {
         const int64_t left = T - t;
+        gemv_args a;
+        a.W = (const uint8_t *)w; a.xq = xq + t * xrow; a.dst = dst + t * dst_stride;
+        a.residual = residual ? residual + t * dst_stride : nullptr; a.dump = nullptr;
+        a.M = (int)M; a.K = (int)K; a.dst_stride = dst_stride;
         int rc;
-        const float *res = residual ? residual + t * dst_stride : nullptr;
-        float *d = dst + t * dst_stride;
-        const uint8_t *x = xq + t * xrow;
-        if (left >= 8)      { rc = launch_tile<WT, 8, false>(st, w, x, d, res, nullptr, M, K, dst_stride); t += 8; }
-        else if (left >= 4) { rc = launch_tile<WT, 4, false>(st, w, x, d, res, nullptr, M, K, dst_stride); t += 4; }
-        else if (left >= 2) { rc = launch_tile<WT, 2, false>(st, w, x, d, res, nullptr, M, K, dst_stride); t += 2; }
-        else                { rc = launch_tile<WT, 1, false>(st, w, x, d, res, nullptr, M, K, dst_stride); t += 1; }
+        if (left >= 8)      { rc = launch_fast_lpr<WT, 8, false>(st, a); t += 8; }
+        else if (left >= 4) { rc = launch_fast_lpr<WT, 4, false>(st, a); t += 4; }
+        else if (left >= 2) { rc = launch_fast_lpr<WT, 2, false>(st, a); t += 2; }
+        else                { rc = launch_fast_lpr<WT, 1, false>(st, a); t += 1; }
         if (rc) return rc;
     }
     return 0;
@@ -290,7 +216,7 @@ static int gemv_tiled_cols(hipStream_t st, const void *w, const uint8_t *xq, flo
 static int check_gemv_args(int wtype, const void *w, const void *xq, const void *dst, int64_t M, int64_t K, int64_t T) {
     SPY_CHECK_ARG(w && xq && dst && M > 0 && K > 0 && T > 0);
     SPY_CHECK_ARG(M < (1ll << 30) && K < (1ll << 24) && T < (1ll << 24));
-    SPY_CHECK_ARG(((uintptr_t)w % 16) == 0 && ((uintptr_t)xq % 2) == 0 && ((uintptr_t)dst % 4) == 0);
+    SPY_CHECK_ARG(((uintptr_t)w % 4) == 0 && ((uintptr_t)xq % 2) == 0 && ((uintptr_t)dst % 4) == 0);
     switch (wtype) {
     case SPY_HIP_Q4_0: case SPY_HIP_Q8_0: SPY_CHECK_ARG(K % 32 == 0); break;
     case SPY_HIP_Q4_K: case SPY_HIP_Q6_K: SPY_CHECK_ARG(K % 256 == 0); break;
@@ -305,14 +231,13 @@ extern "C" int spy_hip_gemv_q8_0act(void *stream, int wtype, const void *w, cons
     if (rc) return rc;
     SPY_CHECK_ARG(dst_stride >= M);
     hipStream_t st = (hipStream_t)stream;
-    const bool tiled = (K % 256 == 0);
     switch (wtype) {
     case SPY_HIP_Q4_0:
-        return tiled ? gemv_tiled_cols<SPY_HIP_Q4_0>(st, w, (const uint8_t *)xq, dst, residual, M, K, T, dst_stride)
-                     : launch_generic<SPY_HIP_Q4_0, false>(st, w, xq, dst, residual, nullptr, M, K, T, dst_stride);
+        return pick_lpr<SPY_HIP_Q4_0>(K) ? gemv_fast_cols<SPY_HIP_Q4_0>(st, w, (const uint8_t *)xq, dst, residual, M, K, T, dst_stride)
+                                         : launch_generic<SPY_HIP_Q4_0, false>(st, w, xq, dst, residual, nullptr, M, K, T, dst_stride);
     case SPY_HIP_Q8_0:
-        return tiled ? gemv_tiled_cols<SPY_HIP_Q8_0>(st, w, (const uint8_t *)xq, dst, residual, M, K, T, dst_stride)
-                     : launch_generic<SPY_HIP_Q8_0, false>(st, w, xq, dst, residual, nullptr, M, K, T, dst_stride);
+        return pick_lpr<SPY_HIP_Q8_0>(K) ? gemv_fast_cols<SPY_HIP_Q8_0>(st, w, (const uint8_t *)xq, dst, residual, M, K, T, dst_stride)
+                                         : launch_generic<SPY_HIP_Q8_0, false>(st, w, xq, dst, residual, nullptr, M, K, T, dst_stride);
     case SPY_HIP_Q4_K: return launch_generic<SPY_HIP_Q4_K, false>(st, w, xq, dst, residual, nullptr, M, K, T, dst_stride);
     case SPY_HIP_Q6_K: return launch_generic<SPY_HIP_Q6_K, false>(st, w, xq, dst, residual, nullptr, M, K, T, dst_stride);
     }
@@ -328,14 +253,16 @@ extern "C" int spy_hip_block_dots(void *stream, int wtype, const void *w, const 
     // the float result goes to a throw-away slot behind the dump: out must hold M*nsub + M ints
     const int64_t nsub = (wtype == SPY_HIP_Q6_K) ? K / 16 : K / 32;
     float *sink = (float *)(out + M * nsub);
-    const bool tiled = (K % 256 == 0);
+    gemv_args a;
+    a.W = (const uint8_t *)w; a.xq = (const uint8_t *)xq; a.dst = sink; a.residual = nullptr; a.dump = out;
+    a.M = (int)M; a.K = (int)K; a.dst_stride = M;
     switch (wtype) {
     case SPY_HIP_Q4_0:
-        return tiled ? launch_tile<SPY_HIP_Q4_0, 1, true>(st, w, xq, sink, nullptr, out, M, K, M)
-                     : launch_generic<SPY_HIP_Q4_0, true>(st, w, xq, sink, nullptr, out, M, K, 1, M);
+        return pick_lpr<SPY_HIP_Q4_0>(K) ? launch_fast_lpr<SPY_HIP_Q4_0, 1, true>(st, a)
+                                         : launch_generic<SPY_HIP_Q4_0, true>(st, w, xq, sink, nullptr, out, M, K, 1, M);
     case SPY_HIP_Q8_0:
-        return tiled ? launch_tile<SPY_HIP_Q8_0, 1, true>(st, w, xq, sink, nullptr, out, M, K, M)
-                     : launch_generic<SPY_HIP_Q8_0, true>(st, w, xq, sink, nullptr, out, M, K, 1, M);
+        return pick_lpr<SPY_HIP_Q8_0>(K) ? launch_fast_lpr<SPY_HIP_Q8_0, 1, true>(st, a)
+                                         : launch_generic<SPY_HIP_Q8_0, true>(st, w, xq, sink, nullptr, out, M, K, 1, M);
     case SPY_HIP_Q4_K: return launch_generic<SPY_HIP_Q4_K, true>(st, w, xq, sink, nullptr, out, M, K, 1, M);
     case SPY_HIP_Q6_K: return launch_generic<SPY_HIP_Q6_K, true>(st, w, xq, sink, nullptr, out, M, K, 1, M);
     }

@@ -1,0 +1,227 @@
+// Device-side building blocks of the quantized matrix x vector kernels (Q4_0 / Q8_0 weights,
+// Q8_0 activations).  Shared by the stand-alone GEMV launchers and the fused token-loop kernels.
+//
+// Work split: LPR (16, 32 or 64) lanes share one weight row, a wave covers 64/LPR rows at once
+// and a 256-thread workgroup 4x that.  A lane owns block PAIRS p = it*LPR + l of its row (a pair
+// of native blocks is 36 / 68 bytes: 4-byte aligned, loaded straight from HBM as dwords, no LDS
+// staging of weights).  All of a tile's weight loads are issued before anything else so the HBM
+// latency overlaps the activation staging; the reduction over the LPR lanes runs on DPP.
+//
+// Activations live in LDS in a "staged" form: int8 q[K] (16-byte aligned) followed by one
+// {float scale, int32 sum(q)} per 32-element block; sum(q) folds the -8 offset of the Q4_0
+// nibbles: sum((n-8)*q) = sum(n*q) - 8*sum(q), keeping the int32 block dot exact.
+#pragma once
+
+#include "common.cuh"
+
+#define GEMV_THREADS 256
+#define GEMV_WAVES 4
+
+template <int WT> struct wt_traits;
+template <> struct wt_traits<SPY_HIP_Q4_0> { static constexpr int BLK = 18, PAIR_DW = 9, NIT_MAX = 6; };
+template <> struct wt_traits<SPY_HIP_Q8_0> { static constexpr int BLK = 34, PAIR_DW = 17, NIT_MAX = 4; };
+
+template <int CTRL> static __device__ __forceinline__ float dpp_add(float v) {
+    return v + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+template <int CTRL> static __device__ __forceinline__ float dpp_max(float v) {
+    return fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true)));
+}
+template <int CTRL> static __device__ __forceinline__ int dpp_add_i(int v) {
+    return v + __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true);
+}
+// Sum over each aligned group of LPR lanes; every lane of the group receives the total.
+template <int LPR> static __device__ __forceinline__ float group_sum(float v) {
+    v = dpp_add<0xB1>(v);    // quad_perm [1,0,3,2]
+    v = dpp_add<0x4E>(v);    // quad_perm [2,3,0,1]
+    v = dpp_add<0x141>(v);   // row_half_mirror
+    v = dpp_add<0x140>(v);   // row_mirror: all 16 lanes of a DPP row now hold the row total
+    if constexpr (LPR >= 32) v += __shfl_xor(v, 16, SPY_WAVE);
+    if constexpr (LPR >= 64) v += __shfl_xor(v, 32, SPY_WAVE);
+    return v;
+}
+// max / sum over aligned groups of 8 lanes (one Q8_0 block = 8 lanes x 4 floats)
+static __device__ __forceinline__ float oct_max(float v) {
+    v = dpp_max<0xB1>(v); v = dpp_max<0x4E>(v); v = dpp_max<0x141>(v);
+    return v;
+}
+static __device__ __forceinline__ int oct_sum_i(int v) {
+    v = dpp_add_i<0xB1>(v); v = dpp_add_i<0x4E>(v); v = dpp_add_i<0x141>(v);
+    return v;
+}
+
+struct staged_act {          // where one activation column lives in LDS
+    const int8_t *q;         // K bytes
+    const int2 *meta;        // K/32 x {bits(float scale), sum(q)}
+};
+static __host__ __device__ inline size_t staged_bytes(int64_t K) { return (size_t)K + (size_t)(K / 32) * 8; }
+
+// ---- activation staging --------------------------------------------------------------------
+
+// native Q8_0 blocks (34 bytes, 2-byte aligned) -> staged LDS form. Ends with __syncthreads().
+static __device__ __forceinline__ void stage_native_q8(const uint8_t *__restrict__ xq, int8_t *s_q, int2 *s_meta, int nblk) {
+    const uint16_t *src = (const uint16_t *)xq;
+    const int total_h = nblk * 17;
+    for (int h = threadIdx.x; h < total_h; h += GEMV_THREADS) {
+        const int b = h / 17, w = h - b * 17;
+        const uint16_t v = src[h];
+        if (w == 0) s_meta[b].x = __float_as_int(h2f(v));
+        else ((uint16_t *)s_q)[b * 16 + (w - 1)] = v;
+    }
+    __syncthreads();
+    for (int b = threadIdx.x; b < nblk; b += GEMV_THREADS) {
+        const int4 *q = (const int4 *)(s_q + b * 32);
+        const int4 q0 = q[0], q1 = q[1];
+        int s = 0;
+        s = __builtin_amdgcn_sdot4(q0.x, 0x01010101, s, false); s = __builtin_amdgcn_sdot4(q0.y, 0x01010101, s, false);
+        s = __builtin_amdgcn_sdot4(q0.z, 0x01010101, s, false); s = __builtin_amdgcn_sdot4(q0.w, 0x01010101, s, false);
+        s = __builtin_amdgcn_sdot4(q1.x, 0x01010101, s, false); s = __builtin_amdgcn_sdot4(q1.y, 0x01010101, s, false);
+        s = __builtin_amdgcn_sdot4(q1.z, 0x01010101, s, false); s = __builtin_amdgcn_sdot4(q1.w, 0x01010101, s, false);
+        s_meta[b].y = s;
+    }
+    __syncthreads();
+}
+
+// Quantize 4 consecutive floats held by each of 8 consecutive lanes (one 32-element block) the
+// way Quantizator<FP32,Q8_0>::transform does (vec_convert.h:197-260 in the Spy tree): amax,
+// d = amax/127 (stored as fp16), id = 127/amax, q = rint(x*id) saturated to int8.
+// Returns the 4 quants packed in a dword; lane 0 of the octet also gets {scale bits, sum q}.
+static __device__ __forceinline__ uint32_t quantize_oct(const float4 v, int2 &meta) {
+    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    amax = oct_max(amax);
+    const float d  = amax / 127.0f;
+    const float id = (amax != 0.0f) ? 127.0f / amax : 0.0f;
+    int q0 = (int)rintf(v.x * id), q1 = (int)rintf(v.y * id), q2 = (int)rintf(v.z * id), q3 = (int)rintf(v.w * id);
+    q0 = min(127, max(-128, q0)); q1 = min(127, max(-128, q1)); q2 = min(127, max(-128, q2)); q3 = min(127, max(-128, q3));
+    const int s = oct_sum_i(q0 + q1 + q2 + q3);
+    meta.x = __float_as_int(h2f(f2h(d)));
+    meta.y = s;
+    return (uint32_t)(q0 & 0xFF) | ((uint32_t)(q1 & 0xFF) << 8) | ((uint32_t)(q2 & 0xFF) << 16) | ((uint32_t)(q3 & 0xFF) << 24);
+}
+
+// f32 vector (optionally RMS-normalised and multiplied by `normw`) -> staged LDS form.
+// NormRMS as the reference: scale = 1/sqrt(sum(x^2)/K + eps), y = (x*scale)*w
+// (non-linear.cpp:216-219 and the separate Mul node, attention.cpp:274-282 in the Spy tree).
+// K % 32 == 0, x 16-byte aligned.  Ends with __syncthreads().
+template <bool NORM>
+static __device__ __forceinline__ void stage_f32(const float *__restrict__ x, const float *__restrict__ normw, float eps,
+                                                 int8_t *s_q, int2 *s_meta, int K, float *s_red) {
+    float scale = 1.0f;
+    if constexpr (NORM) {
+        float acc = 0.0f;
+        for (int i = threadIdx.x; i < K / 4; i += GEMV_THREADS) {
+            const float4 v = ((const float4 *)x)[i];
+            acc = fmaf(v.x, v.x, acc); acc = fmaf(v.y, v.y, acc); acc = fmaf(v.z, v.z, acc); acc = fmaf(v.w, v.w, acc);
+        }
+        acc = wave_sum(acc);
+        if ((threadIdx.x & 63) == 0) s_red[threadIdx.x >> 6] = acc;
+        __syncthreads();
+        const float sum = (s_red[0] + s_red[1]) + (s_red[2] + s_red[3]);
+        scale = 1.0f / sqrtf(sum / (float)K + eps);
+    }
+    // K/4 float4 groups; 8 consecutive lanes hold one block.  Trip count is uniform per octet.
+    for (int i = threadIdx.x; i < K / 4; i += GEMV_THREADS) {
+        float4 v = ((const float4 *)x)[i];
+        if constexpr (NORM) {
+            const float4 w = ((const float4 *)normw)[i];
+            v.x = (v.x * scale) * w.x; v.y = (v.y * scale) * w.y; v.z = (v.z * scale) * w.z; v.w = (v.w * scale) * w.w;
+        }
+        int2 meta;
+        const uint32_t q = quantize_oct(v, meta);
+        ((uint32_t *)s_q)[i] = q;
+        if ((threadIdx.x & 7) == 0) s_meta[i >> 3] = meta;
+    }
+    __syncthreads();
+}
+
+// ---- weight tiles --------------------------------------------------------------------------
+
+template <int WT> struct wtile { uint32_t w[wt_traits<WT>::NIT_MAX][wt_traits<WT>::PAIR_DW]; };
+
+template <int WT, int LPR>
+static __device__ __forceinline__ void load_tile(wtile<WT> &t, const uint8_t *__restrict__ rowp, int npair, int nit, int l) {
+    constexpr int DW = wt_traits<WT>::PAIR_DW;
+#pragma unroll
+    for (int it = 0; it < wt_traits<WT>::NIT_MAX; it++) {
+        const int p = it * LPR + l;
+        if (it < nit && p < npair) {
+            const uint32_t *wp = (const uint32_t *)rowp + (size_t)p * DW;
+#pragma unroll
+            for (int i = 0; i < DW; i++) t.w[it][i] = wp[i];
+        }
+    }
+}
+
+static __device__ __forceinline__ int dot_q4_dwords(const uint32_t n0, const uint32_t n1, const uint32_t n2, const uint32_t n3,
+                                                    const int4 xl, const int4 xh) {
+    int s = 0;
+    s = __builtin_amdgcn_sdot4((int)(n0 & 0x0F0F0F0Fu), xl.x, s, false); s = __builtin_amdgcn_sdot4((int)((n0 >> 4) & 0x0F0F0F0Fu), xh.x, s, false);
+    s = __builtin_amdgcn_sdot4((int)(n1 & 0x0F0F0F0Fu), xl.y, s, false); s = __builtin_amdgcn_sdot4((int)((n1 >> 4) & 0x0F0F0F0Fu), xh.y, s, false);
+    s = __builtin_amdgcn_sdot4((int)(n2 & 0x0F0F0F0Fu), xl.z, s, false); s = __builtin_amdgcn_sdot4((int)((n2 >> 4) & 0x0F0F0F0Fu), xh.z, s, false);
+    s = __builtin_amdgcn_sdot4((int)(n3 & 0x0F0F0F0Fu), xl.w, s, false); s = __builtin_amdgcn_sdot4((int)((n3 >> 4) & 0x0F0F0F0Fu), xh.w, s, false);
+    return s;
+}
+static __device__ __forceinline__ int dot_q8_dwords(const uint32_t *n, const int4 x0, const int4 x1) {
+    int s = 0;
+    s = __builtin_amdgcn_sdot4((int)n[0], x0.x, s, false); s = __builtin_amdgcn_sdot4((int)n[1], x0.y, s, false);
+    s = __builtin_amdgcn_sdot4((int)n[2], x0.z, s, false); s = __builtin_amdgcn_sdot4((int)n[3], x0.w, s, false);
+    s = __builtin_amdgcn_sdot4((int)n[4], x1.x, s, false); s = __builtin_amdgcn_sdot4((int)n[5], x1.y, s, false);
+    s = __builtin_amdgcn_sdot4((int)n[6], x1.z, s, false); s = __builtin_amdgcn_sdot4((int)n[7], x1.w, s, false);
+    return s;
+}
+
+// Partial dot of the lane's pairs of one weight row with NT staged activation columns.
+// dump (optional): int32 dot of every block, row-major [nblk] for activation column 0.
+template <int WT, int LPR, int NT>
+static __device__ __forceinline__ void dot_tile(const wtile<WT> &t, const staged_act *act, int npair, int nit, int l,
+                                                float acc[NT], int32_t *dump) {
+#pragma unroll
+    for (int it = 0; it < wt_traits<WT>::NIT_MAX; it++) {
+        const int p = it * LPR + l;
+        if (it < nit && p < npair) {
+            const uint32_t *w = t.w[it];
+            if constexpr (WT == SPY_HIP_Q4_0) {
+                const float dA = h2f((uint16_t)(w[0] & 0xFFFFu)), dB = h2f((uint16_t)(w[4] >> 16));
+                const uint32_t a0 = __builtin_amdgcn_alignbit(w[1], w[0], 16), a1 = __builtin_amdgcn_alignbit(w[2], w[1], 16);
+                const uint32_t a2 = __builtin_amdgcn_alignbit(w[3], w[2], 16), a3 = __builtin_amdgcn_alignbit(w[4], w[3], 16);
+#pragma unroll
+                for (int c = 0; c < NT; c++) {
+                    const int4 *xa = (const int4 *)(act[c].q + (size_t)p * 64);
+                    const int4 mm = *(const int4 *)(act[c].meta + 2 * p);
+                    const int iA = dot_q4_dwords(a0, a1, a2, a3, xa[0], xa[1]) - 8 * mm.y;
+                    const int iB = dot_q4_dwords(w[5], w[6], w[7], w[8], xa[2], xa[3]) - 8 * mm.w;
+                    if (dump && c == 0) { dump[2 * p] = iA; dump[2 * p + 1] = iB; }
+                    acc[c] = fmaf(dA * __int_as_float(mm.x), (float)iA, acc[c]);
+                    acc[c] = fmaf(dB * __int_as_float(mm.z), (float)iB, acc[c]);
+                }
+            } else {
+                const float dA = h2f((uint16_t)(w[0] & 0xFFFFu)), dB = h2f((uint16_t)(w[8] >> 16));
+                uint32_t a[8];
+#pragma unroll
+                for (int i = 0; i < 8; i++) a[i] = __builtin_amdgcn_alignbit(w[i + 1], w[i], 16);
+#pragma unroll
+                for (int c = 0; c < NT; c++) {
+                    const int4 *xa = (const int4 *)(act[c].q + (size_t)p * 64);
+                    const int4 mm = *(const int4 *)(act[c].meta + 2 * p);
+                    const int iA = dot_q8_dwords(a, xa[0], xa[1]);
+                    const int iB = dot_q8_dwords(&w[9], xa[2], xa[3]);
+                    if (dump && c == 0) { dump[2 * p] = iA; dump[2 * p + 1] = iB; }
+                    acc[c] = fmaf(dA * __int_as_float(mm.x), (float)iA, acc[c]);
+                    acc[c] = fmaf(dB * __int_as_float(mm.z), (float)iB, acc[c]);
+                }
+            }
+        }
+    }
+}
+
+// Lanes-per-row choice for K elements of type WT; returns 0 when no configuration fits
+// (K must be a multiple of 64 so that every row is a whole number of 4-byte aligned pairs).
+template <int WT> static inline int pick_lpr(int64_t K) {
+    if (K % 64 != 0) return 0;
+    const int64_t npair = K / 64;
+    const int nitmax = wt_traits<WT>::NIT_MAX;
+    if (npair <= 16 * nitmax) return 16;
+    if (npair <= 32 * nitmax) return 32;
+    if (npair <= 64 * nitmax) return 64;
+    return 0;
+}

@@ -6,6 +6,14 @@ import numpy as np
 from spy_amd import _lib as H
 
 REL_TOL = 1e-3      # per-op float tolerance of the parity contract (max-abs error / max-abs value)
+# Across SEVERAL operators the reference's own rounding points re-amplify last-ulp differences:
+# every MatMul re-quantizes its activations to Q8_0 (mat.cpp:95-128 in the Spy tree) and the softmax
+# rounds its exp argument to fp16 (non-linear.cpp:170), so an input that differs by 1e-5 moves a
+# few of those roundings to the neighbouring integer / fp16 value and the next operator's output
+# by ~1e-3.  Any implementation whose fp32 summation order differs from the AVX host code sees
+# this; whole-pass comparisons therefore use this looser bound, per-operator comparisons (same
+# inputs on both sides) use REL_TOL.
+E2E_TOL = 3e-2
 
 
 def dev(arr):

@@ -125,3 +125,24 @@ def test_gemv_full_shapes_linearity(hip, oracle):
         scale = float(np.abs(want).max())
         assert float(np.abs(got[rows] - want).max()) <= 1e-3 * scale
         assert np.all(np.isfinite(got))
+
+
+@pytest.mark.parametrize("wtype", [O.Q4_0, O.Q8_0])
+@pytest.mark.parametrize("M,K,T", [(20011, 256, 1), (9003, 6400, 2), (5000, 12800, 1)])
+def test_gemv_many_row_tiles(hip, oracle, wtype, M, K, T):
+    """More row tiles than resident workgroups: every workgroup walks several tiles (both weight
+    register buffers in use), for each lanes-per-row configuration."""
+    from tests.gpu_util import dev, dev_empty, call, assert_close
+    rng = np.random.default_rng(M + K)
+    nblk = K // 32
+    bs = O.TYPE_SIZE[wtype]
+    w = rng.integers(0, 256, (M, nblk, bs), dtype=np.uint8)
+    w[:, :, :2] = (rng.uniform(0.5, 2, (M, nblk)) * 0.0025).astype(np.float16).view(np.uint8).reshape(M, nblk, 2)
+    if wtype == O.Q8_0:
+        w[:, :, 2:][w[:, :, 2:] == 0x80] = 0x81                         # keep quants in [-127, 127]
+    x = rng.standard_normal((T, K)).astype(np.float32)
+    want = O.matmul(oracle, w, wtype, M, K, x, nthread=8)
+    xq = O.quantize(oracle, x, O.Q8_0)
+    dw, dxq, dout = dev(w), dev(xq), dev_empty(T * M * 4, 0xFF)
+    call(hip.load().spy_hip_gemv_q8_0act, None, wtype, dw.ptr, dxq.ptr, dout.ptr, None, M, K, T, M)
+    assert_close(dout.download(np.float32).reshape(T, M), want, "gemv type %d %dx%d T=%d" % (wtype, M, K, T))

@@ -1,0 +1,182 @@
+"""GPU parity of the token loop: prefill (operator by operator), the fused single-token pass, the
+KV caches and the greedy tokens, against the CPU oracle on the same synthetic model."""
+import numpy as np
+import pytest
+
+from tests import oracle_lib as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _mk(cfg, seed=7, nthread=8):
+    from spy_amd import model as M
+    from tests.model_util import OracleModel, k_quant_quantizer
+    tensors = M.synth_model(cfg, seed=seed, quantizer=k_quant_quantizer)
+    return M.Engine(cfg, tensors), OracleModel(cfg, tensors, nthread=nthread), tensors
+
+
+def _f16(a):
+    return a.view(np.float16).astype(np.float32)
+
+
+def _close(got, want, what, tol=1e-3):
+    from tests.gpu_util import assert_close
+    assert_close(got, want, what, tol)
+
+
+@pytest.mark.parametrize("wtype,t_out,t_emb", [(O.Q4_0, O.Q4_0, O.F32), (O.Q8_0, O.Q8_0, O.Q8_0), (O.Q4_0, O.Q6_K, O.F32)])
+def test_small_model_prefill_decode_and_tokens(wtype, t_out, t_emb):
+    from spy_amd import model as M
+    cfg = M.Config(n_layer=2, n_embd=256, n_head=2, n_ff=768, n_vocab=512, n_ctx=64, wtype=wtype, t_out=t_out, t_tok_embd=t_emb)
+    eng, ora, _ = _mk(cfg)
+    rng = np.random.default_rng(3)
+    prompt = rng.integers(0, cfg.n_vocab, 5).astype(np.int32)
+    # prefill: logits of every prompt token, and the caches it leaves behind
+    lg_g = eng.forward(prompt, 0)
+    lg_o = ora.forward(prompt, 0)
+    _close(lg_g, lg_o, "prefill logits (type %d)" % wtype)
+    for il in range(cfg.n_layer):
+        kg, ko = _f16(eng.read_buffer("k_cache", il, np.uint16)), _f16(ora.k_cache[il])
+        vg, vo = _f16(eng.read_buffer("v_cache", il, np.uint16)), _f16(ora.v_cache[il])
+        _close(kg, ko, "K cache layer %d" % il, 2e-3)       # fp16 storage: one ulp = 2^-11 relative
+        _close(vg, vo, "V cache layer %d" % il, 2e-3)
+        assert np.array_equal(kg == 0, ko == 0) and np.array_equal(vg == 0, vo == 0)     # same slots written
+    # fused single-token pass on top of that cache
+    tok = int(np.argmax(lg_o[-1]))
+    lg1_g = eng.forward(np.array([tok], np.int32), 5)[0]
+    lg1_o = ora.forward(np.array([tok], np.int32), 5)[0]
+    _close(lg1_g, lg1_o, "fused decode logits (type %d)" % wtype)
+    eng.close()
+
+
+def _comfortable_prompt(ora, cfg, n_prompt, n_predict, min_margin, tries=40):
+    """A seeded random prompt whose greedy continuation on the CPU path has the widest top-1/top-2
+    logit gaps (stops early once the smallest gap exceeds min_margin logit standard deviations):
+    random-init models have nearly flat logits, and a near-tie is decided by the last ulp of either
+    implementation."""
+    best = None
+    for seed in range(tries):
+        prompt = np.random.default_rng(1000 + seed).integers(0, cfg.n_vocab, n_prompt).astype(np.int32)
+        margins = []
+        toks = ora.generate(prompt, n_predict, margins)
+        sd = float(ora.forward(prompt, 0)[-1].std())
+        if best is None or min(margins) / sd > best[2] / best[3]:
+            best = (prompt, toks, min(margins), sd)
+        if min(margins) > min_margin * sd:
+            break
+    return best
+
+
+def test_greedy_tokens_identical_small():
+    """Single-token passes one by one against the oracle, then the free-running greedy loop.
+    The reference's softmax rounds its exp argument to fp16 (non-linear.cpp:170 in the Spy tree), so a
+    last-ulp difference in a score occasionally moves that argument to the neighbouring fp16 value
+    (0.1-0.8 % on one probability).  With the handful of cached tokens of this test one probability
+    carries a lot of weight, hence the end-to-end bound below is looser than the per-operator 1e-3
+    (which the operator tests hold on identical inputs); the greedy tokens must still be identical."""
+    from spy_amd import model as M
+    from tests.gpu_util import rel_err
+    cfg = M.Config(n_layer=3, n_embd=512, n_head=4, n_ff=1024, n_vocab=1024, n_ctx=64, wtype=O.Q4_0)
+    eng, ora, _ = _mk(cfg, seed=11)
+    prompt, want, margin, sd = _comfortable_prompt(ora, cfg, 8, 32, 0.05)
+    print("prompt", prompt.tolist(), "min margin %.3e, logit std %.3e" % (margin, sd), flush=True)
+    lg_o = ora.forward(prompt, 0)[-1]
+    lg_g = eng.forward(prompt, 0)[-1]
+    errs = []
+    for step in range(32):
+        errs.append(rel_err(lg_g, lg_o))
+        print("step %2d n_kv %2d: logits max-abs err / max |logit| = %.2e" % (step, len(prompt) + step, errs[-1]), flush=True)
+        assert int(np.argmax(lg_g)) == int(want[step])
+        lg_o = ora.forward(want[step:step + 1], len(prompt) + step)[0]
+        lg_g = eng.forward(want[step:step + 1], len(prompt) + step)[0]
+    assert max(errs) < 3e-2
+    # free-running greedy loop on the device: direct launches, then HIP-graph replay
+    got_direct = eng.decode_greedy(int(want[0]), len(prompt), 31, use_graph=False)
+    assert np.array_equal(got_direct, want[1:])
+    got_graph = eng.decode_greedy(int(want[0]), len(prompt), 31, use_graph=True)
+    assert np.array_equal(got_graph, want[1:])
+    assert np.array_equal(eng.generate(prompt, 32), want)
+    eng.close()
+
+
+def test_fused_decode_real_widths_long_cache():
+    """d = 4096, F = 11008, 32 heads, one layer: the single-token pass over a cache filled to
+    n_past = 700 (random fp16 K/V uploaded to both sides).  The attention output (inputs identical
+    on both sides up to fp16 flips of q) is held to the per-operator bound, the cache slots written
+    to one fp16 ulp, the rest of the pass to the whole-pass bound."""
+    from spy_amd import model as M
+    from tests.gpu_util import E2E_TOL
+    cfg = M.Config(n_layer=1, n_embd=4096, n_head=32, n_ff=11008, n_vocab=4096, n_ctx=1024, wtype=O.Q4_0)
+    eng, ora, _ = _mk(cfg, seed=21, nthread=16)
+    rng = np.random.default_rng(9)
+    for P in (700, 0, 1023):
+        k = (rng.standard_normal(cfg.n_ctx * cfg.n_embd) * 0.5).astype(np.float16).view(np.uint16)
+        v = (rng.standard_normal(cfg.n_ctx * cfg.n_embd) * 0.5).astype(np.float16).view(np.uint16)
+        ora.k_cache[0][:] = k; ora.v_cache[0][:] = v
+        eng.write_buffer("k_cache", 0, k); eng.write_buffer("v_cache", 0, v)
+        ora.clear_taps()
+        kqv, layer_out = ora.tap("kqv", 0, cfg.n_embd), ora.tap("layer_out", 0, cfg.n_embd)
+        tok = np.array([123], np.int32)
+        lg_g = eng.forward(tok, P)[0]
+        lg_o = ora.forward(tok, P)[0]
+        ora.clear_taps()
+        _close(eng.read_buffer("attn_out", 0, np.float32), kqv, "attention output, n_kv = %d" % (P + 1))
+        _close(eng.read_buffer("x", 0, np.float32), layer_out, "layer output, n_kv = %d" % (P + 1), E2E_TOL)
+        _close(lg_g, lg_o, "logits, n_kv = %d" % (P + 1), E2E_TOL)
+        kg = _f16(eng.read_buffer("k_cache", 0, np.uint16)).reshape(cfg.n_ctx, cfg.n_embd)
+        ko = _f16(ora.k_cache[0]).reshape(cfg.n_ctx, cfg.n_embd)
+        _close(kg[P], ko[P], "K row written at pos %d" % P, 2e-3)
+        assert np.array_equal(np.delete(kg, P, axis=0), np.delete(ko, P, axis=0))           # every other slot untouched
+        vg = _f16(eng.read_buffer("v_cache", 0, np.uint16)).reshape(cfg.n_embd, cfg.n_ctx)
+        vo = _f16(ora.v_cache[0]).reshape(cfg.n_embd, cfg.n_ctx)
+        _close(vg[:, P], vo[:, P], "V column written at pos %d" % P, 2e-3)
+        assert np.array_equal(np.delete(vg, P, axis=1), np.delete(vo, P, axis=1))
+    eng.close()
+
+
+@pytest.mark.timeout(900)
+def test_llama2_7b_q4_0_greedy_32_tokens():
+    """Config 1: the 7B shape, Q4_0, 8 random prompt tokens, 32 greedy steps.
+
+    Every MatMul of the reference re-quantizes its activations to Q8_0, so two implementations whose
+    fp32 sums are not bit-identical decorrelate their Q8_0 rounding noise within a few layers and
+    then differ by that noise itself: about 0.7 % per MatMul output, a few percent of the largest
+    logit after 32 layers of a random-init model.  The test therefore (a) bounds the per-pass logits
+    difference by that noise level, (b) requires the same argmax at every teacher-forced step whose
+    top-1/top-2 gap on the CPU path exceeds twice the measured difference, and (c) requires the
+    free-running device loop to emit the CPU path's tokens up to the first step that is not
+    decidable in that sense.  It prints how many of the 32 tokens are identical."""
+    import os
+    from spy_amd import model as M
+    from tests.gpu_util import rel_err
+    cfg = M.Config.llama2_7b(n_ctx=48, wtype=O.Q4_0)
+    ncpu = min(16, os.cpu_count() or 8)
+    eng, ora, _ = _mk(cfg, seed=1234, nthread=ncpu)
+    prompt, want, margin, sd = _comfortable_prompt(ora, cfg, 8, 32, 0.05, tries=8)
+    print("7B Q4_0: prompt", prompt.tolist(), "min top-1/top-2 margin %.3e, logit std %.3e" % (margin, sd), flush=True)
+    print("oracle tokens:", want.tolist(), flush=True)
+    margins = []
+    ora.generate(prompt, 32, margins)
+    lg_o = ora.forward(prompt, 0)
+    lg_g = eng.forward(prompt, 0)
+    _close(lg_g, lg_o, "7B prefill logits (8 tokens)", 0.15)
+    lg_o, lg_g = lg_o[-1], lg_g[-1]
+    errs, abs_errs, same = [], [], []
+    for step in range(32):
+        errs.append(rel_err(lg_g, lg_o))
+        abs_errs.append(float(np.abs(lg_g - lg_o).max()))
+        same.append(int(np.argmax(lg_g)) == int(want[step]))
+        lg_o = ora.forward(want[step:step + 1], len(prompt) + step)[0]
+        lg_g = eng.forward(want[step:step + 1], len(prompt) + step)[0]
+    noise = max(abs_errs)
+    decidable = [m > 2 * noise for m in margins]
+    print("per-pass logits max-abs err / max |logit|: median %.2e max %.2e; max-abs err %.3e; %d of 32 steps decidable, %d of 32 teacher-forced argmax identical"
+          % (float(np.median(errs)), max(errs), noise, sum(decidable), sum(same)), flush=True)
+    assert max(errs) < 0.15
+    assert all(s for s, d in zip(same, decidable) if d)
+    got = eng.generate(prompt, 32)
+    n_same = int(np.argmin(np.concatenate([got == want, [False]])))
+    first_undecidable = decidable.index(False) if False in decidable else 32
+    print("hip tokens:   ", got.tolist(), "\nfree-running: first %d tokens identical (first undecidable step: %d)" % (n_same, first_undecidable), flush=True)
+    assert n_same >= first_undecidable
+    eng.close()
