@@ -1,0 +1,150 @@
+#!/usr/bin/env python3
+"""Headline benchmark: single-sequence greedy decode of a LLaMA-2-7B shaped Q4_0 model with the
+f16 KV cache filled to 4096 tokens, on one MI355X.
+
+A "step" is one single-token forward pass (all 32 layers + output head + greedy sampling) at
+n_kv = 4096 + step; weights and KV cache are resident in HBM before the timed region starts.
+Prints ONE JSON line (see the keys below).  The CPU baseline is the oracle (a port of the reference's
+host backend path) timed on this machine's cores on a bounded sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK = 8.0e12          # MI355X HBM3E, bytes/s
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--ctx-fill", type=int, default=4096, help="tokens in the KV cache before the first timed step")
+    ap.add_argument("--prefill", choices=["real", "synthetic"], default="real",
+                    help="real: run the prompt through the model; synthetic: fill the caches with random fp16 (quick runs)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-steps", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=32, help="debug only: fewer layers (result is then not the headline config)")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs the token loop on ONE GPU (no sharding, no collectives); --gpus %d is not supported" % args.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    from spy_amd import _lib as H
+    from spy_amd import model as M
+
+    H.init(0)
+    info = H.device_info()
+    log("device:", info)
+    steps, warmup, fill = args.steps, args.warmup, args.ctx_fill
+    n_ctx = (fill + warmup + steps + 8 + 7) // 8 * 8
+    cfg = M.Config.llama2_7b(n_ctx=n_ctx, wtype=H.Q4_0)
+    cfg.n_layer = args.layers
+    t0 = time.time()
+    tensors = M.synth_model(cfg, seed=1234)
+    log("synthetic model: %.1f s, %.2f GB of weights streamed per token" % (time.time() - t0, cfg.weight_bytes() / 1e9))
+    eng = M.Engine(cfg, tensors)
+    rng = np.random.default_rng(4096)
+    prompt = rng.integers(0, cfg.n_vocab, fill).astype(np.int32)
+    t0 = time.time()
+    if args.prefill == "real":
+        logits = eng.forward(prompt, 0, want_logits=False)
+        last = eng.forward(prompt[-1:], fill - 1)          # re-run the last prompt token alone to get its logits
+        first = int(np.argmax(last[0]))
+    else:
+        for il in range(cfg.n_layer):
+            eng.write_buffer("k_cache", il, (rng.standard_normal(fill * cfg.n_embd) * 1.3).astype(np.float16).view(np.uint16))
+            v = np.zeros((cfg.n_embd, cfg.n_ctx), np.float16)
+            v[:, :fill] = (rng.standard_normal((cfg.n_embd, fill)) * 1.3).astype(np.float16)
+            eng.write_buffer("v_cache", il, v.view(np.uint16))
+        first = int(prompt[-1])
+    H.sync()
+    log("prefill (%s) of %d tokens: %.1f s" % (args.prefill, fill, time.time() - t0))
+
+    # warm-up (also captures the HIP graph), then the timed region: exactly `steps` passes
+    pos = fill
+    toks = eng.decode_greedy(first, pos, warmup, use_graph=True)
+    pos += warmup
+    eng.timing()
+    H.sync()
+    t0 = time.perf_counter()
+    toks = eng.decode_greedy(int(toks[-1]), pos, steps, use_graph=True)
+    H.sync()
+    wall = time.perf_counter() - t0
+    ev_ms, n_timed = eng.timing()
+    assert n_timed == steps
+    ms_per_step = wall * 1e3 / steps
+    tok_s = steps / wall
+    n_kv_mid = pos + steps / 2.0
+    kv_bytes = 2 * cfg.n_embd * 2 * cfg.n_layer           # K and V, fp16, per cached token
+    bytes_per_token = cfg.weight_bytes() + kv_bytes * n_kv_mid
+    frac = bytes_per_token / (wall / steps) / HBM_PEAK
+    log("decode: %.3f ms/step wall, %.3f ms/step by HIP events, %.1f tok/s, %.2f GB/token -> %.1f%% of 8 TB/s"
+        % (ms_per_step, ev_ms, tok_s, bytes_per_token / 1e9, 100 * frac))
+
+    # dominant kernel: the gate|up projection with the fused RMSNorm / Q8_0 / SiLU epilogue
+    per_kernel = {}
+    for name in ("qkv", "scores", "pv", "wo", "gate_up", "down", "head"):
+        per_kernel[name] = eng.kernel_time_us(name, reps=4)
+    d, F, V = cfg.n_embd, cfg.n_ff, cfg.n_vocab
+    n_kv_end = pos + steps
+    alg = {"qkv": 3 * d * d * 18 // 32, "wo": d * d * 18 // 32, "gate_up": 2 * F * d * 18 // 32, "down": F * d * 18 // 32,
+           "head": V * d * 18 // 32, "scores": n_kv_end * d * 2, "pv": n_kv_end * d * 2}
+    log("per-kernel (HIP events, walking the layers):")
+    for k, us in per_kernel.items():
+        log("  %-8s %8.2f us  %7.1f GB/s  (%.1f%% of 8 TB/s)" % (k, us, alg[k] / us / 1e3, alg[k] / us / 1e3 / 80))
+    dom = "gate_up"
+    achieved = alg[dom] / (per_kernel[dom] * 1e-6) / 1e9
+    roofline = {"kernel": "fused_gemv_kernel<Q4_0, gate|up + SiLU>", "bound": "hbm", "achieved": round(achieved, 1), "peak": 8000.0,
+                "unit": "GB/s", "frac": round(achieved / 8000.0, 4), "traffic": None,
+                "bytes_per_launch": alg[dom], "us_per_launch": round(per_kernel[dom], 3)}
+
+    cpu = None
+    if not args.no_cpu:
+        from tests import oracle_lib as O            # the checker, timed as the CPU baseline
+        from tests.model_util import OracleModel
+        ncpu = min(16, os.cpu_count() or 1)
+        ora = OracleModel(cfg, tensors, nthread=ncpu)
+        for il in range(cfg.n_layer):                # same cache contents as the GPU run
+            ora.k_cache[il][:] = eng.read_buffer("k_cache", il, np.uint16)
+            ora.v_cache[il][:] = eng.read_buffer("v_cache", il, np.uint16)
+        tok = np.array([first], np.int32)
+        ora.forward(tok, fill)                        # untimed warm-up pass (cli.h:78-82)
+        t0 = time.perf_counter()
+        for i in range(args.cpu_steps):
+            lg = ora.forward(tok, fill + i)
+            tok = np.array([int(np.argmax(lg[0]))], np.int32)
+        cpu_wall = time.perf_counter() - t0
+        cpu = {"value": round(args.cpu_steps / cpu_wall, 3), "unit": "tok/s", "cores": ncpu, "kind": "port",
+               "sample": "%d single-token passes of the same model at n_kv = %d.. (AVX2 port of Spy's host backend, OpenMP)" % (args.cpu_steps, fill + 1)}
+        log("cpu baseline: %.3f tok/s on %d threads" % (cpu["value"], ncpu))
+
+    out = {
+        "metric": "decode tok/s + % HBM roofline, LLaMA-2-7B Q4_0 ctx 4096, 1xMI355X",
+        "value": round(tok_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8 dot (Q4_0 x Q8_0), fp32 accumulate, fp16 KV", "data": "synthetic",
+        "config": {"workload": "LLaMA-2-7B shape (32 layers, d 4096, 32 heads x 128, FFN 11008, vocab 32000), Q4_0 weights incl. head, "
+                               "f16 KV cache prefilled to %d tokens (%s), greedy single-sequence decode" % (fill, args.prefill),
+                   "n_layer": cfg.n_layer, "n_kv_first": pos + 1, "n_kv_last": pos + steps, "bytes_per_token": int(bytes_per_token)},
+        "hbm_roofline_frac": round(frac, 4), "ms_per_step_hip_events": round(ev_ms, 4),
+        "kernel_us": {k: round(v, 2) for k, v in per_kernel.items()},
+        "roofline": roofline, "cpu_baseline": cpu,
+    }
+    print(json.dumps(out), flush=True)
+    eng.close()
+
+
+if __name__ == "__main__":
+    main()

@@ -172,6 +172,10 @@ int spy_hip_llama_buffer(spy_hip_llama *m, const char *name, int32_t layer, void
 /* average duration (ms) of the HIP-event-timed single-token passes since the last call, and their
  * count; timing is recorded around every pass of spy_hip_llama_decode_greedy */
 int spy_hip_llama_timing(spy_hip_llama *m, float *ms_per_pass, int32_t *n_pass);
+/* average duration (microseconds) of one kernel of the single-token pass, HIP events around
+ * reps x n_layer launches that walk the layers (fresh weights / caches every launch); which:
+ * "qkv", "scores", "pv", "wo", "gate_up", "down", "head".  Uses the position of the last pass. */
+int spy_hip_llama_kernel_time(spy_hip_llama *m, void *stream, const char *which, int32_t reps, float *us_per_launch);
 
 #ifdef __cplusplus
 }

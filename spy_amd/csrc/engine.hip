@@ -172,59 +172,76 @@ static bool fused_ok(const spy_hip_llama *m) {
     return m->hd == 128 && (m->lpr_d == 16 || m->lpr_d == 32) && m->lpr_ff != 0 && m->desc.n_embd % 4 == 0;
 }
 
+enum { K_QKV = 0, K_SCORES, K_PV, K_WO, K_GATEUP, K_DOWN, K_HEAD, K_COUNT };
+
+// one kernel of layer il of the single-token pass
 template <int WT>
-static int enqueue_pass(spy_hip_llama *m, hipStream_t st, bool sample) {
+static int enqueue_kernel(spy_hip_llama *m, hipStream_t st, int which, int il) {
     const spy_hip_llama_desc &c = m->desc;
     const int d = c.n_embd, F = c.n_ff, C = c.n_ctx, H = c.n_head;
-    embed_kernel<<<dim3(1), dim3(256), 0, st>>>(m->st, (const uint8_t *)c.tok_embd, c.t_tok_embd == SPY_HIP_Q8_0, d, c.n_vocab, m->x,
-                                                m->rope_cs, m->theta_scale, m->hd);
-    RC_TRY(SPY_LAUNCH_RC());
     const float scale = 1.0f / sqrtf((float)m->hd);                     // SoftmaxParam::scale (attention.cpp:113)
     const size_t pv_lds = (size_t)C * 4 + (size_t)C * 2 + 16;
-    for (int il = 0; il < c.n_layer; il++) {
-        const spy_hip_llama_layer &L = m->layers[il];
-        fused_args a;
-        memset(&a, 0, sizeof(a));
-        a.st = m->st; a.rope_cs = m->rope_cs; a.q16 = m->q16; a.kc = m->k_cache[il]; a.vc = m->v_cache[il];
-        a.n_ctx = C; a.d = d; a.hd = m->hd; a.eps = c.eps;
-        // attn_norm, attn_norm_linear, Q/K/V_project, rope, KV-cache copies
+    const spy_hip_llama_layer &L = m->layers[il];
+    fused_args a;
+    memset(&a, 0, sizeof(a));
+    a.st = m->st; a.rope_cs = m->rope_cs; a.q16 = m->q16; a.kc = m->k_cache[il]; a.vc = m->v_cache[il];
+    a.n_ctx = C; a.d = d; a.hd = m->hd; a.eps = c.eps;
+    switch (which) {
+    case K_QKV:      // attn_norm, attn_norm_linear, Q/K/V_project, rope, KV-cache copies
         a.W0 = (const uint8_t *)L.wq; a.W1 = (const uint8_t *)L.wk; a.W2 = (const uint8_t *)L.wv;
         a.M = 3 * d; a.K = d; a.x_in = m->x; a.normw = L.attn_norm;
-        RC_TRY((launch_fused_lpr<WT, true, EPI_QKV>(m, st, m->lpr_d, a)));
-        // attn_score
+        return launch_fused_lpr<WT, true, EPI_QKV>(m, st, m->lpr_d, a);
+    case K_SCORES:   // attn_score
         attn_scores_kernel<<<dim3((unsigned)((C + ATT_TCH - 1) / ATT_TCH)), dim3(256), 0, st>>>(m->st, m->q16, m->k_cache[il], m->scores, H, C, scale);
-        RC_TRY(SPY_LAUNCH_RC());
-        // softmax, KQV (+ permute/contiguous: attn_out is already [hd, H] contiguous)
+        return SPY_LAUNCH_RC();
+    case K_PV:       // softmax, KQV (+ permute/contiguous: attn_out is already [hd, H] contiguous)
         attn_pv_kernel<<<dim3((unsigned)(H * 8)), dim3(256), pv_lds, st>>>(m->st, m->scores, m->v_cache[il], m->attn_out, C);
-        RC_TRY(SPY_LAUNCH_RC());
-        // KQV_linear + ffn_input
+        return SPY_LAUNCH_RC();
+    case K_WO:       // KQV_linear + ffn_input
         a.W0 = (const uint8_t *)L.wo; a.M = d; a.K = d; a.x_in = m->attn_out; a.resid = m->x; a.out = m->x1;
-        RC_TRY((launch_fused_lpr<WT, false, EPI_RESID>(m, st, m->lpr_d, a)));
-        // ffn_norm, ffn_up, ffn_gate, silu, ffn_par
+        return launch_fused_lpr<WT, false, EPI_RESID>(m, st, m->lpr_d, a);
+    case K_GATEUP:   // ffn_norm, ffn_up, ffn_gate, silu, ffn_par
         a.W0 = (const uint8_t *)L.w_gate; a.W1 = (const uint8_t *)L.w_up; a.M = 2 * F; a.K = d; a.x_in = m->x1; a.normw = L.ffn_norm; a.out = m->hbuf;
-        RC_TRY((launch_fused_lpr<WT, true, EPI_GATEUP>(m, st, m->lpr_d, a)));
-        // ffn_down + logit_output (the next layer's input)
+        return launch_fused_lpr<WT, true, EPI_GATEUP>(m, st, m->lpr_d, a);
+    case K_DOWN:     // ffn_down + logit_output (the next layer's input)
         a.W0 = (const uint8_t *)L.w_down; a.M = d; a.K = F; a.x_in = m->hbuf; a.resid = m->x1; a.out = m->x;
-        RC_TRY((launch_fused_lpr<WT, false, EPI_RESID>(m, st, m->lpr_ff, a)));
+        return launch_fused_lpr<WT, false, EPI_RESID>(m, st, m->lpr_ff, a);
     }
-    // result_norm, result_linear, output
+    return SPY_HIP_EINVAL;
+}
+
+// result_norm, result_linear, output
+template <int WT>
+static int enqueue_head(spy_hip_llama *m, hipStream_t st) {
+    const spy_hip_llama_desc &c = m->desc;
+    const int d = c.n_embd;
     if (c.t_out == c.wtype) {
         fused_args a;
         memset(&a, 0, sizeof(a));
         a.W0 = (const uint8_t *)c.w_out; a.M = c.n_vocab; a.K = d; a.x_in = m->x; a.normw = c.out_norm; a.eps = c.eps; a.out = m->logits;
-        RC_TRY((launch_fused_lpr<WT, true, EPI_STORE>(m, st, m->lpr_d, a)));
-    } else {
-        // head in another type (e.g. Q6_K): norm + weight + Q8_0 through the operator kernels
-        spy_hip_tensor tx, tw, txn;
-        memset(&tx, 0, sizeof(tx));
-        tx.type = SPY_HIP_F32; tx.dim = 1; tx.ne[0] = d; tx.ne[1] = tx.ne[2] = tx.ne[3] = 1; tx.nb[0] = 4; tx.nb[1] = tx.nb[2] = tx.nb[3] = 4 * d;
-        tw = tx; txn = tx;
-        tx.data = m->x; tw.data = (void *)c.out_norm; txn.data = m->x1;
-        RC_TRY(spy_hip_op_norm_rms(st, &tx, &txn, c.eps));
-        RC_TRY(spy_hip_op_binary(st, 2, &txn, &tw, &txn));
-        RC_TRY(spy_hip_quantize_q8_0(st, m->x1, 4 * d, m->xq_head, 1, d));
-        RC_TRY(spy_hip_gemv_q8_0act(st, c.t_out, c.w_out, m->xq_head, m->logits, nullptr, c.n_vocab, d, 1, c.n_vocab));
+        return launch_fused_lpr<WT, true, EPI_STORE>(m, st, m->lpr_d, a);
     }
+    // head in another type (e.g. Q6_K): norm + weight + Q8_0 through the operator kernels
+    spy_hip_tensor tx, tw, txn;
+    memset(&tx, 0, sizeof(tx));
+    tx.type = SPY_HIP_F32; tx.dim = 1; tx.ne[0] = d; tx.ne[1] = tx.ne[2] = tx.ne[3] = 1; tx.nb[0] = 4; tx.nb[1] = tx.nb[2] = tx.nb[3] = 4 * d;
+    tw = tx; txn = tx;
+    tx.data = m->x; tw.data = (void *)c.out_norm; txn.data = m->x1;
+    RC_TRY(spy_hip_op_norm_rms(st, &tx, &txn, c.eps));
+    RC_TRY(spy_hip_op_binary(st, 2, &txn, &tw, &txn));
+    RC_TRY(spy_hip_quantize_q8_0(st, m->x1, 4 * d, m->xq_head, 1, d));
+    return spy_hip_gemv_q8_0act(st, c.t_out, c.w_out, m->xq_head, m->logits, nullptr, c.n_vocab, d, 1, c.n_vocab);
+}
+
+template <int WT>
+static int enqueue_pass(spy_hip_llama *m, hipStream_t st, bool sample) {
+    const spy_hip_llama_desc &c = m->desc;
+    embed_kernel<<<dim3(1), dim3(256), 0, st>>>(m->st, (const uint8_t *)c.tok_embd, c.t_tok_embd == SPY_HIP_Q8_0, c.n_embd, c.n_vocab, m->x,
+                                                m->rope_cs, m->theta_scale, m->hd);
+    RC_TRY(SPY_LAUNCH_RC());
+    for (int il = 0; il < c.n_layer; il++)
+        for (int k = K_QKV; k <= K_DOWN; k++) RC_TRY(enqueue_kernel<WT>(m, st, k, il));
+    RC_TRY(enqueue_head<WT>(m, st));
     if (sample) {
         sample_advance_kernel<<<dim3(1), dim3(1024), 0, st>>>(m->st, m->logits, c.n_vocab, m->tokens_out, m->max_out);
         RC_TRY(SPY_LAUNCH_RC());
@@ -414,5 +431,33 @@ extern "C" int spy_hip_llama_decode_greedy(spy_hip_llama *m, void *stream, int32
     HIP_TRY(hipMemcpy(&back, m->st, sizeof(back), hipMemcpyDeviceToHost));
     if (back.err) return SPY_HIP_EINVAL;
     if (tokens_host) HIP_TRY(hipMemcpy(tokens_host, m->tokens_out, (size_t)n_steps * 4, hipMemcpyDeviceToHost));
+    return 0;
+}
+
+// Average duration of ONE kernel of the single-token pass, measured with HIP events on the stream it
+// is launched on: the kernel is launched for layer 0, 1, .. n_layer-1 (different weights and
+// caches every launch, so nothing is served from a cache that the token loop would not have),
+// `reps` times over.  The position used is the one left by the last pass.  which: "qkv", "scores",
+// "pv", "wo", "gate_up", "down", "head".
+extern "C" int spy_hip_llama_kernel_time(spy_hip_llama *m, void *stream, const char *which, int32_t reps, float *us_per_launch) {
+    SPY_CHECK_ARG(m && which && reps > 0 && us_per_launch);
+    if (!fused_ok(m)) return SPY_HIP_EUNSUPPORTED;
+    static const char *names[K_COUNT] = {"qkv", "scores", "pv", "wo", "gate_up", "down", "head"};
+    int k = -1;
+    for (int i = 0; i < K_COUNT; i++) if (!strcmp(which, names[i])) k = i;
+    SPY_CHECK_ARG(k >= 0);
+    hipStream_t st = stream ? (hipStream_t)stream : m->own_stream;
+    const bool q4 = m->desc.wtype == SPY_HIP_Q4_0;
+    auto once = [&](int il) { return k == K_HEAD ? (q4 ? enqueue_head<SPY_HIP_Q4_0>(m, st) : enqueue_head<SPY_HIP_Q8_0>(m, st))
+                                                 : (q4 ? enqueue_kernel<SPY_HIP_Q4_0>(m, st, k, il) : enqueue_kernel<SPY_HIP_Q8_0>(m, st, k, il)); };
+    for (int il = 0; il < m->desc.n_layer; il++) RC_TRY(once(il));           // warm-up
+    HIP_TRY(hipEventRecord(m->ev0, st));
+    for (int r = 0; r < reps; r++)
+        for (int il = 0; il < m->desc.n_layer; il++) RC_TRY(once(il));
+    HIP_TRY(hipEventRecord(m->ev1, st));
+    HIP_TRY(hipEventSynchronize(m->ev1));
+    float ms = 0.0f;
+    HIP_TRY(hipEventElapsedTime(&ms, m->ev0, m->ev1));
+    *us_per_launch = ms * 1000.0f / (float)(reps * m->desc.n_layer);
     return 0;
 }

@@ -158,6 +158,11 @@ class Engine:
         H.check(self.L.spy_hip_llama_timing(self.handle, C.byref(ms), C.byref(n)), "spy_hip_llama_timing")
         return ms.value, n.value
 
+    def kernel_time_us(self, which, reps=4):
+        us = C.c_float()
+        H.check(self.L.spy_hip_llama_kernel_time(self.handle, None, which.encode(), reps, C.byref(us)), "spy_hip_llama_kernel_time")
+        return us.value
+
     def buffer(self, name, layer=0):
         p, n = C.c_void_p(), C.c_size_t()
         H.check(self.L.spy_hip_llama_buffer(self.handle, name.encode(), layer, C.byref(p), C.byref(n)), "spy_hip_llama_buffer")
