@@ -18,42 +18,40 @@ struct dev_state {           // lives in device memory so that a captured graph 
     int32_t err;
 };
 
-// ---- persistent GEMV over row tiles with double-buffered weight registers ----------------------
-template <int WT, int LPR> struct gemv_stream {
+// ---- persistent GEMV over row tiles with two tiles' weights always in flight ---------------------
+template <int WT, int LPR, int NIT> struct gemv_stream {
     static constexpr int RPW = SPY_WAVE / LPR, RPT = GEMV_WAVES * RPW;
-    wtile<WT> A, B;
-    int tile, ntiles, G, npair, nit, l, g, rofs, M;
-    size_t RB;
+    wtile<WT, NIT> A, B;
+    int tile, ntiles, G, npair, l, g, rofs, M;
 
+    template <class RowPtr> __device__ __forceinline__ void fetch(wtile<WT, NIT> &t, int tl, RowPtr rowptr) {
+        if (tl < ntiles && tl * RPT + rofs < M) load_tile<WT, LPR, NIT>(t, rowptr(tl * RPT + rofs), npair, l);
+    }
     template <class RowPtr> __device__ __forceinline__ void begin(int M_, int K, RowPtr rowptr) {
         M = M_;
-        const int nblk = K / 32;
-        npair = K / 64; nit = (npair + LPR - 1) / LPR;
-        RB = (size_t)nblk * wt_traits<WT>::BLK;
+        npair = K / 64;
         const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
         l = lane % LPR; g = lane / LPR; rofs = wave * RPW + g;
         ntiles = (M + RPT - 1) / RPT; G = gridDim.x; tile = blockIdx.x;
-        if (tile < ntiles && tile * RPT + rofs < M) load_tile<WT, LPR>(A, rowptr(tile * RPT + rofs), npair, nit, l);
+        fetch(A, tile, rowptr);
+        fetch(B, tile + G, rowptr);
     }
-
     // epi(r, total, valid): called by every lane; `total` is the row's dot, present in all LPR lanes
     template <class RowPtr, class Epi> __device__ __forceinline__ void run(const staged_act &act, RowPtr rowptr, Epi epi) {
-        auto finish = [&](const wtile<WT> &t, int tl) {
+        auto finish = [&](const wtile<WT, NIT> &t, int tl) {
             const int r = tl * RPT + rofs;
             float acc[1] = {0.0f};
-            if (r < M) dot_tile<WT, LPR, 1>(t, &act, npair, nit, l, acc, nullptr);
+            if (r < M) dot_tile<WT, LPR, NIT, 1>(t, &act, npair, l, acc, nullptr);
             epi(r, group_sum<LPR>(acc[0]), r < M);
         };
         while (tile < ntiles) {
-            int tn = tile + G;
-            if (tn < ntiles && tn * RPT + rofs < M) load_tile<WT, LPR>(B, rowptr(tn * RPT + rofs), npair, nit, l);
             finish(A, tile);
-            tile = tn;
+            fetch(A, tile + 2 * G, rowptr);
+            tile += G;
             if (tile >= ntiles) break;
-            tn = tile + G;
-            if (tn < ntiles && tn * RPT + rofs < M) load_tile<WT, LPR>(A, rowptr(tn * RPT + rofs), npair, nit, l);
             finish(B, tile);
-            tile = tn;
+            fetch(B, tile + 2 * G, rowptr);
+            tile += G;
         }
     }
 };
@@ -62,29 +60,6 @@ template <int WT, int LPR> struct gemv_stream {
 static __device__ __forceinline__ float silu_lut(float x) {
     const float v = h2f(f2h(x));
     return v / (1.0f + expf(-v));
-}
-
-// ---- token embedding + RoPE table ---------------------------------------------------------------
-// GetRow (view.cpp:33-81): F32 copy or Q8_0 dequant.  The cos/sin table of this position follows
-// the reference's recurrence: theta_0 = pos, theta_{k+1} = theta_k * theta_scale in fp32
-// (non-linear.cpp:304-309), cosf / sinf of it.
-__global__ __launch_bounds__(256) void embed_kernel(dev_state *st, const uint8_t *__restrict__ table, int q8, int d, int n_vocab,
-                                                    float *__restrict__ x, float *__restrict__ rope_cs, float theta_scale, int hd) {
-    int tok = st->token;
-    if (tok < 0 || tok >= n_vocab) { if (threadIdx.x == 0) st->err = 1; tok = 0; }
-    if (!q8) {
-        const float *row = (const float *)table + (size_t)tok * d;
-        for (int i = threadIdx.x; i < d; i += 256) x[i] = row[i];
-    } else {
-        const blk_q8_0 *row = (const blk_q8_0 *)(table + (size_t)tok * (d / 32) * 34);
-        for (int i = threadIdx.x; i < d; i += 256) x[i] = (float)row[i >> 5].qs[i & 31] * h2f(row[i >> 5].d);
-    }
-    for (int k = threadIdx.x; k < hd / 2; k += 256) {
-        float theta = (float)st->pos;
-        for (int j = 0; j < k; j++) theta *= theta_scale;
-        rope_cs[2 * k] = cosf(theta);
-        rope_cs[2 * k + 1] = sinf(theta);
-    }
 }
 
 // ---- fused GEMVs ----------------------------------------------------------------------------------
@@ -100,7 +75,8 @@ struct fused_args {
 
 enum { EPI_QKV = 0, EPI_RESID = 1, EPI_GATEUP = 2, EPI_STORE = 3 };
 
-template <int WT, int LPR, bool NORM, int EPI>
+// SIT > 0: RMSNorm * weight prologue with SIT float4 of x per thread (K <= 1024*SIT); SIT == 0: plain
+template <int WT, int LPR, int NIT, int SIT, int EPI>
 __global__ __launch_bounds__(GEMV_THREADS) void fused_gemv_kernel(fused_args a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     __shared__ float s_red[4];
@@ -110,12 +86,18 @@ __global__ __launch_bounds__(GEMV_THREADS) void fused_gemv_kernel(fused_args a) 
         else if constexpr (EPI == EPI_GATEUP) return ((r & 1) ? a.W1 : a.W0) + (size_t)(r >> 1) * RB;
         else return a.W0 + (size_t)r * RB;
     };
-    gemv_stream<WT, LPR> gs;
-    gs.begin(a.M, a.K, rowptr);                      // first tile's weights are in flight from here on
+    gemv_stream<WT, LPR, NIT> gs;
+    gs.begin(a.M, a.K, rowptr);                      // the first two tiles' weights are in flight from here on
 
     int8_t *s_q = (int8_t *)smem;
     int2 *s_meta = (int2 *)(smem + a.K);
-    stage_f32<NORM>(a.x_in, a.normw, a.eps, s_q, s_meta, a.K, s_red);
+    if constexpr (SIT > 0) {
+        stage_regs<SIT> sr;
+        stage_norm_load<SIT>(sr, a.x_in, a.normw, a.K);
+        stage_norm_finish<SIT>(sr, a.eps, s_q, s_meta, a.K, s_red);
+    } else {
+        stage_f32_plain(a.x_in, s_q, s_meta, a.K);
+    }
     staged_act act; act.q = s_q; act.meta = s_meta;
 
     const int l = gs.l;
@@ -145,9 +127,35 @@ __global__ __launch_bounds__(GEMV_THREADS) void fused_gemv_kernel(fused_args a) 
     gs.run(act, rowptr, epi);
 }
 
+#ifdef SPY_DECODE_COMMON_KERNELS   // type-independent kernels: compiled by one translation unit only
+
+// ---- token embedding + RoPE table ---------------------------------------------------------------
+// GetRow (view.cpp:33-81): F32 copy or Q8_0 dequant.  The cos/sin table of this position follows
+// the reference's recurrence: theta_0 = pos, theta_{k+1} = theta_k * theta_scale in fp32
+// (non-linear.cpp:304-309), cosf / sinf of it.
+__global__ __launch_bounds__(256) void embed_kernel(dev_state *st, const uint8_t *__restrict__ table, int q8, int d, int n_vocab,
+                                                    float *__restrict__ x, float *__restrict__ rope_cs, float theta_scale, int hd) {
+    int tok = st->token;
+    if (tok < 0 || tok >= n_vocab) { if (threadIdx.x == 0) st->err = 1; tok = 0; }
+    if (!q8) {
+        const float *row = (const float *)table + (size_t)tok * d;
+        for (int i = threadIdx.x; i < d; i += 256) x[i] = row[i];
+    } else {
+        const blk_q8_0 *row = (const blk_q8_0 *)(table + (size_t)tok * (d / 32) * 34);
+        for (int i = threadIdx.x; i < d; i += 256) x[i] = (float)row[i >> 5].qs[i & 31] * h2f(row[i >> 5].d);
+    }
+    for (int k = threadIdx.x; k < hd / 2; k += 256) {
+        float theta = (float)st->pos;
+        for (int j = 0; j < k; j++) theta *= theta_scale;
+        rope_cs[2 * k] = cosf(theta);
+        rope_cs[2 * k + 1] = sinf(theta);
+    }
+}
+
 // ---- attention scores ---------------------------------------------------------------------------
 // One workgroup per chunk of ATT_TCH cached tokens, all heads: a (token, head) key is 256 bytes
-// = 16 lanes x 128-bit.  t = (K.q + mask) * scale with mask = 0 for every cached token of a
+// = 16 lanes x 128-bit; a thread covers two heads (h and h+16) so that 2*ATT_TCH loads are in
+// flight per thread.  t = (K.q + mask) * scale with mask = 0 for every cached token of a
 // single-token pass (llama.cpp:248-257), i.e. t = dot * scale.
 #define ATT_TCH 8
 __global__ __launch_bounds__(256) void attn_scores_kernel(const dev_state *st, const uint16_t *__restrict__ q16, const uint16_t *__restrict__ kc,
@@ -156,82 +164,102 @@ __global__ __launch_bounds__(256) void attn_scores_kernel(const dev_state *st, c
     const int t0 = blockIdx.x * ATT_TCH;
     if (t0 >= n_kv) return;
     const int d = n_head * 128;
-    const int piece = threadIdx.x & 15, hsel = threadIdx.x >> 4;     // 16 heads per pass over the workgroup
-    for (int h0 = 0; h0 < n_head; h0 += 16) {
-        const int head = h0 + hsel;
-        const bool hok = head < n_head;
-        float qf[8];
-        {
-            const uint4 qv = hok ? *(const uint4 *)(q16 + head * 128 + piece * 8) : make_uint4(0, 0, 0, 0);
-            const uint32_t qw[4] = {qv.x, qv.y, qv.z, qv.w};
+    const int piece = threadIdx.x & 15, hsel = threadIdx.x >> 4;     // 2 x 16 heads per pass over the workgroup
+    for (int h0 = 0; h0 < n_head; h0 += 32) {
+        uint4 kv[2][ATT_TCH];
+        uint4 qv[2];
+#pragma unroll
+        for (int hh = 0; hh < 2; hh++) {
+            const int head = h0 + hsel + 16 * hh;
+            if (head < n_head) {
+#pragma unroll
+                for (int tt = 0; tt < ATT_TCH; tt++)
+                    if (t0 + tt < n_kv) kv[hh][tt] = *(const uint4 *)(kc + (size_t)(t0 + tt) * d + head * 128 + piece * 8);
+                qv[hh] = *(const uint4 *)(q16 + head * 128 + piece * 8);
+            }
+        }
+#pragma unroll
+        for (int hh = 0; hh < 2; hh++) {
+            const int head = h0 + hsel + 16 * hh;
+            const bool hok = head < n_head;
+            float qf[8];
+            const uint32_t qw[4] = {qv[hh].x, qv[hh].y, qv[hh].z, qv[hh].w};
 #pragma unroll
             for (int j = 0; j < 4; j++) { qf[2 * j] = h2f((uint16_t)(qw[j] & 0xFFFFu)); qf[2 * j + 1] = h2f((uint16_t)(qw[j] >> 16)); }
-        }
-        uint4 kv[ATT_TCH];
 #pragma unroll
-        for (int tt = 0; tt < ATT_TCH; tt++)
-            if (hok && t0 + tt < n_kv) kv[tt] = *(const uint4 *)(kc + (size_t)(t0 + tt) * d + head * 128 + piece * 8);
+            for (int tt = 0; tt < ATT_TCH; tt++) {
+                float s = 0.0f;
+                if (hok && t0 + tt < n_kv) {
+                    const uint32_t kw[4] = {kv[hh][tt].x, kv[hh][tt].y, kv[hh][tt].z, kv[hh][tt].w};
 #pragma unroll
-        for (int tt = 0; tt < ATT_TCH; tt++) {
-            float s = 0.0f;
-            if (hok && t0 + tt < n_kv) {
-                const uint32_t kw[4] = {kv[tt].x, kv[tt].y, kv[tt].z, kv[tt].w};
-#pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    s = fmaf(h2f((uint16_t)(kw[j] & 0xFFFFu)), qf[2 * j], s);
-                    s = fmaf(h2f((uint16_t)(kw[j] >> 16)), qf[2 * j + 1], s);
+                    for (int j = 0; j < 4; j++) {
+                        s = fmaf(h2f((uint16_t)(kw[j] & 0xFFFFu)), qf[2 * j], s);
+                        s = fmaf(h2f((uint16_t)(kw[j] >> 16)), qf[2 * j + 1], s);
+                    }
                 }
+                s = group_sum<16>(s);
+                if (hok && piece == 0 && t0 + tt < n_kv) scores[(size_t)head * n_ctx + t0 + tt] = s * scale;
             }
-            s = group_sum<16>(s);
-            if (hok && piece == 0 && t0 + tt < n_kv) scores[(size_t)head * n_ctx + t0 + tt] = s * scale;
         }
     }
 }
 
 // ---- softmax + P.V ------------------------------------------------------------------------------
-// One workgroup per (head, 16 head dims).  The softmax of the head's row is recomputed by each of
-// the 8 workgroups of a head (n_kv expf per workgroup): m = max t; e = expf(float(fp16(t - m)));
-// p = e * (1/sum e) (non-linear.cpp:158-176); P is rounded to fp16 for the KQV product
-// (mat.cpp:37, vec_dot.h:117-146).  V^T rows are contiguous along tokens: 16 lanes x 128-bit.
-__global__ __launch_bounds__(256) void attn_pv_kernel(const dev_state *st, const float *__restrict__ scores, const uint16_t *__restrict__ vc,
-                                                      float *__restrict__ attn_out, int n_ctx) {
+// One 1024-thread workgroup per (head, 16 head dims): wave w owns V^T row head*128 + dgrp*16 + w,
+// contiguous along tokens, 64 lanes x 128-bit per step; the first PV_PIECES steps of the row are
+// put in flight before the softmax so that the HBM latency hides behind it.  The softmax of the
+// head's row is recomputed by each of the 8 workgroups of a head: m = max t;
+// e = expf(float(fp16(t - m))); p = e * (1/sum e) (non-linear.cpp:158-176); P is rounded to fp16 for the
+// KQV product (mat.cpp:37, vec_dot.h:117-146).
+#define PV_THREADS 1024
+#define PV_PIECES 10            // 128-bit pieces per lane per chunk: 10*64*8 = 5120 tokens per chunk
+__global__ __launch_bounds__(PV_THREADS) void attn_pv_kernel(const dev_state *st, const float *__restrict__ scores, const uint16_t *__restrict__ vc,
+                                                             float *__restrict__ attn_out, int n_ctx) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    __shared__ float s_part[4];
+    __shared__ float s_part[16];
     const int n_kv = st->pos + 1;
     const int head = blockIdx.x >> 3, dgrp = blockIdx.x & 7;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int row = head * 128 + dgrp * 16 + wave;
+    const uint16_t *vrow = vc + (size_t)row * n_ctx;
+    const int n_pad = (n_kv + 7) & ~7, npiece = n_pad >> 3;
+    uint4 vv[PV_PIECES];
+#pragma unroll
+    for (int u = 0; u < PV_PIECES; u++) { const int pc = u * 64 + lane; if (pc < npiece) vv[u] = *(const uint4 *)(vrow + pc * 8); }
+
     float *s_t = (float *)smem;                               // n_ctx floats
     uint16_t *s_p = (uint16_t *)(smem + (size_t)n_ctx * 4);    // n_ctx halfs (+ pad)
     const float *srow = scores + (size_t)head * n_ctx;
     float mx = -INFINITY;
-    for (int j = threadIdx.x; j < n_kv; j += 256) { const float t = srow[j]; s_t[j] = t; mx = fmaxf(mx, t); }
+    for (int j = threadIdx.x; j < n_kv; j += PV_THREADS) { const float t = srow[j]; s_t[j] = t; mx = fmaxf(mx, t); }
     mx = wave_max(mx);
-    if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = mx;
+    if (lane == 0) s_part[wave] = mx;
     __syncthreads();
-    mx = fmaxf(fmaxf(s_part[0], s_part[1]), fmaxf(s_part[2], s_part[3]));
+    mx = s_part[0];
+#pragma unroll
+    for (int w = 1; w < 16; w++) mx = fmaxf(mx, s_part[w]);
     __syncthreads();
     float sum = 0.0f;
-    for (int j = threadIdx.x; j < n_kv; j += 256) { const float e = expf(h2f(f2h(s_t[j] - mx))); s_t[j] = e; sum += e; }
-    sum = wave_sum(sum);
-    if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = sum;
+    for (int j = threadIdx.x; j < n_kv; j += PV_THREADS) { const float e = expf(h2f(f2h(s_t[j] - mx))); s_t[j] = e; sum += e; }
+    sum = group_sum<64>(sum);
+    if (lane == 0) s_part[wave] = sum;
     __syncthreads();
-    sum = (s_part[0] + s_part[1]) + (s_part[2] + s_part[3]);
+    sum = 0.0f;
+#pragma unroll
+    for (int w = 0; w < 16; w++) sum += s_part[w];
     const float inv = 1.0f / sum;
-    const int n_pad = (n_kv + 7) & ~7;
-    for (int j = threadIdx.x; j < n_pad; j += 256) s_p[j] = j < n_kv ? f2h(s_t[j] * inv) : (uint16_t)0;
+    for (int j = threadIdx.x; j < n_pad; j += PV_THREADS) s_p[j] = j < n_kv ? f2h(s_t[j] * inv) : (uint16_t)0;
     __syncthreads();
 
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l = lane & 15, g = lane >> 4;
-    const int row = head * 128 + dgrp * 16 + wave * 4 + g;
-    const uint16_t *vrow = vc + (size_t)row * n_ctx;
-    const int npiece = n_pad >> 3;
     float acc = 0.0f;
-    for (int pc0 = 0; pc0 < npiece; pc0 += 64) {
-        uint4 vv[4];
+    for (int pc0 = 0; pc0 < npiece; pc0 += PV_PIECES * 64) {
+        if (pc0 > 0) {
 #pragma unroll
-        for (int u = 0; u < 4; u++) { const int pc = pc0 + u * 16 + l; if (pc < npiece) vv[u] = *(const uint4 *)(vrow + pc * 8); }
+            for (int u = 0; u < PV_PIECES; u++) { const int pc = pc0 + u * 64 + lane; if (pc < npiece) vv[u] = *(const uint4 *)(vrow + pc * 8); }
+        }
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
-            const int pc = pc0 + u * 16 + l;
+        for (int u = 0; u < PV_PIECES; u++) {
+            const int pc = pc0 + u * 64 + lane;
             if (pc < npiece) {
                 const uint4 pp = *(const uint4 *)(s_p + pc * 8);
                 const uint32_t vw[4] = {vv[u].x, vv[u].y, vv[u].z, vv[u].w}, pw[4] = {pp.x, pp.y, pp.z, pp.w};
@@ -244,8 +272,8 @@ __global__ __launch_bounds__(256) void attn_pv_kernel(const dev_state *st, const
             }
         }
     }
-    acc = group_sum<16>(acc);
-    if (l == 0) attn_out[row] = acc;
+    acc = group_sum<64>(acc);
+    if (lane == 0) attn_out[row] = acc;
 }
 
 // ---- greedy sampling + loop advance -------------------------------------------------------------
@@ -279,3 +307,5 @@ __global__ __launch_bounds__(1024) void sample_advance_kernel(dev_state *st, con
         st->step = step + 1;
     }
 }
+
+#endif  // SPY_DECODE_COMMON_KERNELS

@@ -1,0 +1,110 @@
+// Launchers of the fused single-token-pass kernels, templated on the layer-weight type; included by
+// one translation unit per type.
+#pragma once
+
+#include "engine_types.cuh"
+
+#include <math.h>
+#include <string.h>
+
+template <int WT, int LPR, int NIT, int SIT, int EPI>
+static int launch_fused(spy_hip_llama *m, hipStream_t st, const fused_args &a) {
+    constexpr int RPT = GEMV_WAVES * (SPY_WAVE / LPR);
+    static int cap = 0;                                   // workgroups resident at once (persistent grid)
+    const size_t lds = staged_bytes(a.K);
+    auto kern = fused_gemv_kernel<WT, LPR, NIT, SIT, EPI>;
+    if (!cap) {
+        if (lds > 48 * 1024) HIP_TRY(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        int per_cu = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, GEMV_THREADS, lds) != hipSuccess || per_cu < 1) per_cu = 1;
+        cap = per_cu * m->num_cu;
+    }
+    if (m->dry) return 0;
+    const int ntiles = (a.M + RPT - 1) / RPT;
+    kern<<<dim3((unsigned)(ntiles < cap ? ntiles : cap)), dim3(GEMV_THREADS), lds, st>>>(a);
+    return SPY_LAUNCH_RC();
+}
+
+// RMSNorm-prologue kernels (K = n_embd): x and the norm weight stay in registers, 4 or 8 float4 each
+template <int WT, int EPI>
+static int launch_fused_norm(spy_hip_llama *m, hipStream_t st, gemv_cfg cfg, const fused_args &a) {
+    int rc = SPY_HIP_EUNSUPPORTED;
+    const bool big = a.K > 4096;
+    if (a.K > 8192) return rc;
+#define CALL(LPR, NIT) rc = big ? launch_fused<WT, LPR, NIT, 8, EPI>(m, st, a) : launch_fused<WT, LPR, NIT, 4, EPI>(m, st, a)
+    switch (cfg.lpr * 8 + cfg.nit) {
+    case 16 * 8 + 1: CALL(16, 1); break; case 16 * 8 + 2: CALL(16, 2); break;
+    case 16 * 8 + 3: CALL(16, 3); break; case 16 * 8 + 4: CALL(16, 4); break;
+    case 32 * 8 + 3: CALL(32, 3); break; case 32 * 8 + 4: CALL(32, 4); break;
+    default: break;
+    }
+#undef CALL
+    return rc;
+}
+
+template <int WT>
+static int launch_fused_resid(spy_hip_llama *m, hipStream_t st, gemv_cfg cfg, const fused_args &a) {
+    int rc = SPY_HIP_EUNSUPPORTED;
+#define CALL(LPR, NIT) rc = launch_fused<WT, LPR, NIT, 0, EPI_RESID>(m, st, a)
+    GEMV_DISPATCH_CFG(cfg, CALL)
+#undef CALL
+    return rc;
+}
+
+// one kernel of layer il of the single-token pass
+template <int WT>
+static int enqueue_kernel(spy_hip_llama *m, hipStream_t st, int which, int il) {
+    const spy_hip_llama_desc &c = m->desc;
+    const int d = c.n_embd, F = c.n_ff, C = c.n_ctx;
+    const spy_hip_llama_layer &L = m->layers[il];
+    fused_args a;
+    memset(&a, 0, sizeof(a));
+    a.st = m->st; a.rope_cs = m->rope_cs; a.q16 = m->q16; a.kc = m->k_cache[il]; a.vc = m->v_cache[il];
+    a.n_ctx = C; a.d = d; a.hd = m->hd; a.eps = c.eps;
+    switch (which) {
+    case K_QKV:      // attn_norm, attn_norm_linear, Q/K/V_project, rope, KV-cache copies
+        a.W0 = (const uint8_t *)L.wq; a.W1 = (const uint8_t *)L.wk; a.W2 = (const uint8_t *)L.wv;
+        a.M = 3 * d; a.K = d; a.x_in = m->x; a.normw = L.attn_norm;
+        return launch_fused_norm<WT, EPI_QKV>(m, st, m->cfg_d, a);
+    case K_WO:       // KQV_linear + ffn_input
+        a.W0 = (const uint8_t *)L.wo; a.M = d; a.K = d; a.x_in = m->attn_out; a.resid = m->x; a.out = m->x1;
+        return launch_fused_resid<WT>(m, st, m->cfg_d, a);
+    case K_GATEUP:   // ffn_norm, ffn_up, ffn_gate, silu, ffn_par
+        a.W0 = (const uint8_t *)L.w_gate; a.W1 = (const uint8_t *)L.w_up; a.M = 2 * F; a.K = d; a.x_in = m->x1; a.normw = L.ffn_norm; a.out = m->hbuf;
+        return launch_fused_norm<WT, EPI_GATEUP>(m, st, m->cfg_d, a);
+    case K_DOWN:     // ffn_down + logit_output (the next layer's input)
+        a.W0 = (const uint8_t *)L.w_down; a.M = d; a.K = F; a.x_in = m->hbuf; a.resid = m->x1; a.out = m->x;
+        return launch_fused_resid<WT>(m, st, m->cfg_ff, a);
+    }
+    return SPY_HIP_EINVAL;
+}
+
+// result_norm, result_linear, output
+template <int WT>
+static int enqueue_head(spy_hip_llama *m, hipStream_t st) {
+    const spy_hip_llama_desc &c = m->desc;
+    const int d = c.n_embd;
+    if (c.t_out == c.wtype) {
+        fused_args a;
+        memset(&a, 0, sizeof(a));
+        a.W0 = (const uint8_t *)c.w_out; a.M = c.n_vocab; a.K = d; a.x_in = m->x; a.normw = c.out_norm; a.eps = c.eps; a.out = m->logits;
+        return launch_fused_norm<WT, EPI_STORE>(m, st, m->cfg_d, a);
+    }
+    // head in another type (e.g. Q6_K): norm + weight + Q8_0 through the operator kernels
+    if (m->dry) return 0;
+    spy_hip_tensor tx, tw, txn;
+    memset(&tx, 0, sizeof(tx));
+    tx.type = SPY_HIP_F32; tx.dim = 1; tx.ne[0] = d; tx.ne[1] = tx.ne[2] = tx.ne[3] = 1; tx.nb[0] = 4; tx.nb[1] = tx.nb[2] = tx.nb[3] = 4 * d;
+    tw = tx; txn = tx;
+    tx.data = m->x; tw.data = (void *)c.out_norm; txn.data = m->x1;
+    RC_TRY(spy_hip_op_norm_rms(st, &tx, &txn, c.eps));
+    RC_TRY(spy_hip_op_binary(st, 2, &txn, &tw, &txn));
+    RC_TRY(spy_hip_quantize_q8_0(st, m->x1, 4 * d, m->xq_head, 1, d));
+    return spy_hip_gemv_q8_0act(st, c.t_out, c.w_out, m->xq_head, m->logits, nullptr, c.n_vocab, d, 1, c.n_vocab);
+}
+
+
+template <int WT>
+static int enqueue_any(spy_hip_llama *m, hipStream_t st, int which, int il) {
+    return which == K_HEAD ? enqueue_head<WT>(m, st) : enqueue_kernel<WT>(m, st, which, il);
+}

@@ -4,39 +4,17 @@
 // whole pass captured once as a HIP graph and replayed per token.  Passes over several tokens
 // (prompts) run operator by operator through the spy_hip_op_* entry points, exactly as the graph
 // lists them.
-#include "decode_kernels.cuh"
+#define SPY_DECODE_COMMON_KERNELS
+#include "engine_types.cuh"
 
 #include <math.h>
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
-#include <vector>
 
-#define HIP_TRY(x) do { hipError_t e_ = (x); if (e_ != hipSuccess) return (int)e_; } while (0)
-#define RC_TRY(x) do { int rc_ = (x); if (rc_) return rc_; } while (0)
 
-struct spy_hip_llama {
-    spy_hip_llama_desc desc;
-    std::vector<spy_hip_llama_layer> layers;
-    int hd = 0, lpr_d = 0, lpr_ff = 0;
-    std::vector<uint16_t *> k_cache, v_cache;
-    float *x = nullptr, *x1 = nullptr, *attn_out = nullptr, *hbuf = nullptr, *scores = nullptr, *logits = nullptr, *rope_cs = nullptr;
-    uint16_t *q16 = nullptr;
-    uint8_t *xq_head = nullptr;          // native Q8_0 activations for a K-quant output head
-    dev_state *st = nullptr;
-    int32_t *tokens_out = nullptr;
-    int max_out = 0;
-    int num_cu = 256;
-    float theta_scale = 0.0f;
-    // op-by-op path scratch (sized lazily for the largest chunk seen)
-    uint8_t *ops_buf = nullptr; size_t ops_bytes = 0;
-    // graph of one single-token pass
-    hipGraph_t graph = nullptr; hipGraphExec_t graph_exec = nullptr; hipStream_t graph_stream = nullptr;
-    hipStream_t own_stream = nullptr;
-    hipEvent_t ev0 = nullptr, ev1 = nullptr;
-    double timed_ms = 0.0; int timed_pass = 0;
-    std::vector<void *> owned;
-};
+static bool fused_ok(const spy_hip_llama *m);
+static int enqueue_pass_any(spy_hip_llama *m, hipStream_t st, bool sample);
 
 static int dalloc(spy_hip_llama *m, void **p, size_t bytes, bool zero) {
     HIP_TRY(hipMalloc(p, bytes));
@@ -79,8 +57,8 @@ extern "C" int spy_hip_llama_create(const spy_hip_llama_desc *desc, spy_hip_llam
         const spy_hip_llama_layer &L = m->layers[i];
         if (!L.attn_norm || !L.ffn_norm || !L.wq || !L.wk || !L.wv || !L.wo || !L.w_gate || !L.w_up || !L.w_down) { delete m; return SPY_HIP_EINVAL; }
     }
-    m->lpr_d  = c.wtype == SPY_HIP_Q4_0 ? pick_lpr<SPY_HIP_Q4_0>(c.n_embd) : pick_lpr<SPY_HIP_Q8_0>(c.n_embd);
-    m->lpr_ff = c.wtype == SPY_HIP_Q4_0 ? pick_lpr<SPY_HIP_Q4_0>(c.n_ff) : pick_lpr<SPY_HIP_Q8_0>(c.n_ff);
+    m->cfg_d  = pick_cfg(c.n_embd, 32);
+    m->cfg_ff = pick_cfg(c.n_ff);
     {
         int dev = 0; hipDeviceProp_t prop;
         if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0) m->num_cu = prop.multiProcessorCount;
@@ -113,6 +91,7 @@ extern "C" int spy_hip_llama_create(const spy_hip_llama_desc *desc, spy_hip_llam
         if (!rc && pv_lds > 160 * 1024) rc = SPY_HIP_EUNSUPPORTED;
         if (!rc && pv_lds > 48 * 1024) rc = (int)hipFuncSetAttribute((const void *)attn_pv_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)pv_lds);
     }
+    if (!rc && fused_ok(m)) { m->dry = true; rc = enqueue_pass_any(m, m->own_stream, true); m->dry = false; }   // sizes the persistent grids
     if (rc) { spy_hip_llama_destroy(m); return rc; }
     *out = m;
     return 0;
@@ -143,114 +122,45 @@ extern "C" int spy_hip_llama_timing(spy_hip_llama *m, float *ms_per_pass, int32_
     return 0;
 }
 
-// ---- the fused single-token pass -----------------------------------------------------------------
-template <int WT, int LPR, bool NORM, int EPI>
-static int launch_fused(spy_hip_llama *m, hipStream_t st, const fused_args &a) {
-    constexpr int RPT = GEMV_WAVES * (SPY_WAVE / LPR);
-    const size_t lds = staged_bytes(a.K);
-    auto kern = fused_gemv_kernel<WT, LPR, NORM, EPI>;
-    if (lds > 48 * 1024) HIP_TRY(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    const int ntiles = (a.M + RPT - 1) / RPT;
-    const int cap = 4 * m->num_cu;
-    kern<<<dim3((unsigned)(ntiles < cap ? ntiles : cap)), dim3(GEMV_THREADS), lds, st>>>(a);
-    return SPY_LAUNCH_RC();
-}
-
-template <int WT, bool NORM, int EPI>
-static int launch_fused_lpr(spy_hip_llama *m, hipStream_t st, int lpr, const fused_args &a) {
-    switch (lpr) {
-    case 16: return launch_fused<WT, 16, NORM, EPI>(m, st, a);
-    case 32: return launch_fused<WT, 32, NORM, EPI>(m, st, a);
-    case 64: if constexpr (EPI == EPI_RESID || EPI == EPI_STORE) return launch_fused<WT, 64, NORM, EPI>(m, st, a); else break;
-    }
-    return SPY_HIP_EUNSUPPORTED;
-}
-
 static bool fused_ok(const spy_hip_llama *m) {
-    // the fused kernels assume 128-wide heads (one key = 16 lanes x 128 bit) and row pairs that
-    // share a wave in the qkv / gate-up epilogues
-    return m->hd == 128 && (m->lpr_d == 16 || m->lpr_d == 32) && m->lpr_ff != 0 && m->desc.n_embd % 4 == 0;
+    // the fused kernels assume 128-wide heads (one key = 16 lanes x 128 bit), row pairs that share a
+    // wave in the qkv / gate-up epilogues (<= 32 lanes per row) and n_embd <= 8192
+    return m->hd == 128 && (m->cfg_d.lpr == 16 || m->cfg_d.lpr == 32) && m->cfg_ff.lpr != 0 && m->desc.n_embd % 4 == 0 && m->desc.n_embd <= 8192;
 }
 
-enum { K_QKV = 0, K_SCORES, K_PV, K_WO, K_GATEUP, K_DOWN, K_HEAD, K_COUNT };
-
-// one kernel of layer il of the single-token pass
-template <int WT>
-static int enqueue_kernel(spy_hip_llama *m, hipStream_t st, int which, int il) {
+static int enqueue_one(spy_hip_llama *m, hipStream_t st, int which, int il) {
     const spy_hip_llama_desc &c = m->desc;
-    const int d = c.n_embd, F = c.n_ff, C = c.n_ctx, H = c.n_head;
-    const float scale = 1.0f / sqrtf((float)m->hd);                     // SoftmaxParam::scale (attention.cpp:113)
-    const size_t pv_lds = (size_t)C * 4 + (size_t)C * 2 + 16;
-    const spy_hip_llama_layer &L = m->layers[il];
-    fused_args a;
-    memset(&a, 0, sizeof(a));
-    a.st = m->st; a.rope_cs = m->rope_cs; a.q16 = m->q16; a.kc = m->k_cache[il]; a.vc = m->v_cache[il];
-    a.n_ctx = C; a.d = d; a.hd = m->hd; a.eps = c.eps;
-    switch (which) {
-    case K_QKV:      // attn_norm, attn_norm_linear, Q/K/V_project, rope, KV-cache copies
-        a.W0 = (const uint8_t *)L.wq; a.W1 = (const uint8_t *)L.wk; a.W2 = (const uint8_t *)L.wv;
-        a.M = 3 * d; a.K = d; a.x_in = m->x; a.normw = L.attn_norm;
-        return launch_fused_lpr<WT, true, EPI_QKV>(m, st, m->lpr_d, a);
-    case K_SCORES:   // attn_score
-        attn_scores_kernel<<<dim3((unsigned)((C + ATT_TCH - 1) / ATT_TCH)), dim3(256), 0, st>>>(m->st, m->q16, m->k_cache[il], m->scores, H, C, scale);
+    if (which == K_SCORES) {            // attn_score
+        if (m->dry) return 0;
+        const float scale = 1.0f / sqrtf((float)m->hd);                     // SoftmaxParam::scale (attention.cpp:113)
+        attn_scores_kernel<<<dim3((unsigned)((c.n_ctx + ATT_TCH - 1) / ATT_TCH)), dim3(256), 0, st>>>(m->st, m->q16, m->k_cache[il], m->scores,
+                                                                                                      c.n_head, c.n_ctx, scale);
         return SPY_LAUNCH_RC();
-    case K_PV:       // softmax, KQV (+ permute/contiguous: attn_out is already [hd, H] contiguous)
-        attn_pv_kernel<<<dim3((unsigned)(H * 8)), dim3(256), pv_lds, st>>>(m->st, m->scores, m->v_cache[il], m->attn_out, C);
+    }
+    if (which == K_PV) {                // softmax, KQV (+ permute/contiguous: attn_out is already [hd, H] contiguous)
+        if (m->dry) return 0;
+        const size_t pv_lds = (size_t)c.n_ctx * 4 + (size_t)c.n_ctx * 2 + 16;
+        attn_pv_kernel<<<dim3((unsigned)(c.n_head * 8)), dim3(PV_THREADS), pv_lds, st>>>(m->st, m->scores, m->v_cache[il], m->attn_out, c.n_ctx);
         return SPY_LAUNCH_RC();
-    case K_WO:       // KQV_linear + ffn_input
-        a.W0 = (const uint8_t *)L.wo; a.M = d; a.K = d; a.x_in = m->attn_out; a.resid = m->x; a.out = m->x1;
-        return launch_fused_lpr<WT, false, EPI_RESID>(m, st, m->lpr_d, a);
-    case K_GATEUP:   // ffn_norm, ffn_up, ffn_gate, silu, ffn_par
-        a.W0 = (const uint8_t *)L.w_gate; a.W1 = (const uint8_t *)L.w_up; a.M = 2 * F; a.K = d; a.x_in = m->x1; a.normw = L.ffn_norm; a.out = m->hbuf;
-        return launch_fused_lpr<WT, true, EPI_GATEUP>(m, st, m->lpr_d, a);
-    case K_DOWN:     // ffn_down + logit_output (the next layer's input)
-        a.W0 = (const uint8_t *)L.w_down; a.M = d; a.K = F; a.x_in = m->hbuf; a.resid = m->x1; a.out = m->x;
-        return launch_fused_lpr<WT, false, EPI_RESID>(m, st, m->lpr_ff, a);
     }
-    return SPY_HIP_EINVAL;
+    return m->desc.wtype == SPY_HIP_Q4_0 ? spy_enqueue_kernel_q4_0(m, st, which, il) : spy_enqueue_kernel_q8_0(m, st, which, il);
 }
 
-// result_norm, result_linear, output
-template <int WT>
-static int enqueue_head(spy_hip_llama *m, hipStream_t st) {
+static int enqueue_pass_any(spy_hip_llama *m, hipStream_t st, bool sample) {
     const spy_hip_llama_desc &c = m->desc;
-    const int d = c.n_embd;
-    if (c.t_out == c.wtype) {
-        fused_args a;
-        memset(&a, 0, sizeof(a));
-        a.W0 = (const uint8_t *)c.w_out; a.M = c.n_vocab; a.K = d; a.x_in = m->x; a.normw = c.out_norm; a.eps = c.eps; a.out = m->logits;
-        return launch_fused_lpr<WT, true, EPI_STORE>(m, st, m->lpr_d, a);
+    if (!m->dry) {
+        embed_kernel<<<dim3(1), dim3(256), 0, st>>>(m->st, (const uint8_t *)c.tok_embd, c.t_tok_embd == SPY_HIP_Q8_0, c.n_embd, c.n_vocab, m->x,
+                                                    m->rope_cs, m->theta_scale, m->hd);
+        RC_TRY(SPY_LAUNCH_RC());
     }
-    // head in another type (e.g. Q6_K): norm + weight + Q8_0 through the operator kernels
-    spy_hip_tensor tx, tw, txn;
-    memset(&tx, 0, sizeof(tx));
-    tx.type = SPY_HIP_F32; tx.dim = 1; tx.ne[0] = d; tx.ne[1] = tx.ne[2] = tx.ne[3] = 1; tx.nb[0] = 4; tx.nb[1] = tx.nb[2] = tx.nb[3] = 4 * d;
-    tw = tx; txn = tx;
-    tx.data = m->x; tw.data = (void *)c.out_norm; txn.data = m->x1;
-    RC_TRY(spy_hip_op_norm_rms(st, &tx, &txn, c.eps));
-    RC_TRY(spy_hip_op_binary(st, 2, &txn, &tw, &txn));
-    RC_TRY(spy_hip_quantize_q8_0(st, m->x1, 4 * d, m->xq_head, 1, d));
-    return spy_hip_gemv_q8_0act(st, c.t_out, c.w_out, m->xq_head, m->logits, nullptr, c.n_vocab, d, 1, c.n_vocab);
-}
-
-template <int WT>
-static int enqueue_pass(spy_hip_llama *m, hipStream_t st, bool sample) {
-    const spy_hip_llama_desc &c = m->desc;
-    embed_kernel<<<dim3(1), dim3(256), 0, st>>>(m->st, (const uint8_t *)c.tok_embd, c.t_tok_embd == SPY_HIP_Q8_0, c.n_embd, c.n_vocab, m->x,
-                                                m->rope_cs, m->theta_scale, m->hd);
-    RC_TRY(SPY_LAUNCH_RC());
     for (int il = 0; il < c.n_layer; il++)
-        for (int k = K_QKV; k <= K_DOWN; k++) RC_TRY(enqueue_kernel<WT>(m, st, k, il));
-    RC_TRY(enqueue_head<WT>(m, st));
-    if (sample) {
+        for (int k = K_QKV; k <= K_DOWN; k++) RC_TRY(enqueue_one(m, st, k, il));
+    RC_TRY(enqueue_one(m, st, K_HEAD, 0));
+    if (sample && !m->dry) {
         sample_advance_kernel<<<dim3(1), dim3(1024), 0, st>>>(m->st, m->logits, c.n_vocab, m->tokens_out, m->max_out);
         RC_TRY(SPY_LAUNCH_RC());
     }
     return 0;
-}
-
-static int enqueue_pass_any(spy_hip_llama *m, hipStream_t st, bool sample) {
-    return m->desc.wtype == SPY_HIP_Q4_0 ? enqueue_pass<SPY_HIP_Q4_0>(m, st, sample) : enqueue_pass<SPY_HIP_Q8_0>(m, st, sample);
 }
 
 // ---- passes over several tokens: operator by operator --------------------------------------------
@@ -447,9 +357,7 @@ extern "C" int spy_hip_llama_kernel_time(spy_hip_llama *m, void *stream, const c
     for (int i = 0; i < K_COUNT; i++) if (!strcmp(which, names[i])) k = i;
     SPY_CHECK_ARG(k >= 0);
     hipStream_t st = stream ? (hipStream_t)stream : m->own_stream;
-    const bool q4 = m->desc.wtype == SPY_HIP_Q4_0;
-    auto once = [&](int il) { return k == K_HEAD ? (q4 ? enqueue_head<SPY_HIP_Q4_0>(m, st) : enqueue_head<SPY_HIP_Q8_0>(m, st))
-                                                 : (q4 ? enqueue_kernel<SPY_HIP_Q4_0>(m, st, k, il) : enqueue_kernel<SPY_HIP_Q8_0>(m, st, k, il)); };
+    auto once = [&](int il) { return enqueue_one(m, st, k, il); };
     for (int il = 0; il < m->desc.n_layer; il++) RC_TRY(once(il));           // warm-up
     HIP_TRY(hipEventRecord(m->ev0, st));
     for (int r = 0; r < reps; r++)

@@ -1,0 +1,4 @@
+// Single-token-pass kernels instantiated for Q8_0 layer weights.
+#include "decode_launch.cuh"
+
+int spy_enqueue_kernel_q8_0(spy_hip_llama *m, hipStream_t st, int which, int il) { return enqueue_any<SPY_HIP_Q8_0>(m, st, which, il); }

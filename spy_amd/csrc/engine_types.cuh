@@ -1,0 +1,42 @@
+// Shared declarations of the token-loop engine (state, per-kernel launch entry points).
+#pragma once
+
+#include "decode_kernels.cuh"
+
+#include <vector>
+
+#define HIP_TRY(x) do { hipError_t e_ = (x); if (e_ != hipSuccess) return (int)e_; } while (0)
+#define RC_TRY(x) do { int rc_ = (x); if (rc_) return rc_; } while (0)
+
+struct spy_hip_llama {
+    spy_hip_llama_desc desc;
+    std::vector<spy_hip_llama_layer> layers;
+    int hd = 0;
+    gemv_cfg cfg_d = {0, 0}, cfg_ff = {0, 0};   // lanes-per-row / pairs-per-lane for K = n_embd and K = n_ff
+    bool dry = false;
+    std::vector<uint16_t *> k_cache, v_cache;
+    float *x = nullptr, *x1 = nullptr, *attn_out = nullptr, *hbuf = nullptr, *scores = nullptr, *logits = nullptr, *rope_cs = nullptr;
+    uint16_t *q16 = nullptr;
+    uint8_t *xq_head = nullptr;          // native Q8_0 activations for a K-quant output head
+    dev_state *st = nullptr;
+    int32_t *tokens_out = nullptr;
+    int max_out = 0;
+    int num_cu = 256;
+    float theta_scale = 0.0f;
+    // op-by-op path scratch (sized lazily for the largest chunk seen)
+    uint8_t *ops_buf = nullptr; size_t ops_bytes = 0;
+    // graph of one single-token pass
+    hipGraph_t graph = nullptr; hipGraphExec_t graph_exec = nullptr; hipStream_t graph_stream = nullptr;
+    hipStream_t own_stream = nullptr;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    double timed_ms = 0.0; int timed_pass = 0;
+    std::vector<void *> owned;
+};
+
+
+enum { K_QKV = 0, K_SCORES, K_PV, K_WO, K_GATEUP, K_DOWN, K_HEAD, K_COUNT };
+
+// One kernel of layer il of the single-token pass (K_HEAD: il ignored), for each layer-weight type.
+// With m->dry set nothing is launched: the call only sizes the persistent grids.
+int spy_enqueue_kernel_q4_0(spy_hip_llama *m, hipStream_t st, int which, int il);
+int spy_enqueue_kernel_q8_0(spy_hip_llama *m, hipStream_t st, int which, int il);

@@ -18,21 +18,25 @@ struct gemv_args {
     int64_t dst_stride;
 };
 
-// Persistent workgroups: each strides over row tiles with the next tile's weights already in
-// flight (two register buffers) while the current one is reduced.
-template <int WT, int LPR, int NT, bool DUMP>
+// Persistent workgroups: each strides over row tiles, always with two tiles' weights in flight
+// (two register buffers).
+template <int WT, int LPR, int NIT, int NT, bool DUMP>
 __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(gemv_args a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     constexpr int RPW = SPY_WAVE / LPR, RPT = GEMV_WAVES * RPW;
-    const int K = a.K, nblk = K / 32, npair = K / 64, nit = (npair + LPR - 1) / LPR;
+    const int K = a.K, nblk = K / 32, npair = K / 64;
     const size_t RB = (size_t)nblk * wt_traits<WT>::BLK;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l = lane % LPR, g = lane / LPR;
     const int ntiles = (a.M + RPT - 1) / RPT, G = gridDim.x;
     const int rofs = wave * RPW + g;
 
-    wtile<WT> A, B;
+    wtile<WT, NIT> A, B;
     int tile = blockIdx.x;
-    if (tile < ntiles && tile * RPT + rofs < a.M) load_tile<WT, LPR>(A, a.W + (size_t)(tile * RPT + rofs) * RB, npair, nit, l);
+    auto fetch = [&](wtile<WT, NIT> &t, int tl) {
+        if (tl < ntiles && tl * RPT + rofs < a.M) load_tile<WT, LPR, NIT>(t, a.W + (size_t)(tl * RPT + rofs) * RB, npair, l);
+    };
+    fetch(A, tile);
+    fetch(B, tile + G);
 
     staged_act act[NT];
 #pragma unroll
@@ -43,12 +47,12 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(gemv_args a) {
         act[c].q = q; act[c].meta = meta;
     }
 
-    auto finish = [&](const wtile<WT> &t, int tl) {
+    auto finish = [&](const wtile<WT, NIT> &t, int tl) {
         const int r = tl * RPT + rofs;
         float acc[NT];
 #pragma unroll
         for (int c = 0; c < NT; c++) acc[c] = 0.0f;
-        if (r < a.M) dot_tile<WT, LPR, NT>(t, act, npair, nit, l, acc, DUMP ? a.dump + (size_t)r * nblk : nullptr);
+        if (r < a.M) dot_tile<WT, LPR, NIT, NT>(t, act, npair, l, acc, DUMP ? a.dump + (size_t)r * nblk : nullptr);
 #pragma unroll
         for (int c = 0; c < NT; c++) {
             const float s = group_sum<LPR>(acc[c]);
@@ -60,15 +64,13 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(gemv_args a) {
     };
 
     while (tile < ntiles) {
-        int tn = tile + G;
-        if (tn < ntiles && tn * RPT + rofs < a.M) load_tile<WT, LPR>(B, a.W + (size_t)(tn * RPT + rofs) * RB, npair, nit, l);
         finish(A, tile);
-        tile = tn;
+        fetch(A, tile + 2 * G);
+        tile += G;
         if (tile >= ntiles) break;
-        tn = tile + G;
-        if (tn < ntiles && tn * RPT + rofs < a.M) load_tile<WT, LPR>(A, a.W + (size_t)(tn * RPT + rofs) * RB, npair, nit, l);
         finish(B, tile);
-        tile = tn;
+        fetch(B, tile + 2 * G);
+        tile += G;
     }
 }
 
@@ -155,31 +157,38 @@ static int num_cu() {
     return g_num_cu;
 }
 
-template <int WT, int LPR, int NT, bool DUMP>
+// workgroups of `kern` that fit on the device at once (persistent kernels launch exactly that many)
+template <class Kern>
+static int resident_blocks(Kern kern, size_t lds) {
+    int per_cu = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, GEMV_THREADS, lds) != hipSuccess || per_cu < 1) per_cu = 1;
+    return per_cu * num_cu();
+}
+
+template <int WT, int LPR, int NIT, int NT, bool DUMP>
 static int launch_fast(hipStream_t st, const gemv_args &a) {
     constexpr int RPT = GEMV_WAVES * (SPY_WAVE / LPR);
     const size_t lds = (size_t)NT * staged_bytes(a.K);
     if (lds > 160 * 1024) return SPY_HIP_EUNSUPPORTED;
-    auto kern = gemv_kernel<WT, LPR, NT, DUMP>;
+    auto kern = gemv_kernel<WT, LPR, NIT, NT, DUMP>;
     if (lds > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return (int)e;
     }
     const int ntiles = (a.M + RPT - 1) / RPT;
-    const int cap = 4 * num_cu();
-    const unsigned grid = (unsigned)(ntiles < cap ? ntiles : cap);
-    kern<<<dim3(grid), dim3(GEMV_THREADS), lds, st>>>(a);
+    const int cap = resident_blocks(kern, lds);
+    kern<<<dim3((unsigned)(ntiles < cap ? ntiles : cap)), dim3(GEMV_THREADS), lds, st>>>(a);
     return SPY_LAUNCH_RC();
 }
 
 template <int WT, int NT, bool DUMP>
 static int launch_fast_lpr(hipStream_t st, const gemv_args &a) {
-    switch (pick_lpr<WT>(a.K)) {
-    case 16: return launch_fast<WT, 16, NT, DUMP>(st, a);
-    case 32: return launch_fast<WT, 32, NT, DUMP>(st, a);
-    case 64: return launch_fast<WT, 64, NT, DUMP>(st, a);
-    }
-    return SPY_HIP_EUNSUPPORTED;
+    const gemv_cfg cfg = pick_cfg(a.K);
+    int rc = SPY_HIP_EUNSUPPORTED;
+#define CALL(LPR, NIT) rc = launch_fast<WT, LPR, NIT, NT, DUMP>(st, a)
+    GEMV_DISPATCH_CFG(cfg, CALL)
+#undef CALL
+    return rc;
 }
 
 template <int WT, bool DUMP>
@@ -233,10 +242,10 @@ extern "C" int spy_hip_gemv_q8_0act(void *stream, int wtype, const void *w, cons
     hipStream_t st = (hipStream_t)stream;
     switch (wtype) {
     case SPY_HIP_Q4_0:
-        return pick_lpr<SPY_HIP_Q4_0>(K) ? gemv_fast_cols<SPY_HIP_Q4_0>(st, w, (const uint8_t *)xq, dst, residual, M, K, T, dst_stride)
+        return pick_cfg(K).lpr ? gemv_fast_cols<SPY_HIP_Q4_0>(st, w, (const uint8_t *)xq, dst, residual, M, K, T, dst_stride)
                                          : launch_generic<SPY_HIP_Q4_0, false>(st, w, xq, dst, residual, nullptr, M, K, T, dst_stride);
     case SPY_HIP_Q8_0:
-        return pick_lpr<SPY_HIP_Q8_0>(K) ? gemv_fast_cols<SPY_HIP_Q8_0>(st, w, (const uint8_t *)xq, dst, residual, M, K, T, dst_stride)
+        return pick_cfg(K).lpr ? gemv_fast_cols<SPY_HIP_Q8_0>(st, w, (const uint8_t *)xq, dst, residual, M, K, T, dst_stride)
                                          : launch_generic<SPY_HIP_Q8_0, false>(st, w, xq, dst, residual, nullptr, M, K, T, dst_stride);
     case SPY_HIP_Q4_K: return launch_generic<SPY_HIP_Q4_K, false>(st, w, xq, dst, residual, nullptr, M, K, T, dst_stride);
     case SPY_HIP_Q6_K: return launch_generic<SPY_HIP_Q6_K, false>(st, w, xq, dst, residual, nullptr, M, K, T, dst_stride);
@@ -258,10 +267,10 @@ extern "C" int spy_hip_block_dots(void *stream, int wtype, const void *w, const 
     a.M = (int)M; a.K = (int)K; a.dst_stride = M;
     switch (wtype) {
     case SPY_HIP_Q4_0:
-        return pick_lpr<SPY_HIP_Q4_0>(K) ? launch_fast_lpr<SPY_HIP_Q4_0, 1, true>(st, a)
+        return pick_cfg(K).lpr ? launch_fast_lpr<SPY_HIP_Q4_0, 1, true>(st, a)
                                          : launch_generic<SPY_HIP_Q4_0, true>(st, w, xq, sink, nullptr, out, M, K, 1, M);
     case SPY_HIP_Q8_0:
-        return pick_lpr<SPY_HIP_Q8_0>(K) ? launch_fast_lpr<SPY_HIP_Q8_0, 1, true>(st, a)
+        return pick_cfg(K).lpr ? launch_fast_lpr<SPY_HIP_Q8_0, 1, true>(st, a)
                                          : launch_generic<SPY_HIP_Q8_0, true>(st, w, xq, sink, nullptr, out, M, K, 1, M);
     case SPY_HIP_Q4_K: return launch_generic<SPY_HIP_Q4_K, true>(st, w, xq, sink, nullptr, out, M, K, 1, M);
     case SPY_HIP_Q6_K: return launch_generic<SPY_HIP_Q6_K, true>(st, w, xq, sink, nullptr, out, M, K, 1, M);

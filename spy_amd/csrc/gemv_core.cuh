@@ -18,8 +18,9 @@
 #define GEMV_WAVES 4
 
 template <int WT> struct wt_traits;
-template <> struct wt_traits<SPY_HIP_Q4_0> { static constexpr int BLK = 18, PAIR_DW = 9, NIT_MAX = 6; };
-template <> struct wt_traits<SPY_HIP_Q8_0> { static constexpr int BLK = 34, PAIR_DW = 17, NIT_MAX = 4; };
+template <> struct wt_traits<SPY_HIP_Q4_0> { static constexpr int BLK = 18, PAIR_DW = 9; };
+template <> struct wt_traits<SPY_HIP_Q8_0> { static constexpr int BLK = 34, PAIR_DW = 17; };
+#define GEMV_NIT_MAX 4        // block pairs per lane per row tile: 1..4 (exact value is a template parameter)
 
 template <int CTRL> static __device__ __forceinline__ float dpp_add(float v) {
     return v + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
@@ -99,52 +100,77 @@ static __device__ __forceinline__ uint32_t quantize_oct(const float4 v, int2 &me
     return (uint32_t)(q0 & 0xFF) | ((uint32_t)(q1 & 0xFF) << 8) | ((uint32_t)(q2 & 0xFF) << 16) | ((uint32_t)(q3 & 0xFF) << 24);
 }
 
-// f32 vector (optionally RMS-normalised and multiplied by `normw`) -> staged LDS form.
-// NormRMS as the reference: scale = 1/sqrt(sum(x^2)/K + eps), y = (x*scale)*w
-// (non-linear.cpp:216-219 and the separate Mul node, attention.cpp:274-282 in the Spy tree).
-// K % 32 == 0, x 16-byte aligned.  Ends with __syncthreads().
-template <bool NORM>
-static __device__ __forceinline__ void stage_f32(const float *__restrict__ x, const float *__restrict__ normw, float eps,
-                                                 int8_t *s_q, int2 *s_meta, int K, float *s_red) {
-    float scale = 1.0f;
-    if constexpr (NORM) {
-        float acc = 0.0f;
-        for (int i = threadIdx.x; i < K / 4; i += GEMV_THREADS) {
-            const float4 v = ((const float4 *)x)[i];
-            acc = fmaf(v.x, v.x, acc); acc = fmaf(v.y, v.y, acc); acc = fmaf(v.z, v.z, acc); acc = fmaf(v.w, v.w, acc);
-        }
-        acc = wave_sum(acc);
-        if ((threadIdx.x & 63) == 0) s_red[threadIdx.x >> 6] = acc;
-        __syncthreads();
-        const float sum = (s_red[0] + s_red[1]) + (s_red[2] + s_red[3]);
-        scale = 1.0f / sqrtf(sum / (float)K + eps);
-    }
-    // K/4 float4 groups; 8 consecutive lanes hold one block.  Trip count is uniform per octet.
+// f32 vector -> staged LDS form, one pass (no normalisation).  K % 32 == 0, x 16-byte aligned.
+// Ends with __syncthreads().
+static __device__ __forceinline__ void stage_f32_plain(const float *__restrict__ x, int8_t *s_q, int2 *s_meta, int K) {
+    // 8 consecutive lanes hold one 32-element block; the trip count is uniform per octet
     for (int i = threadIdx.x; i < K / 4; i += GEMV_THREADS) {
-        float4 v = ((const float4 *)x)[i];
-        if constexpr (NORM) {
-            const float4 w = ((const float4 *)normw)[i];
-            v.x = (v.x * scale) * w.x; v.y = (v.y * scale) * w.y; v.z = (v.z * scale) * w.z; v.w = (v.w * scale) * w.w;
-        }
         int2 meta;
-        const uint32_t q = quantize_oct(v, meta);
+        const uint32_t q = quantize_oct(((const float4 *)x)[i], meta);
         ((uint32_t *)s_q)[i] = q;
         if ((threadIdx.x & 7) == 0) s_meta[i >> 3] = meta;
     }
     __syncthreads();
 }
 
+// RMS-normalised, weighted f32 vector -> staged LDS form.  NormRMS as the reference:
+// scale = 1/sqrt(sum(x^2)/K + eps), y = (x*scale)*w (non-linear.cpp:216-219 and the separate Mul
+// node, attention.cpp:274-282 in the Spy tree).  Split in two so that a kernel can put the global
+// loads in flight first (load), do other work, and finish later; x and w stay in registers
+// (SIT float4 each per thread: K <= 1024*SIT).  finish ends with __syncthreads().
+template <int SIT> struct stage_regs { float4 x[SIT]; float4 w[SIT]; };
+
+template <int SIT>
+static __device__ __forceinline__ void stage_norm_load(stage_regs<SIT> &r, const float *__restrict__ x, const float *__restrict__ normw, int K) {
+#pragma unroll
+    for (int j = 0; j < SIT; j++) {
+        const int i = threadIdx.x + j * GEMV_THREADS;
+        if (i < K / 4) { r.x[j] = ((const float4 *)x)[i]; r.w[j] = ((const float4 *)normw)[i]; }
+    }
+}
+
+template <int SIT>
+static __device__ __forceinline__ void stage_norm_finish(stage_regs<SIT> &r, float eps, int8_t *s_q, int2 *s_meta, int K, float *s_red) {
+    float acc = 0.0f;
+#pragma unroll
+    for (int j = 0; j < SIT; j++) {
+        if (threadIdx.x + j * GEMV_THREADS < K / 4) {
+            const float4 v = r.x[j];
+            acc = fmaf(v.x, v.x, acc); acc = fmaf(v.y, v.y, acc); acc = fmaf(v.z, v.z, acc); acc = fmaf(v.w, v.w, acc);
+        }
+    }
+    acc = group_sum<64>(acc);
+    if ((threadIdx.x & 63) == 0) s_red[threadIdx.x >> 6] = acc;
+    __syncthreads();
+    const float sum = (s_red[0] + s_red[1]) + (s_red[2] + s_red[3]);
+    const float scale = 1.0f / sqrtf(sum / (float)K + eps);
+#pragma unroll
+    for (int j = 0; j < SIT; j++) {
+        const int i = threadIdx.x + j * GEMV_THREADS;
+        if (i < K / 4) {
+            float4 v = r.x[j];
+            const float4 w = r.w[j];
+            v.x = (v.x * scale) * w.x; v.y = (v.y * scale) * w.y; v.z = (v.z * scale) * w.z; v.w = (v.w * scale) * w.w;
+            int2 meta;
+            const uint32_t q = quantize_oct(v, meta);
+            ((uint32_t *)s_q)[i] = q;
+            if ((threadIdx.x & 7) == 0) s_meta[i >> 3] = meta;
+        }
+    }
+    __syncthreads();
+}
+
 // ---- weight tiles --------------------------------------------------------------------------
 
-template <int WT> struct wtile { uint32_t w[wt_traits<WT>::NIT_MAX][wt_traits<WT>::PAIR_DW]; };
+template <int WT, int NIT> struct wtile { uint32_t w[NIT][wt_traits<WT>::PAIR_DW]; };
 
-template <int WT, int LPR>
-static __device__ __forceinline__ void load_tile(wtile<WT> &t, const uint8_t *__restrict__ rowp, int npair, int nit, int l) {
+template <int WT, int LPR, int NIT>
+static __device__ __forceinline__ void load_tile(wtile<WT, NIT> &t, const uint8_t *__restrict__ rowp, int npair, int l) {
     constexpr int DW = wt_traits<WT>::PAIR_DW;
 #pragma unroll
-    for (int it = 0; it < wt_traits<WT>::NIT_MAX; it++) {
+    for (int it = 0; it < NIT; it++) {
         const int p = it * LPR + l;
-        if (it < nit && p < npair) {
+        if (p < npair) {
             const uint32_t *wp = (const uint32_t *)rowp + (size_t)p * DW;
 #pragma unroll
             for (int i = 0; i < DW; i++) t.w[it][i] = wp[i];
@@ -172,13 +198,13 @@ static __device__ __forceinline__ int dot_q8_dwords(const uint32_t *n, const int
 
 // Partial dot of the lane's pairs of one weight row with NT staged activation columns.
 // dump (optional): int32 dot of every block, row-major [nblk] for activation column 0.
-template <int WT, int LPR, int NT>
-static __device__ __forceinline__ void dot_tile(const wtile<WT> &t, const staged_act *act, int npair, int nit, int l,
+template <int WT, int LPR, int NIT, int NT>
+static __device__ __forceinline__ void dot_tile(const wtile<WT, NIT> &t, const staged_act *act, int npair, int l,
                                                 float acc[NT], int32_t *dump) {
 #pragma unroll
-    for (int it = 0; it < wt_traits<WT>::NIT_MAX; it++) {
+    for (int it = 0; it < NIT; it++) {
         const int p = it * LPR + l;
-        if (it < nit && p < npair) {
+        if (p < npair) {
             const uint32_t *w = t.w[it];
             if constexpr (WT == SPY_HIP_Q4_0) {
                 const float dA = h2f((uint16_t)(w[0] & 0xFFFFu)), dB = h2f((uint16_t)(w[4] >> 16));
@@ -214,14 +240,27 @@ static __device__ __forceinline__ void dot_tile(const wtile<WT> &t, const staged
     }
 }
 
-// Lanes-per-row choice for K elements of type WT; returns 0 when no configuration fits
-// (K must be a multiple of 64 so that every row is a whole number of 4-byte aligned pairs).
-template <int WT> static inline int pick_lpr(int64_t K) {
-    if (K % 64 != 0) return 0;
+// (lanes per row, block pairs per lane) for K elements: the smallest lane count whose pairs-per-lane
+// fits GEMV_NIT_MAX; lpr = 0 when nothing fits (K must be a multiple of 64 so that every row is a
+// whole number of 4-byte aligned block pairs).
+struct gemv_cfg { int lpr, nit; };
+static inline gemv_cfg pick_cfg(int64_t K, int max_lpr = 64) {
+    gemv_cfg c = {0, 0};
+    if (K % 64 != 0 || K <= 0) return c;
     const int64_t npair = K / 64;
-    const int nitmax = wt_traits<WT>::NIT_MAX;
-    if (npair <= 16 * nitmax) return 16;
-    if (npair <= 32 * nitmax) return 32;
-    if (npair <= 64 * nitmax) return 64;
-    return 0;
+    for (int lpr = 16; lpr <= max_lpr; lpr *= 2) {
+        const int64_t nit = (npair + lpr - 1) / lpr;
+        if (nit <= GEMV_NIT_MAX) { c.lpr = lpr; c.nit = (int)nit; return c; }
+    }
+    return c;
 }
+
+// dispatch a callable templated on <LPR, NIT> from run-time values
+#define GEMV_DISPATCH_CFG(cfg, CALL)                                                       \
+    switch ((cfg).lpr * 8 + (cfg).nit) {                                                   \
+    case 16 * 8 + 1: CALL(16, 1); break; case 16 * 8 + 2: CALL(16, 2); break;              \
+    case 16 * 8 + 3: CALL(16, 3); break; case 16 * 8 + 4: CALL(16, 4); break;              \
+    case 32 * 8 + 3: CALL(32, 3); break; case 32 * 8 + 4: CALL(32, 4); break;              \
+    case 64 * 8 + 3: CALL(64, 3); break; case 64 * 8 + 4: CALL(64, 4); break;              \
+    default: break;                                                                        \
+    }
