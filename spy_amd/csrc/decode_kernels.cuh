@@ -19,38 +19,46 @@ struct dev_state {           // lives in device memory so that a captured graph 
 };
 
 // ---- persistent GEMV over row tiles with two tiles' weights always in flight ---------------------
-template <int WT, int LPR, int NIT> struct gemv_stream {
+// SIDE: one float per row (the residual) travels with the row's tile, so that the epilogue does not
+// issue a load of its own (which would have to wait for every older load, i.e. the next tile).
+template <int WT, int LPR, int NIT, bool SIDE = false> struct gemv_stream {
     static constexpr int RPW = SPY_WAVE / LPR, RPT = GEMV_WAVES * RPW;
     wtile<WT, NIT> A, B;
+    float sideA, sideB;
+    const float *side;
     int tile, ntiles, G, npair, l, g, rofs, M;
 
-    template <class RowPtr> __device__ __forceinline__ void fetch(wtile<WT, NIT> &t, int tl, RowPtr rowptr) {
-        if (tl < ntiles && tl * RPT + rofs < M) load_tile<WT, LPR, NIT>(t, rowptr(tl * RPT + rofs), npair, l);
+    // unconditional: a tile index beyond the matrix re-reads the last row (never used)
+    template <class RowPtr> __device__ __forceinline__ void fetch(wtile<WT, NIT> &t, float &sd, int tl, RowPtr rowptr) {
+        int r = tl * RPT + rofs;
+        r = (tl < ntiles && r < M) ? r : M - 1;
+        load_tile<WT, LPR, NIT>(t, rowptr(r), npair, l);
+        if constexpr (SIDE) sd = side[r];
     }
-    template <class RowPtr> __device__ __forceinline__ void begin(int M_, int K, RowPtr rowptr) {
-        M = M_;
+    template <class RowPtr> __device__ __forceinline__ void begin(int M_, int K, RowPtr rowptr, const float *side_ = nullptr) {
+        M = M_; side = side_;
         npair = K / 64;
         const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
         l = lane % LPR; g = lane / LPR; rofs = wave * RPW + g;
         ntiles = (M + RPT - 1) / RPT; G = gridDim.x; tile = blockIdx.x;
-        fetch(A, tile, rowptr);
-        fetch(B, tile + G, rowptr);
+        fetch(A, sideA, tile, rowptr);
+        fetch(B, sideB, tile + G, rowptr);
     }
-    // epi(r, total, valid): called by every lane; `total` is the row's dot, present in all LPR lanes
+    // epi(r, total, side, valid): called by every lane; `total` is the row's dot, present in all LPR lanes
     template <class RowPtr, class Epi> __device__ __forceinline__ void run(const staged_act &act, RowPtr rowptr, Epi epi) {
-        auto finish = [&](const wtile<WT, NIT> &t, int tl) {
+        auto finish = [&](const wtile<WT, NIT> &t, float sd, int tl) {
             const int r = tl * RPT + rofs;
             float acc[1] = {0.0f};
             if (r < M) dot_tile<WT, LPR, NIT, 1>(t, &act, npair, l, acc, nullptr);
-            epi(r, group_sum<LPR>(acc[0]), r < M);
+            epi(r, group_sum<LPR>(acc[0]), sd, r < M);
         };
         while (tile < ntiles) {
-            finish(A, tile);
-            fetch(A, tile + 2 * G, rowptr);
+            finish(A, sideA, tile);
+            fetch(A, sideA, tile + 2 * G, rowptr);
             tile += G;
             if (tile >= ntiles) break;
-            finish(B, tile);
-            fetch(B, tile + 2 * G, rowptr);
+            finish(B, sideB, tile);
+            fetch(B, sideB, tile + 2 * G, rowptr);
             tile += G;
         }
     }
@@ -75,34 +83,45 @@ struct fused_args {
 
 enum { EPI_QKV = 0, EPI_RESID = 1, EPI_GATEUP = 2, EPI_STORE = 3 };
 
-// SIT > 0: RMSNorm * weight prologue with SIT float4 of x per thread (K <= 1024*SIT); SIT == 0: plain
+// Prologue: EPI_RESID stages the plain f32 input, every other epilogue the RMS-normalised, weighted
+// one; either way SIT float4 of x per thread (K <= 1024*SIT) are requested before the weight tiles.
 template <int WT, int LPR, int NIT, int SIT, int EPI>
 __global__ __launch_bounds__(GEMV_THREADS) void fused_gemv_kernel(fused_args a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    __shared__ float s_red[4];
+    __shared__ float s_red[GEMV_WAVES];
+    constexpr bool NORM = (EPI != EPI_RESID);
     const size_t RB = (size_t)(a.K / 32) * wt_traits<WT>::BLK;
+    // the matrix bases are selected by arithmetic on wave-uniform differences: a select between
+    // the kernel arguments themselves becomes a per-lane load from the argument block
+    const ptrdiff_t dW1 = a.W1 - a.W0, dW2 = a.W2 - a.W0;
     auto rowptr = [&](int r) -> const uint8_t * {
-        if constexpr (EPI == EPI_QKV) { const int m = r / a.d, row = r - m * a.d; return (m == 0 ? a.W0 : (m == 1 ? a.W1 : a.W2)) + (size_t)row * RB; }
-        else if constexpr (EPI == EPI_GATEUP) return ((r & 1) ? a.W1 : a.W0) + (size_t)(r >> 1) * RB;
+        if constexpr (EPI == EPI_QKV) {
+            const int m = (r >= a.d) + (r >= 2 * a.d);
+            return a.W0 + (m == 0 ? (ptrdiff_t)0 : (m == 1 ? dW1 : dW2)) + (ptrdiff_t)(r - m * a.d) * (ptrdiff_t)RB;
+        } else if constexpr (EPI == EPI_GATEUP) return a.W0 + ((r & 1) ? dW1 : (ptrdiff_t)0) + (ptrdiff_t)(r >> 1) * (ptrdiff_t)RB;
         else return a.W0 + (size_t)r * RB;
     };
-    gemv_stream<WT, LPR, NIT> gs;
-    gs.begin(a.M, a.K, rowptr);                      // the first two tiles' weights are in flight from here on
+    stage_regs<NORM ? SIT : 1> sr;
+    plain_regs<NORM ? 1 : SIT> pr;
+    if constexpr (NORM) stage_norm_load<SIT>(sr, a.x_in, a.normw, a.K);
+    else stage_plain_load<SIT>(pr, a.x_in, a.K);
+    float rope_v = 0.0f;
+    if constexpr (EPI == EPI_QKV) rope_v = a.rope_cs[min((int)threadIdx.x, a.hd - 1)];   // cos/sin table of this position -> LDS
+    gemv_stream<WT, LPR, NIT, EPI == EPI_RESID> gs;
+    gs.begin(a.M, a.K, rowptr, a.resid);             // the first two tiles' weights are in flight from here on
 
     int8_t *s_q = (int8_t *)smem;
-    int2 *s_meta = (int2 *)(smem + a.K);
-    if constexpr (SIT > 0) {
-        stage_regs<SIT> sr;
-        stage_norm_load<SIT>(sr, a.x_in, a.normw, a.K);
-        stage_norm_finish<SIT>(sr, a.eps, s_q, s_meta, a.K, s_red);
-    } else {
-        stage_f32_plain(a.x_in, s_q, s_meta, a.K);
-    }
+    int2 *s_meta = (int2 *)(smem + staged_q_bytes(a.K));
+    float *s_rope = (float *)(smem + staged_bytes(a.K));
+    if constexpr (EPI == EPI_QKV) { if ((int)threadIdx.x < a.hd) s_rope[threadIdx.x] = rope_v; }
+    if constexpr (NORM) stage_norm_finish<SIT>(sr, a.eps, s_q, s_meta, a.K, s_red);
+    else stage_plain_finish<SIT>(pr, s_q, s_meta, a.K);
     staged_act act; act.q = s_q; act.meta = s_meta;
 
     const int l = gs.l;
-    auto epi = [&](int r, float s, bool valid) {
-        if constexpr (EPI == EPI_RESID) { if (valid && l == 0) a.out[r] = s + a.resid[r]; }
+    const int pos = (EPI == EPI_QKV) ? a.st->pos : 0;
+    auto epi = [&](int r, float s, float side, bool valid) {
+        if constexpr (EPI == EPI_RESID) { if (valid && l == 0) a.out[r] = s + side; }
         else if constexpr (EPI == EPI_STORE) { if (valid && l == 0) a.out[r] = s; }
         else if constexpr (EPI == EPI_GATEUP) {
             // rows 2i (gate) and 2i+1 (up) sit in neighbouring lane groups
@@ -111,11 +130,11 @@ __global__ __launch_bounds__(GEMV_THREADS) void fused_gemv_kernel(fused_args a) 
         } else {
             const float other = __shfl_xor(s, LPR, SPY_WAVE);
             if (valid && l == 0) {
-                const int m = r / a.d, row = r - m * a.d, pos = a.st->pos;
+                const int m = (r >= a.d) + (r >= 2 * a.d), row = r - m * a.d;
                 if (m == 2) a.vc[(size_t)row * a.n_ctx + pos] = f2h(s);                    // VCache_cpy: [d][C] column pos
                 else {
                     const int k = (row % a.hd) >> 1;
-                    const float c = a.rope_cs[2 * k], sn = a.rope_cs[2 * k + 1];
+                    const float c = s_rope[2 * k], sn = s_rope[2 * k + 1];
                     // (x0, x1) -> (x0*c - x1*s, x0*s + x1*c) on adjacent rows (non-linear.cpp:359-363)
                     const float v = (row & 1) ? (other * sn + s * c) : (s * c - other * sn);
                     if (m == 0) a.q16[row] = f2h(v);                                       // attn_score rounds Q to fp16 (mat.cpp:37)

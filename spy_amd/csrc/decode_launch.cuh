@@ -11,7 +11,7 @@ template <int WT, int LPR, int NIT, int SIT, int EPI>
 static int launch_fused(spy_hip_llama *m, hipStream_t st, const fused_args &a) {
     constexpr int RPT = GEMV_WAVES * (SPY_WAVE / LPR);
     static int cap = 0;                                   // workgroups resident at once (persistent grid)
-    const size_t lds = staged_bytes(a.K);
+    const size_t lds = staged_bytes(a.K) + (EPI == EPI_QKV ? 4 * (size_t)a.hd : 0);      // + the RoPE cos|sin table
     auto kern = fused_gemv_kernel<WT, LPR, NIT, SIT, EPI>;
     if (!cap) {
         if (lds > 48 * 1024) HIP_TRY(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
@@ -31,7 +31,7 @@ static int launch_fused_norm(spy_hip_llama *m, hipStream_t st, gemv_cfg cfg, con
     int rc = SPY_HIP_EUNSUPPORTED;
     const bool big = a.K > 4096;
     if (a.K > 8192) return rc;
-#define CALL(LPR, NIT) rc = big ? launch_fused<WT, LPR, NIT, 8, EPI>(m, st, a) : launch_fused<WT, LPR, NIT, 4, EPI>(m, st, a)
+#define CALL(LPR, NIT) rc = big ? launch_fused<WT, LPR, NIT, GEMV_SIT_FOR(8192), EPI>(m, st, a) : launch_fused<WT, LPR, NIT, GEMV_SIT_FOR(4096), EPI>(m, st, a)
     switch (cfg.lpr * 8 + cfg.nit) {
     case 16 * 8 + 1: CALL(16, 1); break; case 16 * 8 + 2: CALL(16, 2); break;
     case 16 * 8 + 3: CALL(16, 3); break; case 16 * 8 + 4: CALL(16, 4); break;
@@ -45,7 +45,8 @@ static int launch_fused_norm(spy_hip_llama *m, hipStream_t st, gemv_cfg cfg, con
 template <int WT>
 static int launch_fused_resid(spy_hip_llama *m, hipStream_t st, gemv_cfg cfg, const fused_args &a) {
     int rc = SPY_HIP_EUNSUPPORTED;
-#define CALL(LPR, NIT) rc = launch_fused<WT, LPR, NIT, 0, EPI_RESID>(m, st, a)
+    // input registers per thread follow the tile shape: K <= 64 * LPR * NIT
+#define CALL(LPR, NIT) rc = launch_fused<WT, LPR, NIT, GEMV_SIT_FOR(64 * LPR * NIT), EPI_RESID>(m, st, a)
     GEMV_DISPATCH_CFG(cfg, CALL)
 #undef CALL
     return rc;

@@ -32,8 +32,9 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(gemv_args a) {
 
     wtile<WT, NIT> A, B;
     int tile = blockIdx.x;
-    auto fetch = [&](wtile<WT, NIT> &t, int tl) {
-        if (tl < ntiles && tl * RPT + rofs < a.M) load_tile<WT, LPR, NIT>(t, a.W + (size_t)(tl * RPT + rofs) * RB, npair, l);
+    auto fetch = [&](wtile<WT, NIT> &t, int tl) {             // unconditional: beyond the matrix re-reads the last row
+        const int r = tl * RPT + rofs;
+        load_tile<WT, LPR, NIT>(t, a.W + (size_t)(tl < ntiles && r < a.M ? r : a.M - 1) * RB, npair, l);
     };
     fetch(A, tile);
     fetch(B, tile + G);
@@ -42,7 +43,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(gemv_args a) {
 #pragma unroll
     for (int c = 0; c < NT; c++) {
         int8_t *q = (int8_t *)(smem + (size_t)c * staged_bytes(K));
-        int2 *meta = (int2 *)(q + K);
+        int2 *meta = (int2 *)(q + staged_q_bytes(K));
         stage_native_q8(a.xq + (size_t)c * nblk * 34, q, meta, nblk);
         act[c].q = q; act[c].meta = meta;
     }

@@ -14,8 +14,12 @@
 
 #include "common.cuh"
 
+#ifndef GEMV_THREADS
 #define GEMV_THREADS 256
-#define GEMV_WAVES 4
+#endif
+#define GEMV_WAVES (GEMV_THREADS / 64)
+// float4 of input per thread that cover K elements in the staging prologues
+#define GEMV_SIT_FOR(K) (((K) + 4 * GEMV_THREADS - 1) / (4 * GEMV_THREADS))
 
 template <int WT> struct wt_traits;
 template <> struct wt_traits<SPY_HIP_Q4_0> { static constexpr int BLK = 18, PAIR_DW = 9; };
@@ -51,11 +55,21 @@ static __device__ __forceinline__ int oct_sum_i(int v) {
     return v;
 }
 
-struct staged_act {          // where one activation column lives in LDS
-    const int8_t *q;         // K bytes
+// One staged activation column in LDS.  The 64 int8 of block pair p are kept as four 16-byte parts,
+// part j at byte (j * (npair + 1) + p) * 16: consecutive lanes own consecutive pairs, so each
+// 128-bit LDS read of a wave touches consecutive words (no bank conflicts), and the +1 skews the
+// four parts over different banks for the staging writes.
+struct staged_act {
+    const int8_t *q;         // K + 64 bytes, swizzled as above
     const int2 *meta;        // K/32 x {bits(float scale), sum(q)}
 };
-static __host__ __device__ inline size_t staged_bytes(int64_t K) { return (size_t)K + (size_t)(K / 32) * 8; }
+static __host__ __device__ inline size_t staged_q_bytes(int64_t K) { return (size_t)K + 64; }
+static __host__ __device__ inline size_t staged_bytes(int64_t K) { return staged_q_bytes(K) + (size_t)(K / 32) * 8; }
+// dword index in LDS of natural dword i (= element index / 4) of the activation vector
+static __device__ __forceinline__ int act_dw(int i, int npair) { return (((((i >> 2) & 3) * (npair + 1)) + (i >> 4)) << 2) + (i & 3); }
+static __device__ __forceinline__ const int4 *act_part(const int8_t *q, int p, int j, int npair) {
+    return (const int4 *)(q + (size_t)(j * (npair + 1) + p) * 16);
+}
 
 // ---- activation staging --------------------------------------------------------------------
 
@@ -67,12 +81,11 @@ static __device__ __forceinline__ void stage_native_q8(const uint8_t *__restrict
         const int b = h / 17, w = h - b * 17;
         const uint16_t v = src[h];
         if (w == 0) s_meta[b].x = __float_as_int(h2f(v));
-        else ((uint16_t *)s_q)[b * 16 + (w - 1)] = v;
+        else { const int hw = b * 16 + (w - 1); ((uint16_t *)s_q)[2 * act_dw(hw >> 1, nblk >> 1) + (hw & 1)] = v; }
     }
     __syncthreads();
     for (int b = threadIdx.x; b < nblk; b += GEMV_THREADS) {
-        const int4 *q = (const int4 *)(s_q + b * 32);
-        const int4 q0 = q[0], q1 = q[1];
+        const int4 q0 = *act_part(s_q, b >> 1, 2 * (b & 1), nblk >> 1), q1 = *act_part(s_q, b >> 1, 2 * (b & 1) + 1, nblk >> 1);
         int s = 0;
         s = __builtin_amdgcn_sdot4(q0.x, 0x01010101, s, false); s = __builtin_amdgcn_sdot4(q0.y, 0x01010101, s, false);
         s = __builtin_amdgcn_sdot4(q0.z, 0x01010101, s, false); s = __builtin_amdgcn_sdot4(q0.w, 0x01010101, s, false);
@@ -107,8 +120,37 @@ static __device__ __forceinline__ void stage_f32_plain(const float *__restrict__
     for (int i = threadIdx.x; i < K / 4; i += GEMV_THREADS) {
         int2 meta;
         const uint32_t q = quantize_oct(((const float4 *)x)[i], meta);
-        ((uint32_t *)s_q)[i] = q;
+        ((uint32_t *)s_q)[act_dw(i, K >> 6)] = q;
         if ((threadIdx.x & 7) == 0) s_meta[i >> 3] = meta;
+    }
+    __syncthreads();
+}
+
+// The same with the global loads split off, so that a kernel can issue them BEFORE its weight-tile
+// loads: the memory counter retires loads in order, and a prologue whose loads were issued after the
+// tiles' would wait for the tiles as well.  SIT float4 per thread: K <= 1024*SIT.
+template <int SIT> struct plain_regs { float4 x[SIT]; };
+
+template <int SIT>
+static __device__ __forceinline__ void stage_plain_load(plain_regs<SIT> &r, const float *__restrict__ x, int K) {
+#pragma unroll
+    for (int j = 0; j < SIT; j++) {
+        const int i = min((int)threadIdx.x + j * GEMV_THREADS, K / 4 - 1);      // unconditional (see load_tile)
+        r.x[j] = ((const float4 *)x)[i];
+    }
+}
+
+template <int SIT>
+static __device__ __forceinline__ void stage_plain_finish(const plain_regs<SIT> &r, int8_t *s_q, int2 *s_meta, int K) {
+#pragma unroll
+    for (int j = 0; j < SIT; j++) {
+        const int i = threadIdx.x + j * GEMV_THREADS;
+        if (i < K / 4) {
+            int2 meta;
+            const uint32_t q = quantize_oct(r.x[j], meta);
+            ((uint32_t *)s_q)[act_dw(i, K >> 6)] = q;
+            if ((threadIdx.x & 7) == 0) s_meta[i >> 3] = meta;
+        }
     }
     __syncthreads();
 }
@@ -124,8 +166,8 @@ template <int SIT>
 static __device__ __forceinline__ void stage_norm_load(stage_regs<SIT> &r, const float *__restrict__ x, const float *__restrict__ normw, int K) {
 #pragma unroll
     for (int j = 0; j < SIT; j++) {
-        const int i = threadIdx.x + j * GEMV_THREADS;
-        if (i < K / 4) { r.x[j] = ((const float4 *)x)[i]; r.w[j] = ((const float4 *)normw)[i]; }
+        const int i = min((int)threadIdx.x + j * GEMV_THREADS, K / 4 - 1);      // unconditional (see load_tile)
+        r.x[j] = ((const float4 *)x)[i]; r.w[j] = ((const float4 *)normw)[i];
     }
 }
 
@@ -142,7 +184,9 @@ static __device__ __forceinline__ void stage_norm_finish(stage_regs<SIT> &r, flo
     acc = group_sum<64>(acc);
     if ((threadIdx.x & 63) == 0) s_red[threadIdx.x >> 6] = acc;
     __syncthreads();
-    const float sum = (s_red[0] + s_red[1]) + (s_red[2] + s_red[3]);
+    float sum = 0.0f;
+#pragma unroll
+    for (int w = 0; w < GEMV_WAVES; w += 4) sum += (s_red[w] + s_red[w + 1]) + (s_red[w + 2] + s_red[w + 3]);
     const float scale = 1.0f / sqrtf(sum / (float)K + eps);
 #pragma unroll
     for (int j = 0; j < SIT; j++) {
@@ -153,7 +197,7 @@ static __device__ __forceinline__ void stage_norm_finish(stage_regs<SIT> &r, flo
             v.x = (v.x * scale) * w.x; v.y = (v.y * scale) * w.y; v.z = (v.z * scale) * w.z; v.w = (v.w * scale) * w.w;
             int2 meta;
             const uint32_t q = quantize_oct(v, meta);
-            ((uint32_t *)s_q)[i] = q;
+            ((uint32_t *)s_q)[act_dw(i, K >> 6)] = q;
             if ((threadIdx.x & 7) == 0) s_meta[i >> 3] = meta;
         }
     }
@@ -164,17 +208,18 @@ static __device__ __forceinline__ void stage_norm_finish(stage_regs<SIT> &r, flo
 
 template <int WT, int NIT> struct wtile { uint32_t w[NIT][wt_traits<WT>::PAIR_DW]; };
 
+// Branch-free on purpose: the memory counter retires loads in order, and the compiler can only
+// wait for "all but the N youngest" loads when those N are issued unconditionally.  Lanes whose
+// pair index lies beyond the row re-read the last pair (a cache hit that dot_tile ignores).
 template <int WT, int LPR, int NIT>
 static __device__ __forceinline__ void load_tile(wtile<WT, NIT> &t, const uint8_t *__restrict__ rowp, int npair, int l) {
     constexpr int DW = wt_traits<WT>::PAIR_DW;
 #pragma unroll
     for (int it = 0; it < NIT; it++) {
-        const int p = it * LPR + l;
-        if (p < npair) {
-            const uint32_t *wp = (const uint32_t *)rowp + (size_t)p * DW;
+        const int p = min(it * LPR + l, npair - 1);
+        const uint32_t *wp = (const uint32_t *)rowp + (size_t)p * DW;
 #pragma unroll
-            for (int i = 0; i < DW; i++) t.w[it][i] = wp[i];
-        }
+        for (int i = 0; i < DW; i++) t.w[it][i] = wp[i];
     }
 }
 
@@ -212,10 +257,10 @@ static __device__ __forceinline__ void dot_tile(const wtile<WT, NIT> &t, const s
                 const uint32_t a2 = __builtin_amdgcn_alignbit(w[3], w[2], 16), a3 = __builtin_amdgcn_alignbit(w[4], w[3], 16);
 #pragma unroll
                 for (int c = 0; c < NT; c++) {
-                    const int4 *xa = (const int4 *)(act[c].q + (size_t)p * 64);
+                    const int8_t *xq = act[c].q;
                     const int4 mm = *(const int4 *)(act[c].meta + 2 * p);
-                    const int iA = dot_q4_dwords(a0, a1, a2, a3, xa[0], xa[1]) - 8 * mm.y;
-                    const int iB = dot_q4_dwords(w[5], w[6], w[7], w[8], xa[2], xa[3]) - 8 * mm.w;
+                    const int iA = dot_q4_dwords(a0, a1, a2, a3, *act_part(xq, p, 0, npair), *act_part(xq, p, 1, npair)) - 8 * mm.y;
+                    const int iB = dot_q4_dwords(w[5], w[6], w[7], w[8], *act_part(xq, p, 2, npair), *act_part(xq, p, 3, npair)) - 8 * mm.w;
                     if (dump && c == 0) { dump[2 * p] = iA; dump[2 * p + 1] = iB; }
                     acc[c] = fmaf(dA * __int_as_float(mm.x), (float)iA, acc[c]);
                     acc[c] = fmaf(dB * __int_as_float(mm.z), (float)iB, acc[c]);
@@ -227,10 +272,10 @@ static __device__ __forceinline__ void dot_tile(const wtile<WT, NIT> &t, const s
                 for (int i = 0; i < 8; i++) a[i] = __builtin_amdgcn_alignbit(w[i + 1], w[i], 16);
 #pragma unroll
                 for (int c = 0; c < NT; c++) {
-                    const int4 *xa = (const int4 *)(act[c].q + (size_t)p * 64);
+                    const int8_t *xq = act[c].q;
                     const int4 mm = *(const int4 *)(act[c].meta + 2 * p);
-                    const int iA = dot_q8_dwords(a, xa[0], xa[1]);
-                    const int iB = dot_q8_dwords(&w[9], xa[2], xa[3]);
+                    const int iA = dot_q8_dwords(a, *act_part(xq, p, 0, npair), *act_part(xq, p, 1, npair));
+                    const int iB = dot_q8_dwords(&w[9], *act_part(xq, p, 2, npair), *act_part(xq, p, 3, npair));
                     if (dump && c == 0) { dump[2 * p] = iA; dump[2 * p + 1] = iB; }
                     acc[c] = fmaf(dA * __int_as_float(mm.x), (float)iA, acc[c]);
                     acc[c] = fmaf(dB * __int_as_float(mm.z), (float)iB, acc[c]);
