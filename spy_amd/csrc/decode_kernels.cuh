@@ -146,6 +146,131 @@ __global__ __launch_bounds__(GEMV_THREADS) void fused_gemv_kernel(fused_args a) 
     gs.run(act, rowptr, epi);
 }
 
+// ---- one weight row per wave ------------------------------------------------------------------------
+// 1024-thread workgroups, one per compute unit: every wave owns whole rows (64 lanes x NITK block
+// pairs), all of them requested at kernel start right after the activation vector, which the 1024
+// threads then stage together (one float4 each for K = 4096).  Compared with fused_gemv_kernel this
+// quarters the redundant activation reads and the staging work per thread; it is used where a row
+// fits 64 lanes x NITK pairs (K <= 4096 * NITK).
+//   EPI_QKV   : wave j -> rows 2j, 2j+1 of [W0; W1] (a RoPE pair) and row j of W2          (grid covers d waves)
+//   EPI_GATEUP: wave   -> NR pairs (W0 row i, W1 row i), i = gw + k*NW
+//   EPI_RESID / EPI_STORE: wave -> NR rows r = gw + k*NW of W0
+#define WGV_THREADS 1024
+#define WGV_WAVES 16
+template <int WT, int NITK, int NR, int EPI>
+__global__ __launch_bounds__(WGV_THREADS) void wave_gemv_kernel(fused_args a) {
+    constexpr bool NORM = (EPI != EPI_RESID);
+    constexpr int NB = EPI == EPI_QKV ? 3 : (EPI == EPI_GATEUP ? 2 * NR : NR);
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    __shared__ float s_red[WGV_WAVES];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int NW = (int)gridDim.x * WGV_WAVES, gw = (int)blockIdx.x * WGV_WAVES + wave;
+    const int K = a.K, npair = K / 64;
+    const size_t RB = (size_t)(K / 32) * wt_traits<WT>::BLK;
+
+    // 1. the activation vector (and what the epilogue needs), 2. the rows: all unconditional, in this order
+    float4 xv[NITK], wv[NORM ? NITK : 1];
+#pragma unroll
+    for (int j = 0; j < NITK; j++) {
+        const int i = min(tid + j * WGV_THREADS, K / 4 - 1);
+        xv[j] = ((const float4 *)a.x_in)[i];
+        if constexpr (NORM) wv[j] = ((const float4 *)a.normw)[i];
+    }
+    float rope_v = 0.0f, side[EPI == EPI_RESID ? NR : 1];
+    if constexpr (EPI == EPI_QKV) rope_v = a.rope_cs[min(tid, a.hd - 1)];
+    wtile<WT, NITK> t[NB];
+    if constexpr (EPI == EPI_QKV) {
+        const int j = gw % a.d;
+        const uint8_t *p0 = 2 * j < a.d ? a.W0 + (size_t)(2 * j) * RB : a.W1 + (size_t)(2 * j - a.d) * RB;
+        load_tile<WT, 64, NITK>(t[0], p0, npair, lane);
+        load_tile<WT, 64, NITK>(t[1], p0 + RB, npair, lane);
+        load_tile<WT, 64, NITK>(t[2], a.W2 + (size_t)j * RB, npair, lane);
+    } else if constexpr (EPI == EPI_GATEUP) {
+        const int F = a.M / 2;
+#pragma unroll
+        for (int k = 0; k < NR; k++) {
+            const int u = gw + k * NW, i = u < F ? u : gw % F;
+            load_tile<WT, 64, NITK>(t[2 * k], a.W0 + (size_t)i * RB, npair, lane);
+            load_tile<WT, 64, NITK>(t[2 * k + 1], a.W1 + (size_t)i * RB, npair, lane);
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < NR; k++) {
+            const int u = gw + k * NW, r = u < a.M ? u : gw % a.M;
+            load_tile<WT, 64, NITK>(t[k], a.W0 + (size_t)r * RB, npair, lane);
+            if constexpr (EPI == EPI_RESID) side[k] = a.resid[r];
+        }
+    }
+
+    // 3. stage the activations: RMSNorm * weight (non-linear.cpp:216-219 and the separate Mul node) or plain, then Q8_0
+    int8_t *s_q = (int8_t *)smem;
+    int2 *s_meta = (int2 *)(smem + staged_q_bytes(K));
+    float *s_rope = (float *)(smem + staged_bytes(K));
+    if constexpr (EPI == EPI_QKV) { if (tid < a.hd) s_rope[tid] = rope_v; }
+    float scale = 1.0f;
+    if constexpr (NORM) {
+        float acc = 0.0f;
+#pragma unroll
+        for (int j = 0; j < NITK; j++) {
+            if (tid + j * WGV_THREADS < K / 4) { const float4 v = xv[j]; acc = fmaf(v.x, v.x, acc); acc = fmaf(v.y, v.y, acc); acc = fmaf(v.z, v.z, acc); acc = fmaf(v.w, v.w, acc); }
+        }
+        acc = group_sum<64>(acc);
+        if (lane == 0) s_red[wave] = acc;
+        __syncthreads();
+        const float sum = (((s_red[0] + s_red[1]) + (s_red[2] + s_red[3])) + ((s_red[4] + s_red[5]) + (s_red[6] + s_red[7]))) +
+                          (((s_red[8] + s_red[9]) + (s_red[10] + s_red[11])) + ((s_red[12] + s_red[13]) + (s_red[14] + s_red[15])));
+        scale = 1.0f / sqrtf(sum / (float)K + a.eps);
+    }
+#pragma unroll
+    for (int j = 0; j < NITK; j++) {
+        const int i = tid + j * WGV_THREADS;
+        if (i < K / 4) {
+            float4 v = xv[j];
+            if constexpr (NORM) { const float4 w = wv[j]; v.x = (v.x * scale) * w.x; v.y = (v.y * scale) * w.y; v.z = (v.z * scale) * w.z; v.w = (v.w * scale) * w.w; }
+            int2 meta;
+            const uint32_t q = quantize_oct(v, meta);
+            ((uint32_t *)s_q)[act_dw(i, K >> 6)] = q;
+            if ((tid & 7) == 0) s_meta[i >> 3] = meta;
+        }
+    }
+    __syncthreads();
+    staged_act act; act.q = s_q; act.meta = s_meta;
+    auto row_dot = [&](const wtile<WT, NITK> &tl) -> float {
+        float acc[1] = {0.0f};
+        dot_tile<WT, 64, NITK, 1>(tl, &act, npair, lane, acc, nullptr);
+        return group_sum<64>(acc[0]);
+    };
+
+    // 4. dots and epilogues
+    if constexpr (EPI == EPI_QKV) {
+        const float s0 = row_dot(t[0]), s1 = row_dot(t[1]), s2 = row_dot(t[2]);
+        if (lane == 0 && gw < a.d) {
+            const int j = gw, row = (2 * j) % a.d, k = (row % a.hd) >> 1, pos = a.st->pos;
+            const float c = s_rope[2 * k], sn = s_rope[2 * k + 1];
+            // (x0, x1) -> (x0*c - x1*s, x0*s + x1*c) on adjacent rows (non-linear.cpp:359-363)
+            const uint32_t pr = (uint32_t)f2h(s0 * c - s1 * sn) | ((uint32_t)f2h(s0 * sn + s1 * c) << 16);
+            if (2 * j < a.d) ((uint32_t *)a.q16)[j] = pr;                                        // attn_score rounds Q to fp16 (mat.cpp:37)
+            else ((uint32_t *)(a.kc + (size_t)pos * a.d))[j - a.d / 2] = pr;                      // KCache_cpy: [token][head][hd]
+            a.vc[(size_t)j * a.n_ctx + pos] = f2h(s2);                                           // VCache_cpy: [d][C] column pos
+        }
+    } else if constexpr (EPI == EPI_GATEUP) {
+        const int F = a.M / 2;
+#pragma unroll
+        for (int k = 0; k < NR; k++) {
+            const float g = row_dot(t[2 * k]), u = row_dot(t[2 * k + 1]);
+            const int i = gw + k * NW;
+            if (lane == 0 && i < F) a.out[i] = u * silu_lut(g);                                   // Mul(ffn_up, silu(ffn_gate)) (ffn.cpp:24-35)
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < NR; k++) {
+            const float s = row_dot(t[k]);
+            const int r = gw + k * NW;
+            if (lane == 0 && r < a.M) { if constexpr (EPI == EPI_RESID) a.out[r] = s + side[k]; else a.out[r] = s; }
+        }
+    }
+}
+
 #ifdef SPY_DECODE_COMMON_KERNELS   // type-independent kernels: compiled by one translation unit only
 
 // ---- token embedding + RoPE table ---------------------------------------------------------------

@@ -52,6 +52,33 @@ static int launch_fused_resid(spy_hip_llama *m, hipStream_t st, gemv_cfg cfg, co
     return rc;
 }
 
+
+// ---- one-row-per-wave kernels (K <= 4096 * NITK) ---------------------------------------------------
+template <int WT, int NITK, int NR, int EPI>
+static int launch_wave(spy_hip_llama *m, hipStream_t st, const fused_args &a) {
+    const size_t lds = staged_bytes(a.K) + (EPI == EPI_QKV ? 4 * (size_t)a.hd : 0);
+    auto kern = wave_gemv_kernel<WT, NITK, NR, EPI>;
+    static size_t lds_set = 0;
+    if (lds > 48 * 1024 && lds > lds_set) { HIP_TRY(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); lds_set = lds; }
+    if (m->dry) return 0;
+    const int units = EPI == EPI_QKV ? a.d : (EPI == EPI_GATEUP ? a.M / 2 : a.M);       // one per wave and step
+    const int grid = (units + WGV_WAVES * NR - 1) / (WGV_WAVES * NR);
+    kern<<<dim3((unsigned)grid), dim3(WGV_THREADS), lds, st>>>(a);
+    return SPY_LAUNCH_RC();
+}
+template <int WT> struct wave_rows { static constexpr int HEAD = (WT == SPY_HIP_Q4_0) ? 8 : 4, GATEUP = (WT == SPY_HIP_Q4_0) ? 3 : 2; };
+
+template <int WT>
+static int launch_wave_resid(spy_hip_llama *m, hipStream_t st, const fused_args &a) {
+    switch ((a.K + 4095) / 4096) {
+    case 1: return launch_wave<WT, 1, 1, EPI_RESID>(m, st, a);
+    case 2: return launch_wave<WT, 2, 1, EPI_RESID>(m, st, a);
+    case 3: return launch_wave<WT, 3, 1, EPI_RESID>(m, st, a);
+    case 4: return launch_wave<WT, 4, 1, EPI_RESID>(m, st, a);
+    default: return SPY_HIP_EUNSUPPORTED;
+    }
+}
+
 // one kernel of layer il of the single-token pass
 template <int WT>
 static int enqueue_kernel(spy_hip_llama *m, hipStream_t st, int which, int il) {
@@ -66,15 +93,19 @@ static int enqueue_kernel(spy_hip_llama *m, hipStream_t st, int which, int il) {
     case K_QKV:      // attn_norm, attn_norm_linear, Q/K/V_project, rope, KV-cache copies
         a.W0 = (const uint8_t *)L.wq; a.W1 = (const uint8_t *)L.wk; a.W2 = (const uint8_t *)L.wv;
         a.M = 3 * d; a.K = d; a.x_in = m->x; a.normw = L.attn_norm;
+        if (m->wave) return launch_wave<WT, 1, 1, EPI_QKV>(m, st, a);
         return launch_fused_norm<WT, EPI_QKV>(m, st, m->cfg_d, a);
     case K_WO:       // KQV_linear + ffn_input
         a.W0 = (const uint8_t *)L.wo; a.M = d; a.K = d; a.x_in = m->attn_out; a.resid = m->x; a.out = m->x1;
+        if (m->wave) return launch_wave_resid<WT>(m, st, a);
         return launch_fused_resid<WT>(m, st, m->cfg_d, a);
     case K_GATEUP:   // ffn_norm, ffn_up, ffn_gate, silu, ffn_par
         a.W0 = (const uint8_t *)L.w_gate; a.W1 = (const uint8_t *)L.w_up; a.M = 2 * F; a.K = d; a.x_in = m->x1; a.normw = L.ffn_norm; a.out = m->hbuf;
+        if (m->wave) return launch_wave<WT, 1, wave_rows<WT>::GATEUP, EPI_GATEUP>(m, st, a);
         return launch_fused_norm<WT, EPI_GATEUP>(m, st, m->cfg_d, a);
     case K_DOWN:     // ffn_down + logit_output (the next layer's input)
         a.W0 = (const uint8_t *)L.w_down; a.M = d; a.K = F; a.x_in = m->hbuf; a.resid = m->x1; a.out = m->x;
+        if (m->wave) return launch_wave_resid<WT>(m, st, a);
         return launch_fused_resid<WT>(m, st, m->cfg_ff, a);
     }
     return SPY_HIP_EINVAL;
@@ -89,6 +120,7 @@ static int enqueue_head(spy_hip_llama *m, hipStream_t st) {
         fused_args a;
         memset(&a, 0, sizeof(a));
         a.W0 = (const uint8_t *)c.w_out; a.M = c.n_vocab; a.K = d; a.x_in = m->x; a.normw = c.out_norm; a.eps = c.eps; a.out = m->logits;
+        if (m->wave) return launch_wave<WT, 1, wave_rows<WT>::HEAD, EPI_STORE>(m, st, a);
         return launch_fused_norm<WT, EPI_STORE>(m, st, m->cfg_d, a);
     }
     // head in another type (e.g. Q6_K): norm + weight + Q8_0 through the operator kernels
@@ -108,4 +140,48 @@ static int enqueue_head(spy_hip_llama *m, hipStream_t st) {
 template <int WT>
 static int enqueue_any(spy_hip_llama *m, hipStream_t st, int which, int il) {
     return which == K_HEAD ? enqueue_head<WT>(m, st) : enqueue_kernel<WT>(m, st, which, il);
+}
+
+
+// ---- the persistent single-kernel pass -----------------------------------------------------------
+template <int WT, int NITF>
+static int mega_launch_nitf(spy_hip_llama *m, hipStream_t st, bool probe, const mega_args &a, size_t lds) {
+    auto kern = mega_decode_kernel<WT, NITF>;
+    static size_t lds_set = 0;
+    if (probe || lds > lds_set) {
+        if (lds > lds_set && lds > 48 * 1024) { HIP_TRY(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); lds_set = lds; }
+        int per_cu = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, MEGA_THREADS, lds) != hipSuccess) per_cu = 0;
+        if (per_cu < 1) return SPY_HIP_EUNSUPPORTED;      // the grid barrier needs every workgroup resident
+    }
+    if (probe) return 0;
+    kern<<<dim3((unsigned)m->num_cu), dim3(MEGA_THREADS), lds, st>>>(a);
+    return SPY_LAUNCH_RC();
+}
+
+template <int WT>
+static int mega_launch(spy_hip_llama *m, hipStream_t st, bool probe) {
+    const spy_hip_llama_desc &c = m->desc;
+    const int NW = m->num_cu * MEGA_WAVES;
+    // one batch of rows per wave and phase (see the work split in mega_kernel.cuh)
+    if (m->hd != 128 || c.n_head % 4 != 0 || c.n_embd % 64 != 0 || c.n_embd > 4096 || c.n_embd > NW || c.n_ff % 64 != 0 || c.t_out != c.wtype) return SPY_HIP_EUNSUPPORTED;
+    if ((c.n_ff + NW - 1) / NW > MEGA_SLOTS || (int64_t)c.n_ctx * (c.n_head / 4) > (int64_t)MEGA_RS * NW || c.n_ctx > MEGA_RV * 512 || c.n_ctx % 8 != 0) return SPY_HIP_EUNSUPPORTED;
+    if (m->num_cu > MEGA_FAN * MEGA_MAX_LEAF) return SPY_HIP_EUNSUPPORTED;
+    mega_args a;
+    memset(&a, 0, sizeof(a));
+    a.layers = m->mega_layers; a.n_layer = c.n_layer; a.d = c.n_embd; a.F = c.n_ff; a.H = c.n_head; a.hd = m->hd; a.n_ctx = c.n_ctx; a.n_vocab = c.n_vocab;
+    a.eps = c.eps; a.theta_scale = m->theta_scale; a.att_scale = 1.0f / sqrtf((float)m->hd);       // SoftmaxParam::scale (attention.cpp:113)
+    a.tok_embd = (const uint8_t *)c.tok_embd; a.embd_q8 = c.t_tok_embd == SPY_HIP_Q8_0;
+    a.out_norm = (const float *)c.out_norm; a.w_out = (const uint8_t *)c.w_out;
+    a.st = m->st; a.sync = m->msync;
+    a.x = m->x; a.x1 = m->x1; a.attn_out = m->attn_out; a.hbuf = m->hbuf; a.scores = m->scores; a.logits = m->logits; a.q16 = m->q16;
+    a.dbg = m->mega_dbg;
+    a.spin_limit = 400000;                                 // ~0.5 s of polling before a pass gives up
+    const size_t lds = mega_lds_bytes(c.n_embd, c.n_ff, m->hd, c.n_ctx);
+    if (lds > 160 * 1024) return SPY_HIP_EUNSUPPORTED;
+    switch ((c.n_ff + 4095) / 4096) {
+    case 1: return mega_launch_nitf<WT, 1>(m, st, probe, a, lds);
+    case 3: return mega_launch_nitf<WT, 3>(m, st, probe, a, lds);
+    default: return SPY_HIP_EUNSUPPORTED;
+    }
 }

@@ -59,6 +59,10 @@ extern "C" int spy_hip_llama_create(const spy_hip_llama_desc *desc, spy_hip_llam
     }
     m->cfg_d  = pick_cfg(c.n_embd, 32);
     m->cfg_ff = pick_cfg(c.n_ff);
+    {   // SPY_HIP_TILED=1 keeps the 256-thread tiled kernels (the only ones for n_embd > 4096)
+        const char *env = getenv("SPY_HIP_TILED");
+        m->wave = wave_ok(m) && !(env && env[0] == '1');
+    }
     {
         int dev = 0; hipDeviceProp_t prop;
         if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0) m->num_cu = prop.multiProcessorCount;
@@ -92,6 +96,22 @@ extern "C" int spy_hip_llama_create(const spy_hip_llama_desc *desc, spy_hip_llam
         if (!rc && pv_lds > 48 * 1024) rc = (int)hipFuncSetAttribute((const void *)attn_pv_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)pv_lds);
     }
     if (!rc && fused_ok(m)) { m->dry = true; rc = enqueue_pass_any(m, m->own_stream, true); m->dry = false; }   // sizes the persistent grids
+    if (!rc && fused_ok(m)) {            // the persistent single-kernel pass: opt-in with SPY_HIP_MEGA=1 (slower than the per-phase kernels so far)
+        std::vector<mega_layer> ml(c.n_layer);
+        for (int i = 0; i < c.n_layer; i++) {
+            const spy_hip_llama_layer &L = m->layers[i];
+            ml[i] = mega_layer{(const uint8_t *)L.wq, (const uint8_t *)L.wk, (const uint8_t *)L.wv, (const uint8_t *)L.wo, (const uint8_t *)L.w_gate,
+                               (const uint8_t *)L.w_up, (const uint8_t *)L.w_down, (const float *)L.attn_norm, (const float *)L.ffn_norm,
+                               m->k_cache[i], m->v_cache[i]};
+        }
+        rc = dalloc(m, (void **)&m->mega_layers, ml.size() * sizeof(mega_layer), false);
+        if (!rc) rc = (int)hipMemcpy(m->mega_layers, ml.data(), ml.size() * sizeof(mega_layer), hipMemcpyHostToDevice);
+        if (!rc) rc = dalloc(m, (void **)&m->msync, sizeof(mega_sync), true);
+        if (!rc && getenv("SPY_HIP_MEGA_STAMPS")) rc = dalloc(m, (void **)&m->mega_dbg, 128 * sizeof(long long), true);
+        const char *env = getenv("SPY_HIP_MEGA");
+        if (!rc && env && env[0] == '1')
+            m->mega = (c.wtype == SPY_HIP_Q4_0 ? spy_enqueue_mega_q4_0(m, m->own_stream, true) : spy_enqueue_mega_q8_0(m, m->own_stream, true)) == 0;
+    }
     if (rc) { spy_hip_llama_destroy(m); return rc; }
     *out = m;
     return 0;
@@ -108,11 +128,14 @@ extern "C" int spy_hip_llama_buffer(spy_hip_llama *m, const char *name, int32_t 
     else if (!strcmp(name, "logits")) { p = m->logits; n = (size_t)m->desc.n_vocab * 4; }
     else if (!strcmp(name, "scores")) { p = m->scores; n = (size_t)m->desc.n_head * C * 4; }
     else if (!strcmp(name, "attn_out")) { p = m->attn_out; n = d * 4; }
+    else if (!strcmp(name, "phase_stamps") && m->mega_dbg) { p = m->mega_dbg; n = 128 * sizeof(long long); }
     else return SPY_HIP_EINVAL;
     *ptr = p;
     if (bytes) *bytes = n;
     return 0;
 }
+
+extern "C" int spy_hip_llama_single_kernel(spy_hip_llama *m) { return m ? (m->mega ? 1 : 0) : SPY_HIP_EINVAL; }
 
 extern "C" int spy_hip_llama_timing(spy_hip_llama *m, float *ms_per_pass, int32_t *n_pass) {
     SPY_CHECK_ARG(m);
@@ -148,6 +171,14 @@ static int enqueue_one(spy_hip_llama *m, hipStream_t st, int which, int il) {
 
 static int enqueue_pass_any(spy_hip_llama *m, hipStream_t st, bool sample) {
     const spy_hip_llama_desc &c = m->desc;
+    if (m->mega && !m->dry) {
+        RC_TRY(c.wtype == SPY_HIP_Q4_0 ? spy_enqueue_mega_q4_0(m, st, false) : spy_enqueue_mega_q8_0(m, st, false));
+        if (sample) {
+            sample_advance_kernel<<<dim3(1), dim3(1024), 0, st>>>(m->st, m->logits, c.n_vocab, m->tokens_out, m->max_out);
+            RC_TRY(SPY_LAUNCH_RC());
+        }
+        return 0;
+    }
     if (!m->dry) {
         embed_kernel<<<dim3(1), dim3(256), 0, st>>>(m->st, (const uint8_t *)c.tok_embd, c.t_tok_embd == SPY_HIP_Q8_0, c.n_embd, c.n_vocab, m->x,
                                                     m->rope_cs, m->theta_scale, m->hd);

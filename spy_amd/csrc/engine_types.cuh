@@ -2,6 +2,7 @@
 #pragma once
 
 #include "decode_kernels.cuh"
+#include "mega_kernel.cuh"
 
 #include <vector>
 
@@ -14,6 +15,7 @@ struct spy_hip_llama {
     int hd = 0;
     gemv_cfg cfg_d = {0, 0}, cfg_ff = {0, 0};   // lanes-per-row / pairs-per-lane for K = n_embd and K = n_ff
     bool dry = false;
+    bool wave = false;                          // one-row-per-wave kernels (1024-thread workgroups) instead of the tiled ones
     std::vector<uint16_t *> k_cache, v_cache;
     float *x = nullptr, *x1 = nullptr, *attn_out = nullptr, *hbuf = nullptr, *scores = nullptr, *logits = nullptr, *rope_cs = nullptr;
     uint16_t *q16 = nullptr;
@@ -30,9 +32,20 @@ struct spy_hip_llama {
     hipStream_t own_stream = nullptr;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     double timed_ms = 0.0; int timed_pass = 0;
+    // persistent single-kernel pass
+    bool mega = false;
+    mega_layer *mega_layers = nullptr;
+    mega_sync *msync = nullptr;
+    long long *mega_dbg = nullptr;
     std::vector<void *> owned;
 };
 
+
+// shapes the one-row-per-wave kernels take
+static inline bool wave_ok(const spy_hip_llama *m) {
+    const spy_hip_llama_desc &c = m->desc;
+    return c.n_embd % 64 == 0 && c.n_embd <= 4096 && c.n_ff % 64 == 0 && c.n_ff <= 16384 && m->hd <= WGV_THREADS && m->hd % 2 == 0 && c.n_embd % 2 == 0;
+}
 
 enum { K_QKV = 0, K_SCORES, K_PV, K_WO, K_GATEUP, K_DOWN, K_HEAD, K_COUNT };
 
@@ -40,3 +53,7 @@ enum { K_QKV = 0, K_SCORES, K_PV, K_WO, K_GATEUP, K_DOWN, K_HEAD, K_COUNT };
 // With m->dry set nothing is launched: the call only sizes the persistent grids.
 int spy_enqueue_kernel_q4_0(spy_hip_llama *m, hipStream_t st, int which, int il);
 int spy_enqueue_kernel_q8_0(spy_hip_llama *m, hipStream_t st, int which, int il);
+// The persistent kernel covering embedding .. output head of one pass.  probe: only check that the
+// kernel for this shape exists and that one workgroup per compute unit is resident.
+int spy_enqueue_mega_q4_0(spy_hip_llama *m, hipStream_t st, bool probe);
+int spy_enqueue_mega_q8_0(spy_hip_llama *m, hipStream_t st, bool probe);

@@ -153,6 +153,10 @@ class Engine:
                                                    out.ctypes.data, 1 if use_graph else 0), "spy_hip_llama_decode_greedy")
         return out
 
+    def uses_single_kernel(self):
+        """True when single-token passes run as one persistent kernel"""
+        return self.L.spy_hip_llama_single_kernel(self.handle) == 1
+
     def timing(self):
         ms, n = C.c_float(), C.c_int32()
         H.check(self.L.spy_hip_llama_timing(self.handle, C.byref(ms), C.byref(n)), "spy_hip_llama_timing")
