@@ -90,6 +90,7 @@ SIGNATURES = {
     "spy_hip_quantize_q8_0": (_i32, [_vp, _vp, _i64, _vp, _i64, _i64]),
     "spy_hip_quantize_f16": (_i32, [_vp, _vp, _i64, _vp, _i64, _i64]),
     "spy_hip_gemv_q8_0act": (_i32, [_vp, _i32, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64]),
+    "spy_hip_gemm_q8_0act": (_i32, [_vp, _i32, _vp, _vp, _vp, _i64, _i64, _i64, _i64]),
     "spy_hip_block_dots": (_i32, [_vp, _i32, _vp, _vp, _vp, _i64, _i64]),
     "spy_hip_llama_create": (_i32, [C.POINTER(LlamaDesc), C.POINTER(_vp)]),
     "spy_hip_llama_destroy": (_i32, [_vp]),

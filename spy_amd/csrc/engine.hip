@@ -330,7 +330,7 @@ extern "C" int spy_hip_llama_forward(spy_hip_llama *m, void *stream, const int32
     }
     // longer passes in chunks: each chunk attends to everything before it, so the result per token
     // is that of one pass over the whole prompt
-    const int CH = 256;
+    const int CH = 1024;
     for (int t0 = 0; t0 < n_token; t0 += CH) {
         const int tc = n_token - t0 < CH ? n_token - t0 : CH;
         RC_TRY(forward_ops(m, st, tokens_host + t0, tc, n_past + t0, logits_host ? logits_host + (size_t)t0 * m->desc.n_vocab : nullptr));

@@ -1,0 +1,263 @@
+// Matrix x matrix for passes over many tokens (prompts): the same dots as the GEMV, but with every
+// weight tile reused for 128 tokens, on the matrix cores.
+//
+//  * gemm_q8act_kernel: Q4_0 / Q8_0 weight rows x Q8_0 activation rows.  Replaces the
+//    Dot<Q4_0,Q8_0> / Dot<Q8_0,Q8_0> loops of OperatorMatMulImpl::execute for ne11 > 1
+//    (backend/host/operator/mat.cpp:130-143, backend/host/include/simd/vec_dot.h:42-115 in the Spy
+//    tree).  One v_mfma_i32_32x32x32_i8 contracts exactly one 32-element quantization block for a
+//    32 x 32 output tile, so the int32 block dots are exact; each is then scaled by
+//    h2f(d_w) * h2f(d_x) and accumulated in fp32 like the reference's fma (vec_dot.h:76-79).
+//    Nibbles are unpacked to int8 (n - 8) on the way into LDS.
+//  * gemm_f16_kernel: fp16 rows x fp16 rows with fp32 accumulation (Dot<FP16,FP16>,
+//    vec_dot.h:117-146) for the attention products of a prompt pass: strided left operand (the K cache
+//    view, the transposed V cache view), right operand converted to fp16 by the caller.
+//
+// Both: 256 threads = 2 x 2 waves, 128 x 128 output tile per workgroup, each wave 2 x 2 MFMA tiles
+// of 32 x 32; operands double-buffered in LDS with a row stride of 80 bytes (conflict-free for the
+// 128-bit fragment reads of 32 consecutive rows).
+#include "common.cuh"
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+#define GEMM_TILE 128
+#define GEMM_ROWB 80             // bytes per LDS row: 64 payload + 16 pad
+
+// 32-bit word of 4 packed nibbles (already masked to 0..15 per byte) -> 4 int8 of (n - 8)
+static __device__ __forceinline__ uint32_t nib_m8(uint32_t lo) { return (lo + 0x78787878u) ^ 0x80808080u; }
+
+template <int WT>
+__global__ __launch_bounds__(256, 2) void gemm_q8act_kernel(const uint8_t *__restrict__ W, const uint8_t *__restrict__ xq, float *__restrict__ dst,
+                                                            int M, int K, int T, int64_t dst_stride) {
+    constexpr int PAIR_DW = (WT == SPY_HIP_Q4_0) ? 9 : 17;       // dwords per pair of weight blocks
+    constexpr int HALF_DW = (WT == SPY_HIP_Q4_0) ? 5 : 9;        // dwords that cover one block of the pair
+    __shared__ __attribute__((aligned(16))) uint8_t sA[2][GEMM_TILE * GEMM_ROWB];
+    __shared__ __attribute__((aligned(16))) uint8_t sB[2][GEMM_TILE * GEMM_ROWB];
+    __shared__ __attribute__((aligned(16))) float sAd[2][2][GEMM_TILE];      // [buffer][block of the pair][row]
+    __shared__ __attribute__((aligned(16))) float sBd[2][2][GEMM_TILE];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
+    const int m0 = blockIdx.x * GEMM_TILE, t0 = blockIdx.y * GEMM_TILE;
+    const int nstage = K / 64;
+    const size_t RBw = (size_t)(K / 32) * (WT == SPY_HIP_Q4_0 ? 18 : 34), RBx = (size_t)(K / 32) * 34;
+
+    // Every thread moves one weight block and one activation block per stage: row tid & 127, block
+    // tid >> 7 of the 4-byte aligned block pair (block 0 starts at byte 0, block 1 in the middle of a
+    // dword: the dwords that cover it are loaded and the scale / quants shifted out).  Rows beyond
+    // the matrix re-read its last row (their outputs are never stored).
+    const int lrow = tid & 127, half = tid >> 7;
+    const uint32_t *gA = (const uint32_t *)(W + (size_t)min(m0 + lrow, M - 1) * RBw) + half * (HALF_DW - 1);
+    const uint32_t *gB = (const uint32_t *)(xq + (size_t)min(t0 + lrow, T - 1) * RBx) + half * 8;
+    uint32_t rawA[HALF_DW], rawB[9];
+    auto gload = [&](int s) {
+#pragma unroll
+        for (int i = 0; i < HALF_DW; i++) rawA[i] = gA[(size_t)s * PAIR_DW + i];
+#pragma unroll
+        for (int i = 0; i < 9; i++) rawB[i] = gB[(size_t)s * 17 + i];
+    };
+    // one Q8_0 block held in 9 dwords -> scale + 8 dwords of int8
+    auto split_q8 = [&](const uint32_t *raw, float &d, uint32_t *q) {
+        d = h2f((uint16_t)(half ? raw[0] >> 16 : raw[0] & 0xFFFFu));
+#pragma unroll
+        for (int i = 0; i < 8; i++) q[i] = half ? raw[i + 1] : __builtin_amdgcn_alignbit(raw[i + 1], raw[i], 16);
+    };
+    auto unpack = [&](int b) {
+        uint32_t q[8];
+        float d;
+        if constexpr (WT == SPY_HIP_Q4_0) {
+            // {d, qs[16]}: element j = low nibble of qs[j], element j+16 = high nibble (quant.h:25-28); stored as n - 8
+            d = h2f((uint16_t)(half ? rawA[0] >> 16 : rawA[0] & 0xFFFFu));
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const uint32_t n = half ? rawA[i + 1] : __builtin_amdgcn_alignbit(rawA[i + 1], rawA[i], 16);
+                q[i] = nib_m8(n & 0x0F0F0F0Fu);
+                q[4 + i] = nib_m8((n >> 4) & 0x0F0F0F0Fu);
+            }
+        } else split_q8(rawA, d, q);
+        uint4 *ra = (uint4 *)(sA[b] + lrow * GEMM_ROWB + half * 32);
+        ra[0] = make_uint4(q[0], q[1], q[2], q[3]); ra[1] = make_uint4(q[4], q[5], q[6], q[7]);
+        sAd[b][half][lrow] = d;
+        split_q8(rawB, d, q);                                // {d, qs[32]} (quant.h:139-142)
+        uint4 *rb = (uint4 *)(sB[b] + lrow * GEMM_ROWB + half * 32);
+        rb[0] = make_uint4(q[0], q[1], q[2], q[3]); rb[1] = make_uint4(q[4], q[5], q[6], q[7]);
+        sBd[b][half][lrow] = d;
+    };
+
+    float acc[2][2][16];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+
+    gload(0);
+    unpack(0);
+    __syncthreads();
+    for (int s = 0; s < nstage; s++) {
+        const int b = s & 1;
+        gload(min(s + 1, nstage - 1));                    // unconditional: the last stage re-reads itself
+#pragma unroll 1
+        for (int blk = 0; blk < 2; blk++) {
+            v4i fa[2], fb[2];
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                fa[i] = *(const v4i *)(sA[b] + (wm * 64 + i * 32 + (lane & 31)) * GEMM_ROWB + blk * 32 + (lane >> 5) * 16);
+                fb[i] = *(const v4i *)(sB[b] + (wn * 64 + i * 32 + (lane & 31)) * GEMM_ROWB + blk * 32 + (lane >> 5) * 16);
+            }
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                float dw[16];
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const float4 v = *(const float4 *)&sAd[b][blk][wm * 64 + i * 32 + g * 8 + (lane >> 5) * 4];
+                    dw[4 * g] = v.x; dw[4 * g + 1] = v.y; dw[4 * g + 2] = v.z; dw[4 * g + 3] = v.w;
+                }
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    const float dx = sBd[b][blk][wn * 64 + j * 32 + (lane & 31)];
+                    v16i z = {0};
+                    const v16i I = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], z, 0, 0, 0);
+#pragma unroll
+                    for (int r = 0; r < 16; r++) acc[i][j][r] = fmaf(dw[r] * dx, (float)I[r], acc[i][j][r]);
+                }
+            }
+        }
+        if (s + 1 < nstage) unpack(b ^ 1);
+        __syncthreads();
+    }
+    // C layout of the 32x32 MFMA: lane -> column (token) lane & 31; register r -> row (r / 4) * 8 + (lane >> 5) * 4 + (r & 3)
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int t = t0 + wn * 64 + j * 32 + (lane & 31);
+            if (t < T) {
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const int m = m0 + wm * 64 + i * 32 + g * 8 + (lane >> 5) * 4;
+                    float *o = dst + (size_t)t * dst_stride + m;
+                    if (m + 3 < M && (((uintptr_t)o) & 15) == 0) *(float4 *)o = make_float4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
+                    else {
+#pragma unroll
+                        for (int e = 0; e < 4; e++) if (m + e < M) o[e] = acc[i][j][4 * g + e];
+                    }
+                }
+            }
+        }
+}
+
+extern "C" int spy_hip_gemm_q8_0act(void *stream, int wtype, const void *w_dev, const void *xq_dev, float *dst_dev,
+                                    int64_t M, int64_t K, int64_t T, int64_t dst_stride) {
+    SPY_CHECK_ARG(w_dev && xq_dev && dst_dev && M > 0 && K > 0 && T > 0 && dst_stride >= M);
+    SPY_CHECK_ARG(K % 64 == 0);
+    SPY_CHECK_ARG((M + GEMM_TILE - 1) / GEMM_TILE <= 0x7fffffff && (T + GEMM_TILE - 1) / GEMM_TILE <= 65535);
+    const dim3 grid((unsigned)((M + GEMM_TILE - 1) / GEMM_TILE), (unsigned)((T + GEMM_TILE - 1) / GEMM_TILE));
+    hipStream_t st = (hipStream_t)stream;
+    if (wtype == SPY_HIP_Q4_0) gemm_q8act_kernel<SPY_HIP_Q4_0><<<grid, dim3(256), 0, st>>>((const uint8_t *)w_dev, (const uint8_t *)xq_dev, dst_dev, (int)M, (int)K, (int)T, dst_stride);
+    else if (wtype == SPY_HIP_Q8_0) gemm_q8act_kernel<SPY_HIP_Q8_0><<<grid, dim3(256), 0, st>>>((const uint8_t *)w_dev, (const uint8_t *)xq_dev, dst_dev, (int)M, (int)K, (int)T, dst_stride);
+    else return SPY_HIP_EUNSUPPORTED;
+    return SPY_LAUNCH_RC();
+}
+
+// ---- fp16 x fp16 -> fp32 ----------------------------------------------------------------------------
+// dst[batch][n][m] = sum_k A[batch][m][k] * B[batch][n][k];  A: fp16, k contiguous, row stride a_nb1 and
+// batch stride a_nb2 in bytes (16-byte aligned rows); B: fp16 [batch][N][K] contiguous (K % 8 == 0);
+// dst: f32, m contiguous, d_nb1 / d_nb2 in bytes.
+struct gemm_f16_args {
+    const uint8_t *A; const uint16_t *B; uint8_t *dst;
+    int M, N, K;
+    int64_t a_nb1, a_nb2, d_nb1, d_nb2;
+};
+
+__global__ __launch_bounds__(256) void gemm_f16_kernel(gemm_f16_args a) {
+    __shared__ __attribute__((aligned(16))) uint8_t sA[2][GEMM_TILE * GEMM_ROWB];     // 128 rows x 32 halfs (+ pad)
+    __shared__ __attribute__((aligned(16))) uint8_t sB[2][GEMM_TILE * GEMM_ROWB];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
+    const int m0 = blockIdx.x * GEMM_TILE, n0 = blockIdx.y * GEMM_TILE, bz = blockIdx.z;
+    const int K = a.K, nstage = (K + 31) / 32;
+    const uint8_t *Ab = a.A + (size_t)bz * a.a_nb2;
+    const uint16_t *Bb = a.B + (size_t)bz * a.N * K;
+    // each thread moves two 16-byte chunks of A and two of B per stage: chunk c = tid + i*256 -> row c / 4, k-chunk c % 4
+    uint4 ra[2], rb[2];
+    auto gload = [&](int s) {
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const int c = tid + i * 256, row = c >> 2, kc = c & 3, k = s * 32 + kc * 8;
+            const int kk = min(k, K - 8);                                           // unconditional loads; chunks past K are zeroed
+            ra[i] = *(const uint4 *)(Ab + (size_t)min(m0 + row, a.M - 1) * a.a_nb1 + (size_t)kk * 2);
+            rb[i] = *(const uint4 *)(Bb + (size_t)min(n0 + row, a.N - 1) * K + kk);
+            if (k >= K) { ra[i] = make_uint4(0, 0, 0, 0); rb[i] = make_uint4(0, 0, 0, 0); }
+        }
+    };
+    auto stash = [&](int b) {
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const int c = tid + i * 256, row = c >> 2, kc = c & 3;
+            *(uint4 *)(sA[b] + row * GEMM_ROWB + kc * 16) = ra[i];
+            *(uint4 *)(sB[b] + row * GEMM_ROWB + kc * 16) = rb[i];
+        }
+    };
+    v16f acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+    gload(0);
+    stash(0);
+    __syncthreads();
+    for (int s = 0; s < nstage; s++) {
+        const int b = s & 1;
+        gload(min(s + 1, nstage - 1));
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++) {
+            v8h fa[2], fb[2];
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                fa[i] = *(const v8h *)(sA[b] + (wm * 64 + i * 32 + (lane & 31)) * GEMM_ROWB + ks * 32 + (lane >> 5) * 16);
+                fb[i] = *(const v8h *)(sB[b] + (wn * 64 + i * 32 + (lane & 31)) * GEMM_ROWB + ks * 32 + (lane >> 5) * 16);
+            }
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+        }
+        if (s + 1 < nstage) stash(b ^ 1);
+        __syncthreads();
+    }
+    uint8_t *Db = a.dst + (size_t)bz * a.d_nb2;
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int n = n0 + wn * 64 + j * 32 + (lane & 31);
+            if (n < a.N) {
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const int m = m0 + wm * 64 + i * 32 + g * 8 + (lane >> 5) * 4;
+                    float *o = (float *)(Db + (size_t)n * a.d_nb1) + m;
+                    if (m + 3 < a.M && (((uintptr_t)o) & 15) == 0) *(float4 *)o = make_float4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
+                    else {
+#pragma unroll
+                        for (int e = 0; e < 4; e++) if (m + e < a.M) o[e] = acc[i][j][4 * g + e];
+                    }
+                }
+            }
+        }
+}
+
+// used by the MatMul operator for (F16, F16) operands with many right-hand rows
+int spy_gemm_f16_launch(hipStream_t st, const void *A, int64_t a_nb1, int64_t a_nb2, const uint16_t *B, void *dst, int64_t d_nb1, int64_t d_nb2,
+                        int64_t M, int64_t N, int64_t K, int64_t nbatch) {
+    SPY_CHECK_ARG(A && B && dst && M > 0 && N > 0 && K >= 8 && nbatch > 0 && K % 8 == 0);
+    SPY_CHECK_ARG(a_nb1 % 16 == 0 && a_nb2 % 16 == 0 && ((uintptr_t)A & 15) == 0 && ((uintptr_t)B & 15) == 0);
+    SPY_CHECK_ARG((N + GEMM_TILE - 1) / GEMM_TILE <= 65535 && nbatch <= 65535);
+    gemm_f16_args a;
+    a.A = (const uint8_t *)A; a.B = B; a.dst = (uint8_t *)dst; a.M = (int)M; a.N = (int)N; a.K = (int)K;
+    a.a_nb1 = a_nb1; a.a_nb2 = a_nb2; a.d_nb1 = d_nb1; a.d_nb2 = d_nb2;
+    gemm_f16_kernel<<<dim3((unsigned)((M + GEMM_TILE - 1) / GEMM_TILE), (unsigned)((N + GEMM_TILE - 1) / GEMM_TILE), (unsigned)nbatch), dim3(256), 0, st>>>(a);
+    return SPY_LAUNCH_RC();
+}

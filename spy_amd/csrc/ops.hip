@@ -383,6 +383,9 @@ __global__ __launch_bounds__(256) void matmul_f16_kernel(tdesc w, const uint16_t
     if (lane == 0) *(float *)at(d, i01, i11, i02, i03) = acc;
 }
 
+int spy_gemm_f16_launch(hipStream_t st, const void *A, int64_t a_nb1, int64_t a_nb2, const uint16_t *B, void *dst, int64_t d_nb1, int64_t d_nb2,
+                        int64_t M, int64_t N, int64_t K, int64_t nbatch);      // gemm.hip
+
 static int mid_type(int t0, int t1) {                                        // target_buffer_type (mat.cpp:32-42) + K-quants
     if (t0 == t1) return t0;
     if (t0 == SPY_HIP_F16 && t1 == SPY_HIP_F32) return SPY_HIP_F16;
@@ -444,12 +447,24 @@ extern "C" int spy_hip_op_matmul(void *stream, const spy_hip_tensor *w, const sp
                 const uint8_t *wp = (const uint8_t *)w->data + i2 * w->nb[2] + i3 * w->nb[3];
                 const uint8_t *xp = xm + ((i3 * ne12 + i2) * ne11) * mid_row;
                 float *dp = (float *)((uint8_t *)dst->data + i2 * dst->nb[2] + i3 * dst->nb[3]);
-                int rc = spy_hip_gemv_q8_0act(stream, t0, wp, xp, dp, nullptr, ne01, ne00, ne11, dst->nb[1] / 4);
+                // many activation rows: matrix cores; few: the bandwidth-bound row kernels
+                const bool mfma = ne11 >= 16 && (t0 == SPY_HIP_Q4_0 || t0 == SPY_HIP_Q8_0) && ne00 % 64 == 0;
+                int rc = mfma ? spy_hip_gemm_q8_0act(stream, t0, wp, xp, dp, ne01, ne00, ne11, dst->nb[1] / 4)
+                              : spy_hip_gemv_q8_0act(stream, t0, wp, xp, dp, nullptr, ne01, ne00, ne11, dst->nb[1] / 4);
                 if (rc) return rc;
             }
         return 0;
     }
     SPY_CHECK_ARG(w->nb[0] == 2);
+    if (ne11 >= 16 && ne01 >= 16 && ne00 % 8 == 0 && w->nb[1] % 16 == 0 && w->nb[2] % 16 == 0 && w->nb[3] % 16 == 0 &&
+        ((uintptr_t)w->data & 15) == 0 && ((uintptr_t)xm & 15) == 0 && dst->nb[1] % 4 == 0 && dst->nb[2] % 4 == 0 && ne02 <= 65535) {
+        for (int64_t i3 = 0; i3 < ne03; i3++) {            // prompt-sized attention products: fp16 MFMA
+            int rc = spy_gemm_f16_launch(st, (const uint8_t *)w->data + i3 * w->nb[3], w->nb[1], w->nb[2], (const uint16_t *)xm + i3 * ne12 * ne11 * ne00,
+                                         (uint8_t *)dst->data + i3 * dst->nb[3], dst->nb[1], dst->nb[2], ne01, ne11, ne00, ne02);
+            if (rc) return rc;
+        }
+        return 0;
+    }
     const int64_t total = ne01 * ne11 * ne02 * ne03;
     CHECK_GRID(total, 4);
     matmul_f16_kernel<<<dim3(grid_for(total, 4)), dim3(256), 0, st>>>(mk(w), (const uint16_t *)xm, mk(dst), ne11, total);
