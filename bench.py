@@ -8,6 +8,7 @@ Prints ONE JSON line (see the keys below).  The CPU baseline is the oracle (a po
 host backend path) timed on this machine's cores on a bounded sample of the same workload.
 """
 import argparse
+import ctypes as C
 import json
 import os
 import sys
@@ -34,6 +35,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-steps", type=int, default=8)
     ap.add_argument("--layers", type=int, default=32, help="debug only: fewer layers (result is then not the headline config)")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also launch a plain copy kernel over 256 MiB three times (a known-size dispatch to scale profiler byte counters by)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs the token loop on ONE GPU (no sharding, no collectives); --gpus %d is not supported" % args.gpus,
@@ -70,7 +73,17 @@ def main():
             eng.write_buffer("v_cache", il, v.view(np.uint16))
         first = int(prompt[-1])
     H.sync()
-    log("prefill (%s) of %d tokens: %.1f s" % (args.prefill, fill, time.time() - t0))
+    prefill_s = time.time() - t0
+    log("prefill (%s) of %d tokens: %.2f s" % (args.prefill, fill, prefill_s))
+    if args.calibrate:
+        n = 64 << 20
+        src, dst = H.DeviceBuffer(n * 4), H.DeviceBuffer(n * 4)
+        src.fill(0)
+        ts, td = H.tensor(src, H.F32, [n]), H.tensor(dst, H.F32, [n])
+        for _ in range(3):
+            H.check(H.load().spy_hip_op_dup(None, C.byref(ts), C.byref(td)), "spy_hip_op_dup")
+        H.sync()
+        log("calibration: dup_kernel over %d bytes read + %d bytes written, 3 launches" % (n * 4, n * 4))
 
     # warm-up (also captures the HIP graph), then the timed region: exactly `steps` passes
     pos = fill
@@ -106,7 +119,7 @@ def main():
         log("  %-8s %8.2f us  %7.1f GB/s  (%.1f%% of 8 TB/s)" % (k, us, alg[k] / us / 1e3, alg[k] / us / 1e3 / 80))
     dom = "gate_up"
     achieved = alg[dom] / (per_kernel[dom] * 1e-6) / 1e9
-    roofline = {"kernel": "fused_gemv_kernel<Q4_0, gate|up + SiLU>", "bound": "hbm", "achieved": round(achieved, 1), "peak": 8000.0,
+    roofline = {"kernel": "wave_gemv_kernel<Q4_0, gate|up + SiLU>", "bound": "hbm", "achieved": round(achieved, 1), "peak": 8000.0,
                 "unit": "GB/s", "frac": round(achieved / 8000.0, 4), "traffic": None,
                 "bytes_per_launch": alg[dom], "us_per_launch": round(per_kernel[dom], 3)}
 
@@ -139,6 +152,7 @@ def main():
                                "f16 KV cache prefilled to %d tokens (%s), greedy single-sequence decode" % (fill, args.prefill),
                    "n_layer": cfg.n_layer, "n_kv_first": pos + 1, "n_kv_last": pos + steps, "bytes_per_token": int(bytes_per_token)},
         "hbm_roofline_frac": round(frac, 4), "ms_per_step_hip_events": round(ev_ms, 4),
+        "prefill": {"tokens": fill, "seconds": round(prefill_s, 3), "tok_s": round(fill / prefill_s, 1)} if args.prefill == "real" else None,
         "kernel_us": {k: round(v, 2) for k, v in per_kernel.items()},
         "roofline": roofline, "cpu_baseline": cpu,
     }

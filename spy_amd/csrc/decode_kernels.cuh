@@ -157,10 +157,17 @@ __global__ __launch_bounds__(GEMV_THREADS) void fused_gemv_kernel(fused_args a) 
 //   EPI_RESID / EPI_STORE: wave -> NR rows r = gw + k*NW of W0
 #define WGV_THREADS 1024
 #define WGV_WAVES 16
+#ifndef WGV_DEPTH_QKV
+#define WGV_DEPTH_QKV 2
+#endif
+#ifndef WGV_DEPTH
+#define WGV_DEPTH 3             // rows per wave requested ahead of their use
+#endif
 template <int WT, int NITK, int NR, int EPI>
 __global__ __launch_bounds__(WGV_THREADS) void wave_gemv_kernel(fused_args a) {
     constexpr bool NORM = (EPI != EPI_RESID);
     constexpr int NB = EPI == EPI_QKV ? 3 : (EPI == EPI_GATEUP ? 2 * NR : NR);
+    constexpr int DEPTH = EPI == EPI_QKV ? WGV_DEPTH_QKV : WGV_DEPTH;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     __shared__ float s_red[WGV_WAVES];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -178,29 +185,27 @@ __global__ __launch_bounds__(WGV_THREADS) void wave_gemv_kernel(fused_args a) {
     }
     float rope_v = 0.0f, side[EPI == EPI_RESID ? NR : 1];
     if constexpr (EPI == EPI_QKV) rope_v = a.rope_cs[min(tid, a.hd - 1)];
+    // Row k of this wave.  Only WGV_DEPTH rows per wave are requested ahead of their use: the compute
+    // unit's vector-memory queue is finite, and a wave that tries to put all its rows in flight at
+    // once sits in the issue stage until the queue drains (most of the kernel), holding up the staging
+    // barriers of everybody else.
     wtile<WT, NITK> t[NB];
-    if constexpr (EPI == EPI_QKV) {
-        const int j = gw % a.d;
-        const uint8_t *p0 = 2 * j < a.d ? a.W0 + (size_t)(2 * j) * RB : a.W1 + (size_t)(2 * j - a.d) * RB;
-        load_tile<WT, 64, NITK>(t[0], p0, npair, lane);
-        load_tile<WT, 64, NITK>(t[1], p0 + RB, npair, lane);
-        load_tile<WT, 64, NITK>(t[2], a.W2 + (size_t)j * RB, npair, lane);
-    } else if constexpr (EPI == EPI_GATEUP) {
-        const int F = a.M / 2;
-#pragma unroll
-        for (int k = 0; k < NR; k++) {
-            const int u = gw + k * NW, i = u < F ? u : gw % F;
-            load_tile<WT, 64, NITK>(t[2 * k], a.W0 + (size_t)i * RB, npair, lane);
-            load_tile<WT, 64, NITK>(t[2 * k + 1], a.W1 + (size_t)i * RB, npair, lane);
-        }
-    } else {
-#pragma unroll
-        for (int k = 0; k < NR; k++) {
+    auto issue = [&](int k) {
+        if constexpr (EPI == EPI_QKV) {
+            const int j = gw % a.d;
+            const uint8_t *p0 = 2 * j < a.d ? a.W0 + (size_t)(2 * j) * RB : a.W1 + (size_t)(2 * j - a.d) * RB;
+            load_tile<WT, 64, NITK>(t[k], k == 2 ? a.W2 + (size_t)j * RB : p0 + (size_t)k * RB, npair, lane);
+        } else if constexpr (EPI == EPI_GATEUP) {
+            const int F = a.M / 2, u = gw + (k >> 1) * NW, i = u < F ? u : gw % F;
+            load_tile<WT, 64, NITK>(t[k], ((k & 1) ? a.W1 : a.W0) + (size_t)i * RB, npair, lane);
+        } else {
             const int u = gw + k * NW, r = u < a.M ? u : gw % a.M;
             load_tile<WT, 64, NITK>(t[k], a.W0 + (size_t)r * RB, npair, lane);
             if constexpr (EPI == EPI_RESID) side[k] = a.resid[r];
         }
-    }
+    };
+#pragma unroll
+    for (int k = 0; k < NB; k++) if (k < DEPTH) issue(k);
 
     // 3. stage the activations: RMSNorm * weight (non-linear.cpp:216-219 and the separate Mul node) or plain, then Q8_0
     int8_t *s_q = (int8_t *)smem;
@@ -235,38 +240,42 @@ __global__ __launch_bounds__(WGV_THREADS) void wave_gemv_kernel(fused_args a) {
     }
     __syncthreads();
     staged_act act; act.q = s_q; act.meta = s_meta;
-    auto row_dot = [&](const wtile<WT, NITK> &tl) -> float {
-        float acc[1] = {0.0f};
-        dot_tile<WT, 64, NITK, 1>(tl, &act, npair, lane, acc, nullptr);
-        return group_sum<64>(acc[0]);
-    };
+    act_frag<NITK> af;                                    // this lane's activations: the same for every row
+    load_act_frag<NITK>(af, act, npair, lane);
+    // partial dots of all rows (requesting the row WGV_DEPTH ahead before each), then their wave reductions
+    // (independent chains); totals land in lane 63
+    float s[NB];
+#pragma unroll
+    for (int k = 0; k < NB; k++) {
+        if (k + DEPTH < NB) issue(k + DEPTH);
+        s[k] = dot_row_frag<WT, NITK>(t[k], af, npair, lane);
+    }
+#pragma unroll
+    for (int k = 0; k < NB; k++) s[k] = wave_total_lane63(s[k]);
 
-    // 4. dots and epilogues
+    // 4. epilogues (lane 63 holds the totals)
     if constexpr (EPI == EPI_QKV) {
-        const float s0 = row_dot(t[0]), s1 = row_dot(t[1]), s2 = row_dot(t[2]);
-        if (lane == 0 && gw < a.d) {
+        if (lane == 63 && gw < a.d) {
             const int j = gw, row = (2 * j) % a.d, k = (row % a.hd) >> 1, pos = a.st->pos;
             const float c = s_rope[2 * k], sn = s_rope[2 * k + 1];
             // (x0, x1) -> (x0*c - x1*s, x0*s + x1*c) on adjacent rows (non-linear.cpp:359-363)
-            const uint32_t pr = (uint32_t)f2h(s0 * c - s1 * sn) | ((uint32_t)f2h(s0 * sn + s1 * c) << 16);
+            const uint32_t pr = (uint32_t)f2h(s[0] * c - s[1] * sn) | ((uint32_t)f2h(s[0] * sn + s[1] * c) << 16);
             if (2 * j < a.d) ((uint32_t *)a.q16)[j] = pr;                                        // attn_score rounds Q to fp16 (mat.cpp:37)
             else ((uint32_t *)(a.kc + (size_t)pos * a.d))[j - a.d / 2] = pr;                      // KCache_cpy: [token][head][hd]
-            a.vc[(size_t)j * a.n_ctx + pos] = f2h(s2);                                           // VCache_cpy: [d][C] column pos
+            a.vc[(size_t)j * a.n_ctx + pos] = f2h(s[2]);                                         // VCache_cpy: [d][C] column pos
         }
     } else if constexpr (EPI == EPI_GATEUP) {
         const int F = a.M / 2;
 #pragma unroll
         for (int k = 0; k < NR; k++) {
-            const float g = row_dot(t[2 * k]), u = row_dot(t[2 * k + 1]);
             const int i = gw + k * NW;
-            if (lane == 0 && i < F) a.out[i] = u * silu_lut(g);                                   // Mul(ffn_up, silu(ffn_gate)) (ffn.cpp:24-35)
+            if (lane == 63 && i < F) a.out[i] = s[2 * k + 1] * silu_lut(s[2 * k]);                 // Mul(ffn_up, silu(ffn_gate)) (ffn.cpp:24-35)
         }
     } else {
 #pragma unroll
         for (int k = 0; k < NR; k++) {
-            const float s = row_dot(t[k]);
             const int r = gw + k * NW;
-            if (lane == 0 && r < a.M) { if constexpr (EPI == EPI_RESID) a.out[r] = s + side[k]; else a.out[r] = s; }
+            if (lane == 63 && r < a.M) { if constexpr (EPI == EPI_RESID) a.out[r] = s[k] + side[k]; else a.out[r] = s[k]; }
         }
     }
 }
@@ -302,6 +311,9 @@ __global__ __launch_bounds__(256) void embed_kernel(dev_state *st, const uint8_t
 // flight per thread.  t = (K.q + mask) * scale with mask = 0 for every cached token of a
 // single-token pass (llama.cpp:248-257), i.e. t = dot * scale.
 #define ATT_TCH 8
+#ifndef ATT_DEPTH
+#define ATT_DEPTH 3             // key loads per thread requested ahead of their use
+#endif
 __global__ __launch_bounds__(256) void attn_scores_kernel(const dev_state *st, const uint16_t *__restrict__ q16, const uint16_t *__restrict__ kc,
                                                           float *__restrict__ scores, int n_head, int n_ctx, float scale) {
     const int n_kv = st->pos + 1;
@@ -310,40 +322,37 @@ __global__ __launch_bounds__(256) void attn_scores_kernel(const dev_state *st, c
     const int d = n_head * 128;
     const int piece = threadIdx.x & 15, hsel = threadIdx.x >> 4;     // 2 x 16 heads per pass over the workgroup
     for (int h0 = 0; h0 < n_head; h0 += 32) {
-        uint4 kv[2][ATT_TCH];
-        uint4 qv[2];
+        // q first, then the keys with ATT_DEPTH loads per thread ahead of their use; every load
+        // unconditional (heads / tokens beyond the range re-read the last one, results not stored)
+        uint4 qv[2], kv[2 * ATT_TCH];
+#pragma unroll
+        for (int hh = 0; hh < 2; hh++) qv[hh] = *(const uint4 *)(q16 + min(h0 + hsel + 16 * hh, n_head - 1) * 128 + piece * 8);
+        auto fetch = [&](int idx) {
+            const int head = min(h0 + hsel + 16 * (idx / ATT_TCH), n_head - 1), tok = min(t0 + idx % ATT_TCH, n_kv - 1);
+            kv[idx] = *(const uint4 *)(kc + (size_t)tok * d + head * 128 + piece * 8);
+        };
+#pragma unroll
+        for (int idx = 0; idx < ATT_DEPTH; idx++) fetch(idx);
+        float qf[2][8];
 #pragma unroll
         for (int hh = 0; hh < 2; hh++) {
-            const int head = h0 + hsel + 16 * hh;
-            if (head < n_head) {
-#pragma unroll
-                for (int tt = 0; tt < ATT_TCH; tt++)
-                    if (t0 + tt < n_kv) kv[hh][tt] = *(const uint4 *)(kc + (size_t)(t0 + tt) * d + head * 128 + piece * 8);
-                qv[hh] = *(const uint4 *)(q16 + head * 128 + piece * 8);
-            }
-        }
-#pragma unroll
-        for (int hh = 0; hh < 2; hh++) {
-            const int head = h0 + hsel + 16 * hh;
-            const bool hok = head < n_head;
-            float qf[8];
             const uint32_t qw[4] = {qv[hh].x, qv[hh].y, qv[hh].z, qv[hh].w};
 #pragma unroll
-            for (int j = 0; j < 4; j++) { qf[2 * j] = h2f((uint16_t)(qw[j] & 0xFFFFu)); qf[2 * j + 1] = h2f((uint16_t)(qw[j] >> 16)); }
+            for (int j = 0; j < 4; j++) { qf[hh][2 * j] = h2f((uint16_t)(qw[j] & 0xFFFFu)); qf[hh][2 * j + 1] = h2f((uint16_t)(qw[j] >> 16)); }
+        }
 #pragma unroll
-            for (int tt = 0; tt < ATT_TCH; tt++) {
-                float s = 0.0f;
-                if (hok && t0 + tt < n_kv) {
-                    const uint32_t kw[4] = {kv[hh][tt].x, kv[hh][tt].y, kv[hh][tt].z, kv[hh][tt].w};
+        for (int idx = 0; idx < 2 * ATT_TCH; idx++) {
+            if (idx + ATT_DEPTH < 2 * ATT_TCH) fetch(idx + ATT_DEPTH);
+            const int hh = idx / ATT_TCH, tt = idx % ATT_TCH, head = h0 + hsel + 16 * hh;
+            const uint32_t kw[4] = {kv[idx].x, kv[idx].y, kv[idx].z, kv[idx].w};
+            float s = 0.0f;
 #pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        s = fmaf(h2f((uint16_t)(kw[j] & 0xFFFFu)), qf[2 * j], s);
-                        s = fmaf(h2f((uint16_t)(kw[j] >> 16)), qf[2 * j + 1], s);
-                    }
-                }
-                s = group_sum<16>(s);
-                if (hok && piece == 0 && t0 + tt < n_kv) scores[(size_t)head * n_ctx + t0 + tt] = s * scale;
+            for (int j = 0; j < 4; j++) {
+                s = fmaf(h2f((uint16_t)(kw[j] & 0xFFFFu)), qf[hh][2 * j], s);
+                s = fmaf(h2f((uint16_t)(kw[j] >> 16)), qf[hh][2 * j + 1], s);
             }
+            s = group_sum<16>(s);
+            if (head < n_head && piece == 0 && t0 + tt < n_kv) scores[(size_t)head * n_ctx + t0 + tt] = s * scale;
         }
     }
 }
@@ -357,6 +366,10 @@ __global__ __launch_bounds__(256) void attn_scores_kernel(const dev_state *st, c
 // KQV product (mat.cpp:37, vec_dot.h:117-146).
 #define PV_THREADS 1024
 #define PV_PIECES 10            // 128-bit pieces per lane per chunk: 10*64*8 = 5120 tokens per chunk
+#ifndef PV_DEPTH
+#define PV_DEPTH 3              // pieces per wave requested ahead of their use
+#endif
+#define PV_NS 5                 // scores per thread kept in registers (5 * 1024 = 5120 tokens; more are read in a loop)
 __global__ __launch_bounds__(PV_THREADS) void attn_pv_kernel(const dev_state *st, const float *__restrict__ scores, const uint16_t *__restrict__ vc,
                                                              float *__restrict__ attn_out, int n_ctx) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -367,15 +380,26 @@ __global__ __launch_bounds__(PV_THREADS) void attn_pv_kernel(const dev_state *st
     const int row = head * 128 + dgrp * 16 + wave;
     const uint16_t *vrow = vc + (size_t)row * n_ctx;
     const int n_pad = (n_kv + 7) & ~7, npiece = n_pad >> 3;
-    uint4 vv[PV_PIECES];
+    // Loads in the order they are needed and all unconditional (indices clamped into the row): the
+    // head's scores first, then the first PV_PIECES steps of the V^T row, so that the softmax below
+    // only waits for the scores while the row streams in.
+    const float *srow = scores + (size_t)head * n_ctx;
+    float sreg[PV_NS];
 #pragma unroll
-    for (int u = 0; u < PV_PIECES; u++) { const int pc = u * 64 + lane; if (pc < npiece) vv[u] = *(const uint4 *)(vrow + pc * 8); }
+    for (int u = 0; u < PV_NS; u++) sreg[u] = srow[min((int)threadIdx.x + u * PV_THREADS, n_ctx - 1)];
+    // only PV_DEPTH pieces per wave ahead of their use (the vector-memory queue of the compute unit is
+    // finite: a wave that asks for everything at once sits in the issue stage and delays the barriers below)
+    uint4 vv[PV_PIECES];
+    auto fetch = [&](int pc0, int u) { vv[u] = *(const uint4 *)(vrow + (size_t)min(pc0 + u * 64 + lane, n_ctx / 8 - 1) * 8); };
+#pragma unroll
+    for (int u = 0; u < PV_DEPTH; u++) fetch(0, u);
 
     float *s_t = (float *)smem;                               // n_ctx floats
     uint16_t *s_p = (uint16_t *)(smem + (size_t)n_ctx * 4);    // n_ctx halfs (+ pad)
-    const float *srow = scores + (size_t)head * n_ctx;
     float mx = -INFINITY;
-    for (int j = threadIdx.x; j < n_kv; j += PV_THREADS) { const float t = srow[j]; s_t[j] = t; mx = fmaxf(mx, t); }
+#pragma unroll
+    for (int u = 0; u < PV_NS; u++) { const int j = threadIdx.x + u * PV_THREADS; if (j < n_kv) { s_t[j] = sreg[u]; mx = fmaxf(mx, sreg[u]); } }
+    for (int j = threadIdx.x + PV_NS * PV_THREADS; j < n_kv; j += PV_THREADS) { const float t = srow[j]; s_t[j] = t; mx = fmaxf(mx, t); }
     mx = wave_max(mx);
     if (lane == 0) s_part[wave] = mx;
     __syncthreads();
@@ -396,13 +420,10 @@ __global__ __launch_bounds__(PV_THREADS) void attn_pv_kernel(const dev_state *st
     __syncthreads();
 
     float acc = 0.0f;
-    for (int pc0 = 0; pc0 < npiece; pc0 += PV_PIECES * 64) {
-        if (pc0 > 0) {
-#pragma unroll
-            for (int u = 0; u < PV_PIECES; u++) { const int pc = pc0 + u * 64 + lane; if (pc < npiece) vv[u] = *(const uint4 *)(vrow + pc * 8); }
-        }
+    auto consume = [&](int pc0) {
 #pragma unroll
         for (int u = 0; u < PV_PIECES; u++) {
+            if (u + PV_DEPTH < PV_PIECES) fetch(pc0, u + PV_DEPTH);
             const int pc = pc0 + u * 64 + lane;
             if (pc < npiece) {
                 const uint4 pp = *(const uint4 *)(s_p + pc * 8);
@@ -415,6 +436,12 @@ __global__ __launch_bounds__(PV_THREADS) void attn_pv_kernel(const dev_state *st
                 }
             }
         }
+    };
+    consume(0);                                                // the pieces requested at the top
+    for (int pc0 = PV_PIECES * 64; pc0 < npiece; pc0 += PV_PIECES * 64) {
+#pragma unroll
+        for (int u = 0; u < PV_DEPTH; u++) fetch(pc0, u);
+        consume(pc0);
     }
     acc = group_sum<64>(acc);
     if (lane == 0) attn_out[row] = acc;

@@ -45,6 +45,16 @@ template <int LPR> static __device__ __forceinline__ float group_sum(float v) {
     if constexpr (LPR >= 64) v += __shfl_xor(v, 32, SPY_WAVE);
     return v;
 }
+// Sum over the whole wave for ONE reader: after the in-row steps every lane of a 16-lane DPP row holds
+// its row total R0..R3; row_bcast15 adds R0 into row 1 and R2 into row 3, row_bcast31 adds R0+R1 into
+// rows 2, 3: lanes 48..63 end up with (R2+R3)+(R0+R1), the same additions as group_sum<64>, without
+// the two LDS permutes.  Only lane 63 (any of 48..63) may use the result.
+static __device__ __forceinline__ float wave_total_lane63(float v) {
+    v = dpp_add<0xB1>(v); v = dpp_add<0x4E>(v); v = dpp_add<0x141>(v); v = dpp_add<0x140>(v);
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x142, 0xA, 0xF, false));   // row_bcast15 -> rows 1, 3
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x143, 0xC, 0xF, false));   // row_bcast31 -> rows 2, 3
+    return v;
+}
 // max / sum over aligned groups of 8 lanes (one Q8_0 block = 8 lanes x 4 floats)
 static __device__ __forceinline__ float oct_max(float v) {
     v = dpp_max<0xB1>(v); v = dpp_max<0x4E>(v); v = dpp_max<0x141>(v);
@@ -243,6 +253,34 @@ static __device__ __forceinline__ int dot_q8_dwords(const uint32_t *n, const int
 
 // Partial dot of the lane's pairs of one weight row with NT staged activation columns.
 // dump (optional): int32 dot of every block, row-major [nblk] for activation column 0.
+// One block pair of a weight row (w: its PAIR_DW dwords) with the matching 64 int8 activations
+// (x0..x3: 16 bytes each) and their meta {scale bits, sum q} x 2: the two exact int32 block dots
+// (optionally dumped), scaled and accumulated like the reference's fma (vec_dot.h:76-79).
+template <int WT>
+static __device__ __forceinline__ float dot_pair(const uint32_t *w, const int4 x0, const int4 x1, const int4 x2, const int4 x3, const int4 mm,
+                                                 float acc, int32_t *dump2) {
+    int iA, iB;
+    float dA, dB;
+    if constexpr (WT == SPY_HIP_Q4_0) {
+        dA = h2f((uint16_t)(w[0] & 0xFFFFu)); dB = h2f((uint16_t)(w[4] >> 16));
+        const uint32_t a0 = __builtin_amdgcn_alignbit(w[1], w[0], 16), a1 = __builtin_amdgcn_alignbit(w[2], w[1], 16);
+        const uint32_t a2 = __builtin_amdgcn_alignbit(w[3], w[2], 16), a3 = __builtin_amdgcn_alignbit(w[4], w[3], 16);
+        iA = dot_q4_dwords(a0, a1, a2, a3, x0, x1) - 8 * mm.y;
+        iB = dot_q4_dwords(w[5], w[6], w[7], w[8], x2, x3) - 8 * mm.w;
+    } else {
+        dA = h2f((uint16_t)(w[0] & 0xFFFFu)); dB = h2f((uint16_t)(w[8] >> 16));
+        uint32_t a[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) a[i] = __builtin_amdgcn_alignbit(w[i + 1], w[i], 16);
+        iA = dot_q8_dwords(a, x0, x1);
+        iB = dot_q8_dwords(&w[9], x2, x3);
+    }
+    if (dump2) { dump2[0] = iA; dump2[1] = iB; }
+    acc = fmaf(dA * __int_as_float(mm.x), (float)iA, acc);
+    acc = fmaf(dB * __int_as_float(mm.z), (float)iB, acc);
+    return acc;
+}
+
 template <int WT, int LPR, int NIT, int NT>
 static __device__ __forceinline__ void dot_tile(const wtile<WT, NIT> &t, const staged_act *act, int npair, int l,
                                                 float acc[NT], int32_t *dump) {
@@ -250,39 +288,37 @@ static __device__ __forceinline__ void dot_tile(const wtile<WT, NIT> &t, const s
     for (int it = 0; it < NIT; it++) {
         const int p = it * LPR + l;
         if (p < npair) {
-            const uint32_t *w = t.w[it];
-            if constexpr (WT == SPY_HIP_Q4_0) {
-                const float dA = h2f((uint16_t)(w[0] & 0xFFFFu)), dB = h2f((uint16_t)(w[4] >> 16));
-                const uint32_t a0 = __builtin_amdgcn_alignbit(w[1], w[0], 16), a1 = __builtin_amdgcn_alignbit(w[2], w[1], 16);
-                const uint32_t a2 = __builtin_amdgcn_alignbit(w[3], w[2], 16), a3 = __builtin_amdgcn_alignbit(w[4], w[3], 16);
 #pragma unroll
-                for (int c = 0; c < NT; c++) {
-                    const int8_t *xq = act[c].q;
-                    const int4 mm = *(const int4 *)(act[c].meta + 2 * p);
-                    const int iA = dot_q4_dwords(a0, a1, a2, a3, *act_part(xq, p, 0, npair), *act_part(xq, p, 1, npair)) - 8 * mm.y;
-                    const int iB = dot_q4_dwords(w[5], w[6], w[7], w[8], *act_part(xq, p, 2, npair), *act_part(xq, p, 3, npair)) - 8 * mm.w;
-                    if (dump && c == 0) { dump[2 * p] = iA; dump[2 * p + 1] = iB; }
-                    acc[c] = fmaf(dA * __int_as_float(mm.x), (float)iA, acc[c]);
-                    acc[c] = fmaf(dB * __int_as_float(mm.z), (float)iB, acc[c]);
-                }
-            } else {
-                const float dA = h2f((uint16_t)(w[0] & 0xFFFFu)), dB = h2f((uint16_t)(w[8] >> 16));
-                uint32_t a[8];
-#pragma unroll
-                for (int i = 0; i < 8; i++) a[i] = __builtin_amdgcn_alignbit(w[i + 1], w[i], 16);
-#pragma unroll
-                for (int c = 0; c < NT; c++) {
-                    const int8_t *xq = act[c].q;
-                    const int4 mm = *(const int4 *)(act[c].meta + 2 * p);
-                    const int iA = dot_q8_dwords(a, *act_part(xq, p, 0, npair), *act_part(xq, p, 1, npair));
-                    const int iB = dot_q8_dwords(&w[9], *act_part(xq, p, 2, npair), *act_part(xq, p, 3, npair));
-                    if (dump && c == 0) { dump[2 * p] = iA; dump[2 * p + 1] = iB; }
-                    acc[c] = fmaf(dA * __int_as_float(mm.x), (float)iA, acc[c]);
-                    acc[c] = fmaf(dB * __int_as_float(mm.z), (float)iB, acc[c]);
-                }
+            for (int c = 0; c < NT; c++) {
+                const int8_t *xq = act[c].q;
+                const int4 mm = *(const int4 *)(act[c].meta + 2 * p);
+                acc[c] = dot_pair<WT>(t.w[it], *act_part(xq, p, 0, npair), *act_part(xq, p, 1, npair), *act_part(xq, p, 2, npair), *act_part(xq, p, 3, npair),
+                                      mm, acc[c], (dump && c == 0) ? dump + 2 * p : nullptr);
             }
         }
     }
+}
+
+// The activations one lane needs when it owns the same block pairs of every row (64 lanes per row):
+// read from LDS once, reused for all rows of the wave.
+template <int NIT> struct act_frag { int4 x[NIT][4]; int4 mm[NIT]; };
+template <int NIT>
+static __device__ __forceinline__ void load_act_frag(act_frag<NIT> &f, const staged_act &act, int npair, int lane) {
+#pragma unroll
+    for (int it = 0; it < NIT; it++) {
+        const int p = min(it * 64 + lane, npair - 1);
+#pragma unroll
+        for (int j = 0; j < 4; j++) f.x[it][j] = *act_part(act.q, p, j, npair);
+        f.mm[it] = *(const int4 *)(act.meta + 2 * p);
+    }
+}
+template <int WT, int NIT>
+static __device__ __forceinline__ float dot_row_frag(const wtile<WT, NIT> &t, const act_frag<NIT> &f, int npair, int lane) {
+    float acc = 0.0f;
+#pragma unroll
+    for (int it = 0; it < NIT; it++)
+        if (it * 64 + lane < npair) acc = dot_pair<WT>(t.w[it], f.x[it][0], f.x[it][1], f.x[it][2], f.x[it][3], f.mm[it], acc, nullptr);
+    return acc;
 }
 
 // (lanes per row, block pairs per lane) for K elements: the smallest lane count whose pairs-per-lane

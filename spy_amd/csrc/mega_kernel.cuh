@@ -31,6 +31,7 @@
 #define MEGA_MAX_LEAF 64
 #define MEGA_RS 10                  // K-cache units per wave in the scores phase
 #define MEGA_RV 10                  // 128-bit pieces per lane of a V^T row (64 lanes x 8 tokens each)
+#define MEGA_DEPTH 3                // gate|up row buffers requested ahead of their use
 #define MEGA_SLOTS 40               // results per wave and phase handed to wave 0 through LDS
 
 struct mega_sync {                  // zero-initialised once; every counter on its own 128-byte line
@@ -268,12 +269,16 @@ __global__ __launch_bounds__(MEGA_THREADS) void mega_decode_kernel(mega_args a) 
         for (int i = 0; i < MEGA_RV; i++) vb[i] = *(const uint4 *)(vrow + (size_t)min(i * 64 + lane, n_ctx / 8 - 1) * 8);
     };
     auto fetch_wo = [&](const mega_layer &L) { load_tile<WT, 64, 1>(wo0, L.wo + (size_t)(gw % d) * RBd, npd, lane); };
-    auto fetch_gateup = [&](const mega_layer &L, int k0) {
+    // buffers [b0, b1) of a gate|up batch: buffer 2k = gate row, 2k+1 = up row of pair k0 + k.  Only
+    // MEGA_DEPTH buffers are requested ahead of their use (the vector-memory queue of a compute unit
+    // is finite; whatever waits behind a deep prefetch -- barrier polls, activation loads -- waits long).
+    auto fetch_gateup = [&](const mega_layer &L, int k0, int b0, int b1) {
 #pragma unroll
-        for (int k = 0; k < RG; k++) {
-            const int u = gw + (k0 + k) * NW, i = u < F ? u : gw % F;
-            load_tile<WT, 64, 1>(wg[2 * k], L.w_gate + (size_t)i * RBd, npd, lane);
-            load_tile<WT, 64, 1>(wg[2 * k + 1], L.w_up + (size_t)i * RBd, npd, lane);
+        for (int b = 0; b < 2 * RG; b++) {
+            if (b >= b0 && b < b1) {
+                const int u = gw + (k0 + (b >> 1)) * NW, i = u < F ? u : gw % F;
+                load_tile<WT, 64, 1>(wg[b], ((b & 1) ? L.w_up : L.w_gate) + (size_t)i * RBd, npd, lane);
+            }
         }
     };
     auto fetch_down = [&](const mega_layer &L) { load_tile<WT, 64, NITF>(wd0, L.w_down + (size_t)(gw % d) * RBf, npf, lane); };
@@ -443,7 +448,7 @@ __global__ __launch_bounds__(MEGA_THREADS) void mega_decode_kernel(mega_args a) 
         stamp();
         {
             const float s = row_dot_d(wo0);
-            if (!late) fetch_gateup(L, 0); else clear_tile(wg);
+            if (!late) fetch_gateup(L, 0, 0, MEGA_DEPTH); else clear_tile(wg);
             if (lane == 0) s_out[wave * MEGA_SLOTS] = s;
         }
         if (!publish_and_sync([&]() {
@@ -452,14 +457,15 @@ __global__ __launch_bounds__(MEGA_THREADS) void mega_decode_kernel(mega_args a) 
             })) return;
 
         // ================= gate|up: ffn_norm, ffn_up, ffn_gate, silu, ffn_par ========================
-        if (late) { load_x4(xv, a.x1); fetch_gateup(L, 0); } else clear_tile(xv);
+        if (late) { load_x4(xv, a.x1); fetch_gateup(L, 0, 0, MEGA_DEPTH); } else clear_tile(xv);
         stage_norm(xv, L.ffn_norm);
         stamp();
         const int ground = (F + NW - 1) / NW;                                  // row pairs per wave (<= MEGA_SLOTS)
         for (int k0 = 0; k0 < ground; k0 += RG) {
-            if (k0 > 0) fetch_gateup(L, k0);                                    // only the first batch is prefetched
+            if (k0 > 0) fetch_gateup(L, k0, 0, MEGA_DEPTH);                     // the first batch was requested before the barrier
 #pragma unroll
             for (int k = 0; k < RG; k++) {
+                fetch_gateup(L, k0, 2 * k + MEGA_DEPTH, 2 * k + 2 + MEGA_DEPTH);
                 const float g = row_dot_d(wg[2 * k]), u = row_dot_d(wg[2 * k + 1]);
                 if (lane == 0 && k0 + k < ground) s_out[wave * MEGA_SLOTS + k0 + k] = u * silu_lut(g);   // Mul(ffn_up, silu(ffn_gate)) (ffn.cpp:24-35)
             }
