@@ -35,6 +35,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-steps", type=int, default=8)
     ap.add_argument("--layers", type=int, default=32, help="debug only: fewer layers (result is then not the headline config)")
+    ap.add_argument("--no-graph", action="store_true", help="launch the kernels of every pass one by one instead of replaying a HIP graph (for profilers)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch a plain copy kernel over 256 MiB three times (a known-size dispatch to scale profiler byte counters by)")
     args = ap.parse_args()
@@ -87,12 +88,12 @@ def main():
 
     # warm-up (also captures the HIP graph), then the timed region: exactly `steps` passes
     pos = fill
-    toks = eng.decode_greedy(first, pos, warmup, use_graph=True)
+    toks = eng.decode_greedy(first, pos, warmup, use_graph=not args.no_graph)
     pos += warmup
     eng.timing()
     H.sync()
     t0 = time.perf_counter()
-    toks = eng.decode_greedy(int(toks[-1]), pos, steps, use_graph=True)
+    toks = eng.decode_greedy(int(toks[-1]), pos, steps, use_graph=not args.no_graph)
     H.sync()
     wall = time.perf_counter() - t0
     ev_ms, n_timed = eng.timing()
@@ -118,9 +119,12 @@ def main():
     for k, us in per_kernel.items():
         log("  %-8s %8.2f us  %7.1f GB/s  (%.1f%% of 8 TB/s)" % (k, us, alg[k] / us / 1e3, alg[k] / us / 1e3 / 80))
     dom = "gate_up"
+    # HBM bytes per launch of that kernel from profiler counters (FETCH_SIZE + WRITE_SIZE scaled by a copy
+    # kernel of known size; profiles/decode_7b_q4_0_ctx4096_hbm_traffic.md): valid for this shape only
+    traffic = 51.18e6 if (cfg.n_embd, cfg.n_ff, cfg.wtype) == (4096, 11008, H.Q4_0) else None
     achieved = alg[dom] / (per_kernel[dom] * 1e-6) / 1e9
     roofline = {"kernel": "wave_gemv_kernel<Q4_0, gate|up + SiLU>", "bound": "hbm", "achieved": round(achieved, 1), "peak": 8000.0,
-                "unit": "GB/s", "frac": round(achieved / 8000.0, 4), "traffic": None,
+                "unit": "GB/s", "frac": round(achieved / 8000.0, 4), "traffic": traffic,
                 "bytes_per_launch": alg[dom], "us_per_launch": round(per_kernel[dom], 3)}
 
     cpu = None
