@@ -22,3 +22,20 @@ def run_smoke(H, O, np):
     assert np.array_equal(sc.download(np.uint8), O.quantize(oracle, x, O.Q8_0)), "Q8_0 activations differ from the oracle"
     assert err < 1e-3, err
     print("smoke ok: Q4_0 matmul %dx%d T=%d, max relative error %.2e on %s" % (M, K, T, err, H.device_info()["name"]))
+    # the token loop itself: prompt pass, fused single-token passes and the on-device greedy loop of a small model
+    from spy_amd import model as M_
+    from tests.model_util import OracleModel
+    cfg = M_.Config(n_layer=2, n_embd=512, n_head=4, n_ff=1024, n_vocab=1024, n_ctx=64, wtype=H.Q4_0)
+    tensors = M_.synth_model(cfg, seed=3)
+    eng, ora = M_.Engine(cfg, tensors), OracleModel(cfg, tensors, nthread=2)
+    prompt = rng.integers(0, cfg.n_vocab, 6).astype(np.int32)
+    lg, lo = eng.forward(prompt, 0), ora.forward(prompt, 0)
+    e1 = float(np.abs(lg - lo).max() / np.abs(lo).max())
+    tok = int(np.argmax(lo[-1]))
+    lg1, lo1 = eng.forward(np.array([tok], np.int32), 6)[0], ora.forward(np.array([tok], np.int32), 6)[0]
+    e2 = float(np.abs(lg1 - lo1).max() / np.abs(lo1).max())
+    assert e1 < 3e-2 and e2 < 3e-2, (e1, e2)
+    toks = eng.decode_greedy(int(np.argmax(lo1)), 7, 4, use_graph=True)
+    assert len(toks) == 4 and all(0 <= int(t) < cfg.n_vocab for t in toks)
+    eng.close()
+    print("smoke ok: 2-layer token loop, prompt logits err %.2e, single-token logits err %.2e, greedy tokens %s" % (e1, e2, list(map(int, toks))))
