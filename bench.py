@@ -115,6 +115,10 @@ def main():
     n_kv_end = pos + steps
     alg = {"qkv": 3 * d * d * 18 // 32, "wo": d * d * 18 // 32, "gate_up": 2 * F * d * 18 // 32, "down": F * d * 18 // 32,
            "head": V * d * 18 // 32, "scores": n_kv_end * d * 2, "pv": n_kv_end * d * 2}
+    if eng.fuses_attention():           # qkv, scores and softmax + KQV are one launch, timed under "qkv"
+        per_kernel["attention (qkv+scores+pv)"] = per_kernel.pop("qkv")
+        alg["attention (qkv+scores+pv)"] = alg["qkv"] + alg["scores"] + alg["pv"]
+        per_kernel.pop("scores"); per_kernel.pop("pv")
     log("per-kernel (HIP events, walking the layers):")
     for k, us in per_kernel.items():
         log("  %-8s %8.2f us  %7.1f GB/s  (%.1f%% of 8 TB/s)" % (k, us, alg[k] / us / 1e3, alg[k] / us / 1e3 / 80))

@@ -181,12 +181,12 @@ int spy_hip_llama_timing(spy_hip_llama *m, float *ms_per_pass, int32_t *n_pass);
  * reps x n_layer launches that walk the layers (fresh weights / caches every launch); which:
  * "qkv", "scores", "pv", "wo", "gate_up", "down", "head".  Uses the position of the last pass. */
 int spy_hip_llama_kernel_time(spy_hip_llama *m, void *stream, const char *which, int32_t reps, float *us_per_launch);
-/* 1 if single-token passes run as ONE persistent kernel (all layers, grid barriers between the
- * phases, the next phase's weight rows requested before each barrier), 0 if as one kernel per
- * phase (the default, and the faster of the two so far).  The persistent kernel is used when the
- * environment variable SPY_HIP_MEGA=1 was set when the engine was created and its shape limits
- * hold (128-wide heads, n_embd <= 4096, n_ctx <= 5120 on a 256-CU device, head in the
- * layer-weight type). */
+/* How single-token passes are launched, as a bit mask (negative: error).
+ * bit 1 (value 2): the attention part of a layer (qkv, scores, softmax + KQV) is ONE launch whose
+ *   workgroups synchronise head by head; used where all its workgroups are resident (128-wide heads,
+ *   8 * n_head <= compute units, n_ctx <= 5120) unless SPY_HIP_ATTN_SPLIT=1 was set at creation.
+ * bit 0 (value 1): the whole pass is ONE persistent kernel with grid barriers between the phases;
+ *   opt-in with SPY_HIP_MEGA=1 at creation (slower than the per-phase kernels so far). */
 int spy_hip_llama_single_kernel(spy_hip_llama *m);
 
 #ifdef __cplusplus

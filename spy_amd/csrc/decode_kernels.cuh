@@ -280,6 +280,238 @@ __global__ __launch_bounds__(WGV_THREADS) void wave_gemv_kernel(fused_args a) {
     }
 }
 
+// ---- the attention part of a layer in one kernel -----------------------------------------------------
+// qkv, scores and softmax + KQV of a layer only depend on each other head by head: head h's scores need
+// rows h*128.. of wq / wk (and the cached keys of head h), its KQV needs those scores and rows of wv.
+// One launch therefore runs all three steps with the 8 workgroups of a head (8 x 16 waves = 128 waves)
+// synchronising among themselves instead of returning to the host queue twice:
+//   A  wave w of the head: RoPE pair w of q (w < 64) or k (w >= 64) and row w of v   (as wave_gemv_kernel<EPI_QKV>)
+//   B  wave w: keys 4u..4u+3, u = w + 128 k, of head h: 64 lanes x 128 bit = 4 keys per load   (as attn_scores_kernel)
+//   C  workgroup g: softmax of the head's scores, then V^T rows h*128 + 16 g + wave             (as attn_pv_kernel)
+// What one step hands to the next crosses workgroups (and XCDs): it is written with agent-scope atomic
+// stores by wave 0 of each workgroup (results pass through LDS), which waits for their completion before
+// thread 0 arrives at the head's counter, and read with agent-scope atomic loads after it.  The counters
+// only ever count up: the target of barrier i is 8 * (launches of this layer so far + 1), the launch count
+// is kept next to them and bumped by workgroup 0 of the head after the last barrier.  Polls are bounded:
+// on expiry the error flag of the device state is raised and the workgroup leaves.
+// All of a launch's workgroups must be resident (grid <= compute units, one 1024-thread workgroup each).
+#define ATL_RS 10                 // groups of 4 keys per wave (n_ctx <= 128 * 4 * ATL_RS)
+#define ATL_RV 10                 // 128-bit pieces per lane of a V^T row (n_ctx <= 512 * ATL_RV)
+#define ATL_DEPTH 3
+struct attn_layer_args {
+    const uint8_t *wq, *wk, *wv;
+    const float *x_in, *normw; float eps;
+    dev_state *st; const float *rope_cs;
+    uint16_t *q16, *kc, *vc;
+    float *scores, *attn_out;
+    uint32_t *sync;               // per head 3 x 32 words: arrivals of barrier 1, of barrier 2, launches so far
+    int d, n_head, n_ctx;
+    float scale; uint32_t spin_limit;
+};
+
+template <int WT>
+__global__ __launch_bounds__(WGV_THREADS) void attn_layer_kernel(attn_layer_args a) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    __shared__ float s_red[WGV_WAVES];
+    __shared__ int s_ok;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int h = blockIdx.x >> 3, g = blockIdx.x & 7, w = g * WGV_WAVES + wave;      // w: wave of the head, 0..127
+    const int d = a.d, npair = d / 64, n_ctx = a.n_ctx;
+    const size_t RB = (size_t)(d / 32) * wt_traits<WT>::BLK;
+    const int pos = a.st->pos, n_kv = pos + 1;
+    uint32_t *sync = a.sync + (size_t)h * 96;
+    const uint32_t target = 8u * (ldc(sync + 64) + 1u);
+
+    int8_t *s_q = (int8_t *)smem;
+    int2 *s_meta = (int2 *)(smem + staged_q_bytes(d));
+    float *s_rope = (float *)(smem + staged_bytes(d));               // 128
+    float *s_out = s_rope + 128;                                     // [WGV_WAVES][4 * ATL_RS]
+    float *s_t = s_out + WGV_WAVES * 4 * ATL_RS;                     // n_ctx
+    uint16_t *s_p = (uint16_t *)(s_t + n_ctx);                       // n_ctx + 8
+
+    // wave 0 writes the workgroup's results, waits for the stores, thread 0 goes through the head's barrier
+    auto publish_and_sync = [&](uint32_t *counter, auto writer) -> bool {
+        __syncthreads();
+        if (wave == 0) {
+            writer();
+            __builtin_amdgcn_s_waitcnt(0);
+            if (lane == 0) {
+                __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                uint32_t spins = 0;
+                int ok = 1;
+                while ((int32_t)(__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - target) < 0) {
+                    if (++spins > a.spin_limit) { __hip_atomic_store(&a.st->err, 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); ok = 0; break; }
+                    __builtin_amdgcn_s_sleep(1);
+                }
+                s_ok = ok;
+            }
+        }
+        __syncthreads();
+        return s_ok != 0;
+    };
+
+    // ================= A: attn_norm, Q/K/V_project of head h, rope, KV-cache copies =================
+    const int i4 = min(tid, d / 4 - 1);
+    const float4 xv = ((const float4 *)a.x_in)[i4], wv = ((const float4 *)a.normw)[i4];
+    const float rope_v = a.rope_cs[min(tid, 127)];
+    wtile<WT, 1> t[3];
+    const int wp = w & 63;                                           // RoPE pair of the head
+    const uint8_t *p0 = (w < 64 ? a.wq : a.wk) + (size_t)(h * 128 + 2 * wp) * RB;
+    load_tile<WT, 64, 1>(t[0], p0, npair, lane);
+    load_tile<WT, 64, 1>(t[1], p0 + RB, npair, lane);
+    if (tid < 128) s_rope[tid] = rope_v;
+    {
+        float acc = 0.0f;
+        if (tid < d / 4) { acc = fmaf(xv.x, xv.x, acc); acc = fmaf(xv.y, xv.y, acc); acc = fmaf(xv.z, xv.z, acc); acc = fmaf(xv.w, xv.w, acc); }
+        acc = group_sum<64>(acc);
+        if (lane == 0) s_red[wave] = acc;
+        __syncthreads();
+        const float sum = (((s_red[0] + s_red[1]) + (s_red[2] + s_red[3])) + ((s_red[4] + s_red[5]) + (s_red[6] + s_red[7]))) +
+                          (((s_red[8] + s_red[9]) + (s_red[10] + s_red[11])) + ((s_red[12] + s_red[13]) + (s_red[14] + s_red[15])));
+        const float scale = 1.0f / sqrtf(sum / (float)d + a.eps);
+        if (tid < d / 4) {
+            float4 v = xv;
+            v.x = (v.x * scale) * wv.x; v.y = (v.y * scale) * wv.y; v.z = (v.z * scale) * wv.z; v.w = (v.w * scale) * wv.w;
+            int2 meta;
+            const uint32_t q = quantize_oct(v, meta);
+            ((uint32_t *)s_q)[act_dw(tid, d >> 6)] = q;
+            if ((tid & 7) == 0) s_meta[tid >> 3] = meta;
+        }
+        __syncthreads();
+    }
+    uint4 kb[ATL_RS];
+    auto fetch_k = [&](int k) {                                      // keys 4u..4u+3 of head h, u = w + 128 k
+        const int tok = min(4 * (w + 128 * k) + (lane >> 4), n_kv - 1);
+        kb[k] = *(const uint4 *)(a.kc + (size_t)tok * d + h * 128 + (lane & 15) * 8);
+    };
+    {
+        staged_act act; act.q = s_q; act.meta = s_meta;
+        act_frag<1> af;
+        load_act_frag<1>(af, act, npair, lane);
+        float s0 = dot_row_frag<WT, 1>(t[0], af, npair, lane);
+        load_tile<WT, 64, 1>(t[2], a.wv + (size_t)(h * 128 + w) * RB, npair, lane);
+        float s1 = dot_row_frag<WT, 1>(t[1], af, npair, lane);
+        float s2 = dot_row_frag<WT, 1>(t[2], af, npair, lane);
+        s0 = wave_total_lane63(s0); s1 = wave_total_lane63(s1); s2 = wave_total_lane63(s2);
+        if (lane == 63) {
+            const float c = s_rope[2 * wp], sn = s_rope[2 * wp + 1];
+            // (x0, x1) -> (x0*c - x1*s, x0*s + x1*c) on adjacent rows (non-linear.cpp:359-363)
+            s_out[wave * 2] = __uint_as_float((uint32_t)f2h(s0 * c - s1 * sn) | ((uint32_t)f2h(s0 * sn + s1 * c) << 16));
+            s_out[wave * 2 + 1] = __uint_as_float((uint32_t)f2h(s2));
+        }
+        if (wave != 0) {
+#pragma unroll
+            for (int k = 0; k < ATL_DEPTH; k++) fetch_k(k);
+        }
+    }
+    if (!publish_and_sync(sync, [&]() {
+            if (lane < WGV_WAVES) {
+                const int ww = g * WGV_WAVES + lane, pp = ww & 63;
+                const uint32_t pr = __float_as_uint(s_out[lane * 2]);
+                if (ww < 64) stc((uint32_t *)a.q16 + h * 64 + pp, pr);                                         // attn_score rounds Q to fp16 (mat.cpp:37)
+                else stc((uint32_t *)(a.kc + (size_t)pos * d) + h * 64 + pp, pr);                               // KCache_cpy: [token][head][hd]
+                stc(a.vc + (size_t)(h * 128 + ww) * n_ctx + pos, (uint16_t)__float_as_uint(s_out[lane * 2 + 1]));   // VCache_cpy: [d][C] column pos
+            }
+        })) return;
+
+    // ================= B: t = (K.q) * scale for head h ================================================
+    const uint16_t *vrow = a.vc + (size_t)(h * 128 + w) * n_ctx;
+    uint4 vb[ATL_RV];
+    auto fetch_v = [&](int i) { vb[i] = *(const uint4 *)(vrow + (size_t)min(i * 64 + lane, n_ctx / 8 - 1) * 8); };
+    {
+        const uint32_t *qp = (const uint32_t *)a.q16 + h * 64 + (lane & 15) * 4;
+        const uint32_t qw[4] = {ldc(qp), ldc(qp + 1), ldc(qp + 2), ldc(qp + 3)};
+        if (wave == 0) {
+#pragma unroll
+            for (int k = 0; k < ATL_DEPTH; k++) fetch_k(k);
+        }
+        float qf[8];
+#pragma unroll
+        for (int j = 0; j < 4; j++) { qf[2 * j] = h2f((uint16_t)(qw[j] & 0xFFFFu)); qf[2 * j + 1] = h2f((uint16_t)(qw[j] >> 16)); }
+#pragma unroll
+        for (int k = 0; k < ATL_RS; k++) {
+            if (k + ATL_DEPTH < ATL_RS) fetch_k(k + ATL_DEPTH);
+            const int tok = 4 * (w + 128 * k) + (lane >> 4);
+            uint4 kv = kb[k];
+            if (tok == pos) {                                        // written in step A by another workgroup: read it coherently
+                const uint32_t *p = (const uint32_t *)(a.kc + (size_t)tok * d + h * 128 + (lane & 15) * 8);
+                kv = make_uint4(ldc(p), ldc(p + 1), ldc(p + 2), ldc(p + 3));
+            }
+            const uint32_t kw[4] = {kv.x, kv.y, kv.z, kv.w};
+            float s = 0.0f;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                s = fmaf(h2f((uint16_t)(kw[j] & 0xFFFFu)), qf[2 * j], s);
+                s = fmaf(h2f((uint16_t)(kw[j] >> 16)), qf[2 * j + 1], s);
+            }
+            s = group_sum<16>(s);
+            if ((lane & 15) == 0) s_out[wave * (4 * ATL_RS) + k * 4 + (lane >> 4)] = s * a.scale;
+        }
+        if (wave != 0) {
+#pragma unroll
+            for (int i = 0; i < ATL_DEPTH; i++) fetch_v(i);
+        }
+    }
+    if (!publish_and_sync(sync + 32, [&]() {
+            for (int idx = lane; idx < WGV_WAVES * 4 * ATL_RS; idx += 64) {
+                const int wv_ = idx / (4 * ATL_RS), r = idx - wv_ * (4 * ATL_RS);
+                const int tok = 4 * (g * WGV_WAVES + wv_ + 128 * (r >> 2)) + (r & 3);
+                if (tok < n_kv) stc(a.scores + (size_t)h * n_ctx + tok, s_out[idx]);
+            }
+        })) return;
+    if (g == 0 && tid == 0) sync[64] = target / 8u;                  // every workgroup of the head has read the old count
+
+    // ================= C: softmax of the head's scores, KQV rows 16 g .. 16 g + 15 ====================
+    // m = max t; e = expf(float(fp16(t - m))); p = e * (1/sum e) (non-linear.cpp:158-176); P is rounded
+    // to fp16 for the KQV product (mat.cpp:37, vec_dot.h:117-146)
+    {
+        const float *srow = a.scores + (size_t)h * n_ctx;
+        const int n_pad = (n_kv + 7) & ~7;
+        float mx = -INFINITY;
+        for (int j = tid; j < n_kv; j += WGV_THREADS) { const float tt = ldc(srow + j); s_t[j] = tt; mx = fmaxf(mx, tt); }
+        if (wave == 0) {
+#pragma unroll
+            for (int i = 0; i < ATL_DEPTH; i++) fetch_v(i);
+        }
+        mx = wave_max(mx);
+        if (lane == 0) s_red[wave] = mx;
+        __syncthreads();
+        mx = s_red[0];
+#pragma unroll
+        for (int i = 1; i < WGV_WAVES; i++) mx = fmaxf(mx, s_red[i]);
+        __syncthreads();
+        float sum = 0.0f;
+        for (int j = tid; j < n_kv; j += WGV_THREADS) { const float e = expf(h2f(f2h(s_t[j] - mx))); s_t[j] = e; sum += e; }
+        sum = group_sum<64>(sum);
+        if (lane == 0) s_red[wave] = sum;
+        __syncthreads();
+        sum = 0.0f;
+#pragma unroll
+        for (int i = 0; i < WGV_WAVES; i++) sum += s_red[i];
+        const float inv = 1.0f / sum;
+        for (int j = tid; j < n_pad; j += WGV_THREADS) s_p[j] = j < n_kv ? f2h(s_t[j] * inv) : (uint16_t)0;
+        __syncthreads();
+        float acc = 0.0f;
+#pragma unroll
+        for (int i = 0; i < ATL_RV; i++) {
+            if (i + ATL_DEPTH < ATL_RV) fetch_v(i + ATL_DEPTH);
+            const int pc = i * 64 + lane;
+            if (pc * 8 < n_kv) {
+                const uint4 pp = *(const uint4 *)(s_p + pc * 8);
+                const uint32_t vw[4] = {vb[i].x, vb[i].y, vb[i].z, vb[i].w}, pw[4] = {pp.x, pp.y, pp.z, pp.w};
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    // cache slots past n_kv hold whatever was there before: never multiply them in
+                    if (pc * 8 + 2 * j < n_kv) acc = fmaf(h2f((uint16_t)(vw[j] & 0xFFFFu)), h2f((uint16_t)(pw[j] & 0xFFFFu)), acc);
+                    if (pc * 8 + 2 * j + 1 < n_kv) acc = fmaf(h2f((uint16_t)(vw[j] >> 16)), h2f((uint16_t)(pw[j] >> 16)), acc);
+                }
+            }
+        }
+        acc = wave_total_lane63(acc);
+        if (lane == 63) a.attn_out[h * 128 + w] = acc;
+    }
+}
+
 #ifdef SPY_DECODE_COMMON_KERNELS   // type-independent kernels: compiled by one translation unit only
 
 // ---- token embedding + RoPE table ---------------------------------------------------------------

@@ -79,6 +79,34 @@ static int launch_wave_resid(spy_hip_llama *m, hipStream_t st, const fused_args 
     }
 }
 
+// qkv + scores + softmax/KQV of one layer in one launch (head-local barriers)
+template <int WT>
+static int launch_attn_layer(spy_hip_llama *m, hipStream_t st, int il, bool probe) {
+    const spy_hip_llama_desc &c = m->desc;
+    const spy_hip_llama_layer &L = m->layers[il];
+    const size_t lds = staged_bytes(c.n_embd) + 512 + (size_t)WGV_WAVES * 4 * ATL_RS * 4 + (size_t)c.n_ctx * 6 + 16;
+    auto kern = attn_layer_kernel<WT>;
+    static size_t lds_set = 0;
+    if (probe || lds > lds_set) {
+        if (lds > 48 * 1024 && lds > lds_set) { HIP_TRY(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); lds_set = lds; }
+        int per_cu = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, WGV_THREADS, lds) != hipSuccess) per_cu = 0;
+        if (per_cu < 1) return SPY_HIP_EUNSUPPORTED;        // the head barriers need every workgroup resident
+    }
+    if (probe || m->dry) return 0;
+    attn_layer_args a;
+    memset(&a, 0, sizeof(a));
+    a.wq = (const uint8_t *)L.wq; a.wk = (const uint8_t *)L.wk; a.wv = (const uint8_t *)L.wv;
+    a.x_in = m->x; a.normw = (const float *)L.attn_norm; a.eps = c.eps;
+    a.st = m->st; a.rope_cs = m->rope_cs; a.q16 = m->q16; a.kc = m->k_cache[il]; a.vc = m->v_cache[il];
+    a.scores = m->scores; a.attn_out = m->attn_out; a.sync = m->attn_sync;
+    a.d = c.n_embd; a.n_head = c.n_head; a.n_ctx = c.n_ctx;
+    a.scale = 1.0f / sqrtf((float)m->hd);                   // SoftmaxParam::scale (attention.cpp:113)
+    a.spin_limit = 400000;
+    kern<<<dim3((unsigned)(c.n_head * 8)), dim3(WGV_THREADS), lds, st>>>(a);
+    return SPY_LAUNCH_RC();
+}
+
 // one kernel of layer il of the single-token pass
 template <int WT>
 static int enqueue_kernel(spy_hip_llama *m, hipStream_t st, int which, int il) {
@@ -93,6 +121,7 @@ static int enqueue_kernel(spy_hip_llama *m, hipStream_t st, int which, int il) {
     case K_QKV:      // attn_norm, attn_norm_linear, Q/K/V_project, rope, KV-cache copies
         a.W0 = (const uint8_t *)L.wq; a.W1 = (const uint8_t *)L.wk; a.W2 = (const uint8_t *)L.wv;
         a.M = 3 * d; a.K = d; a.x_in = m->x; a.normw = L.attn_norm;
+        if (m->attn_fused) return launch_attn_layer<WT>(m, st, il, false);
         if (m->wave) return launch_wave<WT, 1, 1, EPI_QKV>(m, st, a);
         return launch_fused_norm<WT, EPI_QKV>(m, st, m->cfg_d, a);
     case K_WO:       // KQV_linear + ffn_input

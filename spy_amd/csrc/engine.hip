@@ -95,6 +95,12 @@ extern "C" int spy_hip_llama_create(const spy_hip_llama_desc *desc, spy_hip_llam
         if (!rc && pv_lds > 160 * 1024) rc = SPY_HIP_EUNSUPPORTED;
         if (!rc && pv_lds > 48 * 1024) rc = (int)hipFuncSetAttribute((const void *)attn_pv_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)pv_lds);
     }
+    if (!rc && fused_ok(m) && m->wave) {   // one launch for the attention part of a layer where its workgroups are all resident (SPY_HIP_ATTN_SPLIT=1: three launches)
+        const char *env = getenv("SPY_HIP_ATTN_SPLIT");
+        rc = dalloc(m, (void **)&m->attn_sync, (size_t)c.n_head * 96 * 4, true);
+        if (!rc && !(env && env[0] == '1') && m->hd == 128 && c.n_head * 8 <= m->num_cu && c.n_ctx <= 128 * 4 * ATL_RS && c.n_ctx <= 512 * ATL_RV)
+            m->attn_fused = (c.wtype == SPY_HIP_Q4_0 ? spy_probe_attn_layer_q4_0(m) : spy_probe_attn_layer_q8_0(m)) == 0;
+    }
     if (!rc && fused_ok(m)) { m->dry = true; rc = enqueue_pass_any(m, m->own_stream, true); m->dry = false; }   // sizes the persistent grids
     if (!rc && fused_ok(m)) {            // the persistent single-kernel pass: opt-in with SPY_HIP_MEGA=1 (slower than the per-phase kernels so far)
         std::vector<mega_layer> ml(c.n_layer);
@@ -135,7 +141,7 @@ extern "C" int spy_hip_llama_buffer(spy_hip_llama *m, const char *name, int32_t 
     return 0;
 }
 
-extern "C" int spy_hip_llama_single_kernel(spy_hip_llama *m) { return m ? (m->mega ? 1 : 0) : SPY_HIP_EINVAL; }
+extern "C" int spy_hip_llama_single_kernel(spy_hip_llama *m) { return m ? ((m->mega ? 1 : 0) | (m->attn_fused ? 2 : 0)) : SPY_HIP_EINVAL; }
 
 extern "C" int spy_hip_llama_timing(spy_hip_llama *m, float *ms_per_pass, int32_t *n_pass) {
     SPY_CHECK_ARG(m);
@@ -153,6 +159,7 @@ static bool fused_ok(const spy_hip_llama *m) {
 
 static int enqueue_one(spy_hip_llama *m, hipStream_t st, int which, int il) {
     const spy_hip_llama_desc &c = m->desc;
+    if ((which == K_SCORES || which == K_PV) && m->attn_fused) return 0;     // part of the K_QKV launch
     if (which == K_SCORES) {            // attn_score
         if (m->dry) return 0;
         const float scale = 1.0f / sqrtf((float)m->hd);                     // SoftmaxParam::scale (attention.cpp:113)

@@ -15,6 +15,8 @@ struct spy_hip_llama {
     int hd = 0;
     gemv_cfg cfg_d = {0, 0}, cfg_ff = {0, 0};   // lanes-per-row / pairs-per-lane for K = n_embd and K = n_ff
     bool dry = false;
+    bool attn_fused = false;                    // qkv + scores + softmax/KQV of a layer in one launch
+    uint32_t *attn_sync = nullptr;
     bool wave = false;                          // one-row-per-wave kernels (1024-thread workgroups) instead of the tiled ones
     std::vector<uint16_t *> k_cache, v_cache;
     float *x = nullptr, *x1 = nullptr, *attn_out = nullptr, *hbuf = nullptr, *scores = nullptr, *logits = nullptr, *rope_cs = nullptr;
@@ -55,5 +57,7 @@ int spy_enqueue_kernel_q4_0(spy_hip_llama *m, hipStream_t st, int which, int il)
 int spy_enqueue_kernel_q8_0(spy_hip_llama *m, hipStream_t st, int which, int il);
 // The persistent kernel covering embedding .. output head of one pass.  probe: only check that the
 // kernel for this shape exists and that one workgroup per compute unit is resident.
+int spy_probe_attn_layer_q4_0(spy_hip_llama *m);
+int spy_probe_attn_layer_q8_0(spy_hip_llama *m);
 int spy_enqueue_mega_q4_0(spy_hip_llama *m, hipStream_t st, bool probe);
 int spy_enqueue_mega_q8_0(spy_hip_llama *m, hipStream_t st, bool probe);

@@ -21,6 +21,14 @@
 // float4 of input per thread that cover K elements in the staging prologues
 #define GEMV_SIT_FOR(K) (((K) + 4 * GEMV_THREADS - 1) / (4 * GEMV_THREADS))
 
+// agent-scope accesses: coherent between compute units and XCDs
+static __device__ __forceinline__ float ldc(const float *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+static __device__ __forceinline__ uint32_t ldc(const uint32_t *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+static __device__ __forceinline__ void stc(float *p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+static __device__ __forceinline__ void stc(uint32_t *p, uint32_t v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+static __device__ __forceinline__ void stc(uint16_t *p, uint16_t v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+static __device__ __forceinline__ float4 ldc4(const float *p) { return make_float4(ldc(p), ldc(p + 1), ldc(p + 2), ldc(p + 3)); }
+
 template <int WT> struct wt_traits;
 template <> struct wt_traits<SPY_HIP_Q4_0> { static constexpr int BLK = 18, PAIR_DW = 9; };
 template <> struct wt_traits<SPY_HIP_Q8_0> { static constexpr int BLK = 34, PAIR_DW = 17; };

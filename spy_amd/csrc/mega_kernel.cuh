@@ -75,14 +75,6 @@ static __host__ __device__ inline size_t mega_lds_bytes(int d, int F, int hd, in
     return (n + 15) & ~(size_t)15;
 }
 
-// agent-scope accesses: coherent between compute units and XCDs
-static __device__ __forceinline__ float ldc(const float *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-static __device__ __forceinline__ uint32_t ldc(const uint32_t *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-static __device__ __forceinline__ void stc(float *p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-static __device__ __forceinline__ void stc(uint32_t *p, uint32_t v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-static __device__ __forceinline__ void stc(uint16_t *p, uint16_t v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-static __device__ __forceinline__ float4 ldc4(const float *p) { return make_float4(ldc(p), ldc(p + 1), ldc(p + 2), ldc(p + 3)); }
-
 // Grid barrier number b (1-based, counts up over the life of the sync block, wraps).  Called by
 // thread 0 of every workgroup after its stores have completed.  Arrivals go to MEGA_FAN-way leaf
 // counters, the last arrival of a leaf to the top counter, the last of those publishes b in the

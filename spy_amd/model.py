@@ -155,7 +155,11 @@ class Engine:
 
     def uses_single_kernel(self):
         """True when single-token passes run as one persistent kernel"""
-        return self.L.spy_hip_llama_single_kernel(self.handle) == 1
+        return (self.L.spy_hip_llama_single_kernel(self.handle) & 1) == 1
+
+    def fuses_attention(self):
+        """True when qkv, scores and softmax + KQV of a layer run as one launch"""
+        return (self.L.spy_hip_llama_single_kernel(self.handle) & 2) == 2
 
     def timing(self):
         ms, n = C.c_float(), C.c_int32()
