@@ -18,12 +18,15 @@ SYNTH_PATH = os.path.join(HERE, "libspy_synth.so")
 
 class Config:
     def __init__(self, n_layer=32, n_embd=4096, n_head=32, n_ff=11008, n_vocab=32000, n_ctx=4096, eps=1e-5,
-                 rope_freq_base=10000.0, wtype=H.Q4_0, t_out=None, t_tok_embd=H.F32):
+                 rope_freq_base=10000.0, wtype=H.Q4_0, t_out=None, t_tok_embd=H.F32, tensor_types=None):
         self.n_layer, self.n_embd, self.n_head, self.n_ff = n_layer, n_embd, n_head, n_ff
         self.n_vocab, self.n_ctx, self.eps, self.rope_freq_base = n_vocab, n_ctx, eps, rope_freq_base
         self.wtype = wtype
         self.t_out = wtype if t_out is None else t_out
         self.t_tok_embd = t_tok_embd
+        # per-tensor overrides of the layer-weight type, e.g. {"attn_v": Q6_K, "ffn_down": Q6_K} for a
+        # Q4_K_M-style mix; only the operator-by-operator path takes mixed layers
+        self.tensor_types = dict(tensor_types or {})
 
     @classmethod
     def llama2_7b(cls, n_ctx=4352, wtype=H.Q4_0, **kw):
@@ -38,11 +41,12 @@ class Config:
             p = "blk.%d." % i
             out[p + "attn_norm.weight"] = (H.F32, 1, d)
             out[p + "ffn_norm.weight"] = (H.F32, 1, d)
+            tt = lambda n: self.tensor_types.get(n, self.wtype)
             for n in ("attn_q", "attn_k", "attn_v", "attn_output"):
-                out[p + n + ".weight"] = (self.wtype, d, d)
-            out[p + "ffn_gate.weight"] = (self.wtype, F, d)
-            out[p + "ffn_up.weight"] = (self.wtype, F, d)
-            out[p + "ffn_down.weight"] = (self.wtype, d, F)
+                out[p + n + ".weight"] = (tt(n), d, d)
+            out[p + "ffn_gate.weight"] = (tt("ffn_gate"), F, d)
+            out[p + "ffn_up.weight"] = (tt("ffn_up"), F, d)
+            out[p + "ffn_down.weight"] = (tt("ffn_down"), d, F)
         return out
 
     def weight_bytes(self):

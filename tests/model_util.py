@@ -20,7 +20,7 @@ class OracleModel:
             for field, gname, tfield in _FIELDS:
                 setattr(self.layers[i], field, tensors["blk.%d.%s.weight" % (i, gname)].ctypes.data)
                 if tfield:
-                    setattr(self.layers[i], tfield, cfg.wtype)
+                    setattr(self.layers[i], tfield, cfg.tensor_types.get(gname, cfg.wtype))
         d, Cx = cfg.n_embd, cfg.n_ctx
         self.k_cache = [np.zeros(Cx * d, dtype=np.uint16) for _ in range(cfg.n_layer)]
         self.v_cache = [np.zeros(Cx * d, dtype=np.uint16) for _ in range(cfg.n_layer)]

@@ -65,3 +65,28 @@ def test_submit_path_matches_oracle_and_engine(wtype):
     assert st2["n_alloc"] == st2["n_free"], st2
     host.close()
     eng.close()
+
+
+@pytest.mark.gpu
+def test_submit_path_k_quant_mix_with_outliers():
+    """The Q4_K_M-style mix (Q4_K for q, k, o, gate, up; Q6_K for v, down and the head; 0.1 % of the
+    weights x20) through Backend::submit, against the oracle.  The reference has no K-quant arithmetic:
+    both sides follow the public ggml block definitions (parity unpinned against the reference)."""
+    from spy_amd import backend_driver as B
+    from spy_amd import model as M
+    from tests.gpu_util import assert_close
+    from tests.model_util import OracleModel, k_quant_quantizer
+    cfg = M.Config(n_layer=2, n_embd=512, n_head=4, n_ff=1024, n_vocab=768, n_ctx=48, wtype=O.Q4_K, t_out=O.Q6_K,
+                   tensor_types={"attn_v": O.Q6_K, "ffn_down": O.Q6_K})
+    tensors = M.synth_model(cfg, seed=21, outlier_every=1000, quantizer=k_quant_quantizer)
+    host, ora = B.HostModel(cfg, tensors), OracleModel(cfg, tensors)
+    prompt = np.random.default_rng(4).integers(0, cfg.n_vocab, 7).astype(np.int32)
+    lo = ora.forward(prompt, 0)
+    assert_close(host.forward(prompt, 0), lo, "K-quant mix prefill logits", 3e-3)
+    tok = int(np.argmax(lo[-1]))
+    for step in range(3):
+        t = np.array([tok], np.int32)
+        lh, l1 = host.forward(t, 7 + step)[0], ora.forward(t, 7 + step)[0]
+        assert_close(lh, l1, "K-quant mix decode step %d" % step, 3e-3)
+        tok = int(np.argmax(l1))
+    host.close()
