@@ -143,12 +143,16 @@ int spy_hip_block_dots(void *stream, int wtype, const void *w, const void *xq, i
 typedef struct spy_hip_llama_layer {
     const float *attn_norm, *ffn_norm;                         /* f32[n_embd], device          */
     const void  *wq, *wk, *wv, *wo, *w_gate, *w_up, *w_down;   /* native GGUF blocks, device   */
+    /* type of each matrix: Q4_0, Q8_0, Q4_K or Q6_K; 0 = the description's wtype.  Within a layer wq and
+     * wk share a type and so do w_gate and w_up (they are read by the same kernel); wv may be Q6_K next
+     * to Q4_K wq / wk (the Q4_K_M mix). */
+    int32_t t_wq, t_wk, t_wv, t_wo, t_gate, t_up, t_down;
 } spy_hip_llama_layer;
 
 typedef struct spy_hip_llama_desc {
     int32_t n_layer, n_embd, n_head, n_ff, n_vocab, n_ctx;     /* n_ctx % 8 == 0               */
     float   eps, rope_freq_base;
-    int32_t wtype;                                             /* type of the 7 layer matrices: Q4_0 or Q8_0 */
+    int32_t wtype;                                             /* default type of the layer matrices: Q4_0, Q8_0, Q4_K, Q6_K */
     const void  *tok_embd;  int32_t t_tok_embd;                /* F32 or Q8_0 (GetRow, view.cpp:65-77) */
     const float *out_norm;
     const void  *w_out;     int32_t t_out;                     /* Q4_0, Q8_0, Q4_K or Q6_K     */

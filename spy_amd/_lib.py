@@ -37,7 +37,8 @@ class RopeParam(C.Structure):
 
 class LlamaLayer(C.Structure):
     """spy_hip_llama_layer"""
-    _fields_ = [(n, C.c_void_p) for n in ("attn_norm", "ffn_norm", "wq", "wk", "wv", "wo", "w_gate", "w_up", "w_down")]
+    _fields_ = [(n, C.c_void_p) for n in ("attn_norm", "ffn_norm", "wq", "wk", "wv", "wo", "w_gate", "w_up", "w_down")] + \
+               [(n, C.c_int32) for n in ("t_wq", "t_wk", "t_wv", "t_wo", "t_gate", "t_up", "t_down")]
 
 
 class LlamaDesc(C.Structure):

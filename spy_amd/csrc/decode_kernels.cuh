@@ -90,7 +90,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void fused_gemv_kernel(fused_args a) 
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     __shared__ float s_red[GEMV_WAVES];
     constexpr bool NORM = (EPI != EPI_RESID);
-    const size_t RB = (size_t)(a.K / 32) * wt_traits<WT>::BLK;
+    const size_t RB = (size_t)spy_row_size(WT, a.K);
     // the matrix bases are selected by arithmetic on wave-uniform differences: a select between
     // the kernel arguments themselves becomes a per-lane load from the argument block
     const ptrdiff_t dW1 = a.W1 - a.W0, dW2 = a.W2 - a.W0;
@@ -163,7 +163,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void fused_gemv_kernel(fused_args a) 
 #ifndef WGV_DEPTH
 #define WGV_DEPTH 3             // rows per wave requested ahead of their use
 #endif
-template <int WT, int NITK, int NR, int EPI>
+template <int WT, int NITK, int NR, int EPI, int WTV = WT>      // WTV: type of W2 (the v rows of EPI_QKV)
 __global__ __launch_bounds__(WGV_THREADS) void wave_gemv_kernel(fused_args a) {
     constexpr bool NORM = (EPI != EPI_RESID);
     constexpr int NB = EPI == EPI_QKV ? 3 : (EPI == EPI_GATEUP ? 2 * NR : NR);
@@ -173,7 +173,7 @@ __global__ __launch_bounds__(WGV_THREADS) void wave_gemv_kernel(fused_args a) {
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int NW = (int)gridDim.x * WGV_WAVES, gw = (int)blockIdx.x * WGV_WAVES + wave;
     const int K = a.K, npair = K / 64;
-    const size_t RB = (size_t)(K / 32) * wt_traits<WT>::BLK;
+    const size_t RB = (size_t)spy_row_size(WT, K);
 
     // 1. the activation vector (and what the epilogue needs), 2. the rows: all unconditional, in this order
     float4 xv[NITK], wv[NORM ? NITK : 1];
@@ -190,11 +190,13 @@ __global__ __launch_bounds__(WGV_THREADS) void wave_gemv_kernel(fused_args a) {
     // once sits in the issue stage until the queue drains (most of the kernel), holding up the staging
     // barriers of everybody else.
     wtile<WT, NITK> t[NB];
+    wtile<WTV, NITK> tv;
     auto issue = [&](int k) {
         if constexpr (EPI == EPI_QKV) {
             const int j = gw % a.d;
             const uint8_t *p0 = 2 * j < a.d ? a.W0 + (size_t)(2 * j) * RB : a.W1 + (size_t)(2 * j - a.d) * RB;
-            load_tile<WT, 64, NITK>(t[k], k == 2 ? a.W2 + (size_t)j * RB : p0 + (size_t)k * RB, npair, lane);
+            if (k == 2) load_tile<WTV, 64, NITK>(tv, a.W2 + (size_t)j * spy_row_size(WTV, K), npair, lane);
+            else load_tile<WT, 64, NITK>(t[k], p0 + (size_t)k * RB, npair, lane);
         } else if constexpr (EPI == EPI_GATEUP) {
             const int F = a.M / 2, u = gw + (k >> 1) * NW, i = u < F ? u : gw % F;
             load_tile<WT, 64, NITK>(t[k], ((k & 1) ? a.W1 : a.W0) + (size_t)i * RB, npair, lane);
@@ -241,14 +243,17 @@ __global__ __launch_bounds__(WGV_THREADS) void wave_gemv_kernel(fused_args a) {
     __syncthreads();
     staged_act act; act.q = s_q; act.meta = s_meta;
     act_frag<NITK> af;                                    // this lane's activations: the same for every row
-    load_act_frag<NITK>(af, act, npair, lane);
+    load_act_frag<WT, NITK>(af, act, npair, lane);
     // partial dots of all rows (requesting the row WGV_DEPTH ahead before each), then their wave reductions
     // (independent chains); totals land in lane 63
     float s[NB];
 #pragma unroll
     for (int k = 0; k < NB; k++) {
         if (k + DEPTH < NB) issue(k + DEPTH);
-        s[k] = dot_row_frag<WT, NITK>(t[k], af, npair, lane);
+        if (EPI == EPI_QKV && k == 2) {
+            if constexpr (WTV == WT) s[k] = dot_row_frag<WTV, NITK>(tv, af, npair, lane);
+            else { act_frag<NITK> av; load_act_frag<WTV, NITK>(av, act, npair, lane); s[k] = dot_row_frag<WTV, NITK>(tv, av, npair, lane); }
+        } else s[k] = dot_row_frag<WT, NITK>(t[k], af, npair, lane);
     }
 #pragma unroll
     for (int k = 0; k < NB; k++) s[k] = wave_total_lane63(s[k]);
@@ -309,7 +314,7 @@ struct attn_layer_args {
     float scale; uint32_t spin_limit;
 };
 
-template <int WT>
+template <int WT, int WTV>        // types of wq / wk and of wv
 __global__ __launch_bounds__(WGV_THREADS) void attn_layer_kernel(attn_layer_args a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     __shared__ float s_red[WGV_WAVES];
@@ -317,7 +322,7 @@ __global__ __launch_bounds__(WGV_THREADS) void attn_layer_kernel(attn_layer_args
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int h = blockIdx.x >> 3, g = blockIdx.x & 7, w = g * WGV_WAVES + wave;      // w: wave of the head, 0..127
     const int d = a.d, npair = d / 64, n_ctx = a.n_ctx;
-    const size_t RB = (size_t)(d / 32) * wt_traits<WT>::BLK;
+    const size_t RB = (size_t)spy_row_size(WT, d);
     const int pos = a.st->pos, n_kv = pos + 1;
     uint32_t *sync = a.sync + (size_t)h * 96;
     const uint32_t target = 8u * (ldc(sync + 64) + 1u);
@@ -354,7 +359,8 @@ __global__ __launch_bounds__(WGV_THREADS) void attn_layer_kernel(attn_layer_args
     const int i4 = min(tid, d / 4 - 1);
     const float4 xv = ((const float4 *)a.x_in)[i4], wv = ((const float4 *)a.normw)[i4];
     const float rope_v = a.rope_cs[min(tid, 127)];
-    wtile<WT, 1> t[3];
+    wtile<WT, 1> t[2];
+    wtile<WTV, 1> tv;
     const int wp = w & 63;                                           // RoPE pair of the head
     const uint8_t *p0 = (w < 64 ? a.wq : a.wk) + (size_t)(h * 128 + 2 * wp) * RB;
     load_tile<WT, 64, 1>(t[0], p0, npair, lane);
@@ -387,11 +393,13 @@ __global__ __launch_bounds__(WGV_THREADS) void attn_layer_kernel(attn_layer_args
     {
         staged_act act; act.q = s_q; act.meta = s_meta;
         act_frag<1> af;
-        load_act_frag<1>(af, act, npair, lane);
+        load_act_frag<WT, 1>(af, act, npair, lane);
         float s0 = dot_row_frag<WT, 1>(t[0], af, npair, lane);
-        load_tile<WT, 64, 1>(t[2], a.wv + (size_t)(h * 128 + w) * RB, npair, lane);
+        load_tile<WTV, 64, 1>(tv, a.wv + (size_t)(h * 128 + w) * spy_row_size(WTV, d), npair, lane);
         float s1 = dot_row_frag<WT, 1>(t[1], af, npair, lane);
-        float s2 = dot_row_frag<WT, 1>(t[2], af, npair, lane);
+        float s2;
+        if constexpr (WTV == WT) s2 = dot_row_frag<WTV, 1>(tv, af, npair, lane);
+        else { act_frag<1> av; load_act_frag<WTV, 1>(av, act, npair, lane); s2 = dot_row_frag<WTV, 1>(tv, av, npair, lane); }
         s0 = wave_total_lane63(s0); s1 = wave_total_lane63(s1); s2 = wave_total_lane63(s2);
         if (lane == 63) {
             const float c = s_rope[2 * wp], sn = s_rope[2 * wp + 1];

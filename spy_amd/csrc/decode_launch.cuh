@@ -54,10 +54,10 @@ static int launch_fused_resid(spy_hip_llama *m, hipStream_t st, gemv_cfg cfg, co
 
 
 // ---- one-row-per-wave kernels (K <= 4096 * NITK) ---------------------------------------------------
-template <int WT, int NITK, int NR, int EPI>
+template <int WT, int NITK, int NR, int EPI, int WTV = WT>
 static int launch_wave(spy_hip_llama *m, hipStream_t st, const fused_args &a) {
     const size_t lds = staged_bytes(a.K) + (EPI == EPI_QKV ? 4 * (size_t)a.hd : 0);
-    auto kern = wave_gemv_kernel<WT, NITK, NR, EPI>;
+    auto kern = wave_gemv_kernel<WT, NITK, NR, EPI, WTV>;
     static size_t lds_set = 0;
     if (lds > 48 * 1024 && lds > lds_set) { HIP_TRY(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); lds_set = lds; }
     if (m->dry) return 0;
@@ -66,7 +66,12 @@ static int launch_wave(spy_hip_llama *m, hipStream_t st, const fused_args &a) {
     kern<<<dim3((unsigned)grid), dim3(WGV_THREADS), lds, st>>>(a);
     return SPY_LAUNCH_RC();
 }
-template <int WT> struct wave_rows { static constexpr int HEAD = (WT == SPY_HIP_Q4_0) ? 8 : 4, GATEUP = (WT == SPY_HIP_Q4_0) ? 3 : 2; };
+// rows (head) and row pairs (gate|up) per wave: bounded by the row registers, PAIR_DW dwords per row
+template <int WT> struct wave_rows {
+    static constexpr int HEAD = WT == SPY_HIP_Q4_0 ? 8 : (WT == SPY_HIP_Q4_K ? 6 : (WT == SPY_HIP_Q8_0 ? 4 : 3));
+    static constexpr int GATEUP = (WT == SPY_HIP_Q4_0 || WT == SPY_HIP_Q4_K) ? 3 : 2;
+};
+static inline int layer_type(const spy_hip_llama *m, int t) { return t ? t : m->desc.wtype; }
 
 template <int WT>
 static int launch_wave_resid(spy_hip_llama *m, hipStream_t st, const fused_args &a) {
@@ -74,18 +79,18 @@ static int launch_wave_resid(spy_hip_llama *m, hipStream_t st, const fused_args 
     case 1: return launch_wave<WT, 1, 1, EPI_RESID>(m, st, a);
     case 2: return launch_wave<WT, 2, 1, EPI_RESID>(m, st, a);
     case 3: return launch_wave<WT, 3, 1, EPI_RESID>(m, st, a);
-    case 4: return launch_wave<WT, 4, 1, EPI_RESID>(m, st, a);
+    case 4: if constexpr (WT == SPY_HIP_Q4_0 || WT == SPY_HIP_Q8_0) return launch_wave<WT, 4, 1, EPI_RESID>(m, st, a); else return SPY_HIP_EUNSUPPORTED;
     default: return SPY_HIP_EUNSUPPORTED;
     }
 }
 
 // qkv + scores + softmax/KQV of one layer in one launch (head-local barriers)
-template <int WT>
-static int launch_attn_layer(spy_hip_llama *m, hipStream_t st, int il, bool probe) {
+template <int WT, int WTV>
+static int launch_attn_layer_tv(spy_hip_llama *m, hipStream_t st, int il, bool probe) {
     const spy_hip_llama_desc &c = m->desc;
     const spy_hip_llama_layer &L = m->layers[il];
     const size_t lds = staged_bytes(c.n_embd) + 512 + (size_t)WGV_WAVES * 4 * ATL_RS * 4 + (size_t)c.n_ctx * 6 + 16;
-    auto kern = attn_layer_kernel<WT>;
+    auto kern = attn_layer_kernel<WT, WTV>;
     static size_t lds_set = 0;
     if (probe || lds > lds_set) {
         if (lds > 48 * 1024 && lds > lds_set) { HIP_TRY(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); lds_set = lds; }
@@ -107,7 +112,23 @@ static int launch_attn_layer(spy_hip_llama *m, hipStream_t st, int il, bool prob
     return SPY_LAUNCH_RC();
 }
 
-// one kernel of layer il of the single-token pass
+// wq / wk of type WT; wv of the same type or, next to Q4_K, Q6_K
+template <int WT>
+static int launch_attn_layer(spy_hip_llama *m, hipStream_t st, int il, bool probe) {
+    const int tv = layer_type(m, m->layers[il].t_wv);
+    if (tv == WT) return launch_attn_layer_tv<WT, WT>(m, st, il, probe);
+    if constexpr (WT == SPY_HIP_Q4_K) { if (tv == SPY_HIP_Q6_K) return launch_attn_layer_tv<SPY_HIP_Q4_K, SPY_HIP_Q6_K>(m, st, il, probe); }
+    return SPY_HIP_EUNSUPPORTED;
+}
+template <int WT>
+static int launch_wave_qkv(spy_hip_llama *m, hipStream_t st, int il, const fused_args &a) {
+    const int tv = layer_type(m, m->layers[il].t_wv);
+    if (tv == WT) return launch_wave<WT, 1, 1, EPI_QKV>(m, st, a);
+    if constexpr (WT == SPY_HIP_Q4_K) { if (tv == SPY_HIP_Q6_K) return launch_wave<SPY_HIP_Q4_K, 1, 1, EPI_QKV, SPY_HIP_Q6_K>(m, st, a); }
+    return SPY_HIP_EUNSUPPORTED;
+}
+
+// one kernel of layer il of the single-token pass; WT is the type of the kernel's (first) matrix
 template <int WT>
 static int enqueue_kernel(spy_hip_llama *m, hipStream_t st, int which, int il) {
     const spy_hip_llama_desc &c = m->desc;
@@ -122,37 +143,39 @@ static int enqueue_kernel(spy_hip_llama *m, hipStream_t st, int which, int il) {
         a.W0 = (const uint8_t *)L.wq; a.W1 = (const uint8_t *)L.wk; a.W2 = (const uint8_t *)L.wv;
         a.M = 3 * d; a.K = d; a.x_in = m->x; a.normw = L.attn_norm;
         if (m->attn_fused) return launch_attn_layer<WT>(m, st, il, false);
-        if (m->wave) return launch_wave<WT, 1, 1, EPI_QKV>(m, st, a);
-        return launch_fused_norm<WT, EPI_QKV>(m, st, m->cfg_d, a);
+        if (m->wave) return launch_wave_qkv<WT>(m, st, il, a);
+        if constexpr (WT == SPY_HIP_Q4_0 || WT == SPY_HIP_Q8_0) return launch_fused_norm<WT, EPI_QKV>(m, st, m->cfg_d, a);
+        return SPY_HIP_EUNSUPPORTED;
     case K_WO:       // KQV_linear + ffn_input
         a.W0 = (const uint8_t *)L.wo; a.M = d; a.K = d; a.x_in = m->attn_out; a.resid = m->x; a.out = m->x1;
         if (m->wave) return launch_wave_resid<WT>(m, st, a);
-        return launch_fused_resid<WT>(m, st, m->cfg_d, a);
+        if constexpr (WT == SPY_HIP_Q4_0 || WT == SPY_HIP_Q8_0) return launch_fused_resid<WT>(m, st, m->cfg_d, a);
+        return SPY_HIP_EUNSUPPORTED;
     case K_GATEUP:   // ffn_norm, ffn_up, ffn_gate, silu, ffn_par
         a.W0 = (const uint8_t *)L.w_gate; a.W1 = (const uint8_t *)L.w_up; a.M = 2 * F; a.K = d; a.x_in = m->x1; a.normw = L.ffn_norm; a.out = m->hbuf;
         if (m->wave) return launch_wave<WT, 1, wave_rows<WT>::GATEUP, EPI_GATEUP>(m, st, a);
-        return launch_fused_norm<WT, EPI_GATEUP>(m, st, m->cfg_d, a);
+        if constexpr (WT == SPY_HIP_Q4_0 || WT == SPY_HIP_Q8_0) return launch_fused_norm<WT, EPI_GATEUP>(m, st, m->cfg_d, a);
+        return SPY_HIP_EUNSUPPORTED;
     case K_DOWN:     // ffn_down + logit_output (the next layer's input)
         a.W0 = (const uint8_t *)L.w_down; a.M = d; a.K = F; a.x_in = m->hbuf; a.resid = m->x1; a.out = m->x;
         if (m->wave) return launch_wave_resid<WT>(m, st, a);
-        return launch_fused_resid<WT>(m, st, m->cfg_ff, a);
+        if constexpr (WT == SPY_HIP_Q4_0 || WT == SPY_HIP_Q8_0) return launch_fused_resid<WT>(m, st, m->cfg_ff, a);
+        return SPY_HIP_EUNSUPPORTED;
     }
     return SPY_HIP_EINVAL;
 }
 
-// result_norm, result_linear, output
+// result_norm, result_linear, output; WT is the type of the output matrix
 template <int WT>
 static int enqueue_head(spy_hip_llama *m, hipStream_t st) {
     const spy_hip_llama_desc &c = m->desc;
     const int d = c.n_embd;
-    if (c.t_out == c.wtype) {
-        fused_args a;
-        memset(&a, 0, sizeof(a));
-        a.W0 = (const uint8_t *)c.w_out; a.M = c.n_vocab; a.K = d; a.x_in = m->x; a.normw = c.out_norm; a.eps = c.eps; a.out = m->logits;
-        if (m->wave) return launch_wave<WT, 1, wave_rows<WT>::HEAD, EPI_STORE>(m, st, a);
-        return launch_fused_norm<WT, EPI_STORE>(m, st, m->cfg_d, a);
-    }
-    // head in another type (e.g. Q6_K): norm + weight + Q8_0 through the operator kernels
+    fused_args a;
+    memset(&a, 0, sizeof(a));
+    a.W0 = (const uint8_t *)c.w_out; a.M = c.n_vocab; a.K = d; a.x_in = m->x; a.normw = c.out_norm; a.eps = c.eps; a.out = m->logits;
+    if (m->wave) return launch_wave<WT, 1, wave_rows<WT>::HEAD, EPI_STORE>(m, st, a);
+    if constexpr (WT == SPY_HIP_Q4_0 || WT == SPY_HIP_Q8_0) return launch_fused_norm<WT, EPI_STORE>(m, st, m->cfg_d, a);
+    // no row kernel for this shape: norm + weight + Q8_0 through the operator kernels
     if (m->dry) return 0;
     spy_hip_tensor tx, tw, txn;
     memset(&tx, 0, sizeof(tx));
@@ -164,7 +187,6 @@ static int enqueue_head(spy_hip_llama *m, hipStream_t st) {
     RC_TRY(spy_hip_quantize_q8_0(st, m->x1, 4 * d, m->xq_head, 1, d));
     return spy_hip_gemv_q8_0act(st, c.t_out, c.w_out, m->xq_head, m->logits, nullptr, c.n_vocab, d, 1, c.n_vocab);
 }
-
 
 template <int WT>
 static int enqueue_any(spy_hip_llama *m, hipStream_t st, int which, int il) {

@@ -14,6 +14,15 @@
 
 
 static bool fused_ok(const spy_hip_llama *m);
+static int probe_attn(spy_hip_llama *m, int il) {
+    switch (m->layers[il].t_wq) {
+    case SPY_HIP_Q4_0: return spy_probe_attn_layer_q4_0(m, il);
+    case SPY_HIP_Q8_0: return spy_probe_attn_layer_q8_0(m, il);
+    case SPY_HIP_Q4_K: return spy_probe_attn_layer_q4_k(m, il);
+    case SPY_HIP_Q6_K: return spy_probe_attn_layer_q6_k(m, il);
+    }
+    return SPY_HIP_EUNSUPPORTED;
+}
 static int enqueue_pass_any(spy_hip_llama *m, hipStream_t st, bool sample);
 
 static int dalloc(spy_hip_llama *m, void **p, size_t bytes, bool zero) {
@@ -44,7 +53,9 @@ extern "C" int spy_hip_llama_create(const spy_hip_llama_desc *desc, spy_hip_llam
     SPY_CHECK_ARG(c.n_layer > 0 && c.n_embd > 0 && c.n_head > 0 && c.n_ff > 0 && c.n_vocab > 0 && c.n_ctx > 0);
     SPY_CHECK_ARG(c.n_embd % c.n_head == 0 && c.n_ctx % 8 == 0 && c.n_embd % 64 == 0 && c.n_ff % 64 == 0);
     SPY_CHECK_ARG(c.tok_embd && c.out_norm && c.w_out);
-    if (c.wtype != SPY_HIP_Q4_0 && c.wtype != SPY_HIP_Q8_0) return SPY_HIP_EUNSUPPORTED;
+    auto is_wt = [](int t) { return t == SPY_HIP_Q4_0 || t == SPY_HIP_Q8_0 || t == SPY_HIP_Q4_K || t == SPY_HIP_Q6_K; };
+    auto is_kq = [](int t) { return t == SPY_HIP_Q4_K || t == SPY_HIP_Q6_K; };
+    if (!is_wt(c.wtype)) return SPY_HIP_EUNSUPPORTED;
     if (c.t_tok_embd != SPY_HIP_F32 && c.t_tok_embd != SPY_HIP_Q8_0) return SPY_HIP_EUNSUPPORTED;     // GetRow (view.cpp:65-77)
     if (c.t_out != SPY_HIP_Q4_0 && c.t_out != SPY_HIP_Q8_0 && c.t_out != SPY_HIP_Q4_K && c.t_out != SPY_HIP_Q6_K) return SPY_HIP_EUNSUPPORTED;
     if ((c.t_out == SPY_HIP_Q4_K || c.t_out == SPY_HIP_Q6_K) && c.n_embd % 256 != 0) return SPY_HIP_EINVAL;
@@ -53,15 +64,23 @@ extern "C" int spy_hip_llama_create(const spy_hip_llama_desc *desc, spy_hip_llam
     m->layers.assign(c.layers, c.layers + c.n_layer);
     m->desc.layers = m->layers.data();
     m->hd = c.n_embd / c.n_head;
+    m->uniform = (c.wtype == SPY_HIP_Q4_0 || c.wtype == SPY_HIP_Q8_0) && c.t_out == c.wtype;
     for (int i = 0; i < c.n_layer; i++) {
-        const spy_hip_llama_layer &L = m->layers[i];
+        spy_hip_llama_layer &L = m->layers[i];
         if (!L.attn_norm || !L.ffn_norm || !L.wq || !L.wk || !L.wv || !L.wo || !L.w_gate || !L.w_up || !L.w_down) { delete m; return SPY_HIP_EINVAL; }
+        int32_t *tt[7] = {&L.t_wq, &L.t_wk, &L.t_wv, &L.t_wo, &L.t_gate, &L.t_up, &L.t_down};
+        for (int k = 0; k < 7; k++) {
+            if (*tt[k] == 0) *tt[k] = c.wtype;
+            if (!is_wt(*tt[k])) { delete m; return SPY_HIP_EUNSUPPORTED; }
+            if (is_kq(*tt[k]) && (c.n_embd % 256 != 0 || c.n_ff % 256 != 0)) { delete m; return SPY_HIP_EINVAL; }
+            if (*tt[k] != c.wtype) m->uniform = false;
+        }
     }
     m->cfg_d  = pick_cfg(c.n_embd, 32);
     m->cfg_ff = pick_cfg(c.n_ff);
     {   // SPY_HIP_TILED=1 keeps the 256-thread tiled kernels (the only ones for n_embd > 4096)
         const char *env = getenv("SPY_HIP_TILED");
-        m->wave = wave_ok(m) && !(env && env[0] == '1');
+        m->wave = wave_ok(m) && !(env && env[0] == '1' && m->uniform);
     }
     {
         int dev = 0; hipDeviceProp_t prop;
@@ -99,7 +118,11 @@ extern "C" int spy_hip_llama_create(const spy_hip_llama_desc *desc, spy_hip_llam
         const char *env = getenv("SPY_HIP_ATTN_SPLIT");
         rc = dalloc(m, (void **)&m->attn_sync, (size_t)c.n_head * 96 * 4, true);
         if (!rc && !(env && env[0] == '1') && m->hd == 128 && c.n_head * 8 <= m->num_cu && c.n_ctx <= 128 * 4 * ATL_RS && c.n_ctx <= 512 * ATL_RV)
-            m->attn_fused = (c.wtype == SPY_HIP_Q4_0 ? spy_probe_attn_layer_q4_0(m) : spy_probe_attn_layer_q8_0(m)) == 0;
+        {
+            bool ok = true;
+            for (int il = 0; il < c.n_layer && ok; il++) ok = probe_attn(m, il) == 0;
+            m->attn_fused = ok;
+        }
     }
     if (!rc && fused_ok(m)) { m->dry = true; rc = enqueue_pass_any(m, m->own_stream, true); m->dry = false; }   // sizes the persistent grids
     if (!rc && fused_ok(m)) {            // the persistent single-kernel pass: opt-in with SPY_HIP_MEGA=1 (slower than the per-phase kernels so far)
@@ -115,7 +138,7 @@ extern "C" int spy_hip_llama_create(const spy_hip_llama_desc *desc, spy_hip_llam
         if (!rc) rc = dalloc(m, (void **)&m->msync, sizeof(mega_sync), true);
         if (!rc && getenv("SPY_HIP_MEGA_STAMPS")) rc = dalloc(m, (void **)&m->mega_dbg, 128 * sizeof(long long), true);
         const char *env = getenv("SPY_HIP_MEGA");
-        if (!rc && env && env[0] == '1')
+        if (!rc && env && env[0] == '1' && m->uniform)
             m->mega = (c.wtype == SPY_HIP_Q4_0 ? spy_enqueue_mega_q4_0(m, m->own_stream, true) : spy_enqueue_mega_q8_0(m, m->own_stream, true)) == 0;
     }
     if (rc) { spy_hip_llama_destroy(m); return rc; }
@@ -154,7 +177,15 @@ extern "C" int spy_hip_llama_timing(spy_hip_llama *m, float *ms_per_pass, int32_
 static bool fused_ok(const spy_hip_llama *m) {
     // the fused kernels assume 128-wide heads (one key = 16 lanes x 128 bit), row pairs that share a
     // wave in the qkv / gate-up epilogues (<= 32 lanes per row) and n_embd <= 8192
-    return m->hd == 128 && (m->cfg_d.lpr == 16 || m->cfg_d.lpr == 32) && m->cfg_ff.lpr != 0 && m->desc.n_embd % 4 == 0 && m->desc.n_embd <= 8192;
+    if (!(m->hd == 128 && (m->cfg_d.lpr == 16 || m->cfg_d.lpr == 32) && m->cfg_ff.lpr != 0 && m->desc.n_embd % 4 == 0 && m->desc.n_embd <= 8192)) return false;
+    if (m->uniform) return true;
+    // mixed / K-quant layers: only the one-row-per-wave kernels, and the matrices one kernel reads share a type
+    if (!m->wave || m->desc.n_ff > 12288) return false;
+    for (const spy_hip_llama_layer &L : m->layers) {
+        if (L.t_wq != L.t_wk || L.t_gate != L.t_up) return false;
+        if (L.t_wv != L.t_wq && !(L.t_wq == SPY_HIP_Q4_K && L.t_wv == SPY_HIP_Q6_K)) return false;
+    }
+    return true;
 }
 
 static int enqueue_one(spy_hip_llama *m, hipStream_t st, int which, int il) {
@@ -173,7 +204,16 @@ static int enqueue_one(spy_hip_llama *m, hipStream_t st, int which, int il) {
         attn_pv_kernel<<<dim3((unsigned)(c.n_head * 8)), dim3(PV_THREADS), pv_lds, st>>>(m->st, m->scores, m->v_cache[il], m->attn_out, c.n_ctx);
         return SPY_LAUNCH_RC();
     }
-    return m->desc.wtype == SPY_HIP_Q4_0 ? spy_enqueue_kernel_q4_0(m, st, which, il) : spy_enqueue_kernel_q8_0(m, st, which, il);
+    // dispatch on the type of the kernel's (first) matrix
+    const spy_hip_llama_layer &L = m->layers[which == K_HEAD ? 0 : il];
+    const int t = which == K_QKV ? L.t_wq : which == K_WO ? L.t_wo : which == K_GATEUP ? L.t_gate : which == K_DOWN ? L.t_down : c.t_out;
+    switch (t) {
+    case SPY_HIP_Q4_0: return spy_enqueue_kernel_q4_0(m, st, which, il);
+    case SPY_HIP_Q8_0: return spy_enqueue_kernel_q8_0(m, st, which, il);
+    case SPY_HIP_Q4_K: return spy_enqueue_kernel_q4_k(m, st, which, il);
+    case SPY_HIP_Q6_K: return spy_enqueue_kernel_q6_k(m, st, which, il);
+    }
+    return SPY_HIP_EUNSUPPORTED;
 }
 
 static int enqueue_pass_any(spy_hip_llama *m, hipStream_t st, bool sample) {
@@ -274,9 +314,9 @@ static int forward_ops(spy_hip_llama *m, hipStream_t st, const int32_t *tokens_h
         spy_hip_tensor t_nw = T2(SPY_HIP_F32, (void *)L.attn_norm, d, 1); t_nw.dim = 1;
         RC_TRY(spy_hip_op_norm_rms(st, &t_x, &t_xn, c.eps));
         RC_TRY(spy_hip_op_binary(st, 2, &t_xn, &t_nw, &t_xn));
-        RC_TRY(mm(L.wq, c.wtype, d, d, &t_xn, &t_q));
-        RC_TRY(mm(L.wk, c.wtype, d, d, &t_xn, &t_k));
-        RC_TRY(mm(L.wv, c.wtype, d, d, &t_xn, &t_v));
+        RC_TRY(mm(L.wq, L.t_wq, d, d, &t_xn, &t_q));
+        RC_TRY(mm(L.wk, L.t_wk, d, d, &t_xn, &t_k));
+        RC_TRY(mm(L.wv, L.t_wv, d, d, &t_xn, &t_v));
         spy_hip_tensor t_q3 = T3s(SPY_HIP_F32, q, hd, H, T, 4, 4 * hd, 4 * d), t_k3 = T3s(SPY_HIP_F32, k, hd, H, T, 4, 4 * hd, 4 * d);
         RC_TRY(spy_hip_op_rope(st, &t_q3, &t_pos, &t_q3, &rp));
         RC_TRY(spy_hip_op_rope(st, &t_k3, &t_pos, &t_k3, &rp));
@@ -297,16 +337,16 @@ static int forward_ops(spy_hip_llama *m, hipStream_t st, const int32_t *tokens_h
         spy_hip_tensor t_Op = T3s(SPY_HIP_F32, o, hd, H, T, 4, 4 * hd * T, 4 * hd);                    // Permute {0,2,1,3}
         spy_hip_tensor t_o2c = T3s(SPY_HIP_F32, o2, hd, H, T, 4, 4 * hd, 4 * d);
         RC_TRY(spy_hip_op_contiguous(st, &t_Op, &t_o2c));
-        RC_TRY(mm(L.wo, c.wtype, d, d, &t_o2, &t_t1));
+        RC_TRY(mm(L.wo, L.t_wo, d, d, &t_o2, &t_t1));
         RC_TRY(spy_hip_op_binary(st, 0, &t_t1, &t_x, &t_t1));
         t_nw.data = (void *)L.ffn_norm;
         RC_TRY(spy_hip_op_norm_rms(st, &t_t1, &t_xn, c.eps));
         RC_TRY(spy_hip_op_binary(st, 2, &t_xn, &t_nw, &t_xn));
-        RC_TRY(mm(L.w_up, c.wtype, d, F, &t_xn, &t_up));
-        RC_TRY(mm(L.w_gate, c.wtype, d, F, &t_xn, &t_gate));
+        RC_TRY(mm(L.w_up, L.t_up, d, F, &t_xn, &t_up));
+        RC_TRY(mm(L.w_gate, L.t_gate, d, F, &t_xn, &t_gate));
         RC_TRY(spy_hip_op_silu(st, &t_gate, &t_gate));
         RC_TRY(spy_hip_op_binary(st, 2, &t_up, &t_gate, &t_par));
-        RC_TRY(mm(L.w_down, c.wtype, F, d, &t_par, &t_od));
+        RC_TRY(mm(L.w_down, L.t_down, F, d, &t_par, &t_od));
         RC_TRY(spy_hip_op_binary(st, 0, &t_t1, &t_od, &t_x));
     }
     {

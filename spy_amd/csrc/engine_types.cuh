@@ -17,6 +17,7 @@ struct spy_hip_llama {
     bool dry = false;
     bool attn_fused = false;                    // qkv + scores + softmax/KQV of a layer in one launch
     uint32_t *attn_sync = nullptr;
+    bool uniform = true;                        // every layer matrix and the head in desc.wtype, Q4_0 or Q8_0
     bool wave = false;                          // one-row-per-wave kernels (1024-thread workgroups) instead of the tiled ones
     std::vector<uint16_t *> k_cache, v_cache;
     float *x = nullptr, *x1 = nullptr, *attn_out = nullptr, *hbuf = nullptr, *scores = nullptr, *logits = nullptr, *rope_cs = nullptr;
@@ -55,9 +56,13 @@ enum { K_QKV = 0, K_SCORES, K_PV, K_WO, K_GATEUP, K_DOWN, K_HEAD, K_COUNT };
 // With m->dry set nothing is launched: the call only sizes the persistent grids.
 int spy_enqueue_kernel_q4_0(spy_hip_llama *m, hipStream_t st, int which, int il);
 int spy_enqueue_kernel_q8_0(spy_hip_llama *m, hipStream_t st, int which, int il);
+int spy_enqueue_kernel_q4_k(spy_hip_llama *m, hipStream_t st, int which, int il);
+int spy_enqueue_kernel_q6_k(spy_hip_llama *m, hipStream_t st, int which, int il);
 // The persistent kernel covering embedding .. output head of one pass.  probe: only check that the
 // kernel for this shape exists and that one workgroup per compute unit is resident.
-int spy_probe_attn_layer_q4_0(spy_hip_llama *m);
-int spy_probe_attn_layer_q8_0(spy_hip_llama *m);
+int spy_probe_attn_layer_q4_0(spy_hip_llama *m, int il);
+int spy_probe_attn_layer_q8_0(spy_hip_llama *m, int il);
+int spy_probe_attn_layer_q4_k(spy_hip_llama *m, int il);
+int spy_probe_attn_layer_q6_k(spy_hip_llama *m, int il);
 int spy_enqueue_mega_q4_0(spy_hip_llama *m, hipStream_t st, bool probe);
 int spy_enqueue_mega_q8_0(spy_hip_llama *m, hipStream_t st, bool probe);

@@ -75,6 +75,99 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_kernel(gemv_args a) {
     }
 }
 
+// ---- one weight row per wave, 1024-thread workgroups (all four weight types; K <= 4096 * NITK) ------
+// The standalone form of the single-token kernels: native Q8_0 activation row(s) staged into LDS by
+// the whole workgroup, every wave owns rows r = gw + k*NW with 64 lanes x NITK 64-element units each,
+// WROW_DEPTH rows requested ahead of their use.  T activation rows are handled one after the other
+// against the same row registers (the weights are read once per launch for up to WROW_T rows).
+#define WROW_THREADS 1024
+#define WROW_DEPTH 3
+#define WROW_T 4
+template <int WT, int NITK, int NR>
+__global__ __launch_bounds__(WROW_THREADS) void wave_row_kernel(gemv_args a, int T) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int NW = (int)gridDim.x * (WROW_THREADS / 64), gw = (int)blockIdx.x * (WROW_THREADS / 64) + wave;
+    const int K = a.K, nblk = K / 32, npair = K / 64;
+    const size_t RB = (size_t)spy_row_size(WT, K);
+    wtile<WT, NITK> t[NR];
+    auto issue = [&](int k) {
+        const int u = gw + k * NW, r = u < a.M ? u : gw % a.M;
+        load_tile<WT, 64, NITK>(t[k], a.W + (size_t)r * RB, npair, lane);
+    };
+#pragma unroll
+    for (int k = 0; k < NR; k++) if (k < WROW_DEPTH) issue(k);
+    staged_act act[WROW_T];
+#pragma unroll
+    for (int c = 0; c < WROW_T; c++) {
+        int8_t *q = (int8_t *)(smem + (size_t)c * staged_bytes(K));
+        int2 *meta = (int2 *)(q + staged_q_bytes(K));
+        if (c < T) stage_native_q8<WROW_THREADS>(a.xq + (size_t)c * nblk * 34, q, meta, nblk);
+        act[c].q = q; act[c].meta = meta;
+    }
+    constexpr bool HOIST = NR > 1;                          // keep the lane's activations in registers across rows
+    act_frag<HOIST ? NITK : 1> af;
+    if constexpr (HOIST) load_act_frag<WT, NITK>(af, act[0], npair, lane);
+#pragma unroll
+    for (int k = 0; k < NR; k++) {
+        if (k + WROW_DEPTH < NR) issue(k + WROW_DEPTH);
+        const int r = gw + k * NW;
+        float s;
+        if constexpr (HOIST) s = wave_total_lane63(dot_row_frag<WT, NITK>(t[k], af, npair, lane));
+        else s = wave_total_lane63(dot_row_lds<WT, NITK>(t[k], act[0], npair, lane));
+        if (lane == 63 && r < a.M) a.dst[r] = a.residual ? s + a.residual[r] : s;
+        for (int c = 1; c < T; c++) {                       // further activation rows against the same weight registers
+            s = wave_total_lane63(dot_row_lds<WT, NITK>(t[k], act[c], npair, lane));
+            const size_t o = (size_t)c * a.dst_stride + r;
+            if (lane == 63 && r < a.M) a.dst[o] = a.residual ? s + a.residual[o] : s;
+        }
+    }
+}
+
+template <int WT, int NITK>
+static int launch_wave_row_nitk(hipStream_t st, const gemv_args &a, int T) {
+    constexpr int NRMAX = (WT == SPY_HIP_Q4_0 || WT == SPY_HIP_Q4_K) ? 6 : 3;      // rows per wave: row registers = NR * NITK * PAIR_DW
+    constexpr int NR = NITK == 1 ? NRMAX : 1;
+    static int num_cu = 0;
+    if (!num_cu) { int dev = 0; hipDeviceProp_t prop; num_cu = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) ? prop.multiProcessorCount : 256; }
+    const size_t lds = (size_t)T * staged_bytes(a.K);
+    auto kern1 = wave_row_kernel<WT, NITK, 1>;
+    auto kernN = wave_row_kernel<WT, NITK, NR>;
+    static size_t lds_set = 0;
+    if (lds > 48 * 1024 && lds > lds_set) {
+        { hipError_t e_ = hipFuncSetAttribute((const void *)kern1, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); if (e_ != hipSuccess) return (int)e_; }
+        { hipError_t e_ = hipFuncSetAttribute((const void *)kernN, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); if (e_ != hipSuccess) return (int)e_; }
+        lds_set = lds;
+    }
+    // few rows: one per wave over as many workgroups as needed; many rows: NR per wave
+    const int waves = WROW_THREADS / 64;
+    if ((int64_t)a.M <= (int64_t)num_cu * waves) kern1<<<dim3((unsigned)((a.M + waves - 1) / waves)), dim3(WROW_THREADS), lds, st>>>(a, T);
+    else kernN<<<dim3((unsigned)((a.M + waves * NR - 1) / (waves * NR))), dim3(WROW_THREADS), lds, st>>>(a, T);
+    return SPY_LAUNCH_RC();
+}
+
+// K % 64 == 0 (Q4_0 / Q8_0) or K % 256 == 0 (K-quants), K <= 12288
+template <int WT>
+static int launch_wave_rows(hipStream_t st, const void *w, const uint8_t *xq, float *dst, const float *residual, int64_t M, int64_t K, int64_t T, int64_t dst_stride) {
+    const int64_t xrow = (K / 32) * 34;
+    for (int64_t t = 0; t < T; t += WROW_T) {
+        gemv_args a;
+        a.W = (const uint8_t *)w; a.xq = xq + t * xrow; a.dst = dst + t * dst_stride;
+        a.residual = residual ? residual + t * dst_stride : nullptr; a.dump = nullptr;
+        a.M = (int)M; a.K = (int)K; a.dst_stride = dst_stride;
+        const int tc = (int)(T - t < WROW_T ? T - t : WROW_T);
+        int rc;
+        switch ((K + 4095) / 4096) {
+        case 1: rc = launch_wave_row_nitk<WT, 1>(st, a, tc); break;
+        case 2: rc = launch_wave_row_nitk<WT, 2>(st, a, tc); break;
+        case 3: rc = launch_wave_row_nitk<WT, 3>(st, a, tc); break;
+        default: return SPY_HIP_EUNSUPPORTED;
+        }
+        if (rc) return rc;
+    }
+    return 0;
+}
+
 // ---- generic path: any K % 32 == 0 (Q4_0 / Q8_0) or K % 256 == 0 (Q4_K / Q6_K); one wave per
 // row, lanes stride over Q8_0 activation blocks and read weights from global memory bytewise.
 // Used for shapes the tiled kernel does not take and for the K-quants.
@@ -248,8 +341,12 @@ extern "C" int spy_hip_gemv_q8_0act(void *stream, int wtype, const void *w, cons
     case SPY_HIP_Q8_0:
         return pick_cfg(K).lpr ? gemv_fast_cols<SPY_HIP_Q8_0>(st, w, (const uint8_t *)xq, dst, residual, M, K, T, dst_stride)
                                          : launch_generic<SPY_HIP_Q8_0, false>(st, w, xq, dst, residual, nullptr, M, K, T, dst_stride);
-    case SPY_HIP_Q4_K: return launch_generic<SPY_HIP_Q4_K, false>(st, w, xq, dst, residual, nullptr, M, K, T, dst_stride);
-    case SPY_HIP_Q6_K: return launch_generic<SPY_HIP_Q6_K, false>(st, w, xq, dst, residual, nullptr, M, K, T, dst_stride);
+    case SPY_HIP_Q4_K:
+        return K <= 12288 ? launch_wave_rows<SPY_HIP_Q4_K>(st, w, (const uint8_t *)xq, dst, residual, M, K, T, dst_stride)
+                          : launch_generic<SPY_HIP_Q4_K, false>(st, w, xq, dst, residual, nullptr, M, K, T, dst_stride);
+    case SPY_HIP_Q6_K:
+        return K <= 12288 ? launch_wave_rows<SPY_HIP_Q6_K>(st, w, (const uint8_t *)xq, dst, residual, M, K, T, dst_stride)
+                          : launch_generic<SPY_HIP_Q6_K, false>(st, w, xq, dst, residual, nullptr, M, K, T, dst_stride);
     }
     return SPY_HIP_EUNSUPPORTED;
 }

@@ -32,6 +32,12 @@ static __device__ __forceinline__ float4 ldc4(const float *p) { return make_floa
 template <int WT> struct wt_traits;
 template <> struct wt_traits<SPY_HIP_Q4_0> { static constexpr int BLK = 18, PAIR_DW = 9; };
 template <> struct wt_traits<SPY_HIP_Q8_0> { static constexpr int BLK = 34, PAIR_DW = 17; };
+// K-quants (64 lanes per row only): a lane's unit is a quarter super-block = 64 elements, the same
+// span as a block pair.  Q4_K: the 16-byte header {d, dmin, scales[12]} + the 32 nibble bytes of sub-blocks
+// 2j, 2j+1.  Q6_K (super-blocks only 2-byte aligned): three 16-byte chunks (ql, ql + 32, qh) as 5 raw
+// dwords each, 8 scale bytes as 3 raw dwords, d, and the byte shift of the super-block (0 or 16 bits).
+template <> struct wt_traits<SPY_HIP_Q4_K> { static constexpr int PAIR_DW = 12; };
+template <> struct wt_traits<SPY_HIP_Q6_K> { static constexpr int PAIR_DW = 20; };
 #define GEMV_NIT_MAX 4        // block pairs per lane per row tile: 1..4 (exact value is a template parameter)
 
 template <int CTRL> static __device__ __forceinline__ float dpp_add(float v) {
@@ -92,17 +98,18 @@ static __device__ __forceinline__ const int4 *act_part(const int8_t *q, int p, i
 // ---- activation staging --------------------------------------------------------------------
 
 // native Q8_0 blocks (34 bytes, 2-byte aligned) -> staged LDS form. Ends with __syncthreads().
+template <int THREADS = GEMV_THREADS>
 static __device__ __forceinline__ void stage_native_q8(const uint8_t *__restrict__ xq, int8_t *s_q, int2 *s_meta, int nblk) {
     const uint16_t *src = (const uint16_t *)xq;
     const int total_h = nblk * 17;
-    for (int h = threadIdx.x; h < total_h; h += GEMV_THREADS) {
+    for (int h = threadIdx.x; h < total_h; h += THREADS) {
         const int b = h / 17, w = h - b * 17;
         const uint16_t v = src[h];
         if (w == 0) s_meta[b].x = __float_as_int(h2f(v));
         else { const int hw = b * 16 + (w - 1); ((uint16_t *)s_q)[2 * act_dw(hw >> 1, nblk >> 1) + (hw & 1)] = v; }
     }
     __syncthreads();
-    for (int b = threadIdx.x; b < nblk; b += GEMV_THREADS) {
+    for (int b = threadIdx.x; b < nblk; b += THREADS) {
         const int4 q0 = *act_part(s_q, b >> 1, 2 * (b & 1), nblk >> 1), q1 = *act_part(s_q, b >> 1, 2 * (b & 1) + 1, nblk >> 1);
         int s = 0;
         s = __builtin_amdgcn_sdot4(q0.x, 0x01010101, s, false); s = __builtin_amdgcn_sdot4(q0.y, 0x01010101, s, false);
@@ -235,9 +242,36 @@ static __device__ __forceinline__ void load_tile(wtile<WT, NIT> &t, const uint8_
 #pragma unroll
     for (int it = 0; it < NIT; it++) {
         const int p = min(it * LPR + l, npair - 1);
-        const uint32_t *wp = (const uint32_t *)rowp + (size_t)p * DW;
+        if constexpr (WT == SPY_HIP_Q4_K) {
+            static_assert(WT != SPY_HIP_Q4_K || LPR == 64, "K-quant tiles use 64 lanes per row");
+            const uint8_t *sb = rowp + (size_t)(p >> 2) * 144;
+            const uint4 hdr = *(const uint4 *)sb, q0 = *(const uint4 *)(sb + 16 + 32 * (p & 3)), q1 = *(const uint4 *)(sb + 32 + 32 * (p & 3));
+            t.w[it][0] = hdr.x; t.w[it][1] = hdr.y; t.w[it][2] = hdr.z; t.w[it][3] = hdr.w;
+            t.w[it][4] = q0.x; t.w[it][5] = q0.y; t.w[it][6] = q0.z; t.w[it][7] = q0.w;
+            t.w[it][8] = q1.x; t.w[it][9] = q1.y; t.w[it][10] = q1.z; t.w[it][11] = q1.w;
+        } else if constexpr (WT == SPY_HIP_Q6_K) {
+            static_assert(WT != SPY_HIP_Q6_K || LPR == 64, "K-quant tiles use 64 lanes per row");
+            // lane (n = half of the super-block, e = 16-element slice): ql[64n + 16e ..], ql[64n + 32 + 16e ..], qh[32n + 16e ..],
+            // scales[8n ..]; every chunk read as aligned dwords around it (the last dword index is clamped
+            // when the chunk is aligned, so nothing beyond the super-block is touched)
+            const int j = p & 3, n = j >> 1, e = j & 1;
+            const uint8_t *sb = rowp + (size_t)(p >> 2) * 210;
+            const uint32_t sh = ((uint32_t)(uintptr_t)sb & 2u) ? 16u : 0u;
+            const uint32_t *base = (const uint32_t *)((uintptr_t)sb & ~(uintptr_t)3);        // sb - (0 | 2) bytes
+            const int last4 = sh ? 4 : 3, last2 = sh ? 2 : 1;
+            const uint32_t *ca = base + (64 * n + 16 * e) / 4, *cb = base + (64 * n + 32 + 16 * e) / 4, *ch = base + (128 + 32 * n + 16 * e) / 4;
+            const uint32_t *cs = base + (192 + 8 * n) / 4;
 #pragma unroll
-        for (int i = 0; i < DW; i++) t.w[it][i] = wp[i];
+            for (int i = 0; i < 4; i++) { t.w[it][i] = ca[i]; t.w[it][5 + i] = cb[i]; t.w[it][10 + i] = ch[i]; }
+            t.w[it][4] = ca[last4]; t.w[it][9] = cb[last4]; t.w[it][14] = ch[last4];
+            t.w[it][15] = cs[0]; t.w[it][16] = cs[1]; t.w[it][17] = cs[last2];
+            t.w[it][18] = *(const uint16_t *)(sb + 208);
+            t.w[it][19] = sh;
+        } else {
+            const uint32_t *wp = (const uint32_t *)rowp + (size_t)p * DW;
+#pragma unroll
+            for (int i = 0; i < DW; i++) t.w[it][i] = wp[i];
+        }
     }
 }
 
@@ -264,9 +298,75 @@ static __device__ __forceinline__ int dot_q8_dwords(const uint32_t *n, const int
 // One block pair of a weight row (w: its PAIR_DW dwords) with the matching 64 int8 activations
 // (x0..x3: 16 bytes each) and their meta {scale bits, sum q} x 2: the two exact int32 block dots
 // (optionally dumped), scaled and accumulated like the reference's fma (vec_dot.h:76-79).
+// byte k (0..11) of three dwords
+static __device__ __forceinline__ uint32_t byte_of3(uint32_t a, uint32_t b, uint32_t c, int k) {
+    const uint32_t w = k < 4 ? a : (k < 8 ? b : c);
+    return (w >> (8 * (k & 3))) & 0xFFu;
+}
+// 4 packed 6-bit values (0..63 per byte) -> 4 int8 of (v - 32)
+static __device__ __forceinline__ uint32_t q6_m32(uint32_t v) { return (v + 0x60606060u) ^ 0x80808080u; }
+
 template <int WT>
-static __device__ __forceinline__ float dot_pair(const uint32_t *w, const int4 x0, const int4 x1, const int4 x2, const int4 x3, const int4 mm,
-                                                 float acc, int32_t *dump2) {
+static __device__ __forceinline__ float dot_pair(const uint32_t *w, const int4 x0, const int4 x1, const int4 x2, const int4 x3, const int4 mm, const int4 mm2,
+                                                 int p, float acc, int32_t *dump2) {
+    if constexpr (WT == SPY_HIP_Q4_K) {
+        // sub-blocks a = 2j (low nibbles) and a + 1 (high nibbles) of the super-block; 6-bit scale / min pairs
+        // from scales[12]; value = d*sc*q - dmin*m (k-quant.h:101-111 holds the layout only)
+        const int j = p & 3, a = 2 * j;
+        const float d = h2f((uint16_t)(w[0] & 0xFFFFu)), dmin = h2f((uint16_t)(w[0] >> 16));
+        int scA, mA, scB, mB;
+        if (j < 2) {
+            scA = byte_of3(w[1], w[2], w[3], a) & 63;     mA = byte_of3(w[1], w[2], w[3], a + 4) & 63;
+            scB = byte_of3(w[1], w[2], w[3], a + 1) & 63; mB = byte_of3(w[1], w[2], w[3], a + 5) & 63;
+        } else {
+            const uint32_t hA = byte_of3(w[1], w[2], w[3], a + 4), hB = byte_of3(w[1], w[2], w[3], a + 5);
+            scA = (hA & 0x0F) | ((byte_of3(w[1], w[2], w[3], a - 4) >> 6) << 4); mA = (hA >> 4) | ((byte_of3(w[1], w[2], w[3], a) >> 6) << 4);
+            scB = (hB & 0x0F) | ((byte_of3(w[1], w[2], w[3], a - 3) >> 6) << 4); mB = (hB >> 4) | ((byte_of3(w[1], w[2], w[3], a + 1) >> 6) << 4);
+        }
+        int iA = 0, iB = 0;
+        const int xa[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w}, xb[8] = {x2.x, x2.y, x2.z, x2.w, x3.x, x3.y, x3.z, x3.w};
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            iA = __builtin_amdgcn_sdot4((int)(w[4 + i] & 0x0F0F0F0Fu), xa[i], iA, false);
+            iB = __builtin_amdgcn_sdot4((int)((w[4 + i] >> 4) & 0x0F0F0F0Fu), xb[i], iB, false);
+        }
+        if (dump2) { dump2[0] = iA; dump2[1] = iB; }
+        acc = fmaf(__int_as_float(mm.x), d * (float)(scA * iA) - dmin * (float)(mA * mm.y), acc);
+        acc = fmaf(__int_as_float(mm.z), d * (float)(scB * iB) - dmin * (float)(mB * mm.w), acc);
+        return acc;
+    } else if constexpr (WT == SPY_HIP_Q6_K) {
+        // lane (n, e): elements l + 32 m, l in [16e, 16e + 16), m = 0..3 of half n: 6-bit quants from the low /
+        // high nibbles of ql / ql + 32 and bit pairs 2m of qh, minus 32; scale = d * scales[8n + e + 2m]
+        const uint32_t sh = w[19];
+        uint32_t qa[4], qb[4], qh[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            qa[i] = __builtin_amdgcn_alignbit(w[i + 1], w[i], sh);
+            qb[i] = __builtin_amdgcn_alignbit(w[6 + i], w[5 + i], sh);
+            qh[i] = __builtin_amdgcn_alignbit(w[11 + i], w[10 + i], sh);
+        }
+        const uint32_t s0 = __builtin_amdgcn_alignbit(w[16], w[15], sh), s1 = __builtin_amdgcn_alignbit(w[17], w[16], sh);
+        const int e = p & 1;
+        const float d = h2f((uint16_t)(w[18] & 0xFFFFu));
+        int isum[4] = {0, 0, 0, 0};
+        const int xm[4][4] = {{x0.x, x0.y, x0.z, x0.w}, {x1.x, x1.y, x1.z, x1.w}, {x2.x, x2.y, x2.z, x2.w}, {x3.x, x3.y, x3.z, x3.w}};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t h = qh[i];
+            isum[0] = __builtin_amdgcn_sdot4((int)q6_m32((qa[i] & 0x0F0F0F0Fu) | ((h & 0x03030303u) << 4)), xm[0][i], isum[0], false);
+            isum[1] = __builtin_amdgcn_sdot4((int)q6_m32((qb[i] & 0x0F0F0F0Fu) | ((h & 0x0C0C0C0Cu) << 2)), xm[1][i], isum[1], false);
+            isum[2] = __builtin_amdgcn_sdot4((int)q6_m32(((qa[i] >> 4) & 0x0F0F0F0Fu) | (h & 0x30303030u)), xm[2][i], isum[2], false);
+            isum[3] = __builtin_amdgcn_sdot4((int)q6_m32(((qb[i] >> 4) & 0x0F0F0F0Fu) | ((h >> 2) & 0x30303030u)), xm[3][i], isum[3], false);
+        }
+        const float dx[4] = {__int_as_float(mm.x), __int_as_float(mm.z), __int_as_float(mm2.x), __int_as_float(mm2.z)};
+#pragma unroll
+        for (int m = 0; m < 4; m++) {
+            const int k = e + 2 * m;                                     // scale byte of the half (0..7)
+            const int sc = (int)(int8_t)(((k < 4 ? s0 : s1) >> (8 * (k & 3))) & 0xFFu);
+            acc = fmaf(dx[m] * d, (float)(sc * isum[m]), acc);
+        }
+        return acc;
+    } else {
     int iA, iB;
     float dA, dB;
     if constexpr (WT == SPY_HIP_Q4_0) {
@@ -287,6 +387,7 @@ static __device__ __forceinline__ float dot_pair(const uint32_t *w, const int4 x
     acc = fmaf(dA * __int_as_float(mm.x), (float)iA, acc);
     acc = fmaf(dB * __int_as_float(mm.z), (float)iB, acc);
     return acc;
+    }
 }
 
 template <int WT, int LPR, int NIT, int NT>
@@ -301,7 +402,7 @@ static __device__ __forceinline__ void dot_tile(const wtile<WT, NIT> &t, const s
                 const int8_t *xq = act[c].q;
                 const int4 mm = *(const int4 *)(act[c].meta + 2 * p);
                 acc[c] = dot_pair<WT>(t.w[it], *act_part(xq, p, 0, npair), *act_part(xq, p, 1, npair), *act_part(xq, p, 2, npair), *act_part(xq, p, 3, npair),
-                                      mm, acc[c], (dump && c == 0) ? dump + 2 * p : nullptr);
+                                      mm, mm, p, acc[c], (dump && c == 0) ? dump + 2 * p : nullptr);
             }
         }
     }
@@ -309,15 +410,25 @@ static __device__ __forceinline__ void dot_tile(const wtile<WT, NIT> &t, const s
 
 // The activations one lane needs when it owns the same block pairs of every row (64 lanes per row):
 // read from LDS once, reused for all rows of the wave.
-template <int NIT> struct act_frag { int4 x[NIT][4]; int4 mm[NIT]; };
-template <int NIT>
+template <int NIT> struct act_frag { int4 x[NIT][4]; int4 mm[NIT]; int4 mm2[NIT]; };
+template <int WT, int NIT>
 static __device__ __forceinline__ void load_act_frag(act_frag<NIT> &f, const staged_act &act, int npair, int lane) {
 #pragma unroll
     for (int it = 0; it < NIT; it++) {
         const int p = min(it * 64 + lane, npair - 1);
+        if constexpr (WT == SPY_HIP_Q6_K) {
+            // 16-element slices e and 2 + e of the two pairs (= four 32-element blocks) of the lane's half
+            const int pa = p & ~1, pb = p | 1, e = p & 1;
+            f.x[it][0] = *act_part(act.q, pa, e, npair); f.x[it][1] = *act_part(act.q, pa, 2 + e, npair);
+            f.x[it][2] = *act_part(act.q, pb, e, npair); f.x[it][3] = *act_part(act.q, pb, 2 + e, npair);
+            f.mm[it] = *(const int4 *)(act.meta + 2 * pa);
+            f.mm2[it] = *(const int4 *)(act.meta + 2 * pb);
+        } else {
 #pragma unroll
-        for (int j = 0; j < 4; j++) f.x[it][j] = *act_part(act.q, p, j, npair);
-        f.mm[it] = *(const int4 *)(act.meta + 2 * p);
+            for (int j = 0; j < 4; j++) f.x[it][j] = *act_part(act.q, p, j, npair);
+            f.mm[it] = *(const int4 *)(act.meta + 2 * p);
+            f.mm2[it] = f.mm[it];
+        }
     }
 }
 template <int WT, int NIT>
@@ -325,7 +436,24 @@ static __device__ __forceinline__ float dot_row_frag(const wtile<WT, NIT> &t, co
     float acc = 0.0f;
 #pragma unroll
     for (int it = 0; it < NIT; it++)
-        if (it * 64 + lane < npair) acc = dot_pair<WT>(t.w[it], f.x[it][0], f.x[it][1], f.x[it][2], f.x[it][3], f.mm[it], acc, nullptr);
+        if (it * 64 + lane < npair) acc = dot_pair<WT>(t.w[it], f.x[it][0], f.x[it][1], f.x[it][2], f.x[it][3], f.mm[it], f.mm2[it], it * 64 + lane, acc, nullptr);
+    return acc;
+}
+
+// The same dot with the activations read from LDS unit by unit (single-row waves with several units per
+// lane: keeps the register footprint to one unit's activations).
+template <int WT, int NIT>
+static __device__ __forceinline__ float dot_row_lds(const wtile<WT, NIT> &t, const staged_act &act, int npair, int lane) {
+    float acc = 0.0f;
+#pragma unroll
+    for (int it = 0; it < NIT; it++) {
+        const int p = it * 64 + lane;
+        if (p < npair) {
+            act_frag<1> f;
+            load_act_frag<WT, 1>(f, act, npair, p);
+            acc = dot_pair<WT>(t.w[it], f.x[0][0], f.x[0][1], f.x[0][2], f.x[0][3], f.mm[0], f.mm2[0], p, acc, nullptr);
+        }
+    }
     return acc;
 }
 

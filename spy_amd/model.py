@@ -116,6 +116,8 @@ def synth_model(cfg, seed=1234, std=0.02, outlier_every=0, quantizer=None, norm_
 
 LlamaLayer, LlamaDesc = H.LlamaLayer, H.LlamaDesc
 
+_LAYER_TYPES = [("t_wq", "attn_q"), ("t_wk", "attn_k"), ("t_wv", "attn_v"), ("t_wo", "attn_output"), ("t_gate", "ffn_gate"),
+                ("t_up", "ffn_up"), ("t_down", "ffn_down")]
 _LAYER_FIELDS = [("attn_norm", "attn_norm"), ("ffn_norm", "ffn_norm"), ("wq", "attn_q"), ("wk", "attn_k"), ("wv", "attn_v"),
                  ("wo", "attn_output"), ("w_gate", "ffn_gate"), ("w_up", "ffn_up"), ("w_down", "ffn_down")]
 
@@ -136,6 +138,8 @@ class Engine:
         for i in range(cfg.n_layer):
             for field, gname in _LAYER_FIELDS:
                 setattr(self._layers[i], field, self.dev["blk.%d.%s.weight" % (i, gname)].ptr)
+            for tfield, gname in _LAYER_TYPES:
+                setattr(self._layers[i], tfield, cfg.tensor_types.get(gname, 0))
         d = LlamaDesc(cfg.n_layer, cfg.n_embd, cfg.n_head, cfg.n_ff, cfg.n_vocab, cfg.n_ctx, cfg.eps, cfg.rope_freq_base,
                       cfg.wtype, self.dev["token_embd.weight"].ptr, cfg.t_tok_embd, self.dev["output_norm.weight"].ptr,
                       self.dev["output.weight"].ptr, cfg.t_out, self._layers)

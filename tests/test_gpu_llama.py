@@ -180,3 +180,46 @@ def test_llama2_7b_q4_0_greedy_32_tokens():
     print("hip tokens:   ", got.tolist(), "\nfree-running: first %d tokens identical (first undecidable step: %d)" % (n_same, first_undecidable), flush=True)
     assert n_same >= first_undecidable
     eng.close()
+
+
+@pytest.mark.parametrize("name,kw", [
+    ("Q4_K + Q6_K head", dict(wtype=O.Q4_K, t_out=O.Q6_K)),
+    ("Q6_K", dict(wtype=O.Q6_K)),
+    ("Q4_K_M mix", dict(wtype=O.Q4_K, t_out=O.Q6_K, tensor_types={"attn_v": O.Q6_K, "ffn_down": O.Q6_K})),
+    ("Q8_0 body, Q4_K gate|up", dict(wtype=O.Q8_0, tensor_types={"ffn_gate": O.Q4_K, "ffn_up": O.Q4_K})),
+])
+@pytest.mark.parametrize("dims", [(2, 512, 4, 1024, 768, 48), (1, 4096, 32, 11008, 2048, 1024)])
+def test_k_quant_layers_in_the_fused_pass(name, kw, dims):
+    """K-quant and mixed-type layers through the fused single-token kernels (and the prompt path) against
+    the oracle.  The reference has no K-quant arithmetic: both sides follow the public ggml block layouts
+    (parity unpinned against the reference itself)."""
+    from spy_amd import model as M
+    from tests.gpu_util import E2E_TOL          # whole passes: see the note on re-quantization there
+    from tests.model_util import OracleModel, k_quant_quantizer
+    n_layer, d, H_, F, V, C_ = dims
+    cfg = M.Config(n_layer=n_layer, n_embd=d, n_head=H_, n_ff=F, n_vocab=V, n_ctx=C_, **kw)
+    tensors = M.synth_model(cfg, seed=31, outlier_every=1000, quantizer=k_quant_quantizer)
+    eng, ora = M.Engine(cfg, tensors), OracleModel(cfg, tensors)
+    rng = np.random.default_rng(8)
+    n_prompt = 9 if C_ < 512 else C_ - 10
+    if C_ < 512:
+        prompt = rng.integers(0, V, n_prompt).astype(np.int32)
+        _close(eng.forward(prompt, 0), ora.forward(prompt, 0), "%s prefill logits" % name, E2E_TOL)
+    else:
+        for il in range(n_layer):
+            k = (rng.standard_normal(n_prompt * d) * 1.2).astype(np.float16).view(np.uint16)
+            v = np.zeros((d, C_), np.float16)
+            v[:, :n_prompt] = (rng.standard_normal((d, n_prompt)) * 1.2).astype(np.float16)
+            eng.write_buffer("k_cache", il, np.concatenate([k, np.zeros((C_ - n_prompt) * d, np.uint16)]))
+            eng.write_buffer("v_cache", il, v.view(np.uint16))
+            ora.k_cache[il][:n_prompt * d] = k
+            ora.v_cache[il][:] = v.view(np.uint16).reshape(-1)
+    tok = int(rng.integers(0, V))
+    for step in range(3):
+        t = np.array([tok], np.int32)
+        lg, lo = eng.forward(t, n_prompt + step)[0], ora.forward(t, n_prompt + step)[0]
+        _close(lg, lo, "%s single-token logits, step %d" % (name, step), E2E_TOL)
+        tok = int(np.argmax(lo))
+    toks = eng.decode_greedy(tok, n_prompt + 3, 3, use_graph=True)
+    assert len(toks) == 3
+    eng.close()
