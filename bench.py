@@ -35,6 +35,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-steps", type=int, default=8)
     ap.add_argument("--layers", type=int, default=32, help="debug only: fewer layers (result is then not the headline config)")
+    ap.add_argument("--model", choices=["q4_0", "q8_0", "q4_k_m"], default="q4_0",
+                    help="q4_0: the headline workload; q8_0 / q4_k_m (Q4_K with Q6_K attn_v, ffn_down and head): the other 7B configurations")
     ap.add_argument("--no-graph", action="store_true", help="launch the kernels of every pass one by one instead of replaying a HIP graph (for profilers)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch a plain copy kernel over 256 MiB three times (a known-size dispatch to scale profiler byte counters by)")
@@ -53,10 +55,16 @@ def main():
     log("device:", info)
     steps, warmup, fill = args.steps, args.warmup, args.ctx_fill
     n_ctx = (fill + warmup + steps + 8 + 7) // 8 * 8
-    cfg = M.Config.llama2_7b(n_ctx=n_ctx, wtype=H.Q4_0)
+    if args.model == "q4_0":
+        cfg = M.Config.llama2_7b(n_ctx=n_ctx, wtype=H.Q4_0)
+    elif args.model == "q8_0":
+        cfg = M.Config.llama2_7b(n_ctx=n_ctx, wtype=H.Q8_0)
+    else:
+        cfg = M.Config.llama2_7b(n_ctx=n_ctx, wtype=H.Q4_K, t_out=H.Q6_K, tensor_types={"attn_v": H.Q6_K, "ffn_down": H.Q6_K})
     cfg.n_layer = args.layers
     t0 = time.time()
-    tensors = M.synth_model(cfg, seed=1234)
+    # K-quant matrices: random well-formed blocks (this package has no K-quant quantizer; timing only)
+    tensors = M.synth_model(cfg, seed=1234, quantizer=M.random_k_blocks if args.model == "q4_k_m" else None)
     log("synthetic model: %.1f s, %.2f GB of weights streamed per token" % (time.time() - t0, cfg.weight_bytes() / 1e9))
     eng = M.Engine(cfg, tensors)
     rng = np.random.default_rng(4096)
@@ -113,8 +121,11 @@ def main():
         per_kernel[name] = eng.kernel_time_us(name, reps=4)
     d, F, V = cfg.n_embd, cfg.n_ff, cfg.n_vocab
     n_kv_end = pos + steps
-    alg = {"qkv": 3 * d * d * 18 // 32, "wo": d * d * 18 // 32, "gate_up": 2 * F * d * 18 // 32, "down": F * d * 18 // 32,
-           "head": V * d * 18 // 32, "scores": n_kv_end * d * 2, "pv": n_kv_end * d * 2}
+    tt = lambda n: cfg.tensor_types.get(n, cfg.wtype)
+    rs = H.row_size
+    alg = {"qkv": d * (rs(tt("attn_q"), d) + rs(tt("attn_k"), d) + rs(tt("attn_v"), d)), "wo": d * rs(tt("attn_output"), d),
+           "gate_up": F * (rs(tt("ffn_gate"), d) + rs(tt("ffn_up"), d)), "down": d * rs(tt("ffn_down"), F),
+           "head": V * rs(cfg.t_out, d), "scores": n_kv_end * d * 2, "pv": n_kv_end * d * 2}
     if eng.fuses_attention():           # qkv, scores and softmax + KQV are one launch, timed under "qkv"
         per_kernel["attention (qkv+scores+pv)"] = per_kernel.pop("qkv")
         alg["attention (qkv+scores+pv)"] = alg["qkv"] + alg["scores"] + alg["pv"]
@@ -125,7 +136,7 @@ def main():
     dom = "gate_up"
     # HBM bytes per launch of that kernel from profiler counters (FETCH_SIZE + WRITE_SIZE scaled by a copy
     # kernel of known size; profiles/decode_7b_q4_0_ctx4096_hbm_traffic.md): valid for this shape only
-    traffic = 51.18e6 if (cfg.n_embd, cfg.n_ff, cfg.wtype) == (4096, 11008, H.Q4_0) else None
+    traffic = 51.18e6 if (cfg.n_embd, cfg.n_ff, cfg.wtype, args.model) == (4096, 11008, H.Q4_0, "q4_0") else None
     achieved = alg[dom] / (per_kernel[dom] * 1e-6) / 1e9
     roofline = {"kernel": "wave_gemv_kernel<Q4_0, gate|up + SiLU>", "bound": "hbm", "achieved": round(achieved, 1), "peak": 8000.0,
                 "unit": "GB/s", "frac": round(achieved / 8000.0, 4), "traffic": traffic,
@@ -151,12 +162,14 @@ def main():
                "sample": "%d single-token passes of the same model at n_kv = %d.. (AVX2 port of Spy's host backend, OpenMP)" % (args.cpu_steps, fill + 1)}
         log("cpu baseline: %.3f tok/s on %d threads" % (cpu["value"], ncpu))
 
+    weights_desc = {"q4_0": "Q4_0 weights incl. head", "q8_0": "Q8_0 weights incl. head",
+                    "q4_k_m": "Q4_K weights with Q6_K attn_v / ffn_down / head (random blocks)"}[args.model]
     out = {
-        "metric": "decode tok/s + % HBM roofline, LLaMA-2-7B Q4_0 ctx 4096, 1xMI355X",
+        "metric": "decode tok/s + %% HBM roofline, LLaMA-2-7B %s ctx 4096, 1xMI355X" % {"q4_0": "Q4_0", "q8_0": "Q8_0", "q4_k_m": "Q4_K_M"}[args.model],
         "value": round(tok_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "int8 dot (Q4_0 x Q8_0), fp32 accumulate, fp16 KV", "data": "synthetic",
-        "config": {"workload": "LLaMA-2-7B shape (32 layers, d 4096, 32 heads x 128, FFN 11008, vocab 32000), Q4_0 weights incl. head, "
+        "dtype": "int8 dot (%s x Q8_0), fp32 accumulate, fp16 KV" % {"q4_0": "Q4_0", "q8_0": "Q8_0", "q4_k_m": "Q4_K / Q6_K"}[args.model], "data": "synthetic",
+        "config": {"workload": "LLaMA-2-7B shape (32 layers, d 4096, 32 heads x 128, FFN 11008, vocab 32000), %s, " % weights_desc +
                                "f16 KV cache prefilled to %d tokens (%s), greedy single-sequence decode" % (fill, args.prefill),
                    "n_layer": cfg.n_layer, "n_kv_first": pos + 1, "n_kv_last": pos + steps, "bytes_per_token": int(bytes_per_token)},
         "hbm_roofline_frac": round(frac, 4), "ms_per_step_hip_events": round(ev_ms, 4),

@@ -98,6 +98,25 @@ def synth_tensor(ttype, seed, name, n, std=0.02, outlier_every=0, outlier_mul=20
     return quantizer(x, ttype)
 
 
+def random_k_blocks(x, ttype):
+    """Q4_K / Q6_K blocks with random quants and small random scales for as many elements as x has:
+    well-formed weights for timing runs (the values do not approximate x)."""
+    n = len(x)
+    rng = np.random.default_rng(n * 31 + ttype)
+    nsb = n // 256
+    if ttype == H.Q4_K:
+        b = rng.integers(0, 256, (nsb, 144), dtype=np.uint8)
+        b[:, 0:2] = (rng.uniform(0.5, 1.5, nsb) * 2e-4).astype(np.float16).view(np.uint8).reshape(nsb, 2)
+        b[:, 2:4] = (rng.uniform(0.5, 1.5, nsb) * 1e-4).astype(np.float16).view(np.uint8).reshape(nsb, 2)
+    elif ttype == H.Q6_K:
+        b = rng.integers(0, 256, (nsb, 210), dtype=np.uint8)
+        b[:, 192:208] = rng.integers(1, 64, (nsb, 16), dtype=np.uint8)
+        b[:, 208:210] = (rng.uniform(0.5, 1.5, nsb) * 2e-5).astype(np.float16).view(np.uint8).reshape(nsb, 2)
+    else:
+        raise ValueError("not a K-quant type: %d" % ttype)
+    return b.reshape(-1)
+
+
 def synth_model(cfg, seed=1234, std=0.02, outlier_every=0, quantizer=None, norm_jitter=0.1):
     """Random-init weights of the LLaMA-2 architecture: matrices ~N(0, std) (12-term integer
     approximation, bit-reproducible), norm weights 1 + N(0, norm_jitter), quantized with the GGUF
