@@ -68,7 +68,7 @@ static int launch_wave(spy_hip_llama *m, hipStream_t st, const fused_args &a) {
 }
 // rows (head) and row pairs (gate|up) per wave: bounded by the row registers, PAIR_DW dwords per row
 template <int WT> struct wave_rows {
-    static constexpr int HEAD = WT == SPY_HIP_Q4_0 ? 8 : (WT == SPY_HIP_Q4_K ? 6 : (WT == SPY_HIP_Q8_0 ? 4 : 3));
+    static constexpr int HEAD = WT == SPY_HIP_Q4_0 ? 8 : (WT == SPY_HIP_Q4_K ? 6 : 4);
     static constexpr int GATEUP = (WT == SPY_HIP_Q4_0 || WT == SPY_HIP_Q4_K) ? 3 : 2;
 };
 static inline int layer_type(const spy_hip_llama *m, int t) { return t ? t : m->desc.wtype; }

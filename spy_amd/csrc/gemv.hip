@@ -126,7 +126,7 @@ __global__ __launch_bounds__(WROW_THREADS) void wave_row_kernel(gemv_args a, int
 
 template <int WT, int NITK>
 static int launch_wave_row_nitk(hipStream_t st, const gemv_args &a, int T) {
-    constexpr int NRMAX = (WT == SPY_HIP_Q4_0 || WT == SPY_HIP_Q4_K) ? 6 : 3;      // rows per wave: row registers = NR * NITK * PAIR_DW
+    constexpr int NRMAX = (WT == SPY_HIP_Q4_0 || WT == SPY_HIP_Q4_K) ? 6 : 4;      // rows per wave: row registers = NR * NITK * PAIR_DW
     constexpr int NR = NITK == 1 ? NRMAX : 1;
     static int num_cu = 0;
     if (!num_cu) { int dev = 0; hipDeviceProp_t prop; num_cu = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) ? prop.multiProcessorCount : 256; }

@@ -34,10 +34,10 @@ template <> struct wt_traits<SPY_HIP_Q4_0> { static constexpr int BLK = 18, PAIR
 template <> struct wt_traits<SPY_HIP_Q8_0> { static constexpr int BLK = 34, PAIR_DW = 17; };
 // K-quants (64 lanes per row only): a lane's unit is a quarter super-block = 64 elements, the same
 // span as a block pair.  Q4_K: the 16-byte header {d, dmin, scales[12]} + the 32 nibble bytes of sub-blocks
-// 2j, 2j+1.  Q6_K (super-blocks only 2-byte aligned): three 16-byte chunks (ql, ql + 32, qh) as 5 raw
-// dwords each, 8 scale bytes as 3 raw dwords, d, and the byte shift of the super-block (0 or 16 bits).
+// 2j, 2j+1.  Q6_K (super-blocks only 2-byte aligned; the hardware takes unaligned vector loads): three
+// 16-byte chunks (ql, ql + 32, qh), 8 scale bytes and d.
 template <> struct wt_traits<SPY_HIP_Q4_K> { static constexpr int PAIR_DW = 12; };
-template <> struct wt_traits<SPY_HIP_Q6_K> { static constexpr int PAIR_DW = 20; };
+template <> struct wt_traits<SPY_HIP_Q6_K> { static constexpr int PAIR_DW = 15; };
 #define GEMV_NIT_MAX 4        // block pairs per lane per row tile: 1..4 (exact value is a template parameter)
 
 template <int CTRL> static __device__ __forceinline__ float dpp_add(float v) {
@@ -251,22 +251,19 @@ static __device__ __forceinline__ void load_tile(wtile<WT, NIT> &t, const uint8_
             t.w[it][8] = q1.x; t.w[it][9] = q1.y; t.w[it][10] = q1.z; t.w[it][11] = q1.w;
         } else if constexpr (WT == SPY_HIP_Q6_K) {
             static_assert(WT != SPY_HIP_Q6_K || LPR == 64, "K-quant tiles use 64 lanes per row");
-            // lane (n = half of the super-block, e = 16-element slice): ql[64n + 16e ..], ql[64n + 32 + 16e ..], qh[32n + 16e ..],
-            // scales[8n ..]; every chunk read as aligned dwords around it (the last dword index is clamped
-            // when the chunk is aligned, so nothing beyond the super-block is touched)
+            // lane (n = half of the super-block, e = 16-element slice): ql[64n + 16e ..], ql[64n + 32 + 16e ..], qh[32n + 16e ..], scales[8n ..]
             const int j = p & 3, n = j >> 1, e = j & 1;
             const uint8_t *sb = rowp + (size_t)(p >> 2) * 210;
-            const uint32_t sh = ((uint32_t)(uintptr_t)sb & 2u) ? 16u : 0u;
-            const uint32_t *base = (const uint32_t *)((uintptr_t)sb & ~(uintptr_t)3);        // sb - (0 | 2) bytes
-            const int last4 = sh ? 4 : 3, last2 = sh ? 2 : 1;
-            const uint32_t *ca = base + (64 * n + 16 * e) / 4, *cb = base + (64 * n + 32 + 16 * e) / 4, *ch = base + (128 + 32 * n + 16 * e) / 4;
-            const uint32_t *cs = base + (192 + 8 * n) / 4;
-#pragma unroll
-            for (int i = 0; i < 4; i++) { t.w[it][i] = ca[i]; t.w[it][5 + i] = cb[i]; t.w[it][10 + i] = ch[i]; }
-            t.w[it][4] = ca[last4]; t.w[it][9] = cb[last4]; t.w[it][14] = ch[last4];
-            t.w[it][15] = cs[0]; t.w[it][16] = cs[1]; t.w[it][17] = cs[last2];
-            t.w[it][18] = *(const uint16_t *)(sb + 208);
-            t.w[it][19] = sh;
+            uint4 ca, cb, ch; uint2 cs;
+            __builtin_memcpy(&ca, __builtin_assume_aligned(sb + 64 * n + 16 * e, 2), 16);
+            __builtin_memcpy(&cb, __builtin_assume_aligned(sb + 64 * n + 32 + 16 * e, 2), 16);
+            __builtin_memcpy(&ch, __builtin_assume_aligned(sb + 128 + 32 * n + 16 * e, 2), 16);
+            __builtin_memcpy(&cs, __builtin_assume_aligned(sb + 192 + 8 * n, 2), 8);
+            t.w[it][0] = ca.x; t.w[it][1] = ca.y; t.w[it][2] = ca.z; t.w[it][3] = ca.w;
+            t.w[it][4] = cb.x; t.w[it][5] = cb.y; t.w[it][6] = cb.z; t.w[it][7] = cb.w;
+            t.w[it][8] = ch.x; t.w[it][9] = ch.y; t.w[it][10] = ch.z; t.w[it][11] = ch.w;
+            t.w[it][12] = cs.x; t.w[it][13] = cs.y;
+            t.w[it][14] = *(const uint16_t *)(sb + 208);
         } else {
             const uint32_t *wp = (const uint32_t *)rowp + (size_t)p * DW;
 #pragma unroll
@@ -337,17 +334,10 @@ static __device__ __forceinline__ float dot_pair(const uint32_t *w, const int4 x
     } else if constexpr (WT == SPY_HIP_Q6_K) {
         // lane (n, e): elements l + 32 m, l in [16e, 16e + 16), m = 0..3 of half n: 6-bit quants from the low /
         // high nibbles of ql / ql + 32 and bit pairs 2m of qh, minus 32; scale = d * scales[8n + e + 2m]
-        const uint32_t sh = w[19];
-        uint32_t qa[4], qb[4], qh[4];
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            qa[i] = __builtin_amdgcn_alignbit(w[i + 1], w[i], sh);
-            qb[i] = __builtin_amdgcn_alignbit(w[6 + i], w[5 + i], sh);
-            qh[i] = __builtin_amdgcn_alignbit(w[11 + i], w[10 + i], sh);
-        }
-        const uint32_t s0 = __builtin_amdgcn_alignbit(w[16], w[15], sh), s1 = __builtin_amdgcn_alignbit(w[17], w[16], sh);
+        const uint32_t *qa = w, *qb = w + 4, *qh = w + 8;
+        const uint32_t s0 = w[12], s1 = w[13];
         const int e = p & 1;
-        const float d = h2f((uint16_t)(w[18] & 0xFFFFu));
+        const float d = h2f((uint16_t)(w[14] & 0xFFFFu));
         int isum[4] = {0, 0, 0, 0};
         const int xm[4][4] = {{x0.x, x0.y, x0.z, x0.w}, {x1.x, x1.y, x1.z, x1.w}, {x2.x, x2.y, x2.z, x2.w}, {x3.x, x3.y, x3.z, x3.w}};
 #pragma unroll
