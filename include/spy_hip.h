@@ -124,7 +124,8 @@ int spy_hip_gemv_q8_0act(void *stream, int wtype, const void *w, const void *xq,
                          int64_t M, int64_t K, int64_t T, int64_t dst_stride);
 /* The same dots for many activation rows at once (prompt passes) on the matrix cores: int8 MFMA,
  * one 32-element block per instruction, exact int32 block dots scaled by h2f(d_w)*h2f(d_x) and
- * accumulated in fp32.  Q4_0 / Q8_0 weights, K % 64 == 0; operands as for spy_hip_gemv_q8_0act. */
+ * accumulated in fp32 (K-quants: per sub-block / 16-element group).  K % 64 == 0 (K-quants: K % 256 == 0);
+ * operands as for spy_hip_gemv_q8_0act. */
 int spy_hip_gemm_q8_0act(void *stream, int wtype, const void *w, const void *xq, float *dst,
                          int64_t M, int64_t K, int64_t T, int64_t dst_stride);
 /* the int32 dot of every 32-element block (Q4_0, Q8_0, Q4_K sub-blocks) or 16-element

@@ -148,15 +148,190 @@ __global__ __launch_bounds__(256, 2) void gemm_q8act_kernel(const uint8_t *__res
         }
 }
 
+// ---- K-quant weights ---------------------------------------------------------------------------------
+// Same tiling.  A stage is a quarter super-block (64 elements), a thread unpacks one 32-element half of it:
+//   Q4_K: sub-block a = 2j + half of the super-block: nibbles 0..15 as int8, scale d*sc and minimum dmin*m;
+//         value = d*sc*q - dmin*m, so the tile gets  dx * (d*sc * I - dmin*m * sum(q_x))  per block, with
+//         dx * sum(q_x) prepared once per activation block.
+//   Q6_K: 32 elements l + 32 m (m = 2 (j & 1) + half) of half n = j >> 1: (q - 32) as int8; they span TWO
+//         16-element scale groups, which the 32x32x32 MFMA keeps apart when the right operand is zeroed in
+//         one lane half (lanes 0..31 carry k = 0..15, lanes 32..63 k = 16..31): two MFMAs, I_lo and I_hi,
+//         combined as integers sc_lo * I_lo + sc_hi * I_hi, then scaled by dx * d.
+static __device__ __forceinline__ void q4k_sc_m(const uint32_t h1, const uint32_t h2, const uint32_t h3, int a, int &sc, int &mn) {
+    auto byte = [&](int k) -> uint32_t { const uint32_t w = k < 4 ? h1 : (k < 8 ? h2 : h3); return (w >> (8 * (k & 3))) & 0xFFu; };
+    if (a < 4) { sc = byte(a) & 63; mn = byte(a + 4) & 63; }
+    else { sc = (byte(a + 4) & 0x0F) | ((byte(a - 4) >> 6) << 4); mn = (byte(a + 4) >> 4) | ((byte(a) >> 6) << 4); }
+}
+
+template <int WT>
+__global__ __launch_bounds__(256, 2) void gemm_kq_kernel(const uint8_t *__restrict__ W, const uint8_t *__restrict__ xq, float *__restrict__ dst,
+                                                         int M, int K, int T, int64_t dst_stride) {
+    constexpr bool Q4K = (WT == SPY_HIP_Q4_K);
+    constexpr int RAW = Q4K ? 12 : 18;
+    __shared__ __attribute__((aligned(16))) uint8_t sA[2][GEMM_TILE * GEMM_ROWB];
+    __shared__ __attribute__((aligned(16))) uint8_t sB[2][GEMM_TILE * GEMM_ROWB];
+    __shared__ __attribute__((aligned(16))) float sAd[2][2][GEMM_TILE];      // Q4_K: d*sc          Q6_K: d
+    __shared__ __attribute__((aligned(16))) int sAm[2][2][GEMM_TILE];        // Q4_K: bits of dmin*m Q6_K: sc_lo | sc_hi << 16
+    __shared__ __attribute__((aligned(16))) float sBd[2][2][GEMM_TILE];      // dx
+    __shared__ __attribute__((aligned(16))) float sBs[2][2][GEMM_TILE];      // dx * sum(q_x)
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
+    const int m0 = blockIdx.x * GEMM_TILE, t0 = blockIdx.y * GEMM_TILE;
+    const int nstage = K / 64;
+    const size_t RBw = (size_t)spy_row_size(WT, K), RBx = (size_t)(K / 32) * 34;
+    const int lrow = tid & 127, half = tid >> 7;
+    const uint8_t *gA = W + (size_t)min(m0 + lrow, M - 1) * RBw;
+    const uint32_t *gB = (const uint32_t *)(xq + (size_t)min(t0 + lrow, T - 1) * RBx) + half * 8;
+    uint32_t rawA[RAW], rawB[9];
+    auto gload = [&](int s) {
+        const int sbi = s >> 2, j = s & 3;
+        if constexpr (Q4K) {
+            const uint8_t *sb = gA + (size_t)sbi * 144;
+            const uint4 hdr = *(const uint4 *)sb, q0 = *(const uint4 *)(sb + 16 + 32 * j), q1 = *(const uint4 *)(sb + 32 + 32 * j);
+            rawA[0] = hdr.x; rawA[1] = hdr.y; rawA[2] = hdr.z; rawA[3] = hdr.w;
+            rawA[4] = q0.x; rawA[5] = q0.y; rawA[6] = q0.z; rawA[7] = q0.w; rawA[8] = q1.x; rawA[9] = q1.y; rawA[10] = q1.z; rawA[11] = q1.w;
+        } else {
+            const int n = j >> 1, m = 2 * (j & 1) + half;
+            const uint8_t *sb = gA + (size_t)sbi * 210;
+            uint4 l0, l1, h0, h1;
+            __builtin_memcpy(&l0, __builtin_assume_aligned(sb + 64 * n + 32 * (m & 1), 2), 16);
+            __builtin_memcpy(&l1, __builtin_assume_aligned(sb + 64 * n + 32 * (m & 1) + 16, 2), 16);
+            __builtin_memcpy(&h0, __builtin_assume_aligned(sb + 128 + 32 * n, 2), 16);
+            __builtin_memcpy(&h1, __builtin_assume_aligned(sb + 128 + 32 * n + 16, 2), 16);
+            rawA[0] = l0.x; rawA[1] = l0.y; rawA[2] = l0.z; rawA[3] = l0.w; rawA[4] = l1.x; rawA[5] = l1.y; rawA[6] = l1.z; rawA[7] = l1.w;
+            rawA[8] = h0.x; rawA[9] = h0.y; rawA[10] = h0.z; rawA[11] = h0.w; rawA[12] = h1.x; rawA[13] = h1.y; rawA[14] = h1.z; rawA[15] = h1.w;
+            rawA[16] = *(const uint16_t *)(sb + 192 + 8 * n + 2 * m);
+            rawA[17] = *(const uint16_t *)(sb + 208);
+        }
+#pragma unroll
+        for (int i = 0; i < 9; i++) rawB[i] = gB[(size_t)s * 17 + i];
+    };
+    auto unpack = [&](int b, int s) {
+        const int j = s & 3;
+        uint32_t q[8];
+        if constexpr (Q4K) {
+            int sc, mn;
+            q4k_sc_m(rawA[1], rawA[2], rawA[3], 2 * j + half, sc, mn);
+#pragma unroll
+            for (int i = 0; i < 8; i++) q[i] = half ? (rawA[4 + i] >> 4) & 0x0F0F0F0Fu : rawA[4 + i] & 0x0F0F0F0Fu;
+            sAd[b][half][lrow] = h2f((uint16_t)(rawA[0] & 0xFFFFu)) * (float)sc;
+            sAm[b][half][lrow] = __float_as_int(h2f((uint16_t)(rawA[0] >> 16)) * (float)mn);
+        } else {
+            const int m = 2 * (j & 1) + half;
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const uint32_t lo = (m & 2) ? (rawA[i] >> 4) & 0x0F0F0F0Fu : rawA[i] & 0x0F0F0F0Fu;
+                const uint32_t hi = (rawA[8 + i] >> (2 * m)) & 0x03030303u;
+                q[i] = (lo | (hi << 4)) + 0x60606060u ^ 0x80808080u;
+            }
+            sAd[b][half][lrow] = h2f((uint16_t)(rawA[17] & 0xFFFFu));
+            sAm[b][half][lrow] = (int)(uint16_t)(int16_t)(int8_t)(rawA[16] & 0xFFu) | ((int)(int8_t)((rawA[16] >> 8) & 0xFFu) << 16);
+        }
+        uint4 *ra = (uint4 *)(sA[b] + lrow * GEMM_ROWB + half * 32);
+        ra[0] = make_uint4(q[0], q[1], q[2], q[3]); ra[1] = make_uint4(q[4], q[5], q[6], q[7]);
+        // activations: {d, qs[32]} (quant.h:139-142)
+        const float dx = h2f((uint16_t)(half ? rawB[0] >> 16 : rawB[0] & 0xFFFFu));
+        int bsum = 0;
+#pragma unroll
+        for (int i = 0; i < 8; i++) { q[i] = half ? rawB[i + 1] : __builtin_amdgcn_alignbit(rawB[i + 1], rawB[i], 16); bsum = __builtin_amdgcn_sdot4((int)q[i], 0x01010101, bsum, false); }
+        uint4 *rb = (uint4 *)(sB[b] + lrow * GEMM_ROWB + half * 32);
+        rb[0] = make_uint4(q[0], q[1], q[2], q[3]); rb[1] = make_uint4(q[4], q[5], q[6], q[7]);
+        sBd[b][half][lrow] = dx;
+        sBs[b][half][lrow] = dx * (float)bsum;
+    };
+
+    float acc[2][2][16];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+
+    gload(0);
+    unpack(0, 0);
+    __syncthreads();
+    for (int s = 0; s < nstage; s++) {
+        const int b = s & 1;
+        gload(min(s + 1, nstage - 1));
+#pragma unroll 1
+        for (int blk = 0; blk < 2; blk++) {
+            v4i fa[2], fb[2];
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                fa[i] = *(const v4i *)(sA[b] + (wm * 64 + i * 32 + (lane & 31)) * GEMM_ROWB + blk * 32 + (lane >> 5) * 16);
+                fb[i] = *(const v4i *)(sB[b] + (wn * 64 + i * 32 + (lane & 31)) * GEMM_ROWB + blk * 32 + (lane >> 5) * 16);
+            }
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                float dw[16]; int am[16];
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const float4 v = *(const float4 *)&sAd[b][blk][wm * 64 + i * 32 + g * 8 + (lane >> 5) * 4];
+                    const int4 u = *(const int4 *)&sAm[b][blk][wm * 64 + i * 32 + g * 8 + (lane >> 5) * 4];
+                    dw[4 * g] = v.x; dw[4 * g + 1] = v.y; dw[4 * g + 2] = v.z; dw[4 * g + 3] = v.w;
+                    am[4 * g] = u.x; am[4 * g + 1] = u.y; am[4 * g + 2] = u.z; am[4 * g + 3] = u.w;
+                }
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    const int col = wn * 64 + j * 32 + (lane & 31);
+                    const float dx = sBd[b][blk][col];
+                    v16i z = {0};
+                    if constexpr (Q4K) {
+                        const float dxs = sBs[b][blk][col];
+                        const v16i I = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], z, 0, 0, 0);
+#pragma unroll
+                        for (int r = 0; r < 16; r++) {
+                            acc[i][j][r] = fmaf(dw[r] * dx, (float)I[r], acc[i][j][r]);
+                            acc[i][j][r] = fmaf(-__int_as_float(am[r]), dxs, acc[i][j][r]);
+                        }
+                    } else {
+                        const v4i zero4 = {0, 0, 0, 0};
+                        const v4i blo = lane < 32 ? fb[j] : zero4, bhi = lane < 32 ? zero4 : fb[j];
+                        const v16i Ilo = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], blo, z, 0, 0, 0);
+                        const v16i Ihi = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], bhi, z, 0, 0, 0);
+#pragma unroll
+                        for (int r = 0; r < 16; r++) {
+                            const int sv = (int)(int16_t)(am[r] & 0xFFFF) * Ilo[r] + (am[r] >> 16) * Ihi[r];
+                            acc[i][j][r] = fmaf(dw[r] * dx, (float)sv, acc[i][j][r]);
+                        }
+                    }
+                }
+            }
+        }
+        if (s + 1 < nstage) unpack(b ^ 1, s + 1);
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int t = t0 + wn * 64 + j * 32 + (lane & 31);
+            if (t < T) {
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const int m = m0 + wm * 64 + i * 32 + g * 8 + (lane >> 5) * 4;
+                    float *o = dst + (size_t)t * dst_stride + m;
+                    if (m + 3 < M && (((uintptr_t)o) & 15) == 0) *(float4 *)o = make_float4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
+                    else {
+#pragma unroll
+                        for (int e = 0; e < 4; e++) if (m + e < M) o[e] = acc[i][j][4 * g + e];
+                    }
+                }
+            }
+        }
+}
+
 extern "C" int spy_hip_gemm_q8_0act(void *stream, int wtype, const void *w_dev, const void *xq_dev, float *dst_dev,
                                     int64_t M, int64_t K, int64_t T, int64_t dst_stride) {
     SPY_CHECK_ARG(w_dev && xq_dev && dst_dev && M > 0 && K > 0 && T > 0 && dst_stride >= M);
-    SPY_CHECK_ARG(K % 64 == 0);
+    SPY_CHECK_ARG(K % 64 == 0 && ((wtype != SPY_HIP_Q4_K && wtype != SPY_HIP_Q6_K) || K % 256 == 0));
     SPY_CHECK_ARG((M + GEMM_TILE - 1) / GEMM_TILE <= 0x7fffffff && (T + GEMM_TILE - 1) / GEMM_TILE <= 65535);
     const dim3 grid((unsigned)((M + GEMM_TILE - 1) / GEMM_TILE), (unsigned)((T + GEMM_TILE - 1) / GEMM_TILE));
     hipStream_t st = (hipStream_t)stream;
     if (wtype == SPY_HIP_Q4_0) gemm_q8act_kernel<SPY_HIP_Q4_0><<<grid, dim3(256), 0, st>>>((const uint8_t *)w_dev, (const uint8_t *)xq_dev, dst_dev, (int)M, (int)K, (int)T, dst_stride);
     else if (wtype == SPY_HIP_Q8_0) gemm_q8act_kernel<SPY_HIP_Q8_0><<<grid, dim3(256), 0, st>>>((const uint8_t *)w_dev, (const uint8_t *)xq_dev, dst_dev, (int)M, (int)K, (int)T, dst_stride);
+    else if (wtype == SPY_HIP_Q4_K) gemm_kq_kernel<SPY_HIP_Q4_K><<<grid, dim3(256), 0, st>>>((const uint8_t *)w_dev, (const uint8_t *)xq_dev, dst_dev, (int)M, (int)K, (int)T, dst_stride);
+    else if (wtype == SPY_HIP_Q6_K) gemm_kq_kernel<SPY_HIP_Q6_K><<<grid, dim3(256), 0, st>>>((const uint8_t *)w_dev, (const uint8_t *)xq_dev, dst_dev, (int)M, (int)K, (int)T, dst_stride);
     else return SPY_HIP_EUNSUPPORTED;
     return SPY_LAUNCH_RC();
 }

@@ -448,7 +448,7 @@ extern "C" int spy_hip_op_matmul(void *stream, const spy_hip_tensor *w, const sp
                 const uint8_t *xp = xm + ((i3 * ne12 + i2) * ne11) * mid_row;
                 float *dp = (float *)((uint8_t *)dst->data + i2 * dst->nb[2] + i3 * dst->nb[3]);
                 // many activation rows: matrix cores; few: the bandwidth-bound row kernels
-                const bool mfma = ne11 >= 16 && (t0 == SPY_HIP_Q4_0 || t0 == SPY_HIP_Q8_0) && ne00 % 64 == 0;
+                const bool mfma = ne11 >= 16 && ne00 % 64 == 0;
                 int rc = mfma ? spy_hip_gemm_q8_0act(stream, t0, wp, xp, dp, ne01, ne00, ne11, dst->nb[1] / 4)
                               : spy_hip_gemv_q8_0act(stream, t0, wp, xp, dp, nullptr, ne01, ne00, ne11, dst->nb[1] / 4);
                 if (rc) return rc;

@@ -33,6 +33,27 @@ def test_gemm_q8_0act_matches_oracle(hip, oracle, wtype, M, K, T):
     assert_close(dout.download(np.float32).reshape(T, M), want, "gemm type %d %dx%d T=%d" % (wtype, M, K, T))
 
 
+@pytest.mark.parametrize("wtype", [O.Q4_K, O.Q6_K])
+@pytest.mark.parametrize("M,K,T", [(128, 4096, 128), (256, 256, 16), (200, 11008, 77), (130, 512, 129), (4096, 4096, 256)])
+def test_gemm_k_quants_match_oracle(hip, oracle, wtype, M, K, T):
+    """Super-block weights: every sub-block scale / minimum (Q4_K) and both 16-element groups of a
+    32-element MFMA block (Q6_K) take part; weights with offsets and outliers so that minima and the
+    6-bit scale fields above index 3 are not trivial."""
+    from tests.gpu_util import dev, dev_empty, call, assert_close
+    rng = np.random.default_rng(wtype * 977 + M + K + T)
+    wf = (rng.standard_normal((M, K)) * 0.02).astype(np.float32)
+    wf += (rng.standard_normal((M, K // 32, 1)) * 0.03).astype(np.float32).repeat(32, 2).reshape(M, K)
+    wf[rng.random((M, K)) < 0.01] *= 8.0
+    w = O.quantize(oracle, wf, wtype)
+    x = rng.standard_normal((T, K)).astype(np.float32)
+    x[:, : K // 2] *= 3.0
+    want = O.matmul(oracle, w, wtype, M, K, x, nthread=8)
+    xq = O.quantize(oracle, x, O.Q8_0)
+    dw, dxq, dout = dev(w), dev(xq), dev_empty(T * M * 4, 0xFF)
+    call(hip.load().spy_hip_gemm_q8_0act, None, wtype, dw.ptr, dxq.ptr, dout.ptr, M, K, T, M)
+    assert_close(dout.download(np.float32).reshape(T, M), want, "gemm type %d %dx%d T=%d" % (wtype, M, K, T))
+
+
 def test_gemm_integer_scales_is_exact(hip, oracle):
     """With power-of-two scales and small integers every product and sum is exact in fp32: the GEMM
     must then equal the integer matrix product bit for bit (pins the MFMA operand / result layout)."""
