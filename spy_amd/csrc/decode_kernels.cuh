@@ -302,7 +302,12 @@ __global__ __launch_bounds__(WGV_THREADS) void wave_gemv_kernel(fused_args a) {
 // All of a launch's workgroups must be resident (grid <= compute units, one 1024-thread workgroup each).
 #define ATL_RS 10                 // groups of 4 keys per wave (n_ctx <= 128 * 4 * ATL_RS)
 #define ATL_RV 10                 // 128-bit pieces per lane of a V^T row (n_ctx <= 512 * ATL_RV)
-#define ATL_DEPTH 3
+#ifndef ATL_DEPTH_K
+#define ATL_DEPTH_K 3               // key groups / V^T pieces per wave requested ahead of their use
+#endif
+#ifndef ATL_DEPTH_V
+#define ATL_DEPTH_V 3
+#endif
 struct attn_layer_args {
     const uint8_t *wq, *wk, *wv;
     const float *x_in, *normw; float eps;
@@ -312,7 +317,15 @@ struct attn_layer_args {
     uint32_t *sync;               // per head 3 x 32 words: arrivals of barrier 1, of barrier 2, launches so far
     int d, n_head, n_ctx;
     float scale; uint32_t spin_limit;
+#ifdef ATL_STAMPS
+    long long *dbg;               // measurement builds only: wall-clock stamps (10 ns units) of workgroups 0 and 100
+#endif
 };
+#ifdef ATL_STAMPS
+#define ATL_STAMP(i) do { if (a.dbg && tid == 0 && (blockIdx.x == 0 || blockIdx.x == 100)) a.dbg[(blockIdx.x ? 64 : 0) + (i)] = wall_clock64(); } while (0)
+#else
+#define ATL_STAMP(i) do { } while (0)
+#endif
 
 template <int WT, int WTV>        // types of wq / wk and of wv
 __global__ __launch_bounds__(WGV_THREADS) void attn_layer_kernel(attn_layer_args a) {
@@ -325,7 +338,10 @@ __global__ __launch_bounds__(WGV_THREADS) void attn_layer_kernel(attn_layer_args
     const size_t RB = (size_t)spy_row_size(WT, d);
     const int pos = a.st->pos, n_kv = pos + 1;
     uint32_t *sync = a.sync + (size_t)h * 96;
-    const uint32_t target = 8u * (ldc(sync + 64) + 1u);
+    // the launch count was written by the previous launch: an ordinary (scalar) load sees it, and stays out of
+    // the vector-memory queue in which the first activation loads would otherwise wait behind it
+    const uint32_t target = 8u * (sync[64] + 1u);
+    ATL_STAMP(0);
 
     int8_t *s_q = (int8_t *)smem;
     int2 *s_meta = (int2 *)(smem + staged_q_bytes(d));
@@ -370,8 +386,10 @@ __global__ __launch_bounds__(WGV_THREADS) void attn_layer_kernel(attn_layer_args
         float acc = 0.0f;
         if (tid < d / 4) { acc = fmaf(xv.x, xv.x, acc); acc = fmaf(xv.y, xv.y, acc); acc = fmaf(xv.z, xv.z, acc); acc = fmaf(xv.w, xv.w, acc); }
         acc = group_sum<64>(acc);
+        ATL_STAMP(9);
         if (lane == 0) s_red[wave] = acc;
         __syncthreads();
+        ATL_STAMP(10);
         const float sum = (((s_red[0] + s_red[1]) + (s_red[2] + s_red[3])) + ((s_red[4] + s_red[5]) + (s_red[6] + s_red[7]))) +
                           (((s_red[8] + s_red[9]) + (s_red[10] + s_red[11])) + ((s_red[12] + s_red[13]) + (s_red[14] + s_red[15])));
         const float scale = 1.0f / sqrtf(sum / (float)d + a.eps);
@@ -385,6 +403,7 @@ __global__ __launch_bounds__(WGV_THREADS) void attn_layer_kernel(attn_layer_args
         }
         __syncthreads();
     }
+    ATL_STAMP(1);
     uint4 kb[ATL_RS];
     auto fetch_k = [&](int k) {                                      // keys 4u..4u+3 of head h, u = w + 128 k
         const int tok = min(4 * (w + 128 * k) + (lane >> 4), n_kv - 1);
@@ -409,9 +428,10 @@ __global__ __launch_bounds__(WGV_THREADS) void attn_layer_kernel(attn_layer_args
         }
         if (wave != 0) {
 #pragma unroll
-            for (int k = 0; k < ATL_DEPTH; k++) fetch_k(k);
+            for (int k = 0; k < ATL_DEPTH_K; k++) fetch_k(k);
         }
     }
+    ATL_STAMP(2);
     if (!publish_and_sync(sync, [&]() {
             if (lane < WGV_WAVES) {
                 const int ww = g * WGV_WAVES + lane, pp = ww & 63;
@@ -421,6 +441,7 @@ __global__ __launch_bounds__(WGV_THREADS) void attn_layer_kernel(attn_layer_args
                 stc(a.vc + (size_t)(h * 128 + ww) * n_ctx + pos, (uint16_t)__float_as_uint(s_out[lane * 2 + 1]));   // VCache_cpy: [d][C] column pos
             }
         })) return;
+    ATL_STAMP(3);
 
     // ================= B: t = (K.q) * scale for head h ================================================
     const uint16_t *vrow = a.vc + (size_t)(h * 128 + w) * n_ctx;
@@ -431,14 +452,14 @@ __global__ __launch_bounds__(WGV_THREADS) void attn_layer_kernel(attn_layer_args
         const uint32_t qw[4] = {ldc(qp), ldc(qp + 1), ldc(qp + 2), ldc(qp + 3)};
         if (wave == 0) {
 #pragma unroll
-            for (int k = 0; k < ATL_DEPTH; k++) fetch_k(k);
+            for (int k = 0; k < ATL_DEPTH_K; k++) fetch_k(k);
         }
         float qf[8];
 #pragma unroll
         for (int j = 0; j < 4; j++) { qf[2 * j] = h2f((uint16_t)(qw[j] & 0xFFFFu)); qf[2 * j + 1] = h2f((uint16_t)(qw[j] >> 16)); }
 #pragma unroll
         for (int k = 0; k < ATL_RS; k++) {
-            if (k + ATL_DEPTH < ATL_RS) fetch_k(k + ATL_DEPTH);
+            if (k + ATL_DEPTH_K < ATL_RS) fetch_k(k + ATL_DEPTH_K);
             const int tok = 4 * (w + 128 * k) + (lane >> 4);
             uint4 kv = kb[k];
             if (tok == pos) {                                        // written in step A by another workgroup: read it coherently
@@ -457,9 +478,10 @@ __global__ __launch_bounds__(WGV_THREADS) void attn_layer_kernel(attn_layer_args
         }
         if (wave != 0) {
 #pragma unroll
-            for (int i = 0; i < ATL_DEPTH; i++) fetch_v(i);
+            for (int i = 0; i < ATL_DEPTH_V; i++) fetch_v(i);
         }
     }
+    ATL_STAMP(4);
     if (!publish_and_sync(sync + 32, [&]() {
             for (int idx = lane; idx < WGV_WAVES * 4 * ATL_RS; idx += 64) {
                 const int wv_ = idx / (4 * ATL_RS), r = idx - wv_ * (4 * ATL_RS);
@@ -467,6 +489,7 @@ __global__ __launch_bounds__(WGV_THREADS) void attn_layer_kernel(attn_layer_args
                 if (tok < n_kv) stc(a.scores + (size_t)h * n_ctx + tok, s_out[idx]);
             }
         })) return;
+    ATL_STAMP(5);
     if (g == 0 && tid == 0) sync[64] = target / 8u;                  // every workgroup of the head has read the old count
 
     // ================= C: softmax of the head's scores, KQV rows 16 g .. 16 g + 15 ====================
@@ -479,11 +502,12 @@ __global__ __launch_bounds__(WGV_THREADS) void attn_layer_kernel(attn_layer_args
         for (int j = tid; j < n_kv; j += WGV_THREADS) { const float tt = ldc(srow + j); s_t[j] = tt; mx = fmaxf(mx, tt); }
         if (wave == 0) {
 #pragma unroll
-            for (int i = 0; i < ATL_DEPTH; i++) fetch_v(i);
+            for (int i = 0; i < ATL_DEPTH_V; i++) fetch_v(i);
         }
         mx = wave_max(mx);
         if (lane == 0) s_red[wave] = mx;
         __syncthreads();
+        ATL_STAMP(6);
         mx = s_red[0];
 #pragma unroll
         for (int i = 1; i < WGV_WAVES; i++) mx = fmaxf(mx, s_red[i]);
@@ -499,10 +523,11 @@ __global__ __launch_bounds__(WGV_THREADS) void attn_layer_kernel(attn_layer_args
         const float inv = 1.0f / sum;
         for (int j = tid; j < n_pad; j += WGV_THREADS) s_p[j] = j < n_kv ? f2h(s_t[j] * inv) : (uint16_t)0;
         __syncthreads();
+        ATL_STAMP(7);
         float acc = 0.0f;
 #pragma unroll
         for (int i = 0; i < ATL_RV; i++) {
-            if (i + ATL_DEPTH < ATL_RV) fetch_v(i + ATL_DEPTH);
+            if (i + ATL_DEPTH_V < ATL_RV) fetch_v(i + ATL_DEPTH_V);
             const int pc = i * 64 + lane;
             if (pc * 8 < n_kv) {
                 const uint4 pp = *(const uint4 *)(s_p + pc * 8);
@@ -517,6 +542,7 @@ __global__ __launch_bounds__(WGV_THREADS) void attn_layer_kernel(attn_layer_args
         }
         acc = wave_total_lane63(acc);
         if (lane == 63) a.attn_out[h * 128 + w] = acc;
+        ATL_STAMP(8);
     }
 }
 

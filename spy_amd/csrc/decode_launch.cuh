@@ -108,6 +108,9 @@ static int launch_attn_layer_tv(spy_hip_llama *m, hipStream_t st, int il, bool p
     a.d = c.n_embd; a.n_head = c.n_head; a.n_ctx = c.n_ctx;
     a.scale = 1.0f / sqrtf((float)m->hd);                   // SoftmaxParam::scale (attention.cpp:113)
     a.spin_limit = 400000;
+#ifdef ATL_STAMPS
+    a.dbg = m->mega_dbg;
+#endif
     kern<<<dim3((unsigned)(c.n_head * 8)), dim3(WGV_THREADS), lds, st>>>(a);
     return SPY_LAUNCH_RC();
 }
