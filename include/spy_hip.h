@@ -134,6 +134,14 @@ int spy_hip_gemm_q8_0act(void *stream, int wtype, const void *w, const void *xq,
  * the last M slots receive the float results and are scratch. */
 int spy_hip_block_dots(void *stream, int wtype, const void *w, const void *xq, int32_t *out, int64_t M, int64_t K);
 
+/* ---- measured ceilings of the part (no counterpart in the reference; they back the roofline denominators
+ *      printed by the operator sweep and are called by nothing else) ---- */
+/* int8 matrix-core rate in TOP/s (2 operations per multiply-accumulate): waves issuing only
+ * v_mfma_i32_32x32x32_i8 on register operands, iters x 4 per wave */
+int spy_hip_measure_mfma_i8(void *stream, int32_t iters, float *tops);
+/* read rate in GB/s over `bytes` of device memory (16-byte aligned, >= 1 MiB; use >= 1 GiB), reps passes */
+int spy_hip_measure_hbm_read(void *stream, const void *buf, size_t bytes, int32_t reps, float *gbps);
+
 /* ---- the token loop: replaces the per-operator dispatch of one forward pass
  *      (DefaultGraphScheduler::execute, backend/distributor/include/scheduler/default_scheduler.h:46-111,
  *      over the graph LLAMAModel::build_graph wires, model/src/llm/model/llama.cpp:86-264) and the

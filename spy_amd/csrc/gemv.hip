@@ -90,61 +90,96 @@ __global__ __launch_bounds__(WROW_THREADS) void wave_row_kernel(gemv_args a, int
     const int NW = (int)gridDim.x * (WROW_THREADS / 64), gw = (int)blockIdx.x * (WROW_THREADS / 64) + wave;
     const int K = a.K, nblk = K / 32, npair = K / 64;
     const size_t RB = (size_t)spy_row_size(WT, K);
-    wtile<WT, NITK> t[NR];
+    // ring of row registers: row k lives in t[k % RING] and is requested RING - 1 rows ahead of its use
+    constexpr int RING = NR < (NITK == 1 ? 4 : 2) ? NR : (NITK == 1 ? 4 : 2);
+    constexpr int DEPTH = RING > 1 ? RING - 1 : 1;
+    wtile<WT, NITK> t[RING];
     auto issue = [&](int k) {
         const int u = gw + k * NW, r = u < a.M ? u : gw % a.M;
-        load_tile<WT, 64, NITK>(t[k], a.W + (size_t)r * RB, npair, lane);
+        load_tile<WT, 64, NITK>(t[k % RING], a.W + (size_t)r * RB, npair, lane);
     };
+    // activation row 0 is requested first, the first weight rows behind it
+    uint32_t xr[NITK + 1];
+    stage_native_q8_load<WROW_THREADS, NITK + 1>(a.xq, nblk, xr);
 #pragma unroll
-    for (int k = 0; k < NR; k++) if (k < WROW_DEPTH) issue(k);
-    staged_act act[WROW_T];
-#pragma unroll
-    for (int c = 0; c < WROW_T; c++) {
+    for (int k = 0; k < NR; k++) if (k < DEPTH) issue(k);
+    auto act_of = [&](int c) {                              // staged activation row c (computed, not kept: no private array)
+        staged_act s;
         int8_t *q = (int8_t *)(smem + (size_t)c * staged_bytes(K));
-        int2 *meta = (int2 *)(q + staged_q_bytes(K));
-        if (c < T) stage_native_q8<WROW_THREADS>(a.xq + (size_t)c * nblk * 34, q, meta, nblk);
-        act[c].q = q; act[c].meta = meta;
+        s.q = q; s.meta = (const int2 *)(q + staged_q_bytes(K));
+        return s;
+    };
+    stage_native_q8_finish<WROW_THREADS, NITK + 1>(xr, (int8_t *)smem, (int2 *)(smem + staged_q_bytes(K)), nblk);
+    for (int c = 1; c < T; c++) {
+        int8_t *q = (int8_t *)(smem + (size_t)c * staged_bytes(K));
+        stage_native_q8<WROW_THREADS>(a.xq + (size_t)c * nblk * 34, q, (int2 *)(q + staged_q_bytes(K)), nblk);
     }
-    constexpr bool HOIST = NR > 1;                          // keep the lane's activations in registers across rows
+    const staged_act act0 = act_of(0);
+    constexpr bool HOIST = NR > 1 && NITK == 1;             // keep the lane's activations in registers across rows
     act_frag<HOIST ? NITK : 1> af;
-    if constexpr (HOIST) load_act_frag<WT, NITK>(af, act[0], npair, lane);
+    if constexpr (HOIST) load_act_frag<WT, NITK>(af, act0, npair, lane);
 #pragma unroll
     for (int k = 0; k < NR; k++) {
-        if (k + WROW_DEPTH < NR) issue(k + WROW_DEPTH);
+        if (RING > 1 && k + DEPTH < NR) issue(k + DEPTH);
         const int r = gw + k * NW;
         float s;
-        if constexpr (HOIST) s = wave_total_lane63(dot_row_frag<WT, NITK>(t[k], af, npair, lane));
-        else s = wave_total_lane63(dot_row_lds<WT, NITK>(t[k], act[0], npair, lane));
+        if constexpr (HOIST) s = wave_total_lane63(dot_row_frag<WT, NITK>(t[k % RING], af, npair, lane));
+        else s = wave_total_lane63(dot_row_lds<WT, NITK>(t[k % RING], act0, npair, lane));
         if (lane == 63 && r < a.M) a.dst[r] = a.residual ? s + a.residual[r] : s;
         for (int c = 1; c < T; c++) {                       // further activation rows against the same weight registers
-            s = wave_total_lane63(dot_row_lds<WT, NITK>(t[k], act[c], npair, lane));
+            s = wave_total_lane63(dot_row_lds<WT, NITK>(t[k % RING], act_of(c), npair, lane));
             const size_t o = (size_t)c * a.dst_stride + r;
             if (lane == 63 && r < a.M) a.dst[o] = a.residual ? s + a.residual[o] : s;
         }
     }
 }
 
+template <int WT, int NITK, int NR>
+static int launch_wave_row_nr(hipStream_t st, const gemv_args &a, int T, size_t lds, int grid) {
+    auto kern = wave_row_kernel<WT, NITK, NR>;
+    static size_t lds_set = 0;
+    if (lds > 48 * 1024 && lds > lds_set) {
+        hipError_t e_ = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e_ != hipSuccess) return (int)e_;
+        lds_set = lds;
+    }
+    kern<<<dim3((unsigned)grid), dim3(WROW_THREADS), lds, st>>>(a, T);
+    return SPY_LAUNCH_RC();
+}
+
+// Rows per wave: the fewest of {1, 2, 3, 4, 6, 8} that covers M with at most one workgroup per compute
+// unit (an even spread; more workgroups than compute units would leave some of them with twice the work);
+// matrices beyond 8 rows per wave take more workgroups.
 template <int WT, int NITK>
 static int launch_wave_row_nitk(hipStream_t st, const gemv_args &a, int T) {
-    constexpr int NRMAX = (WT == SPY_HIP_Q4_0 || WT == SPY_HIP_Q4_K) ? 6 : 4;      // rows per wave: row registers = NR * NITK * PAIR_DW
-    constexpr int NR = NITK == 1 ? NRMAX : 1;
     static int num_cu = 0;
     if (!num_cu) { int dev = 0; hipDeviceProp_t prop; num_cu = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) ? prop.multiProcessorCount : 256; }
     const size_t lds = (size_t)T * staged_bytes(a.K);
-    auto kern1 = wave_row_kernel<WT, NITK, 1>;
-    auto kernN = wave_row_kernel<WT, NITK, NR>;
-    static size_t lds_set = 0;
-    if (lds > 48 * 1024 && lds > lds_set) {
-        { hipError_t e_ = hipFuncSetAttribute((const void *)kern1, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); if (e_ != hipSuccess) return (int)e_; }
-        { hipError_t e_ = hipFuncSetAttribute((const void *)kernN, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); if (e_ != hipSuccess) return (int)e_; }
-        lds_set = lds;
-    }
-    // few rows: one per wave over as many workgroups as needed; many rows: NR per wave
     const int waves = WROW_THREADS / 64;
-    if ((int64_t)a.M <= (int64_t)num_cu * waves) kern1<<<dim3((unsigned)((a.M + waves - 1) / waves)), dim3(WROW_THREADS), lds, st>>>(a, T);
-    else kernN<<<dim3((unsigned)((a.M + waves * NR - 1) / (waves * NR))), dim3(WROW_THREADS), lds, st>>>(a, T);
-    return SPY_LAUNCH_RC();
+    const int64_t need = ((int64_t)a.M + (int64_t)num_cu * waves - 1) / ((int64_t)num_cu * waves);
+    // rows of more than 4096 elements take one row per wave (several 64-element units per lane: the registers
+    // go to the row itself); Q6_K rows (15 dwords per unit) at most 4
+    constexpr int NRMAX = NITK > 1 ? 1 : (WT == SPY_HIP_Q6_K ? 4 : 8);
+    int nr = need <= 1 ? 1 : need <= 2 ? 2 : need <= 3 ? 3 : need <= 4 ? 4 : need <= 6 ? 6 : 8;
+    if (nr > NRMAX) nr = NRMAX;
+    const int grid = (int)(((int64_t)a.M + (int64_t)waves * nr - 1) / ((int64_t)waves * nr));
+    if constexpr (NRMAX >= 4) {
+        switch (nr) {
+        case 2: return launch_wave_row_nr<WT, NITK, 2>(st, a, T, lds, grid);
+        case 3: return launch_wave_row_nr<WT, NITK, 3>(st, a, T, lds, grid);
+        case 4: return launch_wave_row_nr<WT, NITK, 4>(st, a, T, lds, grid);
+        default: break;
+        }
+    }
+    if constexpr (NRMAX >= 8) {
+        if (nr == 6) return launch_wave_row_nr<WT, NITK, 6>(st, a, T, lds, grid);
+        if (nr == 8) return launch_wave_row_nr<WT, NITK, 8>(st, a, T, lds, grid);
+    }
+    return launch_wave_row_nr<WT, NITK, 1>(st, a, T, lds, grid);
 }
+
+// the one-row-per-wave kernels take K % 64 == 0, K <= 12288 and 4-byte aligned activation rows
+static bool wave_rows_ok(int64_t K, const void *xq) { return K % 64 == 0 && K <= 12288 && (((uintptr_t)xq) & 3) == 0; }
 
 // K % 64 == 0 (Q4_0 / Q8_0) or K % 256 == 0 (K-quants), K <= 12288
 template <int WT>
@@ -336,16 +371,18 @@ extern "C" int spy_hip_gemv_q8_0act(void *stream, int wtype, const void *w, cons
     hipStream_t st = (hipStream_t)stream;
     switch (wtype) {
     case SPY_HIP_Q4_0:
+        if (wave_rows_ok(K, xq)) return launch_wave_rows<SPY_HIP_Q4_0>(st, w, (const uint8_t *)xq, dst, residual, M, K, T, dst_stride);
         return pick_cfg(K).lpr ? gemv_fast_cols<SPY_HIP_Q4_0>(st, w, (const uint8_t *)xq, dst, residual, M, K, T, dst_stride)
                                          : launch_generic<SPY_HIP_Q4_0, false>(st, w, xq, dst, residual, nullptr, M, K, T, dst_stride);
     case SPY_HIP_Q8_0:
+        if (wave_rows_ok(K, xq)) return launch_wave_rows<SPY_HIP_Q8_0>(st, w, (const uint8_t *)xq, dst, residual, M, K, T, dst_stride);
         return pick_cfg(K).lpr ? gemv_fast_cols<SPY_HIP_Q8_0>(st, w, (const uint8_t *)xq, dst, residual, M, K, T, dst_stride)
                                          : launch_generic<SPY_HIP_Q8_0, false>(st, w, xq, dst, residual, nullptr, M, K, T, dst_stride);
     case SPY_HIP_Q4_K:
-        return K <= 12288 ? launch_wave_rows<SPY_HIP_Q4_K>(st, w, (const uint8_t *)xq, dst, residual, M, K, T, dst_stride)
+        return wave_rows_ok(K, xq) ? launch_wave_rows<SPY_HIP_Q4_K>(st, w, (const uint8_t *)xq, dst, residual, M, K, T, dst_stride)
                           : launch_generic<SPY_HIP_Q4_K, false>(st, w, xq, dst, residual, nullptr, M, K, T, dst_stride);
     case SPY_HIP_Q6_K:
-        return K <= 12288 ? launch_wave_rows<SPY_HIP_Q6_K>(st, w, (const uint8_t *)xq, dst, residual, M, K, T, dst_stride)
+        return wave_rows_ok(K, xq) ? launch_wave_rows<SPY_HIP_Q6_K>(st, w, (const uint8_t *)xq, dst, residual, M, K, T, dst_stride)
                           : launch_generic<SPY_HIP_Q6_K, false>(st, w, xq, dst, residual, nullptr, M, K, T, dst_stride);
     }
     return SPY_HIP_EUNSUPPORTED;

@@ -121,6 +121,46 @@ static __device__ __forceinline__ void stage_native_q8(const uint8_t *__restrict
     __syncthreads();
 }
 
+// The same in two steps, so that the activation loads can be requested BEFORE the first weight rows (the
+// compute unit serves its memory requests in order: activations requested behind the rows arrive behind
+// them) and turned into the staged form afterwards.  The row must be 4-byte aligned (nblk even); a thread
+// holds NDW dwords, NDW * THREADS >= nblk * 17 / 2.
+template <int THREADS, int NDW>
+static __device__ __forceinline__ void stage_native_q8_load(const uint8_t *__restrict__ xq, int nblk, uint32_t (&r)[NDW]) {
+    const uint32_t *src = (const uint32_t *)xq;
+    const int total = (nblk * 17) >> 1;
+#pragma unroll
+    for (int i = 0; i < NDW; i++) r[i] = src[min((int)threadIdx.x + i * THREADS, total - 1)];
+}
+template <int THREADS, int NDW>
+static __device__ __forceinline__ void stage_native_q8_finish(const uint32_t (&r)[NDW], int8_t *s_q, int2 *s_meta, int nblk) {
+    const int total = (nblk * 17) >> 1;
+#pragma unroll
+    for (int i = 0; i < NDW; i++) {
+        const int dw = (int)threadIdx.x + i * THREADS;
+        if (dw < total) {
+#pragma unroll
+            for (int e = 0; e < 2; e++) {
+                const int h = 2 * dw + e, b = h / 17, w = h - b * 17;
+                const uint16_t v = (uint16_t)(e ? r[i] >> 16 : r[i] & 0xFFFFu);
+                if (w == 0) s_meta[b].x = __float_as_int(h2f(v));
+                else { const int hw = b * 16 + (w - 1); ((uint16_t *)s_q)[2 * act_dw(hw >> 1, nblk >> 1) + (hw & 1)] = v; }
+            }
+        }
+    }
+    __syncthreads();
+    for (int b = threadIdx.x; b < nblk; b += THREADS) {
+        const int4 q0 = *act_part(s_q, b >> 1, 2 * (b & 1), nblk >> 1), q1 = *act_part(s_q, b >> 1, 2 * (b & 1) + 1, nblk >> 1);
+        int s = 0;
+        s = __builtin_amdgcn_sdot4(q0.x, 0x01010101, s, false); s = __builtin_amdgcn_sdot4(q0.y, 0x01010101, s, false);
+        s = __builtin_amdgcn_sdot4(q0.z, 0x01010101, s, false); s = __builtin_amdgcn_sdot4(q0.w, 0x01010101, s, false);
+        s = __builtin_amdgcn_sdot4(q1.x, 0x01010101, s, false); s = __builtin_amdgcn_sdot4(q1.y, 0x01010101, s, false);
+        s = __builtin_amdgcn_sdot4(q1.z, 0x01010101, s, false); s = __builtin_amdgcn_sdot4(q1.w, 0x01010101, s, false);
+        s_meta[b].y = s;
+    }
+    __syncthreads();
+}
+
 // Quantize 4 consecutive floats held by each of 8 consecutive lanes (one 32-element block) the
 // way Quantizator<FP32,Q8_0>::transform does (vec_convert.h:197-260 in the Spy tree): amax,
 // d = amax/127 (stored as fp16), id = 127/amax, q = rint(x*id) saturated to int8.

@@ -1,0 +1,102 @@
+// Measured ceilings of the part, next to the published peaks the rooflines divide by:
+//   * int8 matrix cores: waves that do nothing but v_mfma_i32_32x32x32_i8 on register operands;
+//   * HBM read: every lane streams 16-byte pieces of a large buffer, nothing else.
+// They back the denominators printed by the operator sweep; no product path calls them.
+#include "common.cuh"
+
+#define HIP_TRY(x) do { hipError_t e_ = (x); if (e_ != hipSuccess) return (int)e_; } while (0)
+
+typedef int v4i_p __attribute__((ext_vector_type(4)));
+typedef int v16i_p __attribute__((ext_vector_type(16)));
+
+#define PEAK_MFMA_CHAINS 4
+__global__ __launch_bounds__(256) void peak_mfma_i8_kernel(int iters, int *sink) {
+    v4i_p a = {(int)threadIdx.x, 0x01010101, 0x02020202, (int)blockIdx.x}, b = {0x01010101, (int)threadIdx.x, 0x03030303, 0x01010101};
+    v16i_p acc[PEAK_MFMA_CHAINS];
+#pragma unroll
+    for (int c = 0; c < PEAK_MFMA_CHAINS; c++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[c][r] = c + r;
+    for (int i = 0; i < iters; i++) {
+#pragma unroll
+        for (int c = 0; c < PEAK_MFMA_CHAINS; c++) acc[c] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc[c], 0, 0, 0);
+    }
+    int s = 0;
+#pragma unroll
+    for (int c = 0; c < PEAK_MFMA_CHAINS; c++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) s ^= acc[c][r];
+    if (s == 0x7fffffff) sink[0] = s;                       // keeps the chains alive, practically never taken
+}
+
+// Achieved int8 MFMA rate in TOP/s (2 operations per multiply-accumulate), `iters` x 4 MFMAs per wave,
+// 8 workgroups of 4 waves per compute unit.
+extern "C" int spy_hip_measure_mfma_i8(void *stream, int32_t iters, float *tops) {
+    SPY_CHECK_ARG(iters > 0 && iters <= (1 << 22) && tops);
+    hipStream_t st = (hipStream_t)stream;
+    hipDeviceProp_t prop;
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    HIP_TRY(hipGetDeviceProperties(&prop, dev));
+    int *sink = nullptr;
+    HIP_TRY(hipMalloc(&sink, 64));
+    hipEvent_t e0, e1;
+    HIP_TRY(hipEventCreate(&e0)); HIP_TRY(hipEventCreate(&e1));
+    const int grid = prop.multiProcessorCount * 8;
+    peak_mfma_i8_kernel<<<grid, 256, 0, st>>>(16, sink);    // warm-up
+    HIP_TRY(hipEventRecord(e0, st));
+    peak_mfma_i8_kernel<<<grid, 256, 0, st>>>(iters, sink);
+    HIP_TRY(hipEventRecord(e1, st));
+    HIP_TRY(hipEventSynchronize(e1));
+    float ms = 0.0f;
+    HIP_TRY(hipEventElapsedTime(&ms, e0, e1));
+    const double ops = (double)grid * 4.0 * (double)iters * PEAK_MFMA_CHAINS * 2.0 * 32.0 * 32.0 * 32.0;
+    *tops = (float)(ops / ((double)ms * 1e-3) / 1e12);
+    (void)hipEventDestroy(e0); (void)hipEventDestroy(e1);
+    HIP_TRY(hipFree(sink));
+    return SPY_LAUNCH_RC();
+}
+
+#define PEAK_READ_UNROLL 8
+__global__ __launch_bounds__(256) void peak_read_kernel(const uint4 *__restrict__ p, size_t n16, uint32_t *sink) {
+    const size_t stride = (size_t)gridDim.x * 256;
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    uint32_t x = 0;
+    for (; i + (PEAK_READ_UNROLL - 1) * stride < n16; i += PEAK_READ_UNROLL * stride) {
+        uint4 v[PEAK_READ_UNROLL];
+#pragma unroll
+        for (int u = 0; u < PEAK_READ_UNROLL; u++) v[u] = p[i + u * stride];
+#pragma unroll
+        for (int u = 0; u < PEAK_READ_UNROLL; u++) x ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+    }
+    for (; i < n16; i += stride) { const uint4 v = p[i]; x ^= v.x ^ v.y ^ v.z ^ v.w; }
+    if (x == 0x12345679u) sink[0] = x;
+}
+
+// Achieved read rate in GB/s over `bytes` of device memory at `buf` (contents irrelevant; 16-byte aligned),
+// averaged over `reps` passes.  Use a buffer far larger than the caches (>= 1 GiB).
+extern "C" int spy_hip_measure_hbm_read(void *stream, const void *buf, size_t bytes, int32_t reps, float *gbps) {
+    SPY_CHECK_ARG(buf && bytes >= (1u << 20) && (((uintptr_t)buf) & 15) == 0 && reps > 0 && gbps);
+    hipStream_t st = (hipStream_t)stream;
+    hipDeviceProp_t prop;
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    HIP_TRY(hipGetDeviceProperties(&prop, dev));
+    uint32_t *sink = nullptr;
+    HIP_TRY(hipMalloc(&sink, 64));
+    hipEvent_t e0, e1;
+    HIP_TRY(hipEventCreate(&e0)); HIP_TRY(hipEventCreate(&e1));
+    const int grid = prop.multiProcessorCount * 8;
+    const size_t n16 = bytes / 16;
+    peak_read_kernel<<<grid, 256, 0, st>>>((const uint4 *)buf, n16, sink);
+    HIP_TRY(hipEventRecord(e0, st));
+    for (int r = 0; r < reps; r++) peak_read_kernel<<<grid, 256, 0, st>>>((const uint4 *)buf, n16, sink);
+    HIP_TRY(hipEventRecord(e1, st));
+    HIP_TRY(hipEventSynchronize(e1));
+    float ms = 0.0f;
+    HIP_TRY(hipEventElapsedTime(&ms, e0, e1));
+    *gbps = (float)((double)n16 * 16.0 * reps / ((double)ms * 1e-3) / 1e9);
+    (void)hipEventDestroy(e0); (void)hipEventDestroy(e1);
+    HIP_TRY(hipFree(sink));
+    return SPY_LAUNCH_RC();
+}
