@@ -446,7 +446,8 @@ __global__ __launch_bounds__(WGV_THREADS) void attn_layer_kernel(attn_layer_args
     // ================= B: t = (K.q) * scale for head h ================================================
     const uint16_t *vrow = a.vc + (size_t)(h * 128 + w) * n_ctx;
     uint4 vb[ATL_RV];
-    auto fetch_v = [&](int i) { vb[i] = *(const uint4 *)(vrow + (size_t)min(i * 64 + lane, n_ctx / 8 - 1) * 8); };
+    // pieces past the last cached token re-read the last piece (same cache line: no memory traffic for the unused part of the row)
+    auto fetch_v = [&](int i) { vb[i] = *(const uint4 *)(vrow + (size_t)min(i * 64 + lane, (n_kv - 1) >> 3) * 8); };
     {
         const uint32_t *qp = (const uint32_t *)a.q16 + h * 64 + (lane & 15) * 4;
         const uint32_t qw[4] = {ldc(qp), ldc(qp + 1), ldc(qp + 2), ldc(qp + 3)};
@@ -656,7 +657,7 @@ __global__ __launch_bounds__(PV_THREADS) void attn_pv_kernel(const dev_state *st
     // only PV_DEPTH pieces per wave ahead of their use (the vector-memory queue of the compute unit is
     // finite: a wave that asks for everything at once sits in the issue stage and delays the barriers below)
     uint4 vv[PV_PIECES];
-    auto fetch = [&](int pc0, int u) { vv[u] = *(const uint4 *)(vrow + (size_t)min(pc0 + u * 64 + lane, n_ctx / 8 - 1) * 8); };
+    auto fetch = [&](int pc0, int u) { vv[u] = *(const uint4 *)(vrow + (size_t)min(pc0 + u * 64 + lane, npiece - 1) * 8); };   // past the last token: the last piece again (no traffic)
 #pragma unroll
     for (int u = 0; u < PV_DEPTH; u++) fetch(0, u);
 

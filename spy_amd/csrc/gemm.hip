@@ -16,6 +16,8 @@
 // of 32 x 32; operands double-buffered in LDS with a row stride of 80 bytes (conflict-free for the
 // 128-bit fragment reads of 32 consecutive rows).
 #include "common.cuh"
+#include <stdlib.h>
+#include <string.h>
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
@@ -23,7 +25,11 @@ typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
 #define GEMM_TILE 128
+#define GEMM_SKINNY_MAX_TILES 160 // the 32-row kernel is used up to 64 activation rows and wherever the 128 x 128 tiling would give at most this many workgroups (measured crossover)
 #define GEMM_ROWB 80             // bytes per LDS row: 64 payload + 16 pad
+#ifndef GEMM_PF
+#define GEMM_PF 1                // stages of global loads in flight per thread (the kernel is bound by its scale epilogue on the vector units: 2 and 3 measured the same)
+#endif
 
 // 32-bit word of 4 packed nibbles (already masked to 0..15 per byte) -> 4 int8 of (n - 8)
 static __device__ __forceinline__ uint32_t nib_m8(uint32_t lo) { return (lo + 0x78787878u) ^ 0x80808080u; }
@@ -49,12 +55,12 @@ __global__ __launch_bounds__(256, 2) void gemm_q8act_kernel(const uint8_t *__res
     const int lrow = tid & 127, half = tid >> 7;
     const uint32_t *gA = (const uint32_t *)(W + (size_t)min(m0 + lrow, M - 1) * RBw) + half * (HALF_DW - 1);
     const uint32_t *gB = (const uint32_t *)(xq + (size_t)min(t0 + lrow, T - 1) * RBx) + half * 8;
-    uint32_t rawA[HALF_DW], rawB[9];
-    auto gload = [&](int s) {
-#pragma unroll
-        for (int i = 0; i < HALF_DW; i++) rawA[i] = gA[(size_t)s * PAIR_DW + i];
-#pragma unroll
-        for (int i = 0; i < 9; i++) rawB[i] = gB[(size_t)s * 17 + i];
+    // Global loads run GEMM_PF stages ahead of the stage being multiplied (a ring of raw registers): with one
+    // stage ahead a workgroup advances one stage per memory round trip, whatever the matrix cores could do.
+    uint32_t rawA[GEMM_PF][HALF_DW], rawB[GEMM_PF][9];
+    auto gload = [&](int slot, int s) {                      // 4-byte aligned: 128-bit loads + one dword
+        __builtin_memcpy(rawA[slot], __builtin_assume_aligned(gA + (size_t)s * PAIR_DW, 4), HALF_DW * 4);
+        __builtin_memcpy(rawB[slot], __builtin_assume_aligned(gB + (size_t)s * 17, 4), 36);
     };
     // one Q8_0 block held in 9 dwords -> scale + 8 dwords of int8
     auto split_q8 = [&](const uint32_t *raw, float &d, uint32_t *q) {
@@ -62,23 +68,23 @@ __global__ __launch_bounds__(256, 2) void gemm_q8act_kernel(const uint8_t *__res
 #pragma unroll
         for (int i = 0; i < 8; i++) q[i] = half ? raw[i + 1] : __builtin_amdgcn_alignbit(raw[i + 1], raw[i], 16);
     };
-    auto unpack = [&](int b) {
+    auto unpack = [&](int b, int slot) {
         uint32_t q[8];
         float d;
         if constexpr (WT == SPY_HIP_Q4_0) {
             // {d, qs[16]}: element j = low nibble of qs[j], element j+16 = high nibble (quant.h:25-28); stored as n - 8
-            d = h2f((uint16_t)(half ? rawA[0] >> 16 : rawA[0] & 0xFFFFu));
+            d = h2f((uint16_t)(half ? rawA[slot][0] >> 16 : rawA[slot][0] & 0xFFFFu));
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                const uint32_t n = half ? rawA[i + 1] : __builtin_amdgcn_alignbit(rawA[i + 1], rawA[i], 16);
+                const uint32_t n = half ? rawA[slot][i + 1] : __builtin_amdgcn_alignbit(rawA[slot][i + 1], rawA[slot][i], 16);
                 q[i] = nib_m8(n & 0x0F0F0F0Fu);
                 q[4 + i] = nib_m8((n >> 4) & 0x0F0F0F0Fu);
             }
-        } else split_q8(rawA, d, q);
+        } else split_q8(rawA[slot], d, q);
         uint4 *ra = (uint4 *)(sA[b] + lrow * GEMM_ROWB + half * 32);
         ra[0] = make_uint4(q[0], q[1], q[2], q[3]); ra[1] = make_uint4(q[4], q[5], q[6], q[7]);
         sAd[b][half][lrow] = d;
-        split_q8(rawB, d, q);                                // {d, qs[32]} (quant.h:139-142)
+        split_q8(rawB[slot], d, q);                          // {d, qs[32]} (quant.h:139-142)
         uint4 *rb = (uint4 *)(sB[b] + lrow * GEMM_ROWB + half * 32);
         rb[0] = make_uint4(q[0], q[1], q[2], q[3]); rb[1] = make_uint4(q[4], q[5], q[6], q[7]);
         sBd[b][half][lrow] = d;
@@ -92,12 +98,7 @@ __global__ __launch_bounds__(256, 2) void gemm_q8act_kernel(const uint8_t *__res
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
-    gload(0);
-    unpack(0);
-    __syncthreads();
-    for (int s = 0; s < nstage; s++) {
-        const int b = s & 1;
-        gload(min(s + 1, nstage - 1));                    // unconditional: the last stage re-reads itself
+    auto multiply = [&](int b) {
 #pragma unroll 1
         for (int blk = 0; blk < 2; blk++) {
             v4i fa[2], fb[2];
@@ -124,8 +125,23 @@ __global__ __launch_bounds__(256, 2) void gemm_q8act_kernel(const uint8_t *__res
                 }
             }
         }
-        if (s + 1 < nstage) unpack(b ^ 1);
-        __syncthreads();
+    };
+
+#pragma unroll
+    for (int j = 0; j < GEMM_PF; j++) gload(j, min(j, nstage - 1));
+    unpack(0, 0);
+    __syncthreads();
+    for (int s0 = 0; s0 < nstage; s0 += GEMM_PF) {
+#pragma unroll
+        for (int j = 0; j < GEMM_PF; j++) {
+            const int s = s0 + j;                              // stage in LDS buffer s & 1; its raw registers (slot j) are free
+            if (s < nstage) {
+                gload(j, min(s + GEMM_PF, nstage - 1));      // unconditional: the last stages re-read the last one
+                multiply(s & 1);
+                if (s + 1 < nstage) unpack((s & 1) ^ 1, (j + 1) % GEMM_PF);
+                __syncthreads();
+            }
+        }
     }
     // C layout of the 32x32 MFMA: lane -> column (token) lane & 31; register r -> row (r / 4) * 8 + (lane >> 5) * 4 + (r & 3)
 #pragma unroll
@@ -146,6 +162,185 @@ __global__ __launch_bounds__(256, 2) void gemm_q8act_kernel(const uint8_t *__res
                 }
             }
         }
+}
+
+// ---- few activation rows (16 .. 128 tokens) ----------------------------------------------------------
+// The 128 x 128 tile leaves most of the part idle when T is small (M / 128 workgroups, most of each tile
+// padding).  Here a workgroup owns 32 weight rows and its 4 waves work independently of each other: wave =
+// (token sub-tile of 32) x (contiguous slice of K), NTW x KS = 4.  A wave copies a chunk of 8 blocks of its
+// 32 weight rows and 32 activation rows into its own LDS area with 16-byte loads that run along the rows
+// (9 or 17 consecutive lanes per row: a row-per-lane pattern would touch 64 cache lines per instruction),
+// one chunk ahead in registers; lane (row = lane & 31, half = lane >> 5) then picks its MFMA fragment out of
+// the raw blocks (4-byte aligned LDS reads + a 16-bit funnel shift where a block starts mid-dword).  The weight
+// scales of the 32 rows go through a wave-private LDS line so that a lane can read those of its 16
+// accumulator rows.  No workgroup barrier until the K slices are summed (through LDS, in a fixed order).
+#define GSK_CH 8                  // blocks per chunk (K % 256 == 0)
+template <int WT> struct gsk_traits {
+    static constexpr int WBLK = (WT == SPY_HIP_Q4_0) ? 18 : 34;
+    static constexpr int WP = GSK_CH * WBLK / 16;                        // 16-byte pieces per weight row and chunk: 9 / 17
+    static constexpr int WS = (WT == SPY_HIP_Q4_0) ? 176 : 272;          // LDS row strides: 16-byte aligned, 2-way bank conflicts at worst
+    static constexpr int XP = 17, XS = 272;
+    static constexpr int NWI = (32 * WP + 63) / 64, NXI = (32 * XP + 63) / 64;
+    static constexpr int WAVE_LDS = 32 * WS + 32 * XS + GSK_CH * 128;   // weights, activations, weight scales [block][row]
+};
+// 16 int8 of half `kh` of Q8_0 block bb (34 bytes each, chunk-relative) of an LDS row, and the block's scale
+static __device__ __forceinline__ void gsk_frag_q8(const uint8_t *row, int bb, int kh, v4i &q, float &d) {
+    if ((bb & 1) == 0) {                                   // block at 34 bb = 0 mod 4: quants start mid-dword
+        const uint32_t *p = (const uint32_t *)(row + 34 * bb + 16 * kh);
+        const uint32_t w0 = p[0], w1 = p[1], w2 = p[2], w3 = p[3], w4 = p[4];
+        q = v4i{(int)__builtin_amdgcn_alignbit(w1, w0, 16), (int)__builtin_amdgcn_alignbit(w2, w1, 16),
+                (int)__builtin_amdgcn_alignbit(w3, w2, 16), (int)__builtin_amdgcn_alignbit(w4, w3, 16)};
+        d = h2f((uint16_t)(*(const uint32_t *)(row + 34 * bb) & 0xFFFFu));
+    } else {                                               // block at 34 bb = 2 mod 4: quants dword-aligned
+        const uint32_t *p = (const uint32_t *)(row + 34 * bb + 2 + 16 * kh);
+        q = v4i{(int)p[0], (int)p[1], (int)p[2], (int)p[3]};
+        d = h2f((uint16_t)(*(const uint32_t *)(row + 34 * bb - 2) >> 16));
+    }
+}
+template <int WT, int NTW>
+__global__ __launch_bounds__(256, 2) void gemm_skinny_kernel(const uint8_t *__restrict__ W, const uint8_t *__restrict__ xq, float *__restrict__ dst,
+                                                          int M, int K, int T, int64_t dst_stride) {
+    using TR = gsk_traits<WT>;
+    constexpr int KS = 4 / NTW;
+    extern __shared__ __attribute__((aligned(16))) uint8_t gsk_smem[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), tw = wave % NTW, ks = wave / NTW;
+    const int row = lane & 31, kh = lane >> 5;
+    const int m0 = blockIdx.x * 32, t0 = blockIdx.y * (32 * NTW) + tw * 32;
+    const int nblk = K / 32, nchunk = nblk / GSK_CH;
+    const int c_begin = ks * nchunk / KS, c_end = (ks + 1) * nchunk / KS;
+    uint8_t *sw = gsk_smem + (size_t)wave * TR::WAVE_LDS, *sx = sw + 32 * TR::WS;
+    float *s_dw = (float *)(sx + 32 * TR::XS);
+    const size_t RBw = (size_t)nblk * TR::WBLK, RBx = (size_t)nblk * 34;
+
+    // piece p = lane + 64 i of the chunk: row p / WP, 16 bytes at column p % WP (clamped: the last lanes repeat the last piece)
+    uint4 rw[TR::NWI], rx[TR::NXI];
+    int wofs[TR::NWI], xofs[TR::NXI];
+    uint32_t wgo[TR::NWI], xgo[TR::NXI];                    // byte offsets into W / xq (the launcher checks that they fit)
+#pragma unroll
+    for (int i = 0; i < TR::NWI; i++) {
+        const int p = min(lane + 64 * i, 32 * TR::WP - 1), r = p / TR::WP, c = p - r * TR::WP;
+        wofs[i] = r * TR::WS + c * 16;
+        wgo[i] = (uint32_t)((size_t)min(m0 + r, M - 1) * RBw + c * 16);
+    }
+#pragma unroll
+    for (int i = 0; i < TR::NXI; i++) {
+        const int p = min(lane + 64 * i, 32 * TR::XP - 1), r = p / TR::XP, c = p - r * TR::XP;
+        xofs[i] = r * TR::XS + c * 16;
+        xgo[i] = (uint32_t)((size_t)min(t0 + r, T - 1) * RBx + c * 16);
+    }
+    auto gload = [&](int c) {
+        const uint8_t *wb = W + (size_t)c * (GSK_CH * TR::WBLK), *xb = xq + (size_t)c * (GSK_CH * 34);
+#pragma unroll
+        for (int i = 0; i < TR::NWI; i++) { uint4 v; __builtin_memcpy(&v, __builtin_assume_aligned(wb + wgo[i], 2), 16); rw[i] = v; }
+#pragma unroll
+        for (int i = 0; i < TR::NXI; i++) { uint4 v; __builtin_memcpy(&v, __builtin_assume_aligned(xb + xgo[i], 2), 16); rx[i] = v; }
+    };
+    float acc[16];
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0.0f;
+    if (c_begin < c_end) gload(c_begin);
+    for (int c = c_begin; c < c_end; c++) {
+#pragma unroll
+        for (int i = 0; i < TR::NWI; i++) *(uint4 *)(sw + wofs[i]) = rw[i];
+#pragma unroll
+        for (int i = 0; i < TR::NXI; i++) *(uint4 *)(sx + xofs[i]) = rx[i];
+        gload(min(c + 1, c_end - 1));                        // unconditional: the last chunk re-reads itself
+        // weight scales of the chunk as floats [block][row], written once per chunk (half kh takes blocks 4 kh .. 4 kh + 3)
+#pragma unroll
+        for (int j = 0; j < GSK_CH / 2; j++) {
+            const int bb = kh * (GSK_CH / 2) + j;
+            const uint32_t dd = *(const uint32_t *)(sw + row * TR::WS + bb * TR::WBLK - ((j & 1) ? 2 : 0));
+            s_dw[bb * 32 + row] = h2f((uint16_t)((j & 1) ? dd >> 16 : dd & 0xFFFFu));
+        }
+#pragma unroll 1
+        for (int bp = 0; bp < GSK_CH / 2; bp++) {             // block pairs: the even block starts dword-aligned, the odd one mid-dword
+            const uint8_t *wr = sw + row * TR::WS + bp * (2 * TR::WBLK), *xr = sx + row * TR::XS + bp * 68;
+#pragma unroll
+            for (int bb = 0; bb < 2; bb++) {
+                v4i fa, fb;
+                float dwf = 0.0f, dxf;
+                gsk_frag_q8(xr, bb, kh, fb, dxf);
+                if constexpr (WT == SPY_HIP_Q4_0) {
+                    // {d, qs[16]}: element j = low nibble of qs[j], element j + 16 = high nibble (quant.h:25-28)
+                    uint32_t n0, n1, n2, n3;
+                    if (bb == 0) {
+                        const uint32_t *p = (const uint32_t *)wr;
+                        const uint32_t w0 = p[0], w1 = p[1], w2 = p[2], w3 = p[3], w4 = p[4];
+                        n0 = __builtin_amdgcn_alignbit(w1, w0, 16); n1 = __builtin_amdgcn_alignbit(w2, w1, 16);
+                        n2 = __builtin_amdgcn_alignbit(w3, w2, 16); n3 = __builtin_amdgcn_alignbit(w4, w3, 16);
+                    } else {
+                        const uint32_t *p = (const uint32_t *)(wr + 16);
+                        n0 = p[1]; n1 = p[2]; n2 = p[3]; n3 = p[4];
+                    }
+                    const int sh = kh * 4;
+                    fa = v4i{(int)nib_m8((n0 >> sh) & 0x0F0F0F0Fu), (int)nib_m8((n1 >> sh) & 0x0F0F0F0Fu),
+                             (int)nib_m8((n2 >> sh) & 0x0F0F0F0Fu), (int)nib_m8((n3 >> sh) & 0x0F0F0F0Fu)};
+                } else gsk_frag_q8(wr, bb, kh, fa, dwf);
+                (void)dwf;
+                v16i z = {0};
+                const v16i I = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa, fb, z, 0, 0, 0);
+                float dw[16];
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const float4 v = *(const float4 *)&s_dw[(2 * bp + bb) * 32 + g * 8 + kh * 4];
+                    dw[4 * g] = v.x; dw[4 * g + 1] = v.y; dw[4 * g + 2] = v.z; dw[4 * g + 3] = v.w;
+                }
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[r] = fmaf(dw[r] * dxf, (float)I[r], acc[r]);
+            }
+        }
+    }
+    if constexpr (KS > 1) {
+        // the slices of K meet in the waves with ks == 0: the others park their sums in their own (now idle) LDS area
+        float *park = (float *)sw;
+        if (ks > 0) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) park[r * 64 + lane] = acc[r];
+        }
+        __syncthreads();
+        if (ks > 0) return;
+#pragma unroll
+        for (int k = 1; k < KS; k++) {
+            const float *other = (const float *)(gsk_smem + (size_t)(k * NTW + tw) * TR::WAVE_LDS);
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[r] += other[r * 64 + lane];
+        }
+    }
+    // C layout of the 32x32 MFMA: lane -> column (token) lane & 31; register r -> row (r / 4) * 8 + (lane >> 5) * 4 + (r & 3)
+    const int t = t0 + row;
+    if (t < T) {
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const int m = m0 + g * 8 + kh * 4;
+            float *o = dst + (size_t)t * dst_stride + m;
+            if (m + 3 < M && (((uintptr_t)o) & 15) == 0) *(float4 *)o = make_float4(acc[4 * g], acc[4 * g + 1], acc[4 * g + 2], acc[4 * g + 3]);
+            else {
+#pragma unroll
+                for (int e = 0; e < 4; e++) if (m + e < M) o[e] = acc[4 * g + e];
+            }
+        }
+    }
+}
+
+template <int WT, int NTW>
+static int launch_gemm_skinny_ntw(hipStream_t st, const void *w, const void *xq, float *dst, int64_t M, int64_t K, int64_t T, int64_t dst_stride) {
+    auto kern = gemm_skinny_kernel<WT, NTW>;
+    constexpr size_t lds = 4 * (size_t)gsk_traits<WT>::WAVE_LDS;
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e_ = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e_ != hipSuccess) return (int)e_;
+        attr_set = true;
+    }
+    kern<<<dim3((unsigned)((M + 31) / 32), (unsigned)((T + 32 * NTW - 1) / (32 * NTW))), dim3(256), lds, st>>>(
+        (const uint8_t *)w, (const uint8_t *)xq, dst, (int)M, (int)K, (int)T, dst_stride);
+    return SPY_LAUNCH_RC();
+}
+template <int WT>
+static int launch_gemm_skinny(hipStream_t st, const void *w, const void *xq, float *dst, int64_t M, int64_t K, int64_t T, int64_t dst_stride) {
+    if (T <= 32) return launch_gemm_skinny_ntw<WT, 1>(st, w, xq, dst, M, K, T, dst_stride);
+    if (T <= 64) return launch_gemm_skinny_ntw<WT, 2>(st, w, xq, dst, M, K, T, dst_stride);
+    return launch_gemm_skinny_ntw<WT, 4>(st, w, xq, dst, M, K, T, dst_stride);
 }
 
 // ---- K-quant weights ---------------------------------------------------------------------------------
@@ -328,6 +523,10 @@ extern "C" int spy_hip_gemm_q8_0act(void *stream, int wtype, const void *w_dev, 
     SPY_CHECK_ARG((M + GEMM_TILE - 1) / GEMM_TILE <= 0x7fffffff && (T + GEMM_TILE - 1) / GEMM_TILE <= 65535);
     const dim3 grid((unsigned)((M + GEMM_TILE - 1) / GEMM_TILE), (unsigned)((T + GEMM_TILE - 1) / GEMM_TILE));
     hipStream_t st = (hipStream_t)stream;
+    const char *force = getenv("SPY_HIP_GEMM");           // "tile" / "skinny": measurement switch
+    const bool skinny = K % 256 == 0 && M * (K / 32) * 34 < (int64_t)1 << 31 && T * (K / 32) * 34 < (int64_t)1 << 31 && (force ? !strcmp(force, "skinny") : (T <= 64 || (int64_t)grid.x * grid.y <= GEMM_SKINNY_MAX_TILES));
+    if (skinny && wtype == SPY_HIP_Q4_0) return launch_gemm_skinny<SPY_HIP_Q4_0>(st, w_dev, xq_dev, dst_dev, M, K, T, dst_stride);
+    if (skinny && wtype == SPY_HIP_Q8_0) return launch_gemm_skinny<SPY_HIP_Q8_0>(st, w_dev, xq_dev, dst_dev, M, K, T, dst_stride);
     if (wtype == SPY_HIP_Q4_0) gemm_q8act_kernel<SPY_HIP_Q4_0><<<grid, dim3(256), 0, st>>>((const uint8_t *)w_dev, (const uint8_t *)xq_dev, dst_dev, (int)M, (int)K, (int)T, dst_stride);
     else if (wtype == SPY_HIP_Q8_0) gemm_q8act_kernel<SPY_HIP_Q8_0><<<grid, dim3(256), 0, st>>>((const uint8_t *)w_dev, (const uint8_t *)xq_dev, dst_dev, (int)M, (int)K, (int)T, dst_stride);
     else if (wtype == SPY_HIP_Q4_K) gemm_kq_kernel<SPY_HIP_Q4_K><<<grid, dim3(256), 0, st>>>((const uint8_t *)w_dev, (const uint8_t *)xq_dev, dst_dev, (int)M, (int)K, (int)T, dst_stride);

@@ -19,7 +19,8 @@ def hip():
 
 
 @pytest.mark.parametrize("wtype", [O.Q4_0, O.Q8_0])
-@pytest.mark.parametrize("M,K,T", [(128, 4096, 128), (256, 256, 16), (200, 11008, 77), (130, 64, 129), (4096, 4096, 256)])
+@pytest.mark.parametrize("M,K,T", [(128, 4096, 128), (256, 256, 16), (200, 11008, 77), (130, 64, 129), (4096, 4096, 256),
+                                   (96, 4096, 33), (70, 1024, 64), (33, 64, 17), (1000, 2048, 31)])
 def test_gemm_q8_0act_matches_oracle(hip, oracle, wtype, M, K, T):
     from tests.gpu_util import dev, dev_empty, call, assert_close
     rng = np.random.default_rng(wtype * 131 + M + K + T)
