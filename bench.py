@@ -37,6 +37,8 @@ def main():
     ap.add_argument("--layers", type=int, default=32, help="debug only: fewer layers (result is then not the headline config)")
     ap.add_argument("--model", choices=["q4_0", "q8_0", "q4_k_m"], default="q4_0",
                     help="q4_0: the headline workload; q8_0 / q4_k_m (Q4_K with Q6_K attn_v, ffn_down and head): the other 7B configurations")
+    ap.add_argument("--via-gguf", metavar="PATH", default=None,
+                    help="write the synthetic model to PATH as a GGUF file and run the model loaded from it (file -> HBM times are reported)")
     ap.add_argument("--no-graph", action="store_true", help="launch the kernels of every pass one by one instead of replaying a HIP graph (for profilers)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch a plain copy kernel over 256 MiB three times (a known-size dispatch to scale profiler byte counters by)")
@@ -66,7 +68,20 @@ def main():
     # K-quant matrices: random well-formed blocks (this package has no K-quant quantizer; timing only)
     tensors = M.synth_model(cfg, seed=1234, quantizer=M.random_k_blocks if args.model == "q4_k_m" else None)
     log("synthetic model: %.1f s, %.2f GB of weights streamed per token" % (time.time() - t0, cfg.weight_bytes() / 1e9))
-    eng = M.Engine(cfg, tensors)
+    load_info, loaded = None, None
+    if args.via_gguf:
+        from spy_amd import gguf as G
+        t0 = time.time()
+        G.write_llama(args.via_gguf, cfg, tensors)
+        t_write = time.time() - t0
+        loaded = G.GGUFModel(args.via_gguf, n_ctx=n_ctx)
+        eng = loaded.engine
+        load_info = {"file_bytes": os.path.getsize(args.via_gguf), "parse_ms": round(loaded.parse_ms, 2), "upload_ms": round(loaded.upload_ms, 1),
+                     "create_ms": round(loaded.create_ms, 1), "upload_GBps": round(loaded.weight_bytes / loaded.upload_ms / 1e6, 2)}
+        log("GGUF: wrote %.2f GB in %.1f s; parse %.1f ms, upload to HBM %.0f ms (%.1f GB/s from the page cache), token loop set-up %.0f ms"
+            % (load_info["file_bytes"] / 1e9, t_write, loaded.parse_ms, loaded.upload_ms, load_info["upload_GBps"], loaded.create_ms))
+    else:
+        eng = M.Engine(cfg, tensors)
     rng = np.random.default_rng(4096)
     prompt = rng.integers(0, cfg.n_vocab, fill).astype(np.int32)
     t0 = time.time()
@@ -177,8 +192,12 @@ def main():
         "kernel_us": {k: round(v, 2) for k, v in per_kernel.items()},
         "roofline": roofline, "cpu_baseline": cpu,
     }
+    if load_info:
+        out["gguf_load"] = load_info
     print(json.dumps(out), flush=True)
     eng.close()
+    if loaded:
+        loaded.close()
 
 
 if __name__ == "__main__":

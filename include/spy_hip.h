@@ -148,7 +148,7 @@ int spy_hip_measure_hbm_read(void *stream, const void *buf, size_t bytes, int32_
  *      greedy loop of AutoModelGenerator::generate (app/cli/include/cli.h:88-128) for single-token
  *      passes.  Same operators, same rounding points, same KV-cache layouts
  *      (K: f16 [n_ctx][n_head][hd], V: f16 [n_embd][n_ctx]; model/src/llm/plugin/attention.cpp:188-262);
- *      fused into six kernels per layer and replayed as a HIP graph. ----------------------------- */
+ *      fused into four kernels per layer and replayed as a HIP graph. ----------------------------- */
 typedef struct spy_hip_llama_layer {
     const float *attn_norm, *ffn_norm;                         /* f32[n_embd], device          */
     const void  *wq, *wk, *wv, *wo, *w_gate, *w_up, *w_down;   /* native GGUF blocks, device   */

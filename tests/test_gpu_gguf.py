@@ -1,0 +1,56 @@
+"""GGUF file -> HBM -> token loop on the GPU: a model loaded from a file computes exactly what the same
+model built from arrays computes, and agrees with the oracle."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("name,kw", [
+    ("q4_0, f32 embeddings", dict()),
+    ("q8_0, q8_0 embeddings", dict(wtype=8, t_tok_embd=8)),
+    ("q4_k body, q6_k wv / down / head", dict(wtype=12, t_out=14, tensor_types={"attn_v": 14, "ffn_down": 14})),
+])
+def test_loaded_model_equals_the_model_built_from_arrays(tmp_path, oracle, name, kw):
+    from spy_amd import gguf as G, model as M
+    from tests.gpu_util import E2E_TOL
+    from tests.model_util import OracleModel, k_quant_quantizer
+    kw = dict(kw)
+    kw.setdefault("wtype", 2)
+    cfg = M.Config(n_layer=2, n_embd=512, n_head=4, n_ff=1024, n_vocab=640, n_ctx=64, **kw)
+    tensors = M.synth_model(cfg, seed=17, outlier_every=500, quantizer=k_quant_quantizer)
+    path = G.write_llama(str(tmp_path / "m.gguf"), cfg, tensors, alignment=64)
+    loaded = G.GGUFModel(path)
+    assert loaded.weight_bytes == sum(t.nbytes for t in tensors.values())
+    d = loaded.desc
+    assert (d.n_layer, d.n_embd, d.n_head, d.n_ff, d.n_vocab, d.n_ctx) == (2, 512, 4, 1024, 640, 64)
+    assert d.eps == np.float32(cfg.eps) and d.rope_freq_base == np.float32(cfg.rope_freq_base)
+    assert loaded.file.get_arr_str("tokenizer.ggml.tokens", 5) == b"<t5>"
+    direct = M.Engine(cfg, tensors)
+    rng = np.random.default_rng(3)
+    prompt = rng.integers(0, cfg.n_vocab, 7).astype(np.int32)
+    a, b = loaded.engine.forward(prompt, 0), direct.forward(prompt, 0)
+    assert np.array_equal(a, b), name
+    ora = OracleModel(cfg, tensors)
+    lo = ora.forward(prompt, 0)
+    assert float(np.abs(a - lo).max() / np.abs(lo).max()) < E2E_TOL
+    tok = int(np.argmax(a[-1]))
+    ta, tb = loaded.engine.decode_greedy(tok, 7, 6), direct.decode_greedy(tok, 7, 6)
+    assert np.array_equal(ta, tb), name
+    assert np.array_equal(loaded.engine.generate(prompt, 5), direct.generate(prompt, 5))
+    direct.close()
+    loaded.close()
+
+
+def test_context_argument_and_reload(tmp_path):
+    """n_ctx = 0 takes the file's context length; another n_ctx sizes the KV caches (rounded up to 8)."""
+    from spy_amd import gguf as G, model as M
+    cfg = M.Config(n_layer=1, n_embd=256, n_head=2, n_ff=512, n_vocab=320, n_ctx=40, wtype=2)
+    path = G.write_llama(str(tmp_path / "c.gguf"), cfg, M.synth_model(cfg, seed=2))
+    m0 = G.GGUFModel(path)
+    assert m0.desc.n_ctx == 40
+    m1 = G.GGUFModel(path, n_ctx=21)
+    assert m1.desc.n_ctx == 24
+    t = np.array([3, 1, 4, 1, 5], np.int32)
+    assert np.array_equal(m0.engine.forward(t, 0), m1.engine.forward(t, 0))
+    m0.close(); m1.close()
