@@ -300,6 +300,12 @@ __global__ __launch_bounds__(WGV_THREADS) void wave_gemv_kernel(fused_args a) {
 // is kept next to them and bumped by workgroup 0 of the head after the last barrier.  Polls are bounded:
 // on expiry the error flag of the device state is raised and the workgroup leaves.
 // All of a launch's workgroups must be resident (grid <= compute units, one 1024-thread workgroup each).
+#ifndef ATL_WAVES
+#define ATL_WAVES 16              // waves per workgroup: 16 (one workgroup per compute unit) or 8 (two; measured 8 % slower, also with the second one started late)
+#endif
+#define ATL_THREADS (ATL_WAVES * 64)
+#define ATL_GPH (128 / ATL_WAVES)  // workgroups per head
+#define ATL_NX (1024 / ATL_THREADS)
 #define ATL_RS 10                 // groups of 4 keys per wave (n_ctx <= 128 * 4 * ATL_RS)
 #define ATL_RV 10                 // 128-bit pieces per lane of a V^T row (n_ctx <= 512 * ATL_RV)
 #ifndef ATL_DEPTH_K
@@ -322,32 +328,34 @@ struct attn_layer_args {
 #endif
 };
 #ifdef ATL_STAMPS
-#define ATL_STAMP(i) do { if (a.dbg && tid == 0 && (blockIdx.x == 0 || blockIdx.x == 100)) a.dbg[(blockIdx.x ? 64 : 0) + (i)] = wall_clock64(); } while (0)
+#define ATL_STAMP(i) do { if (a.dbg && tid == 0) { if (blockIdx.x == 0 || blockIdx.x == 100) a.dbg[(blockIdx.x ? 64 : 0) + (i)] = wall_clock64(); \
+                                                    if ((i) == 0 || (i) == 3 || (i) == 5 || (i) == 8) a.dbg[128 + blockIdx.x * 8 + ((i) == 0 ? 0 : (i) == 3 ? 1 : (i) == 5 ? 2 : 3)] = wall_clock64(); \
+                                                    if ((i) == 0) { a.dbg[128 + blockIdx.x * 8 + 4] = __builtin_amdgcn_s_getreg((31 << 11) | 4); a.dbg[128 + blockIdx.x * 8 + 5] = __builtin_amdgcn_s_getreg((31 << 11) | 20); } } } while (0)
 #else
 #define ATL_STAMP(i) do { } while (0)
 #endif
 
 template <int WT, int WTV>        // types of wq / wk and of wv
-__global__ __launch_bounds__(WGV_THREADS) void attn_layer_kernel(attn_layer_args a) {
+__global__ __launch_bounds__(ATL_THREADS, 4) void attn_layer_kernel(attn_layer_args a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    __shared__ float s_red[WGV_WAVES];
+    __shared__ float s_red[16];
     __shared__ int s_ok;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int h = blockIdx.x >> 3, g = blockIdx.x & 7, w = g * WGV_WAVES + wave;      // w: wave of the head, 0..127
+    const int h = blockIdx.x / ATL_GPH, g = blockIdx.x % ATL_GPH, w = g * ATL_WAVES + wave;      // w: wave of the head, 0..127
     const int d = a.d, npair = d / 64, n_ctx = a.n_ctx;
     const size_t RB = (size_t)spy_row_size(WT, d);
     const int pos = a.st->pos, n_kv = pos + 1;
     uint32_t *sync = a.sync + (size_t)h * 96;
     // the launch count was written by the previous launch: an ordinary (scalar) load sees it, and stays out of
     // the vector-memory queue in which the first activation loads would otherwise wait behind it
-    const uint32_t target = 8u * (sync[64] + 1u);
+    const uint32_t target = (uint32_t)ATL_GPH * (sync[64] + 1u);
     ATL_STAMP(0);
 
     int8_t *s_q = (int8_t *)smem;
     int2 *s_meta = (int2 *)(smem + staged_q_bytes(d));
     float *s_rope = (float *)(smem + staged_bytes(d));               // 128
-    float *s_out = s_rope + 128;                                     // [WGV_WAVES][4 * ATL_RS]
-    float *s_t = s_out + WGV_WAVES * 4 * ATL_RS;                     // n_ctx
+    float *s_out = s_rope + 128;                                     // [ATL_WAVES][4 * ATL_RS]
+    float *s_t = s_out + ATL_WAVES * 4 * ATL_RS;                     // n_ctx
     uint16_t *s_p = (uint16_t *)(s_t + n_ctx);                       // n_ctx + 8
 
     // wave 0 writes the workgroup's results, waits for the stores, thread 0 goes through the head's barrier
@@ -372,8 +380,13 @@ __global__ __launch_bounds__(WGV_THREADS) void attn_layer_kernel(attn_layer_args
     };
 
     // ================= A: attn_norm, Q/K/V_project of head h, rope, KV-cache copies =================
-    const int i4 = min(tid, d / 4 - 1);
-    const float4 xv = ((const float4 *)a.x_in)[i4], wv = ((const float4 *)a.normw)[i4];
+    // the 1024 float4 of x (d <= 4096) are spread over the workgroup's threads: ATL_NX each, float4 tid + j * ATL_THREADS
+    float4 xv[ATL_NX], wv[ATL_NX];
+#pragma unroll
+    for (int j = 0; j < ATL_NX; j++) {
+        const int i4 = min(tid + j * ATL_THREADS, d / 4 - 1);
+        xv[j] = ((const float4 *)a.x_in)[i4]; wv[j] = ((const float4 *)a.normw)[i4];
+    }
     const float rope_v = a.rope_cs[min(tid, 127)];
     wtile<WT, 1> t[2];
     wtile<WTV, 1> tv;
@@ -383,23 +396,31 @@ __global__ __launch_bounds__(WGV_THREADS) void attn_layer_kernel(attn_layer_args
     load_tile<WT, 64, 1>(t[1], p0 + RB, npair, lane);
     if (tid < 128) s_rope[tid] = rope_v;
     {
-        float acc = 0.0f;
-        if (tid < d / 4) { acc = fmaf(xv.x, xv.x, acc); acc = fmaf(xv.y, xv.y, acc); acc = fmaf(xv.z, xv.z, acc); acc = fmaf(xv.w, xv.w, acc); }
-        acc = group_sum<64>(acc);
+        // sums of squares per 64 float4 (one entry of s_red each), added in the same order whatever the workgroup size
+#pragma unroll
+        for (int j = 0; j < ATL_NX; j++) {
+            float acc = 0.0f;
+            if (tid + j * ATL_THREADS < d / 4) { const float4 v = xv[j]; acc = fmaf(v.x, v.x, acc); acc = fmaf(v.y, v.y, acc); acc = fmaf(v.z, v.z, acc); acc = fmaf(v.w, v.w, acc); }
+            acc = group_sum<64>(acc);
+            if (lane == 0) s_red[wave + j * ATL_WAVES] = acc;
+        }
         ATL_STAMP(9);
-        if (lane == 0) s_red[wave] = acc;
         __syncthreads();
         ATL_STAMP(10);
         const float sum = (((s_red[0] + s_red[1]) + (s_red[2] + s_red[3])) + ((s_red[4] + s_red[5]) + (s_red[6] + s_red[7]))) +
                           (((s_red[8] + s_red[9]) + (s_red[10] + s_red[11])) + ((s_red[12] + s_red[13]) + (s_red[14] + s_red[15])));
         const float scale = 1.0f / sqrtf(sum / (float)d + a.eps);
-        if (tid < d / 4) {
-            float4 v = xv;
-            v.x = (v.x * scale) * wv.x; v.y = (v.y * scale) * wv.y; v.z = (v.z * scale) * wv.z; v.w = (v.w * scale) * wv.w;
-            int2 meta;
-            const uint32_t q = quantize_oct(v, meta);
-            ((uint32_t *)s_q)[act_dw(tid, d >> 6)] = q;
-            if ((tid & 7) == 0) s_meta[tid >> 3] = meta;
+#pragma unroll
+        for (int j = 0; j < ATL_NX; j++) {
+            const int i = tid + j * ATL_THREADS;
+            if (i < d / 4) {
+                float4 v = xv[j];
+                v.x = (v.x * scale) * wv[j].x; v.y = (v.y * scale) * wv[j].y; v.z = (v.z * scale) * wv[j].z; v.w = (v.w * scale) * wv[j].w;
+                int2 meta;
+                const uint32_t q = quantize_oct(v, meta);
+                ((uint32_t *)s_q)[act_dw(i, d >> 6)] = q;
+                if ((i & 7) == 0) s_meta[i >> 3] = meta;
+            }
         }
         __syncthreads();
     }
@@ -433,8 +454,8 @@ __global__ __launch_bounds__(WGV_THREADS) void attn_layer_kernel(attn_layer_args
     }
     ATL_STAMP(2);
     if (!publish_and_sync(sync, [&]() {
-            if (lane < WGV_WAVES) {
-                const int ww = g * WGV_WAVES + lane, pp = ww & 63;
+            if (lane < ATL_WAVES) {
+                const int ww = g * ATL_WAVES + lane, pp = ww & 63;
                 const uint32_t pr = __float_as_uint(s_out[lane * 2]);
                 if (ww < 64) stc((uint32_t *)a.q16 + h * 64 + pp, pr);                                         // attn_score rounds Q to fp16 (mat.cpp:37)
                 else stc((uint32_t *)(a.kc + (size_t)pos * d) + h * 64 + pp, pr);                               // KCache_cpy: [token][head][hd]
@@ -484,14 +505,14 @@ __global__ __launch_bounds__(WGV_THREADS) void attn_layer_kernel(attn_layer_args
     }
     ATL_STAMP(4);
     if (!publish_and_sync(sync + 32, [&]() {
-            for (int idx = lane; idx < WGV_WAVES * 4 * ATL_RS; idx += 64) {
+            for (int idx = lane; idx < ATL_WAVES * 4 * ATL_RS; idx += 64) {
                 const int wv_ = idx / (4 * ATL_RS), r = idx - wv_ * (4 * ATL_RS);
-                const int tok = 4 * (g * WGV_WAVES + wv_ + 128 * (r >> 2)) + (r & 3);
+                const int tok = 4 * (g * ATL_WAVES + wv_ + 128 * (r >> 2)) + (r & 3);
                 if (tok < n_kv) stc(a.scores + (size_t)h * n_ctx + tok, s_out[idx]);
             }
         })) return;
     ATL_STAMP(5);
-    if (g == 0 && tid == 0) sync[64] = target / 8u;                  // every workgroup of the head has read the old count
+    if (g == 0 && tid == 0) sync[64] = target / (uint32_t)ATL_GPH;                  // every workgroup of the head has read the old count
 
     // ================= C: softmax of the head's scores, KQV rows 16 g .. 16 g + 15 ====================
     // m = max t; e = expf(float(fp16(t - m))); p = e * (1/sum e) (non-linear.cpp:158-176); P is rounded
@@ -500,7 +521,7 @@ __global__ __launch_bounds__(WGV_THREADS) void attn_layer_kernel(attn_layer_args
         const float *srow = a.scores + (size_t)h * n_ctx;
         const int n_pad = (n_kv + 7) & ~7;
         float mx = -INFINITY;
-        for (int j = tid; j < n_kv; j += WGV_THREADS) { const float tt = ldc(srow + j); s_t[j] = tt; mx = fmaxf(mx, tt); }
+        for (int j = tid; j < n_kv; j += ATL_THREADS) { const float tt = ldc(srow + j); s_t[j] = tt; mx = fmaxf(mx, tt); }
         if (wave == 0) {
 #pragma unroll
             for (int i = 0; i < ATL_DEPTH_V; i++) fetch_v(i);
@@ -511,18 +532,23 @@ __global__ __launch_bounds__(WGV_THREADS) void attn_layer_kernel(attn_layer_args
         ATL_STAMP(6);
         mx = s_red[0];
 #pragma unroll
-        for (int i = 1; i < WGV_WAVES; i++) mx = fmaxf(mx, s_red[i]);
+        for (int i = 1; i < ATL_WAVES; i++) mx = fmaxf(mx, s_red[i]);
+        __syncthreads();
+        // partial sums per residue class j mod 1024 (thread tid + c * ATL_THREADS of a 1024-thread workgroup), one entry of
+        // s_red per 64 classes: the same additions in the same order whatever the workgroup size
+#pragma unroll
+        for (int c = 0; c < ATL_NX; c++) {
+            float sum = 0.0f;
+            for (int j = tid + c * ATL_THREADS; j < n_kv; j += 1024) { const float e = expf(h2f(f2h(s_t[j] - mx))); s_t[j] = e; sum += e; }
+            sum = group_sum<64>(sum);
+            if (lane == 0) s_red[wave + c * ATL_WAVES] = sum;
+        }
         __syncthreads();
         float sum = 0.0f;
-        for (int j = tid; j < n_kv; j += WGV_THREADS) { const float e = expf(h2f(f2h(s_t[j] - mx))); s_t[j] = e; sum += e; }
-        sum = group_sum<64>(sum);
-        if (lane == 0) s_red[wave] = sum;
-        __syncthreads();
-        sum = 0.0f;
 #pragma unroll
-        for (int i = 0; i < WGV_WAVES; i++) sum += s_red[i];
+        for (int i = 0; i < 16; i++) sum += s_red[i];
         const float inv = 1.0f / sum;
-        for (int j = tid; j < n_pad; j += WGV_THREADS) s_p[j] = j < n_kv ? f2h(s_t[j] * inv) : (uint16_t)0;
+        for (int j = tid; j < n_pad; j += ATL_THREADS) s_p[j] = j < n_kv ? f2h(s_t[j] * inv) : (uint16_t)0;
         __syncthreads();
         ATL_STAMP(7);
         float acc = 0.0f;

@@ -89,14 +89,14 @@ template <int WT, int WTV>
 static int launch_attn_layer_tv(spy_hip_llama *m, hipStream_t st, int il, bool probe) {
     const spy_hip_llama_desc &c = m->desc;
     const spy_hip_llama_layer &L = m->layers[il];
-    const size_t lds = staged_bytes(c.n_embd) + 512 + (size_t)WGV_WAVES * 4 * ATL_RS * 4 + (size_t)c.n_ctx * 6 + 16;
+    const size_t lds = staged_bytes(c.n_embd) + 512 + (size_t)ATL_WAVES * 4 * ATL_RS * 4 + (size_t)c.n_ctx * 6 + 16;
     auto kern = attn_layer_kernel<WT, WTV>;
     static size_t lds_set = 0;
     if (probe || lds > lds_set) {
         if (lds > 48 * 1024 && lds > lds_set) { HIP_TRY(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); lds_set = lds; }
         int per_cu = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, WGV_THREADS, lds) != hipSuccess) per_cu = 0;
-        if (per_cu < 1) return SPY_HIP_EUNSUPPORTED;        // the head barriers need every workgroup resident
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, ATL_THREADS, lds) != hipSuccess) per_cu = 0;
+        if (per_cu * m->num_cu < c.n_head * ATL_GPH) return SPY_HIP_EUNSUPPORTED;        // the head barriers need every workgroup resident
     }
     if (probe || m->dry) return 0;
     attn_layer_args a;
@@ -111,7 +111,7 @@ static int launch_attn_layer_tv(spy_hip_llama *m, hipStream_t st, int il, bool p
 #ifdef ATL_STAMPS
     a.dbg = m->mega_dbg;
 #endif
-    kern<<<dim3((unsigned)(c.n_head * 8)), dim3(WGV_THREADS), lds, st>>>(a);
+    kern<<<dim3((unsigned)(c.n_head * ATL_GPH)), dim3(ATL_THREADS), lds, st>>>(a);
     return SPY_LAUNCH_RC();
 }
 

@@ -136,7 +136,7 @@ extern "C" int spy_hip_llama_create(const spy_hip_llama_desc *desc, spy_hip_llam
         rc = dalloc(m, (void **)&m->mega_layers, ml.size() * sizeof(mega_layer), false);
         if (!rc) rc = (int)hipMemcpy(m->mega_layers, ml.data(), ml.size() * sizeof(mega_layer), hipMemcpyHostToDevice);
         if (!rc) rc = dalloc(m, (void **)&m->msync, sizeof(mega_sync), true);
-        if (!rc && getenv("SPY_HIP_MEGA_STAMPS")) rc = dalloc(m, (void **)&m->mega_dbg, 128 * sizeof(long long), true);
+        if (!rc && getenv("SPY_HIP_MEGA_STAMPS")) rc = dalloc(m, (void **)&m->mega_dbg, (128 + 512 * 8) * sizeof(long long), true);
         const char *env = getenv("SPY_HIP_MEGA");
         if (!rc && env && env[0] == '1' && m->uniform)
             m->mega = (c.wtype == SPY_HIP_Q4_0 ? spy_enqueue_mega_q4_0(m, m->own_stream, true) : spy_enqueue_mega_q8_0(m, m->own_stream, true)) == 0;
@@ -157,7 +157,7 @@ extern "C" int spy_hip_llama_buffer(spy_hip_llama *m, const char *name, int32_t 
     else if (!strcmp(name, "logits")) { p = m->logits; n = (size_t)m->desc.n_vocab * 4; }
     else if (!strcmp(name, "scores")) { p = m->scores; n = (size_t)m->desc.n_head * C * 4; }
     else if (!strcmp(name, "attn_out")) { p = m->attn_out; n = d * 4; }
-    else if (!strcmp(name, "phase_stamps") && m->mega_dbg) { p = m->mega_dbg; n = 128 * sizeof(long long); }
+    else if (!strcmp(name, "phase_stamps") && m->mega_dbg) { p = m->mega_dbg; n = (128 + 512 * 8) * sizeof(long long); }
     else return SPY_HIP_EINVAL;
     *ptr = p;
     if (bytes) *bytes = n;
