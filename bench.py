@@ -37,6 +37,8 @@ def main():
     ap.add_argument("--layers", type=int, default=32, help="debug only: fewer layers (result is then not the headline config)")
     ap.add_argument("--model", choices=["q4_0", "q8_0", "q4_k_m"], default="q4_0",
                     help="q4_0: the headline workload; q8_0 / q4_k_m (Q4_K with Q6_K attn_v, ffn_down and head): the other 7B configurations")
+    ap.add_argument("--head", choices=["q6_k", "body"], default="q6_k",
+                    help="--model q4_0 only: output head in Q6_K (the named configuration; default) or in the body's Q4_0 (the variant Spy's CPU backend can run)")
     ap.add_argument("--via-gguf", metavar="PATH", default=None,
                     help="write the synthetic model to PATH as a GGUF file and run the model loaded from it (file -> HBM times are reported)")
     ap.add_argument("--no-graph", action="store_true", help="launch the kernels of every pass one by one instead of replaying a HIP graph (for profilers)")
@@ -58,7 +60,7 @@ def main():
     steps, warmup, fill = args.steps, args.warmup, args.ctx_fill
     n_ctx = (fill + warmup + steps + 8 + 7) // 8 * 8
     if args.model == "q4_0":
-        cfg = M.Config.llama2_7b(n_ctx=n_ctx, wtype=H.Q4_0)
+        cfg = M.Config.llama2_7b(n_ctx=n_ctx, wtype=H.Q4_0, t_out=H.Q4_0 if args.head == "body" else H.Q6_K)
     elif args.model == "q8_0":
         cfg = M.Config.llama2_7b(n_ctx=n_ctx, wtype=H.Q8_0)
     else:
@@ -66,7 +68,7 @@ def main():
     cfg.n_layer = args.layers
     t0 = time.time()
     # K-quant matrices: random well-formed blocks (this package has no K-quant quantizer; timing only)
-    tensors = M.synth_model(cfg, seed=1234, quantizer=M.random_k_blocks if args.model == "q4_k_m" else None)
+    tensors = M.synth_model(cfg, seed=1234, quantizer=M.random_k_blocks)
     log("synthetic model: %.1f s, %.2f GB of weights streamed per token" % (time.time() - t0, cfg.weight_bytes() / 1e9))
     load_info, loaded = None, None
     if args.via_gguf:
@@ -177,7 +179,7 @@ def main():
                "sample": "%d single-token passes of the same model at n_kv = %d.. (AVX2 port of Spy's host backend, OpenMP)" % (args.cpu_steps, fill + 1)}
         log("cpu baseline: %.3f tok/s on %d threads" % (cpu["value"], ncpu))
 
-    weights_desc = {"q4_0": "Q4_0 weights incl. head", "q8_0": "Q8_0 weights incl. head",
+    weights_desc = {"q4_0": "Q4_0 weights, output head Q6_K (random well-formed blocks)" if cfg.t_out == H.Q6_K else "Q4_0 weights incl. head", "q8_0": "Q8_0 weights incl. head",
                     "q4_k_m": "Q4_K weights with Q6_K attn_v / ffn_down / head (random blocks)"}[args.model]
     out = {
         "metric": "decode tok/s + %% HBM roofline, LLaMA-2-7B %s ctx 4096, 1xMI355X" % {"q4_0": "Q4_0", "q8_0": "Q8_0", "q4_k_m": "Q4_K_M"}[args.model],

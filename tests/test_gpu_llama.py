@@ -183,6 +183,7 @@ def test_llama2_7b_q4_0_greedy_32_tokens():
 
 
 @pytest.mark.parametrize("name,kw", [
+    ("Q4_0 body, Q6_K head", dict(wtype=O.Q4_0, t_out=O.Q6_K)),
     ("Q4_K + Q6_K head", dict(wtype=O.Q4_K, t_out=O.Q6_K)),
     ("Q6_K", dict(wtype=O.Q6_K)),
     ("Q4_K_M mix", dict(wtype=O.Q4_K, t_out=O.Q6_K, tensor_types={"attn_v": O.Q6_K, "ffn_down": O.Q6_K})),
