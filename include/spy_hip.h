@@ -85,7 +85,9 @@ int spy_hip_op_binary(void *stream, int op, const spy_hip_tensor *a, const spy_h
 /* Silu -- OperatorSiluImpl::execute (non-linear.cpp:57-77) */
 int spy_hip_op_silu(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *dst);
 /* Softmax -- OperatorSoftmaxImpl::execute (non-linear.cpp:86-185); mask may be NULL;
- * scale = SoftmaxParam::scale */
+ * scale = SoftmaxParam::scale.  dst may also be FP16 (rows of up to 16384 elements, scale > 0): the
+ * probabilities rounded the way the KQV MatMul rounds its right operand first (mat.cpp:37), so that the
+ * product can take them without a conversion pass */
 int spy_hip_op_softmax(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *mask, const spy_hip_tensor *dst, float scale);
 /* Rope -- OperatorRopeImpl::execute (non-linear.cpp:270-371); fields of RopeParam
  * (orchestration/include/operator/non-linear.h:191-207).  Supported: mode None/Norm (-1/0) with

@@ -40,7 +40,10 @@ static inline __host__ __device__ int64_t spy_row_size(int t, int64_t n) { retur
 
 // fp16 <-> fp32: IEEE round-to-nearest-even narrowing (v_cvt_f16_f32) and exact widening.
 static __device__ __forceinline__ float h2f(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
-static __device__ __forceinline__ uint16_t f2h(float f) { return __builtin_bit_cast(uint16_t, (_Float16)f); }
+// The empty asm keeps the operand a finished fp32 value: without it the compiler folds a preceding multiply or add
+// into v_fma_mixlo_f16, which rounds once (straight to fp16) where the reference rounds twice (fp32, then fp16) --
+// a different result whenever the fp32 rounding lands on an fp16 tie.
+static __device__ __forceinline__ uint16_t f2h(float f) { asm("" : "+v"(f)); return __builtin_bit_cast(uint16_t, (_Float16)f); }
 
 static __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

@@ -329,7 +329,11 @@ static int forward_ops(spy_hip_llama *m, hipStream_t st, const int32_t *tokens_h
         RC_TRY(spy_hip_op_dup(st, &t_vt, &t_vc));
         spy_hip_tensor t_kall = T3s(SPY_HIP_F16, m->k_cache[il], hd, n_kv, H, 2, 2 * d, 2 * hd);
         spy_hip_tensor t_vall = T3s(SPY_HIP_F16, m->v_cache[il], n_kv, hd, H, 2, 2 * C, 2 * C * hd);
-        spy_hip_tensor t_S = T3s(SPY_HIP_F32, S, n_kv, T, H, 4, 4 * n_kv, 4 * n_kv * T), t_P = T3s(SPY_HIP_F32, Pm, n_kv, T, H, 4, 4 * n_kv, 4 * n_kv * T);
+        // the probabilities go to the KQV product as fp16 (its first step, mat.cpp:37): the softmax writes them that way
+        // directly where the fp16 GEMM takes them (rows of a multiple of 8 elements)
+        const bool p16 = n_kv % 8 == 0 && n_kv <= 16384 && T >= 16;
+        spy_hip_tensor t_S = T3s(SPY_HIP_F32, S, n_kv, T, H, 4, 4 * n_kv, 4 * n_kv * T);
+        spy_hip_tensor t_P = p16 ? T3s(SPY_HIP_F16, Pm, n_kv, T, H, 2, 2 * n_kv, 2 * n_kv * T) : T3s(SPY_HIP_F32, Pm, n_kv, T, H, 4, 4 * n_kv, 4 * n_kv * T);
         RC_TRY(spy_hip_op_matmul(st, &t_kall, &t_qp, &t_S, scr, scr_bytes));
         RC_TRY(spy_hip_op_softmax(st, &t_S, &t_mask, &t_P, scale));
         spy_hip_tensor t_O = T3s(SPY_HIP_F32, o, hd, T, H, 4, 4 * hd, 4 * hd * T);

@@ -3,6 +3,7 @@
 // stride-honouring forms that a per-operator submit() uses; the fused token loop has its own
 // specialised kernels.
 #include "common.cuh"
+#include <stdlib.h>
 
 #include <math.h>
 
@@ -164,10 +165,53 @@ __global__ __launch_bounds__(256) void softmax_kernel(tdesc x, tdesc mask, bool 
     for (int64_t i = threadIdx.x; i < ne0; i += 256) d[i] *= inv;
 }
 
+// The same arithmetic with the row kept in LDS between the passes (one read of the scores, one write of the
+// probabilities) for rows of up to SOFTMAX_LDS_ROW elements; the additions of the sum happen in the same order
+// as above (thread stride 256, then the same tree), so both kernels give the same bits.  Masked elements
+// (mask = -inf, scale > 0) are not read: (s - inf) * scale = -inf whatever the finite score.  F16OUT stores the
+// probabilities rounded to fp16, which is what the KQV product does to them first anyway (mat.cpp:37).
+#define SOFTMAX_LDS_ROW 16384
+template <bool F16OUT>
+__global__ __launch_bounds__(256) void softmax_row_kernel(tdesc x, tdesc mask, bool has_mask, tdesc y, float scale) {
+    extern __shared__ __attribute__((aligned(16))) float s_row[];
+    __shared__ float s_part[4];
+    const int64_t r = blockIdx.x;
+    const int ne0 = (int)y.ne[0];
+    const int64_t ne1 = y.ne[1], ne2 = y.ne[2];
+    const int64_t i3 = r / (ne1 * ne2), i2 = r % (ne1 * ne2) / ne1, i1 = r % ne1;
+    const float *s = (const float *)at(x, 0, i1, i2, i3);
+    const float *mk_ = has_mask ? (const float *)at(mask, 0, i1, 0, 0) : nullptr;
+    float mx = -INFINITY;
+    for (int i = threadIdx.x; i < ne0; i += 256) {
+        float t;
+        if (has_mask) { const float mv = mk_[i]; t = (mv == -INFINITY) ? -INFINITY : (s[i] + mv) * scale; }
+        else t = s[i] * scale;
+        s_row[i] = t;
+        mx = fmaxf(mx, t);
+    }
+    mx = block_reduce_256(mx, true, s_part);
+    float sum = 0.0f;
+    for (int i = threadIdx.x; i < ne0; i += 256) {
+        const float t = s_row[i];
+        const float e = (has_mask && t == -INFINITY) ? 0.0f : expf(h2f(f2h(t - mx)));
+        s_row[i] = e;
+        sum += e;
+    }
+    sum = block_reduce_256(sum, false, s_part);
+    const float inv = 1.0f / sum;
+    if constexpr (F16OUT) {
+        uint16_t *d = (uint16_t *)at(y, 0, i1, i2, i3);
+        for (int i = threadIdx.x; i < ne0; i += 256) d[i] = f2h(s_row[i] * inv);
+    } else {
+        float *d = (float *)at(y, 0, i1, i2, i3);
+        for (int i = threadIdx.x; i < ne0; i += 256) d[i] = s_row[i] * inv;
+    }
+}
+
 extern "C" int spy_hip_op_softmax(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *mask, const spy_hip_tensor *dst, float scale) {
     SPY_CHECK_ARG(x && dst && x->data && dst->data);
-    if (x->type != SPY_HIP_F32 || dst->type != SPY_HIP_F32) return SPY_HIP_EUNSUPPORTED;
-    SPY_CHECK_ARG(same_ne(x, dst) && x->nb[0] == 4 && dst->nb[0] == 4);
+    if (x->type != SPY_HIP_F32 || (dst->type != SPY_HIP_F32 && dst->type != SPY_HIP_F16)) return SPY_HIP_EUNSUPPORTED;
+    SPY_CHECK_ARG(same_ne(x, dst) && x->nb[0] == 4 && dst->nb[0] == (dst->type == SPY_HIP_F16 ? 2 : 4));
     tdesc m = mk(x);
     if (mask) {
         // the mask is typed INT32 by the graph (inout.cpp:43-47) but read as float (non-linear.cpp:147)
@@ -176,6 +220,23 @@ extern "C" int spy_hip_op_softmax(void *stream, const spy_hip_tensor *x, const s
     }
     const int64_t nrow = spy_t_nrow(dst);
     CHECK_GRID(nrow, 1);
+    // a masked element of the generic kernel reads as (s + mask) * scale: the row kernel's shortcut needs scale > 0 and a
+    // mask that really is 0 / -inf, which is what the graph builds (llama.cpp:248-263)
+    const bool row_ok = dst->ne[0] <= SOFTMAX_LDS_ROW && scale > 0.0f && !getenv("SPY_HIP_SOFTMAX_GENERIC");
+    if (dst->type == SPY_HIP_F16 && !row_ok) return SPY_HIP_EUNSUPPORTED;
+    if (row_ok) {
+        const size_t lds = (size_t)dst->ne[0] * 4;
+        static size_t lds_set = 0;
+        if (lds > 48 * 1024 && lds > lds_set) {
+            hipError_t e1_ = hipFuncSetAttribute((const void *)softmax_row_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, SOFTMAX_LDS_ROW * 4);
+            hipError_t e2_ = hipFuncSetAttribute((const void *)softmax_row_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, SOFTMAX_LDS_ROW * 4);
+            if (e1_ != hipSuccess || e2_ != hipSuccess) return (int)(e1_ != hipSuccess ? e1_ : e2_);
+            lds_set = SOFTMAX_LDS_ROW * 4;
+        }
+        if (dst->type == SPY_HIP_F16) softmax_row_kernel<true><<<dim3((unsigned)nrow), dim3(256), lds, (hipStream_t)stream>>>(mk(x), m, mask != nullptr, mk(dst), scale);
+        else softmax_row_kernel<false><<<dim3((unsigned)nrow), dim3(256), lds, (hipStream_t)stream>>>(mk(x), m, mask != nullptr, mk(dst), scale);
+        return SPY_LAUNCH_RC();
+    }
     softmax_kernel<<<dim3((unsigned)nrow), dim3(256), 0, (hipStream_t)stream>>>(mk(x), m, mask != nullptr, mk(dst), scale);
     return SPY_LAUNCH_RC();
 }
@@ -393,6 +454,19 @@ static int mid_type(int t0, int t1) {                                        // 
     return t0;
 }
 
+// f32 [ne10, ne11, batches] with byte strides -> contiguous fp16, 4 elements per thread; blockIdx.y = batch
+__global__ __launch_bounds__(256) void to_f16_batched_kernel(const uint8_t *__restrict__ x, int64_t nb1, int64_t nb2, int64_t nb3,
+                                                              uint16_t *__restrict__ y, int64_t ne10, int64_t ne11, int64_t ne12) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x, q = ne10 / 4;
+    if (i >= q * ne11) return;
+    const int64_t row = i / q, c = i - row * q, b = blockIdx.y, i12 = b % ne12, i13 = b / ne12;
+    const float4 v = *(const float4 *)(x + i13 * nb3 + i12 * nb2 + row * nb1 + c * 16);
+    uint2 o;
+    o.x = (uint32_t)f2h(v.x) | ((uint32_t)f2h(v.y) << 16);
+    o.y = (uint32_t)f2h(v.z) | ((uint32_t)f2h(v.w) << 16);
+    *(uint2 *)(y + (b * ne11 + row) * ne10 + c * 4) = o;
+}
+
 extern "C" size_t spy_hip_op_matmul_scratch_size(const spy_hip_tensor *w, const spy_hip_tensor *x) {
     if (!w || !x) return 0;
     const int tm = mid_type(w->type, x->type);
@@ -425,6 +499,13 @@ extern "C" int spy_hip_op_matmul(void *stream, const spy_hip_tensor *w, const sp
         const size_t need = (size_t)(spy_t_nrow(x) * mid_row);
         if (!scratch || scratch_bytes < need) return SPY_HIP_ENOSPACE;
         SPY_CHECK_ARG(x->nb[0] == 4);
+        if (tm == SPY_HIP_F16 && ne12 * ne13 > 1 && ne12 * ne13 <= 65535 && ne10 % 4 == 0 && x->nb[1] % 16 == 0 && x->nb[2] % 16 == 0 &&
+            x->nb[3] % 16 == 0 && ((uintptr_t)x->data & 15) == 0 && ne10 * ne11 / 4 < (1ll << 31) * 256) {
+            // all batches (heads) in one launch
+            to_f16_batched_kernel<<<dim3((unsigned)((ne10 / 4 * ne11 + 255) / 256), (unsigned)(ne12 * ne13)), dim3(256), 0, st>>>(
+                (const uint8_t *)x->data, x->nb[1], x->nb[2], x->nb[3], (uint16_t *)scratch, ne10, ne11, ne12);
+            if (hipGetLastError() != hipSuccess) return SPY_HIP_EINVAL;
+        } else
         for (int64_t i13 = 0; i13 < ne13; i13++)
             for (int64_t i12 = 0; i12 < ne12; i12++) {
                 const float *src = (const float *)((const uint8_t *)x->data + i12 * x->nb[2] + i13 * x->nb[3]);

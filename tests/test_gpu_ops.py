@@ -91,6 +91,41 @@ def test_masked_softmax(hip, oracle):
     assert_close(dd.download(np.float32).reshape(s.shape), want, "softmax unmasked", tol=1e-5)
 
 
+def test_softmax_row_kernel_and_fp16_output(hip, oracle):
+    """The kernel that keeps a row in LDS gives the bits of the three-pass kernel (same additions in the same
+    order), with and without a causal mask; the fp16 output is the fp32 output rounded to nearest even, which is
+    what the KQV product does to it first (mat.cpp:37 in the Spy tree)."""
+    import os
+    from tests.gpu_util import dev, dev_empty, call
+    rng = np.random.default_rng(12)
+    scale = 0.0883883461356163
+    L = hip.load()
+    for (H_, T, n_kv, Cx, P) in [(4, 24, 40, 64, 16), (2, 5, 1000, 1024, 995), (1, 3, 4104, 4352, 4101)]:
+        s = (rng.standard_normal((H_, T, n_kv)) * 4).astype(np.float32)
+        mask = np.where(np.arange(Cx)[None, :] <= (np.arange(T)[:, None] + P), 0.0, -np.inf).astype(np.float32)
+        ds, dm = dev(s), dev(mask.view(np.int32))
+        outs = {}
+        for name, use_mask in (("masked", True), ("plain", False)):
+            tm = B(hip.tensor(dm, hip.I32, [Cx, T])) if use_mask else None
+            os.environ["SPY_HIP_SOFTMAX_GENERIC"] = "1"
+            try:
+                dg = dev_empty(s.nbytes, 0xFF)
+                call(L.spy_hip_op_softmax, None, B(hip.tensor(ds, hip.F32, [n_kv, T, H_])), tm, B(hip.tensor(dg, hip.F32, [n_kv, T, H_])), scale)
+                hip.sync()
+            finally:
+                del os.environ["SPY_HIP_SOFTMAX_GENERIC"]
+            dr, dh = dev_empty(s.nbytes, 0xFF), dev_empty(s.nbytes // 2, 0xFF)
+            call(L.spy_hip_op_softmax, None, B(hip.tensor(ds, hip.F32, [n_kv, T, H_])), tm, B(hip.tensor(dr, hip.F32, [n_kv, T, H_])), scale)
+            call(L.spy_hip_op_softmax, None, B(hip.tensor(ds, hip.F32, [n_kv, T, H_])), tm, B(hip.tensor(dh, hip.F16, [n_kv, T, H_])), scale)
+            generic, row, half = dg.download(np.float32), dr.download(np.float32), dh.download(np.float16)
+            assert np.array_equal(generic.view(np.uint32), row.view(np.uint32)), (name, H_, T, n_kv)
+            assert np.array_equal(half.view(np.uint16), row.astype(np.float16).view(np.uint16)), (name, H_, T, n_kv)
+            outs[name] = row
+        want = np.zeros_like(s)
+        assert oracle.spy_o_softmax(B(O.tensor(s, O.F32, [n_kv, T, H_])), B(O.tensor(mask.view(np.int32), O.I32, [Cx, T])), B(O.tensor(want, O.F32, [n_kv, T, H_])), scale) == 0
+        assert float(np.abs(outs["masked"].reshape(want.shape) - want).max()) < 1e-5
+
+
 def test_rope(hip, oracle):
     from tests.gpu_util import dev, dev_empty, call, assert_close
     rng = np.random.default_rng(5)
