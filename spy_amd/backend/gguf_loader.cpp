@@ -63,6 +63,17 @@ struct TensorInfo {
 
 }  // namespace
 
+// the same for the other sources of this library (tokenizer.cpp)
+int spy_gguf_fail(int code, const char *fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    g_error = buf;
+    return code;
+}
+
 struct spy_gguf {
     int fd = -1;
     const uint8_t *base = nullptr;

@@ -241,7 +241,24 @@ class GGUFModel:
         eng.close = lambda: None                                 # the loaded model owns the token loop
         self.engine = eng
 
+    @property
+    def vocab(self):
+        """SentencePiece vocabulary of the file (built on first use)."""
+        if getattr(self, "_vocab", None) is None:
+            self._vocab = Vocab(self.file)
+        return self._vocab
+
+    def generate_text(self, prompt, n_predict):
+        """What AutoModelGenerator::generate does with a prompt (app/cli/include/cli.h:60-129 in the Spy tree):
+        tokenize(prompt, bos = true, special = false), prompt pass, greedy loop; returns (ids, text of the new tokens)."""
+        ids = self.vocab.tokenize(prompt, add_bos=True, special=False)
+        new = self.engine.generate(np.asarray(ids, dtype=np.int32), n_predict)
+        return [int(t) for t in new], self.vocab.detokenize([int(t) for t in new])
+
     def close(self):
+        if getattr(self, "_vocab", None) is not None:
+            self._vocab.close()
+            self._vocab = None
         if getattr(self, "h", None):
             self.engine.handle = None
             self.L.spy_gguf_model_free(self.h)
@@ -252,3 +269,79 @@ class GGUFModel:
             self.close()
         except Exception:
             pass
+
+
+# ---- SentencePiece vocabulary (include/spy_vocab.h) --------------------------------------------------
+VOCAB_SIGNATURES = {
+    "spy_vocab_from_gguf": (C.c_int, [_vp, _P(_vp)]),
+    "spy_vocab_free": (None, [_vp]),
+    "spy_vocab_size": (_i32, [_vp]),
+    "spy_vocab_special_ids": (C.c_int, [_vp, _P(_i32), _P(_i32), _P(_i32), _P(_i32), _P(_i32), _P(_i32)]),
+    "spy_vocab_token": (C.c_int, [_vp, _i32, _P(_vp), _P(_u64), _P(C.c_float), _P(_i32)]),
+    "spy_vocab_tokenize": (_i64, [_vp, C.c_char_p, _u64, _i32, _i32, _P(_i32), _u64]),
+    "spy_vocab_token_to_piece": (_i64, [_vp, _i32, C.c_char_p, _u64]),
+    "spy_vocab_detokenize": (_i64, [_vp, _P(_i32), _u64, C.c_char_p, _u64]),
+}
+
+
+class Vocab:
+    """SentencePiece vocabulary of a GGUF file: tokenize / detokenize as spy::SentencePieceVocab does."""
+
+    def __init__(self, gguf_file):
+        self.L = load()
+        for name, (res, args) in VOCAB_SIGNATURES.items():
+            fn = getattr(self.L, name)
+            fn.restype, fn.argtypes = res, args
+        h = _vp()
+        _check(self.L.spy_vocab_from_gguf(gguf_file.h, C.byref(h)), "spy_vocab_from_gguf")
+        self.h = h.value
+
+    def close(self):
+        if getattr(self, "h", None):
+            self.L.spy_vocab_free(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def __len__(self):
+        return self.L.spy_vocab_size(self.h)
+
+    def special_ids(self):
+        v = [_i32() for _ in range(6)]
+        _check(self.L.spy_vocab_special_ids(self.h, *v), "spy_vocab_special_ids")
+        return dict(zip(("bos", "eos", "unk", "sep", "pad", "linefeed"), (x.value for x in v)))
+
+    def token(self, i):
+        p, n, s, t = _vp(), _u64(), C.c_float(), _i32()
+        _check(self.L.spy_vocab_token(self.h, i, p, n, s, t), "spy_vocab_token(%d)" % i)
+        return C.string_at(p.value, n.value), s.value, t.value
+
+    def tokenize(self, text, add_bos=True, special=False):
+        raw = text if isinstance(text, bytes) else text.encode("utf-8")
+        cap = 3 * len(raw) + 8
+        ids = (_i32 * cap)()
+        n = self.L.spy_vocab_tokenize(self.h, raw, len(raw), int(add_bos), int(special), ids, cap)
+        if n < 0:
+            raise GGUFError(int(n), "spy_vocab_tokenize")
+        return list(ids[:n])
+
+    def piece(self, i):
+        buf = C.create_string_buffer(256)
+        n = self.L.spy_vocab_token_to_piece(self.h, i, buf, 256)
+        return buf.raw[:n]
+
+    def detokenize(self, ids):
+        arr = (_i32 * max(len(ids), 1))(*ids)
+        cap = 64 + 16 * len(ids)
+        while True:
+            buf = C.create_string_buffer(cap)
+            n = self.L.spy_vocab_detokenize(self.h, arr, len(ids), buf, cap)
+            if n < 0:
+                raise GGUFError(int(n), "spy_vocab_detokenize")
+            if n <= cap:
+                return buf.raw[:n]
+            cap = int(n)

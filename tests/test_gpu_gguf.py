@@ -54,3 +54,28 @@ def test_context_argument_and_reload(tmp_path):
     t = np.array([3, 1, 4, 1, 5], np.int32)
     assert np.array_equal(m0.engine.forward(t, 0), m1.engine.forward(t, 0))
     m0.close(); m1.close()
+
+
+def test_text_in_text_out(tmp_path, capsys):
+    """Prompt text -> SentencePiece ids -> prompt pass + greedy loop -> text, and the command line around it."""
+    from spy_amd import cli, gguf as G, model as M
+    cfg = M.Config(n_layer=2, n_embd=256, n_head=2, n_ff=512, n_vocab=3 + 256 + 40, n_ctx=64, wtype=2)
+    tensors = M.synth_model(cfg, seed=9)
+    words = ["▁", "a", "b", "c", "d", "e", "t", "h", "▁t", "he", "▁the", "▁a", "at", "▁c", "▁cat", "ca", "▁s", "sa", "s"]
+    toks = ["<unk>", "<s>", "</s>"] + ["<0x%02X>" % b for b in range(256)] + words + ["<pad%d>" % i for i in range(40 - len(words))]
+    kv = G.llama_kv(cfg, toks) + [("tokenizer.ggml.scores", G.ARRAY, (G.F32, [0.0] * 259 + [-float(i) for i in range(40)])),
+                                  ("tokenizer.ggml.token_type", G.ARRAY, (G.I32, [2, 3, 3] + [6] * 256 + [1] * 40))]
+    infos = [(n, t, [c] if r == 1 else [c, r], tensors[n]) for n, (t, r, c) in cfg.tensor_shapes().items()]
+    path = G.write_gguf(str(tmp_path / "t.gguf"), kv, infos)
+    m = G.GGUFModel(path)
+    ids = m.vocab.tokenize("the cat sat")
+    assert ids[0] == 1 and m.vocab.detokenize(ids) == b" the cat sat"
+    new, text = m.generate_text("the cat sat", 8)
+    direct = M.Engine(cfg, tensors)
+    want = direct.generate(np.asarray(ids, np.int32), 8)
+    assert new == [int(t) for t in want] and text == m.vocab.detokenize(new)
+    direct.close()
+    m.close()
+    cli.main([path, "-p", "the cat sat", "-n", "8"])
+    out = capsys.readouterr()
+    assert out.out == "the cat sat" + text.decode("utf-8", "replace") + "\n" and "generation: 8 tokens" in out.err
