@@ -189,20 +189,23 @@ __global__ __launch_bounds__(WGV_THREADS) void wave_gemv_kernel(fused_args a) {
     // unit's vector-memory queue is finite, and a wave that tries to put all its rows in flight at
     // once sits in the issue stage until the queue drains (most of the kernel), holding up the staging
     // barriers of everybody else.
-    wtile<WT, NITK> t[NB];
+    // Row k lives in slot k % RING: the slot is free again by the time row k + RING is requested (rows up to k + RING - DEPTH - 1
+    // have been multiplied by then), so the registers hold DEPTH + 1 rows whatever the number of rows per wave.
+    constexpr int RING = NB < DEPTH + 1 ? NB : DEPTH + 1;
+    wtile<WT, NITK> t[RING];
     wtile<WTV, NITK> tv;
     auto issue = [&](int k) {
         if constexpr (EPI == EPI_QKV) {
             const int j = gw % a.d;
             const uint8_t *p0 = 2 * j < a.d ? a.W0 + (size_t)(2 * j) * RB : a.W1 + (size_t)(2 * j - a.d) * RB;
             if (k == 2) load_tile<WTV, 64, NITK>(tv, a.W2 + (size_t)j * spy_row_size(WTV, K), npair, lane);
-            else load_tile<WT, 64, NITK>(t[k], p0 + (size_t)k * RB, npair, lane);
+            else load_tile<WT, 64, NITK>(t[k % RING], p0 + (size_t)k * RB, npair, lane);
         } else if constexpr (EPI == EPI_GATEUP) {
             const int F = a.M / 2, u = gw + (k >> 1) * NW, i = u < F ? u : gw % F;
-            load_tile<WT, 64, NITK>(t[k], ((k & 1) ? a.W1 : a.W0) + (size_t)i * RB, npair, lane);
+            load_tile<WT, 64, NITK>(t[k % RING], ((k & 1) ? a.W1 : a.W0) + (size_t)i * RB, npair, lane);
         } else {
             const int u = gw + k * NW, r = u < a.M ? u : gw % a.M;
-            load_tile<WT, 64, NITK>(t[k], a.W0 + (size_t)r * RB, npair, lane);
+            load_tile<WT, 64, NITK>(t[k % RING], a.W0 + (size_t)r * RB, npair, lane);
             if constexpr (EPI == EPI_RESID) side[k] = a.resid[r];
         }
     };
@@ -249,11 +252,12 @@ __global__ __launch_bounds__(WGV_THREADS) void wave_gemv_kernel(fused_args a) {
     float s[NB];
 #pragma unroll
     for (int k = 0; k < NB; k++) {
+        if constexpr (NB > DEPTH + 1) __builtin_amdgcn_sched_barrier(0);     // keep the requests where they are: hoisted, they would need more than the ring
         if (k + DEPTH < NB) issue(k + DEPTH);
         if (EPI == EPI_QKV && k == 2) {
             if constexpr (WTV == WT) s[k] = dot_row_frag<WTV, NITK>(tv, af, npair, lane);
             else { act_frag<NITK> av; load_act_frag<WTV, NITK>(av, act, npair, lane); s[k] = dot_row_frag<WTV, NITK>(tv, av, npair, lane); }
-        } else s[k] = dot_row_frag<WT, NITK>(t[k], af, npair, lane);
+        } else s[k] = dot_row_frag<WT, NITK>(t[k % RING], af, npair, lane);
     }
 #pragma unroll
     for (int k = 0; k < NB; k++) s[k] = wave_total_lane63(s[k]);

@@ -66,9 +66,11 @@ static int launch_wave(spy_hip_llama *m, hipStream_t st, const fused_args &a) {
     kern<<<dim3((unsigned)grid), dim3(WGV_THREADS), lds, st>>>(a);
     return SPY_LAUNCH_RC();
 }
-// rows (head) and row pairs (gate|up) per wave: bounded by the row registers, PAIR_DW dwords per row
+// rows (head) and row pairs (gate|up) per wave.  The kernel keeps a ring of DEPTH + 1 rows in registers; 8 rows per wave give
+// 250 workgroups for 32000 rows, one per compute unit.  The wide rows of Q8_0 / Q6_K (17 / 15 dwords per lane) stay at 4:
+// with 8 the kernel spills a dozen registers and measured 24.3 instead of 21.5 us (Q6_K), 27.3 instead of 20.8 us (Q8_0)
 template <int WT> struct wave_rows {
-    static constexpr int HEAD = WT == SPY_HIP_Q4_0 ? 8 : (WT == SPY_HIP_Q4_K ? 6 : 4);
+    static constexpr int HEAD = (WT == SPY_HIP_Q4_0 || WT == SPY_HIP_Q4_K) ? 8 : 4;
     static constexpr int GATEUP = (WT == SPY_HIP_Q4_0 || WT == SPY_HIP_Q4_K) ? 3 : 2;
 };
 static inline int layer_type(const spy_hip_llama *m, int t) { return t ? t : m->desc.wtype; }
