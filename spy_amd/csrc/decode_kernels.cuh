@@ -747,15 +747,36 @@ __global__ __launch_bounds__(PV_THREADS) void attn_pv_kernel(const dev_state *st
 // ---- greedy sampling + loop advance -------------------------------------------------------------
 // argmax with std::max_element's first-maximum rule (greedy.h:20-25), then the loop step of
 // AutoModelGenerator::generate (cli.h:121-123): the sampled token becomes the next input at pos+1.
+// With `table` != nullptr the kernel goes on to what the next pass starts with: the embedding row of the sampled
+// token and the RoPE table of the next position (embed_kernel's work), so that a greedy step is one launch shorter.
 __global__ __launch_bounds__(1024) void sample_advance_kernel(dev_state *st, const float *__restrict__ logits, int n, int32_t *__restrict__ tokens_out,
-                                                              int max_out) {
+                                                              int max_out, const uint8_t *__restrict__ table, int q8, int d, float *__restrict__ x,
+                                                              float *__restrict__ rope_cs, float theta_scale, int hd) {
     __shared__ float s_v[16];
     __shared__ int s_i[16];
+    __shared__ int s_next[1];
     float best = -INFINITY;
     int bi = 0x7fffffff;
-    for (int i = threadIdx.x; i < n; i += 1024) {
-        const float v = logits[i];
-        if (v > best || (bi == 0x7fffffff && !(v < best))) { best = v; bi = i; }
+    const int step = st->step, pos = st->pos + 1;
+    // 16 logits per thread requested together (one at a time, the loop is 32 memory round trips long)
+    for (int base = 0; base < n; base += 16 * 1024) {
+        float v[16];
+#pragma unroll
+        for (int u = 0; u < 16; u++) v[u] = logits[min(base + (int)threadIdx.x + u * 1024, n - 1)];
+#pragma unroll
+        for (int u = 0; u < 16; u++) {
+            const int i = base + (int)threadIdx.x + u * 1024;
+            if (i < n && (v[u] > best || (bi == 0x7fffffff && !(v[u] < best)))) { best = v[u]; bi = i; }
+        }
+    }
+    if (table != nullptr) {
+        // the RoPE table of the next position does not depend on the token: computed while the maximum is being reduced
+        for (int k = threadIdx.x; k < hd / 2; k += 1024) {
+            float theta = (float)pos;
+            for (int j = 0; j < k; j++) theta *= theta_scale;
+            rope_cs[2 * k] = cosf(theta);
+            rope_cs[2 * k + 1] = sinf(theta);
+        }
     }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {
@@ -768,11 +789,21 @@ __global__ __launch_bounds__(1024) void sample_advance_kernel(dev_state *st, con
     if (threadIdx.x == 0) {
         for (int w = 1; w < 16; w++) if (s_v[w] > best || (s_v[w] == best && s_i[w] < bi)) { best = s_v[w]; bi = s_i[w]; }
         if (bi == 0x7fffffff) bi = 0;
-        const int step = st->step;
         if (step < max_out) tokens_out[step] = bi;
         st->token = bi;
-        st->pos = st->pos + 1;
+        st->pos = pos;
         st->step = step + 1;
+        s_next[0] = bi;
+    }
+    if (table == nullptr) return;
+    __syncthreads();
+    const int tok = s_next[0];                 // an index of the logits: always a valid row
+    if (!q8) {
+        const float *row = (const float *)table + (size_t)tok * d;
+        for (int i = threadIdx.x; i < d; i += 1024) x[i] = row[i];
+    } else {
+        const blk_q8_0 *row = (const blk_q8_0 *)(table + (size_t)tok * (d / 32) * 34);
+        for (int i = threadIdx.x; i < d; i += 1024) x[i] = (float)row[i >> 5].qs[i & 31] * h2f(row[i >> 5].d);
     }
 }
 

@@ -23,7 +23,8 @@ static int probe_attn(spy_hip_llama *m, int il) {
     }
     return SPY_HIP_EUNSUPPORTED;
 }
-static int enqueue_pass_any(spy_hip_llama *m, hipStream_t st, bool sample);
+enum { PASS_LOGITS = 0, PASS_GREEDY = 1 };
+static int enqueue_pass_any(spy_hip_llama *m, hipStream_t st, int mode);
 
 static int dalloc(spy_hip_llama *m, void **p, size_t bytes, bool zero) {
     HIP_TRY(hipMalloc(p, bytes));
@@ -124,7 +125,7 @@ extern "C" int spy_hip_llama_create(const spy_hip_llama_desc *desc, spy_hip_llam
             m->attn_fused = ok;
         }
     }
-    if (!rc && fused_ok(m)) { m->dry = true; rc = enqueue_pass_any(m, m->own_stream, true); m->dry = false; }   // sizes the persistent grids
+    if (!rc && fused_ok(m)) { m->dry = true; rc = enqueue_pass_any(m, m->own_stream, PASS_GREEDY); m->dry = false; }   // sizes the persistent grids
     if (!rc && fused_ok(m)) {            // the persistent single-kernel pass: opt-in with SPY_HIP_MEGA=1 (slower than the per-phase kernels so far)
         std::vector<mega_layer> ml(c.n_layer);
         for (int i = 0; i < c.n_layer; i++) {
@@ -216,28 +217,34 @@ static int enqueue_one(spy_hip_llama *m, hipStream_t st, int which, int il) {
     return SPY_HIP_EUNSUPPORTED;
 }
 
-static int enqueue_pass_any(spy_hip_llama *m, hipStream_t st, bool sample) {
+static int enqueue_embed(spy_hip_llama *m, hipStream_t st) {
     const spy_hip_llama_desc &c = m->desc;
-    if (m->mega && !m->dry) {
+    embed_kernel<<<dim3(1), dim3(256), 0, st>>>(m->st, (const uint8_t *)c.tok_embd, c.t_tok_embd == SPY_HIP_Q8_0, c.n_embd, c.n_vocab, m->x,
+                                                m->rope_cs, m->theta_scale, m->hd);
+    return SPY_LAUNCH_RC();
+}
+
+// One single-token pass.  PASS_LOGITS: embedding, layers, head (spy_hip_llama_forward).  PASS_GREEDY: layers, head, and one
+// launch that samples, advances the position and prepares the next pass's embedding and RoPE table -- the first pass of a
+// greedy run is preceded by enqueue_embed.
+static int enqueue_pass_any(spy_hip_llama *m, hipStream_t st, int mode) {
+    const spy_hip_llama_desc &c = m->desc;
+    auto sample = [&](bool embed_next) {
+        sample_advance_kernel<<<dim3(1), dim3(1024), 0, st>>>(m->st, m->logits, c.n_vocab, m->tokens_out, m->max_out,
+                                                              embed_next ? (const uint8_t *)c.tok_embd : nullptr, c.t_tok_embd == SPY_HIP_Q8_0, c.n_embd,
+                                                              m->x, m->rope_cs, m->theta_scale, m->hd);
+        return SPY_LAUNCH_RC();
+    };
+    if (m->mega && !m->dry) {            // the persistent kernel does its own embedding
         RC_TRY(c.wtype == SPY_HIP_Q4_0 ? spy_enqueue_mega_q4_0(m, st, false) : spy_enqueue_mega_q8_0(m, st, false));
-        if (sample) {
-            sample_advance_kernel<<<dim3(1), dim3(1024), 0, st>>>(m->st, m->logits, c.n_vocab, m->tokens_out, m->max_out);
-            RC_TRY(SPY_LAUNCH_RC());
-        }
+        if (mode == PASS_GREEDY) RC_TRY(sample(false));
         return 0;
     }
-    if (!m->dry) {
-        embed_kernel<<<dim3(1), dim3(256), 0, st>>>(m->st, (const uint8_t *)c.tok_embd, c.t_tok_embd == SPY_HIP_Q8_0, c.n_embd, c.n_vocab, m->x,
-                                                    m->rope_cs, m->theta_scale, m->hd);
-        RC_TRY(SPY_LAUNCH_RC());
-    }
+    if (mode == PASS_LOGITS && !m->dry) RC_TRY(enqueue_embed(m, st));
     for (int il = 0; il < c.n_layer; il++)
         for (int k = K_QKV; k <= K_DOWN; k++) RC_TRY(enqueue_one(m, st, k, il));
     RC_TRY(enqueue_one(m, st, K_HEAD, 0));
-    if (sample && !m->dry) {
-        sample_advance_kernel<<<dim3(1), dim3(1024), 0, st>>>(m->st, m->logits, c.n_vocab, m->tokens_out, m->max_out);
-        RC_TRY(SPY_LAUNCH_RC());
-    }
+    if (mode == PASS_GREEDY && !m->dry) RC_TRY(sample(true));
     return 0;
 }
 
@@ -382,7 +389,7 @@ extern "C" int spy_hip_llama_forward(spy_hip_llama *m, void *stream, const int32
     if (n_token == 1 && fused_ok(m) && !getenv("SPY_HIP_FORCE_OPS")) {
         dev_state h = {tokens_host[0], n_past, 0, 0};
         HIP_TRY(hipMemcpyAsync(m->st, &h, sizeof(h), hipMemcpyHostToDevice, st));
-        RC_TRY(enqueue_pass_any(m, st, false));
+        RC_TRY(enqueue_pass_any(m, st, PASS_LOGITS));
         if (logits_host) HIP_TRY(hipMemcpyAsync(logits_host, m->logits, (size_t)m->desc.n_vocab * 4, hipMemcpyDeviceToHost, st));
         HIP_TRY(hipStreamSynchronize(st));
         return 0;
@@ -413,17 +420,18 @@ extern "C" int spy_hip_llama_decode_greedy(spy_hip_llama *m, void *stream, int32
         if (m->graph_exec) { (void)hipGraphExecDestroy(m->graph_exec); m->graph_exec = nullptr; }
         if (m->graph) { (void)hipGraphDestroy(m->graph); m->graph = nullptr; }
         HIP_TRY(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
-        const int rc = enqueue_pass_any(m, st, true);
+        const int rc = enqueue_pass_any(m, st, PASS_GREEDY);
         hipError_t e = hipStreamEndCapture(st, &m->graph);
         if (rc) return rc;
         if (e != hipSuccess) return (int)e;
         HIP_TRY(hipGraphInstantiate(&m->graph_exec, m->graph, nullptr, nullptr, 0));
         m->graph_stream = st;
     }
+    if (!m->mega) RC_TRY(enqueue_embed(m, st));              // embedding of the first token; every step prepares the next one's
     HIP_TRY(hipEventRecord(m->ev0, st));
     for (int i = 0; i < n_steps; i++) {
         if (use_graph) HIP_TRY(hipGraphLaunch(m->graph_exec, st));
-        else RC_TRY(enqueue_pass_any(m, st, true));
+        else RC_TRY(enqueue_pass_any(m, st, PASS_GREEDY));
     }
     HIP_TRY(hipEventRecord(m->ev1, st));
     HIP_TRY(hipEventSynchronize(m->ev1));
