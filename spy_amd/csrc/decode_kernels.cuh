@@ -209,6 +209,10 @@ __global__ __launch_bounds__(WGV_THREADS) void wave_gemv_kernel(fused_args a) {
             if constexpr (EPI == EPI_RESID) side[k] = a.resid[r];
         }
     };
+    // The compute unit serves its memory requests in order: every wave's activation request goes into the queue before any
+    // wave's first row (the barrier waits for the requests to be issued, not for the data).  Without it the last waves' x arrives
+    // behind 15 waves' worth of rows, and the staging barrier with it.
+    __builtin_amdgcn_s_barrier();
 #pragma unroll
     for (int k = 0; k < NB; k++) if (k < DEPTH) issue(k);
 
@@ -310,6 +314,7 @@ __global__ __launch_bounds__(WGV_THREADS) void wave_gemv_kernel(fused_args a) {
 #define ATL_THREADS (ATL_WAVES * 64)
 #define ATL_GPH (128 / ATL_WAVES)  // workgroups per head
 #define ATL_NX (1024 / ATL_THREADS)
+#define ATL_NS (5120 / ATL_THREADS) // scores per thread of the softmax step (n_ctx <= 5120)
 #define ATL_RS 10                 // groups of 4 keys per wave (n_ctx <= 128 * 4 * ATL_RS)
 #define ATL_RV 10                 // 128-bit pieces per lane of a V^T row (n_ctx <= 512 * ATL_RV)
 #ifndef ATL_DEPTH_K
@@ -396,6 +401,7 @@ __global__ __launch_bounds__(ATL_THREADS, 4) void attn_layer_kernel(attn_layer_a
     wtile<WTV, 1> tv;
     const int wp = w & 63;                                           // RoPE pair of the head
     const uint8_t *p0 = (w < 64 ? a.wq : a.wk) + (size_t)(h * 128 + 2 * wp) * RB;
+    __builtin_amdgcn_s_barrier();            // x of every wave ahead of every wave's rows in the compute unit's memory queue
     load_tile<WT, 64, 1>(t[0], p0, npair, lane);
     load_tile<WT, 64, 1>(t[1], p0 + RB, npair, lane);
     if (tid < 128) s_rope[tid] = rope_v;
@@ -451,7 +457,7 @@ __global__ __launch_bounds__(ATL_THREADS, 4) void attn_layer_kernel(attn_layer_a
             s_out[wave * 2] = __uint_as_float((uint32_t)f2h(s0 * c - s1 * sn) | ((uint32_t)f2h(s0 * sn + s1 * c) << 16));
             s_out[wave * 2 + 1] = __uint_as_float((uint32_t)f2h(s2));
         }
-        if (wave != 0) {
+        if (wave != 0) {                     // (requesting the keys only after the barrier, behind q, measured 1 us slower)
 #pragma unroll
             for (int k = 0; k < ATL_DEPTH_K; k++) fetch_k(k);
         }
@@ -502,10 +508,6 @@ __global__ __launch_bounds__(ATL_THREADS, 4) void attn_layer_kernel(attn_layer_a
             s = group_sum<16>(s);
             if ((lane & 15) == 0) s_out[wave * (4 * ATL_RS) + k * 4 + (lane >> 4)] = s * a.scale;
         }
-        if (wave != 0) {
-#pragma unroll
-            for (int i = 0; i < ATL_DEPTH_V; i++) fetch_v(i);
-        }
     }
     ATL_STAMP(4);
     if (!publish_and_sync(sync + 32, [&]() {
@@ -525,11 +527,16 @@ __global__ __launch_bounds__(ATL_THREADS, 4) void attn_layer_kernel(attn_layer_a
         const float *srow = a.scores + (size_t)h * n_ctx;
         const int n_pad = (n_kv + 7) & ~7;
         float mx = -INFINITY;
-        for (int j = tid; j < n_kv; j += ATL_THREADS) { const float tt = ldc(srow + j); s_t[j] = tt; mx = fmaxf(mx, tt); }
-        if (wave == 0) {
+        // the head's scores first, for every wave (they are what the softmax waits for), the first V^T pieces behind them; no
+        // V^T request before the barrier above: its stores, atomics and polls would wait behind them in the memory queue
+        float sreg[ATL_NS];
 #pragma unroll
-            for (int i = 0; i < ATL_DEPTH_V; i++) fetch_v(i);
-        }
+        for (int u = 0; u < ATL_NS; u++) sreg[u] = ldc(srow + min(tid + u * ATL_THREADS, n_ctx - 1));
+        __builtin_amdgcn_s_barrier();
+#pragma unroll
+        for (int i = 0; i < ATL_DEPTH_V; i++) fetch_v(i);
+#pragma unroll
+        for (int u = 0; u < ATL_NS; u++) { const int j = tid + u * ATL_THREADS; if (j < n_kv) { s_t[j] = sreg[u]; mx = fmaxf(mx, sreg[u]); } }
         mx = wave_max(mx);
         if (lane == 0) s_red[wave] = mx;
         __syncthreads();
