@@ -101,6 +101,7 @@ __global__ __launch_bounds__(WROW_THREADS) void wave_row_kernel(gemv_args a, int
     // activation row 0 is requested first, the first weight rows behind it
     uint32_t xr[NITK + 1];
     stage_native_q8_load<WROW_THREADS, NITK + 1>(a.xq, nblk, xr);
+    __builtin_amdgcn_s_barrier();          // every wave's activation request is queued before any wave's first row (issue order, not data)
 #pragma unroll
     for (int k = 0; k < NR; k++) if (k < DEPTH) issue(k);
     auto act_of = [&](int c) {                              // staged activation row c (computed, not kept: no private array)
