@@ -86,6 +86,23 @@ __global__ __launch_bounds__(256) void binary_kernel(int op, tdesc a, tdesc b, t
     *(float *)at(d, i0, i1, i2, i3) = v;
 }
 
+// The shapes the LLaMA graph uses -- contiguous a and dst, b either of the same shape or one contiguous row repeated over
+// the rows (a norm weight) -- four elements per thread, no index arithmetic beyond one remainder.
+__global__ __launch_bounds__(256) void binary_rows_kernel(int op, const float4 *a, const float4 *b, float4 *d,      /* dst may be a or b */
+                                                          int64_t total4, int64_t b4) {
+    const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (g >= total4) return;
+    const float4 va = a[g], vb = b[b4 == total4 ? g : g % b4];
+    float4 v;
+    switch (op) {
+    case 0: v = make_float4(va.x + vb.x, va.y + vb.y, va.z + vb.z, va.w + vb.w); break;
+    case 1: v = make_float4(va.x - vb.x, va.y - vb.y, va.z - vb.z, va.w - vb.w); break;
+    case 2: v = make_float4(va.x * vb.x, va.y * vb.y, va.z * vb.z, va.w * vb.w); break;
+    default: v = make_float4(va.x / vb.x, va.y / vb.y, va.z / vb.z, va.w / vb.w); break;
+    }
+    d[g] = v;
+}
+
 extern "C" int spy_hip_op_binary(void *stream, int op, const spy_hip_tensor *a, const spy_hip_tensor *b, const spy_hip_tensor *dst) {
     SPY_CHECK_ARG(a && b && dst && a->data && b->data && dst->data && op >= 0 && op <= 3);
     if (a->type != SPY_HIP_F32 || b->type != SPY_HIP_F32 || dst->type != SPY_HIP_F32) return SPY_HIP_EUNSUPPORTED;
@@ -93,6 +110,15 @@ extern "C" int spy_hip_op_binary(void *stream, int op, const spy_hip_tensor *a, 
     for (int i = 0; i < 4; i++) SPY_CHECK_ARG(b->ne[i] > 0 && a->ne[i] % b->ne[i] == 0);   // Shape::can_repeat (tensor.h:186-190)
     const int64_t total = spy_t_nelem(a);
     CHECK_GRID(total, 256);
+    const int64_t nb_ = spy_t_nelem(b);
+    const bool b_row = b->ne[1] == 1 && b->ne[2] == 1 && b->ne[3] == 1 && b->nb[0] == 4;          // one row, repeated
+    const bool b_same = nb_ == total && same_ne(a, b) && spy_t_contiguous(b);
+    if (spy_t_contiguous(a) && spy_t_contiguous(dst) && (b_row || b_same) && a->ne[0] % 4 == 0 && b->ne[0] % 4 == 0 && (b_same || a->ne[0] == b->ne[0]) &&
+        (((uintptr_t)a->data | (uintptr_t)b->data | (uintptr_t)dst->data) & 15) == 0) {
+        binary_rows_kernel<<<dim3(grid_for(total / 4, 256)), dim3(256), 0, (hipStream_t)stream>>>(op, (const float4 *)a->data, (const float4 *)b->data,
+                                                                                                (float4 *)dst->data, total / 4, (b_same ? total : b->ne[0]) / 4);
+        return SPY_LAUNCH_RC();
+    }
     binary_kernel<<<dim3(grid_for(total, 256)), dim3(256), 0, (hipStream_t)stream>>>(op, mk(a), mk(b), mk(dst), total);
     return SPY_LAUNCH_RC();
 }
@@ -114,12 +140,23 @@ __global__ __launch_bounds__(256) void silu_kernel(tdesc x, tdesc d, int64_t tot
     *(float *)at(d, i0, i1, i2, i3) = silu_ref(*(const float *)at(x, i0, i1, i2, i3));
 }
 
+__global__ __launch_bounds__(256) void silu_flat_kernel(const float4 *x, float4 *d, int64_t total4)      /* in place allowed */ {
+    const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (g >= total4) return;
+    const float4 v = x[g];
+    d[g] = make_float4(silu_ref(v.x), silu_ref(v.y), silu_ref(v.z), silu_ref(v.w));
+}
+
 extern "C" int spy_hip_op_silu(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *dst) {
     SPY_CHECK_ARG(x && dst && x->data && dst->data);
     if (x->type != SPY_HIP_F32 || dst->type != SPY_HIP_F32) return SPY_HIP_EUNSUPPORTED;
     SPY_CHECK_ARG(same_ne(x, dst));
     const int64_t total = spy_t_nelem(x);
     CHECK_GRID(total, 256);
+    if (spy_t_contiguous(x) && spy_t_contiguous(dst) && total % 4 == 0 && (((uintptr_t)x->data | (uintptr_t)dst->data) & 15) == 0) {
+        silu_flat_kernel<<<dim3(grid_for(total / 4, 256)), dim3(256), 0, (hipStream_t)stream>>>((const float4 *)x->data, (float4 *)dst->data, total / 4);
+        return SPY_LAUNCH_RC();
+    }
     silu_kernel<<<dim3(grid_for(total, 256)), dim3(256), 0, (hipStream_t)stream>>>(mk(x), mk(dst), total);
     return SPY_LAUNCH_RC();
 }
