@@ -6,7 +6,10 @@
 //    (backend/host/operator/mat.cpp:130-143, backend/host/include/simd/vec_dot.h:42-115 in the Spy
 //    tree).  One v_mfma_i32_32x32x32_i8 contracts exactly one 32-element quantization block for a
 //    32 x 32 output tile, so the int32 block dots are exact; each is then scaled by
-//    h2f(d_w) * h2f(d_x) and accumulated in fp32 like the reference's fma (vec_dot.h:76-79).
+//    h2f(d_w) * h2f(d_x) and accumulated in fp32 like the reference's fma (vec_dot.h:76-79).  The scale
+//    products of a tile come from an fp16 MFMA (outer product of the two scale vectors, exact in fp32):
+//    matrix and vector instructions of a SIMD were measured to add up rather than overlap here, and the
+//    MFMA costs half the cycles of the 16 multiplications it replaces.
 //    Nibbles are unpacked to int8 (n - 8) on the way into LDS.
 //  * gemm_f16_kernel: fp16 rows x fp16 rows with fp32 accumulation (Dot<FP16,FP16>,
 //    vec_dot.h:117-146) for the attention products of a prompt pass: strided left operand (the K cache
@@ -22,11 +25,16 @@
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
 #define GEMM_TILE 128
 #define GEMM_SKINNY_MAX_TILES 160 // the 32-row kernel is used up to 64 activation rows and wherever the 128 x 128 tiling would give at most this many workgroups (measured crossover)
 #define GEMM_ROWB 80             // bytes per LDS row: 64 payload + 16 pad
+#ifndef GEMM_WGS
+#define GEMM_WGS 3                // workgroups per CU the tile kernel is compiled for (register budget 512 / GEMM_WGS per lane)
+#endif
 #ifndef GEMM_PF
 #define GEMM_PF 1                // stages of global loads in flight per thread (the kernel is bound by its scale epilogue on the vector units: 2 and 3 measured the same)
 #endif
@@ -35,14 +43,14 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 static __device__ __forceinline__ uint32_t nib_m8(uint32_t lo) { return (lo + 0x78787878u) ^ 0x80808080u; }
 
 template <int WT>
-__global__ __launch_bounds__(256, 2) void gemm_q8act_kernel(const uint8_t *__restrict__ W, const uint8_t *__restrict__ xq, float *__restrict__ dst,
+__global__ __launch_bounds__(256, GEMM_WGS) void gemm_q8act_kernel(const uint8_t *__restrict__ W, const uint8_t *__restrict__ xq, float *__restrict__ dst,
                                                             int M, int K, int T, int64_t dst_stride) {
     constexpr int PAIR_DW = (WT == SPY_HIP_Q4_0) ? 9 : 17;       // dwords per pair of weight blocks
     constexpr int HALF_DW = (WT == SPY_HIP_Q4_0) ? 5 : 9;        // dwords that cover one block of the pair
     __shared__ __attribute__((aligned(16))) uint8_t sA[2][GEMM_TILE * GEMM_ROWB];
     __shared__ __attribute__((aligned(16))) uint8_t sB[2][GEMM_TILE * GEMM_ROWB];
-    __shared__ __attribute__((aligned(16))) float sAd[2][2][GEMM_TILE];      // [buffer][block of the pair][row]
-    __shared__ __attribute__((aligned(16))) float sBd[2][2][GEMM_TILE];
+    __shared__ uint16_t sAd[2][2][GEMM_TILE];                                // fp16 block scales [buffer][block of the pair][row]
+    __shared__ uint16_t sBd[2][2][GEMM_TILE];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
     const int m0 = blockIdx.x * GEMM_TILE, t0 = blockIdx.y * GEMM_TILE;
     const int nstage = K / 64;
@@ -50,9 +58,11 @@ __global__ __launch_bounds__(256, 2) void gemm_q8act_kernel(const uint8_t *__res
 
     // Every thread moves one weight block and one activation block per stage: row tid & 127, block
     // tid >> 7 of the 4-byte aligned block pair (block 0 starts at byte 0, block 1 in the middle of a
-    // dword: the dwords that cover it are loaded and the scale / quants shifted out).  Rows beyond
-    // the matrix re-read its last row (their outputs are never stored).
-    const int lrow = tid & 127, half = tid >> 7;
+    // dword: the dwords that cover it are loaded and the scale / quants picked out with byte selectors that
+    // are the same for a whole wave).  Rows beyond the matrix re-read its last row (their outputs are never stored).
+    const int lrow = tid & 127, half = __builtin_amdgcn_readfirstlane(tid >> 7);
+    const uint32_t qsel = half ? 0x07060504u : 0x05040302u;  // v_perm_b32 selector over {raw[i+1], raw[i]}: quants dword-aligned / starting mid-dword
+    const uint32_t dshift = half ? 16 : 0;                    // the fp16 scale sits in the upper / lower half of raw[0]
     const uint32_t *gA = (const uint32_t *)(W + (size_t)min(m0 + lrow, M - 1) * RBw) + half * (HALF_DW - 1);
     const uint32_t *gB = (const uint32_t *)(xq + (size_t)min(t0 + lrow, T - 1) * RBx) + half * 8;
     // Global loads run GEMM_PF stages ahead of the stage being multiplied (a ring of raw registers): with one
@@ -62,32 +72,28 @@ __global__ __launch_bounds__(256, 2) void gemm_q8act_kernel(const uint8_t *__res
         __builtin_memcpy(rawA[slot], __builtin_assume_aligned(gA + (size_t)s * PAIR_DW, 4), HALF_DW * 4);
         __builtin_memcpy(rawB[slot], __builtin_assume_aligned(gB + (size_t)s * 17, 4), 36);
     };
-    // one Q8_0 block held in 9 dwords -> scale + 8 dwords of int8
-    auto split_q8 = [&](const uint32_t *raw, float &d, uint32_t *q) {
-        d = h2f((uint16_t)(half ? raw[0] >> 16 : raw[0] & 0xFFFFu));
-#pragma unroll
-        for (int i = 0; i < 8; i++) q[i] = half ? raw[i + 1] : __builtin_amdgcn_alignbit(raw[i + 1], raw[i], 16);
-    };
     auto unpack = [&](int b, int slot) {
         uint32_t q[8];
-        float d;
         if constexpr (WT == SPY_HIP_Q4_0) {
             // {d, qs[16]}: element j = low nibble of qs[j], element j+16 = high nibble (quant.h:25-28); stored as n - 8
-            d = h2f((uint16_t)(half ? rawA[slot][0] >> 16 : rawA[slot][0] & 0xFFFFu));
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                const uint32_t n = half ? rawA[slot][i + 1] : __builtin_amdgcn_alignbit(rawA[slot][i + 1], rawA[slot][i], 16);
+                const uint32_t n = __builtin_amdgcn_perm(rawA[slot][i + 1], rawA[slot][i], qsel);
                 q[i] = nib_m8(n & 0x0F0F0F0Fu);
                 q[4 + i] = nib_m8((n >> 4) & 0x0F0F0F0Fu);
             }
-        } else split_q8(rawA[slot], d, q);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; i++) q[i] = __builtin_amdgcn_perm(rawA[slot][i + 1], rawA[slot][i], qsel);
+        }
         uint4 *ra = (uint4 *)(sA[b] + lrow * GEMM_ROWB + half * 32);
         ra[0] = make_uint4(q[0], q[1], q[2], q[3]); ra[1] = make_uint4(q[4], q[5], q[6], q[7]);
-        sAd[b][half][lrow] = d;
-        split_q8(rawB[slot], d, q);                          // {d, qs[32]} (quant.h:139-142)
+        sAd[b][half][lrow] = (uint16_t)(rawA[slot][0] >> dshift);
+#pragma unroll
+        for (int i = 0; i < 8; i++) q[i] = __builtin_amdgcn_perm(rawB[slot][i + 1], rawB[slot][i], qsel);   // {d, qs[32]} (quant.h:139-142)
         uint4 *rb = (uint4 *)(sB[b] + lrow * GEMM_ROWB + half * 32);
         rb[0] = make_uint4(q[0], q[1], q[2], q[3]); rb[1] = make_uint4(q[4], q[5], q[6], q[7]);
-        sBd[b][half][lrow] = d;
+        sBd[b][half][lrow] = (uint16_t)(rawB[slot][0] >> dshift);
     };
 
     float acc[2][2][16];
@@ -98,32 +104,36 @@ __global__ __launch_bounds__(256, 2) void gemm_q8act_kernel(const uint8_t *__res
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
+    // Per block and 32 x 32 tile: the int32 block dots from one int8 MFMA, and the scale products
+    // h2f(d_w) * h2f(d_x) of the same tile from one fp16 MFMA whose operands hold the scales at k = 0 and zeros
+    // elsewhere (an outer product; fp16 x fp16 is exact in fp32, so these are the bits of the scalar product).
+    // That leaves a conversion and an fma per output on the vector units, which bound this kernel.
+    const int k0mask = lane < 32 ? 0xFFFF : 0;
     auto multiply = [&](int b) {
 #pragma unroll 1
         for (int blk = 0; blk < 2; blk++) {
             v4i fa[2], fb[2];
+            v4h ha[2], hb[2];
 #pragma unroll
             for (int i = 0; i < 2; i++) {
                 fa[i] = *(const v4i *)(sA[b] + (wm * 64 + i * 32 + (lane & 31)) * GEMM_ROWB + blk * 32 + (lane >> 5) * 16);
                 fb[i] = *(const v4i *)(sB[b] + (wn * 64 + i * 32 + (lane & 31)) * GEMM_ROWB + blk * 32 + (lane >> 5) * 16);
+                const int da = sAd[b][blk][wm * 64 + i * 32 + (lane & 31)];
+                const int dx = sBd[b][blk][wn * 64 + i * 32 + (lane & 31)] & k0mask;             // lanes 32..63 carry k = 4..7: zero
+                ha[i] = __builtin_bit_cast(v4h, v2i{da, 0});
+                hb[i] = __builtin_bit_cast(v4h, v2i{dx, 0});
             }
 #pragma unroll
-            for (int i = 0; i < 2; i++) {
-                float dw[16];
-#pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    const float4 v = *(const float4 *)&sAd[b][blk][wm * 64 + i * 32 + g * 8 + (lane >> 5) * 4];
-                    dw[4 * g] = v.x; dw[4 * g + 1] = v.y; dw[4 * g + 2] = v.z; dw[4 * g + 3] = v.w;
-                }
+            for (int i = 0; i < 2; i++)
 #pragma unroll
                 for (int j = 0; j < 2; j++) {
-                    const float dx = sBd[b][blk][wn * 64 + j * 32 + (lane & 31)];
                     v16i z = {0};
+                    v16f zf = {0};
                     const v16i I = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], z, 0, 0, 0);
+                    const v16f S = __builtin_amdgcn_mfma_f32_32x32x8f16(ha[i], hb[j], zf, 0, 0, 0);
 #pragma unroll
-                    for (int r = 0; r < 16; r++) acc[i][j][r] = fmaf(dw[r] * dx, (float)I[r], acc[i][j][r]);
+                    for (int r = 0; r < 16; r++) acc[i][j][r] = fmaf(S[r], (float)I[r], acc[i][j][r]);
                 }
-            }
         }
     };
 
@@ -373,7 +383,7 @@ __global__ __launch_bounds__(256, 2) void gemm_kq_kernel(const uint8_t *__restri
     const int m0 = blockIdx.x * GEMM_TILE, t0 = blockIdx.y * GEMM_TILE;
     const int nstage = K / 64;
     const size_t RBw = (size_t)spy_row_size(WT, K), RBx = (size_t)(K / 32) * 34;
-    const int lrow = tid & 127, half = tid >> 7;
+    const int lrow = tid & 127, half = __builtin_amdgcn_readfirstlane(tid >> 7);   // the same for all lanes of a wave
     const uint8_t *gA = W + (size_t)min(m0 + lrow, M - 1) * RBw;
     const uint32_t *gB = (const uint32_t *)(xq + (size_t)min(t0 + lrow, T - 1) * RBx) + half * 8;
     uint32_t rawA[RAW], rawB[9];
