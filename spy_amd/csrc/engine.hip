@@ -264,6 +264,8 @@ static spy_hip_tensor T3s(int type, void *p, int64_t e0, int64_t e1, int64_t e2,
     return t;
 }
 
+int spy_softmax_causal_launch(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *dst, float scale, int n_past);   // ops.hip
+
 // KQ mask of a pass over tokens P .. P + T - 1 (llama.cpp:248-263): row i allows the cached positions j <= P + i
 __global__ __launch_bounds__(256) void causal_mask_kernel(float *__restrict__ mask, int C, int P) {
     const int j = blockIdx.x * 256 + threadIdx.x, i = blockIdx.y;
@@ -350,7 +352,11 @@ static int forward_ops(spy_hip_llama *m, hipStream_t st, const int32_t *tokens_h
         spy_hip_tensor t_S = T3s(SPY_HIP_F32, S, n_kv, T, H, 4, 4 * n_kv, 4 * n_kv * T);
         spy_hip_tensor t_P = p16 ? T3s(SPY_HIP_F16, Pm, n_kv, T, H, 2, 2 * n_kv, 2 * n_kv * T) : T3s(SPY_HIP_F32, Pm, n_kv, T, H, 4, 4 * n_kv, 4 * n_kv * T);
         RC_TRY(spy_hip_op_matmul(st, &t_kall, &t_qp, &t_S, scr, scr_bytes));
-        RC_TRY(spy_hip_op_softmax(st, &t_S, &t_mask, &t_P, scale));
+        {   // the mask of this pass is the causal one filled above: the row kernel takes its shape as a number
+            int rc = spy_softmax_causal_launch(st, &t_S, &t_P, scale, P);
+            if (rc == SPY_HIP_EUNSUPPORTED) rc = spy_hip_op_softmax(st, &t_S, &t_mask, &t_P, scale);
+            RC_TRY(rc);
+        }
         spy_hip_tensor t_O = T3s(SPY_HIP_F32, o, hd, T, H, 4, 4 * hd, 4 * hd * T);
         RC_TRY(spy_hip_op_matmul(st, &t_vall, &t_P, &t_O, scr, scr_bytes));
         spy_hip_tensor t_Op = T3s(SPY_HIP_F32, o, hd, H, T, 4, 4 * hd * T, 4 * hd);                    // Permute {0,2,1,3}

@@ -209,7 +209,7 @@ __global__ __launch_bounds__(256) void softmax_kernel(tdesc x, tdesc mask, bool 
 // probabilities rounded to fp16, which is what the KQV product does to them first anyway (mat.cpp:37).
 #define SOFTMAX_LDS_ROW 16384
 template <bool F16OUT>
-__global__ __launch_bounds__(256) void softmax_row_kernel(tdesc x, tdesc mask, bool has_mask, tdesc y, float scale) {
+__global__ __launch_bounds__(256) void softmax_row_kernel(tdesc x, tdesc mask, bool has_mask, tdesc y, float scale, int causal_past) {
     extern __shared__ __attribute__((aligned(16))) float s_row[];
     __shared__ float s_part[4];
     const int64_t r = blockIdx.x;
@@ -217,20 +217,24 @@ __global__ __launch_bounds__(256) void softmax_row_kernel(tdesc x, tdesc mask, b
     const int64_t ne1 = y.ne[1], ne2 = y.ne[2];
     const int64_t i3 = r / (ne1 * ne2), i2 = r % (ne1 * ne2) / ne1, i1 = r % ne1;
     const float *s = (const float *)at(x, 0, i1, i2, i3);
-    const float *mk_ = has_mask ? (const float *)at(mask, 0, i1, 0, 0) : nullptr;
+    // causal_past >= 0: the mask is known to be the causal one of a pass that starts at position causal_past (row i1 sees
+    // the first causal_past + i1 + 1 elements) and is not read; the elements beyond contribute -inf to the maximum and 0
+    // to the sum, i.e. nothing, so the bits are those of the masked path
+    const int nv = causal_past >= 0 ? (int)min((int64_t)ne0, causal_past + i1 + 1) : ne0;
+    const float *mk_ = (has_mask && causal_past < 0) ? (const float *)at(mask, 0, i1, 0, 0) : nullptr;
     float mx = -INFINITY;
-    for (int i = threadIdx.x; i < ne0; i += 256) {
+    for (int i = threadIdx.x; i < nv; i += 256) {
         float t;
-        if (has_mask) { const float mv = mk_[i]; t = (mv == -INFINITY) ? -INFINITY : (s[i] + mv) * scale; }
+        if (mk_) { const float mv = mk_[i]; t = (mv == -INFINITY) ? -INFINITY : (s[i] + mv) * scale; }
         else t = s[i] * scale;
         s_row[i] = t;
         mx = fmaxf(mx, t);
     }
     mx = block_reduce_256(mx, true, s_part);
     float sum = 0.0f;
-    for (int i = threadIdx.x; i < ne0; i += 256) {
+    for (int i = threadIdx.x; i < nv; i += 256) {
         const float t = s_row[i];
-        const float e = (has_mask && t == -INFINITY) ? 0.0f : expf(h2f(f2h(t - mx)));
+        const float e = (mk_ && t == -INFINITY) ? 0.0f : expf(h2f(f2h(t - mx)));
         s_row[i] = e;
         sum += e;
     }
@@ -238,14 +242,27 @@ __global__ __launch_bounds__(256) void softmax_row_kernel(tdesc x, tdesc mask, b
     const float inv = 1.0f / sum;
     if constexpr (F16OUT) {
         uint16_t *d = (uint16_t *)at(y, 0, i1, i2, i3);
-        for (int i = threadIdx.x; i < ne0; i += 256) d[i] = f2h(s_row[i] * inv);
+        for (int i = threadIdx.x; i < ne0; i += 256) d[i] = i < nv ? f2h(s_row[i] * inv) : (uint16_t)0;
     } else {
         float *d = (float *)at(y, 0, i1, i2, i3);
-        for (int i = threadIdx.x; i < ne0; i += 256) d[i] = s_row[i] * inv;
+        for (int i = threadIdx.x; i < ne0; i += 256) d[i] = i < nv ? s_row[i] * inv : 0.0f;
     }
 }
 
+static int softmax_launch(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *mask, const spy_hip_tensor *dst, float scale, int causal_past);
+// Softmax under the causal mask of a pass that starts at position n_past, without reading a mask tensor (the token
+// loop fills its masks itself and knows their shape).  Same bits as spy_hip_op_softmax with that mask.
+int spy_softmax_causal_launch(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *dst, float scale, int n_past) {
+    SPY_CHECK_ARG(n_past >= 0 && dst && scale > 0.0f);
+    if (dst->ne[0] > SOFTMAX_LDS_ROW) return SPY_HIP_EUNSUPPORTED;      // the caller falls back to the operator with a mask tensor
+    return softmax_launch(stream, x, nullptr, dst, scale, n_past);
+}
+
 extern "C" int spy_hip_op_softmax(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *mask, const spy_hip_tensor *dst, float scale) {
+    return softmax_launch(stream, x, mask, dst, scale, -1);
+}
+
+static int softmax_launch(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *mask, const spy_hip_tensor *dst, float scale, int causal_past) {
     SPY_CHECK_ARG(x && dst && x->data && dst->data);
     if (x->type != SPY_HIP_F32 || (dst->type != SPY_HIP_F32 && dst->type != SPY_HIP_F16)) return SPY_HIP_EUNSUPPORTED;
     SPY_CHECK_ARG(same_ne(x, dst) && x->nb[0] == 4 && dst->nb[0] == (dst->type == SPY_HIP_F16 ? 2 : 4));
@@ -270,10 +287,11 @@ extern "C" int spy_hip_op_softmax(void *stream, const spy_hip_tensor *x, const s
             if (e1_ != hipSuccess || e2_ != hipSuccess) return (int)(e1_ != hipSuccess ? e1_ : e2_);
             lds_set = SOFTMAX_LDS_ROW * 4;
         }
-        if (dst->type == SPY_HIP_F16) softmax_row_kernel<true><<<dim3((unsigned)nrow), dim3(256), lds, (hipStream_t)stream>>>(mk(x), m, mask != nullptr, mk(dst), scale);
-        else softmax_row_kernel<false><<<dim3((unsigned)nrow), dim3(256), lds, (hipStream_t)stream>>>(mk(x), m, mask != nullptr, mk(dst), scale);
+        if (dst->type == SPY_HIP_F16) softmax_row_kernel<true><<<dim3((unsigned)nrow), dim3(256), lds, (hipStream_t)stream>>>(mk(x), m, mask != nullptr, mk(dst), scale, causal_past);
+        else softmax_row_kernel<false><<<dim3((unsigned)nrow), dim3(256), lds, (hipStream_t)stream>>>(mk(x), m, mask != nullptr, mk(dst), scale, causal_past);
         return SPY_LAUNCH_RC();
     }
+    if (causal_past >= 0) return SPY_HIP_EINVAL;
     softmax_kernel<<<dim3((unsigned)nrow), dim3(256), 0, (hipStream_t)stream>>>(mk(x), m, mask != nullptr, mk(dst), scale);
     return SPY_LAUNCH_RC();
 }
