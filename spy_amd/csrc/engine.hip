@@ -264,7 +264,10 @@ static spy_hip_tensor T3s(int type, void *p, int64_t e0, int64_t e1, int64_t e2,
     return t;
 }
 
+int spy_matmul_causal(void *stream, const spy_hip_tensor *w, const spy_hip_tensor *x, const spy_hip_tensor *dst, void *scratch, size_t scratch_bytes,
+                      int which, int past);                                                                                  // ops.hip
 int spy_softmax_causal_launch(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *dst, float scale, int n_past);   // ops.hip
+int spy_softmax_row_ok(int64_t ne0);                                                                                         // ops.hip
 
 // KQ mask of a pass over tokens P .. P + T - 1 (llama.cpp:248-263): row i allows the cached positions j <= P + i
 __global__ __launch_bounds__(256) void causal_mask_kernel(float *__restrict__ mask, int C, int P) {
@@ -346,19 +349,19 @@ static int forward_ops(spy_hip_llama *m, hipStream_t st, const int32_t *tokens_h
         RC_TRY(spy_hip_op_dup(st, &t_vt, &t_vc));
         spy_hip_tensor t_kall = T3s(SPY_HIP_F16, m->k_cache[il], hd, n_kv, H, 2, 2 * d, 2 * hd);
         spy_hip_tensor t_vall = T3s(SPY_HIP_F16, m->v_cache[il], n_kv, hd, H, 2, 2 * C, 2 * C * hd);
+        // causal_ok: the softmax below takes the row kernel, which reads no score beyond a row's causal length and writes
+        // zeros there: the two products may then leave out what the mask removes
+        const bool causal_ok = spy_softmax_row_ok(n_kv) != 0;
         // the probabilities go to the KQV product as fp16 (its first step, mat.cpp:37): the softmax writes them that way
         // directly where the fp16 GEMM takes them (rows of a multiple of 8 elements)
-        const bool p16 = n_kv % 8 == 0 && n_kv <= 16384 && T >= 16;
+        const bool p16 = n_kv % 8 == 0 && causal_ok && T >= 16;
         spy_hip_tensor t_S = T3s(SPY_HIP_F32, S, n_kv, T, H, 4, 4 * n_kv, 4 * n_kv * T);
         spy_hip_tensor t_P = p16 ? T3s(SPY_HIP_F16, Pm, n_kv, T, H, 2, 2 * n_kv, 2 * n_kv * T) : T3s(SPY_HIP_F32, Pm, n_kv, T, H, 4, 4 * n_kv, 4 * n_kv * T);
-        RC_TRY(spy_hip_op_matmul(st, &t_kall, &t_qp, &t_S, scr, scr_bytes));
-        {   // the mask of this pass is the causal one filled above: the row kernel takes its shape as a number
-            int rc = spy_softmax_causal_launch(st, &t_S, &t_P, scale, P);
-            if (rc == SPY_HIP_EUNSUPPORTED) rc = spy_hip_op_softmax(st, &t_S, &t_mask, &t_P, scale);
-            RC_TRY(rc);
-        }
+        RC_TRY(causal_ok ? spy_matmul_causal(st, &t_kall, &t_qp, &t_S, scr, scr_bytes, 0, P) : spy_hip_op_matmul(st, &t_kall, &t_qp, &t_S, scr, scr_bytes));
+        // the mask of this pass is the causal one filled above: the row kernel takes its shape as a number
+        RC_TRY(causal_ok ? spy_softmax_causal_launch(st, &t_S, &t_P, scale, P) : spy_hip_op_softmax(st, &t_S, &t_mask, &t_P, scale));
         spy_hip_tensor t_O = T3s(SPY_HIP_F32, o, hd, T, H, 4, 4 * hd, 4 * hd * T);
-        RC_TRY(spy_hip_op_matmul(st, &t_vall, &t_P, &t_O, scr, scr_bytes));
+        RC_TRY(causal_ok ? spy_matmul_causal(st, &t_vall, &t_P, &t_O, scr, scr_bytes, 1, P) : spy_hip_op_matmul(st, &t_vall, &t_P, &t_O, scr, scr_bytes));
         spy_hip_tensor t_Op = T3s(SPY_HIP_F32, o, hd, H, T, 4, 4 * hd * T, 4 * hd);                    // Permute {0,2,1,3}
         spy_hip_tensor t_o2c = T3s(SPY_HIP_F32, o2, hd, H, T, 4, 4 * hd, 4 * d);
         RC_TRY(spy_hip_op_contiguous(st, &t_Op, &t_o2c));

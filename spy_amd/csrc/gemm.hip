@@ -368,6 +368,8 @@ static __device__ __forceinline__ void q4k_sc_m(const uint32_t h1, const uint32_
     else { sc = (byte(a + 4) & 0x0F) | ((byte(a - 4) >> 6) << 4); mn = (byte(a + 4) >> 4) | ((byte(a) >> 6) << 4); }
 }
 
+template <bool Q4K> struct kq_scale { typedef float type; };
+template <> struct kq_scale<false> { typedef uint16_t type; };
 template <int WT>
 __global__ __launch_bounds__(256, 2) void gemm_kq_kernel(const uint8_t *__restrict__ W, const uint8_t *__restrict__ xq, float *__restrict__ dst,
                                                          int M, int K, int T, int64_t dst_stride) {
@@ -375,15 +377,16 @@ __global__ __launch_bounds__(256, 2) void gemm_kq_kernel(const uint8_t *__restri
     constexpr int RAW = Q4K ? 12 : 18;
     __shared__ __attribute__((aligned(16))) uint8_t sA[2][GEMM_TILE * GEMM_ROWB];
     __shared__ __attribute__((aligned(16))) uint8_t sB[2][GEMM_TILE * GEMM_ROWB];
-    __shared__ __attribute__((aligned(16))) float sAd[2][2][GEMM_TILE];      // Q4_K: d*sc          Q6_K: d
+    using scale_t = typename kq_scale<Q4K>::type;
+    __shared__ __attribute__((aligned(16))) scale_t sAd[2][2][GEMM_TILE];    // Q4_K: d*sc (float)  Q6_K: d (fp16 bits)
     __shared__ __attribute__((aligned(16))) int sAm[2][2][GEMM_TILE];        // Q4_K: bits of dmin*m Q6_K: sc_lo | sc_hi << 16
-    __shared__ __attribute__((aligned(16))) float sBd[2][2][GEMM_TILE];      // dx
+    __shared__ __attribute__((aligned(16))) scale_t sBd[2][2][GEMM_TILE];    // dx (Q4_K: float, Q6_K: fp16 bits)
     __shared__ __attribute__((aligned(16))) float sBs[2][2][GEMM_TILE];      // dx * sum(q_x)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
     const int m0 = blockIdx.x * GEMM_TILE, t0 = blockIdx.y * GEMM_TILE;
     const int nstage = K / 64;
     const size_t RBw = (size_t)spy_row_size(WT, K), RBx = (size_t)(K / 32) * 34;
-    const int lrow = tid & 127, half = __builtin_amdgcn_readfirstlane(tid >> 7);   // the same for all lanes of a wave
+    const int lrow = tid & 127, half = tid >> 7;
     const uint8_t *gA = W + (size_t)min(m0 + lrow, M - 1) * RBw;
     const uint32_t *gB = (const uint32_t *)(xq + (size_t)min(t0 + lrow, T - 1) * RBx) + half * 8;
     uint32_t rawA[RAW], rawB[9];
@@ -428,20 +431,21 @@ __global__ __launch_bounds__(256, 2) void gemm_kq_kernel(const uint8_t *__restri
                 const uint32_t hi = (rawA[8 + i] >> (2 * m)) & 0x03030303u;
                 q[i] = (lo | (hi << 4)) + 0x60606060u ^ 0x80808080u;
             }
-            sAd[b][half][lrow] = h2f((uint16_t)(rawA[17] & 0xFFFFu));
+            sAd[b][half][lrow] = (uint16_t)(rawA[17] & 0xFFFFu);
             sAm[b][half][lrow] = (int)(uint16_t)(int16_t)(int8_t)(rawA[16] & 0xFFu) | ((int)(int8_t)((rawA[16] >> 8) & 0xFFu) << 16);
         }
         uint4 *ra = (uint4 *)(sA[b] + lrow * GEMM_ROWB + half * 32);
         ra[0] = make_uint4(q[0], q[1], q[2], q[3]); ra[1] = make_uint4(q[4], q[5], q[6], q[7]);
         // activations: {d, qs[32]} (quant.h:139-142)
-        const float dx = h2f((uint16_t)(half ? rawB[0] >> 16 : rawB[0] & 0xFFFFu));
+        const uint16_t dxh = (uint16_t)(half ? rawB[0] >> 16 : rawB[0] & 0xFFFFu);
+        const float dx = h2f(dxh);
         int bsum = 0;
 #pragma unroll
         for (int i = 0; i < 8; i++) { q[i] = half ? rawB[i + 1] : __builtin_amdgcn_alignbit(rawB[i + 1], rawB[i], 16); bsum = __builtin_amdgcn_sdot4((int)q[i], 0x01010101, bsum, false); }
         uint4 *rb = (uint4 *)(sB[b] + lrow * GEMM_ROWB + half * 32);
         rb[0] = make_uint4(q[0], q[1], q[2], q[3]); rb[1] = make_uint4(q[4], q[5], q[6], q[7]);
-        sBd[b][half][lrow] = dx;
-        sBs[b][half][lrow] = dx * (float)bsum;
+        if constexpr (Q4K) { sBd[b][half][lrow] = dx; sBs[b][half][lrow] = dx * (float)bsum; }
+        else sBd[b][half][lrow] = dxh;
     };
 
     float acc[2][2][16];
@@ -452,6 +456,7 @@ __global__ __launch_bounds__(256, 2) void gemm_kq_kernel(const uint8_t *__restri
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
+    const int k0mask = lane < 32 ? 0xFFFF : 0;
     gload(0);
     unpack(0, 0);
     __syncthreads();
@@ -468,37 +473,50 @@ __global__ __launch_bounds__(256, 2) void gemm_kq_kernel(const uint8_t *__restri
             }
 #pragma unroll
             for (int i = 0; i < 2; i++) {
-                float dw[16]; int am[16];
+                int am[16];
 #pragma unroll
                 for (int g = 0; g < 4; g++) {
-                    const float4 v = *(const float4 *)&sAd[b][blk][wm * 64 + i * 32 + g * 8 + (lane >> 5) * 4];
                     const int4 u = *(const int4 *)&sAm[b][blk][wm * 64 + i * 32 + g * 8 + (lane >> 5) * 4];
-                    dw[4 * g] = v.x; dw[4 * g + 1] = v.y; dw[4 * g + 2] = v.z; dw[4 * g + 3] = v.w;
                     am[4 * g] = u.x; am[4 * g + 1] = u.y; am[4 * g + 2] = u.z; am[4 * g + 3] = u.w;
                 }
+                if constexpr (Q4K) {
+                    float dw[16];
 #pragma unroll
-                for (int j = 0; j < 2; j++) {
-                    const int col = wn * 64 + j * 32 + (lane & 31);
-                    const float dx = sBd[b][blk][col];
-                    v16i z = {0};
-                    if constexpr (Q4K) {
-                        const float dxs = sBs[b][blk][col];
+                    for (int g = 0; g < 4; g++) {
+                        const float4 v = *(const float4 *)&sAd[b][blk][wm * 64 + i * 32 + g * 8 + (lane >> 5) * 4];
+                        dw[4 * g] = v.x; dw[4 * g + 1] = v.y; dw[4 * g + 2] = v.z; dw[4 * g + 3] = v.w;
+                    }
+#pragma unroll
+                    for (int j = 0; j < 2; j++) {
+                        const int col = wn * 64 + j * 32 + (lane & 31);
+                        const float dx = sBd[b][blk][col], dxs = sBs[b][blk][col];
+                        v16i z = {0};
                         const v16i I = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], z, 0, 0, 0);
 #pragma unroll
                         for (int r = 0; r < 16; r++) {
                             acc[i][j][r] = fmaf(dw[r] * dx, (float)I[r], acc[i][j][r]);
                             acc[i][j][r] = fmaf(-__int_as_float(am[r]), dxs, acc[i][j][r]);
                         }
-                    } else {
+                    }
+                } else {
+                    // d (fp16) x dx (fp16) for the whole tile from one fp16 MFMA: scales at k = 0, zeros elsewhere (exact in fp32)
+                    const v4h ha = __builtin_bit_cast(v4h, v2i{(int)sAd[b][blk][wm * 64 + i * 32 + (lane & 31)], 0});
+#pragma unroll
+                    for (int j = 0; j < 2; j++) {
+                        const v4h hb = __builtin_bit_cast(v4h, v2i{(int)sBd[b][blk][wn * 64 + j * 32 + (lane & 31)] & k0mask, 0});
+                        v16i z = {0};
+                        v16f zf = {0};
                         const v4i zero4 = {0, 0, 0, 0};
                         const v4i blo = lane < 32 ? fb[j] : zero4, bhi = lane < 32 ? zero4 : fb[j];
                         const v16i Ilo = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], blo, z, 0, 0, 0);
                         const v16i Ihi = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], bhi, z, 0, 0, 0);
+                        const v16f S = __builtin_amdgcn_mfma_f32_32x32x8f16(ha, hb, zf, 0, 0, 0);
 #pragma unroll
                         for (int r = 0; r < 16; r++) {
                             const int sv = (int)(int16_t)(am[r] & 0xFFFF) * Ilo[r] + (am[r] >> 16) * Ihi[r];
-                            acc[i][j][r] = fmaf(dw[r] * dx, (float)sv, acc[i][j][r]);
+                            acc[i][j][r] = fmaf(S[r], (float)sv, acc[i][j][r]);
                         }
+                        __builtin_amdgcn_sched_barrier(0);       // one tile's three MFMA results at a time: two would not fit the register file
                     }
                 }
             }
@@ -557,6 +575,13 @@ struct gemm_f16_args {
     const uint8_t *A; const uint16_t *B; uint8_t *dst;
     int M, N, K;
     int64_t a_nb1, a_nb2, d_nb1, d_nb2;
+    // causal structure of the attention products of a pass that starts at position `past` (column n = token past + n,
+    // which sees positions 0 .. past + n); -1 = none.
+    //  skip_past:  rows m are cache positions (scores): tiles whose rows are all beyond what their columns see are not
+    //              computed (the softmax that follows never reads them)
+    //  klimit_past: the contraction runs over cache positions (probabilities x V^T): it stops where the tile's
+    //              probabilities are all zero (adding the zero products would not change a bit)
+    int skip_past, klimit_past;
 };
 
 __global__ __launch_bounds__(256) void gemm_f16_kernel(gemm_f16_args a) {
@@ -564,7 +589,9 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(gemm_f16_args a) {
     __shared__ __attribute__((aligned(16))) uint8_t sB[2][GEMM_TILE * GEMM_ROWB];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
     const int m0 = blockIdx.x * GEMM_TILE, n0 = blockIdx.y * GEMM_TILE, bz = blockIdx.z;
-    const int K = a.K, nstage = (K + 31) / 32;
+    const int K = a.K, n_last = min(n0 + GEMM_TILE - 1, a.N - 1);
+    if (a.skip_past >= 0 && m0 > a.skip_past + n_last) return;
+    const int nstage = ((a.klimit_past >= 0 ? min(K, a.klimit_past + n_last + 1) : K) + 31) / 32;
     const uint8_t *Ab = a.A + (size_t)bz * a.a_nb2;
     const uint16_t *Bb = a.B + (size_t)bz * a.N * K;
     // each thread moves two 16-byte chunks of A and two of B per stage: chunk c = tid + i*256 -> row c / 4, k-chunk c % 4
@@ -639,13 +666,13 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(gemm_f16_args a) {
 
 // used by the MatMul operator for (F16, F16) operands with many right-hand rows
 int spy_gemm_f16_launch(hipStream_t st, const void *A, int64_t a_nb1, int64_t a_nb2, const uint16_t *B, void *dst, int64_t d_nb1, int64_t d_nb2,
-                        int64_t M, int64_t N, int64_t K, int64_t nbatch) {
+                        int64_t M, int64_t N, int64_t K, int64_t nbatch, int skip_past, int klimit_past) {
     SPY_CHECK_ARG(A && B && dst && M > 0 && N > 0 && K >= 8 && nbatch > 0 && K % 8 == 0);
     SPY_CHECK_ARG(a_nb1 % 16 == 0 && a_nb2 % 16 == 0 && ((uintptr_t)A & 15) == 0 && ((uintptr_t)B & 15) == 0);
     SPY_CHECK_ARG((N + GEMM_TILE - 1) / GEMM_TILE <= 65535 && nbatch <= 65535);
     gemm_f16_args a;
     a.A = (const uint8_t *)A; a.B = B; a.dst = (uint8_t *)dst; a.M = (int)M; a.N = (int)N; a.K = (int)K;
-    a.a_nb1 = a_nb1; a.a_nb2 = a_nb2; a.d_nb1 = d_nb1; a.d_nb2 = d_nb2;
+    a.a_nb1 = a_nb1; a.a_nb2 = a_nb2; a.d_nb1 = d_nb1; a.d_nb2 = d_nb2; a.skip_past = skip_past; a.klimit_past = klimit_past;
     gemm_f16_kernel<<<dim3((unsigned)((M + GEMM_TILE - 1) / GEMM_TILE), (unsigned)((N + GEMM_TILE - 1) / GEMM_TILE), (unsigned)nbatch), dim3(256), 0, st>>>(a);
     return SPY_LAUNCH_RC();
 }

@@ -252,9 +252,9 @@ __global__ __launch_bounds__(256) void softmax_row_kernel(tdesc x, tdesc mask, b
 static int softmax_launch(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *mask, const spy_hip_tensor *dst, float scale, int causal_past);
 // Softmax under the causal mask of a pass that starts at position n_past, without reading a mask tensor (the token
 // loop fills its masks itself and knows their shape).  Same bits as spy_hip_op_softmax with that mask.
+int spy_softmax_row_ok(int64_t ne0) { return ne0 <= SOFTMAX_LDS_ROW && !getenv("SPY_HIP_SOFTMAX_GENERIC"); }   // rows of ne0 elements take the row kernel
 int spy_softmax_causal_launch(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *dst, float scale, int n_past) {
-    SPY_CHECK_ARG(n_past >= 0 && dst && scale > 0.0f);
-    if (dst->ne[0] > SOFTMAX_LDS_ROW) return SPY_HIP_EUNSUPPORTED;      // the caller falls back to the operator with a mask tensor
+    SPY_CHECK_ARG(n_past >= 0 && dst && scale > 0.0f && spy_softmax_row_ok(dst->ne[0]));
     return softmax_launch(stream, x, nullptr, dst, scale, n_past);
 }
 
@@ -276,7 +276,7 @@ static int softmax_launch(void *stream, const spy_hip_tensor *x, const spy_hip_t
     CHECK_GRID(nrow, 1);
     // a masked element of the generic kernel reads as (s + mask) * scale: the row kernel's shortcut needs scale > 0 and a
     // mask that really is 0 / -inf, which is what the graph builds (llama.cpp:248-263)
-    const bool row_ok = dst->ne[0] <= SOFTMAX_LDS_ROW && scale > 0.0f && !getenv("SPY_HIP_SOFTMAX_GENERIC");
+    const bool row_ok = spy_softmax_row_ok(dst->ne[0]) && scale > 0.0f;
     if (dst->type == SPY_HIP_F16 && !row_ok) return SPY_HIP_EUNSUPPORTED;
     if (row_ok) {
         const size_t lds = (size_t)dst->ne[0] * 4;
@@ -500,7 +500,7 @@ __global__ __launch_bounds__(256) void matmul_f16_kernel(tdesc w, const uint16_t
 }
 
 int spy_gemm_f16_launch(hipStream_t st, const void *A, int64_t a_nb1, int64_t a_nb2, const uint16_t *B, void *dst, int64_t d_nb1, int64_t d_nb2,
-                        int64_t M, int64_t N, int64_t K, int64_t nbatch);      // gemm.hip
+                        int64_t M, int64_t N, int64_t K, int64_t nbatch, int skip_past, int klimit_past);      // gemm.hip
 
 static int mid_type(int t0, int t1) {                                        // target_buffer_type (mat.cpp:32-42) + K-quants
     if (t0 == t1) return t0;
@@ -531,8 +531,23 @@ extern "C" size_t spy_hip_op_matmul_scratch_size(const spy_hip_tensor *w, const 
     return (size_t)(spy_t_nrow(x) * spy_row_size(tm, x->ne[0]));
 }
 
+static int matmul_impl(void *stream, const spy_hip_tensor *w, const spy_hip_tensor *x, const spy_hip_tensor *dst, void *scratch, size_t scratch_bytes,
+                       int skip_past, int klimit_past);
 extern "C" int spy_hip_op_matmul(void *stream, const spy_hip_tensor *w, const spy_hip_tensor *x, const spy_hip_tensor *dst,
                                  void *scratch, size_t scratch_bytes) {
+    return matmul_impl(stream, w, x, dst, scratch, scratch_bytes, -1, -1);
+}
+// The two attention products of a prompt pass that starts at position `past`, told about the causal structure so that
+// the fp16 GEMM leaves out what the mask removes anyway: which = 0: scores (rows of w = cache positions; tiles the
+// softmax will never read are not computed), which = 1: probabilities x V^T (the contraction stops where the
+// probabilities of a tile are all zero).  Other shapes / types run as the plain operator.
+int spy_matmul_causal(void *stream, const spy_hip_tensor *w, const spy_hip_tensor *x, const spy_hip_tensor *dst, void *scratch, size_t scratch_bytes,
+                      int which, int past) {
+    SPY_CHECK_ARG(past >= 0 && (which == 0 || which == 1));
+    return matmul_impl(stream, w, x, dst, scratch, scratch_bytes, which == 0 ? past : -1, which == 1 ? past : -1);
+}
+static int matmul_impl(void *stream, const spy_hip_tensor *w, const spy_hip_tensor *x, const spy_hip_tensor *dst, void *scratch, size_t scratch_bytes,
+                       int skip_past, int klimit_past) {
     SPY_CHECK_ARG(w && x && dst && w->data && x->data && dst->data);
     const int t0 = w->type, t1 = x->type, tm = mid_type(t0, t1);
     if (dst->type != SPY_HIP_F32) return SPY_HIP_EUNSUPPORTED;
@@ -596,7 +611,7 @@ extern "C" int spy_hip_op_matmul(void *stream, const spy_hip_tensor *w, const sp
         ((uintptr_t)w->data & 15) == 0 && ((uintptr_t)xm & 15) == 0 && dst->nb[1] % 4 == 0 && dst->nb[2] % 4 == 0 && ne02 <= 65535) {
         for (int64_t i3 = 0; i3 < ne03; i3++) {            // prompt-sized attention products: fp16 MFMA
             int rc = spy_gemm_f16_launch(st, (const uint8_t *)w->data + i3 * w->nb[3], w->nb[1], w->nb[2], (const uint16_t *)xm + i3 * ne12 * ne11 * ne00,
-                                         (uint8_t *)dst->data + i3 * dst->nb[3], dst->nb[1], dst->nb[2], ne01, ne11, ne00, ne02);
+                                         (uint8_t *)dst->data + i3 * dst->nb[3], dst->nb[1], dst->nb[2], ne01, ne11, ne00, ne02, skip_past, klimit_past);
             if (rc) return rc;
         }
         return 0;

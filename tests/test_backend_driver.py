@@ -69,16 +69,20 @@ def test_submit_path_matches_oracle_and_engine(wtype):
 
 @pytest.mark.gpu
 def test_engine_prompt_softmax_without_mask_tensor_matches_submit_path():
-    """The engine's prompt pass tells its softmax the causal shape as a number (no mask tensor read) and
-    hands the probabilities over as fp16; the submit path runs Softmax with the graph's mask tensor
-    (llama.cpp:248-263).  Same bits, also for a second pass on top of a filled cache."""
+    """The engine's prompt pass tells its softmax and its two attention products the causal shape as a number (no
+    mask tensor read, tiles above the diagonal left out) and hands the probabilities over as fp16; the submit path
+    runs MatMul / Softmax / MatMul with the graph's mask tensor (llama.cpp:248-263).  Same bits, also for passes on
+    top of a filled cache."""
     from spy_amd import backend_driver as B
     from spy_amd import model as M
-    cfg = M.Config(n_layer=2, n_embd=256, n_head=2, n_ff=768, n_vocab=512, n_ctx=96, wtype=O.Q4_0)
+    cfg = M.Config(n_layer=2, n_embd=256, n_head=2, n_ff=768, n_vocab=512, n_ctx=448, wtype=O.Q4_0)
     tensors = M.synth_model(cfg, seed=11)
     host, eng = B.HostModel(cfg, tensors), M.Engine(cfg, tensors)
-    prompt = np.random.default_rng(5).integers(0, cfg.n_vocab, 72).astype(np.int32)
-    for start, stop in ((0, 40), (40, 72)):                # 40 and 32 tokens: rows of 40 and 72 cached positions
+    prompt = np.random.default_rng(5).integers(0, cfg.n_vocab, 438).astype(np.int32)
+    # passes of 168, 136 and 134 tokens: the attention products span several 128 x 128 tiles, some of them entirely
+    # above the causal diagonal (left out by the engine); the last pass has rows of 438 positions (not a multiple of 8:
+    # probabilities handed over as fp32)
+    for start, stop in ((0, 168), (168, 304), (304, 438)):
         lg_h, lg_e = host.forward(prompt[start:stop], start), eng.forward(prompt[start:stop], start)
         assert np.isfinite(lg_e).all()
         assert np.array_equal(lg_h, lg_e), (start, stop)
