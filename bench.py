@@ -132,7 +132,7 @@ def main():
     log("decode: %.3f ms/step wall, %.3f ms/step by HIP events, %.1f tok/s, %.2f GB/token -> %.1f%% of 8 TB/s"
         % (ms_per_step, ev_ms, tok_s, bytes_per_token / 1e9, 100 * frac))
 
-    # dominant kernel: the gate|up projection with the fused RMSNorm / Q8_0 / SiLU epilogue
+    # per-kernel times: HIP events around repeated launches of each kernel of a layer, on the stream they run on
     per_kernel = {}
     for name in ("qkv", "scores", "pv", "wo", "gate_up", "down", "head"):
         per_kernel[name] = eng.kernel_time_us(name, reps=4)
@@ -150,14 +150,25 @@ def main():
     log("per-kernel (HIP events, walking the layers):")
     for k, us in per_kernel.items():
         log("  %-8s %8.2f us  %7.1f GB/s  (%.1f%% of 8 TB/s)" % (k, us, alg[k] / us / 1e3, alg[k] / us / 1e3 / 80))
-    dom = "gate_up"
-    # HBM bytes per launch of that kernel from profiler counters (FETCH_SIZE + WRITE_SIZE scaled by a copy
-    # kernel of known size; profiles/decode_7b_q4_0_ctx4096_hbm_traffic.md): valid for this shape only
-    traffic = 51.18e6 if (cfg.n_embd, cfg.n_ff, cfg.wtype, args.model) == (4096, 11008, H.Q4_0, "q4_0") else None
-    achieved = alg[dom] / (per_kernel[dom] * 1e-6) / 1e9
-    roofline = {"kernel": "wave_gemv_kernel<Q4_0, gate|up + SiLU>", "bound": "hbm", "achieved": round(achieved, 1), "peak": 8000.0,
-                "unit": "GB/s", "frac": round(achieved / 8000.0, 4), "traffic": traffic,
-                "bytes_per_launch": alg[dom], "us_per_launch": round(per_kernel[dom], 3)}
+    # dominant kernel = largest share of the step: launches per token x time per launch
+    count = {k: (1 if k == "head" else cfg.n_layer) for k in per_kernel}
+    dom = max(per_kernel, key=lambda k: per_kernel[k] * count[k])
+    names = {"attention (qkv+scores+pv)": "attn_layer_kernel<Q4_0> (RMSNorm, Q8_0, wq|wk|wv, RoPE, cache write, q.K, softmax, P.V^T)",
+             "gate_up": "wave_gemv_kernel<gate|up + SiLU>", "down": "wave_gemv_kernel<down + residual>", "wo": "wave_gemv_kernel<wo + residual>",
+             "head": "wave_gemv_kernel<output head>", "qkv": "wave_gemv_kernel<qkv>", "scores": "attn_scores_kernel", "pv": "attn_pv_kernel"}
+    # HBM bytes per launch from profiler counters (FETCH_SIZE + WRITE_SIZE, each scaled by what the same counter reads for a
+    # copy kernel of known size; profiles/decode_7b_q4_0_ctx4096_hbm_traffic.md): measured for this model shape only.  The
+    # attention launch was counted at n_kv = 4103 (101.6 MB for 95.5 MB algorithmic); its traffic is scaled to this run's n_kv.
+    measured = {"gate_up": 51.18e6, "down": 25.83e6, "wo": 9.65e6, "head": 108.26e6,
+                "attention (qkv+scores+pv)": 101.6e6 * alg.get("attention (qkv+scores+pv)", 0) / (28311552 + 2 * 4103 * 8192)}
+    shape_ok = (cfg.n_embd, cfg.n_ff, cfg.wtype, args.model, cfg.t_out) == (4096, 11008, H.Q4_0, "q4_0", H.Q6_K) and cfg.n_layer == 32
+    def roof(k):
+        ach = alg[k] / (per_kernel[k] * 1e-6) / 1e9
+        return {"kernel": names.get(k, k), "bound": "hbm", "achieved": round(ach, 1), "peak": 8000.0, "unit": "GB/s", "frac": round(ach / 8000.0, 4),
+                "traffic": round(measured[k]) if shape_ok and k in measured else None, "bytes_per_launch": int(alg[k]),
+                "us_per_launch": round(per_kernel[k], 3), "launches_per_token": count[k], "share_of_step": round(per_kernel[k] * count[k] / (ev_ms * 1e3), 3)}
+    roofline = roof(dom)
+    roofline_others = {k: roof(k) for k in per_kernel if k != dom}
 
     cpu = None
     if not args.no_cpu:
@@ -192,7 +203,7 @@ def main():
         "hbm_roofline_frac": round(frac, 4), "ms_per_step_hip_events": round(ev_ms, 4),
         "prefill": {"tokens": fill, "seconds": round(prefill_s, 3), "tok_s": round(fill / prefill_s, 1)} if args.prefill == "real" else None,
         "kernel_us": {k: round(v, 2) for k, v in per_kernel.items()},
-        "roofline": roofline, "cpu_baseline": cpu,
+        "roofline": roofline, "roofline_other_kernels": roofline_others, "cpu_baseline": cpu,
     }
     if load_info:
         out["gguf_load"] = load_info
