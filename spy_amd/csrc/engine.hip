@@ -266,6 +266,8 @@ static spy_hip_tensor T3s(int type, void *p, int64_t e0, int64_t e1, int64_t e2,
 
 int spy_matmul_causal(void *stream, const spy_hip_tensor *w, const spy_hip_tensor *x, const spy_hip_tensor *dst, void *scratch, size_t scratch_bytes,
                       int which, int past);                                                                                  // ops.hip
+int spy_norm_mul_q8_launch(hipStream_t st, const float *x, int64_t x_stride, const float *w, float eps, void *y, int64_t nrow, int64_t K);   // prompt_fused.hip
+int spy_silu_mul_q8_launch(hipStream_t st, const float *gate, const float *up, void *y, int64_t nrow, int64_t F);                           // prompt_fused.hip
 int spy_softmax_causal_launch(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *dst, float scale, int n_past);   // ops.hip
 int spy_softmax_row_ok(int64_t ne0);                                                                                         // ops.hip
 
@@ -329,14 +331,24 @@ static int forward_ops(spy_hip_llama *m, hipStream_t st, const int32_t *tokens_h
         spy_hip_tensor tw = T2(wt, (void *)w, K, M);
         return spy_hip_op_matmul(st, &tw, xin, out, scr, scr_bytes);
     };
+    // Passes over many tokens (every MatMul on the matrix cores): the elementwise operators between two MatMuls write the
+    // next MatMul's Q8_0 activations directly (same bytes as the separate operators: prompt_fused.hip)
+    const bool fuse_act = T >= 16 && d % 64 == 0 && F % 64 == 0 && !getenv("SPY_HIP_PROMPT_UNFUSED");
     for (int il = 0; il < c.n_layer; il++) {
         const spy_hip_llama_layer &L = m->layers[il];
         spy_hip_tensor t_nw = T2(SPY_HIP_F32, (void *)L.attn_norm, d, 1); t_nw.dim = 1;
-        RC_TRY(spy_hip_op_norm_rms(st, &t_x, &t_xn, c.eps));
-        RC_TRY(spy_hip_op_binary(st, 2, &t_xn, &t_nw, &t_xn));
-        RC_TRY(mm(L.wq, L.t_wq, d, d, &t_xn, &t_q));
-        RC_TRY(mm(L.wk, L.t_wk, d, d, &t_xn, &t_k));
-        RC_TRY(mm(L.wv, L.t_wv, d, d, &t_xn, &t_v));
+        if (fuse_act) {           // NormRMS -> Mul -> Q8_0 in one kernel, quantized once for the three MatMuls
+            RC_TRY(spy_norm_mul_q8_launch(st, x, 4 * d, (const float *)L.attn_norm, c.eps, scr, T, d));
+            RC_TRY(spy_hip_gemm_q8_0act(st, L.t_wq, L.wq, scr, q, d, d, T, d));
+            RC_TRY(spy_hip_gemm_q8_0act(st, L.t_wk, L.wk, scr, k, d, d, T, d));
+            RC_TRY(spy_hip_gemm_q8_0act(st, L.t_wv, L.wv, scr, v, d, d, T, d));
+        } else {
+            RC_TRY(spy_hip_op_norm_rms(st, &t_x, &t_xn, c.eps));
+            RC_TRY(spy_hip_op_binary(st, 2, &t_xn, &t_nw, &t_xn));
+            RC_TRY(mm(L.wq, L.t_wq, d, d, &t_xn, &t_q));
+            RC_TRY(mm(L.wk, L.t_wk, d, d, &t_xn, &t_k));
+            RC_TRY(mm(L.wv, L.t_wv, d, d, &t_xn, &t_v));
+        }
         spy_hip_tensor t_q3 = T3s(SPY_HIP_F32, q, hd, H, T, 4, 4 * hd, 4 * d), t_k3 = T3s(SPY_HIP_F32, k, hd, H, T, 4, 4 * hd, 4 * d);
         RC_TRY(spy_hip_op_rope(st, &t_q3, &t_pos, &t_q3, &rp));
         RC_TRY(spy_hip_op_rope(st, &t_k3, &t_pos, &t_k3, &rp));
@@ -368,13 +380,21 @@ static int forward_ops(spy_hip_llama *m, hipStream_t st, const int32_t *tokens_h
         RC_TRY(mm(L.wo, L.t_wo, d, d, &t_o2, &t_t1));
         RC_TRY(spy_hip_op_binary(st, 0, &t_t1, &t_x, &t_t1));
         t_nw.data = (void *)L.ffn_norm;
-        RC_TRY(spy_hip_op_norm_rms(st, &t_t1, &t_xn, c.eps));
-        RC_TRY(spy_hip_op_binary(st, 2, &t_xn, &t_nw, &t_xn));
-        RC_TRY(mm(L.w_up, L.t_up, d, F, &t_xn, &t_up));
-        RC_TRY(mm(L.w_gate, L.t_gate, d, F, &t_xn, &t_gate));
-        RC_TRY(spy_hip_op_silu(st, &t_gate, &t_gate));
-        RC_TRY(spy_hip_op_binary(st, 2, &t_up, &t_gate, &t_par));
-        RC_TRY(mm(L.w_down, L.t_down, F, d, &t_par, &t_od));
+        if (fuse_act) {
+            RC_TRY(spy_norm_mul_q8_launch(st, t1, 4 * d, (const float *)L.ffn_norm, c.eps, scr, T, d));
+            RC_TRY(spy_hip_gemm_q8_0act(st, L.t_up, L.w_up, scr, up, F, d, T, F));
+            RC_TRY(spy_hip_gemm_q8_0act(st, L.t_gate, L.w_gate, scr, gate, F, d, T, F));
+            RC_TRY(spy_silu_mul_q8_launch(st, gate, up, scr, T, F));        // Silu -> Mul -> Q8_0
+            RC_TRY(spy_hip_gemm_q8_0act(st, L.t_down, L.w_down, scr, o, d, F, T, d));
+        } else {
+            RC_TRY(spy_hip_op_norm_rms(st, &t_t1, &t_xn, c.eps));
+            RC_TRY(spy_hip_op_binary(st, 2, &t_xn, &t_nw, &t_xn));
+            RC_TRY(mm(L.w_up, L.t_up, d, F, &t_xn, &t_up));
+            RC_TRY(mm(L.w_gate, L.t_gate, d, F, &t_xn, &t_gate));
+            RC_TRY(spy_hip_op_silu(st, &t_gate, &t_gate));
+            RC_TRY(spy_hip_op_binary(st, 2, &t_up, &t_gate, &t_par));
+            RC_TRY(mm(L.w_down, L.t_down, F, d, &t_par, &t_od));
+        }
         RC_TRY(spy_hip_op_binary(st, 0, &t_t1, &t_od, &t_x));
     }
     {
