@@ -268,6 +268,9 @@ int spy_matmul_causal(void *stream, const spy_hip_tensor *w, const spy_hip_tenso
                       int which, int past);                                                                                  // ops.hip
 int spy_norm_mul_q8_launch(hipStream_t st, const float *x, int64_t x_stride, const float *w, float eps, void *y, int64_t nrow, int64_t K);   // prompt_fused.hip
 int spy_silu_mul_q8_launch(hipStream_t st, const float *gate, const float *up, void *y, int64_t nrow, int64_t F);                           // prompt_fused.hip
+int spy_rope_table_launch(hipStream_t st, float *table, int past, int T, int hd, float freq_base, float freq_scale, float mscale);       // prompt_fused.hip
+int spy_rope_store_launch(hipStream_t st, const float *q, const float *k, const float *table, uint16_t *q16, uint16_t *kc, int T, int H, int hd);
+int spy_vt_store_launch(hipStream_t st, const float *v, uint16_t *vc, int T, int d, int64_t n_ctx);
 int spy_softmax_causal_launch(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *dst, float scale, int n_past);   // ops.hip
 int spy_softmax_row_ok(int64_t ne0);                                                                                         // ops.hip
 
@@ -289,7 +292,7 @@ static int forward_ops(spy_hip_llama *m, hipStream_t st, const int32_t *tokens_h
     const size_t o_x = take(d * T * 4), o_xn = take(d * T * 4), o_q = take(d * T * 4), o_k = take(d * T * 4), o_v = take(d * T * 4),
                  o_o = take(d * T * 4), o_o2 = take(d * T * 4), o_t1 = take(d * T * 4), o_up = take(F * T * 4), o_gate = take(F * T * 4),
                  o_par = take(F * T * 4), o_S = take(n_kv * T * H * 4), o_P = take(n_kv * T * H * 4), o_mask = take(C * T * 4),
-                 o_ids = take(T * 4), o_pos = take(T * 4), o_logits = take(V * T * 4);
+                 o_ids = take(T * 4), o_pos = take(T * 4), o_logits = take(V * T * 4), o_rt = take(T * hd * 4);
     const size_t act_q8 = (size_t)T * ((F > d ? F : d) / 32) * 34;
     const size_t act_f16 = (size_t)n_kv * T * H * 2 > (size_t)d * T * 2 ? (size_t)n_kv * T * H * 2 : (size_t)d * T * 2;
     const size_t o_scr = take(act_q8 > act_f16 ? act_q8 : act_f16);
@@ -334,6 +337,8 @@ static int forward_ops(spy_hip_llama *m, hipStream_t st, const int32_t *tokens_h
     // Passes over many tokens (every MatMul on the matrix cores): the elementwise operators between two MatMuls write the
     // next MatMul's Q8_0 activations directly (same bytes as the separate operators: prompt_fused.hip)
     const bool fuse_act = T >= 16 && d % 64 == 0 && F % 64 == 0 && !getenv("SPY_HIP_PROMPT_UNFUSED");
+    float *rope_tab = (float *)(B + o_rt);
+    if (fuse_act) RC_TRY(spy_rope_table_launch(st, rope_tab, P, T, (int)hd, rp.freq_base, rp.freq_scale, rp.attention_factor));
     for (int il = 0; il < c.n_layer; il++) {
         const spy_hip_llama_layer &L = m->layers[il];
         spy_hip_tensor t_nw = T2(SPY_HIP_F32, (void *)L.attn_norm, d, 1); t_nw.dim = 1;
@@ -349,16 +354,23 @@ static int forward_ops(spy_hip_llama *m, hipStream_t st, const int32_t *tokens_h
             RC_TRY(mm(L.wk, L.t_wk, d, d, &t_xn, &t_k));
             RC_TRY(mm(L.wv, L.t_wv, d, d, &t_xn, &t_v));
         }
-        spy_hip_tensor t_q3 = T3s(SPY_HIP_F32, q, hd, H, T, 4, 4 * hd, 4 * d), t_k3 = T3s(SPY_HIP_F32, k, hd, H, T, 4, 4 * hd, 4 * d);
-        RC_TRY(spy_hip_op_rope(st, &t_q3, &t_pos, &t_q3, &rp));
-        RC_TRY(spy_hip_op_rope(st, &t_k3, &t_pos, &t_k3, &rp));
-        spy_hip_tensor t_qp = T3s(SPY_HIP_F32, q, hd, T, H, 4, 4 * d, 4 * hd);                         // Permute {0,2,1,3}
-        spy_hip_tensor t_vt = T2(SPY_HIP_F32, v, T, d); t_vt.nb[0] = 4 * d; t_vt.nb[1] = 4; t_vt.nb[2] = t_vt.nb[3] = 4 * d * T;   // Transpose
-        spy_hip_tensor t_kc = T2(SPY_HIP_F16, (uint8_t *)m->k_cache[il] + 2 * d * P, (int64_t)T * d, 1); t_kc.dim = 1;
-        RC_TRY(spy_hip_op_dup(st, &t_k3, &t_kc));
-        spy_hip_tensor t_vc = T2(SPY_HIP_F16, (uint8_t *)m->v_cache[il] + 2 * (int64_t)P, T, d);
-        t_vc.nb[0] = 2; t_vc.nb[1] = 2 * C; t_vc.nb[2] = t_vc.nb[3] = d * 2 * C;
-        RC_TRY(spy_hip_op_dup(st, &t_vt, &t_vc));
+        spy_hip_tensor t_qp;
+        if (fuse_act) {           // Rope(q), Rope(k), the fp16 conversion of q and both cache writes in two kernels (prompt_fused.hip)
+            RC_TRY(spy_rope_store_launch(st, q, k, rope_tab, (uint16_t *)xn, (uint16_t *)m->k_cache[il] + d * P, T, (int)H, (int)hd));
+            RC_TRY(spy_vt_store_launch(st, v, (uint16_t *)m->v_cache[il] + P, T, (int)d, C));
+            t_qp = T3s(SPY_HIP_F16, xn, hd, T, H, 2, 2 * hd, 2 * hd * T);
+        } else {
+            spy_hip_tensor t_q3 = T3s(SPY_HIP_F32, q, hd, H, T, 4, 4 * hd, 4 * d), t_k3 = T3s(SPY_HIP_F32, k, hd, H, T, 4, 4 * hd, 4 * d);
+            RC_TRY(spy_hip_op_rope(st, &t_q3, &t_pos, &t_q3, &rp));
+            RC_TRY(spy_hip_op_rope(st, &t_k3, &t_pos, &t_k3, &rp));
+            t_qp = T3s(SPY_HIP_F32, q, hd, T, H, 4, 4 * d, 4 * hd);                                        // Permute {0,2,1,3}
+            spy_hip_tensor t_vt = T2(SPY_HIP_F32, v, T, d); t_vt.nb[0] = 4 * d; t_vt.nb[1] = 4; t_vt.nb[2] = t_vt.nb[3] = 4 * d * T;   // Transpose
+            spy_hip_tensor t_kc = T2(SPY_HIP_F16, (uint8_t *)m->k_cache[il] + 2 * d * P, (int64_t)T * d, 1); t_kc.dim = 1;
+            RC_TRY(spy_hip_op_dup(st, &t_k3, &t_kc));
+            spy_hip_tensor t_vc = T2(SPY_HIP_F16, (uint8_t *)m->v_cache[il] + 2 * (int64_t)P, T, d);
+            t_vc.nb[0] = 2; t_vc.nb[1] = 2 * C; t_vc.nb[2] = t_vc.nb[3] = d * 2 * C;
+            RC_TRY(spy_hip_op_dup(st, &t_vt, &t_vc));
+        }
         spy_hip_tensor t_kall = T3s(SPY_HIP_F16, m->k_cache[il], hd, n_kv, H, 2, 2 * d, 2 * hd);
         spy_hip_tensor t_vall = T3s(SPY_HIP_F16, m->v_cache[il], n_kv, hd, H, 2, 2 * C, 2 * C * hd);
         // causal_ok: the softmax below takes the row kernel, which reads no score beyond a row's causal length and writes
@@ -372,11 +384,15 @@ static int forward_ops(spy_hip_llama *m, hipStream_t st, const int32_t *tokens_h
         RC_TRY(causal_ok ? spy_matmul_causal(st, &t_kall, &t_qp, &t_S, scr, scr_bytes, 0, P) : spy_hip_op_matmul(st, &t_kall, &t_qp, &t_S, scr, scr_bytes));
         // the mask of this pass is the causal one filled above: the row kernel takes its shape as a number
         RC_TRY(causal_ok ? spy_softmax_causal_launch(st, &t_S, &t_P, scale, P) : spy_hip_op_softmax(st, &t_S, &t_mask, &t_P, scale));
-        spy_hip_tensor t_O = T3s(SPY_HIP_F32, o, hd, T, H, 4, 4 * hd, 4 * hd * T);
+        // fused: the product writes [hd, T, H] through the strides of the permuted view, i.e. straight into the contiguous
+        // [hd, H, T] buffer the next MatMul reads (Permute {0,2,1,3} + Contiguous without a copy)
+        spy_hip_tensor t_O = fuse_act ? T3s(SPY_HIP_F32, o2, hd, T, H, 4, 4 * d, 4 * hd) : T3s(SPY_HIP_F32, o, hd, T, H, 4, 4 * hd, 4 * hd * T);
         RC_TRY(causal_ok ? spy_matmul_causal(st, &t_vall, &t_P, &t_O, scr, scr_bytes, 1, P) : spy_hip_op_matmul(st, &t_vall, &t_P, &t_O, scr, scr_bytes));
-        spy_hip_tensor t_Op = T3s(SPY_HIP_F32, o, hd, H, T, 4, 4 * hd * T, 4 * hd);                    // Permute {0,2,1,3}
-        spy_hip_tensor t_o2c = T3s(SPY_HIP_F32, o2, hd, H, T, 4, 4 * hd, 4 * d);
-        RC_TRY(spy_hip_op_contiguous(st, &t_Op, &t_o2c));
+        if (!fuse_act) {
+            spy_hip_tensor t_Op = T3s(SPY_HIP_F32, o, hd, H, T, 4, 4 * hd * T, 4 * hd);                // Permute {0,2,1,3}
+            spy_hip_tensor t_o2c = T3s(SPY_HIP_F32, o2, hd, H, T, 4, 4 * hd, 4 * d);
+            RC_TRY(spy_hip_op_contiguous(st, &t_Op, &t_o2c));
+        }
         RC_TRY(mm(L.wo, L.t_wo, d, d, &t_o2, &t_t1));
         RC_TRY(spy_hip_op_binary(st, 0, &t_t1, &t_x, &t_t1));
         t_nw.data = (void *)L.ffn_norm;
@@ -399,10 +415,15 @@ static int forward_ops(spy_hip_llama *m, hipStream_t st, const int32_t *tokens_h
     }
     {
         spy_hip_tensor t_nw = T2(SPY_HIP_F32, (void *)c.out_norm, d, 1); t_nw.dim = 1;
-        RC_TRY(spy_hip_op_norm_rms(st, &t_x, &t_xn, c.eps));
-        RC_TRY(spy_hip_op_binary(st, 2, &t_xn, &t_nw, &t_xn));
         spy_hip_tensor t_l = T2(SPY_HIP_F32, lg, V, T);
-        RC_TRY(mm(c.w_out, c.t_out, d, V, &t_xn, &t_l));
+        if (fuse_act) {
+            RC_TRY(spy_norm_mul_q8_launch(st, x, 4 * d, (const float *)c.out_norm, c.eps, scr, T, d));
+            RC_TRY(spy_hip_gemm_q8_0act(st, c.t_out, c.w_out, scr, lg, V, d, T, V));
+        } else {
+            RC_TRY(spy_hip_op_norm_rms(st, &t_x, &t_xn, c.eps));
+            RC_TRY(spy_hip_op_binary(st, 2, &t_xn, &t_nw, &t_xn));
+            RC_TRY(mm(c.w_out, c.t_out, d, V, &t_xn, &t_l));
+        }
     }
     if (logits_host) HIP_TRY(hipMemcpyAsync(logits_host, lg, (size_t)V * T * 4, hipMemcpyDeviceToHost, st));
     HIP_TRY(hipStreamSynchronize(st));

@@ -78,3 +78,72 @@ int spy_silu_mul_q8_launch(hipStream_t st, const float *gate, const float *up, v
     silu_mul_q8_kernel<<<dim3((unsigned)((total4 + 255) / 256)), dim3(256), 0, st>>>((const float4 *)gate, (const float4 *)up, (uint8_t *)y, total4);
     return SPY_LAUNCH_RC();
 }
+
+// ---- RoPE + cache writes of a prompt pass -----------------------------------------------------------
+// Rope (non-linear.cpp:270-371, default branch) rotates q and k of every layer by angles that depend on
+// the position and the pair index only: they are computed once per pass into a table, with the
+// arithmetic of the operator kernel (theta built by k successive fp32 multiplications, :304-309; cosf /
+// sinf of theta * freq_scale, times the attention factor).  Per layer one kernel then rotates q and k
+// and stores them where the next operators read them: q as fp16 [head][token][hd] (the conversion the
+// score product applies to its right operand, mat.cpp:37) and k as fp16 into the K cache rows of the
+// pass (the Copy of view.cpp:83-227); a second kernel transposes v into the V^T cache.
+__global__ __launch_bounds__(64) void rope_table_kernel(float2 *__restrict__ table, int past, int npair, float theta_scale, float freq_scale, float mscale) {
+    const int t = blockIdx.x;
+    const float p = (float)(past + t);
+    for (int k = threadIdx.x; k < npair; k += 64) {
+        float theta = p;
+        for (int j = 0; j < k; j++) theta *= theta_scale;
+        const float ang = freq_scale * theta;
+        table[(size_t)t * npair + k] = make_float2(cosf(ang) * mscale, sinf(ang) * mscale);
+    }
+}
+
+// grid (T, H); q, k: f32 [T][H * hd]; q16: fp16 [H][T][hd]; kc: K cache row of the pass's first token, fp16 [T][H * hd]
+__global__ __launch_bounds__(64) void rope_store_kernel(const float *__restrict__ q, const float *__restrict__ k, const float2 *__restrict__ table,
+                                                        uint16_t *__restrict__ q16, uint16_t *__restrict__ kc, int T, int H, int hd) {
+    const int t = blockIdx.x, h = blockIdx.y, npair = hd / 2;
+    const size_t row = ((size_t)t * H + h) * hd;
+    for (int p = threadIdx.x; p < npair; p += 64) {
+        const float2 cs = table[(size_t)t * npair + p];
+        const float2 a = *(const float2 *)(q + row + 2 * p), b = *(const float2 *)(k + row + 2 * p);
+        const float q0 = a.x * cs.x - a.y * cs.y, q1 = a.x * cs.y + a.y * cs.x;
+        const float k0 = b.x * cs.x - b.y * cs.y, k1 = b.x * cs.y + b.y * cs.x;
+        *(uint32_t *)(q16 + ((size_t)h * T + t) * hd + 2 * p) = (uint32_t)f2h(q0) | ((uint32_t)f2h(q1) << 16);
+        *(uint32_t *)(kc + row + 2 * p) = (uint32_t)f2h(k0) | ((uint32_t)f2h(k1) << 16);
+    }
+}
+
+// v: f32 [T][d] -> V^T cache: fp16 vc[col * n_ctx + t] for t < T (vc points at the pass's first position); 64 x 64 tiles through LDS
+__global__ __launch_bounds__(256) void vt_store_kernel(const float *__restrict__ v, uint16_t *__restrict__ vc, int T, int d, int64_t n_ctx) {
+    __shared__ uint16_t tile[64][66];
+    const int t0 = blockIdx.x * 64, c0 = blockIdx.y * 64;
+    for (int i = threadIdx.x; i < 64 * 64; i += 256) {
+        const int tt = i >> 6, cc = i & 63;
+        tile[tt][cc] = (t0 + tt < T && c0 + cc < d) ? f2h(v[(size_t)(t0 + tt) * d + c0 + cc]) : (uint16_t)0;
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < 64 * 64; i += 256) {
+        const int cc = i >> 6, tt = i & 63;
+        if (t0 + tt < T && c0 + cc < d) vc[(size_t)(c0 + cc) * n_ctx + t0 + tt] = tile[tt][cc];
+    }
+}
+
+int spy_rope_table_launch(hipStream_t st, float *table, int past, int T, int hd, float freq_base, float freq_scale, float mscale) {
+    SPY_CHECK_ARG(table && past >= 0 && T > 0 && hd > 0 && hd % 2 == 0);
+    const float theta_scale = powf(freq_base, -2.0f / (float)hd);             // host libm, as the reference (:282)
+    rope_table_kernel<<<dim3((unsigned)T), dim3(64), 0, st>>>((float2 *)table, past, hd / 2, theta_scale, freq_scale, mscale);
+    return SPY_LAUNCH_RC();
+}
+
+int spy_rope_store_launch(hipStream_t st, const float *q, const float *k, const float *table, uint16_t *q16, uint16_t *kc, int T, int H, int hd) {
+    SPY_CHECK_ARG(q && k && table && q16 && kc && T > 0 && H > 0 && H < 65536 && hd > 0 && hd % 2 == 0);
+    SPY_CHECK_ARG(((uintptr_t)q % 8) == 0 && ((uintptr_t)k % 8) == 0 && ((uintptr_t)table % 8) == 0 && ((uintptr_t)q16 % 4) == 0 && ((uintptr_t)kc % 4) == 0);
+    rope_store_kernel<<<dim3((unsigned)T, (unsigned)H), dim3(64), 0, st>>>(q, k, (const float2 *)table, q16, kc, T, H, hd);
+    return SPY_LAUNCH_RC();
+}
+
+int spy_vt_store_launch(hipStream_t st, const float *v, uint16_t *vc, int T, int d, int64_t n_ctx) {
+    SPY_CHECK_ARG(v && vc && T > 0 && d > 0 && n_ctx >= T && (d + 63) / 64 < 65536);
+    vt_store_kernel<<<dim3((unsigned)((T + 63) / 64), (unsigned)((d + 63) / 64)), dim3(256), 0, st>>>(v, vc, T, d, n_ctx);
+    return SPY_LAUNCH_RC();
+}
