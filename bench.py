@@ -88,9 +88,7 @@ def main():
     prompt = rng.integers(0, cfg.n_vocab, fill).astype(np.int32)
     t0 = time.time()
     if args.prefill == "real":
-        logits = eng.forward(prompt, 0, want_logits=False)
-        last = eng.forward(prompt[-1:], fill - 1)          # re-run the last prompt token alone to get its logits
-        first = int(np.argmax(last[0]))
+        first = int(np.argmax(eng.forward_last(prompt, 0)))   # the prompt pass; output head on the last token only
     else:
         for il in range(cfg.n_layer):
             eng.write_buffer("k_cache", il, (rng.standard_normal(fill * cfg.n_embd) * 1.3).astype(np.float16).view(np.uint16))

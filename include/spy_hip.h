@@ -181,6 +181,12 @@ int spy_hip_llama_destroy(spy_hip_llama *m);
  * than one token run operator by operator).  logits_host: NULL or n_vocab*n_token floats. */
 int spy_hip_llama_forward(spy_hip_llama *m, void *stream, const int32_t *tokens_host, int32_t n_token, int32_t n_past,
                           float *logits_host);
+/* The same pass with the output head applied to the last token only: logits_last_host receives
+ * n_vocab floats (NULL: no head at all).  What a token loop needs from a prompt: the reference's graph
+ * computes the logits of every prompt token (llama.cpp:86-313) and the loop then samples from the last
+ * row (cli.h:88-100); the other rows, n_vocab*(n_token-1) floats, are neither computed nor copied here. */
+int spy_hip_llama_forward_last(spy_hip_llama *m, void *stream, const int32_t *tokens_host, int32_t n_token, int32_t n_past,
+                               float *logits_last_host);
 /* n_steps single-token passes with greedy sampling on the device: step i consumes the token
  * sampled by step i-1 (the first consumes first_token at position n_past) and tokens_host[i]
  * receives the token sampled by step i.  use_graph: replay a captured HIP graph. */

@@ -98,6 +98,7 @@ SIGNATURES = {
     "spy_hip_llama_create": (_i32, [C.POINTER(LlamaDesc), C.POINTER(_vp)]),
     "spy_hip_llama_destroy": (_i32, [_vp]),
     "spy_hip_llama_forward": (_i32, [_vp, _vp, _vp, _i32, _i32, _vp]),
+    "spy_hip_llama_forward_last": (_i32, [_vp, _vp, _vp, _i32, _i32, _vp]),
     "spy_hip_llama_decode_greedy": (_i32, [_vp, _vp, _i32, _i32, _i32, _vp, _i32]),
     "spy_hip_llama_buffer": (_i32, [_vp, C.c_char_p, _i32, C.POINTER(_vp), C.POINTER(_sz)]),
     "spy_hip_llama_timing": (_i32, [_vp, C.POINTER(_f32), C.POINTER(_i32)]),

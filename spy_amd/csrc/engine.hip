@@ -283,7 +283,8 @@ __global__ __launch_bounds__(256) void causal_mask_kernel(float *__restrict__ ma
 #ifndef SPY_PREFILL_CHUNK
 #define SPY_PREFILL_CHUNK 2048        // tokens per operator-by-operator pass of a long prompt (4096-token prompt: 0.33 s with 512, 0.27 with 1024, 0.24 with 2048, 0.25 with 4096)
 #endif
-static int forward_ops(spy_hip_llama *m, hipStream_t st, const int32_t *tokens_host, int T, int P, float *logits_host) {
+enum { HEAD_ALL = 0, HEAD_NONE = 1, HEAD_LAST = 2 };     // output head of a pass: every token's logits (the reference's graph), none, the last token's
+static int forward_ops(spy_hip_llama *m, hipStream_t st, const int32_t *tokens_host, int T, int P, float *logits_host, int head) {
     const spy_hip_llama_desc &c = m->desc;
     const int64_t d = c.n_embd, F = c.n_ff, C = c.n_ctx, H = c.n_head, hd = m->hd, V = c.n_vocab, n_kv = (int64_t)P + T;
     // scratch layout (bytes)
@@ -413,7 +414,7 @@ static int forward_ops(spy_hip_llama *m, hipStream_t st, const int32_t *tokens_h
         }
         RC_TRY(spy_hip_op_binary(st, 0, &t_t1, &t_od, &t_x));
     }
-    {
+    if (head == HEAD_ALL) {
         spy_hip_tensor t_nw = T2(SPY_HIP_F32, (void *)c.out_norm, d, 1); t_nw.dim = 1;
         spy_hip_tensor t_l = T2(SPY_HIP_F32, lg, V, T);
         if (fuse_act) {
@@ -424,14 +425,20 @@ static int forward_ops(spy_hip_llama *m, hipStream_t st, const int32_t *tokens_h
             RC_TRY(spy_hip_op_binary(st, 2, &t_xn, &t_nw, &t_xn));
             RC_TRY(mm(c.w_out, c.t_out, d, V, &t_xn, &t_l));
         }
+    } else if (head == HEAD_LAST) {         // the three head operators on the last token's row only
+        spy_hip_tensor t_nw = T2(SPY_HIP_F32, (void *)c.out_norm, d, 1); t_nw.dim = 1;
+        spy_hip_tensor t_x1 = T2(SPY_HIP_F32, x + (size_t)(T - 1) * d, d, 1), t_xn1 = T2(SPY_HIP_F32, xn, d, 1), t_l1 = T2(SPY_HIP_F32, lg, V, 1);
+        RC_TRY(spy_hip_op_norm_rms(st, &t_x1, &t_xn1, c.eps));
+        RC_TRY(spy_hip_op_binary(st, 2, &t_xn1, &t_nw, &t_xn1));
+        RC_TRY(mm(c.w_out, c.t_out, d, V, &t_xn1, &t_l1));
+        if (logits_host) HIP_TRY(hipMemcpyAsync(logits_host, lg, (size_t)V * 4, hipMemcpyDeviceToHost, st));
     }
-    if (logits_host) HIP_TRY(hipMemcpyAsync(logits_host, lg, (size_t)V * T * 4, hipMemcpyDeviceToHost, st));
+    if (head == HEAD_ALL && logits_host) HIP_TRY(hipMemcpyAsync(logits_host, lg, (size_t)V * T * 4, hipMemcpyDeviceToHost, st));
     HIP_TRY(hipStreamSynchronize(st));
     return 0;
 }
 
-extern "C" int spy_hip_llama_forward(spy_hip_llama *m, void *stream, const int32_t *tokens_host, int32_t n_token, int32_t n_past,
-                                     float *logits_host) {
+static int forward_any(spy_hip_llama *m, void *stream, const int32_t *tokens_host, int32_t n_token, int32_t n_past, float *logits_host, bool last_only) {
     SPY_CHECK_ARG(m && tokens_host && n_token > 0 && n_past >= 0);
     SPY_CHECK_ARG((int64_t)n_past + n_token <= m->desc.n_ctx);                  // llama.cpp:249
     hipStream_t st = stream ? (hipStream_t)stream : m->own_stream;
@@ -452,9 +459,22 @@ extern "C" int spy_hip_llama_forward(spy_hip_llama *m, void *stream, const int32
     const int CH = ch_req >= 16 ? ch_req : SPY_PREFILL_CHUNK;
     for (int t0 = 0; t0 < n_token; t0 += CH) {
         const int tc = n_token - t0 < CH ? n_token - t0 : CH;
-        RC_TRY(forward_ops(m, st, tokens_host + t0, tc, n_past + t0, logits_host ? logits_host + (size_t)t0 * m->desc.n_vocab : nullptr));
+        // logits nobody asked for are not computed: no buffer -> no head; last_only -> the head runs on the last row of the last chunk
+        const int head = !logits_host ? HEAD_NONE : !last_only ? HEAD_ALL : (t0 + tc == n_token ? HEAD_LAST : HEAD_NONE);
+        float *dst = !logits_host ? nullptr : last_only ? logits_host : logits_host + (size_t)t0 * m->desc.n_vocab;
+        RC_TRY(forward_ops(m, st, tokens_host + t0, tc, n_past + t0, dst, head));
     }
     return 0;
+}
+
+extern "C" int spy_hip_llama_forward(spy_hip_llama *m, void *stream, const int32_t *tokens_host, int32_t n_token, int32_t n_past,
+                                     float *logits_host) {
+    return forward_any(m, stream, tokens_host, n_token, n_past, logits_host, false);
+}
+
+extern "C" int spy_hip_llama_forward_last(spy_hip_llama *m, void *stream, const int32_t *tokens_host, int32_t n_token, int32_t n_past,
+                                          float *logits_last_host) {
+    return forward_any(m, stream, tokens_host, n_token, n_past, logits_last_host, true);
 }
 
 extern "C" int spy_hip_llama_decode_greedy(spy_hip_llama *m, void *stream, int32_t first_token, int32_t n_past, int32_t n_steps,

@@ -174,6 +174,14 @@ class Engine:
                                              logits.ctypes.data if want_logits else None), "spy_hip_llama_forward")
         return logits
 
+    def forward_last(self, tokens, n_past):
+        """The pass of forward() with the output head on the last token only: n_vocab logits."""
+        tokens = np.ascontiguousarray(tokens, dtype=np.int32)
+        logits = np.empty(self.cfg.n_vocab, dtype=np.float32)
+        H.check(self.L.spy_hip_llama_forward_last(self.handle, None, tokens.ctypes.data, len(tokens), n_past, logits.ctypes.data),
+                "spy_hip_llama_forward_last")
+        return logits
+
     def decode_greedy(self, first_token, n_past, n_steps, use_graph=True):
         out = np.empty(n_steps, dtype=np.int32)
         H.check(self.L.spy_hip_llama_decode_greedy(self.handle, None, int(first_token), int(n_past), int(n_steps),
@@ -219,8 +227,8 @@ class Engine:
         """Prefill + greedy loop of AutoModelGenerator::generate (cli.h:60-129): returns the
         n_predict sampled tokens."""
         prompt = np.asarray(prompt_tokens, dtype=np.int32)
-        logits = self.forward(prompt, 0)
-        first = int(np.argmax(logits[-1]))          # np.argmax returns the first maximum, like greedy.h:20-25
+        logits = self.forward_last(prompt, 0)
+        first = int(np.argmax(logits))              # np.argmax returns the first maximum, like greedy.h:20-25
         if n_predict == 1:
             return np.array([first], dtype=np.int32)
         rest = self.decode_greedy(first, len(prompt), n_predict - 1)

@@ -67,6 +67,37 @@ def _comfortable_prompt(ora, cfg, n_prompt, n_predict, min_margin, tries=40):
     return best
 
 
+@pytest.mark.parametrize("n_prompt,chunk", [(6, None), (40, None), (72, "32")])
+def test_forward_last_is_the_last_row_of_forward(n_prompt, chunk, monkeypatch):
+    """spy_hip_llama_forward_last = the pass of spy_hip_llama_forward with the head on the last token only: same
+    KV caches, and the logits of the last row (same kernels for a prompt below 16 tokens, the one-row head kernel
+    against the matrix-core one above: 1e-3), also when the prompt goes through in chunks."""
+    from spy_amd import model as M
+    if chunk:
+        monkeypatch.setenv("SPY_HIP_PREFILL_CHUNK", chunk)
+    cfg = M.Config(n_layer=2, n_embd=256, n_head=2, n_ff=768, n_vocab=512, n_ctx=96, wtype=O.Q4_0)
+    tensors = M.synth_model(cfg, seed=5)
+    a, b = M.Engine(cfg, tensors), M.Engine(cfg, tensors)
+    prompt = np.random.default_rng(9).integers(0, cfg.n_vocab, n_prompt).astype(np.int32)
+    full = a.forward(prompt, 0)
+    last = b.forward_last(prompt, 0)
+    assert last.shape == (cfg.n_vocab,)
+    if n_prompt < 16:
+        assert np.array_equal(last, full[-1])
+    else:
+        _close(last, full[-1], "last-row logits")
+        assert int(np.argmax(last)) == int(np.argmax(full[-1]))
+    for il in range(cfg.n_layer):
+        for name in ("k_cache", "v_cache"):
+            assert np.array_equal(a.read_buffer(name, il), b.read_buffer(name, il)), (name, il)
+    # a pass without any logits leaves the same caches too
+    c = M.Engine(cfg, tensors)
+    assert c.forward(prompt, 0, want_logits=False) is None
+    assert np.array_equal(c.read_buffer("k_cache", 1), a.read_buffer("k_cache", 1))
+    for e in (a, b, c):
+        e.close()
+
+
 def test_greedy_tokens_identical_small():
     """Single-token passes one by one against the oracle, then the free-running greedy loop.
     The reference's softmax rounds its exp argument to fp16 (non-linear.cpp:170 in the Spy tree), so a
