@@ -130,6 +130,14 @@ int spy_hip_gemv_q8_0act(void *stream, int wtype, const void *w, const void *xq,
  * operands as for spy_hip_gemv_q8_0act. */
 int spy_hip_gemm_q8_0act(void *stream, int wtype, const void *w, const void *xq, float *dst,
                          int64_t M, int64_t K, int64_t T, int64_t dst_stride);
+/* Causal attention of a pass over T tokens at positions past .. past+T-1, all heads, in one kernel: the
+ * operator sequence MatMul(K cache view, q) -> Softmax(causal mask, scale) -> MatMul(V^T cache view, P) of
+ * the LLaMA graph (attention.cpp:25-302; mat.cpp:32-146; non-linear.cpp:129-180) without the score and
+ * probability matrices in memory.  q16: rotated queries as fp16 [H][T][hd]; k_cache: fp16 [n_ctx][H*hd];
+ * v_cache: fp16 [H*hd][n_ctx], both already holding the pass's own rows; out: f32 [T][H*hd].
+ * hd must be 128 and n_ctx a multiple of 8 (else SPY_HIP_EUNSUPPORTED). */
+int spy_hip_prompt_attention(void *stream, const void *q16, const void *k_cache, const void *v_cache, float *out,
+                             int32_t T, int32_t H, int32_t hd, int32_t past, int64_t n_ctx, float scale);
 /* the int32 dot of every 32-element block (Q4_0, Q8_0, Q4_K sub-blocks) or 16-element
  * sub-block (Q6_K) of every weight row with activation row 0: out[m*nsub + b], written by the
  * GEMV kernels themselves (same code path, dump switch on).  `out` must hold M*nsub + M int32:

@@ -92,6 +92,7 @@ SIGNATURES = {
     "spy_hip_quantize_f16": (_i32, [_vp, _vp, _i64, _vp, _i64, _i64]),
     "spy_hip_gemv_q8_0act": (_i32, [_vp, _i32, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64]),
     "spy_hip_gemm_q8_0act": (_i32, [_vp, _i32, _vp, _vp, _vp, _i64, _i64, _i64, _i64]),
+    "spy_hip_prompt_attention": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i64, C.c_float]),
     "spy_hip_block_dots": (_i32, [_vp, _i32, _vp, _vp, _vp, _i64, _i64]),
     "spy_hip_measure_mfma_i8": (_i32, [_vp, _i32, C.POINTER(_f32)]),
     "spy_hip_measure_hbm_read": (_i32, [_vp, _vp, _sz, _i32, C.POINTER(_f32)]),

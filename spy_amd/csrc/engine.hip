@@ -271,6 +271,8 @@ int spy_silu_mul_q8_launch(hipStream_t st, const float *gate, const float *up, v
 int spy_rope_table_launch(hipStream_t st, float *table, int past, int T, int hd, float freq_base, float freq_scale, float mscale);       // prompt_fused.hip
 int spy_rope_store_launch(hipStream_t st, const float *q, const float *k, const float *table, uint16_t *q16, uint16_t *kc, int T, int H, int hd);
 int spy_vt_store_launch(hipStream_t st, const float *v, uint16_t *vc, int T, int d, int64_t n_ctx);
+int spy_prompt_attn_launch(hipStream_t st, const uint16_t *q16, const uint16_t *k_cache, const uint16_t *v_cache, float *out,
+                           int T, int H, int hd, int past, int64_t n_ctx, float scale);                                       // prompt_attn.hip
 int spy_softmax_causal_launch(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *dst, float scale, int n_past);   // ops.hip
 int spy_softmax_row_ok(int64_t ne0);                                                                                         // ops.hip
 
@@ -338,6 +340,9 @@ static int forward_ops(spy_hip_llama *m, hipStream_t st, const int32_t *tokens_h
     // Passes over many tokens (every MatMul on the matrix cores): the elementwise operators between two MatMuls write the
     // next MatMul's Q8_0 activations directly (same bytes as the separate operators: prompt_fused.hip)
     const bool fuse_act = T >= 16 && d % 64 == 0 && F % 64 == 0 && !getenv("SPY_HIP_PROMPT_UNFUSED");
+    // SPY_HIP_PROMPT_ATTN=0: the attention of a prompt pass as MatMul -> Softmax -> MatMul (bit-identical to the operator path)
+    const char *pa_env = getenv("SPY_HIP_PROMPT_ATTN");
+    const bool fuse_attn = fuse_act && !(pa_env && pa_env[0] == '0');
     float *rope_tab = (float *)(B + o_rt);
     if (fuse_act) RC_TRY(spy_rope_table_launch(st, rope_tab, P, T, (int)hd, rp.freq_base, rp.freq_scale, rp.attention_factor));
     for (int il = 0; il < c.n_layer; il++) {
@@ -372,6 +377,13 @@ static int forward_ops(spy_hip_llama *m, hipStream_t st, const int32_t *tokens_h
             t_vc.nb[0] = 2; t_vc.nb[1] = 2 * C; t_vc.nb[2] = t_vc.nb[3] = d * 2 * C;
             RC_TRY(spy_hip_op_dup(st, &t_vt, &t_vc));
         }
+        bool attn_done = false;
+        if (fuse_attn) {          // scores, masked softmax and the product with V^T in one kernel: no score / probability matrix in memory
+            const int rc = spy_prompt_attn_launch(st, (const uint16_t *)xn, (const uint16_t *)m->k_cache[il], (const uint16_t *)m->v_cache[il], o2,
+                                                  T, (int)H, (int)hd, P, C, scale);
+            if (rc != SPY_HIP_EUNSUPPORTED) { RC_TRY(rc); attn_done = true; }
+        }
+        if (!attn_done) {
         spy_hip_tensor t_kall = T3s(SPY_HIP_F16, m->k_cache[il], hd, n_kv, H, 2, 2 * d, 2 * hd);
         spy_hip_tensor t_vall = T3s(SPY_HIP_F16, m->v_cache[il], n_kv, hd, H, 2, 2 * C, 2 * C * hd);
         // causal_ok: the softmax below takes the row kernel, which reads no score beyond a row's causal length and writes
@@ -393,6 +405,7 @@ static int forward_ops(spy_hip_llama *m, hipStream_t st, const int32_t *tokens_h
             spy_hip_tensor t_Op = T3s(SPY_HIP_F32, o, hd, H, T, 4, 4 * hd * T, 4 * hd);                // Permute {0,2,1,3}
             spy_hip_tensor t_o2c = T3s(SPY_HIP_F32, o2, hd, H, T, 4, 4 * hd, 4 * d);
             RC_TRY(spy_hip_op_contiguous(st, &t_Op, &t_o2c));
+        }
         }
         RC_TRY(mm(L.wo, L.t_wo, d, d, &t_o2, &t_t1));
         RC_TRY(spy_hip_op_binary(st, 0, &t_t1, &t_x, &t_t1));

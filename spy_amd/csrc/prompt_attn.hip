@@ -1,0 +1,172 @@
+// Causal attention of a prompt pass in one kernel: scores, masked softmax and the product with V^T
+// for a tile of 64 queries of one head, without writing the score or probability matrices to memory.
+//
+// Replaces, for passes over many tokens, the operator sequence MatMul(K, q) -> Softmax(mask, scale) ->
+// MatMul(V^T, P) of the LLaMA graph (attention.cpp:25-302; mat.cpp:32-146 with Dot<FP16,FP16>,
+// vec_dot.h:117-146; non-linear.cpp:129-180 in the Spy tree).  The arithmetic per element is that of
+// those operators: fp16 x fp16 products accumulated in fp32 over the head dimension in ascending order;
+// t = s * scale; m = max t over the row; e = expf(float(fp16(t - m))); p = e * (1 / sum e), rounded to
+// fp16 as the second MatMul rounds its right operand (mat.cpp:37); fp32 accumulation over the cached
+// positions in ascending order.  The softmax needs the row maximum before any exponential and the row
+// sum before any probability, so the scores of a tile are computed three times (cheap on the matrix
+// cores) instead of being kept: pass 1 maximum, pass 2 sum, pass 3 probabilities and the product.
+// Only the order in which a row's exponentials are added differs from softmax_row_kernel (last-bit
+// differences of the sum).
+//
+// 256 threads = 2 x 2 waves; a score tile is 64 cached positions x 64 queries, one 32 x 32 MFMA tile per
+// wave (positions along the accumulator registers, queries along the lanes, so a lane owns one query);
+// the output tile is 128 head dimensions x 64 queries, two 32 x 32 tiles per wave.
+#include "common.cuh"
+
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+#define PA_KROW 272     // LDS bytes per K row: 128 halfs + 16 pad
+#define PA_VROW 144     // LDS bytes per V^T / P row: 64 halfs + 16 pad
+
+struct pattn_args {
+    const uint16_t *q16;   // [H][T][128] fp16 (rotated queries)
+    const uint16_t *kc;    // K cache, fp16 [n_ctx][H * 128]
+    const uint16_t *vc;    // V^T cache, fp16 [H * 128][n_ctx]
+    float *out;            // f32 [T][H * 128]
+    int T, H, past, n_ctx;
+    float scale;
+};
+
+__global__ __launch_bounds__(256, 2) void prompt_attn_kernel(pattn_args a) {
+    __shared__ __attribute__((aligned(16))) uint8_t sK[2][64 * PA_KROW];
+    __shared__ __attribute__((aligned(16))) uint8_t sV[128 * PA_VROW];
+    __shared__ __attribute__((aligned(16))) uint8_t sP[64 * PA_VROW];
+    __shared__ float s_stat[2][64];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
+    const int q0 = blockIdx.x * 64, h = blockIdx.y, T = a.T, H = a.H;
+    const size_t d = (size_t)H * 128;
+    const int n_kv = a.past + T;
+    const int ql = wn * 32 + (lane & 31), t = q0 + ql, tq = min(t, T - 1);
+    const int limit = a.past + tq;                                  // last cached position this lane's query sees
+    const int kv_end = a.past + min(q0 + 63, T - 1) + 1;            // positions any query of the tile sees (<= n_kv)
+    const int ntile = (kv_end + 63) / 64;
+    const float scale = a.scale;
+
+    v8h fq[8];                                                      // this lane's query: B operand of the score MFMAs
+#pragma unroll
+    for (int ks = 0; ks < 8; ks++) fq[ks] = *(const v8h *)(a.q16 + ((size_t)h * T + tq) * 128 + ks * 16 + (lane >> 5) * 8);
+
+    // scores of tile j: K rows j*64 .. +63 -> LDS (rows past the cache end re-read its last row: masked below)
+    auto load_k = [&](int j, int b) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int c = tid + i * 256, row = c >> 4, piece = c & 15;
+            const uint4 v = *(const uint4 *)(a.kc + (size_t)min(j * 64 + row, n_kv - 1) * d + (size_t)h * 128 + piece * 8);
+            *(uint4 *)(sK[b] + row * PA_KROW + piece * 16) = v;
+        }
+    };
+    auto scores = [&](int b) {
+        v16f acc = {0};
+#pragma unroll
+        for (int ks = 0; ks < 8; ks++) {
+            const v8h fa = *(const v8h *)(sK[b] + (wm * 32 + (lane & 31)) * PA_KROW + ks * 32 + (lane >> 5) * 16);
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa, fq[ks], acc, 0, 0, 0);
+        }
+        return acc;
+    };
+    // accumulator register r of tile j holds position j*64 + wm*32 + (r/4)*8 + (lane>>5)*4 + (r&3)
+    const int pos0 = wm * 32 + (lane >> 5) * 4;
+
+    // pass 1: row maximum of t = s * scale
+    float m = -INFINITY;
+    for (int j = 0; j < ntile; j++) {
+        load_k(j, j & 1);
+        __syncthreads();
+        const v16f s = scores(j & 1);
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int pos = j * 64 + pos0 + (r >> 2) * 8 + (r & 3);
+            if (pos <= limit) m = fmaxf(m, s[r] * scale);
+        }
+    }
+    m = fmaxf(m, __shfl_xor(m, 32, SPY_WAVE));
+    if (lane < 32) s_stat[wm][ql] = m;
+    __syncthreads();
+    m = fmaxf(s_stat[0][ql], s_stat[1][ql]);
+    __syncthreads();
+
+    // pass 2: row sum of e = expf(fp16(t - m))
+    float sum = 0.0f;
+    for (int j = 0; j < ntile; j++) {
+        load_k(j, j & 1);
+        __syncthreads();
+        const v16f s = scores(j & 1);
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int pos = j * 64 + pos0 + (r >> 2) * 8 + (r & 3);
+            if (pos <= limit) sum += expf(h2f(f2h(s[r] * scale - m)));
+        }
+    }
+    sum += __shfl_xor(sum, 32, SPY_WAVE);
+    if (lane < 32) s_stat[wm][ql] = sum;
+    __syncthreads();
+    const float inv = 1.0f / (s_stat[0][ql] + s_stat[1][ql]);
+
+    // pass 3: probabilities (fp16) through LDS, times V^T
+    v16f oacc[2] = {{0}, {0}};
+    for (int j = 0; j < ntile; j++) {
+        load_k(j, j & 1);
+        __syncthreads();                                            // K tile stored; every wave is done with the previous tile's sP / sV
+        const v16f s = scores(j & 1);
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            uint16_t p[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int pos = j * 64 + pos0 + g * 8 + e;
+                p[e] = pos <= limit ? f2h(expf(h2f(f2h(s[4 * g + e] * scale - m))) * inv) : (uint16_t)0;
+            }
+            *(uint2 *)(sP + ql * PA_VROW + (pos0 + g * 8) * 2) = make_uint2((uint32_t)p[0] | ((uint32_t)p[1] << 16), (uint32_t)p[2] | ((uint32_t)p[3] << 16));
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) {                               // V^T tile: 128 rows x 64 positions
+            const int c = tid + i * 256, row = c >> 3, piece = c & 7;
+            const int col = min(j * 64 + piece * 8, a.n_ctx - 8);   // groups of 8 past the cache end carry zero probabilities
+            const uint4 v = *(const uint4 *)(a.vc + ((size_t)h * 128 + row) * a.n_ctx + col);
+            *(uint4 *)(sV + row * PA_VROW + piece * 16) = v;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int ks = 0; ks < 4; ks++) {
+                const v8h fa = *(const v8h *)(sV + (wm * 64 + i * 32 + (lane & 31)) * PA_VROW + ks * 32 + (lane >> 5) * 16);
+                const v8h fb = *(const v8h *)(sP + ql * PA_VROW + ks * 32 + (lane >> 5) * 16);
+                oacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa, fb, oacc[i], 0, 0, 0);
+            }
+    }
+    if (t < T) {
+        float *o = a.out + ((size_t)t * H + h) * 128;
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int dd = wm * 64 + i * 32 + g * 8 + (lane >> 5) * 4;
+                *(float4 *)(o + dd) = make_float4(oacc[i][4 * g], oacc[i][4 * g + 1], oacc[i][4 * g + 2], oacc[i][4 * g + 3]);
+            }
+    }
+}
+
+// q16: rotated queries as fp16 [H][T][128]; k_cache / v_cache: the layer's caches with the pass's rows already stored;
+// out: f32 [T][H * 128] (the layout of the attention output after Permute + Contiguous)
+int spy_prompt_attn_launch(hipStream_t st, const uint16_t *q16, const uint16_t *k_cache, const uint16_t *v_cache, float *out,
+                           int T, int H, int hd, int past, int64_t n_ctx, float scale) {
+    SPY_CHECK_ARG(q16 && k_cache && v_cache && out && T > 0 && H > 0 && H < 65536 && past >= 0);
+    if (hd != 128 || n_ctx % 8 != 0 || n_ctx < 64 || n_ctx >= (1ll << 31)) return SPY_HIP_EUNSUPPORTED;
+    SPY_CHECK_ARG((int64_t)past + T <= n_ctx && ((uintptr_t)q16 % 16) == 0 && ((uintptr_t)k_cache % 16) == 0 && ((uintptr_t)v_cache % 16) == 0 && ((uintptr_t)out % 16) == 0);
+    pattn_args a;
+    a.q16 = q16; a.kc = k_cache; a.vc = v_cache; a.out = out; a.T = T; a.H = H; a.past = past; a.n_ctx = (int)n_ctx; a.scale = scale;
+    prompt_attn_kernel<<<dim3((unsigned)((T + 63) / 64), (unsigned)H), dim3(256), 0, st>>>(a);
+    return SPY_LAUNCH_RC();
+}
+
+extern "C" int spy_hip_prompt_attention(void *stream, const void *q16, const void *k_cache, const void *v_cache, float *out,
+                                        int32_t T, int32_t H, int32_t hd, int32_t past, int64_t n_ctx, float scale) {
+    return spy_prompt_attn_launch((hipStream_t)stream, (const uint16_t *)q16, (const uint16_t *)k_cache, (const uint16_t *)v_cache, out, T, H, hd, past, n_ctx, scale);
+}

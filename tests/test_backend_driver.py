@@ -68,11 +68,41 @@ def test_submit_path_matches_oracle_and_engine(wtype):
 
 
 @pytest.mark.gpu
-def test_engine_prompt_softmax_without_mask_tensor_matches_submit_path():
+@pytest.mark.parametrize("passes", [((0, 168), (168, 304), (304, 438)), ((0, 64),), ((0, 17), (17, 100), (100, 163)), ((0, 130), (130, 131), (131, 200))])
+def test_engine_fused_prompt_attention_against_submit_path(passes):
+    """Default prompt pass of the engine: scores, masked softmax and P.V^T of a layer in one kernel (no score matrix in
+    memory).  Same arithmetic per element as the three operators of the submit path except for the order in which a
+    row's exponentials are added: a probability now and then lands on the other side of an fp16 rounding boundary
+    (tests/test_gpu_ops.py bounds that at the kernel), and the Q8_0 re-quantization of the following MatMuls turns such
+    a difference into their rounding noise, as for any two implementations whose sums are not bit-identical.  Hence a
+    bound at that noise level (5e-3 of the largest logit) and the same argmax on nearly every row.  Tile edges: passes
+    that are not multiples of 64 tokens, caches that are not multiples of 64 positions, a single-token pass (the fused
+    single-token kernels) in between."""
+    from spy_amd import backend_driver as B
+    from spy_amd import model as M
+    from tests.gpu_util import rel_err
+    cfg = M.Config(n_layer=2, n_embd=256, n_head=2, n_ff=768, n_vocab=512, n_ctx=448, wtype=O.Q4_0)
+    tensors = M.synth_model(cfg, seed=11)
+    host, eng = B.HostModel(cfg, tensors), M.Engine(cfg, tensors)
+    prompt = np.random.default_rng(5).integers(0, cfg.n_vocab, passes[-1][1]).astype(np.int32)
+    for start, stop in passes:
+        print("pass", start, stop, flush=True)
+        lg_h, lg_e = host.forward(prompt[start:stop], start), eng.forward(prompt[start:stop], start)
+        assert np.isfinite(lg_e).all()
+        err = rel_err(lg_e, lg_h)
+        print("  max-abs err / max |logit| = %.2e" % err, flush=True)
+        assert err < 5e-3, (start, stop, err)
+        assert (np.argmax(lg_e, axis=1) == np.argmax(lg_h, axis=1)).mean() > 0.98
+    host.close()
+
+
+@pytest.mark.gpu
+def test_engine_prompt_softmax_without_mask_tensor_matches_submit_path(monkeypatch):
     """The engine's prompt pass tells its softmax and its two attention products the causal shape as a number (no
     mask tensor read, tiles above the diagonal left out) and hands the probabilities over as fp16; the submit path
     runs MatMul / Softmax / MatMul with the graph's mask tensor (llama.cpp:248-263).  Same bits, also for passes on
     top of a filled cache."""
+    monkeypatch.setenv("SPY_HIP_PROMPT_ATTN", "0")          # attention as MatMul -> Softmax -> MatMul, not the single kernel
     from spy_amd import backend_driver as B
     from spy_amd import model as M
     cfg = M.Config(n_layer=2, n_embd=256, n_head=2, n_ff=768, n_vocab=512, n_ctx=448, wtype=O.Q4_0)

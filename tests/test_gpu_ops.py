@@ -262,3 +262,52 @@ def test_op_matmul_attention_views(hip, oracle):
     assert_close(dO.download(np.float32).reshape(O_want.shape), O_want, "KQV", tol=1e-5)
     # F32 x F32 has no hip implementation: reported, not aborted
     assert L.spy_hip_op_matmul(None, B(tq), B(tq), B(tS), None, 0) == hip.EUNSUPPORTED
+
+
+@pytest.mark.parametrize("H_,T,past,n_ctx", [(2, 40, 0, 64), (3, 136, 168, 448), (2, 200, 57, 320), (1, 64, 4032, 4096), (2, 1, 77, 128), (1, 130, 0, 136)])
+def test_prompt_attention_kernel_against_operator_sequence(hip, H_, T, past, n_ctx):
+    """spy_hip_prompt_attention = MatMul(K view, q) -> Softmax(causal mask, scale) -> MatMul(V^T view, P) of the
+    operator ABI on the same fp16 inputs.  The products accumulate in the same order and the maximum is exact, so the
+    only difference is the order in which a row's exponentials are added: the results agree to a few fp32 ulps except
+    where that moves a probability across an fp16 rounding boundary (2^-11 of that probability)."""
+    from tests.gpu_util import dev, dev_empty, call, rel_err
+    hd, n_kv = 128, past + T
+    d = H_ * hd
+    rng = np.random.default_rng(1000 * T + past)
+    scale = 1.0 / np.sqrt(hd)
+    q = rng.standard_normal((H_, T, hd)).astype(np.float16)
+    kc = np.zeros((n_ctx, d), np.float16); kc[:n_kv] = rng.standard_normal((n_kv, d)).astype(np.float16)
+    vc = np.zeros((d, n_ctx), np.float16); vc[:, :n_kv] = rng.standard_normal((d, n_kv)).astype(np.float16)
+    dq, dk, dv = dev(q), dev(kc), dev(vc)
+    L = hip.load()
+    fused = dev_empty(T * d * 4, 0xFF)
+    call(L.spy_hip_prompt_attention, None, dq.ptr, dk.ptr, dv.ptr, fused.ptr, T, H_, hd, past, n_ctx, scale)
+    # the operator sequence, tensors as the LLaMA graph views them
+    mask = np.where(np.arange(n_ctx)[None, :] <= (np.arange(T)[:, None] + past), 0.0, -np.inf).astype(np.float32)
+    dm = dev(mask.view(np.int32))
+    tk = hip.tensor(dk, hip.F16, [hd, n_kv, H_], nb=[2, 2 * d, 2 * hd])
+    tq = hip.tensor(dq, hip.F16, [hd, T, H_])
+    dS, dP, ref = dev_empty(n_kv * T * H_ * 4, 0xFF), dev_empty(n_kv * T * H_ * 4, 0xFF), dev_empty(T * d * 4, 0xFF)
+    tS, tP = hip.tensor(dS, hip.F32, [n_kv, T, H_]), hip.tensor(dP, hip.F32, [n_kv, T, H_])
+    tv = hip.tensor(dv, hip.F16, [n_kv, hd, H_], nb=[2, 2 * n_ctx, 2 * n_ctx * hd])
+    tO = hip.tensor(ref, hip.F32, [hd, T, H_], nb=[4, 4 * d, 4 * hd])
+    need = max(L.spy_hip_op_matmul_scratch_size(B(tk), B(tq)), L.spy_hip_op_matmul_scratch_size(B(tv), B(tP)), 256)
+    sc = dev_empty(need)
+    call(L.spy_hip_op_matmul, None, B(tk), B(tq), B(tS), sc.ptr, need)
+    call(L.spy_hip_op_softmax, None, B(tS), B(hip.tensor(dm, hip.I32, [n_ctx, T])), B(tP), scale)
+    call(L.spy_hip_op_matmul, None, B(tv), B(tP), B(tO), sc.ptr, need)
+    hip.sync()
+    got, want = fused.download(np.float32).reshape(T, d), ref.download(np.float32).reshape(T, d)
+    assert np.isfinite(got).all()
+    err = rel_err(got, want)
+    frac_equal = float((got.view(np.uint32) == want.view(np.uint32)).mean())
+    print("H %d T %d past %d: max-abs err / max |out| = %.2e, %.1f %% of the outputs bit-identical" % (H_, T, past, err, 100 * frac_equal), flush=True)
+    assert err < 2e-4
+    # and against the definition in float64 on the same fp16 inputs
+    for h in range(H_):
+        qf, kf, vf = q[h].astype(np.float64), kc[:n_kv, h * hd:(h + 1) * hd].astype(np.float64), vc[h * hd:(h + 1) * hd, :n_kv].astype(np.float64)
+        t = (qf @ kf.T) * scale
+        t[np.arange(n_kv)[None, :] > (np.arange(T)[:, None] + past)] = -np.inf
+        e = np.exp((t - t.max(axis=1, keepdims=True)).astype(np.float16).astype(np.float64))
+        p = (e / e.sum(axis=1, keepdims=True)).astype(np.float16).astype(np.float64)
+        assert rel_err(got[:, h * hd:(h + 1) * hd], p @ vf.T) < 1e-3
