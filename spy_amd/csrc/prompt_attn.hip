@@ -39,7 +39,13 @@ __global__ __launch_bounds__(256, 2) void prompt_attn_kernel(pattn_args a) {
     __shared__ __attribute__((aligned(16))) uint8_t sP[64 * PA_VROW];
     __shared__ float s_stat[2][64];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
-    const int q0 = blockIdx.x * 64, h = blockIdx.y, T = a.T, H = a.H;
+    const int T = a.T, H = a.H, NQ = (T + 63) / 64;
+    // Workgroup b runs on XCD b % 8, each with its own L2: all query tiles of a head go to one XCD, so that the head's K and
+    // V^T rows (read by every tile, three times) stay in that L2.  Head counts that are not a multiple of 8 use the plain order.
+    int h, qt;
+    if (H % 8 == 0) { const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3; h = (slot / NQ) * 8 + xcd; qt = slot % NQ; }
+    else { h = blockIdx.x / NQ; qt = blockIdx.x % NQ; }
+    const int q0 = (NQ - 1 - qt) * 64;                              // late queries (most cached positions) first
     const size_t d = (size_t)H * 128;
     const int n_kv = a.past + T;
     const int ql = wn * 32 + (lane & 31), t = q0 + ql, tq = min(t, T - 1);
@@ -52,14 +58,27 @@ __global__ __launch_bounds__(256, 2) void prompt_attn_kernel(pattn_args a) {
 #pragma unroll
     for (int ks = 0; ks < 8; ks++) fq[ks] = *(const v8h *)(a.q16 + ((size_t)h * T + tq) * 128 + ks * 16 + (lane >> 5) * 8);
 
-    // scores of tile j: K rows j*64 .. +63 -> LDS (rows past the cache end re-read its last row: masked below)
-    auto load_k = [&](int j, int b) {
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int c = tid + i * 256, row = c >> 4, piece = c & 15;
-            const uint4 v = *(const uint4 *)(a.kc + (size_t)min(j * 64 + row, n_kv - 1) * d + (size_t)h * 128 + piece * 8);
-            *(uint4 *)(sK[b] + row * PA_KROW + piece * 16) = v;
-        }
+    // K rows j*64 .. +63 of the head -> registers -> LDS (rows past the cache end re-read its last row: masked below).
+    // The loads of tile j + 1 are issued before tile j is multiplied, so that their latency is covered.
+    struct quad { uint4 a, b, c, d; };
+    quad rk, rv;
+    const uint16_t *kbase = a.kc + (size_t)h * 128 + (tid & 15) * 8;         // thread's 16-byte piece of rows (tid >> 4) + 16 i
+    const uint16_t *vbase = a.vc + ((size_t)h * 128 + (tid >> 3)) * a.n_ctx;   // thread's piece (tid & 7) of rows (tid >> 3) + 32 i
+    auto krow = [&](int j, int i) { return (const uint4 *)(kbase + (size_t)min(j * 64 + (tid >> 4) + 16 * i, n_kv - 1) * d); };
+    auto gload_k = [&](int j) -> quad { return quad{*krow(j, 0), *krow(j, 1), *krow(j, 2), *krow(j, 3)}; };
+    auto store_k = [&](int b, const quad &r) {
+        uint8_t *p = sK[b] + (tid >> 4) * PA_KROW + (tid & 15) * 16;
+        *(uint4 *)p = r.a; *(uint4 *)(p + 16 * PA_KROW) = r.b; *(uint4 *)(p + 32 * PA_KROW) = r.c; *(uint4 *)(p + 48 * PA_KROW) = r.d;
+    };
+    auto gload_v = [&](int j) -> quad {                             // V^T tile: 128 rows x 64 positions
+        const int col = min(j * 64 + (tid & 7) * 8, a.n_ctx - 8);   // groups of 8 past the cache end carry zero probabilities
+        const uint16_t *p = vbase + col;
+        const size_t rs = (size_t)32 * a.n_ctx;
+        return quad{*(const uint4 *)p, *(const uint4 *)(p + rs), *(const uint4 *)(p + 2 * rs), *(const uint4 *)(p + 3 * rs)};
+    };
+    auto store_v = [&](const quad &r) {
+        uint8_t *p = sV + (tid >> 3) * PA_VROW + (tid & 7) * 16;
+        *(uint4 *)p = r.a; *(uint4 *)(p + 32 * PA_VROW) = r.b; *(uint4 *)(p + 64 * PA_VROW) = r.c; *(uint4 *)(p + 96 * PA_VROW) = r.d;
     };
     auto scores = [&](int b) {
         v16f acc = {0};
@@ -75,15 +94,15 @@ __global__ __launch_bounds__(256, 2) void prompt_attn_kernel(pattn_args a) {
 
     // pass 1: row maximum of t = s * scale
     float m = -INFINITY;
+    rk = gload_k(0);
     for (int j = 0; j < ntile; j++) {
-        load_k(j, j & 1);
+        store_k(j & 1, rk);
+        rk = gload_k(min(j + 1, ntile - 1));                        // unconditional: the last tile re-reads itself
         __syncthreads();
         const v16f s = scores(j & 1);
+        const int room = limit - (j * 64 + pos0);                   // register r is visible to this lane's query iff (r/4)*8 + (r&3) <= room
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const int pos = j * 64 + pos0 + (r >> 2) * 8 + (r & 3);
-            if (pos <= limit) m = fmaxf(m, s[r] * scale);
-        }
+        for (int r = 0; r < 16; r++) m = fmaxf(m, ((r >> 2) * 8 + (r & 3) <= room) ? s[r] * scale : -INFINITY);
     }
     m = fmaxf(m, __shfl_xor(m, 32, SPY_WAVE));
     if (lane < 32) s_stat[wm][ql] = m;
@@ -93,15 +112,20 @@ __global__ __launch_bounds__(256, 2) void prompt_attn_kernel(pattn_args a) {
 
     // pass 2: row sum of e = expf(fp16(t - m))
     float sum = 0.0f;
+    rk = gload_k(0);
     for (int j = 0; j < ntile; j++) {
-        load_k(j, j & 1);
+        store_k(j & 1, rk);
+        rk = gload_k(min(j + 1, ntile - 1));
         __syncthreads();
         const v16f s = scores(j & 1);
+        // every exponential is evaluated (no divergent branches: the 16 evaluations interleave) and the masked ones are
+        // replaced by 0 afterwards; adding those zeros changes nothing
+        const int room = limit - (j * 64 + pos0);
+        float e[16];
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const int pos = j * 64 + pos0 + (r >> 2) * 8 + (r & 3);
-            if (pos <= limit) sum += expf(h2f(f2h(s[r] * scale - m)));
-        }
+        for (int r = 0; r < 16; r++) e[r] = expf(h2f(f2h(s[r] * scale - m)));
+#pragma unroll
+        for (int r = 0; r < 16; r++) sum += ((r >> 2) * 8 + (r & 3) <= room) ? e[r] : 0.0f;
     }
     sum += __shfl_xor(sum, 32, SPY_WAVE);
     if (lane < 32) s_stat[wm][ql] = sum;
@@ -110,27 +134,25 @@ __global__ __launch_bounds__(256, 2) void prompt_attn_kernel(pattn_args a) {
 
     // pass 3: probabilities (fp16) through LDS, times V^T
     v16f oacc[2] = {{0}, {0}};
+    rk = gload_k(0);
     for (int j = 0; j < ntile; j++) {
-        load_k(j, j & 1);
+        store_k(j & 1, rk);
+        rk = gload_k(min(j + 1, ntile - 1));
+        rv = gload_v(j);                                            // needed after the scores of this tile
         __syncthreads();                                            // K tile stored; every wave is done with the previous tile's sP / sV
         const v16f s = scores(j & 1);
+        const int room = limit - (j * 64 + pos0);
+        float e[16];
+#pragma unroll
+        for (int r = 0; r < 16; r++) e[r] = expf(h2f(f2h(s[r] * scale - m)));
 #pragma unroll
         for (int g = 0; g < 4; g++) {
-            uint16_t p[4];
+            uint32_t p[4];
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                const int pos = j * 64 + pos0 + g * 8 + e;
-                p[e] = pos <= limit ? f2h(expf(h2f(f2h(s[4 * g + e] * scale - m))) * inv) : (uint16_t)0;
-            }
-            *(uint2 *)(sP + ql * PA_VROW + (pos0 + g * 8) * 2) = make_uint2((uint32_t)p[0] | ((uint32_t)p[1] << 16), (uint32_t)p[2] | ((uint32_t)p[3] << 16));
+            for (int k = 0; k < 4; k++) p[k] = f2h((g * 8 + k <= room) ? e[4 * g + k] * inv : 0.0f);
+            *(uint2 *)(sP + ql * PA_VROW + (pos0 + g * 8) * 2) = make_uint2(p[0] | (p[1] << 16), p[2] | (p[3] << 16));
         }
-#pragma unroll
-        for (int i = 0; i < 4; i++) {                               // V^T tile: 128 rows x 64 positions
-            const int c = tid + i * 256, row = c >> 3, piece = c & 7;
-            const int col = min(j * 64 + piece * 8, a.n_ctx - 8);   // groups of 8 past the cache end carry zero probabilities
-            const uint4 v = *(const uint4 *)(a.vc + ((size_t)h * 128 + row) * a.n_ctx + col);
-            *(uint4 *)(sV + row * PA_VROW + piece * 16) = v;
-        }
+        store_v(rv);
         __syncthreads();
 #pragma unroll
         for (int i = 0; i < 2; i++)
@@ -157,12 +179,12 @@ __global__ __launch_bounds__(256, 2) void prompt_attn_kernel(pattn_args a) {
 // out: f32 [T][H * 128] (the layout of the attention output after Permute + Contiguous)
 int spy_prompt_attn_launch(hipStream_t st, const uint16_t *q16, const uint16_t *k_cache, const uint16_t *v_cache, float *out,
                            int T, int H, int hd, int past, int64_t n_ctx, float scale) {
-    SPY_CHECK_ARG(q16 && k_cache && v_cache && out && T > 0 && H > 0 && H < 65536 && past >= 0);
+    SPY_CHECK_ARG(q16 && k_cache && v_cache && out && T > 0 && H > 0 && H < 65536 && past >= 0 && (int64_t)((T + 63) / 64) * H < (1ll << 31));
     if (hd != 128 || n_ctx % 8 != 0 || n_ctx < 64 || n_ctx >= (1ll << 31)) return SPY_HIP_EUNSUPPORTED;
     SPY_CHECK_ARG((int64_t)past + T <= n_ctx && ((uintptr_t)q16 % 16) == 0 && ((uintptr_t)k_cache % 16) == 0 && ((uintptr_t)v_cache % 16) == 0 && ((uintptr_t)out % 16) == 0);
     pattn_args a;
     a.q16 = q16; a.kc = k_cache; a.vc = v_cache; a.out = out; a.T = T; a.H = H; a.past = past; a.n_ctx = (int)n_ctx; a.scale = scale;
-    prompt_attn_kernel<<<dim3((unsigned)((T + 63) / 64), (unsigned)H), dim3(256), 0, st>>>(a);
+    prompt_attn_kernel<<<dim3((unsigned)(((T + 63) / 64) * H)), dim3(256), 0, st>>>(a);
     return SPY_LAUNCH_RC();
 }
 
