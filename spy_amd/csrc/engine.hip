@@ -289,15 +289,24 @@ enum { HEAD_ALL = 0, HEAD_NONE = 1, HEAD_LAST = 2 };     // output head of a pas
 static int forward_ops(spy_hip_llama *m, hipStream_t st, const int32_t *tokens_host, int T, int P, float *logits_host, int head) {
     const spy_hip_llama_desc &c = m->desc;
     const int64_t d = c.n_embd, F = c.n_ff, C = c.n_ctx, H = c.n_head, hd = m->hd, V = c.n_vocab, n_kv = (int64_t)P + T;
-    // scratch layout (bytes)
+    // Passes over many tokens (every MatMul on the matrix cores): the elementwise operators between two MatMuls write the
+    // next MatMul's Q8_0 activations directly (same bytes as the separate operators: prompt_fused.hip)
+    const bool fuse_act = T >= 16 && d % 64 == 0 && F % 64 == 0 && !getenv("SPY_HIP_PROMPT_UNFUSED");
+    // ... and the attention of a layer is one kernel (prompt_attn.hip) where its shape conditions hold;
+    // SPY_HIP_PROMPT_ATTN=0: attention as MatMul -> Softmax -> MatMul (bit-identical to the operator path)
+    const char *pa_env = getenv("SPY_HIP_PROMPT_ATTN");
+    const bool fuse_attn = fuse_act && hd == 128 && C % 8 == 0 && C >= 64 && !(pa_env && pa_env[0] == '0');
+    // scratch layout (bytes); the score / probability matrices and the mask exist only without the attention kernel,
+    // the logits of every row only when they were asked for
     size_t off = 0;
     auto take = [&](size_t bytes) { size_t o = off; off += (bytes + 255) & ~(size_t)255; return o; };
+    const size_t sp_bytes = fuse_attn ? 0 : (size_t)n_kv * T * H * 4;
     const size_t o_x = take(d * T * 4), o_xn = take(d * T * 4), o_q = take(d * T * 4), o_k = take(d * T * 4), o_v = take(d * T * 4),
                  o_o = take(d * T * 4), o_o2 = take(d * T * 4), o_t1 = take(d * T * 4), o_up = take(F * T * 4), o_gate = take(F * T * 4),
-                 o_par = take(F * T * 4), o_S = take(n_kv * T * H * 4), o_P = take(n_kv * T * H * 4), o_mask = take(C * T * 4),
-                 o_ids = take(T * 4), o_pos = take(T * 4), o_logits = take(V * T * 4), o_rt = take(T * hd * 4);
+                 o_par = take(F * T * 4), o_S = take(sp_bytes), o_P = take(sp_bytes), o_mask = take(fuse_attn ? 0 : C * T * 4),
+                 o_ids = take(T * 4), o_pos = take(T * 4), o_logits = take(head == HEAD_ALL ? V * T * 4 : V * 4), o_rt = take(T * hd * 4);
     const size_t act_q8 = (size_t)T * ((F > d ? F : d) / 32) * 34;
-    const size_t act_f16 = (size_t)n_kv * T * H * 2 > (size_t)d * T * 2 ? (size_t)n_kv * T * H * 2 : (size_t)d * T * 2;
+    const size_t act_f16 = sp_bytes / 2 > (size_t)d * T * 2 ? sp_bytes / 2 : (size_t)d * T * 2;
     const size_t o_scr = take(act_q8 > act_f16 ? act_q8 : act_f16);
     const size_t scr_bytes = off - o_scr;
     if (off > m->ops_bytes) {
@@ -318,8 +327,10 @@ static int forward_ops(spy_hip_llama *m, hipStream_t st, const int32_t *tokens_h
         for (int i = 0; i < T; i++) hp[i] = P + i;
         HIP_TRY(hipMemcpyAsync(ids, tokens_host, (size_t)T * 4, hipMemcpyHostToDevice, st));
         HIP_TRY(hipMemcpyAsync(pos, hp.data(), (size_t)T * 4, hipMemcpyHostToDevice, st));
-        causal_mask_kernel<<<dim3((unsigned)((C + 255) / 256), (unsigned)T), dim3(256), 0, st>>>(mask, (int)C, P);   // filled on the device: 35 MB per 2048-token chunk
-        HIP_TRY(hipGetLastError());
+        if (!fuse_attn) {
+            causal_mask_kernel<<<dim3((unsigned)((C + 255) / 256), (unsigned)T), dim3(256), 0, st>>>(mask, (int)C, P);   // filled on the device: 35 MB per 2048-token chunk
+            HIP_TRY(hipGetLastError());
+        }
         HIP_TRY(hipStreamSynchronize(st));
     }
     spy_hip_tensor t_ids = T2(SPY_HIP_I32, ids, T, 1), t_pos = t_ids, t_mask = T2(SPY_HIP_I32, mask, C, T);
@@ -337,12 +348,6 @@ static int forward_ops(spy_hip_llama *m, hipStream_t st, const int32_t *tokens_h
         spy_hip_tensor tw = T2(wt, (void *)w, K, M);
         return spy_hip_op_matmul(st, &tw, xin, out, scr, scr_bytes);
     };
-    // Passes over many tokens (every MatMul on the matrix cores): the elementwise operators between two MatMuls write the
-    // next MatMul's Q8_0 activations directly (same bytes as the separate operators: prompt_fused.hip)
-    const bool fuse_act = T >= 16 && d % 64 == 0 && F % 64 == 0 && !getenv("SPY_HIP_PROMPT_UNFUSED");
-    // SPY_HIP_PROMPT_ATTN=0: the attention of a prompt pass as MatMul -> Softmax -> MatMul (bit-identical to the operator path)
-    const char *pa_env = getenv("SPY_HIP_PROMPT_ATTN");
-    const bool fuse_attn = fuse_act && !(pa_env && pa_env[0] == '0');
     float *rope_tab = (float *)(B + o_rt);
     if (fuse_act) RC_TRY(spy_rope_table_launch(st, rope_tab, P, T, (int)hd, rp.freq_base, rp.freq_scale, rp.attention_factor));
     for (int il = 0; il < c.n_layer; il++) {
@@ -377,13 +382,10 @@ static int forward_ops(spy_hip_llama *m, hipStream_t st, const int32_t *tokens_h
             t_vc.nb[0] = 2; t_vc.nb[1] = 2 * C; t_vc.nb[2] = t_vc.nb[3] = d * 2 * C;
             RC_TRY(spy_hip_op_dup(st, &t_vt, &t_vc));
         }
-        bool attn_done = false;
         if (fuse_attn) {          // scores, masked softmax and the product with V^T in one kernel: no score / probability matrix in memory
-            const int rc = spy_prompt_attn_launch(st, (const uint16_t *)xn, (const uint16_t *)m->k_cache[il], (const uint16_t *)m->v_cache[il], o2,
-                                                  T, (int)H, (int)hd, P, C, scale);
-            if (rc != SPY_HIP_EUNSUPPORTED) { RC_TRY(rc); attn_done = true; }
-        }
-        if (!attn_done) {
+            RC_TRY(spy_prompt_attn_launch(st, (const uint16_t *)xn, (const uint16_t *)m->k_cache[il], (const uint16_t *)m->v_cache[il], o2,
+                                          T, (int)H, (int)hd, P, C, scale));
+        } else {
         spy_hip_tensor t_kall = T3s(SPY_HIP_F16, m->k_cache[il], hd, n_kv, H, 2, 2 * d, 2 * hd);
         spy_hip_tensor t_vall = T3s(SPY_HIP_F16, m->v_cache[il], n_kv, hd, H, 2, 2 * C, 2 * C * hd);
         // causal_ok: the softmax below takes the row kernel, which reads no score beyond a row's causal length and writes
