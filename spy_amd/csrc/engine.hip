@@ -273,6 +273,8 @@ int spy_rope_store_launch(hipStream_t st, const float *q, const float *k, const 
 int spy_vt_store_launch(hipStream_t st, const float *v, uint16_t *vc, int T, int d, int64_t n_ctx);
 int spy_prompt_attn_launch(hipStream_t st, const uint16_t *q16, const uint16_t *k_cache, const uint16_t *v_cache, float *out,
                            int T, int H, int hd, int past, int64_t n_ctx, float scale);                                       // prompt_attn.hip
+int spy_gemm_q8act_pair(hipStream_t st, int wtype, const void *w1, const void *w2, const void *xq, float *dst1, float *dst2,
+                        int64_t M, int64_t K, int64_t T, int64_t dst_stride);                                                  // gemm.hip
 int spy_softmax_causal_launch(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *dst, float scale, int n_past);   // ops.hip
 int spy_softmax_row_ok(int64_t ne0);                                                                                         // ops.hip
 
@@ -414,8 +416,11 @@ static int forward_ops(spy_hip_llama *m, hipStream_t st, const int32_t *tokens_h
         t_nw.data = (void *)L.ffn_norm;
         if (fuse_act) {
             RC_TRY(spy_norm_mul_q8_launch(st, t1, 4 * d, (const float *)L.ffn_norm, c.eps, scr, T, d));
-            RC_TRY(spy_hip_gemm_q8_0act(st, L.t_up, L.w_up, scr, up, F, d, T, F));
-            RC_TRY(spy_hip_gemm_q8_0act(st, L.t_gate, L.w_gate, scr, gate, F, d, T, F));
+            if (L.t_up == L.t_gate) RC_TRY(spy_gemm_q8act_pair(st, L.t_up, L.w_up, L.w_gate, scr, up, gate, F, d, T, F));   // one grid for both
+            else {
+                RC_TRY(spy_hip_gemm_q8_0act(st, L.t_up, L.w_up, scr, up, F, d, T, F));
+                RC_TRY(spy_hip_gemm_q8_0act(st, L.t_gate, L.w_gate, scr, gate, F, d, T, F));
+            }
             RC_TRY(spy_silu_mul_q8_launch(st, gate, up, scr, T, F));        // Silu -> Mul -> Q8_0
             RC_TRY(spy_hip_gemm_q8_0act(st, L.t_down, L.w_down, scr, o, d, F, T, d));
         } else {

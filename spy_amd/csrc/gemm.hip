@@ -43,8 +43,15 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 static __device__ __forceinline__ uint32_t nib_m8(uint32_t lo) { return (lo + 0x78787878u) ^ 0x80808080u; }
 
 template <int WT>
-__global__ __launch_bounds__(256, GEMM_WGS) void gemm_q8act_kernel(const uint8_t *__restrict__ W, const uint8_t *__restrict__ xq, float *__restrict__ dst,
-                                                            int M, int K, int T, int64_t dst_stride) {
+__global__ __launch_bounds__(256, GEMM_WGS) void gemm_q8act_kernel(const uint8_t *__restrict__ W1, const uint8_t *__restrict__ xq, float *__restrict__ dst1,
+                                                            int M, int K, int T, int64_t dst_stride, const uint8_t *__restrict__ W2, float *__restrict__ dst2) {
+    // Optionally two weight matrices of the same shape against the same activations in one grid (gate and up): the
+    // workgroups of the second follow those of the first, which halves the share of the grid's tail.
+    const int tiles1 = (M + GEMM_TILE - 1) / GEMM_TILE;
+    const bool second = W2 != nullptr && (int)blockIdx.x >= tiles1;
+    const uint8_t *W = second ? W2 : W1;
+    float *dst = second ? dst2 : dst1;
+    const int bx = second ? (int)blockIdx.x - tiles1 : (int)blockIdx.x;
     constexpr int PAIR_DW = (WT == SPY_HIP_Q4_0) ? 9 : 17;       // dwords per pair of weight blocks
     constexpr int HALF_DW = (WT == SPY_HIP_Q4_0) ? 5 : 9;        // dwords that cover one block of the pair
     __shared__ __attribute__((aligned(16))) uint8_t sA[2][GEMM_TILE * GEMM_ROWB];
@@ -52,7 +59,7 @@ __global__ __launch_bounds__(256, GEMM_WGS) void gemm_q8act_kernel(const uint8_t
     __shared__ uint16_t sAd[2][2][GEMM_TILE];                                // fp16 block scales [buffer][block of the pair][row]
     __shared__ uint16_t sBd[2][2][GEMM_TILE];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
-    const int m0 = blockIdx.x * GEMM_TILE, t0 = blockIdx.y * GEMM_TILE;
+    const int m0 = bx * GEMM_TILE, t0 = blockIdx.y * GEMM_TILE;
     const int nstage = K / 64;
     const size_t RBw = (size_t)(K / 32) * (WT == SPY_HIP_Q4_0 ? 18 : 34), RBx = (size_t)(K / 32) * 34;
 
@@ -559,11 +566,29 @@ extern "C" int spy_hip_gemm_q8_0act(void *stream, int wtype, const void *w_dev, 
     // weights) beat the 128 x 128 tile, which leaves most of the part idle there (T = 16: 32 us against 130-230 us)
     if ((wtype == SPY_HIP_Q4_K || wtype == SPY_HIP_Q6_K) && T <= 32 && K <= 12288 && !force)
         return spy_hip_gemv_q8_0act(stream, wtype, w_dev, xq_dev, dst_dev, nullptr, M, K, T, dst_stride);
-    if (wtype == SPY_HIP_Q4_0) gemm_q8act_kernel<SPY_HIP_Q4_0><<<grid, dim3(256), 0, st>>>((const uint8_t *)w_dev, (const uint8_t *)xq_dev, dst_dev, (int)M, (int)K, (int)T, dst_stride);
-    else if (wtype == SPY_HIP_Q8_0) gemm_q8act_kernel<SPY_HIP_Q8_0><<<grid, dim3(256), 0, st>>>((const uint8_t *)w_dev, (const uint8_t *)xq_dev, dst_dev, (int)M, (int)K, (int)T, dst_stride);
+    if (wtype == SPY_HIP_Q4_0) gemm_q8act_kernel<SPY_HIP_Q4_0><<<grid, dim3(256), 0, st>>>((const uint8_t *)w_dev, (const uint8_t *)xq_dev, dst_dev, (int)M, (int)K, (int)T, dst_stride, nullptr, nullptr);
+    else if (wtype == SPY_HIP_Q8_0) gemm_q8act_kernel<SPY_HIP_Q8_0><<<grid, dim3(256), 0, st>>>((const uint8_t *)w_dev, (const uint8_t *)xq_dev, dst_dev, (int)M, (int)K, (int)T, dst_stride, nullptr, nullptr);
     else if (wtype == SPY_HIP_Q4_K) gemm_kq_kernel<SPY_HIP_Q4_K><<<grid, dim3(256), 0, st>>>((const uint8_t *)w_dev, (const uint8_t *)xq_dev, dst_dev, (int)M, (int)K, (int)T, dst_stride);
     else if (wtype == SPY_HIP_Q6_K) gemm_kq_kernel<SPY_HIP_Q6_K><<<grid, dim3(256), 0, st>>>((const uint8_t *)w_dev, (const uint8_t *)xq_dev, dst_dev, (int)M, (int)K, (int)T, dst_stride);
     else return SPY_HIP_EUNSUPPORTED;
+    return SPY_LAUNCH_RC();
+}
+
+// Two weight matrices of the same type and shape against the same activations (gate and up of a layer): one grid
+// where the 128 x 128 tile kernel applies, else two launches.  Same results as two calls of spy_hip_gemm_q8_0act.
+int spy_gemm_q8act_pair(hipStream_t st, int wtype, const void *w1, const void *w2, const void *xq, float *dst1, float *dst2,
+                        int64_t M, int64_t K, int64_t T, int64_t dst_stride) {
+    SPY_CHECK_ARG(w1 && w2 && xq && dst1 && dst2 && M > 0 && K > 0 && T > 0 && dst_stride >= M);
+    const int64_t tiles = (M + GEMM_TILE - 1) / GEMM_TILE, ttiles = (T + GEMM_TILE - 1) / GEMM_TILE;
+    const bool tile_kernel = (wtype == SPY_HIP_Q4_0 || wtype == SPY_HIP_Q8_0) && K % 64 == 0 && T > 64 && tiles * ttiles > GEMM_SKINNY_MAX_TILES &&
+                             2 * tiles <= 0x7fffffff && ttiles <= 65535 && !getenv("SPY_HIP_GEMM");
+    if (!tile_kernel) {
+        int rc = spy_hip_gemm_q8_0act(st, wtype, w1, xq, dst1, M, K, T, dst_stride);
+        return rc ? rc : spy_hip_gemm_q8_0act(st, wtype, w2, xq, dst2, M, K, T, dst_stride);
+    }
+    const dim3 grid((unsigned)(2 * tiles), (unsigned)ttiles);
+    if (wtype == SPY_HIP_Q4_0) gemm_q8act_kernel<SPY_HIP_Q4_0><<<grid, dim3(256), 0, st>>>((const uint8_t *)w1, (const uint8_t *)xq, dst1, (int)M, (int)K, (int)T, dst_stride, (const uint8_t *)w2, dst2);
+    else gemm_q8act_kernel<SPY_HIP_Q8_0><<<grid, dim3(256), 0, st>>>((const uint8_t *)w1, (const uint8_t *)xq, dst1, (int)M, (int)K, (int)T, dst_stride, (const uint8_t *)w2, dst2);
     return SPY_LAUNCH_RC();
 }
 

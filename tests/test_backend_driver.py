@@ -120,6 +120,22 @@ def test_engine_prompt_softmax_without_mask_tensor_matches_submit_path(monkeypat
 
 
 @pytest.mark.gpu
+def test_engine_prompt_pass_wide_layer_matches_submit_path(monkeypatch):
+    """A layer wide enough (and a pass long enough) for the 128 x 128 tile GEMM, where the engine runs gate and up as
+    one grid: same bits as the submit path's separate MatMuls (attention as MatMul -> Softmax -> MatMul for this test)."""
+    monkeypatch.setenv("SPY_HIP_PROMPT_ATTN", "0")
+    from spy_amd import backend_driver as B
+    from spy_amd import model as M
+    cfg = M.Config(n_layer=1, n_embd=512, n_head=4, n_ff=2816, n_vocab=512, n_ctx=1040, wtype=O.Q4_0)
+    tensors = M.synth_model(cfg, seed=3)
+    host, eng = B.HostModel(cfg, tensors), M.Engine(cfg, tensors)
+    prompt = np.random.default_rng(8).integers(0, cfg.n_vocab, 1024).astype(np.int32)
+    lg_h, lg_e = host.forward(prompt, 0), eng.forward(prompt, 0)
+    assert np.isfinite(lg_e).all() and np.array_equal(lg_h, lg_e)
+    host.close()
+
+
+@pytest.mark.gpu
 def test_submit_path_k_quant_mix_with_outliers():
     """The Q4_K_M-style mix (Q4_K for q, k, o, gate, up; Q6_K for v, down and the head; 0.1 % of the
     weights x20) through Backend::submit, against the oracle.  The reference has no K-quant arithmetic:
