@@ -121,18 +121,20 @@ def test_engine_prompt_softmax_without_mask_tensor_matches_submit_path(monkeypat
 
 @pytest.mark.gpu
 def test_engine_prompt_pass_wide_layer_matches_submit_path(monkeypatch):
-    """A layer wide enough (and a pass long enough) for the 128 x 128 tile GEMM, where the engine runs gate and up as
+    """Layers wide enough (and passes long enough) for the 128 x 128 tile GEMM, where the engine runs gate and up as
     one grid: same bits as the submit path's separate MatMuls (attention as MatMul -> Softmax -> MatMul for this test)."""
     monkeypatch.setenv("SPY_HIP_PROMPT_ATTN", "0")
     from spy_amd import backend_driver as B
     from spy_amd import model as M
-    cfg = M.Config(n_layer=1, n_embd=512, n_head=4, n_ff=2816, n_vocab=512, n_ctx=1040, wtype=O.Q4_0)
-    tensors = M.synth_model(cfg, seed=3)
-    host, eng = B.HostModel(cfg, tensors), M.Engine(cfg, tensors)
-    prompt = np.random.default_rng(8).integers(0, cfg.n_vocab, 1024).astype(np.int32)
-    lg_h, lg_e = host.forward(prompt, 0), eng.forward(prompt, 0)
-    assert np.isfinite(lg_e).all() and np.array_equal(lg_h, lg_e)
-    host.close()
+    for wtype, dims in ((O.Q4_0, (512, 4, 2816, 1024)), (O.Q8_0, (2048, 16, 2816, 1408))):
+        n_embd, n_head, n_ff, n_tok = dims       # the second: wq, wk, wv, wo and down wide enough for the tile kernel too
+        cfg = M.Config(n_layer=1, n_embd=n_embd, n_head=n_head, n_ff=n_ff, n_vocab=512, n_ctx=n_tok + 16, wtype=wtype)
+        tensors = M.synth_model(cfg, seed=3)
+        host, eng = B.HostModel(cfg, tensors), M.Engine(cfg, tensors)
+        prompt = np.random.default_rng(8).integers(0, cfg.n_vocab, n_tok).astype(np.int32)
+        lg_h, lg_e = host.forward(prompt, 0), eng.forward(prompt, 0)
+        assert np.isfinite(lg_e).all() and np.array_equal(lg_h, lg_e), dims
+        host.close(); eng.close()
 
 
 @pytest.mark.gpu
