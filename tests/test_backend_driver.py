@@ -126,7 +126,7 @@ def test_engine_prompt_pass_wide_layer_matches_submit_path(monkeypatch):
     monkeypatch.setenv("SPY_HIP_PROMPT_ATTN", "0")
     from spy_amd import backend_driver as B
     from spy_amd import model as M
-    for wtype, dims in ((O.Q4_0, (512, 4, 2816, 1024)), (O.Q8_0, (2048, 16, 2816, 1408))):
+    for wtype, dims in ((O.Q4_0, (512, 4, 2816, 1024)), (O.Q8_0, (2048, 16, 2816, 1408)), (O.Q4_0, (2048, 16, 2816, 1408))):
         n_embd, n_head, n_ff, n_tok = dims       # the second: wq, wk, wv, wo and down wide enough for the tile kernel too
         cfg = M.Config(n_layer=1, n_embd=n_embd, n_head=n_head, n_ff=n_ff, n_vocab=512, n_ctx=n_tok + 16, wtype=wtype)
         tensors = M.synth_model(cfg, seed=3)
