@@ -49,6 +49,33 @@ def test_small_model_prefill_decode_and_tokens(wtype, t_out, t_emb):
     eng.close()
 
 
+@pytest.mark.parametrize("name,kw", [
+    ("Q4_0", dict(wtype=O.Q4_0)),
+    ("Q8_0, Q8_0 embeddings", dict(wtype=O.Q8_0, t_tok_embd=O.Q8_0)),
+    ("Q4_K_M mix", dict(wtype=O.Q4_K, t_out=O.Q6_K, tensor_types={"attn_v": O.Q6_K, "ffn_down": O.Q6_K})),
+])
+def test_prompt_passes_of_many_tokens_against_oracle(name, kw):
+    """Passes of 16 tokens and more take the matrix-core GEMMs, the fused activation producers and the attention
+    kernel: logits of every token and both caches against the CPU oracle, for a first pass and for one on top of
+    a filled cache (head dimension 128, as the attention kernel requires)."""
+    from spy_amd import model as M
+    from tests.gpu_util import E2E_TOL
+    cfg = M.Config(n_layer=2, n_embd=256, n_head=2, n_ff=768, n_vocab=512, n_ctx=96, **kw)
+    eng, ora, _ = _mk(cfg, seed=13)
+    prompt = np.random.default_rng(17).integers(0, cfg.n_vocab, 88).astype(np.int32)
+    for start, stop in ((0, 48), (48, 88)):
+        lg_g, lg_o = eng.forward(prompt[start:stop], start), ora.forward(prompt[start:stop], start)
+        _close(lg_g, lg_o, "%s: logits of the pass over tokens %d..%d" % (name, start, stop), E2E_TOL)
+        assert (np.argmax(lg_g, axis=1) == np.argmax(lg_o, axis=1)).mean() > 0.9
+    for il in range(cfg.n_layer):
+        kg, ko = _f16(eng.read_buffer("k_cache", il, np.uint16)), _f16(ora.k_cache[il])
+        vg, vo = _f16(eng.read_buffer("v_cache", il, np.uint16)), _f16(ora.v_cache[il])
+        _close(kg, ko, "K cache layer %d" % il, E2E_TOL if il else 2e-3)      # layer 0: one fp16 ulp; deeper layers carry the pass's noise
+        _close(vg, vo, "V cache layer %d" % il, E2E_TOL if il else 2e-3)
+        assert np.array_equal(kg == 0, ko == 0) and np.array_equal(vg == 0, vo == 0)
+    eng.close()
+
+
 def _comfortable_prompt(ora, cfg, n_prompt, n_predict, min_margin, tries=40):
     """A seeded random prompt whose greedy continuation on the CPU path has the widest top-1/top-2
     logit gaps (stops early once the smallest gap exceeds min_margin logit standard deviations):
