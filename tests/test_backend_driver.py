@@ -120,6 +120,22 @@ def test_engine_prompt_softmax_without_mask_tensor_matches_submit_path(monkeypat
 
 
 @pytest.mark.gpu
+def test_engine_prompt_pass_heads_of_64():
+    """Heads the attention kernel does not take (it is built for 128-wide heads): the engine falls back to
+    MatMul -> Softmax -> MatMul by itself, bit-identical to the submit path."""
+    from spy_amd import backend_driver as B
+    from spy_amd import model as M
+    cfg = M.Config(n_layer=2, n_embd=256, n_head=4, n_ff=768, n_vocab=512, n_ctx=96, wtype=O.Q8_0)
+    tensors = M.synth_model(cfg, seed=19)
+    host, eng = B.HostModel(cfg, tensors), M.Engine(cfg, tensors)
+    prompt = np.random.default_rng(6).integers(0, cfg.n_vocab, 90).astype(np.int32)
+    for start, stop in ((0, 50), (50, 90)):
+        lg_h, lg_e = host.forward(prompt[start:stop], start), eng.forward(prompt[start:stop], start)
+        assert np.isfinite(lg_e).all() and np.array_equal(lg_h, lg_e), (start, stop)
+    host.close(); eng.close()
+
+
+@pytest.mark.gpu
 def test_engine_prompt_pass_wide_layer_matches_submit_path(monkeypatch):
     """Layers wide enough (and passes long enough) for the 128 x 128 tile GEMM, where the engine runs gate and up as
     one grid: same bits as the submit path's separate MatMuls (attention as MatMul -> Softmax -> MatMul for this test)."""
