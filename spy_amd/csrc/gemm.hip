@@ -35,8 +35,8 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 #ifndef GEMM_WGS
 #define GEMM_WGS 3                // workgroups per CU the tile kernel is compiled for (register budget 512 / GEMM_WGS per lane)
 #endif
-#ifndef GEMM_PF
-#define GEMM_PF 1                // stages of global loads in flight per thread (the kernel is bound by its scale epilogue on the vector units: 2 and 3 measured the same)
+#ifndef GEMM_PF_Q4_0
+#define GEMM_PF_Q4_0 2           // Q4_0: two stages of global loads in flight (+2-5 % for M >= 11008, the operands come from beyond the L2); Q8_0 keeps one: two would spill
 #endif
 
 // 32-bit word of 4 packed nibbles (already masked to 0..15 per byte) -> 4 int8 of (n - 8)
@@ -52,6 +52,7 @@ __global__ __launch_bounds__(256, GEMM_WGS) void gemm_q8act_kernel(const uint8_t
     const uint8_t *W = second ? W2 : W1;
     float *dst = second ? dst2 : dst1;
     const int bx = second ? (int)blockIdx.x - tiles1 : (int)blockIdx.x;
+    constexpr int PF = (WT == SPY_HIP_Q4_0) ? GEMM_PF_Q4_0 : 1; // stages of global loads in flight per thread
     constexpr int PAIR_DW = (WT == SPY_HIP_Q4_0) ? 9 : 17;       // dwords per pair of weight blocks
     constexpr int HALF_DW = (WT == SPY_HIP_Q4_0) ? 5 : 9;        // dwords that cover one block of the pair
     __shared__ __attribute__((aligned(16))) uint8_t sA[2][GEMM_TILE * GEMM_ROWB];
@@ -72,9 +73,9 @@ __global__ __launch_bounds__(256, GEMM_WGS) void gemm_q8act_kernel(const uint8_t
     const uint32_t dshift = half ? 16 : 0;                    // the fp16 scale sits in the upper / lower half of raw[0]
     const uint32_t *gA = (const uint32_t *)(W + (size_t)min(m0 + lrow, M - 1) * RBw) + half * (HALF_DW - 1);
     const uint32_t *gB = (const uint32_t *)(xq + (size_t)min(t0 + lrow, T - 1) * RBx) + half * 8;
-    // Global loads run GEMM_PF stages ahead of the stage being multiplied (a ring of raw registers): with one
+    // Global loads run PF stages ahead of the stage being multiplied (a ring of raw registers): with one
     // stage ahead a workgroup advances one stage per memory round trip, whatever the matrix cores could do.
-    uint32_t rawA[GEMM_PF][HALF_DW], rawB[GEMM_PF][9];
+    uint32_t rawA[PF][HALF_DW], rawB[PF][9];
     auto gload = [&](int slot, int s) {                      // 4-byte aligned: 128-bit loads + one dword
         __builtin_memcpy(rawA[slot], __builtin_assume_aligned(gA + (size_t)s * PAIR_DW, 4), HALF_DW * 4);
         __builtin_memcpy(rawB[slot], __builtin_assume_aligned(gB + (size_t)s * 17, 4), 36);
@@ -145,17 +146,17 @@ __global__ __launch_bounds__(256, GEMM_WGS) void gemm_q8act_kernel(const uint8_t
     };
 
 #pragma unroll
-    for (int j = 0; j < GEMM_PF; j++) gload(j, min(j, nstage - 1));
+    for (int j = 0; j < PF; j++) gload(j, min(j, nstage - 1));
     unpack(0, 0);
     __syncthreads();
-    for (int s0 = 0; s0 < nstage; s0 += GEMM_PF) {
+    for (int s0 = 0; s0 < nstage; s0 += PF) {
 #pragma unroll
-        for (int j = 0; j < GEMM_PF; j++) {
+        for (int j = 0; j < PF; j++) {
             const int s = s0 + j;                              // stage in LDS buffer s & 1; its raw registers (slot j) are free
             if (s < nstage) {
-                gload(j, min(s + GEMM_PF, nstage - 1));      // unconditional: the last stages re-read the last one
+                gload(j, min(s + PF, nstage - 1));      // unconditional: the last stages re-read the last one
                 multiply(s & 1);
-                if (s + 1 < nstage) unpack((s & 1) ^ 1, (j + 1) % GEMM_PF);
+                if (s + 1 < nstage) unpack((s & 1) ^ 1, (j + 1) % PF);
                 __syncthreads();
             }
         }
