@@ -186,7 +186,9 @@ typedef struct spy_hip_llama spy_hip_llama;
 int spy_hip_llama_create(const spy_hip_llama_desc *desc, spy_hip_llama **out);
 int spy_hip_llama_destroy(spy_hip_llama *m);
 /* One forward pass over n_token tokens at positions n_past.. (any n_token >= 1; passes of more
- * than one token run operator by operator).  logits_host: NULL or n_vocab*n_token floats. */
+ * than one token run the operator kernels one after the other below 16 tokens and, from 16 tokens, the
+ * matrix-core GEMMs with fused activation producers and the attention kernel; long prompts go through in
+ * chunks of 2048 tokens).  logits_host: NULL (no output head is computed) or n_vocab*n_token floats. */
 int spy_hip_llama_forward(spy_hip_llama *m, void *stream, const int32_t *tokens_host, int32_t n_token, int32_t n_past,
                           float *logits_host);
 /* The same pass with the output head applied to the last token only: logits_last_host receives
