@@ -365,7 +365,8 @@ static int launch_gemm_skinny(hipStream_t st, const void *w, const void *xq, flo
 // Same tiling.  A stage is a quarter super-block (64 elements), a thread unpacks one 32-element half of it:
 //   Q4_K: sub-block a = 2j + half of the super-block: nibbles 0..15 as int8, scale d*sc and minimum dmin*m;
 //         value = d*sc*q - dmin*m, so the tile gets  dx * (d*sc * I - dmin*m * sum(q_x))  per block, with
-//         dx * sum(q_x) prepared once per activation block.
+//         dx * sum(q_x) prepared once per activation block.  The minimum terms are an outer product over the
+//         block index: one fp32 MFMA per tile and stage adds those of both blocks (k = block of the pair).
 //   Q6_K: 32 elements l + 32 m (m = 2 (j & 1) + half) of half n = j >> 1: (q - 32) as int8; they span TWO
 //         16-element scale groups, which the 32x32x32 MFMA keeps apart when the right operand is zeroed in
 //         one lane half (lanes 0..31 carry k = 0..15, lanes 32..63 k = 16..31): two MFMAs, I_lo and I_hi,
@@ -482,10 +483,12 @@ __global__ __launch_bounds__(256, 2) void gemm_kq_kernel(const uint8_t *__restri
 #pragma unroll
             for (int i = 0; i < 2; i++) {
                 int am[16];
+                if constexpr (!Q4K) {
 #pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    const int4 u = *(const int4 *)&sAm[b][blk][wm * 64 + i * 32 + g * 8 + (lane >> 5) * 4];
-                    am[4 * g] = u.x; am[4 * g + 1] = u.y; am[4 * g + 2] = u.z; am[4 * g + 3] = u.w;
+                    for (int g = 0; g < 4; g++) {
+                        const int4 u = *(const int4 *)&sAm[b][blk][wm * 64 + i * 32 + g * 8 + (lane >> 5) * 4];
+                        am[4 * g] = u.x; am[4 * g + 1] = u.y; am[4 * g + 2] = u.z; am[4 * g + 3] = u.w;
+                    }
                 }
                 if constexpr (Q4K) {
                     float dw[16];
@@ -496,15 +499,11 @@ __global__ __launch_bounds__(256, 2) void gemm_kq_kernel(const uint8_t *__restri
                     }
 #pragma unroll
                     for (int j = 0; j < 2; j++) {
-                        const int col = wn * 64 + j * 32 + (lane & 31);
-                        const float dx = sBd[b][blk][col], dxs = sBs[b][blk][col];
+                        const float dx = sBd[b][blk][wn * 64 + j * 32 + (lane & 31)];
                         v16i z = {0};
                         const v16i I = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], z, 0, 0, 0);
 #pragma unroll
-                        for (int r = 0; r < 16; r++) {
-                            acc[i][j][r] = fmaf(dw[r] * dx, (float)I[r], acc[i][j][r]);
-                            acc[i][j][r] = fmaf(-__int_as_float(am[r]), dxs, acc[i][j][r]);
-                        }
+                        for (int r = 0; r < 16; r++) acc[i][j][r] = fmaf(dw[r] * dx, (float)I[r], acc[i][j][r]);
                     }
                 } else {
                     // d (fp16) x dx (fp16) for the whole tile from one fp16 MFMA: scales at k = 0, zeros elsewhere (exact in fp32)
@@ -526,6 +525,25 @@ __global__ __launch_bounds__(256, 2) void gemm_kq_kernel(const uint8_t *__restri
                         }
                         __builtin_amdgcn_sched_barrier(0);       // one tile's three MFMA results at a time: two would not fit the register file
                     }
+                }
+            }
+        }
+        if constexpr (Q4K) {
+            // the minimum terms of the stage's two blocks, -(dmin * m)[row][blk] * (dx * sum q_x)[token][blk], are an outer
+            // product over the block index: one fp32 MFMA per tile (k = block of the pair, carried by the lane half)
+            // adds both to the accumulators instead of 32 fmas per lane
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                const float a2 = -__int_as_float(sAm[b][lane >> 5][wm * 64 + i * 32 + (lane & 31)]);
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    const float b2 = sBs[b][lane >> 5][wn * 64 + j * 32 + (lane & 31)];
+                    v16f c;
+#pragma unroll
+                    for (int r = 0; r < 16; r++) c[r] = acc[i][j][r];
+                    c = __builtin_amdgcn_mfma_f32_32x32x2f32(a2, b2, c, 0, 0, 0);
+#pragma unroll
+                    for (int r = 0; r < 16; r++) acc[i][j][r] = c[r];
                 }
             }
         }
