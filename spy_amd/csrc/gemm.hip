@@ -520,7 +520,8 @@ __global__ __launch_bounds__(256, 2) void gemm_kq_kernel(const uint8_t *__restri
                         const v16f S = __builtin_amdgcn_mfma_f32_32x32x8f16(ha, hb, zf, 0, 0, 0);
 #pragma unroll
                         for (int r = 0; r < 16; r++) {
-                            const int sv = (int)(int16_t)(am[r] & 0xFFFF) * Ilo[r] + (am[r] >> 16) * Ihi[r];
+                            // 24-bit multiplies (full rate): |I| <= 16 * 31 * 127 and the scales are int8
+                            const int sv = __mul24((int)(int16_t)(am[r] & 0xFFFF), Ilo[r]) + __mul24(am[r] >> 16, Ihi[r]);
                             acc[i][j][r] = fmaf(S[r], (float)sv, acc[i][j][r]);
                         }
                         __builtin_amdgcn_sched_barrier(0);       // one tile's three MFMA results at a time: two would not fit the register file
