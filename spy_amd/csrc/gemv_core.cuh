@@ -368,8 +368,9 @@ static __device__ __forceinline__ float dot_pair(const uint32_t *w, const int4 x
             iB = __builtin_amdgcn_sdot4((int)((w[4 + i] >> 4) & 0x0F0F0F0Fu), xb[i], iB, false);
         }
         if (dump2) { dump2[0] = iA; dump2[1] = iB; }
-        acc = fmaf(__int_as_float(mm.x), d * (float)(scA * iA) - dmin * (float)(mA * mm.y), acc);
-        acc = fmaf(__int_as_float(mm.z), d * (float)(scB * iB) - dmin * (float)(mB * mm.w), acc);
+        // 24-bit multiplies (full rate): |i| <= 32 * 15 * 127, |sum q_x| <= 32 * 127, scales below 64
+        acc = fmaf(__int_as_float(mm.x), d * (float)__mul24(scA, iA) - dmin * (float)__mul24(mA, mm.y), acc);
+        acc = fmaf(__int_as_float(mm.z), d * (float)__mul24(scB, iB) - dmin * (float)__mul24(mB, mm.w), acc);
         return acc;
     } else if constexpr (WT == SPY_HIP_Q6_K) {
         // lane (n, e): elements l + 32 m, l in [16e, 16e + 16), m = 0..3 of half n: 6-bit quants from the low /
@@ -393,7 +394,7 @@ static __device__ __forceinline__ float dot_pair(const uint32_t *w, const int4 x
         for (int m = 0; m < 4; m++) {
             const int k = e + 2 * m;                                     // scale byte of the half (0..7)
             const int sc = (int)(int8_t)(((k < 4 ? s0 : s1) >> (8 * (k & 3))) & 0xFFu);
-            acc = fmaf(dx[m] * d, (float)(sc * isum[m]), acc);
+            acc = fmaf(dx[m] * d, (float)__mul24(sc, isum[m]), acc);               // |isum| <= 16 * 32 * 127: 24-bit multiply (full rate)
         }
         return acc;
     } else {
