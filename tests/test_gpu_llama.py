@@ -240,6 +240,43 @@ def test_llama2_7b_q4_0_greedy_32_tokens():
     eng.close()
 
 
+@pytest.mark.timeout(600)
+def test_llama2_7b_prompt_4096_properties(monkeypatch):
+    """The headline shape at full size (7B, Q4_0 body, Q6_K head, 4096-token prompt), through properties that need no
+    CPU pass.  (a) Chunking: the prompt in chunks of 2048 (default) and of 1024 tokens gives the same last-row logits
+    bit for bit: every output of the matrix-core kernels is accumulated in an order that does not depend on the
+    tiling, and a query attends to the same cached positions in the same order whatever chunk it arrives in.
+    (b) Causality: the first 2048 tokens alone write the K cache rows (last layer) the full prompt writes.
+    (c) The token loop on top: decode_greedy and one-token forward passes emit the same tokens."""
+    from spy_amd import model as M
+    cfg = M.Config.llama2_7b(n_ctx=4096 + 32, wtype=O.Q4_0, t_out=O.Q6_K)
+    tensors = M.synth_model(cfg, seed=1234, quantizer=M.random_k_blocks)      # K-quant head: random well-formed blocks
+    prompt = np.random.default_rng(4096).integers(0, cfg.n_vocab, 4096).astype(np.int32)
+    eng = M.Engine(cfg, tensors)
+    last_2048 = eng.forward_last(prompt, 0)
+    assert np.isfinite(last_2048).all() and last_2048.std() > 0
+    k_full = eng.read_buffer("k_cache", cfg.n_layer - 1, np.uint16).reshape(cfg.n_ctx, cfg.n_embd)[:2048].copy()
+    first = int(np.argmax(last_2048))
+    toks = eng.decode_greedy(first, 4096, 8)
+    eng.close()
+    eng2 = M.Engine(cfg, tensors)
+    monkeypatch.setenv("SPY_HIP_PREFILL_CHUNK", "1024")
+    last_1024 = eng2.forward_last(prompt, 0)
+    monkeypatch.delenv("SPY_HIP_PREFILL_CHUNK")
+    assert np.array_equal(last_1024, last_2048)
+    tok, own = first, []
+    for i in range(8):
+        tok = int(np.argmax(eng2.forward(np.array([tok], np.int32), 4096 + i)[0]))
+        own.append(tok)
+    assert own == toks.tolist(), (own, toks.tolist())
+    eng2.close()
+    eng3 = M.Engine(cfg, tensors)
+    eng3.forward(prompt[:2048], 0, want_logits=False)
+    k_half = eng3.read_buffer("k_cache", cfg.n_layer - 1, np.uint16).reshape(cfg.n_ctx, cfg.n_embd)[:2048]
+    assert np.array_equal(k_half, k_full)
+    eng3.close()
+
+
 @pytest.mark.parametrize("name,kw", [
     ("Q4_0 body, Q6_K head", dict(wtype=O.Q4_0, t_out=O.Q6_K)),
     ("Q4_K + Q6_K head", dict(wtype=O.Q4_K, t_out=O.Q6_K)),
