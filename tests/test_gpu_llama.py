@@ -241,16 +241,20 @@ def test_llama2_7b_q4_0_greedy_32_tokens():
 
 
 @pytest.mark.timeout(600)
-def test_llama2_7b_prompt_4096_properties(monkeypatch):
-    """The headline shape at full size (7B, Q4_0 body, Q6_K head, 4096-token prompt), through properties that need no
-    CPU pass.  (a) Chunking: the prompt in chunks of 2048 (default) and of 1024 tokens gives the same last-row logits
+@pytest.mark.parametrize("name,kw", [
+    ("Q4_0 body, Q6_K head", dict(wtype=O.Q4_0, t_out=O.Q6_K)),
+    ("Q8_0", dict(wtype=O.Q8_0)),
+    ("Q4_K_M mix", dict(wtype=O.Q4_K, t_out=O.Q6_K, tensor_types={"attn_v": O.Q6_K, "ffn_down": O.Q6_K})),
+])
+def test_llama2_7b_prompt_4096_properties(name, kw, monkeypatch):
+    """The named configurations at full size (7B shape, 4096-token prompt), through properties that need no CPU pass.  (a) Chunking: the prompt in chunks of 2048 (default) and of 1024 tokens gives the same last-row logits
     bit for bit: every output of the matrix-core kernels is accumulated in an order that does not depend on the
     tiling, and a query attends to the same cached positions in the same order whatever chunk it arrives in.
     (b) Causality: the first 2048 tokens alone write the K cache rows (last layer) the full prompt writes.
     (c) The token loop on top: decode_greedy and one-token forward passes emit the same tokens."""
     from spy_amd import model as M
-    cfg = M.Config.llama2_7b(n_ctx=4096 + 32, wtype=O.Q4_0, t_out=O.Q6_K)
-    tensors = M.synth_model(cfg, seed=1234, quantizer=M.random_k_blocks)      # K-quant head: random well-formed blocks
+    cfg = M.Config.llama2_7b(n_ctx=4096 + 32, **kw)
+    tensors = M.synth_model(cfg, seed=1234, quantizer=M.random_k_blocks)      # K-quant matrices: random well-formed blocks
     prompt = np.random.default_rng(4096).integers(0, cfg.n_vocab, 4096).astype(np.int32)
     eng = M.Engine(cfg, tensors)
     last_2048 = eng.forward_last(prompt, 0)
