@@ -357,7 +357,13 @@ __global__ __launch_bounds__(ATL_THREADS, 4) void attn_layer_kernel(attn_layer_a
     uint32_t *sync = a.sync + (size_t)h * 96;
     // the launch count was written by the previous launch: an ordinary (scalar) load sees it, and stays out of
     // the vector-memory queue in which the first activation loads would otherwise wait behind it
-    const uint32_t target = (uint32_t)ATL_GPH * (sync[64] + 1u);
+    const uint32_t epoch = sync[64] + 1u;                            // number of this launch (per head), never 0
+    const uint32_t target = (uint32_t)ATL_GPH * epoch;
+    // q and the new K row of the head travel from the workgroups that compute them to those that use them as 64-bit words
+    // {value, epoch}, written and read with single atomic accesses: the value is valid exactly when its epoch is this
+    // launch's, so the consumers poll the data itself and no barrier (wait for the stores, counter, poll) sits between
+    // the projections and the scores.  128 words per head behind the barrier counters: 0..63 q, 64..127 k (fp16 pairs).
+    uint64_t *xch = (uint64_t *)(a.sync + (size_t)a.n_head * 96) + (size_t)h * 128;
     ATL_STAMP(0);
 
     int8_t *s_q = (int8_t *)smem;
@@ -463,15 +469,15 @@ __global__ __launch_bounds__(ATL_THREADS, 4) void attn_layer_kernel(attn_layer_a
         }
     }
     ATL_STAMP(2);
-    if (!publish_and_sync(sync, [&]() {
-            if (lane < ATL_WAVES) {
-                const int ww = g * ATL_WAVES + lane, pp = ww & 63;
-                const uint32_t pr = __float_as_uint(s_out[lane * 2]);
-                if (ww < 64) stc((uint32_t *)a.q16 + h * 64 + pp, pr);                                         // attn_score rounds Q to fp16 (mat.cpp:37)
-                else stc((uint32_t *)(a.kc + (size_t)pos * d) + h * 64 + pp, pr);                               // KCache_cpy: [token][head][hd]
-                stc(a.vc + (size_t)(h * 128 + ww) * n_ctx + pos, (uint16_t)__float_as_uint(s_out[lane * 2 + 1]));   // VCache_cpy: [d][C] column pos
-            }
-        })) return;
+    __syncthreads();
+    if (wave == 0 && lane < ATL_WAVES) {
+        const int ww = g * ATL_WAVES + lane, pp = ww & 63;
+        const uint32_t pr = __float_as_uint(s_out[lane * 2]);
+        __hip_atomic_store(xch + ww, ((uint64_t)epoch << 32) | pr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // attn_score rounds Q to fp16 (mat.cpp:37)
+        if (ww >= 64) stc((uint32_t *)(a.kc + (size_t)pos * d) + h * 64 + pp, pr);                          // KCache_cpy: [token][head][hd] (for the passes to come)
+        stc(a.vc + (size_t)(h * 128 + ww) * n_ctx + pos, (uint16_t)__float_as_uint(s_out[lane * 2 + 1]));   // VCache_cpy: [d][C] column pos (read after the barrier below)
+    }
+    __syncthreads();                                                 // s_out is written again below
     ATL_STAMP(3);
 
     // ================= B: t = (K.q) * scale for head h ================================================
@@ -480,8 +486,24 @@ __global__ __launch_bounds__(ATL_THREADS, 4) void attn_layer_kernel(attn_layer_a
     // pieces past the last cached token re-read the last piece (same cache line: no memory traffic for the unused part of the row)
     auto fetch_v = [&](int i) { vb[i] = *(const uint4 *)(vrow + (size_t)min(i * 64 + lane, (n_kv - 1) >> 3) * 8); };
     {
-        const uint32_t *qp = (const uint32_t *)a.q16 + h * 64 + (lane & 15) * 4;
-        const uint32_t qw[4] = {ldc(qp), ldc(qp + 1), ldc(qp + 2), ldc(qp + 3)};
+        // four words of q per lane, polled until all four carry this launch's epoch (bounded: the error flag is set and the
+        // pass goes on with what is there)
+        uint32_t qw[4];
+        {
+            const uint64_t *qs = xch + (lane & 15) * 4;
+            uint32_t spins = 0;
+            for (;;) {
+                bool ok = true;
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const uint64_t v = __hip_atomic_load(qs + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    qw[j] = (uint32_t)v; ok = ok && (uint32_t)(v >> 32) == epoch;
+                }
+                if (__all(ok)) break;
+                if (++spins > a.spin_limit) { if (lane == 0) __hip_atomic_store(&a.st->err, 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); break; }
+                __builtin_amdgcn_s_sleep(1);
+            }
+        }
         if (wave == 0) {
 #pragma unroll
             for (int k = 0; k < ATL_DEPTH_K; k++) fetch_k(k);
@@ -494,9 +516,21 @@ __global__ __launch_bounds__(ATL_THREADS, 4) void attn_layer_kernel(attn_layer_a
             if (k + ATL_DEPTH_K < ATL_RS) fetch_k(k + ATL_DEPTH_K);
             const int tok = 4 * (w + 128 * k) + (lane >> 4);
             uint4 kv = kb[k];
-            if (tok == pos) {                                        // written in step A by another workgroup: read it coherently
-                const uint32_t *p = (const uint32_t *)(a.kc + (size_t)tok * d + h * 128 + (lane & 15) * 8);
-                kv = make_uint4(ldc(p), ldc(p + 1), ldc(p + 2), ldc(p + 3));
+            if (tok == pos) {                                        // computed in step A by another workgroup: taken from the exchange words
+                const uint64_t *ks = xch + 64 + (lane & 15) * 4;
+                uint32_t kw4[4], spins = 0;
+                for (;;) {
+                    bool ok = true;
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        const uint64_t v = __hip_atomic_load(ks + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        kw4[j] = (uint32_t)v; ok = ok && (uint32_t)(v >> 32) == epoch;
+                    }
+                    if (ok) break;
+                    if (++spins > a.spin_limit) { __hip_atomic_store(&a.st->err, 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); break; }
+                    __builtin_amdgcn_s_sleep(1);
+                }
+                kv = make_uint4(kw4[0], kw4[1], kw4[2], kw4[3]);
             }
             const uint32_t kw[4] = {kv.x, kv.y, kv.z, kv.w};
             float s = 0.0f;

@@ -117,7 +117,7 @@ extern "C" int spy_hip_llama_create(const spy_hip_llama_desc *desc, spy_hip_llam
     }
     if (!rc && fused_ok(m) && m->wave) {   // one launch for the attention part of a layer where its workgroups are all resident (SPY_HIP_ATTN_SPLIT=1: three launches)
         const char *env = getenv("SPY_HIP_ATTN_SPLIT");
-        rc = dalloc(m, (void **)&m->attn_sync, (size_t)c.n_head * 96 * 4, true);
+        rc = dalloc(m, (void **)&m->attn_sync, (size_t)c.n_head * 96 * 4 + (size_t)c.n_head * 128 * 8, true);   // barrier counters + per head 128 {value, epoch} exchange words
         if (!rc && !(env && env[0] == '1') && m->hd == 128 && c.n_head * 8 <= m->num_cu && c.n_ctx <= 128 * 4 * ATL_RS && c.n_ctx <= 512 * ATL_RV)
         {
             bool ok = true;
