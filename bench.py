@@ -156,9 +156,9 @@ def main():
              "head": "wave_gemv_kernel<output head>", "qkv": "wave_gemv_kernel<qkv>", "scores": "attn_scores_kernel", "pv": "attn_pv_kernel"}
     # HBM bytes per launch from profiler counters (FETCH_SIZE + WRITE_SIZE, each scaled by what the same counter reads for a
     # copy kernel of known size; profiles/decode_7b_q4_0_ctx4096_hbm_traffic.md): measured for this model shape only.  The
-    # attention launch was counted at n_kv = 4103 (101.6 MB for 95.5 MB algorithmic); its traffic is scaled to this run's n_kv.
+    # attention launch was counted at n_kv = 4103 (101.7 MB for 95.5 MB algorithmic); its traffic is scaled to this run's n_kv.
     measured = {"gate_up": 51.18e6, "down": 25.83e6, "wo": 9.65e6, "head": 108.26e6,
-                "attention (qkv+scores+pv)": 101.6e6 * alg.get("attention (qkv+scores+pv)", 0) / (28311552 + 2 * 4103 * 8192)}
+                "attention (qkv+scores+pv)": 101.7e6 * alg.get("attention (qkv+scores+pv)", 0) / (28311552 + 2 * 4103 * 8192)}
     shape_ok = (cfg.n_embd, cfg.n_ff, cfg.wtype, args.model, cfg.t_out) == (4096, 11008, H.Q4_0, "q4_0", H.Q6_K) and cfg.n_layer == 32
     def roof(k):
         ach = alg[k] / (per_kernel[k] * 1e-6) / 1e9
