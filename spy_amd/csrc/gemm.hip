@@ -31,6 +31,7 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 
 #define GEMM_TILE 128
 #define GEMM_SKINNY_MAX_TILES 160 // the 32-row kernel is used up to 64 activation rows and wherever the 128 x 128 tiling would give at most this many workgroups (measured crossover)
+#define GEMM_KQ_SMALL_MAX_TILES 768 // Q4_K / Q6_K: the 64 x 64 tiling is used where it gives at most this many workgroups (3 per CU: all resident at once)
 #define GEMM_ROWB 80             // bytes per LDS row: 64 payload + 16 pad
 #ifndef GEMM_WGS
 #define GEMM_WGS 3                // workgroups per CU the tile kernel is compiled for (register budget 512 / GEMM_WGS per lane)
@@ -379,29 +380,34 @@ static __device__ __forceinline__ void q4k_sc_m(const uint32_t h1, const uint32_
 
 template <bool Q4K> struct kq_scale { typedef float type; };
 template <> struct kq_scale<false> { typedef uint16_t type; };
-template <int WT>
-__global__ __launch_bounds__(256, 2) void gemm_kq_kernel(const uint8_t *__restrict__ W, const uint8_t *__restrict__ xq, float *__restrict__ dst,
+// NI x NI MFMA tiles of 32 x 32 per wave: 2 = the 128 x 128 workgroup tile; 1 = a 64 x 64 tile for shapes that would give the
+// large tile too few workgroups to fill the part (waves 0-1 then move the weights, waves 2-3 the activations).
+template <int WT, int NI>
+__global__ __launch_bounds__(256, NI == 2 ? 2 : 3) void gemm_kq_kernel(const uint8_t *__restrict__ W, const uint8_t *__restrict__ xq, float *__restrict__ dst,
                                                          int M, int K, int T, int64_t dst_stride) {
     constexpr bool Q4K = (WT == SPY_HIP_Q4_K);
     constexpr int RAW = Q4K ? 12 : 18;
-    __shared__ __attribute__((aligned(16))) uint8_t sA[2][GEMM_TILE * GEMM_ROWB];
-    __shared__ __attribute__((aligned(16))) uint8_t sB[2][GEMM_TILE * GEMM_ROWB];
+    constexpr int TILE = 64 * NI, WT32 = 32 * NI;        // rows of the workgroup tile / of a wave's part of it
+    __shared__ __attribute__((aligned(16))) uint8_t sA[2][TILE * GEMM_ROWB];
+    __shared__ __attribute__((aligned(16))) uint8_t sB[2][TILE * GEMM_ROWB];
     using scale_t = typename kq_scale<Q4K>::type;
-    __shared__ __attribute__((aligned(16))) scale_t sAd[2][2][GEMM_TILE];    // Q4_K: d*sc (float)  Q6_K: d (fp16 bits)
-    __shared__ __attribute__((aligned(16))) int sAm[2][2][GEMM_TILE];        // Q4_K: bits of dmin*m Q6_K: sc_lo | sc_hi << 16
-    __shared__ __attribute__((aligned(16))) scale_t sBd[2][2][GEMM_TILE];    // dx (Q4_K: float, Q6_K: fp16 bits)
-    __shared__ __attribute__((aligned(16))) float sBs[2][2][GEMM_TILE];      // dx * sum(q_x)
+    __shared__ __attribute__((aligned(16))) scale_t sAd[2][2][TILE];    // Q4_K: d*sc (float)  Q6_K: d (fp16 bits)
+    __shared__ __attribute__((aligned(16))) int sAm[2][2][TILE];        // Q4_K: bits of dmin*m Q6_K: sc_lo | sc_hi << 16
+    __shared__ __attribute__((aligned(16))) scale_t sBd[2][2][TILE];    // dx (Q4_K: float, Q6_K: fp16 bits)
+    __shared__ __attribute__((aligned(16))) float sBs[2][2][TILE];      // dx * sum(q_x)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
-    const int m0 = blockIdx.x * GEMM_TILE, t0 = blockIdx.y * GEMM_TILE;
+    const int m0 = blockIdx.x * TILE, t0 = blockIdx.y * TILE;
     const int nstage = K / 64;
     const size_t RBw = (size_t)spy_row_size(WT, K), RBx = (size_t)(K / 32) * 34;
-    const int lrow = tid & 127, half = tid >> 7;
+    const int lrow = tid & (TILE - 1), half = NI == 2 ? tid >> 7 : (tid >> 6) & 1;
+    const bool doA = NI == 2 || tid < 128, doB = NI == 2 || tid >= 128;   // wave-uniform
     const uint8_t *gA = W + (size_t)min(m0 + lrow, M - 1) * RBw;
     const uint32_t *gB = (const uint32_t *)(xq + (size_t)min(t0 + lrow, T - 1) * RBx) + half * 8;
     uint32_t rawA[RAW], rawB[9];
     auto gload = [&](int s) {
         const int sbi = s >> 2, j = s & 3;
-        if constexpr (Q4K) {
+        if (!doA) {
+        } else if constexpr (Q4K) {
             const uint8_t *sb = gA + (size_t)sbi * 144;
             const uint4 hdr = *(const uint4 *)sb, q0 = *(const uint4 *)(sb + 16 + 32 * j), q1 = *(const uint4 *)(sb + 32 + 32 * j);
             rawA[0] = hdr.x; rawA[1] = hdr.y; rawA[2] = hdr.z; rawA[3] = hdr.w;
@@ -419,13 +425,16 @@ __global__ __launch_bounds__(256, 2) void gemm_kq_kernel(const uint8_t *__restri
             rawA[16] = *(const uint16_t *)(sb + 192 + 8 * n + 2 * m);
             rawA[17] = *(const uint16_t *)(sb + 208);
         }
+        if (doB) {
 #pragma unroll
-        for (int i = 0; i < 9; i++) rawB[i] = gB[(size_t)s * 17 + i];
+            for (int i = 0; i < 9; i++) rawB[i] = gB[(size_t)s * 17 + i];
+        }
     };
     auto unpack = [&](int b, int s) {
         const int j = s & 3;
         uint32_t q[8];
-        if constexpr (Q4K) {
+        if (!doA) {
+        } else if constexpr (Q4K) {
             int sc, mn;
             q4k_sc_m(rawA[1], rawA[2], rawA[3], 2 * j + half, sc, mn);
 #pragma unroll
@@ -443,8 +452,11 @@ __global__ __launch_bounds__(256, 2) void gemm_kq_kernel(const uint8_t *__restri
             sAd[b][half][lrow] = (uint16_t)(rawA[17] & 0xFFFFu);
             sAm[b][half][lrow] = (int)(uint16_t)(int16_t)(int8_t)(rawA[16] & 0xFFu) | ((int)(int8_t)((rawA[16] >> 8) & 0xFFu) << 16);
         }
-        uint4 *ra = (uint4 *)(sA[b] + lrow * GEMM_ROWB + half * 32);
-        ra[0] = make_uint4(q[0], q[1], q[2], q[3]); ra[1] = make_uint4(q[4], q[5], q[6], q[7]);
+        if (doA) {
+            uint4 *ra = (uint4 *)(sA[b] + lrow * GEMM_ROWB + half * 32);
+            ra[0] = make_uint4(q[0], q[1], q[2], q[3]); ra[1] = make_uint4(q[4], q[5], q[6], q[7]);
+        }
+        if (!doB) return;
         // activations: {d, qs[32]} (quant.h:139-142)
         const uint16_t dxh = (uint16_t)(half ? rawB[0] >> 16 : rawB[0] & 0xFFFFu);
         const float dx = h2f(dxh);
@@ -457,11 +469,11 @@ __global__ __launch_bounds__(256, 2) void gemm_kq_kernel(const uint8_t *__restri
         else sBd[b][half][lrow] = dxh;
     };
 
-    float acc[2][2][16];
+    float acc[NI][NI][16];
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < NI; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++)
+        for (int j = 0; j < NI; j++)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
@@ -474,19 +486,19 @@ __global__ __launch_bounds__(256, 2) void gemm_kq_kernel(const uint8_t *__restri
         gload(min(s + 1, nstage - 1));
 #pragma unroll 1
         for (int blk = 0; blk < 2; blk++) {
-            v4i fa[2], fb[2];
+            v4i fa[NI], fb[NI];
 #pragma unroll
-            for (int i = 0; i < 2; i++) {
-                fa[i] = *(const v4i *)(sA[b] + (wm * 64 + i * 32 + (lane & 31)) * GEMM_ROWB + blk * 32 + (lane >> 5) * 16);
-                fb[i] = *(const v4i *)(sB[b] + (wn * 64 + i * 32 + (lane & 31)) * GEMM_ROWB + blk * 32 + (lane >> 5) * 16);
+            for (int i = 0; i < NI; i++) {
+                fa[i] = *(const v4i *)(sA[b] + (wm * WT32 + i * 32 + (lane & 31)) * GEMM_ROWB + blk * 32 + (lane >> 5) * 16);
+                fb[i] = *(const v4i *)(sB[b] + (wn * WT32 + i * 32 + (lane & 31)) * GEMM_ROWB + blk * 32 + (lane >> 5) * 16);
             }
 #pragma unroll
-            for (int i = 0; i < 2; i++) {
+            for (int i = 0; i < NI; i++) {
                 int am[16];
                 if constexpr (!Q4K) {
 #pragma unroll
                     for (int g = 0; g < 4; g++) {
-                        const int4 u = *(const int4 *)&sAm[b][blk][wm * 64 + i * 32 + g * 8 + (lane >> 5) * 4];
+                        const int4 u = *(const int4 *)&sAm[b][blk][wm * WT32 + i * 32 + g * 8 + (lane >> 5) * 4];
                         am[4 * g] = u.x; am[4 * g + 1] = u.y; am[4 * g + 2] = u.z; am[4 * g + 3] = u.w;
                     }
                 }
@@ -494,12 +506,12 @@ __global__ __launch_bounds__(256, 2) void gemm_kq_kernel(const uint8_t *__restri
                     float dw[16];
 #pragma unroll
                     for (int g = 0; g < 4; g++) {
-                        const float4 v = *(const float4 *)&sAd[b][blk][wm * 64 + i * 32 + g * 8 + (lane >> 5) * 4];
+                        const float4 v = *(const float4 *)&sAd[b][blk][wm * WT32 + i * 32 + g * 8 + (lane >> 5) * 4];
                         dw[4 * g] = v.x; dw[4 * g + 1] = v.y; dw[4 * g + 2] = v.z; dw[4 * g + 3] = v.w;
                     }
 #pragma unroll
-                    for (int j = 0; j < 2; j++) {
-                        const float dx = sBd[b][blk][wn * 64 + j * 32 + (lane & 31)];
+                    for (int j = 0; j < NI; j++) {
+                        const float dx = sBd[b][blk][wn * WT32 + j * 32 + (lane & 31)];
                         v16i z = {0};
                         const v16i I = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], z, 0, 0, 0);
 #pragma unroll
@@ -507,10 +519,10 @@ __global__ __launch_bounds__(256, 2) void gemm_kq_kernel(const uint8_t *__restri
                     }
                 } else {
                     // d (fp16) x dx (fp16) for the whole tile from one fp16 MFMA: scales at k = 0, zeros elsewhere (exact in fp32)
-                    const v4h ha = __builtin_bit_cast(v4h, v2i{(int)sAd[b][blk][wm * 64 + i * 32 + (lane & 31)], 0});
+                    const v4h ha = __builtin_bit_cast(v4h, v2i{(int)sAd[b][blk][wm * WT32 + i * 32 + (lane & 31)], 0});
 #pragma unroll
-                    for (int j = 0; j < 2; j++) {
-                        const v4h hb = __builtin_bit_cast(v4h, v2i{(int)sBd[b][blk][wn * 64 + j * 32 + (lane & 31)] & k0mask, 0});
+                    for (int j = 0; j < NI; j++) {
+                        const v4h hb = __builtin_bit_cast(v4h, v2i{(int)sBd[b][blk][wn * WT32 + j * 32 + (lane & 31)] & k0mask, 0});
                         v16i z = {0};
                         v16f zf = {0};
                         const v4i zero4 = {0, 0, 0, 0};
@@ -534,11 +546,11 @@ __global__ __launch_bounds__(256, 2) void gemm_kq_kernel(const uint8_t *__restri
             // product over the block index: one fp32 MFMA per tile (k = block of the pair, carried by the lane half)
             // adds both to the accumulators instead of 32 fmas per lane
 #pragma unroll
-            for (int i = 0; i < 2; i++) {
-                const float a2 = -__int_as_float(sAm[b][lane >> 5][wm * 64 + i * 32 + (lane & 31)]);
+            for (int i = 0; i < NI; i++) {
+                const float a2 = -__int_as_float(sAm[b][lane >> 5][wm * WT32 + i * 32 + (lane & 31)]);
 #pragma unroll
-                for (int j = 0; j < 2; j++) {
-                    const float b2 = sBs[b][lane >> 5][wn * 64 + j * 32 + (lane & 31)];
+                for (int j = 0; j < NI; j++) {
+                    const float b2 = sBs[b][lane >> 5][wn * WT32 + j * 32 + (lane & 31)];
                     v16f c;
 #pragma unroll
                     for (int r = 0; r < 16; r++) c[r] = acc[i][j][r];
@@ -552,14 +564,14 @@ __global__ __launch_bounds__(256, 2) void gemm_kq_kernel(const uint8_t *__restri
         __syncthreads();
     }
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < NI; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++) {
-            const int t = t0 + wn * 64 + j * 32 + (lane & 31);
+        for (int j = 0; j < NI; j++) {
+            const int t = t0 + wn * WT32 + j * 32 + (lane & 31);
             if (t < T) {
 #pragma unroll
                 for (int g = 0; g < 4; g++) {
-                    const int m = m0 + wm * 64 + i * 32 + g * 8 + (lane >> 5) * 4;
+                    const int m = m0 + wm * WT32 + i * 32 + g * 8 + (lane >> 5) * 4;
                     float *o = dst + (size_t)t * dst_stride + m;
                     if (m + 3 < M && (((uintptr_t)o) & 15) == 0) *(float4 *)o = make_float4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
                     else {
@@ -578,7 +590,7 @@ extern "C" int spy_hip_gemm_q8_0act(void *stream, int wtype, const void *w_dev, 
     SPY_CHECK_ARG((M + GEMM_TILE - 1) / GEMM_TILE <= 0x7fffffff && (T + GEMM_TILE - 1) / GEMM_TILE <= 65535);
     const dim3 grid((unsigned)((M + GEMM_TILE - 1) / GEMM_TILE), (unsigned)((T + GEMM_TILE - 1) / GEMM_TILE));
     hipStream_t st = (hipStream_t)stream;
-    const char *force = getenv("SPY_HIP_GEMM");           // "tile" / "skinny": measurement switch
+    const char *force = getenv("SPY_HIP_GEMM");           // "tile" / "skinny" / "tile64": measurement switch
     const bool skinny = K % 256 == 0 && M * (K / 32) * 34 < (int64_t)1 << 31 && T * (K / 32) * 34 < (int64_t)1 << 31 && (force ? !strcmp(force, "skinny") : (T <= 64 || (int64_t)grid.x * grid.y <= GEMM_SKINNY_MAX_TILES));
     if (skinny && wtype == SPY_HIP_Q4_0) return launch_gemm_skinny<SPY_HIP_Q4_0>(st, w_dev, xq_dev, dst_dev, M, K, T, dst_stride);
     if (skinny && wtype == SPY_HIP_Q8_0) return launch_gemm_skinny<SPY_HIP_Q8_0>(st, w_dev, xq_dev, dst_dev, M, K, T, dst_stride);
@@ -588,9 +600,20 @@ extern "C" int spy_hip_gemm_q8_0act(void *stream, int wtype, const void *w_dev, 
         return spy_hip_gemv_q8_0act(stream, wtype, w_dev, xq_dev, dst_dev, nullptr, M, K, T, dst_stride);
     if (wtype == SPY_HIP_Q4_0) gemm_q8act_kernel<SPY_HIP_Q4_0><<<grid, dim3(256), 0, st>>>((const uint8_t *)w_dev, (const uint8_t *)xq_dev, dst_dev, (int)M, (int)K, (int)T, dst_stride, nullptr, nullptr);
     else if (wtype == SPY_HIP_Q8_0) gemm_q8act_kernel<SPY_HIP_Q8_0><<<grid, dim3(256), 0, st>>>((const uint8_t *)w_dev, (const uint8_t *)xq_dev, dst_dev, (int)M, (int)K, (int)T, dst_stride, nullptr, nullptr);
-    else if (wtype == SPY_HIP_Q4_K) gemm_kq_kernel<SPY_HIP_Q4_K><<<grid, dim3(256), 0, st>>>((const uint8_t *)w_dev, (const uint8_t *)xq_dev, dst_dev, (int)M, (int)K, (int)T, dst_stride);
-    else if (wtype == SPY_HIP_Q6_K) gemm_kq_kernel<SPY_HIP_Q6_K><<<grid, dim3(256), 0, st>>>((const uint8_t *)w_dev, (const uint8_t *)xq_dev, dst_dev, (int)M, (int)K, (int)T, dst_stride);
-    else return SPY_HIP_EUNSUPPORTED;
+    else if (wtype == SPY_HIP_Q4_K || wtype == SPY_HIP_Q6_K) {
+        // 64 x 64 tiles where the 128 x 128 tiling gives too few workgroups to fill the part: 1.8-2.9 x faster up to 512 activation
+        // rows of the 7B shapes, equal where its own workgroups stop being resident all at once, 30 % slower beyond
+        const dim3 grid64((unsigned)((M + 63) / 64), (unsigned)((T + 63) / 64));
+        const bool small = force ? !strcmp(force, "tile64") : (int64_t)grid64.x * grid64.y <= GEMM_KQ_SMALL_MAX_TILES;
+        SPY_CHECK_ARG(!small || (T + 63) / 64 <= 65535);
+        if (wtype == SPY_HIP_Q4_K) {
+            if (small) gemm_kq_kernel<SPY_HIP_Q4_K, 1><<<grid64, dim3(256), 0, st>>>((const uint8_t *)w_dev, (const uint8_t *)xq_dev, dst_dev, (int)M, (int)K, (int)T, dst_stride);
+            else gemm_kq_kernel<SPY_HIP_Q4_K, 2><<<grid, dim3(256), 0, st>>>((const uint8_t *)w_dev, (const uint8_t *)xq_dev, dst_dev, (int)M, (int)K, (int)T, dst_stride);
+        } else {
+            if (small) gemm_kq_kernel<SPY_HIP_Q6_K, 1><<<grid64, dim3(256), 0, st>>>((const uint8_t *)w_dev, (const uint8_t *)xq_dev, dst_dev, (int)M, (int)K, (int)T, dst_stride);
+            else gemm_kq_kernel<SPY_HIP_Q6_K, 2><<<grid, dim3(256), 0, st>>>((const uint8_t *)w_dev, (const uint8_t *)xq_dev, dst_dev, (int)M, (int)K, (int)T, dst_stride);
+        }
+    } else return SPY_HIP_EUNSUPPORTED;
     return SPY_LAUNCH_RC();
 }
 

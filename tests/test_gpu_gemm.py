@@ -34,13 +34,17 @@ def test_gemm_q8_0act_matches_oracle(hip, oracle, wtype, M, K, T):
     assert_close(dout.download(np.float32).reshape(T, M), want, "gemm type %d %dx%d T=%d" % (wtype, M, K, T))
 
 
+@pytest.mark.parametrize("tiling", ["tile", "tile64", None])
 @pytest.mark.parametrize("wtype", [O.Q4_K, O.Q6_K])
 @pytest.mark.parametrize("M,K,T", [(128, 4096, 128), (256, 256, 16), (200, 11008, 77), (130, 512, 129), (4096, 4096, 256)])
-def test_gemm_k_quants_match_oracle(hip, oracle, wtype, M, K, T):
+def test_gemm_k_quants_match_oracle(hip, oracle, wtype, M, K, T, tiling, monkeypatch):
     """Super-block weights: every sub-block scale / minimum (Q4_K) and both 16-element groups of a
     32-element MFMA block (Q6_K) take part; weights with offsets and outliers so that minima and the
-    6-bit scale fields above index 3 are not trivial."""
+    6-bit scale fields above index 3 are not trivial.  Each shape with the 128 x 128 tiling, the 64 x 64
+    tiling and whatever the library picks for it."""
     from tests.gpu_util import dev, dev_empty, call, assert_close
+    if tiling: monkeypatch.setenv("SPY_HIP_GEMM", tiling)
+    else: monkeypatch.delenv("SPY_HIP_GEMM", raising=False)
     rng = np.random.default_rng(wtype * 977 + M + K + T)
     wf = (rng.standard_normal((M, K)) * 0.02).astype(np.float32)
     wf += (rng.standard_normal((M, K // 32, 1)) * 0.03).astype(np.float32).repeat(32, 2).reshape(M, K)
