@@ -37,6 +37,8 @@ extern "C" int spy_hip_llama_destroy(spy_hip_llama *m) {
     if (!m) return 0;
     (void)hipDeviceSynchronize();
     if (m->graph_exec) (void)hipGraphExecDestroy(m->graph_exec);
+    if (m->graph_n_exec) (void)hipGraphExecDestroy(m->graph_n_exec);
+    if (m->graph_n) (void)hipGraphDestroy(m->graph_n);
     if (m->graph) (void)hipGraphDestroy(m->graph);
     if (m->own_stream) (void)hipStreamDestroy(m->own_stream);
     if (m->ev0) (void)hipEventDestroy(m->ev0);
@@ -497,6 +499,9 @@ extern "C" int spy_hip_llama_forward_last(spy_hip_llama *m, void *stream, const 
     return forward_any(m, stream, tokens_host, n_token, n_past, logits_last_host, true);
 }
 
+#ifndef SPY_GRAPH_STEPS
+#define SPY_GRAPH_STEPS 8   // passes per replayed graph of the greedy loop (the remainder runs the one-pass graph)
+#endif
 extern "C" int spy_hip_llama_decode_greedy(spy_hip_llama *m, void *stream, int32_t first_token, int32_t n_past, int32_t n_steps,
                                            int32_t *tokens_host, int32_t use_graph) {
     SPY_CHECK_ARG(m && n_steps > 0 && n_past >= 0 && first_token >= 0 && first_token < m->desc.n_vocab);
@@ -516,12 +521,24 @@ extern "C" int spy_hip_llama_decode_greedy(spy_hip_llama *m, void *stream, int32
         if (e != hipSuccess) return (int)e;
         HIP_TRY(hipGraphInstantiate(&m->graph_exec, m->graph, nullptr, nullptr, 0));
         m->graph_stream = st;
+        // several passes as one graph: nothing in a pass depends on the host (token, position and step count live on the device)
+        if (m->graph_n_exec) { (void)hipGraphExecDestroy(m->graph_n_exec); m->graph_n_exec = nullptr; }
+        if (m->graph_n) { (void)hipGraphDestroy(m->graph_n); m->graph_n = nullptr; }
+        HIP_TRY(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
+        int rcn = 0;
+        for (int i = 0; i < SPY_GRAPH_STEPS && !rcn; i++) rcn = enqueue_pass_any(m, st, PASS_GREEDY);
+        e = hipStreamEndCapture(st, &m->graph_n);
+        if (rcn) return rcn;
+        if (e != hipSuccess) return (int)e;
+        HIP_TRY(hipGraphInstantiate(&m->graph_n_exec, m->graph_n, nullptr, nullptr, 0));
     }
     if (!m->mega) RC_TRY(enqueue_embed(m, st));              // embedding of the first token; every step prepares the next one's
     HIP_TRY(hipEventRecord(m->ev0, st));
-    for (int i = 0; i < n_steps; i++) {
+    for (int i = 0; i < n_steps;) {
+        if (use_graph && n_steps - i >= SPY_GRAPH_STEPS) { HIP_TRY(hipGraphLaunch(m->graph_n_exec, st)); i += SPY_GRAPH_STEPS; continue; }
         if (use_graph) HIP_TRY(hipGraphLaunch(m->graph_exec, st));
         else RC_TRY(enqueue_pass_any(m, st, PASS_GREEDY));
+        i++;
     }
     HIP_TRY(hipEventRecord(m->ev1, st));
     HIP_TRY(hipEventSynchronize(m->ev1));

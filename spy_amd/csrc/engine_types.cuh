@@ -32,6 +32,7 @@ struct spy_hip_llama {
     uint8_t *ops_buf = nullptr; size_t ops_bytes = 0;
     // graph of one single-token pass
     hipGraph_t graph = nullptr; hipGraphExec_t graph_exec = nullptr; hipStream_t graph_stream = nullptr;
+    hipGraph_t graph_n = nullptr; hipGraphExec_t graph_n_exec = nullptr;   // SPY_GRAPH_STEPS passes in one graph
     hipStream_t own_stream = nullptr;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     double timed_ms = 0.0; int timed_pass = 0;
