@@ -59,6 +59,31 @@ def test_gemm_k_quants_match_oracle(hip, oracle, wtype, M, K, T, tiling, monkeyp
     assert_close(dout.download(np.float32).reshape(T, M), want, "gemm type %d %dx%d T=%d" % (wtype, M, K, T))
 
 
+@pytest.mark.parametrize("wtype", [O.Q4_0, O.Q8_0, O.Q4_K, O.Q6_K])
+def test_gemm_random_shapes_strided_destination_and_untouched_padding(hip, oracle, wtype):
+    """Seeded ragged shapes on both sides of every kernel choice (row kernels, 32-row kernel, 64 x 64 and 128 x 128 tiles),
+    written through a destination stride larger than M: the results equal the oracle's and no byte outside the T x M
+    region is written (columns M .. stride-1 of every row, and a guard row behind the last one)."""
+    from tests.gpu_util import dev, dev_empty, call, assert_close
+    rng = np.random.default_rng(4000 + wtype)
+    kq = wtype in (O.Q4_K, O.Q6_K)
+    for case in range(6):
+        M = int(rng.integers(1, 400))
+        K = int(rng.integers(1, 5)) * 256 if (kq or case % 2 == 0) else int(rng.integers(1, 12)) * 64
+        T = int(rng.choice([1, 2, 15, 16, 17, 31, 33, 63, 64, 65, 127, 129, 200, 257]))
+        pad = int(rng.integers(1, 9))
+        stride = M + pad
+        w = O.quantize(oracle, (rng.standard_normal((M, K)) * 0.05).astype(np.float32), wtype)
+        x = (rng.standard_normal((T, K)) * rng.choice([0.1, 1.0, 10.0])).astype(np.float32)
+        want = O.matmul(oracle, w, wtype, M, K, x, nthread=8)
+        xq = O.quantize(oracle, x, O.Q8_0)
+        dw, dxq, dout = dev(w), dev(xq), dev_empty((T + 1) * stride * 4, 0xFF)
+        call(hip.load().spy_hip_gemm_q8_0act, None, wtype, dw.ptr, dxq.ptr, dout.ptr, M, K, T, stride)
+        raw = dout.download(np.uint32).reshape(T + 1, stride)
+        assert np.all(raw[:T, M:] == 0xFFFFFFFF) and np.all(raw[T] == 0xFFFFFFFF), "type %d %dx%d T=%d stride %d: wrote outside the result" % (wtype, M, K, T, stride)
+        assert_close(raw[:T, :M].view(np.float32), want, "gemm type %d %dx%d T=%d stride %d" % (wtype, M, K, T, stride))
+
+
 def test_gemm_integer_scales_is_exact(hip, oracle):
     """With power-of-two scales and small integers every product and sum is exact in fp32: the GEMM
     must then equal the integer matrix product bit for bit (pins the MFMA operand / result layout)."""
