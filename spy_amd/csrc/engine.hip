@@ -511,7 +511,7 @@ extern "C" int spy_hip_llama_decode_greedy(spy_hip_llama *m, void *stream, int32
     dev_state h = {first_token, n_past, 0, 0};
     HIP_TRY(hipMemcpyAsync(m->st, &h, sizeof(h), hipMemcpyHostToDevice, st));
     HIP_TRY(hipStreamSynchronize(st));
-    if (use_graph && (!m->graph_exec || m->graph_stream != st)) {
+    if (use_graph && (!m->graph_exec || !m->graph_n_exec || m->graph_stream != st)) {
         if (m->graph_exec) { (void)hipGraphExecDestroy(m->graph_exec); m->graph_exec = nullptr; }
         if (m->graph) { (void)hipGraphDestroy(m->graph); m->graph = nullptr; }
         HIP_TRY(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
