@@ -71,7 +71,8 @@ static int launch_wave(spy_hip_llama *m, hipStream_t st, const fused_args &a) {
 // with 8 the kernel spills a dozen registers and measured 24.3 instead of 21.5 us (Q6_K), 27.3 instead of 20.8 us (Q8_0).
 // gate|up: 3 pairs per wave for every type = 230 workgroups for 11008 pairs, one round over the compute units (2 pairs gave
 // 344 workgroups, a second round a third full: Q8_0 22.1 -> 18.7 us).  Dealing the 11008 pairs out over 256 workgroups
-// (2 or 3 per wave, the third either re-reading a row or skipped) was slower: 682 -> 664 / 620 tok/s.
+// (2 or 3 per wave; the third re-reading a row, skipped, or left out by a second instantiation of the loop) was slower: 682 -> 664 / 620 / 669 tok/s.
+// The 230 workgroups already draw what the memory system delivers.
 template <int WT> struct wave_rows {
     static constexpr int HEAD = (WT == SPY_HIP_Q4_0 || WT == SPY_HIP_Q4_K) ? 8 : 4;
     static constexpr int GATEUP = 3;
