@@ -107,6 +107,16 @@ int spy_hip_op_contiguous(void *stream, const spy_hip_tensor *src, const spy_hip
  * returned by spy_hip_take_error (the reference asserts, view.cpp:61). */
 int spy_hip_op_get_row(void *stream, const spy_hip_tensor *table, const spy_hip_tensor *ids, const spy_hip_tensor *dst);
 int spy_hip_take_error(int *flag);   /* reads and clears the device error flag (synchronises) */
+/* Exact-order mode of the spy_hip_op_* entry points (on != 0; returns the previous setting; the environment
+ * variable SPY_HIP_EXACT=1 is its initial value).  MatMul, NormRMS, Softmax, Silu and Rope then add their terms
+ * in the order of the host backend's own loops -- the 8-lane accumulators and hsum_float_8 of Dot<Q4_0,Q8_0>,
+ * Dot<Q8_0,Q8_0> and Dot<FP16,FP16> (vec_dot.h:42-146, vec_util.h:75-81), libstdc++'s four-way std::reduce in
+ * NormRMS and Softmax (non-linear.cpp:129-223) -- and take exp / silu from tables and the Rope angles from the
+ * host's libm (lookup_table_impl/non-linear.h:39-47,131-139, non-linear.cpp:270-371), so that every operator
+ * output equals the host backend's bit for bit.  A checking mode, far slower than the default kernels; Rope
+ * synchronises the stream.  The fused token loop (spy_hip_llama_*) only follows it where it runs operator by
+ * operator (prompt passes below 16 tokens). */
+int spy_hip_set_exact_order(int on);
 /* Greedy sampling -- SamplerImpl<Greedy>::sample (model/include/llm/sampler/greedy.h:20-25):
  * index of the FIRST maximum of n logits, written to *out_index (device int32) */
 int spy_hip_argmax(void *stream, const float *logits, int64_t n, int32_t *out_index);

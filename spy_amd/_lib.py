@@ -87,6 +87,7 @@ SIGNATURES = {
     "spy_hip_op_contiguous": (_i32, [_vp, _TP, _TP]),
     "spy_hip_op_get_row": (_i32, [_vp, _TP, _TP, _TP]),
     "spy_hip_take_error": (_i32, [C.POINTER(_i32)]),
+    "spy_hip_set_exact_order": (_i32, [_i32]),
     "spy_hip_argmax": (_i32, [_vp, _vp, _i64, _vp]),
     "spy_hip_quantize_q8_0": (_i32, [_vp, _vp, _i64, _vp, _i64, _i64]),
     "spy_hip_quantize_f16": (_i32, [_vp, _vp, _i64, _vp, _i64, _i64]),

@@ -1,0 +1,444 @@
+// Exact-order forms of the operators whose fp32 results depend on the ORDER of their additions or on
+// the host's libm: the quantized and fp16 dots of MatMul, NormRMS, Softmax, Silu and Rope.
+//
+// The fast kernels add a row's terms in whatever order suits 64 lanes; Spy's host backend adds them in
+// the order of its 8-lane AVX accumulators and of libstdc++'s four-way reduce, and looks exp / silu up
+// in tables that glibc filled.  The results agree to about 1e-7, but every MatMul re-quantizes its
+// activations to Q8_0 (mat.cpp:95-128) and the softmax rounds its exp argument to fp16
+// (non-linear.cpp:170), so a last-ulp difference moves a rounding now and then and the greedy tokens of
+// a model with near-tied logits can differ.  With spy_hip_set_exact_order(1) (or SPY_HIP_EXACT=1) the
+// spy_hip_op_* entry points launch the kernels below instead: one thread (or one serial lane) walks
+// each sum in the host backend's order, the tables and the rotation angles come from the host's libm,
+// and the outputs are the host backend's bit for bit.  This is the checking mode of the operator path,
+// roughly 30x slower than the fast kernels; the fused token loop (spy_hip_llama_*) is not affected.
+#include "common.cuh"
+
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <vector>
+
+namespace {
+
+struct xdesc {
+    uint8_t *p;
+    int64_t ne[4], nb[4];
+};
+xdesc mkx(const spy_hip_tensor *t) {
+    xdesc d;
+    d.p = (uint8_t *)t->data;
+    for (int i = 0; i < 4; i++) { d.ne[i] = t->ne[i]; d.nb[i] = t->nb[i]; }
+    return d;
+}
+__device__ __forceinline__ uint8_t *xat(const xdesc &t, int64_t i0, int64_t i1, int64_t i2, int64_t i3) {
+    return t.p + i0 * t.nb[0] + i1 * t.nb[1] + i2 * t.nb[2] + i3 * t.nb[3];
+}
+
+int g_exact = -1;          // -1: not decided yet (environment), 0 / 1
+float *g_lut = nullptr;    // device: exp table [65536], then silu table [65536]
+float *g_rope = nullptr;   // device: cos / sin pairs per token of the current Rope call
+size_t g_rope_cap = 0;
+
+// IEEE binary16 -> binary32 on the host
+float host_h2f(uint16_t h) {
+    const uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    uint32_t exp = (h >> 10) & 0x1F, mant = h & 0x3FFu, x;
+    if (exp == 0) {
+        if (mant == 0) x = sign;
+        else {
+            int e = -1;
+            do { mant <<= 1; e++; } while (!(mant & 0x400u));
+            x = sign | ((uint32_t)(112 - e) << 23) | ((mant & 0x3FFu) << 13);
+        }
+    } else if (exp == 31) x = sign | 0x7F800000u | (mant << 13);
+    else x = sign | ((exp + 112) << 23) | (mant << 13);
+    float f;
+    memcpy(&f, &x, 4);
+    return f;
+}
+
+// The reference's tables (lookup_table_impl/non-linear.h:39-47,131-139): entry k holds the function of
+// float(half k), evaluated by the host's libm in fp32; the loop stops before k = 0xFFFF, which stays 0.
+int ensure_luts() {
+    if (g_lut) return 0;
+    std::vector<float> h(2 * 65536, 0.0f);
+    for (uint32_t k = 0; k < 0xFFFFu; k++) {
+        const float v = host_h2f((uint16_t)k);
+        h[k] = expf(v);
+        h[65536 + k] = v / (1.0f + expf(-v));
+    }
+    float *d = nullptr;
+    hipError_t e = hipMalloc((void **)&d, h.size() * sizeof(float));
+    if (e != hipSuccess) return (int)e;
+    e = hipMemcpy(d, h.data(), h.size() * sizeof(float), hipMemcpyHostToDevice);
+    if (e != hipSuccess) { (void)hipFree(d); return (int)e; }
+    g_lut = d;
+    return 0;
+}
+
+// conversion.h:39-41: the fp16 -> fp32 table has no entry for 0xFFFF either
+__device__ __forceinline__ float h2f_tab(uint16_t h) { return h == 0xFFFFu ? 0.0f : h2f(h); }
+
+// libstdc++'s std::reduce / std::transform_reduce over a random-access range: groups of four as
+// init = init + ((a0 + a1) + (a2 + a3)), then the remaining elements one by one.  The 256 threads of the
+// workgroup prepare the group sums of up to 4096 elements in LDS, thread 0 adds them in order.
+template <bool SQUARE>
+__device__ float reduce4_block(const float *p, int64_t n, float *s_grp, float *s_out) {
+    const int64_t ngrp = n / 4;
+    float init = 0.0f;
+    for (int64_t g0 = 0; g0 < ngrp; g0 += 1024) {
+        const int cnt = (int)min((int64_t)1024, ngrp - g0);
+        for (int g = threadIdx.x; g < cnt; g += 256) {
+            const float *q = p + (g0 + g) * 4;
+            float a0 = q[0], a1 = q[1], a2 = q[2], a3 = q[3];
+            if (SQUARE) { a0 = a0 * a0; a1 = a1 * a1; a2 = a2 * a2; a3 = a3 * a3; }
+            const float v1 = a0 + a1, v2 = a2 + a3;
+            s_grp[g] = v1 + v2;
+        }
+        __syncthreads();
+        if (threadIdx.x == 0)
+            for (int g = 0; g < cnt; g++) init = init + s_grp[g];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        for (int64_t i = ngrp * 4; i < n; i++) { const float a = p[i]; init = init + (SQUARE ? a * a : a); }
+        *s_out = init;
+    }
+    __syncthreads();
+    return *s_out;
+}
+
+// NormRMS (non-linear.cpp:194-223): one workgroup per row
+__global__ __launch_bounds__(256) void exact_norm_rms_kernel(xdesc x, xdesc y, float eps) {
+    __shared__ float s_grp[1024];
+    __shared__ float s_out;
+    const int64_t r = blockIdx.x;
+    const int64_t ne0 = y.ne[0], ne1 = y.ne[1], ne2 = y.ne[2];
+    const int64_t i3 = r / (ne1 * ne2), i2 = r % (ne1 * ne2) / ne1, i1 = r % ne1;
+    const float *s = (const float *)xat(x, 0, i1, i2, i3);
+    float *d = (float *)xat(y, 0, i1, i2, i3);
+    const float sum = reduce4_block<true>(s, ne0, s_grp, &s_out);
+    const float mean = sum / (float)ne0;
+    const float scale = 1.0f / sqrtf(mean + eps);
+    for (int64_t i = threadIdx.x; i < ne0; i += 256) d[i] = s[i] * scale;
+}
+
+// Silu (non-linear.cpp:11-14,57-77): table look-up on fp16(x)
+__global__ __launch_bounds__(256) void exact_silu_kernel(xdesc x, xdesc d, const float *__restrict__ lut, int64_t total) {
+    const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (g >= total) return;
+    const int64_t i0 = g % x.ne[0], r = g / x.ne[0];
+    const int64_t i1 = r % x.ne[1], i2 = r / x.ne[1] % x.ne[2], i3 = r / (x.ne[1] * x.ne[2]);
+    *(float *)xat(d, i0, i1, i2, i3) = lut[65536 + f2h(*(const float *)xat(x, i0, i1, i2, i3))];
+}
+
+// Softmax (non-linear.cpp:86-180), the row kept in dst between the steps as the reference keeps it
+__global__ __launch_bounds__(256) void exact_softmax_kernel(xdesc x, xdesc mask, bool has_mask, xdesc y, float scale, const float *__restrict__ lut) {
+    __shared__ float s_grp[1024];
+    __shared__ float s_out;
+    __shared__ float s_part[4];
+    const int64_t r = blockIdx.x;
+    const int64_t ne0 = y.ne[0], ne1 = y.ne[1], ne2 = y.ne[2];
+    const int64_t i3 = r / (ne1 * ne2), i2 = r % (ne1 * ne2) / ne1, i1 = r % ne1;
+    const float *s = (const float *)xat(x, 0, i1, i2, i3);
+    const float *mk_ = has_mask ? (const float *)xat(mask, 0, i1, 0, 0) : nullptr;
+    float *d = (float *)xat(y, 0, i1, i2, i3);
+    float mx = -INFINITY;
+    for (int64_t i = threadIdx.x; i < ne0; i += 256) {
+        float t;
+        if (has_mask) { t = s[i] + mk_[i]; t = t * scale; }
+        else t = s[i] * scale;
+        d[i] = t;
+        mx = fmaxf(mx, t);
+    }
+    mx = wave_max(mx);
+    if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(s_part[0], s_part[1]), fmaxf(s_part[2], s_part[3]));
+    for (int64_t i = threadIdx.x; i < ne0; i += 256) {
+        const float t = d[i] - mx;
+        d[i] = (has_mask && mk_[i] == -INFINITY) ? 0.0f : lut[f2h(t)];
+    }
+    __syncthreads();
+    const float sum = reduce4_block<false>(d, ne0, s_grp, &s_out);
+    const float inv = 1.0f / sum;
+    for (int64_t i = threadIdx.x; i < ne0; i += 256) d[i] *= inv;
+}
+
+// Rope (non-linear.cpp:270-371), default branch; tab = cos, sin per pair and token, from the host
+__global__ __launch_bounds__(64) void exact_rope_kernel(xdesc x, xdesc y, const float *__restrict__ tab) {
+    const int64_t i1 = blockIdx.x, i2 = blockIdx.y, i3 = blockIdx.z;
+    const int64_t ne0 = y.ne[0];
+    for (int64_t i0 = 2 * threadIdx.x; i0 < ne0; i0 += 128) {
+        const float c = tab[i2 * ne0 + i0], s = tab[i2 * ne0 + i0 + 1];
+        const float *sp = (const float *)xat(x, i0, i1, i2, i3);
+        float *dp = (float *)xat(y, i0, i1, i2, i3);
+        const float x0 = sp[0], x1 = sp[1];
+        const float a = x0 * c, b = x1 * s, e = x0 * s, f = x1 * c;
+        dp[0] = a - b;
+        dp[1] = e + f;
+    }
+}
+
+// mul_sum_i8_pairs (vec_util.h:101-110) on four int8 pairs: |x| as uint8 times y with the sign of x,
+// adjacent products added with int16 saturation (maddubs), the two sums added as int32 (madd with ones)
+__device__ __forceinline__ int32_t mul_sum4(const int8_t *x, const int8_t *y) {
+    int32_t pair[2];
+#pragma unroll
+    for (int p = 0; p < 2; p++) {
+        int32_t s = 0;
+#pragma unroll
+        for (int k = 0; k < 2; k++) {
+            const int8_t xv = x[2 * p + k], yv = y[2 * p + k];
+            const int32_t ax = (uint8_t)(xv < 0 ? -xv : xv);
+            const int32_t sy = xv < 0 ? (int32_t)(int8_t)(-yv) : (xv == 0 ? 0 : (int32_t)yv);
+            s += ax * sy;
+        }
+        pair[p] = s < -32768 ? -32768 : (s > 32767 ? 32767 : s);
+    }
+    return pair[0] + pair[1];
+}
+
+// hsum_float_8 (vec_util.h:75-81)
+__device__ __forceinline__ float hsum8(const float *a) {
+    const float r0 = a[4] + a[0], r1 = a[5] + a[1], r2 = a[6] + a[2], r3 = a[7] + a[3];
+    const float s0 = r0 + r2, s1 = r1 + r3;
+    return s0 + s1;
+}
+
+// Dot<Q4_0,Q8_0>::exec (vec_dot.h:42-86): accumulators 4..7 take the low-nibble half (elements 0..15),
+// 0..3 the high-nibble half, four products each; acc = fma(d_w * d_x, float(part), acc) block after block
+__device__ float dot_q4_0(const uint8_t *wv, const uint8_t *xv, int64_t n) {
+    const blk_q4_0 *w = (const blk_q4_0 *)wv;
+    const blk_q8_0 *x = (const blk_q8_0 *)xv;
+    float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int64_t i = 0; i < n / 32; i++) {
+        const float d = h2f_tab(w[i].d) * h2f_tab(x[i].d);
+        int8_t lo[16], hi[16], q[32];
+#pragma unroll
+        for (int j = 0; j < 16; j++) { const uint8_t b = w[i].qs[j]; lo[j] = (int8_t)((b & 0x0F) - 8); hi[j] = (int8_t)((b >> 4) - 8); }
+#pragma unroll
+        for (int j = 0; j < 32; j++) q[j] = x[i].qs[j];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            acc[4 + k] = fmaf(d, (float)mul_sum4(lo + 4 * k, q + 4 * k), acc[4 + k]);
+            acc[k] = fmaf(d, (float)mul_sum4(hi + 4 * k, q + 16 + 4 * k), acc[k]);
+        }
+    }
+    return hsum8(acc);
+}
+
+// Dot<Q8_0,Q8_0>::exec (vec_dot.h:88-115): accumulator l takes elements 4l..4l+3
+__device__ float dot_q8_0(const uint8_t *wv, const uint8_t *xv, int64_t n) {
+    const blk_q8_0 *w = (const blk_q8_0 *)wv, *x = (const blk_q8_0 *)xv;
+    float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int64_t i = 0; i < n / 32; i++) {
+        const float d = h2f_tab(w[i].d) * h2f_tab(x[i].d);
+        int8_t a[32], b[32];
+#pragma unroll
+        for (int j = 0; j < 32; j++) { a[j] = w[i].qs[j]; b[j] = x[i].qs[j]; }
+#pragma unroll
+        for (int l = 0; l < 8; l++) acc[l] = fmaf(d, (float)mul_sum4(a + 4 * l, b + 4 * l), acc[l]);
+    }
+    return hsum8(acc);
+}
+
+// Dot<FP16,FP16>::exec (vec_dot.h:117-146): four 8-lane fma accumulators over chunks of 32 while
+// i + 32 < n, FP16::block_reduce (vec_util.h:61-71), the last 1..32 elements as a scalar sum of products
+// through the conversion table, result = tail + simd
+__device__ float dot_f16(const uint8_t *av, const uint8_t *bv, int64_t n) {
+    const uint16_t *a = (const uint16_t *)av, *b = (const uint16_t *)bv;
+    float sum[32];
+#pragma unroll
+    for (int l = 0; l < 32; l++) sum[l] = 0.0f;
+    int64_t i = 0;
+    for (; i + 32 < n; i += 32) {
+#pragma unroll
+        for (int l = 0; l < 32; l++) sum[l] = fmaf(h2f(a[i + l]), h2f(b[i + l]), sum[l]);
+    }
+#pragma unroll
+    for (int l = 0; l < 8; l++) { sum[l] += sum[16 + l]; sum[8 + l] += sum[24 + l]; }
+#pragma unroll
+    for (int l = 0; l < 8; l++) sum[l] += sum[8 + l];
+    const float t0 = sum[0] + sum[4], t1 = sum[1] + sum[5], t2 = sum[2] + sum[6], t3 = sum[3] + sum[7];
+    const float u0 = t0 + t1, u1 = t2 + t3;
+    const float simd = u0 + u1;
+    float tail = 0.0f;
+    for (; i < n; i++) { const float pr = h2f_tab(a[i]) * h2f_tab(b[i]); tail += pr; }
+    return tail + simd;
+}
+
+// K-quant rows against Q8_0 activations.  The reference has no K-quant arithmetic; the order is the one
+// this project defines: one accumulator, sub-block after sub-block.
+__device__ float dot_q4_k(const uint8_t *wv, const uint8_t *xv, int64_t n) {
+    const blk_q4_k *w = (const blk_q4_k *)wv;
+    const blk_q8_0 *x = (const blk_q8_0 *)xv;
+    float acc = 0.0f;
+    for (int64_t b = 0; b < n / 256; b++) {
+        const float d = h2f_tab(w[b].d), dmin = h2f_tab(w[b].dmin);
+        const uint8_t *s = w[b].scales;
+        for (int j = 0; j < 8; j++) {
+            int32_t sc, m;
+            if (j < 4) { sc = s[j] & 63; m = s[j + 4] & 63; }
+            else { sc = (s[j + 4] & 0x0F) | ((s[j - 4] >> 6) << 4); m = (s[j + 4] >> 4) | ((s[j] >> 6) << 4); }
+            const blk_q8_0 *xb = &x[b * 8 + j];
+            int32_t isum = 0, bsum = 0;
+            for (int l = 0; l < 32; l++) {
+                const uint8_t byte = w[b].qs[32 * (j / 2) + l];
+                const int32_t q = (j & 1) ? (byte >> 4) : (byte & 0x0F);
+                const int32_t xq = xb->qs[l];
+                isum += q * xq;
+                bsum += xq;
+            }
+            const float dx = h2f_tab(xb->d);
+            const float pos = d * (float)(sc * isum), neg = dmin * (float)(m * bsum);
+            acc = fmaf(dx, pos - neg, acc);
+        }
+    }
+    return acc;
+}
+
+__device__ __forceinline__ int32_t q6k_get(const blk_q6_k *x, int e) {
+    const int half = e / 128, r = e % 128, grp = r / 32, l = r % 32;
+    const uint8_t *ql = x->ql + 64 * half, *qh = x->qh + 32 * half;
+    int32_t lo;
+    switch (grp) {
+    case 0: lo = ql[l] & 0x0F; break;
+    case 1: lo = ql[l + 32] & 0x0F; break;
+    case 2: lo = ql[l] >> 4; break;
+    default: lo = ql[l + 32] >> 4; break;
+    }
+    const int32_t hi = (qh[l] >> (2 * grp)) & 3;
+    return (lo | (hi << 4)) - 32;
+}
+
+__device__ float dot_q6_k(const uint8_t *wv, const uint8_t *xv, int64_t n) {
+    const blk_q6_k *w = (const blk_q6_k *)wv;
+    const blk_q8_0 *x = (const blk_q8_0 *)xv;
+    float acc = 0.0f;
+    for (int64_t b = 0; b < n / 256; b++) {
+        const float d = h2f_tab(w[b].d);
+        for (int t = 0; t < 8; t++) {
+            const blk_q8_0 *xb = &x[b * 8 + t];
+            int32_t s = 0;
+            for (int h = 0; h < 2; h++) {
+                int32_t isum = 0;
+                for (int l = 0; l < 16; l++) isum += q6k_get(&w[b], 32 * t + 16 * h + l) * (int32_t)xb->qs[16 * h + l];
+                s += (int32_t)w[b].scales[2 * t + h] * isum;
+            }
+            const float dd = h2f_tab(xb->d) * d;
+            acc = fmaf(dd, (float)s, acc);
+        }
+    }
+    return acc;
+}
+
+// MatMul (mat.cpp:130-143): one thread per output element, the output index running fastest along the
+// weight rows; xm = the activations in the intermediate type, contiguous [ne00, ne11, ne02, ne03]
+template <int WT>
+__global__ __launch_bounds__(64) void exact_dots_kernel(xdesc w, const uint8_t *__restrict__ xm, int64_t x_row, xdesc d, int64_t ne11, int64_t total) {
+    const int64_t o = (int64_t)blockIdx.x * 64 + threadIdx.x;
+    if (o >= total) return;
+    const int64_t ne00 = w.ne[0], ne01 = w.ne[1], ne02 = w.ne[2];
+    const int64_t i01 = o % ne01, i11 = o / ne01 % ne11, i02 = o / (ne01 * ne11) % ne02, i03 = o / (ne01 * ne11 * ne02);
+    const uint8_t *wr = xat(w, 0, i01, i02, i03);
+    const uint8_t *xr = xm + ((i03 * ne02 + i02) * ne11 + i11) * x_row;
+    float v;
+    if (WT == SPY_HIP_Q4_0) v = dot_q4_0(wr, xr, ne00);
+    else if (WT == SPY_HIP_Q8_0) v = dot_q8_0(wr, xr, ne00);
+    else if (WT == SPY_HIP_Q4_K) v = dot_q4_k(wr, xr, ne00);
+    else if (WT == SPY_HIP_Q6_K) v = dot_q6_k(wr, xr, ne00);
+    else v = dot_f16(wr, xr, ne00);
+    *(float *)xat(d, i01, i11, i02, i03) = v;
+}
+
+}   // namespace
+
+int spy_exact_on() {
+    if (g_exact < 0) {
+        const char *e = getenv("SPY_HIP_EXACT");
+        g_exact = (e && *e && *e != '0') ? 1 : 0;
+    }
+    return g_exact;
+}
+
+extern "C" int spy_hip_set_exact_order(int on) {
+    const int prev = spy_exact_on();
+    g_exact = on ? 1 : 0;
+    return prev;
+}
+
+// The callers (the spy_hip_op_* entry points) have validated types, shapes and strides.
+int spy_exact_norm_rms(hipStream_t st, const spy_hip_tensor *x, const spy_hip_tensor *dst, float eps) {
+    exact_norm_rms_kernel<<<dim3((unsigned)spy_t_nrow(dst)), dim3(256), 0, st>>>(mkx(x), mkx(dst), eps);
+    return SPY_LAUNCH_RC();
+}
+
+int spy_exact_silu(hipStream_t st, const spy_hip_tensor *x, const spy_hip_tensor *dst) {
+    int rc = ensure_luts();
+    if (rc) return rc;
+    const int64_t total = spy_t_nelem(x);
+    exact_silu_kernel<<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st>>>(mkx(x), mkx(dst), g_lut, total);
+    return SPY_LAUNCH_RC();
+}
+
+int spy_exact_softmax(hipStream_t st, const spy_hip_tensor *x, const spy_hip_tensor *mask, const spy_hip_tensor *dst, float scale) {
+    if (dst->type != SPY_HIP_F32) return SPY_HIP_EUNSUPPORTED;      // the fp16 output is a shortcut of the fast path
+    int rc = ensure_luts();
+    if (rc) return rc;
+    exact_softmax_kernel<<<dim3((unsigned)spy_t_nrow(dst)), dim3(256), 0, st>>>(mkx(x), mkx(mask ? mask : x), mask != nullptr, mkx(dst), scale, g_lut);
+    return SPY_LAUNCH_RC();
+}
+
+int spy_exact_rope(hipStream_t st, const spy_hip_tensor *x, const spy_hip_tensor *pos, const spy_hip_tensor *dst, const spy_hip_rope_param *p) {
+    // The reference computes the rotation of a token on the host: theta starts at the position and is multiplied by
+    // theta_scale once per pair (non-linear.cpp:304-309), cosf / sinf from libm.  The positions live in device
+    // memory, so this form waits for the stream, reads them back and uploads the table.
+    const int64_t ne0 = dst->ne[0], ne2 = dst->ne[2];
+    hipError_t e = hipStreamSynchronize(st);
+    if (e != hipSuccess) return (int)e;
+    std::vector<int32_t> hp((size_t)ne2);
+    if (pos->nb[0] == 4) e = hipMemcpy(hp.data(), pos->data, (size_t)ne2 * 4, hipMemcpyDeviceToHost);
+    else e = hipMemcpy2D(hp.data(), 4, pos->data, (size_t)pos->nb[0], 4, (size_t)ne2, hipMemcpyDeviceToHost);
+    if (e != hipSuccess) return (int)e;
+    const float theta_scale = powf(p->freq_base, -2.0f / (float)p->num_dim);
+    std::vector<float> tab((size_t)(ne2 * ne0));
+    for (int64_t i2 = 0; i2 < ne2; i2++) {
+        float theta = (float)hp[(size_t)i2];
+        for (int64_t i0 = 0; i0 < ne0; i0 += 2) {
+            const float ang = p->freq_scale * theta;
+            tab[(size_t)(i2 * ne0 + i0)] = cosf(ang) * p->attention_factor;
+            tab[(size_t)(i2 * ne0 + i0 + 1)] = sinf(ang) * p->attention_factor;
+            theta *= theta_scale;
+        }
+    }
+    const size_t need = tab.size() * sizeof(float);
+    if (need > g_rope_cap) {
+        if (g_rope) { (void)hipDeviceSynchronize(); (void)hipFree(g_rope); g_rope = nullptr; g_rope_cap = 0; }
+        e = hipMalloc((void **)&g_rope, need);
+        if (e != hipSuccess) return (int)e;
+        g_rope_cap = need;
+    }
+    e = hipMemcpy(g_rope, tab.data(), need, hipMemcpyHostToDevice);
+    if (e != hipSuccess) return (int)e;
+    const dim3 grid((unsigned)dst->ne[1], (unsigned)dst->ne[2], (unsigned)dst->ne[3]);
+    exact_rope_kernel<<<grid, dim3(64), 0, st>>>(mkx(x), mkx(dst), g_rope);
+    if (hipGetLastError() != hipSuccess) return SPY_HIP_EINVAL;
+    return (int)hipStreamSynchronize(st);      // the table is overwritten by the next call
+}
+
+int spy_exact_dots(hipStream_t st, int t0, const spy_hip_tensor *w, const uint8_t *xm, int64_t x_row, int64_t ne11, const spy_hip_tensor *dst) {
+    const int64_t total = w->ne[1] * ne11 * w->ne[2] * w->ne[3];
+    if (total <= 0 || (total + 63) / 64 >= (1ll << 31)) return SPY_HIP_EINVAL;
+    const dim3 grid((unsigned)((total + 63) / 64)), block(64);
+    switch (t0) {
+    case SPY_HIP_Q4_0: exact_dots_kernel<SPY_HIP_Q4_0><<<grid, block, 0, st>>>(mkx(w), xm, x_row, mkx(dst), ne11, total); break;
+    case SPY_HIP_Q8_0: exact_dots_kernel<SPY_HIP_Q8_0><<<grid, block, 0, st>>>(mkx(w), xm, x_row, mkx(dst), ne11, total); break;
+    case SPY_HIP_Q4_K: exact_dots_kernel<SPY_HIP_Q4_K><<<grid, block, 0, st>>>(mkx(w), xm, x_row, mkx(dst), ne11, total); break;
+    case SPY_HIP_Q6_K: exact_dots_kernel<SPY_HIP_Q6_K><<<grid, block, 0, st>>>(mkx(w), xm, x_row, mkx(dst), ne11, total); break;
+    case SPY_HIP_F16: exact_dots_kernel<SPY_HIP_F16><<<grid, block, 0, st>>>(mkx(w), xm, x_row, mkx(dst), ne11, total); break;
+    default: return SPY_HIP_EUNSUPPORTED;
+    }
+    return SPY_LAUNCH_RC();
+}

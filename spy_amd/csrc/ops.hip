@@ -9,6 +9,14 @@
 
 int *spy_hip_err_flag_ptr();
 
+// exact_order.hip: the same operators with every sum in the host backend's order (spy_hip_set_exact_order)
+int spy_exact_on();
+int spy_exact_norm_rms(hipStream_t st, const spy_hip_tensor *x, const spy_hip_tensor *dst, float eps);
+int spy_exact_silu(hipStream_t st, const spy_hip_tensor *x, const spy_hip_tensor *dst);
+int spy_exact_softmax(hipStream_t st, const spy_hip_tensor *x, const spy_hip_tensor *mask, const spy_hip_tensor *dst, float scale);
+int spy_exact_rope(hipStream_t st, const spy_hip_tensor *x, const spy_hip_tensor *pos, const spy_hip_tensor *dst, const spy_hip_rope_param *p);
+int spy_exact_dots(hipStream_t st, int t0, const spy_hip_tensor *w, const uint8_t *xm, int64_t x_row, int64_t ne11, const spy_hip_tensor *dst);
+
 struct tdesc {              // a tensor as the kernels see it
     uint8_t *p;
     int64_t ne[4], nb[4];
@@ -61,6 +69,7 @@ extern "C" int spy_hip_op_norm_rms(void *stream, const spy_hip_tensor *x, const 
     SPY_CHECK_ARG(same_ne(x, dst) && x->nb[0] == 4 && dst->nb[0] == 4);
     const int64_t nrow = spy_t_nrow(dst);
     CHECK_GRID(nrow, 1);
+    if (spy_exact_on()) return spy_exact_norm_rms((hipStream_t)stream, x, dst, eps);
     norm_rms_kernel<<<dim3((unsigned)nrow), dim3(256), 0, (hipStream_t)stream>>>(mk(x), mk(dst), eps);
     return SPY_LAUNCH_RC();
 }
@@ -153,6 +162,7 @@ extern "C" int spy_hip_op_silu(void *stream, const spy_hip_tensor *x, const spy_
     SPY_CHECK_ARG(same_ne(x, dst));
     const int64_t total = spy_t_nelem(x);
     CHECK_GRID(total, 256);
+    if (spy_exact_on()) return spy_exact_silu((hipStream_t)stream, x, dst);
     if (spy_t_contiguous(x) && spy_t_contiguous(dst) && total % 4 == 0 && (((uintptr_t)x->data | (uintptr_t)dst->data) & 15) == 0) {
         silu_flat_kernel<<<dim3(grid_for(total / 4, 256)), dim3(256), 0, (hipStream_t)stream>>>((const float4 *)x->data, (float4 *)dst->data, total / 4);
         return SPY_LAUNCH_RC();
@@ -274,6 +284,7 @@ static int softmax_launch(void *stream, const spy_hip_tensor *x, const spy_hip_t
     }
     const int64_t nrow = spy_t_nrow(dst);
     CHECK_GRID(nrow, 1);
+    if (causal_past < 0 && dst->type == SPY_HIP_F32 && spy_exact_on()) return spy_exact_softmax((hipStream_t)stream, x, mask, dst, scale);
     // a masked element of the generic kernel reads as (s + mask) * scale: the row kernel's shortcut needs scale > 0 and a
     // mask that really is 0 / -inf, which is what the graph builds (llama.cpp:248-263)
     const bool row_ok = spy_softmax_row_ok(dst->ne[0]) && scale > 0.0f;
@@ -331,6 +342,7 @@ extern "C" int spy_hip_op_rope(void *stream, const spy_hip_tensor *x, const spy_
     // CUDA-style grids cap y/z at 65535: put the token index on x when it is the large one
     const dim3 grid((unsigned)dst->ne[1], (unsigned)dst->ne[2], (unsigned)dst->ne[3]);
     SPY_CHECK_ARG(dst->ne[2] < 65536);
+    if (spy_exact_on()) return spy_exact_rope((hipStream_t)stream, x, pos, dst, p);
     rope_kernel<<<grid, dim3(64), 0, (hipStream_t)stream>>>(mk(x), (const int32_t *)pos->data, pos->nb[0], mk(dst), theta_scale,
                                                            p->freq_scale, p->attention_factor);
     return SPY_LAUNCH_RC();
@@ -593,6 +605,7 @@ static int matmul_impl(void *stream, const spy_hip_tensor *w, const spy_hip_tens
     if (quant) {
         SPY_CHECK_ARG(w->nb[0] == spy_type_size(t0) && w->nb[1] == spy_row_size(t0, ne00));   // whole contiguous rows
         SPY_CHECK_ARG(dst->nb[1] % 4 == 0);
+        if (skip_past < 0 && klimit_past < 0 && spy_exact_on()) return spy_exact_dots(st, t0, w, xm, mid_row, ne11, dst);
         for (int64_t i3 = 0; i3 < ne03; i3++)
             for (int64_t i2 = 0; i2 < ne02; i2++) {
                 const uint8_t *wp = (const uint8_t *)w->data + i2 * w->nb[2] + i3 * w->nb[3];
@@ -607,6 +620,7 @@ static int matmul_impl(void *stream, const spy_hip_tensor *w, const spy_hip_tens
         return 0;
     }
     SPY_CHECK_ARG(w->nb[0] == 2);
+    if (skip_past < 0 && klimit_past < 0 && spy_exact_on()) return spy_exact_dots(st, t0, w, xm, mid_row, ne11, dst);
     if (ne11 >= 16 && ne01 >= 16 && ne00 % 8 == 0 && w->nb[1] % 16 == 0 && w->nb[2] % 16 == 0 && w->nb[3] % 16 == 0 &&
         ((uintptr_t)w->data & 15) == 0 && ((uintptr_t)xm & 15) == 0 && dst->nb[1] % 4 == 0 && dst->nb[2] % 4 == 0 && ne02 <= 65535) {
         for (int64_t i3 = 0; i3 < ne03; i3++) {            // prompt-sized attention products: fp16 MFMA

@@ -1,0 +1,228 @@
+"""Exact-order mode of the operator entry points (spy_hip_set_exact_order): every float sum in the order
+of the host backend's loops (vec_dot.h:42-146, vec_util.h:75-81, non-linear.cpp:129-223 in the Spy tree),
+exp / silu / cos / sin from the host's libm.  The bar here is equality of the BITS with the CPU oracle:
+per operator, for a whole model through Backend::submit, and for the greedy tokens of the 7B shape."""
+import ctypes as C
+import os
+
+import numpy as np
+import pytest
+
+from tests import oracle_lib as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture()
+def hip():
+    from spy_amd import _lib as H
+    H.init(0)
+    prev = H.load().spy_hip_set_exact_order(1)
+    yield H
+    H.load().spy_hip_set_exact_order(prev)
+
+
+def B(t):
+    return C.byref(t)
+
+
+def _same_bits(got, want, what):
+    got, want = np.ascontiguousarray(got, np.float32), np.ascontiguousarray(want, np.float32)
+    bad = got.view(np.uint32) != want.view(np.uint32)
+    assert not bad.any(), "%s: %d of %d outputs differ in their bits, largest difference %.3e" % (
+        what, int(bad.sum()), bad.size, float(np.abs(got.astype(np.float64) - want.astype(np.float64))[bad].max()))
+
+
+@pytest.mark.parametrize("wtype", [O.Q4_0, O.Q8_0, O.Q4_K, O.Q6_K])
+@pytest.mark.parametrize("M,K,T", [(96, 4096, 5), (40, 11008, 1), (33, 256, 3)])
+def test_quantized_matmul_bits(hip, oracle, wtype, M, K, T):
+    from tests.gpu_util import dev, dev_empty, call
+    if K % 256 and wtype in (O.Q4_K, O.Q6_K):
+        pytest.skip("K-quant rows are whole super-blocks")
+    rng = np.random.default_rng(100 * wtype + K + T)
+    w = O.quantize(oracle, (rng.standard_normal((M, K)) * 0.02).astype(np.float32), wtype)
+    x = (rng.standard_normal((T, K)) * rng.uniform(0.1, 30.0, (T, 1))).astype(np.float32)
+    want = O.matmul(oracle, w, wtype, M, K, x, nthread=4)
+    dw, dx, dd = dev(w), dev(x), dev_empty(T * M * 4, 0xFF)
+    tw, tx, td = hip.tensor(dw, wtype, [K, M]), hip.tensor(dx, hip.F32, [K, T]), hip.tensor(dd, hip.F32, [M, T])
+    L = hip.load()
+    need = L.spy_hip_op_matmul_scratch_size(B(tw), B(tx))
+    scratch = dev_empty(need, 0)
+    call(L.spy_hip_op_matmul, None, B(tw), B(tx), B(td), scratch.ptr, need)
+    _same_bits(dd.download(np.float32).reshape(T, M), want, "matmul type %d %dx%d T %d" % (wtype, M, K, T))
+
+
+def test_q8_0_weights_of_any_byte(hip, oracle):
+    """Weight bytes a quantizer never writes (-128): the host backend's sign / maddubs sequence
+    (vec_util.h:101-110) gives 128 * -128 for (-128) * (-128); the exact mode follows it."""
+    from tests.gpu_util import dev, dev_empty, call
+    rng = np.random.default_rng(77)
+    M, K, T = 16, 512, 2
+    w = O.quantize(oracle, rng.standard_normal((M, K)).astype(np.float32), O.Q8_0).copy()
+    blocks = w.reshape(M * K // 32, 34)
+    blocks[:, 2:] = rng.integers(0, 256, (blocks.shape[0], 32), dtype=np.uint8)
+    blocks[::3, 2:6] = 0x80
+    x = rng.standard_normal((T, K)).astype(np.float32)
+    want = O.matmul(oracle, w, O.Q8_0, M, K, x, nthread=1)
+    dw, dx, dd = dev(w), dev(x), dev_empty(T * M * 4, 0xFF)
+    tw, tx, td = hip.tensor(dw, O.Q8_0, [K, M]), hip.tensor(dx, hip.F32, [K, T]), hip.tensor(dd, hip.F32, [M, T])
+    L = hip.load()
+    need = L.spy_hip_op_matmul_scratch_size(B(tw), B(tx))
+    scratch = dev_empty(need, 0)
+    call(L.spy_hip_op_matmul, None, B(tw), B(tx), B(td), scratch.ptr, need)
+    _same_bits(dd.download(np.float32).reshape(T, M), want, "Q8_0 with arbitrary weight bytes")
+
+
+@pytest.mark.parametrize("n_kv", [1, 31, 32, 33, 64, 65, 300, 4241])
+def test_attention_products_bits(hip, oracle, n_kv):
+    """attn_score (contraction over 128) and KQV (contraction over n_kv: the strict `i + 32 < n` loop bound
+    and the scalar tail of Dot<FP16,FP16>, vec_dot.h:124-145) through the cache views."""
+    from tests.gpu_util import dev, dev_empty, call
+    rng = np.random.default_rng(9 + n_kv)
+    hd, H_, T = 128, 4, 2
+    Cx = n_kv + 11
+    d = hd * H_
+    kc = rng.standard_normal((Cx, H_, hd)).astype(np.float16)
+    vc = rng.standard_normal((d, Cx)).astype(np.float16)
+    q = rng.standard_normal((T, H_, hd)).astype(np.float32)
+    P = rng.random((H_, T, n_kv)).astype(np.float32)
+    S_want, O_want = np.zeros((H_, T, n_kv), np.float32), np.zeros((H_, T, hd), np.float32)
+    assert oracle.spy_o_matmul(B(O.tensor(kc.view(np.uint16), O.F16, [hd, n_kv, H_], nb=[2, 2 * d, 2 * hd])),
+                               B(O.tensor(q, O.F32, [hd, T, H_], nb=[4, 4 * d, 4 * hd])), B(O.tensor(S_want, O.F32, [n_kv, T, H_])), 2) == 0
+    assert oracle.spy_o_matmul(B(O.tensor(vc.view(np.uint16), O.F16, [n_kv, hd, H_], nb=[2, 2 * Cx, 2 * Cx * hd])),
+                               B(O.tensor(P, O.F32, [n_kv, T, H_])), B(O.tensor(O_want, O.F32, [hd, T, H_])), 2) == 0
+    L = hip.load()
+    dkc, dvc, dq, dP = dev(kc.view(np.uint16)), dev(vc.view(np.uint16)), dev(q), dev(P)
+    dS, dO = dev_empty(S_want.nbytes, 0xFF), dev_empty(O_want.nbytes, 0xFF)
+    tk = hip.tensor(dkc, hip.F16, [hd, n_kv, H_], nb=[2, 2 * d, 2 * hd])
+    tq = hip.tensor(dq, hip.F32, [hd, T, H_], nb=[4, 4 * d, 4 * hd])
+    tS = hip.tensor(dS, hip.F32, [n_kv, T, H_])
+    tv = hip.tensor(dvc, hip.F16, [n_kv, hd, H_], nb=[2, 2 * Cx, 2 * Cx * hd])
+    tP, tO = hip.tensor(dP, hip.F32, [n_kv, T, H_]), hip.tensor(dO, hip.F32, [hd, T, H_])
+    need = max(L.spy_hip_op_matmul_scratch_size(B(tk), B(tq)), L.spy_hip_op_matmul_scratch_size(B(tv), B(tP)), 256)
+    sc = dev_empty(need, 0)
+    call(L.spy_hip_op_matmul, None, B(tk), B(tq), B(tS), sc.ptr, need)
+    _same_bits(dS.download(np.float32).reshape(S_want.shape), S_want, "attn_score n_kv %d" % n_kv)
+    call(L.spy_hip_op_matmul, None, B(tv), B(tP), B(tO), sc.ptr, need)
+    _same_bits(dO.download(np.float32).reshape(O_want.shape), O_want, "KQV n_kv %d" % n_kv)
+
+
+def test_norm_softmax_silu_rope_bits(hip, oracle):
+    from tests.gpu_util import dev, dev_empty, call
+    L = hip.load()
+    rng = np.random.default_rng(21)
+    # NormRMS: rows of whole groups of four, with a remainder, longer than one LDS pass
+    for T, d in [(1, 4096), (7, 4096), (2, 103), (3, 11008), (2, 4099), (1, 3)]:
+        x = (rng.standard_normal((T, d)) * 2.5).astype(np.float32)
+        want = np.zeros_like(x)
+        assert oracle.spy_o_norm_rms(B(O.tensor(x, O.F32, [d, T])), B(O.tensor(want, O.F32, [d, T])), 1e-5) == 0
+        dx, dy = dev(x), dev_empty(x.nbytes, 0xFF)
+        call(L.spy_hip_op_norm_rms, None, B(hip.tensor(dx, hip.F32, [d, T])), B(hip.tensor(dy, hip.F32, [d, T])), 1e-5)
+        _same_bits(dy.download(np.float32).reshape(T, d), want, "norm_rms %dx%d" % (T, d))
+    # Silu: every fp16 bit pattern that is a finite number, and fp32 values between them
+    bits = np.arange(0, 0x10000, dtype=np.uint16)
+    finite = (bits & 0x7C00) != 0x7C00
+    x = np.concatenate([bits[finite].view(np.float16).astype(np.float32), rng.standard_normal(4096).astype(np.float32) * 4])
+    want = np.zeros_like(x)
+    assert oracle.spy_o_silu(B(O.tensor(x, O.F32, [x.size])), B(O.tensor(want, O.F32, [x.size]))) == 0
+    dx, dy = dev(x), dev_empty(x.nbytes, 0xFF)
+    call(L.spy_hip_op_silu, None, B(hip.tensor(dx, hip.F32, [x.size])), B(hip.tensor(dy, hip.F32, [x.size])))
+    _same_bits(dy.download(np.float32), want, "silu")
+    # Softmax: causal mask, no mask, rows shorter and longer than one LDS pass
+    scale = float(1.0 / np.sqrt(128.0))
+    for (H_, T, n_kv, Cx, P) in [(32, 1, 300, 512, 299), (4, 5, 9, 16, 4), (2, 3, 1030, 1100, 1027), (2, 2, 4243, 4352, 4241), (1, 1, 1, 8, 0)]:
+        s = (rng.standard_normal((H_, T, n_kv)) * 12).astype(np.float32)
+        mask = np.where(np.arange(Cx)[None, :] <= (np.arange(T)[:, None] + P), 0.0, -np.inf).astype(np.float32)
+        ds, dm, dd = dev(s), dev(mask), dev_empty(s.nbytes, 0xFF)
+        for use_mask in (True, False):
+            want = np.zeros_like(s)
+            assert oracle.spy_o_softmax(B(O.tensor(s, O.F32, [n_kv, T, H_])), B(O.tensor(mask, O.I32, [Cx, T])) if use_mask else None,
+                                        B(O.tensor(want, O.F32, [n_kv, T, H_])), scale) == 0
+            call(L.spy_hip_op_softmax, None, B(hip.tensor(ds, hip.F32, [n_kv, T, H_])), B(hip.tensor(dm, hip.I32, [Cx, T])) if use_mask else None,
+                 B(hip.tensor(dd, hip.F32, [n_kv, T, H_])), scale)
+            _same_bits(dd.download(np.float32).reshape(s.shape), want, "softmax H%d T%d n_kv%d mask %d" % (H_, T, n_kv, use_mask))
+    # Rope
+    hd, H_, T = 128, 32, 7
+    pos = np.array([0, 1, 7, 100, 2047, 4095, 4351], dtype=np.int32)
+    x = rng.standard_normal((T, H_, hd)).astype(np.float32)
+    want = np.zeros_like(x)
+    rp = O.default_rope(hd, 4352)
+    assert oracle.spy_o_rope(B(O.tensor(x, O.F32, [hd, H_, T])), B(O.tensor(pos, O.I32, [T])), B(O.tensor(want, O.F32, [hd, H_, T])), B(rp)) == 0
+    dx, dp, dy = dev(x), dev(pos), dev_empty(x.nbytes, 0xFF)
+    hp = hip.RopeParam(0, 0, hd, 4352, 4352, 10000.0, 1.0, 0.0, 1.0, 32.0, 1.0, 0.0, 0)
+    call(L.spy_hip_op_rope, None, B(hip.tensor(dx, hip.F32, [hd, H_, T])), B(hip.tensor(dp, hip.I32, [T])), B(hip.tensor(dy, hip.F32, [hd, H_, T])), B(hp))
+    _same_bits(dy.download(np.float32).reshape(x.shape), want, "rope")
+
+
+def test_switch_returns_previous_setting_and_default_is_off():
+    from spy_amd import _lib as H
+    L = H.load()
+    if os.environ.get("SPY_HIP_EXACT", "0") not in ("", "0"):
+        pytest.skip("exact order switched on by the environment")
+    assert L.spy_hip_set_exact_order(1) == 0
+    assert L.spy_hip_set_exact_order(0) == 1
+    assert L.spy_hip_set_exact_order(0) == 0
+
+
+@pytest.mark.parametrize("name,kw", [
+    ("Q4_0", dict(wtype=O.Q4_0)),
+    ("Q8_0", dict(wtype=O.Q8_0)),
+    ("Q4_K/Q6_K mix", dict(wtype=O.Q4_K, t_out=O.Q6_K, tensor_types={"attn_v": O.Q6_K, "ffn_down": O.Q6_K})),
+])
+def test_whole_model_through_submit_has_the_oracle_bits(hip, name, kw):
+    """33 operators per layer through Backend::submit: the logits of a prompt pass and of single-token passes on
+    top of it, and both caches, equal the CPU oracle's bit for bit."""
+    from spy_amd import backend_driver as BD
+    from spy_amd import model as M
+    from tests.model_util import OracleModel, k_quant_quantizer
+    cfg = M.Config(n_layer=3, n_embd=256, n_head=2, n_ff=768, n_vocab=512, n_ctx=64, **kw)
+    tensors = M.synth_model(cfg, seed=11, quantizer=k_quant_quantizer)
+    host, ora = BD.HostModel(cfg, tensors), OracleModel(cfg, tensors)
+    prompt = np.random.default_rng(3).integers(0, cfg.n_vocab, 9).astype(np.int32)
+    _same_bits(host.forward(prompt, 0), ora.forward(prompt, 0), name + ": prompt logits")
+    for il in range(cfg.n_layer):
+        for which, ref in ((0, ora.k_cache[il]), (1, ora.v_cache[il])):
+            assert np.array_equal(host.cache(il, which).view(np.uint16), ref.view(np.uint16)), (name, il, which)
+    toks = ora.generate(prompt, 12)
+    ora2 = OracleModel(cfg, tensors)
+    lg = ora2.forward(prompt, 0)[-1]
+    for step in range(12):
+        assert int(np.argmax(lg)) == int(toks[step])
+        t = toks[step:step + 1]
+        lh, lg = host.forward(t, 9 + step)[0], ora2.forward(t, 9 + step)[0]
+        _same_bits(lh, lg, "%s: single-token pass %d" % (name, step))
+    host.close()
+
+
+@pytest.mark.timeout(900)
+def test_llama2_7b_q4_0_greedy_32_tokens_identical():
+    """The 7B shape, Q4_0, 8 random prompt tokens, 32 greedy steps through Backend::submit in exact order:
+    the 32 tokens are the CPU oracle's, and so are the bits of every pass's logits."""
+    from spy_amd import _lib as H
+    from spy_amd import backend_driver as BD
+    from spy_amd import model as M
+    from tests.model_util import OracleModel
+    H.init(0)
+    cfg = M.Config.llama2_7b(n_ctx=48, wtype=O.Q4_0)
+    tensors = M.synth_model(cfg, seed=1234)
+    ora = OracleModel(cfg, tensors, nthread=min(16, os.cpu_count() or 8))
+    prompt = np.random.default_rng(5).integers(0, cfg.n_vocab, 8).astype(np.int32)
+    prev = H.load().spy_hip_set_exact_order(1)
+    try:
+        host = BD.HostModel(cfg, tensors)
+        lg_o, lg_h = ora.forward(prompt, 0)[-1], host.forward(prompt, 0)[-1]
+        want, got, equal_bits = [], [], 0
+        for step in range(32):
+            equal_bits += int(np.array_equal(lg_o.view(np.uint32), lg_h.view(np.uint32)))
+            want.append(int(ora.L.spy_o_argmax(lg_o.ctypes.data, lg_o.size)))
+            got.append(int(np.argmax(lg_h)))                       # numpy's argmax is the first maximum too
+            if step == 31:
+                break
+            lg_o = ora.forward(np.array([want[-1]], np.int32), 8 + step)[0]
+            lg_h = host.forward(np.array([got[-1]], np.int32), 8 + step)[0]
+        print("oracle tokens:", want, "\nhip tokens:   ", got, "\n%d of 32 passes with bit-identical logits" % equal_bits, flush=True)
+        assert got == want
+        assert equal_bits == 32
+        host.close()
+    finally:
+        H.load().spy_hip_set_exact_order(prev)
