@@ -12,6 +12,9 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <algorithm>
+#include <vector>
+
 
 static bool fused_ok(const spy_hip_llama *m);
 static int probe_attn(spy_hip_llama *m, int il) {
@@ -278,6 +281,7 @@ int spy_prompt_attn_launch(hipStream_t st, const uint16_t *q16, const uint16_t *
 int spy_gemm_q8act_pair(hipStream_t st, int wtype, const void *w1, const void *w2, const void *xq, float *dst1, float *dst2,
                         int64_t M, int64_t K, int64_t T, int64_t dst_stride);                                                  // gemm.hip
 int spy_softmax_causal_launch(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *dst, float scale, int n_past);   // ops.hip
+int spy_exact_on();                                                                                                          // exact_order.hip
 int spy_softmax_row_ok(int64_t ne0);                                                                                         // ops.hip
 
 // KQ mask of a pass over tokens P .. P + T - 1 (llama.cpp:248-263): row i allows the cached positions j <= P + i
@@ -295,7 +299,9 @@ static int forward_ops(spy_hip_llama *m, hipStream_t st, const int32_t *tokens_h
     const int64_t d = c.n_embd, F = c.n_ff, C = c.n_ctx, H = c.n_head, hd = m->hd, V = c.n_vocab, n_kv = (int64_t)P + T;
     // Passes over many tokens (every MatMul on the matrix cores): the elementwise operators between two MatMuls write the
     // next MatMul's Q8_0 activations directly (same bytes as the separate operators: prompt_fused.hip)
-    const bool fuse_act = T >= 16 && d % 64 == 0 && F % 64 == 0 && !getenv("SPY_HIP_PROMPT_UNFUSED");
+    // exact-order mode (spy_hip_set_exact_order): the plain operators only, each in its exact form
+    const bool exact = spy_exact_on() != 0;
+    const bool fuse_act = !exact && T >= 16 && d % 64 == 0 && F % 64 == 0 && !getenv("SPY_HIP_PROMPT_UNFUSED");
     // ... and the attention of a layer is one kernel (prompt_attn.hip) where its shape conditions hold;
     // SPY_HIP_PROMPT_ATTN=0: attention as MatMul -> Softmax -> MatMul (bit-identical to the operator path)
     const char *pa_env = getenv("SPY_HIP_PROMPT_ATTN");
@@ -394,7 +400,7 @@ static int forward_ops(spy_hip_llama *m, hipStream_t st, const int32_t *tokens_h
         spy_hip_tensor t_vall = T3s(SPY_HIP_F16, m->v_cache[il], n_kv, hd, H, 2, 2 * C, 2 * C * hd);
         // causal_ok: the softmax below takes the row kernel, which reads no score beyond a row's causal length and writes
         // zeros there: the two products may then leave out what the mask removes
-        const bool causal_ok = spy_softmax_row_ok(n_kv) != 0;
+        const bool causal_ok = !exact && spy_softmax_row_ok(n_kv) != 0;
         // the probabilities go to the KQV product as fp16 (its first step, mat.cpp:37): the softmax writes them that way
         // directly where the fp16 GEMM takes them (rows of a multiple of 8 elements)
         const bool p16 = n_kv % 8 == 0 && causal_ok && T >= 16;
@@ -465,7 +471,8 @@ static int forward_any(spy_hip_llama *m, void *stream, const int32_t *tokens_hos
     SPY_CHECK_ARG((int64_t)n_past + n_token <= m->desc.n_ctx);                  // llama.cpp:249
     hipStream_t st = stream ? (hipStream_t)stream : m->own_stream;
     for (int i = 0; i < n_token; i++) SPY_CHECK_ARG(tokens_host[i] >= 0 && tokens_host[i] < m->desc.n_vocab);   // view.cpp:61
-    if (n_token == 1 && fused_ok(m) && !getenv("SPY_HIP_FORCE_OPS")) {
+    const bool exact = spy_exact_on() != 0;
+    if (n_token == 1 && fused_ok(m) && !exact && !getenv("SPY_HIP_FORCE_OPS")) {
         dev_state h = {tokens_host[0], n_past, 0, 0};
         HIP_TRY(hipMemcpyAsync(m->st, &h, sizeof(h), hipMemcpyHostToDevice, st));
         RC_TRY(enqueue_pass_any(m, st, PASS_LOGITS));
@@ -478,7 +485,9 @@ static int forward_any(spy_hip_llama *m, void *stream, const int32_t *tokens_hos
     // (the scores of a chunk take n_kv * chunk * n_head * 6 bytes of scratch; larger chunks fill the matrix-core grids better)
     const char *ch_env = getenv("SPY_HIP_PREFILL_CHUNK");
     const int ch_req = ch_env ? atoi(ch_env) : 0;
-    const int CH = ch_req >= 16 ? ch_req : SPY_PREFILL_CHUNK;
+    // exact order: one pass over the whole prompt, as the reference runs it (a chunk boundary moves elements between
+    // the 8-lane part and the scalar tail of the KQV dots and between the groups of four of the softmax sum)
+    const int CH = exact ? n_token : ch_req >= 16 ? ch_req : SPY_PREFILL_CHUNK;
     for (int t0 = 0; t0 < n_token; t0 += CH) {
         const int tc = n_token - t0 < CH ? n_token - t0 : CH;
         // logits nobody asked for are not computed: no buffer -> no head; last_only -> the head runs on the last row of the last chunk
@@ -506,6 +515,18 @@ extern "C" int spy_hip_llama_decode_greedy(spy_hip_llama *m, void *stream, int32
                                            int32_t *tokens_host, int32_t use_graph) {
     SPY_CHECK_ARG(m && n_steps > 0 && n_past >= 0 && first_token >= 0 && first_token < m->desc.n_vocab);
     SPY_CHECK_ARG((int64_t)n_past + n_steps <= m->desc.n_ctx && n_steps <= m->max_out);
+    if (spy_exact_on()) {
+        // exact order: the reference's loop as it stands (cli.h:88-128) -- one operator-by-operator pass per token,
+        // the first maximum of its logits (greedy.h:20-25) taken on the host
+        std::vector<float> lg((size_t)m->desc.n_vocab);
+        int32_t tok = first_token;
+        for (int i = 0; i < n_steps; i++) {
+            RC_TRY(forward_any(m, stream, &tok, 1, n_past + i, lg.data(), false));
+            tok = (int32_t)(std::max_element(lg.begin(), lg.end()) - lg.begin());
+            if (tokens_host) tokens_host[i] = tok;
+        }
+        return 0;
+    }
     if (!fused_ok(m)) return SPY_HIP_EUNSUPPORTED;
     hipStream_t st = stream ? (hipStream_t)stream : m->own_stream;
     dev_state h = {first_token, n_past, 0, 0};

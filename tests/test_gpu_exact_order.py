@@ -194,6 +194,26 @@ def test_whole_model_through_submit_has_the_oracle_bits(hip, name, kw):
     host.close()
 
 
+@pytest.mark.parametrize("n_prompt", [5, 21])
+def test_engine_follows_the_switch(hip, n_prompt):
+    """spy_hip_llama_forward / _forward_last / _decode_greedy in exact order: prompt passes below and above the 16
+    tokens from which the default path fuses operators, single-token passes, and the greedy loop."""
+    from spy_amd import model as M
+    from tests.model_util import OracleModel
+    cfg = M.Config(n_layer=2, n_embd=256, n_head=2, n_ff=768, n_vocab=512, n_ctx=64, wtype=O.Q4_0)
+    tensors = M.synth_model(cfg, seed=5)
+    eng, ora = M.Engine(cfg, tensors), OracleModel(cfg, tensors)
+    prompt = np.random.default_rng(n_prompt).integers(0, cfg.n_vocab, n_prompt).astype(np.int32)
+    lg = ora.forward(prompt, 0)
+    _same_bits(eng.forward(prompt, 0), lg, "engine prompt pass of %d tokens" % n_prompt)
+    _same_bits(eng.forward_last(prompt, 0), lg[-1], "engine prompt pass, last row only")
+    t = np.array([int(np.argmax(lg[-1]))], np.int32)
+    _same_bits(eng.forward(t, n_prompt)[0], ora.forward(t, n_prompt)[0], "engine single-token pass")
+    want = OracleModel(cfg, tensors).generate(prompt, 20)
+    assert eng.generate(prompt, 20).tolist() == want.tolist()
+    eng.close()
+
+
 @pytest.mark.timeout(900)
 def test_llama2_7b_q4_0_greedy_32_tokens_identical():
     """The 7B shape, Q4_0, 8 random prompt tokens, 32 greedy steps through Backend::submit in exact order:
@@ -224,5 +244,11 @@ def test_llama2_7b_q4_0_greedy_32_tokens_identical():
         assert got == want
         assert equal_bits == 32
         host.close()
+        # the token loop of the engine (prompt pass, then its greedy loop) follows the switch: same 32 tokens
+        eng = M.Engine(cfg, tensors)
+        got_eng = eng.generate(prompt, 32).tolist()
+        print("engine tokens:", got_eng, flush=True)
+        assert got_eng == want
+        eng.close()
     finally:
         H.load().spy_hip_set_exact_order(prev)
