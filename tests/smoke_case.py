@@ -37,5 +37,14 @@ def run_smoke(H, O, np):
     assert e1 < 3e-2 and e2 < 3e-2, (e1, e2)
     toks = eng.decode_greedy(int(np.argmax(lo1)), 7, 4, use_graph=True)
     assert len(toks) == 4 and all(0 <= int(t) < cfg.n_vocab for t in toks)
+    # exact-order mode: the same passes with every sum in the host backend's order -- the oracle's bits and tokens
+    prev = L.spy_hip_set_exact_order(1)
+    try:
+        eng2, ora2 = M_.Engine(cfg, tensors), OracleModel(cfg, tensors, nthread=2)
+        assert np.array_equal(eng2.forward(prompt, 0).view(np.uint32), lo.view(np.uint32)), "exact order: prompt logits differ from the oracle's bits"
+        assert eng2.generate(prompt, 8).tolist() == ora2.generate(prompt, 8).tolist(), "exact order: greedy tokens differ from the oracle's"
+        eng2.close()
+    finally:
+        L.spy_hip_set_exact_order(prev)
     eng.close()
-    print("smoke ok: 2-layer token loop, prompt logits err %.2e, single-token logits err %.2e, greedy tokens %s" % (e1, e2, list(map(int, toks))))
+    print("smoke ok: 2-layer token loop, prompt logits err %.2e, single-token logits err %.2e, greedy tokens %s; exact-order mode: logits bit-identical, 8 greedy tokens identical" % (e1, e2, list(map(int, toks))))
