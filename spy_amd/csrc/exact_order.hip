@@ -166,12 +166,19 @@ __global__ __launch_bounds__(256) void exact_softmax_kernel(xdesc x, xdesc mask,
     for (int64_t i = threadIdx.x; i < ne0; i += 256) d[i] *= inv;
 }
 
-// Rope (non-linear.cpp:270-371), default branch; tab = cos, sin per pair and token, from the host
-__global__ __launch_bounds__(64) void exact_rope_kernel(xdesc x, xdesc y, const float *__restrict__ tab) {
+// Rope (non-linear.cpp:270-371), default branch; tab = cos, sin per pair, from the host: one row per token of
+// this call (pos == nullptr) or one row per position 0 .. npos-1, the token's position read here
+__global__ __launch_bounds__(64) void exact_rope_kernel(xdesc x, xdesc y, const float *__restrict__ tab, const uint8_t *__restrict__ pos, int64_t pos_stride,
+                                                        int64_t npos, int *err) {
     const int64_t i1 = blockIdx.x, i2 = blockIdx.y, i3 = blockIdx.z;
     const int64_t ne0 = y.ne[0];
+    int64_t row = i2;
+    if (pos) {
+        row = *(const int32_t *)(pos + i2 * pos_stride);
+        if (row < 0 || row >= npos) { if (threadIdx.x == 0) *err = 1; return; }      // beyond the context the table was built for
+    }
     for (int64_t i0 = 2 * threadIdx.x; i0 < ne0; i0 += 128) {
-        const float c = tab[i2 * ne0 + i0], s = tab[i2 * ne0 + i0 + 1];
+        const float c = tab[row * ne0 + i0], s = tab[row * ne0 + i0 + 1];
         const float *sp = (const float *)xat(x, i0, i1, i2, i3);
         float *dp = (float *)xat(y, i0, i1, i2, i3);
         const float x0 = sp[0], x1 = sp[1];
@@ -353,6 +360,99 @@ __global__ __launch_bounds__(64) void exact_dots_kernel(xdesc w, const uint8_t *
     *(float *)xat(d, i01, i11, i02, i03) = v;
 }
 
+// The same Q4_0 / Q8_0 dots with the eight accumulators of an output element spread over eight lanes: lane l keeps
+// accumulator l (its four products per block), the blocks follow one another in each lane exactly as in the host loop,
+// and hsum_float_8 becomes three exchanges (l ^ 4, l ^ 2, l ^ 1 -- the additions of the tree, whose operands commute).
+// A workgroup computes 32 consecutive output elements; where they all belong to one activation row of at most
+// DOTS8_LDS_BLOCKS blocks, the row is unpacked into LDS once (scale as fp32, quants as aligned words).
+#define DOTS8_LDS_BLOCKS 1024
+__device__ __forceinline__ uint32_t ld_u32_a2(const uint8_t *p) {      // four bytes from a 2-byte-aligned address
+    return (uint32_t)*(const uint16_t *)p | ((uint32_t)*(const uint16_t *)(p + 2) << 16);
+}
+__device__ __forceinline__ int32_t mul_sum4_packed(uint32_t a, uint32_t b) {
+    int8_t x[4], y[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) { x[k] = (int8_t)(a >> (8 * k)); y[k] = (int8_t)(b >> (8 * k)); }
+    return mul_sum4(x, y);
+}
+template <int WT>
+__global__ __launch_bounds__(256) void exact_dots8_kernel(xdesc w, const uint8_t *__restrict__ xm, int64_t x_row, xdesc d, int64_t ne11, int64_t total) {
+    __shared__ float s_d[DOTS8_LDS_BLOCKS];
+    __shared__ uint32_t s_q[DOTS8_LDS_BLOCKS * 8];
+    const int64_t ne00 = w.ne[0], ne01 = w.ne[1], ne02 = w.ne[2];
+    const int64_t nb = ne00 / 32;
+    const int64_t o_first = (int64_t)blockIdx.x * 32, o_last = min(o_first + 31, total - 1);
+    const bool staged = nb <= DOTS8_LDS_BLOCKS && o_first / ne01 == o_last / ne01;      // one (i11, i02, i03) for the workgroup
+    if (staged) {
+        const int64_t xr = o_first / ne01;                                              // = (i03 * ne02 + i02) * ne11 + i11
+        const uint8_t *xb = xm + xr * x_row;
+        for (int64_t i = threadIdx.x; i < nb; i += 256) {
+            const uint8_t *b = xb + i * 34;
+            s_d[i] = h2f_tab(*(const uint16_t *)b);
+#pragma unroll
+            for (int j = 0; j < 8; j++) s_q[i * 8 + j] = ld_u32_a2(b + 2 + 4 * j);
+        }
+        __syncthreads();
+    }
+    const int64_t o = o_first + (threadIdx.x >> 3);
+    if (o >= total) return;                       // whole groups of eight lanes leave together, after the barrier
+    const int l = threadIdx.x & 7;
+    const int64_t i01 = o % ne01, i11 = o / ne01 % ne11, i02 = o / (ne01 * ne11) % ne02, i03 = o / (ne01 * ne11 * ne02);
+    const uint8_t *wr = xat(w, 0, i01, i02, i03);
+    const uint8_t *xr = xm + ((i03 * ne02 + i02) * ne11 + i11) * x_row;
+    // Q4_0: lanes 0..3 take the high nibbles against elements 16..31, lanes 4..7 the low nibbles against 0..15;
+    // Q8_0: lane l takes elements 4l..4l+3
+    const int wo = WT == SPY_HIP_Q4_0 ? 2 + 4 * (l & 3) : 2 + 4 * l;
+    const int xg = WT == SPY_HIP_Q4_0 ? (l < 4 ? 4 : 0) + (l & 3) : l;
+    const int wsz = WT == SPY_HIP_Q4_0 ? 18 : 34;
+    float acc = 0.0f;
+#pragma unroll 4
+    for (int64_t i = 0; i < nb; i++) {
+        const uint8_t *wb = wr + i * wsz;
+        const float dw = h2f_tab(*(const uint16_t *)wb);
+        uint32_t a = ld_u32_a2(wb + wo);
+        if (WT == SPY_HIP_Q4_0) {
+            a = (l < 4 ? (a >> 4) : a) & 0x0F0F0F0Fu;
+            a = (a | 0x80808080u) - 0x08080808u;          // per byte n - 8 without a borrow across bytes ...
+            a ^= 0x80808080u;                             // ... (n + 128 - 8) with the top bit flipped back = n - 8 mod 256
+        }
+        float dx;
+        uint32_t b;
+        if (staged) { dx = s_d[i]; b = s_q[i * 8 + xg]; }
+        else { const uint8_t *xb = xr + i * 34; dx = h2f_tab(*(const uint16_t *)xb); b = ld_u32_a2(xb + 2 + 4 * xg); }
+        acc = fmaf(dw * dx, (float)mul_sum4_packed(a, b), acc);
+    }
+    acc += __shfl_xor(acc, 4, SPY_WAVE);          // r_l = a_l + a_(l+4)
+    acc += __shfl_xor(acc, 2, SPY_WAVE);          // s_0 = r_0 + r_2, s_1 = r_1 + r_3
+    acc += __shfl_xor(acc, 1, SPY_WAVE);          // s_0 + s_1
+    if (l == 0) *(float *)xat(d, i01, i11, i02, i03) = acc;
+}
+
+// Dot<FP16,FP16> with its 4 x 8 accumulators in 32 lanes: lane 8j + l keeps accumulator l of vector j.
+__global__ __launch_bounds__(256) void exact_dots32_kernel(xdesc w, const uint8_t *__restrict__ xm, int64_t x_row, xdesc d, int64_t ne11, int64_t total) {
+    const int64_t o = (int64_t)blockIdx.x * 8 + (threadIdx.x >> 5);
+    if (o >= total) return;                       // whole groups of 32 lanes leave together
+    const int l = threadIdx.x & 31;
+    const int64_t n = w.ne[0], ne01 = w.ne[1], ne02 = w.ne[2];
+    const int64_t i01 = o % ne01, i11 = o / ne01 % ne11, i02 = o / (ne01 * ne11) % ne02, i03 = o / (ne01 * ne11 * ne02);
+    const uint16_t *a = (const uint16_t *)xat(w, 0, i01, i02, i03);
+    const uint16_t *b = (const uint16_t *)(xm + ((i03 * ne02 + i02) * ne11 + i11) * x_row);
+    float acc = 0.0f;
+    int64_t i = 0;
+#pragma unroll 4
+    for (; i + 32 < n; i += 32) acc = fmaf(h2f(a[i + l]), h2f(b[i + l]), acc);
+    acc += __shfl_xor(acc, 16, SPY_WAVE);         // sum[0] += sum[2], sum[1] += sum[3]
+    acc += __shfl_xor(acc, 8, SPY_WAVE);          // sum[0] += sum[1]
+    acc += __shfl_xor(acc, 4, SPY_WAVE);          // t_l = sum[0][l] + sum[0][l + 4]
+    acc += __shfl_xor(acc, 1, SPY_WAVE);          // t_0 + t_1, t_2 + t_3
+    acc += __shfl_xor(acc, 2, SPY_WAVE);          // (t_0 + t_1) + (t_2 + t_3)
+    if (l == 0) {
+        float tail = 0.0f;
+        for (; i < n; i++) { const float pr = h2f_tab(a[i]) * h2f_tab(b[i]); tail += pr; }
+        *(float *)xat(d, i01, i11, i02, i03) = tail + acc;
+    }
+}
+
 }   // namespace
 
 int spy_exact_on() {
@@ -391,28 +491,53 @@ int spy_exact_softmax(hipStream_t st, const spy_hip_tensor *x, const spy_hip_ten
     return SPY_LAUNCH_RC();
 }
 
+// cos / sin of one token: theta starts at the position and is multiplied by theta_scale once per pair
+// (non-linear.cpp:304-309), cosf / sinf from the host's libm as in the reference
+static void rope_row(float *row, int32_t position, int64_t ne0, float theta_scale, const spy_hip_rope_param *p) {
+    float theta = (float)position;
+    for (int64_t i0 = 0; i0 < ne0; i0 += 2) {
+        const float ang = p->freq_scale * theta;
+        row[i0] = cosf(ang) * p->attention_factor;
+        row[i0 + 1] = sinf(ang) * p->attention_factor;
+        theta *= theta_scale;
+    }
+}
+
+int *spy_hip_err_flag_ptr();      // runtime.hip
+
 int spy_exact_rope(hipStream_t st, const spy_hip_tensor *x, const spy_hip_tensor *pos, const spy_hip_tensor *dst, const spy_hip_rope_param *p) {
-    // The reference computes the rotation of a token on the host: theta starts at the position and is multiplied by
-    // theta_scale once per pair (non-linear.cpp:304-309), cosf / sinf from libm.  The positions live in device
-    // memory, so this form waits for the stream, reads them back and uploads the table.
     const int64_t ne0 = dst->ne[0], ne2 = dst->ne[2];
+    const float theta_scale = powf(p->freq_base, -2.0f / (float)p->num_dim);
+    const dim3 grid((unsigned)dst->ne[1], (unsigned)dst->ne[2], (unsigned)dst->ne[3]);
+    // The rotations of every position of the context, built once per parameter set and kept on the device: the kernel
+    // then looks its token's position up itself and the call needs no copy and no wait.
+    static struct { int64_t npos, ne0; float freq_base, freq_scale, factor; int32_t num_dim; float *dev; } cache = {0, 0, 0, 0, 0, 0, nullptr};
+    const int64_t npos = p->num_context;
+    if (npos > 0 && npos * ne0 * 4 <= (64ll << 20) && spy_hip_err_flag_ptr()) {
+        if (!cache.dev || cache.npos != npos || cache.ne0 != ne0 || cache.freq_base != p->freq_base || cache.freq_scale != p->freq_scale ||
+            cache.factor != p->attention_factor || cache.num_dim != p->num_dim) {
+            std::vector<float> tab((size_t)(npos * ne0));
+            for (int64_t q = 0; q < npos; q++) rope_row(&tab[(size_t)(q * ne0)], (int32_t)q, ne0, theta_scale, p);
+            if (cache.dev) { (void)hipDeviceSynchronize(); (void)hipFree(cache.dev); cache.dev = nullptr; }
+            hipError_t e = hipMalloc((void **)&cache.dev, tab.size() * sizeof(float));
+            if (e != hipSuccess) { cache.dev = nullptr; return (int)e; }
+            e = hipMemcpy(cache.dev, tab.data(), tab.size() * sizeof(float), hipMemcpyHostToDevice);
+            if (e != hipSuccess) return (int)e;
+            cache.npos = npos; cache.ne0 = ne0; cache.freq_base = p->freq_base; cache.freq_scale = p->freq_scale;
+            cache.factor = p->attention_factor; cache.num_dim = p->num_dim;
+        }
+        exact_rope_kernel<<<grid, dim3(64), 0, st>>>(mkx(x), mkx(dst), cache.dev, (const uint8_t *)pos->data, pos->nb[0], npos, spy_hip_err_flag_ptr());
+        return SPY_LAUNCH_RC();
+    }
+    // No context length given: wait for the stream, read the positions back and upload the rows of this call's tokens.
     hipError_t e = hipStreamSynchronize(st);
     if (e != hipSuccess) return (int)e;
     std::vector<int32_t> hp((size_t)ne2);
     if (pos->nb[0] == 4) e = hipMemcpy(hp.data(), pos->data, (size_t)ne2 * 4, hipMemcpyDeviceToHost);
     else e = hipMemcpy2D(hp.data(), 4, pos->data, (size_t)pos->nb[0], 4, (size_t)ne2, hipMemcpyDeviceToHost);
     if (e != hipSuccess) return (int)e;
-    const float theta_scale = powf(p->freq_base, -2.0f / (float)p->num_dim);
     std::vector<float> tab((size_t)(ne2 * ne0));
-    for (int64_t i2 = 0; i2 < ne2; i2++) {
-        float theta = (float)hp[(size_t)i2];
-        for (int64_t i0 = 0; i0 < ne0; i0 += 2) {
-            const float ang = p->freq_scale * theta;
-            tab[(size_t)(i2 * ne0 + i0)] = cosf(ang) * p->attention_factor;
-            tab[(size_t)(i2 * ne0 + i0 + 1)] = sinf(ang) * p->attention_factor;
-            theta *= theta_scale;
-        }
-    }
+    for (int64_t i2 = 0; i2 < ne2; i2++) rope_row(&tab[(size_t)(i2 * ne0)], hp[(size_t)i2], ne0, theta_scale, p);
     const size_t need = tab.size() * sizeof(float);
     if (need > g_rope_cap) {
         if (g_rope) { (void)hipDeviceSynchronize(); (void)hipFree(g_rope); g_rope = nullptr; g_rope_cap = 0; }
@@ -422,16 +547,21 @@ int spy_exact_rope(hipStream_t st, const spy_hip_tensor *x, const spy_hip_tensor
     }
     e = hipMemcpy(g_rope, tab.data(), need, hipMemcpyHostToDevice);
     if (e != hipSuccess) return (int)e;
-    const dim3 grid((unsigned)dst->ne[1], (unsigned)dst->ne[2], (unsigned)dst->ne[3]);
-    exact_rope_kernel<<<grid, dim3(64), 0, st>>>(mkx(x), mkx(dst), g_rope);
+    exact_rope_kernel<<<grid, dim3(64), 0, st>>>(mkx(x), mkx(dst), g_rope, nullptr, 0, 0, nullptr);
     if (hipGetLastError() != hipSuccess) return SPY_HIP_EINVAL;
     return (int)hipStreamSynchronize(st);      // the table is overwritten by the next call
 }
 
 int spy_exact_dots(hipStream_t st, int t0, const spy_hip_tensor *w, const uint8_t *xm, int64_t x_row, int64_t ne11, const spy_hip_tensor *dst) {
     const int64_t total = w->ne[1] * ne11 * w->ne[2] * w->ne[3];
-    if (total <= 0 || (total + 63) / 64 >= (1ll << 31)) return SPY_HIP_EINVAL;
+    if (total <= 0 || (total + 7) / 8 >= (1ll << 31)) return SPY_HIP_EINVAL;
     const dim3 grid((unsigned)((total + 63) / 64)), block(64);
+    // SPY_HIP_EXACT_SERIAL=1: one thread per output element for every type (the plain restatement the lane forms are tested against)
+    const bool serial = getenv("SPY_HIP_EXACT_SERIAL") != nullptr;
+    const dim3 grid8((unsigned)((total + 31) / 32)), grid32((unsigned)((total + 7) / 8));
+    if (!serial && t0 == SPY_HIP_Q4_0) { exact_dots8_kernel<SPY_HIP_Q4_0><<<grid8, dim3(256), 0, st>>>(mkx(w), xm, x_row, mkx(dst), ne11, total); return SPY_LAUNCH_RC(); }
+    if (!serial && t0 == SPY_HIP_Q8_0) { exact_dots8_kernel<SPY_HIP_Q8_0><<<grid8, dim3(256), 0, st>>>(mkx(w), xm, x_row, mkx(dst), ne11, total); return SPY_LAUNCH_RC(); }
+    if (!serial && t0 == SPY_HIP_F16) { exact_dots32_kernel<<<grid32, dim3(256), 0, st>>>(mkx(w), xm, x_row, mkx(dst), ne11, total); return SPY_LAUNCH_RC(); }
     switch (t0) {
     case SPY_HIP_Q4_0: exact_dots_kernel<SPY_HIP_Q4_0><<<grid, block, 0, st>>>(mkx(w), xm, x_row, mkx(dst), ne11, total); break;
     case SPY_HIP_Q8_0: exact_dots_kernel<SPY_HIP_Q8_0><<<grid, block, 0, st>>>(mkx(w), xm, x_row, mkx(dst), ne11, total); break;

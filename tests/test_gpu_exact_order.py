@@ -35,8 +35,13 @@ def _same_bits(got, want, what):
 
 @pytest.mark.parametrize("wtype", [O.Q4_0, O.Q8_0, O.Q4_K, O.Q6_K])
 @pytest.mark.parametrize("M,K,T", [(96, 4096, 5), (40, 11008, 1), (33, 256, 3)])
-def test_quantized_matmul_bits(hip, oracle, wtype, M, K, T):
+@pytest.mark.parametrize("serial", [False, True])
+def test_quantized_matmul_bits(hip, oracle, wtype, M, K, T, serial, monkeypatch):
+    """serial: one thread per output element (the plain restatement); otherwise the eight accumulators of an
+    output element in eight lanes (Q4_0 / Q8_0).  Both must give the oracle's bits."""
     from tests.gpu_util import dev, dev_empty, call
+    if serial:
+        monkeypatch.setenv("SPY_HIP_EXACT_SERIAL", "1")
     if K % 256 and wtype in (O.Q4_K, O.Q6_K):
         pytest.skip("K-quant rows are whole super-blocks")
     rng = np.random.default_rng(100 * wtype + K + T)
@@ -74,10 +79,13 @@ def test_q8_0_weights_of_any_byte(hip, oracle):
 
 
 @pytest.mark.parametrize("n_kv", [1, 31, 32, 33, 64, 65, 300, 4241])
-def test_attention_products_bits(hip, oracle, n_kv):
+@pytest.mark.parametrize("serial", [False, True])
+def test_attention_products_bits(hip, oracle, n_kv, serial, monkeypatch):
     """attn_score (contraction over 128) and KQV (contraction over n_kv: the strict `i + 32 < n` loop bound
     and the scalar tail of Dot<FP16,FP16>, vec_dot.h:124-145) through the cache views."""
     from tests.gpu_util import dev, dev_empty, call
+    if serial:
+        monkeypatch.setenv("SPY_HIP_EXACT_SERIAL", "1")
     rng = np.random.default_rng(9 + n_kv)
     hd, H_, T = 128, 4, 2
     Cx = n_kv + 11
@@ -149,9 +157,17 @@ def test_norm_softmax_silu_rope_bits(hip, oracle):
     rp = O.default_rope(hd, 4352)
     assert oracle.spy_o_rope(B(O.tensor(x, O.F32, [hd, H_, T])), B(O.tensor(pos, O.I32, [T])), B(O.tensor(want, O.F32, [hd, H_, T])), B(rp)) == 0
     dx, dp, dy = dev(x), dev(pos), dev_empty(x.nbytes, 0xFF)
-    hp = hip.RopeParam(0, 0, hd, 4352, 4352, 10000.0, 1.0, 0.0, 1.0, 32.0, 1.0, 0.0, 0)
+    # with a context length: one table of all positions kept on the device; without: the positions read back per call
+    for n_ctx in (4352, 0):
+        hp = hip.RopeParam(0, 0, hd, n_ctx, 4352, 10000.0, 1.0, 0.0, 1.0, 32.0, 1.0, 0.0, 0)
+        dy = dev_empty(x.nbytes, 0xFF)
+        call(L.spy_hip_op_rope, None, B(hip.tensor(dx, hip.F32, [hd, H_, T])), B(hip.tensor(dp, hip.I32, [T])), B(hip.tensor(dy, hip.F32, [hd, H_, T])), B(hp))
+        _same_bits(dy.download(np.float32).reshape(x.shape), want, "rope, context %d" % n_ctx)
+    flag = C.c_int32(-1)
+    call(L.spy_hip_take_error, C.byref(flag)); assert flag.value == 0
+    hp = hip.RopeParam(0, 0, hd, 4096, 4096, 10000.0, 1.0, 0.0, 1.0, 32.0, 1.0, 0.0, 0)       # position 4351 lies beyond this context
     call(L.spy_hip_op_rope, None, B(hip.tensor(dx, hip.F32, [hd, H_, T])), B(hip.tensor(dp, hip.I32, [T])), B(hip.tensor(dy, hip.F32, [hd, H_, T])), B(hp))
-    _same_bits(dy.download(np.float32).reshape(x.shape), want, "rope")
+    call(L.spy_hip_take_error, C.byref(flag)); assert flag.value == 1
 
 
 def test_switch_returns_previous_setting_and_default_is_off():
