@@ -113,9 +113,11 @@ int spy_hip_take_error(int *flag);   /* reads and clears the device error flag (
  * Dot<Q8_0,Q8_0> and Dot<FP16,FP16> (vec_dot.h:42-146, vec_util.h:75-81), libstdc++'s four-way std::reduce in
  * NormRMS and Softmax (non-linear.cpp:129-223) -- and take exp / silu from tables and the Rope angles from the
  * host's libm (lookup_table_impl/non-linear.h:39-47,131-139, non-linear.cpp:270-371), so that every operator
- * output equals the host backend's bit for bit.  A checking mode, far slower than the default kernels; Rope
- * synchronises the stream.  The fused token loop (spy_hip_llama_*) only follows it where it runs operator by
- * operator (prompt passes below 16 tokens). */
+ * output equals the host backend's bit for bit.  A checking mode, about 12 x slower than the fused token
+ * loop.  spy_hip_llama_forward / _forward_last / _decode_greedy follow it: every pass runs operator by operator
+ * (the prompt as one pass, the greedy loop with the argmax on the host).  With RopeParam::num_context > 0 the
+ * rotations of all positions are kept in a device table and a position outside it raises the error flag of
+ * spy_hip_take_error; with num_context == 0 Rope reads the positions back and synchronises the stream. */
 int spy_hip_set_exact_order(int on);
 /* Greedy sampling -- SamplerImpl<Greedy>::sample (model/include/llm/sampler/greedy.h:20-25):
  * index of the FIRST maximum of n logits, written to *out_index (device int32) */
