@@ -18,6 +18,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK = 8.0e12          # MI355X HBM3E, bytes/s
+INT8_PEAK = 5.0e15         # MI355X dense int8 MFMA, op/s
 
 
 def log(*a):
@@ -41,6 +42,7 @@ def main():
                     help="--model q4_0 only: output head in Q6_K (the named configuration; default) or in the body's Q4_0 (the variant Spy's CPU backend can run)")
     ap.add_argument("--via-gguf", metavar="PATH", default=None,
                     help="write the synthetic model to PATH as a GGUF file and run the model loaded from it (file -> HBM times are reported)")
+    ap.add_argument("--no-gemm", action="store_true", help="skip the timing of the prompt's quantized GEMM")
     ap.add_argument("--no-graph", action="store_true", help="launch the kernels of every pass one by one instead of replaying a HIP graph (for profilers)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch a plain copy kernel over 256 MiB three times (a known-size dispatch to scale profiler byte counters by)")
@@ -168,6 +170,52 @@ def main():
     roofline = roof(dom)
     roofline_others = {k: roof(k) for k in per_kernel if k != dom}
 
+    # The prompt's dominant kernels against the int8 matrix-core peak: the seven quantized GEMMs of one layer
+    # (wq, wk, wv, wo: 4096 x 4096; gate, up: 11008 x 4096; down: 4096 x 11008) over the 2048 activation rows of a
+    # prompt chunk, HIP events around 4 back-to-back sets.  K-quant bodies have no quantizer in this package: random blocks.
+    gemm_roofline = None
+    if not args.no_gemm:
+        wt_g, Tg = cfg.wtype, 2048
+        d_, F_ = cfg.n_embd, cfg.n_ff
+        L = H.load()
+
+        def wdev(Mg, Kg):
+            wb = M.synth_tensor(wt_g, 7, "bench.gemm.%d.%d" % (Mg, Kg), Mg * Kg) if wt_g in (H.Q4_0, H.Q8_0) else M.random_k_blocks(np.empty(Mg * Kg, np.float32), wt_g)
+            return H.DeviceBuffer.from_numpy(wb)
+
+        def xdev(Kg):
+            xf = H.DeviceBuffer.from_numpy(np.random.default_rng(Kg).standard_normal((Tg, Kg)).astype(np.float32))
+            xq_ = H.DeviceBuffer(Tg * (Kg // 32) * 34)
+            H.check(L.spy_hip_quantize_q8_0(None, xf.ptr, Kg, xq_.ptr, Tg, Kg), "spy_hip_quantize_q8_0")
+            H.sync()
+            xf.free()
+            return xq_
+        w_dd, w_Fd, w_dF, x_d, x_F = wdev(d_, d_), wdev(F_, d_), wdev(d_, F_), xdev(d_), xdev(F_)
+        og = H.DeviceBuffer(Tg * F_ * 4)
+        layer_set = [(w_dd, x_d, d_, d_)] * 4 + [(w_Fd, x_d, F_, d_)] * 2 + [(w_dF, x_F, d_, F_)]
+        e0, e1, ms = C.c_void_p(), C.c_void_p(), C.c_float()
+        H.check(L.spy_hip_event_create(C.byref(e0)), "event")
+        H.check(L.spy_hip_event_create(C.byref(e1)), "event")
+        n_set = 4
+        for timed in (False, True):
+            H.check(L.spy_hip_event_record(e0, None), "record")
+            for i in range(n_set):
+                for (wb_, xb_, Mg, Kg) in layer_set:
+                    H.check(L.spy_hip_gemm_q8_0act(None, wt_g, wb_.ptr, xb_.ptr, og.ptr, Mg, Kg, Tg, Mg), "spy_hip_gemm_q8_0act")
+            H.check(L.spy_hip_event_record(e1, None), "record")
+            H.sync()
+        H.check(L.spy_hip_event_elapsed_ms(e0, e1, C.byref(ms)), "elapsed")
+        us_set = ms.value * 1000.0 / n_set
+        ops_set = 2.0 * Tg * (4 * d_ * d_ + 3 * d_ * F_)
+        tops = ops_set / us_set / 1e6
+        gemm_roofline = {"kernel": "quantized GEMMs of one layer (%s weights x Q8_0 activations, int8 MFMA, per-block scales): 4 x %dx%d, 2 x %dx%d, 1 x %dx%d, %d activation rows"
+                                   % ({H.Q4_0: "Q4_0", H.Q8_0: "Q8_0", H.Q4_K: "Q4_K", H.Q6_K: "Q6_K"}[wt_g], d_, d_, F_, d_, d_, F_, Tg),
+                         "bound": "mfma", "achieved": round(tops, 1), "peak": INT8_PEAK / 1e12, "unit": "TOP/s", "frac": round(tops * 1e12 / INT8_PEAK, 4),
+                         "ops_per_set": ops_set, "us_per_set": round(us_set, 1)}
+        log("prompt GEMMs of a layer, T = %d: %.1f us, %.0f TOP/s (%.1f%% of the int8 MFMA peak)" % (Tg, us_set, tops, 100 * tops * 1e12 / INT8_PEAK))
+        for b in (w_dd, w_Fd, w_dF, x_d, x_F, og):
+            b.free()
+
     cpu = None
     if not args.no_cpu:
         from tests import oracle_lib as O            # the checker, timed as the CPU baseline
@@ -201,7 +249,7 @@ def main():
         "hbm_roofline_frac": round(frac, 4), "ms_per_step_hip_events": round(ev_ms, 4),
         "prefill": {"tokens": fill, "seconds": round(prefill_s, 3), "tok_s": round(fill / prefill_s, 1)} if args.prefill == "real" else None,
         "kernel_us": {k: round(v, 2) for k, v in per_kernel.items()},
-        "roofline": roofline, "roofline_other_kernels": roofline_others, "cpu_baseline": cpu,
+        "roofline": roofline, "roofline_other_kernels": roofline_others, "prompt_gemm_roofline": gemm_roofline, "cpu_baseline": cpu,
     }
     if load_info:
         out["gguf_load"] = load_info
