@@ -453,6 +453,62 @@ __global__ __launch_bounds__(256) void exact_dots8_kernel(xdesc w, const uint8_t
     if (l == 0) *(float *)xat(d, i01, i11, i02, i03) = acc;
 }
 
+// K-quant rows with the eight sub-blocks (Q4_K) or Q8_0 blocks (Q6_K) of a super-block in eight lanes: lane j forms
+// the integer sums and the fp32 term of its part, then every lane walks the ONE accumulator of the project's order
+// through the eight terms in turn (terms broadcast from their lanes), so all eight lanes hold the same sum.
+template <int WT>
+__global__ __launch_bounds__(256) void exact_dotsk_kernel(xdesc w, const uint8_t *__restrict__ xm, int64_t x_row, xdesc d, int64_t ne11, int64_t total) {
+    const int64_t o = (int64_t)blockIdx.x * 32 + (threadIdx.x >> 3);
+    if (o >= total) return;                       // whole groups of eight lanes leave together
+    const int j = threadIdx.x & 7;
+    const int64_t ne00 = w.ne[0], ne01 = w.ne[1], ne02 = w.ne[2];
+    const int64_t i01 = o % ne01, i11 = o / ne01 % ne11, i02 = o / (ne01 * ne11) % ne02, i03 = o / (ne01 * ne11 * ne02);
+    const uint8_t *wr = xat(w, 0, i01, i02, i03);
+    const blk_q8_0 *x = (const blk_q8_0 *)(xm + ((i03 * ne02 + i02) * ne11 + i11) * x_row);
+    float acc = 0.0f;
+    for (int64_t b = 0; b < ne00 / 256; b++) {
+        const blk_q8_0 *xb = &x[b * 8 + j];
+        float scale, term;                        // acc = fma(scale, term, acc), part after part
+        if (WT == SPY_HIP_Q4_K) {
+            const blk_q4_k *wb = (const blk_q4_k *)wr + b;
+            const float dw = h2f_tab(wb->d), dmin = h2f_tab(wb->dmin);
+            const uint8_t *s = wb->scales;
+            int32_t sc, m;
+            if (j < 4) { sc = s[j] & 63; m = s[j + 4] & 63; }
+            else { sc = (s[j + 4] & 0x0F) | ((s[j - 4] >> 6) << 4); m = (s[j + 4] >> 4) | ((s[j] >> 6) << 4); }
+            int32_t isum = 0, bsum = 0;
+#pragma unroll 8
+            for (int l = 0; l < 32; l++) {
+                const uint8_t byte = wb->qs[32 * (j / 2) + l];
+                const int32_t q = (j & 1) ? (byte >> 4) : (byte & 0x0F);
+                const int32_t xq = xb->qs[l];
+                isum += q * xq;
+                bsum += xq;
+            }
+            const float pos = dw * (float)(sc * isum), neg = dmin * (float)(m * bsum);
+            scale = h2f_tab(xb->d);
+            term = pos - neg;
+        } else {
+            const blk_q6_k *wb = (const blk_q6_k *)wr + b;
+            int32_t sv = 0;
+            for (int h = 0; h < 2; h++) {
+                int32_t isum = 0;
+#pragma unroll 8
+                for (int l = 0; l < 16; l++) isum += q6k_get(wb, 32 * j + 16 * h + l) * (int32_t)xb->qs[16 * h + l];
+                sv += (int32_t)wb->scales[2 * j + h] * isum;
+            }
+            scale = h2f_tab(xb->d) * h2f_tab(wb->d);
+            term = (float)sv;
+        }
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+            const float sc_t = __shfl(scale, (threadIdx.x & 56) | t, SPY_WAVE), te_t = __shfl(term, (threadIdx.x & 56) | t, SPY_WAVE);
+            acc = fmaf(sc_t, te_t, acc);
+        }
+    }
+    if (j == 0) *(float *)xat(d, i01, i11, i02, i03) = acc;
+}
+
 // Dot<FP16,FP16> with its 4 x 8 accumulators in 32 lanes: lane 8j + l keeps accumulator l of vector j.
 __global__ __launch_bounds__(256) void exact_dots32_kernel(xdesc w, const uint8_t *__restrict__ xm, int64_t x_row, xdesc d, int64_t ne11, int64_t total) {
     const int64_t o = (int64_t)blockIdx.x * 8 + (threadIdx.x >> 5);
@@ -586,6 +642,8 @@ int spy_exact_dots(hipStream_t st, int t0, const spy_hip_tensor *w, const uint8_
     const dim3 grid8((unsigned)((total + 31) / 32)), grid32((unsigned)((total + 7) / 8));
     if (!serial && t0 == SPY_HIP_Q4_0) { exact_dots8_kernel<SPY_HIP_Q4_0><<<grid8, dim3(256), 0, st>>>(mkx(w), xm, x_row, mkx(dst), ne11, total); return SPY_LAUNCH_RC(); }
     if (!serial && t0 == SPY_HIP_Q8_0) { exact_dots8_kernel<SPY_HIP_Q8_0><<<grid8, dim3(256), 0, st>>>(mkx(w), xm, x_row, mkx(dst), ne11, total); return SPY_LAUNCH_RC(); }
+    if (!serial && t0 == SPY_HIP_Q4_K) { exact_dotsk_kernel<SPY_HIP_Q4_K><<<grid8, dim3(256), 0, st>>>(mkx(w), xm, x_row, mkx(dst), ne11, total); return SPY_LAUNCH_RC(); }
+    if (!serial && t0 == SPY_HIP_Q6_K) { exact_dotsk_kernel<SPY_HIP_Q6_K><<<grid8, dim3(256), 0, st>>>(mkx(w), xm, x_row, mkx(dst), ne11, total); return SPY_LAUNCH_RC(); }
     if (!serial && t0 == SPY_HIP_F16) { exact_dots32_kernel<<<grid32, dim3(256), 0, st>>>(mkx(w), xm, x_row, mkx(dst), ne11, total); return SPY_LAUNCH_RC(); }
     switch (t0) {
     case SPY_HIP_Q4_0: exact_dots_kernel<SPY_HIP_Q4_0><<<grid, block, 0, st>>>(mkx(w), xm, x_row, mkx(dst), ne11, total); break;
