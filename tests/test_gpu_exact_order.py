@@ -231,15 +231,16 @@ def test_engine_follows_the_switch(hip, n_prompt):
 
 
 @pytest.mark.timeout(900)
-def test_llama2_7b_q4_0_greedy_32_tokens_identical():
-    """The 7B shape, Q4_0, 8 random prompt tokens, 32 greedy steps through Backend::submit in exact order:
+@pytest.mark.parametrize("wtype", [O.Q4_0, O.Q8_0])
+def test_llama2_7b_greedy_32_tokens_identical(wtype):
+    """The 7B shape, Q4_0 or Q8_0, 8 random prompt tokens, 32 greedy steps through Backend::submit in exact order:
     the 32 tokens are the CPU oracle's, and so are the bits of every pass's logits."""
     from spy_amd import _lib as H
     from spy_amd import backend_driver as BD
     from spy_amd import model as M
     from tests.model_util import OracleModel
     H.init(0)
-    cfg = M.Config.llama2_7b(n_ctx=48, wtype=O.Q4_0)
+    cfg = M.Config.llama2_7b(n_ctx=48, wtype=wtype)
     tensors = M.synth_model(cfg, seed=1234)
     ora = OracleModel(cfg, tensors, nthread=min(16, os.cpu_count() or 8))
     prompt = np.random.default_rng(5).integers(0, cfg.n_vocab, 8).astype(np.int32)
