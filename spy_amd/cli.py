@@ -15,9 +15,14 @@ def main(argv=None):
     ap.add_argument("-p", "--prompt", default="Once upon a time")
     ap.add_argument("-n", "--n-predict", type=int, default=32)
     ap.add_argument("-c", "--ctx", type=int, default=0, help="context to allocate (0: the file's context_length)")
+    ap.add_argument("--exact", action="store_true",
+                    help="exact-order mode: every float sum in the order of Spy's host backend, so that logits and tokens are the CPU backend's bit for bit (slow)")
     args = ap.parse_args(argv)
     from . import gguf as G
     import numpy as np
+    if args.exact:
+        from . import _lib
+        _lib.load().spy_hip_set_exact_order(1)
     m = G.GGUFModel(args.model, n_ctx=args.ctx)
     print("loaded %.2f GB: parse %.1f ms, upload %.0f ms, set-up %.0f ms" % (m.weight_bytes / 1e9, m.parse_ms, m.upload_ms, m.create_ms), file=sys.stderr)
     ids = m.vocab.tokenize(args.prompt, add_bos=True, special=False)

@@ -245,6 +245,8 @@ class GGUFModel:
     def vocab(self):
         """SentencePiece vocabulary of the file (built on first use)."""
         if getattr(self, "_vocab", None) is None:
+            if not getattr(self, "h", None):
+                raise RuntimeError("the model has been closed")
             self._vocab = Vocab(self.file)
         return self._vocab
 

@@ -75,7 +75,17 @@ def test_text_in_text_out(tmp_path, capsys):
     want = direct.generate(np.asarray(ids, np.int32), 8)
     assert new == [int(t) for t in want] and text == m.vocab.detokenize(new)
     direct.close()
+    from tests.model_util import OracleModel
+    text_cpu = m.vocab.detokenize([int(t) for t in OracleModel(cfg, tensors).generate(np.asarray(ids, np.int32), 8)])
     m.close()
     cli.main([path, "-p", "the cat sat", "-n", "8"])
     out = capsys.readouterr()
     assert out.out == "the cat sat" + text.decode("utf-8", "replace") + "\n" and "generation: 8 tokens" in out.err
+    # --exact: the same file through the exact-order operators gives the CPU oracle's tokens
+    from spy_amd import _lib as H
+    try:
+        cli.main([path, "-p", "the cat sat", "-n", "8", "--exact"])
+    finally:
+        H.load().spy_hip_set_exact_order(0)
+    out = capsys.readouterr()
+    assert out.out == "the cat sat" + text_cpu.decode("utf-8", "replace") + "\n"
