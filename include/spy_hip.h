@@ -32,6 +32,7 @@ extern "C" {
 #define SPY_HIP_EUNSUPPORTED (-1) /* OperatorStatus::Unsupport (backend.h:22-29) */
 #define SPY_HIP_EINVAL       (-2) /* shape / argument check failed (spy_assert in the reference) */
 #define SPY_HIP_ENOSPACE     (-3) /* caller-provided scratch too small */
+#define SPY_HIP_ETIMEOUT     (-4) /* a bounded wait between workgroups of a fused launch expired: the pass's results are void */
 
 /* NumberType ids (orchestration/include/number/number_impl/type.h:12-45) */
 enum spy_hip_type {
@@ -214,6 +215,10 @@ int spy_hip_llama_forward_last(spy_hip_llama *m, void *stream, const int32_t *to
  * receives the token sampled by step i.  use_graph: replay a captured HIP graph. */
 int spy_hip_llama_decode_greedy(spy_hip_llama *m, void *stream, int32_t first_token, int32_t n_past, int32_t n_steps,
                                 int32_t *tokens_host, int32_t use_graph);
+/* Polls a bounded wait between the workgroups of a fused launch may spend before it gives up (default 400000, about
+ * half a second).  On expiry every workgroup still runs to its end, the pass returns SPY_HIP_ETIMEOUT and the hand-over
+ * words are cleared, so the next pass is a clean one.  Captured graphs are dropped (they carry the old limit). */
+int spy_hip_llama_set_spin_limit(spy_hip_llama *m, uint32_t polls);
 /* device pointers of the engine's buffers, for tests and profiling: name one of "k_cache",
  * "v_cache" (layer 0..n_layer-1), "x", "logits", "scores", "attn_out" (layer ignored) */
 int spy_hip_llama_buffer(spy_hip_llama *m, const char *name, int32_t layer, void **ptr, size_t *bytes);
@@ -228,8 +233,7 @@ int spy_hip_llama_kernel_time(spy_hip_llama *m, void *stream, const char *which,
  * bit 1 (value 2): the attention part of a layer (qkv, scores, softmax + KQV) is ONE launch whose
  *   workgroups synchronise head by head; used where all its workgroups are resident (128-wide heads,
  *   8 * n_head <= compute units, n_ctx <= 5120) unless SPY_HIP_ATTN_SPLIT=1 was set at creation.
- * bit 0 (value 1): the whole pass is ONE persistent kernel with grid barriers between the phases;
- *   opt-in with SPY_HIP_MEGA=1 at creation (slower than the per-phase kernels so far). */
+ * bit 0 is reserved (always 0). */
 int spy_hip_llama_single_kernel(spy_hip_llama *m);
 
 #ifdef __cplusplus

@@ -15,7 +15,7 @@ F32, F16, Q4_0, Q8_0, Q4_K, Q6_K, I32 = 0, 1, 2, 8, 12, 14, 26
 TYPE_SIZE = {F32: 4, F16: 2, Q4_0: 18, Q8_0: 34, Q4_K: 144, Q6_K: 210, I32: 4}
 BLOCK_SIZE = {F32: 1, F16: 1, Q4_0: 32, Q8_0: 32, Q4_K: 256, Q6_K: 256, I32: 1}
 
-EUNSUPPORTED, EINVAL, ENOSPACE = -1, -2, -3
+EUNSUPPORTED, EINVAL, ENOSPACE, ETIMEOUT = -1, -2, -3, -4
 
 
 def row_size(t, n):
@@ -102,6 +102,7 @@ SIGNATURES = {
     "spy_hip_llama_forward": (_i32, [_vp, _vp, _vp, _i32, _i32, _vp]),
     "spy_hip_llama_forward_last": (_i32, [_vp, _vp, _vp, _i32, _i32, _vp]),
     "spy_hip_llama_decode_greedy": (_i32, [_vp, _vp, _i32, _i32, _i32, _vp, _i32]),
+    "spy_hip_llama_set_spin_limit": (_i32, [_vp, C.c_uint32]),
     "spy_hip_llama_buffer": (_i32, [_vp, C.c_char_p, _i32, C.POINTER(_vp), C.POINTER(_sz)]),
     "spy_hip_llama_timing": (_i32, [_vp, C.POINTER(_f32), C.POINTER(_i32)]),
     "spy_hip_llama_single_kernel": (_i32, [_vp]),

@@ -160,7 +160,14 @@ int parse(spy_gguf *g) {
         t.n_dim = (int32_t)c.get<uint32_t>();
         if (!c.ok || t.n_dim < 1 || t.n_dim > 4) return fail(SPY_GGUF_EFORMAT, "tensor %s: %d dimensions", t.name.c_str(), t.n_dim);
         uint64_t elems = 1;
-        for (int d = 0; d < t.n_dim; d++) { t.ne[d] = (int64_t)c.get<uint64_t>(); elems *= (uint64_t)t.ne[d]; }
+        bool overflow = false;
+        for (int d = 0; d < t.n_dim; d++) {
+            const uint64_t e = c.get<uint64_t>();
+            t.ne[d] = (int64_t)e;
+            if (e > (uint64_t)INT64_MAX || (e != 0 && elems > UINT64_MAX / e)) overflow = true;       // a crafted shape must not wrap the product
+            else elems *= e;
+        }
+        if (overflow) return fail(SPY_GGUF_EFORMAT, "tensor %s: shape overflows 64 bits", t.name.c_str());
         t.type = (int32_t)c.get<uint32_t>();
         t.offset = c.get<uint64_t>();
         if (!c.ok) return fail(SPY_GGUF_EFORMAT, "truncated tensor infos");
@@ -168,6 +175,7 @@ int parse(spy_gguf *g) {
         if (!type_layout(t.type, bb, be)) return fail(SPY_GGUF_EUNSUPPORTED, "tensor %s: type %d is not one this backend stores", t.name.c_str(), t.type);
         if (elems % be != 0) return fail(SPY_GGUF_EFORMAT, "tensor %s: number of elements (%llu) is not a multiple of the block size (%llu)",
                                          t.name.c_str(), (unsigned long long)elems, (unsigned long long)be);
+        if (elems / be > UINT64_MAX / bb) return fail(SPY_GGUF_EFORMAT, "tensor %s: size overflows 64 bits", t.name.c_str());
         t.nbytes = elems / be * bb;
         g->by_name[t.name] = i;
     }
@@ -179,12 +187,15 @@ int parse(spy_gguf *g) {
     }
     const uint64_t pos = (uint64_t)(c.p - g->base);
     g->data_offset = (pos + g->alignment - 1) / g->alignment * g->alignment;
+    if (g->data_offset > g->size) return fail(SPY_GGUF_EFORMAT, "the tensor data would start beyond the file");
+    const uint64_t room = g->size - g->data_offset;                  // bytes of the data section
     for (const TensorInfo &t : g->tensors) {
-        g->data_bytes += (t.nbytes + g->alignment - 1) / g->alignment * g->alignment;
         if (t.offset % g->alignment != 0) return fail(SPY_GGUF_EFORMAT, "tensor %s: offset %llu is not aligned to %u", t.name.c_str(), (unsigned long long)t.offset, g->alignment);
-        if (g->data_offset + t.offset + t.nbytes > g->size)
+        // subtraction form: none of these can wrap, whatever the file says
+        if (t.offset > room || t.nbytes > room - t.offset)
             return fail(SPY_GGUF_EFORMAT, "tensor %s: data (%llu bytes at %llu) ends beyond the file", t.name.c_str(), (unsigned long long)t.nbytes,
-                        (unsigned long long)(g->data_offset + t.offset));
+                        (unsigned long long)t.offset);
+        g->data_bytes += (t.nbytes + g->alignment - 1) / g->alignment * g->alignment;
     }
     return 0;
 }

@@ -195,13 +195,22 @@ OperatorStatus HIPBackend::run(OperatorNode *op) {
     if (out_io && type != OperatorType::Copy) {                  // e.g. the logits: host-visible before the callback
         rc = spy_hip_download(out_node->tensor.data_ptr, out.data, static_cast<size_t>(out_node->tensor.total_size()), stream_);
         if (rc != 0) { last_error_ = rc; return OperatorStatus::Fail; }
+        // the pass's device-side error flag (a GetRow index outside its table: the reference asserts, view.cpp:61)
+        int flag = 0;
+        rc = spy_hip_take_error(&flag);
+        if (rc != 0 || flag != 0) { last_error_ = rc != 0 ? rc : SPY_HIP_EINVAL; return OperatorStatus::Fail; }
     }
     return OperatorStatus::Success;
 }
 
 void HIPBackend::submit(OperatorNode *op_node_ptr, std::function<void()> &&callback) {
-    const OperatorStatus st = run(op_node_ptr);
-    if (st != OperatorStatus::Success) last_status_ = st;        // the CPU backend asserts here (default_backend.h:175-176)
+    {
+        // one operator at a time: run() touches the constant and staging maps and the one stream.  The callback runs
+        // outside the lock (it frees inputs through dealloc_memory and may submit successors).
+        std::lock_guard<std::mutex> lock(submit_mutex_);
+        const OperatorStatus st = run(op_node_ptr);
+        if (st != OperatorStatus::Success) last_status_ = st;    // the CPU backend asserts here (default_backend.h:175-176)
+    }
     if (callback) callback();
 }
 

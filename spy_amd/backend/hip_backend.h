@@ -46,7 +46,8 @@ private:
 
     int device_id_ = 0;
     void *stream_ = nullptr;
-    std::mutex mutex_;
+    std::mutex mutex_;                                            // the memory pool
+    std::mutex submit_mutex_;                                     // run(): maps, staging buffers, stream order
     std::map<size_t, std::vector<void *>> pool_;                  // bucket size -> free blocks
     std::unordered_map<void *, size_t> bucket_of_;
     std::unordered_map<const void *, void *> constants_;          // host pointer -> device copy

@@ -10,11 +10,11 @@
 template <int WT, int LPR, int NIT, int SIT, int EPI>
 static int launch_fused(spy_hip_llama *m, hipStream_t st, const fused_args &a) {
     constexpr int RPT = GEMV_WAVES * (SPY_WAVE / LPR);
-    static int cap = 0;                                   // workgroups resident at once (persistent grid)
     const size_t lds = staged_bytes(a.K) + (EPI == EPI_QKV ? 4 * (size_t)a.hd : 0);      // + the RoPE cos|sin table
     auto kern = fused_gemv_kernel<WT, LPR, NIT, SIT, EPI>;
+    int &cap = m->grid_cap[(const void *)kern];           // workgroups resident at once (persistent grid)
     if (!cap) {
-        if (lds > 48 * 1024) HIP_TRY(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        RC_TRY(spy_ensure_lds(m, (const void *)kern, lds));
         int per_cu = 0;
         if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, GEMV_THREADS, lds) != hipSuccess || per_cu < 1) per_cu = 1;
         cap = per_cu * m->num_cu;
@@ -58,8 +58,7 @@ template <int WT, int NITK, int NR, int EPI, int WTV = WT>
 static int launch_wave(spy_hip_llama *m, hipStream_t st, const fused_args &a) {
     const size_t lds = staged_bytes(a.K) + (EPI == EPI_QKV ? 4 * (size_t)a.hd : 0);
     auto kern = wave_gemv_kernel<WT, NITK, NR, EPI, WTV>;
-    static size_t lds_set = 0;
-    if (lds > 48 * 1024 && lds > lds_set) { HIP_TRY(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); lds_set = lds; }
+    RC_TRY(spy_ensure_lds(m, (const void *)kern, lds));
     if (m->dry) return 0;
     const int units = EPI == EPI_QKV ? a.d : (EPI == EPI_GATEUP ? a.M / 2 : a.M);       // one per wave and step
     const int grid = (units + WGV_WAVES * NR - 1) / (WGV_WAVES * NR);
@@ -97,9 +96,8 @@ static int launch_attn_layer_tv(spy_hip_llama *m, hipStream_t st, int il, bool p
     const spy_hip_llama_layer &L = m->layers[il];
     const size_t lds = staged_bytes(c.n_embd) + 512 + (size_t)ATL_WAVES * 4 * ATL_RS * 4 + (size_t)c.n_ctx * 6 + 16;
     auto kern = attn_layer_kernel<WT, WTV>;
-    static size_t lds_set = 0;
-    if (probe || lds > lds_set) {
-        if (lds > 48 * 1024 && lds > lds_set) { HIP_TRY(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); lds_set = lds; }
+    if (probe || lds > m->lds_set[(const void *)kern]) {
+        RC_TRY(spy_ensure_lds(m, (const void *)kern, lds));
         int per_cu = 0;
         if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, ATL_THREADS, lds) != hipSuccess) per_cu = 0;
         if (per_cu * m->num_cu < c.n_head * ATL_GPH) return SPY_HIP_EUNSUPPORTED;        // the head barriers need every workgroup resident
@@ -113,9 +111,9 @@ static int launch_attn_layer_tv(spy_hip_llama *m, hipStream_t st, int il, bool p
     a.scores = m->scores; a.attn_out = m->attn_out; a.sync = m->attn_sync;
     a.d = c.n_embd; a.n_head = c.n_head; a.n_ctx = c.n_ctx;
     a.scale = 1.0f / sqrtf((float)m->hd);                   // SoftmaxParam::scale (attention.cpp:113)
-    a.spin_limit = 400000;
+    a.spin_limit = m->spin_limit;
 #ifdef ATL_STAMPS
-    a.dbg = m->mega_dbg;
+    a.dbg = m->stamp_dbg;
 #endif
     kern<<<dim3((unsigned)(c.n_head * ATL_GPH)), dim3(ATL_THREADS), lds, st>>>(a);
     return SPY_LAUNCH_RC();
@@ -200,48 +198,4 @@ static int enqueue_head(spy_hip_llama *m, hipStream_t st) {
 template <int WT>
 static int enqueue_any(spy_hip_llama *m, hipStream_t st, int which, int il) {
     return which == K_HEAD ? enqueue_head<WT>(m, st) : enqueue_kernel<WT>(m, st, which, il);
-}
-
-
-// ---- the persistent single-kernel pass -----------------------------------------------------------
-template <int WT, int NITF>
-static int mega_launch_nitf(spy_hip_llama *m, hipStream_t st, bool probe, const mega_args &a, size_t lds) {
-    auto kern = mega_decode_kernel<WT, NITF>;
-    static size_t lds_set = 0;
-    if (probe || lds > lds_set) {
-        if (lds > lds_set && lds > 48 * 1024) { HIP_TRY(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); lds_set = lds; }
-        int per_cu = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, MEGA_THREADS, lds) != hipSuccess) per_cu = 0;
-        if (per_cu < 1) return SPY_HIP_EUNSUPPORTED;      // the grid barrier needs every workgroup resident
-    }
-    if (probe) return 0;
-    kern<<<dim3((unsigned)m->num_cu), dim3(MEGA_THREADS), lds, st>>>(a);
-    return SPY_LAUNCH_RC();
-}
-
-template <int WT>
-static int mega_launch(spy_hip_llama *m, hipStream_t st, bool probe) {
-    const spy_hip_llama_desc &c = m->desc;
-    const int NW = m->num_cu * MEGA_WAVES;
-    // one batch of rows per wave and phase (see the work split in mega_kernel.cuh)
-    if (m->hd != 128 || c.n_head % 4 != 0 || c.n_embd % 64 != 0 || c.n_embd > 4096 || c.n_embd > NW || c.n_ff % 64 != 0 || c.t_out != c.wtype) return SPY_HIP_EUNSUPPORTED;
-    if ((c.n_ff + NW - 1) / NW > MEGA_SLOTS || (int64_t)c.n_ctx * (c.n_head / 4) > (int64_t)MEGA_RS * NW || c.n_ctx > MEGA_RV * 512 || c.n_ctx % 8 != 0) return SPY_HIP_EUNSUPPORTED;
-    if (m->num_cu > MEGA_FAN * MEGA_MAX_LEAF) return SPY_HIP_EUNSUPPORTED;
-    mega_args a;
-    memset(&a, 0, sizeof(a));
-    a.layers = m->mega_layers; a.n_layer = c.n_layer; a.d = c.n_embd; a.F = c.n_ff; a.H = c.n_head; a.hd = m->hd; a.n_ctx = c.n_ctx; a.n_vocab = c.n_vocab;
-    a.eps = c.eps; a.theta_scale = m->theta_scale; a.att_scale = 1.0f / sqrtf((float)m->hd);       // SoftmaxParam::scale (attention.cpp:113)
-    a.tok_embd = (const uint8_t *)c.tok_embd; a.embd_q8 = c.t_tok_embd == SPY_HIP_Q8_0;
-    a.out_norm = (const float *)c.out_norm; a.w_out = (const uint8_t *)c.w_out;
-    a.st = m->st; a.sync = m->msync;
-    a.x = m->x; a.x1 = m->x1; a.attn_out = m->attn_out; a.hbuf = m->hbuf; a.scores = m->scores; a.logits = m->logits; a.q16 = m->q16;
-    a.dbg = m->mega_dbg;
-    a.spin_limit = 400000;                                 // ~0.5 s of polling before a pass gives up
-    const size_t lds = mega_lds_bytes(c.n_embd, c.n_ff, m->hd, c.n_ctx);
-    if (lds > 160 * 1024) return SPY_HIP_EUNSUPPORTED;
-    switch ((c.n_ff + 4095) / 4096) {
-    case 1: return mega_launch_nitf<WT, 1>(m, st, probe, a, lds);
-    case 3: return mega_launch_nitf<WT, 3>(m, st, probe, a, lds);
-    default: return SPY_HIP_EUNSUPPORTED;
-    }
 }

@@ -131,22 +131,9 @@ extern "C" int spy_hip_llama_create(const spy_hip_llama_desc *desc, spy_hip_llam
         }
     }
     if (!rc && fused_ok(m)) { m->dry = true; rc = enqueue_pass_any(m, m->own_stream, PASS_GREEDY); m->dry = false; }   // sizes the persistent grids
-    if (!rc && fused_ok(m)) {            // the persistent single-kernel pass: opt-in with SPY_HIP_MEGA=1 (slower than the per-phase kernels so far)
-        std::vector<mega_layer> ml(c.n_layer);
-        for (int i = 0; i < c.n_layer; i++) {
-            const spy_hip_llama_layer &L = m->layers[i];
-            ml[i] = mega_layer{(const uint8_t *)L.wq, (const uint8_t *)L.wk, (const uint8_t *)L.wv, (const uint8_t *)L.wo, (const uint8_t *)L.w_gate,
-                               (const uint8_t *)L.w_up, (const uint8_t *)L.w_down, (const float *)L.attn_norm, (const float *)L.ffn_norm,
-                               m->k_cache[i], m->v_cache[i]};
-        }
-        rc = dalloc(m, (void **)&m->mega_layers, ml.size() * sizeof(mega_layer), false);
-        if (!rc) rc = (int)hipMemcpy(m->mega_layers, ml.data(), ml.size() * sizeof(mega_layer), hipMemcpyHostToDevice);
-        if (!rc) rc = dalloc(m, (void **)&m->msync, sizeof(mega_sync), true);
-        if (!rc && getenv("SPY_HIP_MEGA_STAMPS")) rc = dalloc(m, (void **)&m->mega_dbg, (128 + 512 * 8) * sizeof(long long), true);
-        const char *env = getenv("SPY_HIP_MEGA");
-        if (!rc && env && env[0] == '1' && m->uniform)
-            m->mega = (c.wtype == SPY_HIP_Q4_0 ? spy_enqueue_mega_q4_0(m, m->own_stream, true) : spy_enqueue_mega_q8_0(m, m->own_stream, true)) == 0;
-    }
+#ifdef ATL_STAMPS
+    if (!rc && getenv("SPY_HIP_STAMPS")) rc = dalloc(m, (void **)&m->stamp_dbg, (128 + 512 * 8) * sizeof(long long), true);
+#endif
     if (rc) { spy_hip_llama_destroy(m); return rc; }
     *out = m;
     return 0;
@@ -163,14 +150,14 @@ extern "C" int spy_hip_llama_buffer(spy_hip_llama *m, const char *name, int32_t 
     else if (!strcmp(name, "logits")) { p = m->logits; n = (size_t)m->desc.n_vocab * 4; }
     else if (!strcmp(name, "scores")) { p = m->scores; n = (size_t)m->desc.n_head * C * 4; }
     else if (!strcmp(name, "attn_out")) { p = m->attn_out; n = d * 4; }
-    else if (!strcmp(name, "phase_stamps") && m->mega_dbg) { p = m->mega_dbg; n = (128 + 512 * 8) * sizeof(long long); }
+    else if (!strcmp(name, "phase_stamps") && m->stamp_dbg) { p = m->stamp_dbg; n = (128 + 512 * 8) * sizeof(long long); }
     else return SPY_HIP_EINVAL;
     *ptr = p;
     if (bytes) *bytes = n;
     return 0;
 }
 
-extern "C" int spy_hip_llama_single_kernel(spy_hip_llama *m) { return m ? ((m->mega ? 1 : 0) | (m->attn_fused ? 2 : 0)) : SPY_HIP_EINVAL; }
+extern "C" int spy_hip_llama_single_kernel(spy_hip_llama *m) { return m ? (m->attn_fused ? 2 : 0) : SPY_HIP_EINVAL; }
 
 extern "C" int spy_hip_llama_timing(spy_hip_llama *m, float *ms_per_pass, int32_t *n_pass) {
     SPY_CHECK_ARG(m);
@@ -222,6 +209,37 @@ static int enqueue_one(spy_hip_llama *m, hipStream_t st, int which, int il) {
     return SPY_HIP_EUNSUPPORTED;
 }
 
+// After a pass: the device state's error word.  1 = a token id outside the vocabulary; 2, 3 = a bounded wait between
+// workgroups expired, the pass went on with what was there and its results are void.  The head barriers' arrival counters
+// and exchange words are then in an unknown state: they are cleared (fill kernel, stream order) so that the next pass starts
+// from launch number 1 with no stale word carrying a valid-looking number.
+__global__ __launch_bounds__(256) void fill_words_kernel(uint32_t *p, size_t n) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) p[i] = 0u;
+}
+static int check_pass_error(spy_hip_llama *m, hipStream_t st) {
+    dev_state back;
+    HIP_TRY(hipMemcpyAsync(&back, m->st, sizeof(back), hipMemcpyDeviceToHost, st));
+    HIP_TRY(hipStreamSynchronize(st));
+    if (!back.err) return 0;
+    if (back.err != 1 && m->attn_sync) {
+        const size_t words = ((size_t)m->desc.n_head * 96 * 4 + (size_t)m->desc.n_head * 128 * 8) / 4;
+        fill_words_kernel<<<dim3((unsigned)((words + 255) / 256)), dim3(256), 0, st>>>(m->attn_sync, words);
+        HIP_TRY(hipGetLastError());
+        HIP_TRY(hipStreamSynchronize(st));
+    }
+    return back.err == 1 ? SPY_HIP_EINVAL : SPY_HIP_ETIMEOUT;
+}
+
+extern "C" int spy_hip_llama_set_spin_limit(spy_hip_llama *m, uint32_t polls) {
+    SPY_CHECK_ARG(m);
+    m->spin_limit = polls;
+    // captured graphs carry the old limit in their kernel arguments
+    if (m->graph_exec) { (void)hipGraphExecDestroy(m->graph_exec); m->graph_exec = nullptr; }
+    if (m->graph_n_exec) { (void)hipGraphExecDestroy(m->graph_n_exec); m->graph_n_exec = nullptr; }
+    return 0;
+}
+
 static int enqueue_embed(spy_hip_llama *m, hipStream_t st) {
     const spy_hip_llama_desc &c = m->desc;
     embed_kernel<<<dim3(1), dim3(256), 0, st>>>(m->st, (const uint8_t *)c.tok_embd, c.t_tok_embd == SPY_HIP_Q8_0, c.n_embd, c.n_vocab, m->x,
@@ -240,11 +258,6 @@ static int enqueue_pass_any(spy_hip_llama *m, hipStream_t st, int mode) {
                                                               m->x, m->rope_cs, m->theta_scale, m->hd);
         return SPY_LAUNCH_RC();
     };
-    if (m->mega && !m->dry) {            // the persistent kernel does its own embedding
-        RC_TRY(c.wtype == SPY_HIP_Q4_0 ? spy_enqueue_mega_q4_0(m, st, false) : spy_enqueue_mega_q8_0(m, st, false));
-        if (mode == PASS_GREEDY) RC_TRY(sample(false));
-        return 0;
-    }
     if (mode == PASS_LOGITS && !m->dry) RC_TRY(enqueue_embed(m, st));
     for (int il = 0; il < c.n_layer; il++)
         for (int k = K_QKV; k <= K_DOWN; k++) RC_TRY(enqueue_one(m, st, k, il));
@@ -477,8 +490,7 @@ static int forward_any(spy_hip_llama *m, void *stream, const int32_t *tokens_hos
         HIP_TRY(hipMemcpyAsync(m->st, &h, sizeof(h), hipMemcpyHostToDevice, st));
         RC_TRY(enqueue_pass_any(m, st, PASS_LOGITS));
         if (logits_host) HIP_TRY(hipMemcpyAsync(logits_host, m->logits, (size_t)m->desc.n_vocab * 4, hipMemcpyDeviceToHost, st));
-        HIP_TRY(hipStreamSynchronize(st));
-        return 0;
+        return check_pass_error(m, st);
     }
     // longer passes in chunks: each chunk attends to everything before it, so the result per token
     // is that of one pass over the whole prompt
@@ -553,7 +565,7 @@ extern "C" int spy_hip_llama_decode_greedy(spy_hip_llama *m, void *stream, int32
         if (e != hipSuccess) return (int)e;
         HIP_TRY(hipGraphInstantiate(&m->graph_n_exec, m->graph_n, nullptr, nullptr, 0));
     }
-    if (!m->mega) RC_TRY(enqueue_embed(m, st));              // embedding of the first token; every step prepares the next one's
+    RC_TRY(enqueue_embed(m, st));              // embedding of the first token; every step prepares the next one's
     HIP_TRY(hipEventRecord(m->ev0, st));
     for (int i = 0; i < n_steps;) {
         if (use_graph && n_steps - i >= SPY_GRAPH_STEPS) { HIP_TRY(hipGraphLaunch(m->graph_n_exec, st)); i += SPY_GRAPH_STEPS; continue; }
@@ -566,9 +578,7 @@ extern "C" int spy_hip_llama_decode_greedy(spy_hip_llama *m, void *stream, int32
     float ms = 0.0f;
     HIP_TRY(hipEventElapsedTime(&ms, m->ev0, m->ev1));
     m->timed_ms += ms; m->timed_pass += n_steps;
-    dev_state back;
-    HIP_TRY(hipMemcpy(&back, m->st, sizeof(back), hipMemcpyDeviceToHost));
-    if (back.err) return SPY_HIP_EINVAL;
+    RC_TRY(check_pass_error(m, st));
     if (tokens_host) HIP_TRY(hipMemcpy(tokens_host, m->tokens_out, (size_t)n_steps * 4, hipMemcpyDeviceToHost));
     return 0;
 }

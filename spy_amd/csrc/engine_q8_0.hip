@@ -2,5 +2,4 @@
 #include "decode_launch.cuh"
 
 int spy_enqueue_kernel_q8_0(spy_hip_llama *m, hipStream_t st, int which, int il) { return enqueue_any<SPY_HIP_Q8_0>(m, st, which, il); }
-int spy_enqueue_mega_q8_0(spy_hip_llama *m, hipStream_t st, bool probe) { return mega_launch<SPY_HIP_Q8_0>(m, st, probe); }
 int spy_probe_attn_layer_q8_0(spy_hip_llama *m, int il) { return launch_attn_layer<SPY_HIP_Q8_0>(m, nullptr, il, true); }

@@ -2,8 +2,8 @@
 #pragma once
 
 #include "decode_kernels.cuh"
-#include "mega_kernel.cuh"
 
+#include <unordered_map>
 #include <vector>
 
 #define HIP_TRY(x) do { hipError_t e_ = (x); if (e_ != hipSuccess) return (int)e_; } while (0)
@@ -36,14 +36,24 @@ struct spy_hip_llama {
     hipStream_t own_stream = nullptr;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     double timed_ms = 0.0; int timed_pass = 0;
-    // persistent single-kernel pass
-    bool mega = false;
-    mega_layer *mega_layers = nullptr;
-    mega_sync *msync = nullptr;
-    long long *mega_dbg = nullptr;
+    long long *stamp_dbg = nullptr;             // measurement builds (-DATL_STAMPS) only
+    uint32_t spin_limit = 400000;               // polls of a bounded inter-workgroup wait before a pass gives up (~0.5 s)
+    // per engine (= per device) launcher state: dynamic-LDS limit already set for a kernel, resident workgroups of a persistent grid
+    std::unordered_map<const void *, size_t> lds_set;
+    std::unordered_map<const void *, int> grid_cap;
     std::vector<void *> owned;
 };
 
+
+// raise a kernel's dynamic-LDS limit once per engine and size
+static inline int spy_ensure_lds(spy_hip_llama *m, const void *kern, size_t lds) {
+    size_t &have = m->lds_set[kern];
+    if (lds > have) {
+        if (lds > 48 * 1024) HIP_TRY(hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        have = lds;
+    }
+    return 0;
+}
 
 // shapes the one-row-per-wave kernels take
 static inline bool wave_ok(const spy_hip_llama *m) {
@@ -59,11 +69,8 @@ int spy_enqueue_kernel_q4_0(spy_hip_llama *m, hipStream_t st, int which, int il)
 int spy_enqueue_kernel_q8_0(spy_hip_llama *m, hipStream_t st, int which, int il);
 int spy_enqueue_kernel_q4_k(spy_hip_llama *m, hipStream_t st, int which, int il);
 int spy_enqueue_kernel_q6_k(spy_hip_llama *m, hipStream_t st, int which, int il);
-// The persistent kernel covering embedding .. output head of one pass.  probe: only check that the
-// kernel for this shape exists and that one workgroup per compute unit is resident.
+// probe: only check that the fused attention launch for this layer's types exists and that all its workgroups are resident
 int spy_probe_attn_layer_q4_0(spy_hip_llama *m, int il);
 int spy_probe_attn_layer_q8_0(spy_hip_llama *m, int il);
 int spy_probe_attn_layer_q4_k(spy_hip_llama *m, int il);
 int spy_probe_attn_layer_q6_k(spy_hip_llama *m, int il);
-int spy_enqueue_mega_q4_0(spy_hip_llama *m, hipStream_t st, bool probe);
-int spy_enqueue_mega_q8_0(spy_hip_llama *m, hipStream_t st, bool probe);

@@ -128,6 +128,7 @@ extern "C" const char *spy_hip_error_string(int code) {
     case SPY_HIP_EUNSUPPORTED: return "operator or type combination not supported by the hip backend";
     case SPY_HIP_EINVAL: return "invalid argument or shape";
     case SPY_HIP_ENOSPACE: return "scratch buffer too small";
+    case SPY_HIP_ETIMEOUT: return "a bounded wait between workgroups expired; the pass's results are void";
     }
     return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error";
 }

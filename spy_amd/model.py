@@ -188,9 +188,9 @@ class Engine:
                                                    out.ctypes.data, 1 if use_graph else 0), "spy_hip_llama_decode_greedy")
         return out
 
-    def uses_single_kernel(self):
-        """True when single-token passes run as one persistent kernel"""
-        return (self.L.spy_hip_llama_single_kernel(self.handle) & 1) == 1
+    def set_spin_limit(self, polls):
+        """polls a bounded wait between workgroups may spend before the pass gives up (ETIMEOUT)"""
+        H.check(self.L.spy_hip_llama_set_spin_limit(self.handle, int(polls)), "spy_hip_llama_set_spin_limit")
 
     def fuses_attention(self):
         """True when qkv, scores and softmax + KQV of a layer run as one launch"""

@@ -16,3 +16,10 @@ def pytest_configure(config):
 def oracle():
     from tests import oracle_lib
     return oracle_lib.load()
+
+
+@pytest.fixture(scope="session")
+def hip():
+    from spy_amd import _lib as H
+    H.init(0)
+    return H

@@ -140,6 +140,17 @@ def test_broken_files_are_rejected_with_a_message(G, tmp_path):
     # a tensor type this backend does not store (Q5_0 = 6)
     struct.pack_into("<IQIQ", blob, i, 1, 32, 6, 0)
     expect("type.gguf", bytes(blob), G.EUNSUPPORTED, "type 6")
+    # crafted sizes that wrap 64-bit arithmetic must not pass the bounds checks: an offset near 2^64 (aligned), an element
+    # count whose byte size wraps, and a two-dimensional shape whose product wraps to a small number
+    struct.pack_into("<IQIQ", blob, i, 1, 4, H.F32, 2 ** 64 - 32)
+    expect("wrap_offset.gguf", bytes(blob), G.EFORMAT, "beyond the file")
+    struct.pack_into("<IQIQ", blob, i, 1, 2 ** 62, H.F32, 0)
+    expect("wrap_bytes.gguf", bytes(blob), G.EFORMAT, "overflows")
+    two = G.write_gguf(str(tmp_path / "two.gguf"), [], [("w", H.F32, [2, 2], np.zeros(16, np.uint8))])
+    blob2 = bytearray(open(two, "rb").read())
+    j = blob2.index(b"w") + 1
+    struct.pack_into("<IQQIQ", blob2, j, 2, 2 ** 33, 2 ** 31 + 1, H.F32, 0)      # product = 2^64 + 2^33: wraps to 2^33
+    expect("wrap_shape.gguf", bytes(blob2), G.EFORMAT, "overflows")
 
 
 def test_loader_refuses_models_it_does_not_run(G, tmp_path):
