@@ -79,6 +79,15 @@ const char *spy_hip_error_string(int code);
 size_t spy_hip_op_matmul_scratch_size(const spy_hip_tensor *w, const spy_hip_tensor *x);
 int spy_hip_op_matmul(void *stream, const spy_hip_tensor *w, const spy_hip_tensor *x, const spy_hip_tensor *dst,
                       void *scratch, size_t scratch_bytes);
+/* MatMul with no allocation anywhere -- no counterpart in the reference, whose MatMul allocates its activation buffer
+ * per node (mat.cpp:61-68).  For callers that cannot allocate: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  Same operator and same results as spy_hip_op_matmul; the converted activations go
+ * to a fixed array in device memory (spy_hip_op_matmul_noalloc_max_scratch() bytes, 8 MiB, held by every device the
+ * library runs on until the process ends) instead of a caller buffer.  Returns SPY_HIP_ENOSPACE when
+ * spy_hip_op_matmul_scratch_size(w, x) exceeds that.  All calls on a device share the array: calls that overlap on one
+ * device (different streams or threads) race. */
+size_t spy_hip_op_matmul_noalloc_max_scratch(void);
+int spy_hip_op_matmul_noalloc(void *stream, const spy_hip_tensor *w, const spy_hip_tensor *x, const spy_hip_tensor *dst);
 /* NormRMS -- OperatorNormRMSImpl::execute (non-linear.cpp:194-223); eps = NormRMSParam::eps */
 int spy_hip_op_norm_rms(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *dst, float eps);
 /* Add/Sub/Mul/Div -- binary_execution<Op> (basic.cpp:15-50); op: 0 add, 1 sub, 2 mul, 3 div */

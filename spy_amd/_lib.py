@@ -78,6 +78,8 @@ SIGNATURES = {
     "spy_hip_error_string": (C.c_char_p, [_i32]),
     "spy_hip_op_matmul_scratch_size": (_sz, [_TP, _TP]),
     "spy_hip_op_matmul": (_i32, [_vp, _TP, _TP, _TP, _vp, _sz]),
+    "spy_hip_op_matmul_noalloc_max_scratch": (_sz, []),
+    "spy_hip_op_matmul_noalloc": (_i32, [_vp, _TP, _TP, _TP]),
     "spy_hip_op_norm_rms": (_i32, [_vp, _TP, _TP, _f32]),
     "spy_hip_op_binary": (_i32, [_vp, _i32, _TP, _TP, _TP]),
     "spy_hip_op_silu": (_i32, [_vp, _TP, _TP]),

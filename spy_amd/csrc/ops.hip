@@ -635,3 +635,41 @@ static int matmul_impl(void *stream, const spy_hip_tensor *w, const spy_hip_tens
     matmul_f16_kernel<<<dim3(grid_for(total, 4)), dim3(256), 0, st>>>(mk(w), (const uint16_t *)xm, mk(dst), ne11, total);
     return SPY_LAUNCH_RC();
 }
+
+// ---- MatMul for callers that cannot allocate ---------------------------------------------------------
+// spy_hip_op_matmul takes the buffer for the converted activations (Q8_0 blocks or fp16 rows) from its caller, who has to
+// size and allocate it.  Code under HIP graph capture, tight serving loops and harnesses that forbid hipMalloc cannot:
+// for them the same operator runs with that buffer in a fixed array in device memory.  Each device that loads the library
+// holds its own copy of the array until the process ends; every call on a device shares it, so calls that overlap on one
+// device race, and a call sees the bytes the previous call left (the conversion kernels overwrite every byte the dots read).
+#define SPY_STATIC_SCRATCH_BYTES (8u << 20)      // 8 MiB: 512 activation rows of 11008 elements as Q8_0 blocks (5.6 MiB) fit
+#define SPY_STATIC_SCRATCH_MAX_DEVICES 64
+static __device__ __align__(256) uint8_t scratch[SPY_STATIC_SCRATCH_BYTES];
+static void *g_scratch_ptr[SPY_STATIC_SCRATCH_MAX_DEVICES];     // the array's device address, per device
+
+// Called by spy_hip_init with the device current (and by the entry point's first call on a device that never went through
+// it): the array's name is only a host-side handle, its address on the current device comes from the runtime.
+int spy_static_scratch_setup(int device) {
+    if (device < 0 || device >= SPY_STATIC_SCRATCH_MAX_DEVICES) return SPY_HIP_EINVAL;
+    if (g_scratch_ptr[device]) return 0;
+    void *p = nullptr;
+    const hipError_t e = hipGetSymbolAddress((void **)&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (!p) return SPY_HIP_EINVAL;
+    g_scratch_ptr[device] = p;
+    return 0;
+}
+
+extern "C" size_t spy_hip_op_matmul_noalloc_max_scratch(void) { return SPY_STATIC_SCRATCH_BYTES; }
+
+extern "C" int spy_hip_op_matmul_noalloc(void *stream, const spy_hip_tensor *w, const spy_hip_tensor *x, const spy_hip_tensor *dst) {
+    SPY_CHECK_ARG(w && x && dst);
+    int dev = -1;
+    const hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    const int rc = spy_static_scratch_setup(dev);
+    if (rc) return rc;
+    const size_t need = spy_hip_op_matmul_scratch_size(w, x);
+    if (need > SPY_STATIC_SCRATCH_BYTES) return SPY_HIP_ENOSPACE;     // the converted activations do not fit the fixed array
+    return matmul_impl(stream, w, x, dst, g_scratch_ptr[dev], SPY_STATIC_SCRATCH_BYTES, -1, -1);
+}

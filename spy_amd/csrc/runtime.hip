@@ -10,6 +10,7 @@ static int g_device = -1;
 static int *g_err_flag = nullptr;   // device int, raised by kernels that detect bad operands
 
 int *spy_hip_err_flag_ptr() { return g_err_flag; }
+int spy_static_scratch_setup(int device);    // ops.hip: address of the fixed scratch array on the current device
 
 extern "C" int spy_hip_init(int device_id) {
     int n = 0;
@@ -26,7 +27,7 @@ extern "C" int spy_hip_init(int device_id) {
         if (e != hipSuccess) return (int)e;
     }
     g_device = device_id;
-    return 0;
+    return spy_static_scratch_setup(device_id);
 }
 
 extern "C" int spy_hip_device_info(char *name, int name_len, int *num_cu, size_t *total_mem, size_t *free_mem) {
