@@ -44,6 +44,8 @@ def main():
                     help="write the synthetic model to PATH as a GGUF file and run the model loaded from it (file -> HBM times are reported)")
     ap.add_argument("--no-gemm", action="store_true", help="skip the timing of the prompt's quantized GEMM")
     ap.add_argument("--no-graph", action="store_true", help="launch the kernels of every pass one by one instead of replaying a HIP graph (for profilers)")
+    ap.add_argument("--order", type=int, choices=[0, 1], default=1,
+                    help="summation order of the single-token pass: 1 = the host backend's (greedy tokens identical to the CPU reference; default), 0 = this backend's own")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch a plain copy kernel over 256 MiB three times (a known-size dispatch to scale profiler byte counters by)")
     args = ap.parse_args()
@@ -86,6 +88,7 @@ def main():
             % (load_info["file_bytes"] / 1e9, t_write, loaded.parse_ms, loaded.upload_ms, load_info["upload_GBps"], loaded.create_ms))
     else:
         eng = M.Engine(cfg, tensors)
+    eng.set_order(args.order)
     rng = np.random.default_rng(4096)
     prompt = rng.integers(0, cfg.n_vocab, fill).astype(np.int32)
     t0 = time.time()

@@ -166,6 +166,36 @@ int spy_hip_prompt_attention(void *stream, const void *q16, const void *k_cache,
  * the last M slots receive the float results and are scratch. */
 int spy_hip_block_dots(void *stream, int wtype, const void *w, const void *xq, int32_t *out, int64_t M, int64_t K);
 
+/* ---- the kernel families of the fused single-token pass, one launch at a time.  Each runs exactly the launch the token
+ *      loop below uses for that part of a layer (same kernel, same grid), on the caller's buffers; order = 1: the host
+ *      backend's summation order (results equal to the CPU backend's bit for bit), 0: this backend's own.  K (and F) must be
+ *      multiples of 128 for order 1, rows at most 4096 elements wide for the norm prologue (16384 for the plain one). ------- */
+/* RMSNorm * weight -> Q8_0: OperatorNormRMSImpl::execute + the Mul node + Quantizator<FP32,Q8_0>::transform
+ * (non-linear.cpp:194-223, basic.cpp:15-50, vec_convert.h:178-261) as the fused kernels stage their activations;
+ * normw == NULL: the quantization alone.  yq: K/32 native Q8_0 blocks. */
+int spy_hip_rmsnorm_q8_0(void *stream, int32_t order, const float *x, const float *normw, float eps, int64_t K, void *yq);
+/* attn_norm, Q/K/V_project, 2 x Rope, the fp16 rounding of Q and both KV-cache copies of one token at position pos
+ * (attention.cpp:25-265; mat.cpp:71-146; non-linear.cpp:270-371; view.cpp:83-227): q16 = fp16[n_embd], row pos of
+ * k_cache (fp16 [n_ctx][n_embd]) and column pos of v_cache (fp16 [n_embd][n_ctx]).  rope_cs: cos, sin per pair of the
+ * position's angles (hd floats; theta_0 = pos, theta_{k+1} = theta_k * powf(base, -2/hd) in fp32).  wtype_v: type of wv
+ * (0 = wtype; Q6_K next to Q4_K).  xq_dump: NULL or K/32 Q8_0 blocks that receive the staged activations. */
+int spy_hip_rope_kvwrite(void *stream, int32_t order, int32_t wtype, int32_t wtype_v, const void *wq, const void *wk, const void *wv, const float *x,
+                         const float *normw, float eps, int32_t n_embd, int32_t n_head, int32_t pos, int64_t n_ctx, const float *rope_cs,
+                         void *q16, void *k_cache, void *v_cache, void *xq_dump);
+/* attn_score, Softmax, KQV of one token over n_kv cached tokens, all heads (MatMul(K view, q) -> Softmax(mask 0, scale
+ * 1/sqrt(128)) -> MatMul(V^T view, P); mat.cpp:71-146, vec_dot.h:117-146, non-linear.cpp:129-180): two launches (scores;
+ * softmax + P.V^T).  scores: scratch f32 [n_head][n_ctx]; out: f32 [n_head * 128]. */
+int spy_hip_attn_decode(void *stream, int32_t order, const void *q16, const void *k_cache, const void *v_cache, int32_t n_head, int32_t n_kv,
+                        int64_t n_ctx, float *scores, float *out);
+/* One matrix x vector launch with its prologue and epilogue: normw != NULL, resid == NULL: RMSNorm * weight -> Q8_0 -> M rows
+ * of w (result_norm .. output); normw == NULL, resid != NULL: Q8_0(x) -> rows of w -> + resid (KQV_linear + Add, ffn_down
+ * + Add; M % 128 == 0).  Dot<W,Q8_0>::exec per row (vec_dot.h:42-115). */
+int spy_hip_gemv_fused(void *stream, int32_t order, int32_t wtype, const void *w, const float *x, const float *normw, float eps,
+                       const float *resid, float *out, int64_t M, int64_t K, void *xq_dump);
+/* ffn_norm, ffn_gate, ffn_up, Silu, Mul (ffn.cpp:5-42; non-linear.cpp:11-14,57-77): out[i] = up_i * silu(gate_i), F values */
+int spy_hip_ffn_gate_up_silu(void *stream, int32_t order, int32_t wtype, const void *w_gate, const void *w_up, const float *x, const float *normw,
+                             float eps, float *out, int64_t F, int64_t K, void *xq_dump);
+
 /* ---- measured ceilings of the part (no counterpart in the reference; they back the roofline denominators
  *      printed by the operator sweep and are called by nothing else) ---- */
 /* int8 matrix-core rate in TOP/s (2 operations per multiply-accumulate): waves issuing only
@@ -224,6 +254,16 @@ int spy_hip_llama_forward_last(spy_hip_llama *m, void *stream, const int32_t *to
  * receives the token sampled by step i.  use_graph: replay a captured HIP graph. */
 int spy_hip_llama_decode_greedy(spy_hip_llama *m, void *stream, int32_t first_token, int32_t n_past, int32_t n_steps,
                                 int32_t *tokens_host, int32_t use_graph);
+/* Summation order of the fused single-token pass.  1 (the default wherever the kernels take the model: 128-wide heads,
+ * n_embd and n_ff multiples of 128): the host backend's -- the eight accumulators and hsum_float_8 of its quantized dots,
+ * the 4 x 8 accumulators, tree and scalar tail of its fp16 dots (vec_dot.h:42-146), libstdc++'s four-way reduce in
+ * NormRMS and Softmax (non-linear.cpp:129-223), exp / silu from the fp16-indexed tables and the RoPE angles from the
+ * host's libm -- so that logits and greedy tokens equal the CPU backend's bit for bit.  0: this backend's own order
+ * (lane-parallel sums; per-operator results equal to about 1e-7, greedy tokens of a model with near-tied logits may
+ * differ).  The environment variable SPY_HIP_ORDER=own at creation selects 0.  spy_hip_set_exact_order(1) forces 1 for
+ * every engine while it is on.  spy_hip_llama_order returns the order the next single-token pass will use. */
+int spy_hip_llama_set_order(spy_hip_llama *m, int32_t order);
+int spy_hip_llama_order(spy_hip_llama *m);
 /* Polls a bounded wait between the workgroups of a fused launch may spend before it gives up (default 400000, about
  * half a second).  On expiry every workgroup still runs to its end, the pass returns SPY_HIP_ETIMEOUT and the hand-over
  * words are cleared, so the next pass is a clean one.  Captured graphs are dropped (they carry the old limit). */

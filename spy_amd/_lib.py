@@ -97,6 +97,11 @@ SIGNATURES = {
     "spy_hip_gemm_q8_0act": (_i32, [_vp, _i32, _vp, _vp, _vp, _i64, _i64, _i64, _i64]),
     "spy_hip_prompt_attention": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i64, C.c_float]),
     "spy_hip_block_dots": (_i32, [_vp, _i32, _vp, _vp, _vp, _i64, _i64]),
+    "spy_hip_rmsnorm_q8_0": (_i32, [_vp, _i32, _vp, _vp, _f32, _i64, _vp]),
+    "spy_hip_rope_kvwrite": (_i32, [_vp, _i32, _i32, _i32, _vp, _vp, _vp, _vp, _vp, _f32, _i32, _i32, _i32, _i64, _vp, _vp, _vp, _vp, _vp]),
+    "spy_hip_attn_decode": (_i32, [_vp, _i32, _vp, _vp, _vp, _i32, _i32, _i64, _vp, _vp]),
+    "spy_hip_gemv_fused": (_i32, [_vp, _i32, _i32, _vp, _vp, _vp, _f32, _vp, _vp, _i64, _i64, _vp]),
+    "spy_hip_ffn_gate_up_silu": (_i32, [_vp, _i32, _i32, _vp, _vp, _vp, _vp, _f32, _vp, _i64, _i64, _vp]),
     "spy_hip_measure_mfma_i8": (_i32, [_vp, _i32, C.POINTER(_f32)]),
     "spy_hip_measure_hbm_read": (_i32, [_vp, _vp, _sz, _i32, C.POINTER(_f32)]),
     "spy_hip_llama_create": (_i32, [C.POINTER(LlamaDesc), C.POINTER(_vp)]),
@@ -104,6 +109,8 @@ SIGNATURES = {
     "spy_hip_llama_forward": (_i32, [_vp, _vp, _vp, _i32, _i32, _vp]),
     "spy_hip_llama_forward_last": (_i32, [_vp, _vp, _vp, _i32, _i32, _vp]),
     "spy_hip_llama_decode_greedy": (_i32, [_vp, _vp, _i32, _i32, _i32, _vp, _i32]),
+    "spy_hip_llama_set_order": (_i32, [_vp, _i32]),
+    "spy_hip_llama_order": (_i32, [_vp]),
     "spy_hip_llama_set_spin_limit": (_i32, [_vp, C.c_uint32]),
     "spy_hip_llama_buffer": (_i32, [_vp, C.c_char_p, _i32, C.POINTER(_vp), C.POINTER(_sz)]),
     "spy_hip_llama_timing": (_i32, [_vp, C.POINTER(_f32), C.POINTER(_i32)]),

@@ -79,6 +79,8 @@ struct fused_args {
     const float *resid; float *out;
     const dev_state *st; const float *rope_cs; uint16_t *q16; uint16_t *kc; uint16_t *vc;
     int n_ctx, d, hd;
+    int pos_imm;                   // st == nullptr: the position as a number (kernel-family entry points)
+    uint8_t *q8_dump;              // tests: workgroup 0 of a one-row-per-wave launch writes its staged activations here as native Q8_0 blocks
 };
 
 enum { EPI_QKV = 0, EPI_RESID = 1, EPI_GATEUP = 2, EPI_STORE = 3 };
@@ -157,6 +159,42 @@ __global__ __launch_bounds__(GEMV_THREADS) void fused_gemv_kernel(fused_args a) 
 //   EPI_RESID / EPI_STORE: wave -> NR rows r = gw + k*NW of W0
 #define WGV_THREADS 1024
 #define WGV_WAVES 16
+// Activations of a one-row-per-wave kernel: (RMSNorm * weight ->) Q8_0 in the staged LDS form, by all 1024 threads (float4
+// tid + j * 1024 each).  NormRMS (non-linear.cpp:216-219 and the separate Mul node): sums of squares per wave on DPP, the 16
+// wave sums as a tree.  Ends with __syncthreads().
+template <int NITK, bool NORM>
+static __device__ __forceinline__ void wgv_stage(const float4 (&xv)[NITK], const float4 (&wv)[NORM ? NITK : 1], int K, float eps,
+                                                 int8_t *s_q, int2 *s_meta, float *s_red) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    float scale = 1.0f;
+    if constexpr (NORM) {
+        float acc = 0.0f;
+#pragma unroll
+        for (int j = 0; j < NITK; j++) {
+            if (tid + j * WGV_THREADS < K / 4) { const float4 v = xv[j]; acc = fmaf(v.x, v.x, acc); acc = fmaf(v.y, v.y, acc); acc = fmaf(v.z, v.z, acc); acc = fmaf(v.w, v.w, acc); }
+        }
+        acc = group_sum<64>(acc);
+        if (lane == 0) s_red[wave] = acc;
+        __syncthreads();
+        const float sum = (((s_red[0] + s_red[1]) + (s_red[2] + s_red[3])) + ((s_red[4] + s_red[5]) + (s_red[6] + s_red[7]))) +
+                          (((s_red[8] + s_red[9]) + (s_red[10] + s_red[11])) + ((s_red[12] + s_red[13]) + (s_red[14] + s_red[15])));
+        scale = 1.0f / sqrtf(sum / (float)K + eps);
+    }
+#pragma unroll
+    for (int j = 0; j < NITK; j++) {
+        const int i = tid + j * WGV_THREADS;
+        if (i < K / 4) {
+            float4 v = xv[j];
+            if constexpr (NORM) { const float4 w = wv[j]; v.x = (v.x * scale) * w.x; v.y = (v.y * scale) * w.y; v.z = (v.z * scale) * w.z; v.w = (v.w * scale) * w.w; }
+            int2 meta;
+            const uint32_t q = quantize_oct(v, meta);
+            ((uint32_t *)s_q)[act_dw(i, K >> 6)] = q;
+            if ((tid & 7) == 0) s_meta[i >> 3] = meta;
+        }
+    }
+    __syncthreads();
+}
+
 #ifndef WGV_DEPTH_QKV
 #define WGV_DEPTH_QKV 2
 #endif
@@ -221,33 +259,17 @@ __global__ __launch_bounds__(WGV_THREADS) void wave_gemv_kernel(fused_args a) {
     int2 *s_meta = (int2 *)(smem + staged_q_bytes(K));
     float *s_rope = (float *)(smem + staged_bytes(K));
     if constexpr (EPI == EPI_QKV) { if (tid < a.hd) s_rope[tid] = rope_v; }
-    float scale = 1.0f;
-    if constexpr (NORM) {
-        float acc = 0.0f;
-#pragma unroll
-        for (int j = 0; j < NITK; j++) {
-            if (tid + j * WGV_THREADS < K / 4) { const float4 v = xv[j]; acc = fmaf(v.x, v.x, acc); acc = fmaf(v.y, v.y, acc); acc = fmaf(v.z, v.z, acc); acc = fmaf(v.w, v.w, acc); }
-        }
-        acc = group_sum<64>(acc);
-        if (lane == 0) s_red[wave] = acc;
-        __syncthreads();
-        const float sum = (((s_red[0] + s_red[1]) + (s_red[2] + s_red[3])) + ((s_red[4] + s_red[5]) + (s_red[6] + s_red[7]))) +
-                          (((s_red[8] + s_red[9]) + (s_red[10] + s_red[11])) + ((s_red[12] + s_red[13]) + (s_red[14] + s_red[15])));
-        scale = 1.0f / sqrtf(sum / (float)K + a.eps);
-    }
-#pragma unroll
-    for (int j = 0; j < NITK; j++) {
-        const int i = tid + j * WGV_THREADS;
-        if (i < K / 4) {
-            float4 v = xv[j];
-            if constexpr (NORM) { const float4 w = wv[j]; v.x = (v.x * scale) * w.x; v.y = (v.y * scale) * w.y; v.z = (v.z * scale) * w.z; v.w = (v.w * scale) * w.w; }
-            int2 meta;
-            const uint32_t q = quantize_oct(v, meta);
-            ((uint32_t *)s_q)[act_dw(i, K >> 6)] = q;
-            if ((tid & 7) == 0) s_meta[i >> 3] = meta;
+    wgv_stage<NITK, NORM>(xv, wv, K, a.eps, s_q, s_meta, s_red);
+    if (a.q8_dump && blockIdx.x == 0) {
+        for (int b = tid; b < K / 32; b += WGV_THREADS) {
+            uint16_t *dst = (uint16_t *)(a.q8_dump + (size_t)b * 34);
+            dst[0] = f2h(__int_as_float(s_meta[b].x));
+            for (int i = 0; i < 8; i++) {
+                const uint32_t q = ((const uint32_t *)s_q)[act_dw(b * 8 + i, K >> 6)];
+                dst[1 + 2 * i] = (uint16_t)(q & 0xFFFFu); dst[2 + 2 * i] = (uint16_t)(q >> 16);
+            }
         }
     }
-    __syncthreads();
     staged_act act; act.q = s_q; act.meta = s_meta;
     act_frag<NITK> af;                                    // this lane's activations: the same for every row
     load_act_frag<WT, NITK>(af, act, npair, lane);
@@ -269,7 +291,7 @@ __global__ __launch_bounds__(WGV_THREADS) void wave_gemv_kernel(fused_args a) {
     // 4. epilogues (lane 63 holds the totals)
     if constexpr (EPI == EPI_QKV) {
         if (lane == 63 && gw < a.d) {
-            const int j = gw, row = (2 * j) % a.d, k = (row % a.hd) >> 1, pos = a.st->pos;
+            const int j = gw, row = (2 * j) % a.d, k = (row % a.hd) >> 1, pos = a.st ? a.st->pos : a.pos_imm;
             const float c = s_rope[2 * k], sn = s_rope[2 * k + 1];
             // (x0, x1) -> (x0*c - x1*s, x0*s + x1*c) on adjacent rows (non-linear.cpp:359-363)
             const uint32_t pr = (uint32_t)f2h(s[0] * c - s[1] * sn) | ((uint32_t)f2h(s[0] * sn + s[1] * c) << 16);
@@ -652,9 +674,9 @@ __global__ __launch_bounds__(256) void embed_kernel(dev_state *st, const uint8_t
 #ifndef ATT_DEPTH
 #define ATT_DEPTH 3             // key loads per thread requested ahead of their use
 #endif
-__global__ __launch_bounds__(256) void attn_scores_kernel(const dev_state *st, const uint16_t *__restrict__ q16, const uint16_t *__restrict__ kc,
+__global__ __launch_bounds__(256) void attn_scores_kernel(const dev_state *st, int pos_imm, const uint16_t *__restrict__ q16, const uint16_t *__restrict__ kc,
                                                           float *__restrict__ scores, int n_head, int n_ctx, float scale) {
-    const int n_kv = st->pos + 1;
+    const int n_kv = (st ? st->pos : pos_imm) + 1;
     const int t0 = blockIdx.x * ATT_TCH;
     if (t0 >= n_kv) return;
     const int d = n_head * 128;
@@ -708,11 +730,11 @@ __global__ __launch_bounds__(256) void attn_scores_kernel(const dev_state *st, c
 #define PV_DEPTH 3              // pieces per wave requested ahead of their use
 #endif
 #define PV_NS 5                 // scores per thread kept in registers (5 * 1024 = 5120 tokens; more are read in a loop)
-__global__ __launch_bounds__(PV_THREADS) void attn_pv_kernel(const dev_state *st, const float *__restrict__ scores, const uint16_t *__restrict__ vc,
+__global__ __launch_bounds__(PV_THREADS) void attn_pv_kernel(const dev_state *st, int pos_imm, const float *__restrict__ scores, const uint16_t *__restrict__ vc,
                                                              float *__restrict__ attn_out, int n_ctx) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     __shared__ float s_part[16];
-    const int n_kv = st->pos + 1;
+    const int n_kv = (st ? st->pos : pos_imm) + 1;
     const int head = blockIdx.x >> 3, dgrp = blockIdx.x & 7;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int row = head * 128 + dgrp * 16 + wave;

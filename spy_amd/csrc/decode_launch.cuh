@@ -144,7 +144,7 @@ static int enqueue_kernel(spy_hip_llama *m, hipStream_t st, int which, int il) {
     fused_args a;
     memset(&a, 0, sizeof(a));
     a.st = m->st; a.rope_cs = m->rope_cs; a.q16 = m->q16; a.kc = m->k_cache[il]; a.vc = m->v_cache[il];
-    a.n_ctx = C; a.d = d; a.hd = m->hd; a.eps = c.eps;
+    a.n_ctx = C; a.d = d; a.hd = m->hd; a.eps = c.eps; a.pos_imm = m->pos_imm; a.q8_dump = m->q8_dump;
     switch (which) {
     case K_QKV:      // attn_norm, attn_norm_linear, Q/K/V_project, rope, KV-cache copies
         a.W0 = (const uint8_t *)L.wq; a.W1 = (const uint8_t *)L.wk; a.W2 = (const uint8_t *)L.wv;
@@ -179,7 +179,7 @@ static int enqueue_head(spy_hip_llama *m, hipStream_t st) {
     const int d = c.n_embd;
     fused_args a;
     memset(&a, 0, sizeof(a));
-    a.W0 = (const uint8_t *)c.w_out; a.M = c.n_vocab; a.K = d; a.x_in = m->x; a.normw = c.out_norm; a.eps = c.eps; a.out = m->logits;
+    a.W0 = (const uint8_t *)c.w_out; a.M = c.n_vocab; a.K = d; a.x_in = m->x; a.normw = c.out_norm; a.eps = c.eps; a.out = m->logits; a.q8_dump = m->q8_dump;
     if (m->wave) return launch_wave<WT, 1, wave_rows<WT>::HEAD, EPI_STORE>(m, st, a);
     if constexpr (WT == SPY_HIP_Q4_0 || WT == SPY_HIP_Q8_0) return launch_fused_norm<WT, EPI_STORE>(m, st, m->cfg_d, a);
     // no row kernel for this shape: norm + weight + Q8_0 through the operator kernels

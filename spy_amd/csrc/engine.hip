@@ -6,6 +6,7 @@
 // lists them.
 #define SPY_DECODE_COMMON_KERNELS
 #include "engine_types.cuh"
+#include "exact_decode.cuh"
 
 #include <math.h>
 #include <stdio.h>
@@ -27,6 +28,11 @@ static int probe_attn(spy_hip_llama *m, int il) {
     return SPY_HIP_EUNSUPPORTED;
 }
 enum { PASS_LOGITS = 0, PASS_GREEDY = 1 };
+int spy_exact_on();                              // exact_order.hip
+int spy_exact_luts(const float **lut);           // exact_order.hip
+// summation order of the next single-token pass: the host backend's when the engine is set to it or the library-wide
+// exact-order switch is on (and the exact kernels take the model), else this backend's own
+static int pass_order(const spy_hip_llama *m) { return (m->exact_ok && (m->order == 1 || spy_exact_on())) ? 1 : 0; }
 static int enqueue_pass_any(spy_hip_llama *m, hipStream_t st, int mode);
 
 static int dalloc(spy_hip_llama *m, void **p, size_t bytes, bool zero) {
@@ -131,6 +137,33 @@ extern "C" int spy_hip_llama_create(const spy_hip_llama_desc *desc, spy_hip_llam
         }
     }
     if (!rc && fused_ok(m)) { m->dry = true; rc = enqueue_pass_any(m, m->own_stream, PASS_GREEDY); m->dry = false; }   // sizes the persistent grids
+    // the host backend's summation order: cos / sin of every position from the host's libm (theta_0 = pos, theta_{k+1} =
+    // theta_k * theta_scale in fp32, non-linear.cpp:304-309), the exp / silu tables, shapes the kernels take
+    if (!rc && fused_ok(m) && m->wave && m->hd == 128 && c.n_embd % 128 == 0 && c.n_ff % 128 == 0 && c.n_ff <= 16384 &&
+        xattn_pv_lds(c.n_ctx) <= 160 * 1024 && xattn_scores_lds(c.n_head) <= 160 * 1024) {
+        std::vector<float> tab((size_t)c.n_ctx * m->hd);
+        for (int pos = 0; pos < c.n_ctx; pos++) {
+            float theta = (float)pos;
+            for (int i0 = 0; i0 < m->hd; i0 += 2) {
+                tab[(size_t)pos * m->hd + i0] = cosf(theta);
+                tab[(size_t)pos * m->hd + i0 + 1] = sinf(theta);
+                theta *= m->theta_scale;
+            }
+        }
+        rc = dalloc(m, (void **)&m->rope_tab, tab.size() * 4, false);
+        if (!rc) rc = (int)hipMemcpy(m->rope_tab, tab.data(), tab.size() * 4, hipMemcpyHostToDevice);
+        if (!rc) rc = spy_exact_luts(&m->lut);
+        if (!rc) rc = spy_ensure_lds(m, (const void *)xattn_pv_kernel<0>, xattn_pv_lds(c.n_ctx));
+        if (!rc) rc = spy_ensure_lds(m, (const void *)xattn_scores_kernel<0>, xattn_scores_lds(c.n_head));
+        if (!rc) {
+            m->exact_ok = true;
+            m->order = 1;
+            m->dry = true; rc = enqueue_pass_any(m, m->own_stream, PASS_GREEDY); m->dry = false;
+            if (rc == SPY_HIP_EUNSUPPORTED) { rc = 0; m->exact_ok = false; m->order = 0; }
+            const char *env = getenv("SPY_HIP_ORDER");                       // "own": this backend's own summation order by default
+            if (env && env[0] == 'o') m->order = 0;
+        }
+    }
 #ifdef ATL_STAMPS
     if (!rc && getenv("SPY_HIP_STAMPS")) rc = dalloc(m, (void **)&m->stamp_dbg, (128 + 512 * 8) * sizeof(long long), true);
 #endif
@@ -157,7 +190,15 @@ extern "C" int spy_hip_llama_buffer(spy_hip_llama *m, const char *name, int32_t 
     return 0;
 }
 
-extern "C" int spy_hip_llama_single_kernel(spy_hip_llama *m) { return m ? (m->attn_fused ? 2 : 0) : SPY_HIP_EINVAL; }
+extern "C" int spy_hip_llama_single_kernel(spy_hip_llama *m) { return m ? ((m->attn_fused && pass_order(m) == 0) ? 2 : 0) : SPY_HIP_EINVAL; }
+
+extern "C" int spy_hip_llama_set_order(spy_hip_llama *m, int32_t order) {
+    SPY_CHECK_ARG(m && (order == 0 || order == 1));
+    if (order == 1 && !m->exact_ok) return SPY_HIP_EUNSUPPORTED;
+    m->order = order;
+    return 0;
+}
+extern "C" int spy_hip_llama_order(spy_hip_llama *m) { return m ? pass_order(m) : SPY_HIP_EINVAL; }
 
 extern "C" int spy_hip_llama_timing(spy_hip_llama *m, float *ms_per_pass, int32_t *n_pass) {
     SPY_CHECK_ARG(m);
@@ -183,18 +224,40 @@ static bool fused_ok(const spy_hip_llama *m) {
 
 static int enqueue_one(spy_hip_llama *m, hipStream_t st, int which, int il) {
     const spy_hip_llama_desc &c = m->desc;
+    if (pass_order(m) == 1 || (m->dry && m->order == 1)) {      // the host backend's summation order: six launches per layer
+        if (which == K_SCORES) {
+            if (m->dry) return 0;
+            xattn_scores_kernel<0><<<dim3((unsigned)((c.n_ctx + XS_TOK - 1) / XS_TOK)), dim3(256), xattn_scores_lds(c.n_head), st>>>(
+                m->st, m->pos_imm, m->q16, m->k_cache[il], m->scores, c.n_head, c.n_ctx, 1.0f / sqrtf((float)m->hd));   // SoftmaxParam::scale (attention.cpp:113)
+            return SPY_LAUNCH_RC();
+        }
+        if (which == K_PV) {
+            if (m->dry) return 0;
+            xattn_pv_kernel<0><<<dim3((unsigned)(c.n_head * 8)), dim3(XP_THREADS), xattn_pv_lds(c.n_ctx), st>>>(m->st, m->pos_imm, m->scores, m->v_cache[il], m->attn_out, m->lut, c.n_ctx);
+            return SPY_LAUNCH_RC();
+        }
+        const spy_hip_llama_layer &Lx = m->layers[which == K_HEAD ? 0 : il];
+        const int tx = which == K_QKV ? Lx.t_wq : which == K_WO ? Lx.t_wo : which == K_GATEUP ? Lx.t_gate : which == K_DOWN ? Lx.t_down : c.t_out;
+        switch (tx) {
+        case SPY_HIP_Q4_0: return spy_enqueue_exact_q4_0(m, st, which, il);
+        case SPY_HIP_Q8_0: return spy_enqueue_exact_q8_0(m, st, which, il);
+        case SPY_HIP_Q4_K: return spy_enqueue_exact_q4_k(m, st, which, il);
+        case SPY_HIP_Q6_K: return spy_enqueue_exact_q6_k(m, st, which, il);
+        }
+        return SPY_HIP_EUNSUPPORTED;
+    }
     if ((which == K_SCORES || which == K_PV) && m->attn_fused) return 0;     // part of the K_QKV launch
     if (which == K_SCORES) {            // attn_score
         if (m->dry) return 0;
         const float scale = 1.0f / sqrtf((float)m->hd);                     // SoftmaxParam::scale (attention.cpp:113)
-        attn_scores_kernel<<<dim3((unsigned)((c.n_ctx + ATT_TCH - 1) / ATT_TCH)), dim3(256), 0, st>>>(m->st, m->q16, m->k_cache[il], m->scores,
+        attn_scores_kernel<<<dim3((unsigned)((c.n_ctx + ATT_TCH - 1) / ATT_TCH)), dim3(256), 0, st>>>(m->st, m->pos_imm, m->q16, m->k_cache[il], m->scores,
                                                                                                       c.n_head, c.n_ctx, scale);
         return SPY_LAUNCH_RC();
     }
     if (which == K_PV) {                // softmax, KQV (+ permute/contiguous: attn_out is already [hd, H] contiguous)
         if (m->dry) return 0;
         const size_t pv_lds = (size_t)c.n_ctx * 4 + (size_t)c.n_ctx * 2 + 16;
-        attn_pv_kernel<<<dim3((unsigned)(c.n_head * 8)), dim3(PV_THREADS), pv_lds, st>>>(m->st, m->scores, m->v_cache[il], m->attn_out, c.n_ctx);
+        attn_pv_kernel<<<dim3((unsigned)(c.n_head * 8)), dim3(PV_THREADS), pv_lds, st>>>(m->st, m->pos_imm, m->scores, m->v_cache[il], m->attn_out, c.n_ctx);
         return SPY_LAUNCH_RC();
     }
     // dispatch on the type of the kernel's (first) matrix
@@ -485,7 +548,9 @@ static int forward_any(spy_hip_llama *m, void *stream, const int32_t *tokens_hos
     hipStream_t st = stream ? (hipStream_t)stream : m->own_stream;
     for (int i = 0; i < n_token; i++) SPY_CHECK_ARG(tokens_host[i] >= 0 && tokens_host[i] < m->desc.n_vocab);   // view.cpp:61
     const bool exact = spy_exact_on() != 0;
-    if (n_token == 1 && fused_ok(m) && !exact && !getenv("SPY_HIP_FORCE_OPS")) {
+    // single tokens: the fused pass, in the order pass_order() names (with the library-wide exact-order switch on and a
+    // model the exact kernels do not take, operator by operator instead)
+    if (n_token == 1 && fused_ok(m) && (!exact || m->exact_ok) && !getenv("SPY_HIP_FORCE_OPS")) {
         dev_state h = {tokens_host[0], n_past, 0, 0};
         HIP_TRY(hipMemcpyAsync(m->st, &h, sizeof(h), hipMemcpyHostToDevice, st));
         RC_TRY(enqueue_pass_any(m, st, PASS_LOGITS));
@@ -527,8 +592,8 @@ extern "C" int spy_hip_llama_decode_greedy(spy_hip_llama *m, void *stream, int32
                                            int32_t *tokens_host, int32_t use_graph) {
     SPY_CHECK_ARG(m && n_steps > 0 && n_past >= 0 && first_token >= 0 && first_token < m->desc.n_vocab);
     SPY_CHECK_ARG((int64_t)n_past + n_steps <= m->desc.n_ctx && n_steps <= m->max_out);
-    if (spy_exact_on()) {
-        // exact order: the reference's loop as it stands (cli.h:88-128) -- one operator-by-operator pass per token,
+    if (spy_exact_on() && (!m->exact_ok || getenv("SPY_HIP_FORCE_OPS"))) {
+        // exact order for a model the fused exact kernels do not take: the reference's loop as it stands (cli.h:88-128) -- one operator-by-operator pass per token,
         // the first maximum of its logits (greedy.h:20-25) taken on the host
         std::vector<float> lg((size_t)m->desc.n_vocab);
         int32_t tok = first_token;
@@ -544,7 +609,8 @@ extern "C" int spy_hip_llama_decode_greedy(spy_hip_llama *m, void *stream, int32
     dev_state h = {first_token, n_past, 0, 0};
     HIP_TRY(hipMemcpyAsync(m->st, &h, sizeof(h), hipMemcpyHostToDevice, st));
     HIP_TRY(hipStreamSynchronize(st));
-    if (use_graph && (!m->graph_exec || !m->graph_n_exec || m->graph_stream != st)) {
+    if (use_graph && (!m->graph_exec || !m->graph_n_exec || m->graph_stream != st || m->graph_order != pass_order(m))) {
+        m->graph_order = pass_order(m);
         if (m->graph_exec) { (void)hipGraphExecDestroy(m->graph_exec); m->graph_exec = nullptr; }
         if (m->graph) { (void)hipGraphDestroy(m->graph); m->graph = nullptr; }
         HIP_TRY(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
@@ -607,4 +673,151 @@ extern "C" int spy_hip_llama_kernel_time(spy_hip_llama *m, void *stream, const c
     HIP_TRY(hipEventElapsedTime(&ms, m->ev0, m->ev1));
     *us_per_launch = ms * 1000.0f / (float)(reps * m->desc.n_layer);
     return 0;
+}
+
+// ---- the kernel families of the fused single-token pass, one at a time ---------------------------------------------------
+// Each entry point launches exactly what the token loop launches for that part of a layer (same templates, same grids),
+// on the caller's buffers and without a device state: a bare engine description is filled with the caller's pointers and
+// handed to the same enqueue functions.  order: 1 = the host backend's summation order, 0 = this backend's own.
+namespace {
+
+template <int ORDER, int NITK, bool NORM>
+__global__ __launch_bounds__(1024) void stage_dump_kernel(const float *__restrict__ x, const float *__restrict__ normw, float eps, int K, uint8_t *__restrict__ out) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    __shared__ float s_red[16];
+    __shared__ float s_sum;
+    const int tid = threadIdx.x;
+    float4 xv[NITK], wv[NORM ? NITK : 1];
+#pragma unroll
+    for (int j = 0; j < NITK; j++) {
+        const int i = min(tid + j * 1024, K / 4 - 1);
+        xv[j] = ((const float4 *)x)[i];
+        if constexpr (NORM) wv[j] = ((const float4 *)normw)[i];
+    }
+    int8_t *s_q = (int8_t *)smem;
+    int2 *s_meta = (int2 *)(smem + staged_q_bytes(K));
+    float *s_grp = (float *)(smem + ((staged_bytes(K) + 15) & ~(size_t)15));
+    if constexpr (ORDER == 1) xg_stage<NITK, NORM>(xv, wv, K, eps, s_q, s_meta, s_grp, &s_sum);
+    else wgv_stage<NITK, NORM>(xv, wv, K, eps, s_q, s_meta, s_red);
+    xg_dump_q8(s_q, s_meta, K, out);
+}
+
+template <int ORDER, bool NORM>
+int stage_dump(hipStream_t st, const float *x, const float *normw, float eps, int64_t K, void *yq) {
+    const size_t lds = ((staged_bytes(K) + 15) & ~(size_t)15) + (size_t)K;          // + K / 4 group sums
+    switch ((K + 4095) / 4096) {
+    case 1: stage_dump_kernel<ORDER, 1, NORM><<<dim3(1), dim3(1024), lds, st>>>(x, normw, eps, (int)K, (uint8_t *)yq); break;
+    case 2: stage_dump_kernel<ORDER, 2, NORM><<<dim3(1), dim3(1024), lds, st>>>(x, normw, eps, (int)K, (uint8_t *)yq); break;
+    case 3: stage_dump_kernel<ORDER, 3, NORM><<<dim3(1), dim3(1024), lds, st>>>(x, normw, eps, (int)K, (uint8_t *)yq); break;
+    default: return SPY_HIP_EUNSUPPORTED;
+    }
+    return SPY_LAUNCH_RC();
+}
+
+// a bare engine: one layer, the caller's buffers, nothing owned
+struct family_ctx {
+    spy_hip_llama m;
+    int init(int order, int n_embd, int n_head, int n_ff, int n_vocab, int64_t n_ctx, int wtype) {
+        if (order != 0 && order != 1) return SPY_HIP_EINVAL;
+        if (n_embd <= 0 || n_head <= 0 || n_embd % n_head != 0 || n_ctx <= 0 || n_ctx > (1 << 24)) return SPY_HIP_EINVAL;
+        spy_hip_llama_desc &c = m.desc;
+        memset(&c, 0, sizeof(c));
+        c.n_layer = 1; c.n_embd = n_embd; c.n_head = n_head; c.n_ff = n_ff; c.n_vocab = n_vocab; c.n_ctx = (int32_t)n_ctx;
+        c.eps = 0.0f; c.rope_freq_base = 10000.0f; c.wtype = wtype; c.t_out = wtype;
+        m.layers.resize(1);
+        memset(&m.layers[0], 0, sizeof(spy_hip_llama_layer));
+        int32_t *tt[7] = {&m.layers[0].t_wq, &m.layers[0].t_wk, &m.layers[0].t_wv, &m.layers[0].t_wo, &m.layers[0].t_gate, &m.layers[0].t_up, &m.layers[0].t_down};
+        for (int k = 0; k < 7; k++) *tt[k] = wtype;
+        m.desc.layers = m.layers.data();
+        m.hd = n_embd / n_head;
+        m.k_cache.assign(1, nullptr); m.v_cache.assign(1, nullptr);
+        m.wave = wave_ok(&m);
+        if (!m.wave) return SPY_HIP_EUNSUPPORTED;
+        const bool kq = wtype == SPY_HIP_Q4_K || wtype == SPY_HIP_Q6_K;
+        if (wtype != SPY_HIP_Q4_0 && wtype != SPY_HIP_Q8_0 && !kq) return SPY_HIP_EUNSUPPORTED;
+        if (kq && (n_embd % 256 != 0 || n_ff % 256 != 0)) return SPY_HIP_EINVAL;
+        int dev = 0; hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0) m.num_cu = prop.multiProcessorCount;
+        if (order == 1) {
+            if (n_embd % 128 != 0 || n_ff % 128 != 0) return SPY_HIP_EUNSUPPORTED;
+            RC_TRY(spy_exact_luts(&m.lut));
+            m.exact_ok = true; m.order = 1;
+        }
+        return 0;
+    }
+};
+
+}   // namespace
+
+extern "C" int spy_hip_rmsnorm_q8_0(void *stream, int32_t order, const float *x, const float *normw, float eps, int64_t K, void *yq) {
+    SPY_CHECK_ARG(x && yq && K > 0 && K % 64 == 0 && (order == 0 || order == 1));
+    if (order == 1 && K % 128 != 0) return SPY_HIP_EUNSUPPORTED;
+    hipStream_t st = (hipStream_t)stream;
+    if (order == 1) return normw ? stage_dump<1, true>(st, x, normw, eps, K, yq) : stage_dump<1, false>(st, x, normw, eps, K, yq);
+    return normw ? stage_dump<0, true>(st, x, normw, eps, K, yq) : stage_dump<0, false>(st, x, normw, eps, K, yq);
+}
+
+extern "C" int spy_hip_gemv_fused(void *stream, int32_t order, int32_t wtype, const void *w, const float *x, const float *normw, float eps,
+                                  const float *resid, float *out, int64_t M, int64_t K, void *xq_dump) {
+    SPY_CHECK_ARG(w && x && out && M > 0 && K > 0 && M < (1ll << 30) && K < (1ll << 20));
+    family_ctx f;
+    if (normw && !resid) {                       // result_norm, result_linear, output: RMSNorm * weight -> Q8_0 -> rows of w
+        RC_TRY(f.init(order, (int)K, (int)(K / 128), (int)K, (int)M, 8, wtype));
+        f.m.desc.w_out = w; f.m.desc.out_norm = normw; f.m.desc.eps = eps;
+        f.m.x = (float *)x; f.m.logits = out; f.m.q8_dump = (uint8_t *)xq_dump;
+        return enqueue_one(&f.m, (hipStream_t)stream, K_HEAD, 0);
+    }
+    if (!normw && resid) {                       // KQV_linear + Add, ffn_down + Add: Q8_0(x) -> rows of w -> + resid
+        SPY_CHECK_ARG(M % 128 == 0);
+        RC_TRY(f.init(order, (int)M, (int)(M / 128), (int)K, 1, 8, wtype));
+        f.m.layers[0].w_down = w;
+        f.m.hbuf = (float *)x; f.m.x1 = (float *)resid; f.m.x = out; f.m.q8_dump = (uint8_t *)xq_dump;
+        return enqueue_one(&f.m, (hipStream_t)stream, K_DOWN, 0);
+    }
+    return SPY_HIP_EUNSUPPORTED;
+}
+
+extern "C" int spy_hip_ffn_gate_up_silu(void *stream, int32_t order, int32_t wtype, const void *w_gate, const void *w_up, const float *x, const float *normw,
+                                        float eps, float *out, int64_t F, int64_t K, void *xq_dump) {
+    SPY_CHECK_ARG(w_gate && w_up && x && normw && out && F > 0 && K > 0 && K % 128 == 0 && F < (1ll << 24) && K < (1ll << 20));
+    family_ctx f;
+    RC_TRY(f.init(order, (int)K, (int)(K / 128), (int)F, 1, 8, wtype));
+    f.m.layers[0].w_gate = w_gate; f.m.layers[0].w_up = w_up; f.m.layers[0].ffn_norm = normw; f.m.desc.eps = eps;
+    f.m.x1 = (float *)x; f.m.hbuf = out; f.m.q8_dump = (uint8_t *)xq_dump;
+    return enqueue_one(&f.m, (hipStream_t)stream, K_GATEUP, 0);
+}
+
+extern "C" int spy_hip_rope_kvwrite(void *stream, int32_t order, int32_t wtype, int32_t wtype_v, const void *wq, const void *wk, const void *wv, const float *x,
+                                    const float *normw, float eps, int32_t n_embd, int32_t n_head, int32_t pos, int64_t n_ctx, const float *rope_cs,
+                                    void *q16, void *k_cache, void *v_cache, void *xq_dump) {
+    SPY_CHECK_ARG(wq && wk && wv && x && normw && rope_cs && q16 && k_cache && v_cache && pos >= 0 && pos < n_ctx && n_embd % 128 == 0);
+    family_ctx f;
+    RC_TRY(f.init(order, n_embd, n_head, n_embd, 1, n_ctx, wtype));
+    if (f.m.hd != 128) return SPY_HIP_EUNSUPPORTED;
+    spy_hip_llama_layer &L = f.m.layers[0];
+    L.wq = wq; L.wk = wk; L.wv = wv; L.attn_norm = normw; L.t_wv = wtype_v ? wtype_v : wtype;
+    f.m.desc.eps = eps;
+    f.m.x = (float *)x; f.m.q16 = (uint16_t *)q16; f.m.k_cache[0] = (uint16_t *)k_cache; f.m.v_cache[0] = (uint16_t *)v_cache;
+    f.m.rope_cs = (float *)rope_cs; f.m.rope_tab = (float *)rope_cs; f.m.rope_row0 = pos; f.m.pos_imm = pos; f.m.q8_dump = (uint8_t *)xq_dump;
+    return enqueue_one(&f.m, (hipStream_t)stream, K_QKV, 0);
+}
+
+extern "C" int spy_hip_attn_decode(void *stream, int32_t order, const void *q16, const void *k_cache, const void *v_cache, int32_t n_head, int32_t n_kv,
+                                   int64_t n_ctx, float *scores, float *out) {
+    SPY_CHECK_ARG(q16 && k_cache && v_cache && scores && out && n_head > 0 && n_kv > 0 && n_kv <= n_ctx && n_ctx % 8 == 0);
+    family_ctx f;
+    RC_TRY(f.init(order, n_head * 128, n_head, n_head * 128, 1, n_ctx, SPY_HIP_Q4_0));
+    const size_t pv_lds = (size_t)n_ctx * 6 + 16;
+    if (order == 1) {
+        if (xattn_pv_lds((int)n_ctx) > 160 * 1024 || xattn_scores_lds(n_head) > 160 * 1024) return SPY_HIP_EUNSUPPORTED;
+        RC_TRY(spy_ensure_lds(&f.m, (const void *)xattn_pv_kernel<0>, xattn_pv_lds((int)n_ctx)));
+        RC_TRY(spy_ensure_lds(&f.m, (const void *)xattn_scores_kernel<0>, xattn_scores_lds(n_head)));
+    } else {
+        if (pv_lds > 160 * 1024) return SPY_HIP_EUNSUPPORTED;
+        RC_TRY(spy_ensure_lds(&f.m, (const void *)attn_pv_kernel, pv_lds));
+    }
+    f.m.q16 = (uint16_t *)q16; f.m.k_cache[0] = (uint16_t *)k_cache; f.m.v_cache[0] = (uint16_t *)v_cache;
+    f.m.scores = scores; f.m.attn_out = out; f.m.pos_imm = n_kv - 1;
+    RC_TRY(enqueue_one(&f.m, (hipStream_t)stream, K_SCORES, 0));
+    return enqueue_one(&f.m, (hipStream_t)stream, K_PV, 0);
 }

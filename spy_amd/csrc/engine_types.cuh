@@ -33,9 +33,18 @@ struct spy_hip_llama {
     // graph of one single-token pass
     hipGraph_t graph = nullptr; hipGraphExec_t graph_exec = nullptr; hipStream_t graph_stream = nullptr;
     hipGraph_t graph_n = nullptr; hipGraphExec_t graph_n_exec = nullptr;   // SPY_GRAPH_STEPS passes in one graph
+    int graph_order = -1;                                                  // summation order the graphs were captured with
     hipStream_t own_stream = nullptr;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     double timed_ms = 0.0; int timed_pass = 0;
+    // Summation order of the fused single-token pass: 1 = the host backend's (exact_decode.cuh: every output equal to the CPU
+    // backend's bit for bit), 0 = this backend's own (decode_kernels.cuh: faster, equal to about 1e-7 per operator)
+    int order = 0;
+    bool exact_ok = false;                      // the exact-order kernels take this model's shapes
+    float *rope_tab = nullptr;                  // [n_ctx][hd]: cos, sin of every position's angles, from the host's libm (non-linear.cpp:304-309)
+    const float *lut = nullptr;                 // exp table [65536], silu table [65536], filled by the host's libm
+    uint8_t *q8_dump = nullptr;                 // tests: where workgroup 0 of a launch leaves its staged Q8_0 activations
+    int pos_imm = 0, rope_row0 = 0;             // kernel-family entry points (no device state): the position; first position of rope_tab
     long long *stamp_dbg = nullptr;             // measurement builds (-DATL_STAMPS) only
     uint32_t spin_limit = 400000;               // polls of a bounded inter-workgroup wait before a pass gives up (~0.5 s)
     // per engine (= per device) launcher state: dynamic-LDS limit already set for a kernel, resident workgroups of a persistent grid
@@ -69,6 +78,11 @@ int spy_enqueue_kernel_q4_0(spy_hip_llama *m, hipStream_t st, int which, int il)
 int spy_enqueue_kernel_q8_0(spy_hip_llama *m, hipStream_t st, int which, int il);
 int spy_enqueue_kernel_q4_k(spy_hip_llama *m, hipStream_t st, int which, int il);
 int spy_enqueue_kernel_q6_k(spy_hip_llama *m, hipStream_t st, int which, int il);
+// the same in the host backend's summation order (exact_launch.cuh)
+int spy_enqueue_exact_q4_0(spy_hip_llama *m, hipStream_t st, int which, int il);
+int spy_enqueue_exact_q8_0(spy_hip_llama *m, hipStream_t st, int which, int il);
+int spy_enqueue_exact_q4_k(spy_hip_llama *m, hipStream_t st, int which, int il);
+int spy_enqueue_exact_q6_k(spy_hip_llama *m, hipStream_t st, int which, int il);
 // probe: only check that the fused attention launch for this layer's types exists and that all its workgroups are resident
 int spy_probe_attn_layer_q4_0(spy_hip_llama *m, int il);
 int spy_probe_attn_layer_q8_0(spy_hip_llama *m, int il);

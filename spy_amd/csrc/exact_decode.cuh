@@ -1,0 +1,534 @@
+// Kernels of the fused single-token pass in the HOST BACKEND'S SUMMATION ORDER: the same launches as
+// decode_kernels.cuh (weights streamed once, activations quantized in LDS, epilogues fused), but every fp32 sum is
+// added in the order of Spy's CPU loops, so that each output equals the CPU backend's bit for bit:
+//   * quantized dots (vec_dot.h:42-115): eight accumulators per output element, lane l takes four products of every
+//     block, acc[l] = fma(d_w * d_x, float(part[l]), acc[l]) block after block, then hsum_float_8 (vec_util.h:75-81);
+//     K-quant rows: the project's order, one accumulator, one term per 32-element block;
+//   * fp16 dots (vec_dot.h:117-146): 4 x 8 accumulators over chunks of 32 while i + 32 < n, the reduction tree, then
+//     the scalar tail;
+//   * NormRMS and Softmax sums (non-linear.cpp:129-223): libstdc++'s groups of four added to ONE running sum;
+//   * exp and silu from the two fp16-indexed tables filled by the host's libm, the RoPE angles from a host table.
+//
+// How a serial sum is made fast.  The integer block dots stay where they are (64 lanes x v_dot4, one block pair per
+// lane, weights read once, coalesced).  What changes is what follows them: instead of scaling and adding its blocks in
+// lane order, a lane writes the eight partial sums of each of its blocks (as floats) and the block's scale product into
+// LDS, transposed, and after a workgroup barrier ONE lane per accumulator walks its row of LDS block after block:
+// 8 lanes per output element, 64 lanes = 8 output elements per wave, fed by 128-bit LDS reads.  The walk is a chain of
+// dependent fmas (about 4 ns each on this part, whatever else the compute unit does), so a 4096-wide row costs about
+// 0.6 us of latency per batch of rows; batches are as large as LDS allows (32 rows of 128 blocks).
+#pragma once
+
+#include "decode_kernels.cuh"
+
+#define XG_THREADS 1024
+#define XG_WAVES 16
+#define XG_NBS 128                         // blocks per K slab (= 64 lanes x one block pair)
+#ifndef XG_DEPTH
+#define XG_DEPTH 3                         // rows per wave requested ahead of their use
+#endif
+
+template <int WT> struct xg_traits { static constexpr int NCH = (WT == SPY_HIP_Q4_0 || WT == SPY_HIP_Q8_0) ? 8 : 1; };
+// floats of LDS per row slot: NCH rows of partials (+4: bank skew between the rows) and the row of scale products (+4: skew between slots)
+static __host__ __device__ constexpr int xg_slot_floats(int nch) { return nch * (XG_NBS + 4) + XG_NBS + 4; }
+
+struct xg_args {
+    const uint8_t *W0, *W1, *W2;
+    int M, K;                              // output elements (RESID / STORE: rows of W0; GATEUP: rows of W0 = rows of W1; QKV: n_embd), contraction length
+    const float *x_in, *normw; float eps;
+    const float *resid; float *out;
+    const dev_state *st; const float *rope_tab; uint16_t *q16, *kc, *vc;   // rope_tab: [n_ctx][hd] cos, sin per pair, from the host's libm
+    const float *lut;                      // exp table [65536], then silu table [65536] (lookup_table_impl/non-linear.h:39-47,131-139)
+    int n_ctx, d, hd;
+    uint8_t *q8_dump;                      // tests: workgroup 0 writes its staged activations here as native Q8_0 blocks
+    int pos_imm, rope_row0;                // st == nullptr: the position as a number; first position of rope_tab
+};
+
+// ---- activations: f32 vector -> (RMSNorm * weight ->) Q8_0 in LDS, sums in the host order --------------------------
+// NormRMS (non-linear.cpp:194-223): sum = std::transform_reduce(x, x) = groups of four ((x0^2 + x1^2) + (x2^2 + x3^2))
+// added to one running sum in order; scale = 1 / sqrt(sum / n + eps); y = x * scale; then the Mul node: y * w.
+// The 1024 threads form the group sums (one float4 each per 4096 elements), lane 0 of wave 0 adds them.
+template <int NITK, bool NORM>
+static __device__ __forceinline__ void xg_stage(const float4 (&xv)[NITK], const float4 (&wv)[NORM ? NITK : 1], int K, float eps,
+                                                int8_t *s_q, int2 *s_meta, float *s_grp, float *s_sum) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    float scale = 1.0f;
+    if constexpr (NORM) {
+#pragma unroll
+        for (int j = 0; j < NITK; j++) {
+            const int i = tid + j * XG_THREADS;
+            if (i < K / 4) {
+                const float4 v = xv[j];
+                const float a0 = v.x * v.x, a1 = v.y * v.y, a2 = v.z * v.z, a3 = v.w * v.w;
+                const float v1 = a0 + a1, v2 = a2 + a3;
+                s_grp[i] = v1 + v2;
+            }
+        }
+        __syncthreads();
+        if (wave == 0) {
+            float init = 0.0f;
+            const int ng = K / 4;                          // a multiple of 4 (K % 16 == 0)
+            for (int g = 0; g < ng; g += 16) {
+                const float4 a = *(const float4 *)(s_grp + g), b = *(const float4 *)(s_grp + min(g + 4, ng - 4)),
+                             c = *(const float4 *)(s_grp + min(g + 8, ng - 4)), e = *(const float4 *)(s_grp + min(g + 12, ng - 4));
+                init = init + a.x; init = init + a.y; init = init + a.z; init = init + a.w;
+                if (g + 4 < ng) { init = init + b.x; init = init + b.y; init = init + b.z; init = init + b.w; }
+                if (g + 8 < ng) { init = init + c.x; init = init + c.y; init = init + c.z; init = init + c.w; }
+                if (g + 12 < ng) { init = init + e.x; init = init + e.y; init = init + e.z; init = init + e.w; }
+            }
+            if (lane == 0) *s_sum = init;
+        }
+        __syncthreads();
+        const float mean = *s_sum / (float)K;
+        scale = 1.0f / sqrtf(mean + eps);
+    }
+#pragma unroll
+    for (int j = 0; j < NITK; j++) {
+        const int i = tid + j * XG_THREADS;
+        if (i < K / 4) {
+            float4 v = xv[j];
+            if constexpr (NORM) {
+                const float4 w = wv[j];
+                v.x = (v.x * scale) * w.x; v.y = (v.y * scale) * w.y; v.z = (v.z * scale) * w.z; v.w = (v.w * scale) * w.w;
+            }
+            int2 meta;
+            const uint32_t q = quantize_oct(v, meta);
+            ((uint32_t *)s_q)[act_dw(i, K >> 6)] = q;
+            if ((tid & 7) == 0) s_meta[i >> 3] = meta;
+        }
+    }
+    __syncthreads();
+}
+
+// the staged activations of a workgroup as native Q8_0 blocks (tests compare them with Quantizator<FP32,Q8_0>)
+static __device__ __forceinline__ void xg_dump_q8(const int8_t *s_q, const int2 *s_meta, int K, uint8_t *out) {
+    for (int b = threadIdx.x; b < K / 32; b += XG_THREADS) {
+        uint16_t *dst = (uint16_t *)(out + (size_t)b * 34);
+        dst[0] = f2h(__int_as_float(s_meta[b].x));
+        for (int i = 0; i < 8; i++) {
+            const uint32_t q = ((const uint32_t *)s_q)[act_dw(b * 8 + i, K >> 6)];
+            dst[1 + 2 * i] = (uint16_t)(q & 0xFFFFu); dst[2 + 2 * i] = (uint16_t)(q >> 16);
+        }
+    }
+}
+
+// ---- phase 1: a lane's block pair of one weight row -> partial sums and scale products in LDS -------------------------
+// x[0..3]: the 64 int8 activations of the pair (16 bytes each), mm / mm2: their {scale bits, sum q} (see load_act_frag),
+// n8[i] = -8 * (sum of the four bytes of activation dword i): folds the -8 of the Q4_0 nibbles into the accumulator
+// input of v_dot4, so that each partial sum is sum (n - 8) * q exactly as sub_epi8 / maddubs / madd form it.
+// slot: this row's LDS record; pl: the pair's index within the slab (= lane).
+template <int WT>
+static __device__ __forceinline__ void xg_phase1(const uint32_t *w, const act_frag<1> &f, const int (&n8)[16], int p, int pl, float *slot) {
+    constexpr int NCH = xg_traits<WT>::NCH;
+    float *P = slot, *D = slot + NCH * (XG_NBS + 4);
+    const int4 x0 = f.x[0][0], x1 = f.x[0][1], x2 = f.x[0][2], x3 = f.x[0][3], mm = f.mm[0], mm2 = f.mm2[0];
+    if constexpr (WT == SPY_HIP_Q4_0 || WT == SPY_HIP_Q8_0) {
+        int pa[8], pb[8];
+        float sA, sB;
+        if constexpr (WT == SPY_HIP_Q4_0) {
+            sA = h2f((uint16_t)(w[0] & 0xFFFFu)) * __int_as_float(mm.x); sB = h2f((uint16_t)(w[4] >> 16)) * __int_as_float(mm.z);
+            const uint32_t a[4] = {__builtin_amdgcn_alignbit(w[1], w[0], 16), __builtin_amdgcn_alignbit(w[2], w[1], 16),
+                                   __builtin_amdgcn_alignbit(w[3], w[2], 16), __builtin_amdgcn_alignbit(w[4], w[3], 16)};
+            const int xa[4] = {x0.x, x0.y, x0.z, x0.w}, xb[4] = {x1.x, x1.y, x1.z, x1.w}, xc[4] = {x2.x, x2.y, x2.z, x2.w}, xd[4] = {x3.x, x3.y, x3.z, x3.w};
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                // accumulators 4..7: low nibbles against elements 0..15; 0..3: high nibbles against 16..31 (vec_dot.h:62-78)
+                pa[4 + k] = __builtin_amdgcn_sdot4((int)(a[k] & 0x0F0F0F0Fu), xa[k], n8[k], false);
+                pa[k]     = __builtin_amdgcn_sdot4((int)((a[k] >> 4) & 0x0F0F0F0Fu), xb[k], n8[4 + k], false);
+                pb[4 + k] = __builtin_amdgcn_sdot4((int)(w[5 + k] & 0x0F0F0F0Fu), xc[k], n8[8 + k], false);
+                pb[k]     = __builtin_amdgcn_sdot4((int)((w[5 + k] >> 4) & 0x0F0F0F0Fu), xd[k], n8[12 + k], false);
+            }
+        } else {
+            sA = h2f((uint16_t)(w[0] & 0xFFFFu)) * __int_as_float(mm.x); sB = h2f((uint16_t)(w[8] >> 16)) * __int_as_float(mm.z);
+            const int xa[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w}, xb[8] = {x2.x, x2.y, x2.z, x2.w, x3.x, x3.y, x3.z, x3.w};
+#pragma unroll
+            for (int l = 0; l < 8; l++) {               // accumulator l: elements 4l..4l+3 (vec_util.h:126-132)
+                pa[l] = __builtin_amdgcn_sdot4((int)__builtin_amdgcn_alignbit(w[l + 1], w[l], 16), xa[l], 0, false);
+                pb[l] = __builtin_amdgcn_sdot4((int)w[9 + l], xb[l], 0, false);
+            }
+        }
+#pragma unroll
+        for (int l = 0; l < 8; l++) *(float2 *)(P + l * (XG_NBS + 4) + 2 * pl) = make_float2((float)pa[l], (float)pb[l]);
+        *(float2 *)(D + 2 * pl) = make_float2(sA, sB);
+    } else if constexpr (WT == SPY_HIP_Q4_K) {
+        // the two sub-blocks of the lane: term = d * float(sc * isum) - dmin * float(m * sum q), scale = d_x (one accumulator per row)
+        const int j = p & 3, a = 2 * j;
+        const float d = h2f((uint16_t)(w[0] & 0xFFFFu)), dmin = h2f((uint16_t)(w[0] >> 16));
+        int scA, mA, scB, mB;
+        if (j < 2) {
+            scA = byte_of3(w[1], w[2], w[3], a) & 63;     mA = byte_of3(w[1], w[2], w[3], a + 4) & 63;
+            scB = byte_of3(w[1], w[2], w[3], a + 1) & 63; mB = byte_of3(w[1], w[2], w[3], a + 5) & 63;
+        } else {
+            const uint32_t hA = byte_of3(w[1], w[2], w[3], a + 4), hB = byte_of3(w[1], w[2], w[3], a + 5);
+            scA = (hA & 0x0F) | ((byte_of3(w[1], w[2], w[3], a - 4) >> 6) << 4); mA = (hA >> 4) | ((byte_of3(w[1], w[2], w[3], a) >> 6) << 4);
+            scB = (hB & 0x0F) | ((byte_of3(w[1], w[2], w[3], a - 3) >> 6) << 4); mB = (hB >> 4) | ((byte_of3(w[1], w[2], w[3], a + 1) >> 6) << 4);
+        }
+        int iA = 0, iB = 0;
+        const int xa[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w}, xb[8] = {x2.x, x2.y, x2.z, x2.w, x3.x, x3.y, x3.z, x3.w};
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            iA = __builtin_amdgcn_sdot4((int)(w[4 + i] & 0x0F0F0F0Fu), xa[i], iA, false);
+            iB = __builtin_amdgcn_sdot4((int)((w[4 + i] >> 4) & 0x0F0F0F0Fu), xb[i], iB, false);
+        }
+        const float posA = d * (float)__mul24(scA, iA), negA = dmin * (float)__mul24(mA, mm.y);
+        const float posB = d * (float)__mul24(scB, iB), negB = dmin * (float)__mul24(mB, mm.w);
+        *(float2 *)(P + 2 * pl) = make_float2(posA - negA, posB - negB);
+        *(float2 *)(D + 2 * pl) = make_float2(__int_as_float(mm.x), __int_as_float(mm.z));
+    } else {
+        // Q6_K: lane (n, e) holds the 16-element halves e of the four Q8_0 blocks 4n .. 4n+3 of its super-block; the other
+        // halves are in the neighbouring lane.  term of block t = float(sc[2t] * isum(t, 0) + sc[2t+1] * isum(t, 1)), scale = d_x * d
+        const uint32_t *qa = w, *qb = w + 4, *qh = w + 8;
+        const uint32_t s0 = w[12], s1 = w[13];
+        const int e = p & 1;
+        const float d = h2f((uint16_t)(w[14] & 0xFFFFu));
+        int isum[4] = {0, 0, 0, 0};
+        const int xm[4][4] = {{x0.x, x0.y, x0.z, x0.w}, {x1.x, x1.y, x1.z, x1.w}, {x2.x, x2.y, x2.z, x2.w}, {x3.x, x3.y, x3.z, x3.w}};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t h = qh[i];
+            isum[0] = __builtin_amdgcn_sdot4((int)q6_m32((qa[i] & 0x0F0F0F0Fu) | ((h & 0x03030303u) << 4)), xm[0][i], isum[0], false);
+            isum[1] = __builtin_amdgcn_sdot4((int)q6_m32((qb[i] & 0x0F0F0F0Fu) | ((h & 0x0C0C0C0Cu) << 2)), xm[1][i], isum[1], false);
+            isum[2] = __builtin_amdgcn_sdot4((int)q6_m32(((qa[i] >> 4) & 0x0F0F0F0Fu) | (h & 0x30303030u)), xm[2][i], isum[2], false);
+            isum[3] = __builtin_amdgcn_sdot4((int)q6_m32(((qb[i] >> 4) & 0x0F0F0F0Fu) | ((h >> 2) & 0x30303030u)), xm[3][i], isum[3], false);
+        }
+        int sv[4];
+#pragma unroll
+        for (int m = 0; m < 4; m++) {
+            const int k = e + 2 * m;
+            const int sc = (int)(int8_t)(((k < 4 ? s0 : s1) >> (8 * (k & 3))) & 0xFFu);
+            const int v = __mul24(sc, isum[m]);
+            sv[m] = v + __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, true);          // + the neighbour lane's half (quad_perm [1,0,3,2]); integer, order-free
+        }
+        const float dx[4] = {__int_as_float(mm.x), __int_as_float(mm.z), __int_as_float(mm2.x), __int_as_float(mm2.z)};
+        // lane e writes blocks m = 2e, 2e+1 of the four: global block 2p, 2p+1
+        const float t0 = (float)(e ? sv[2] : sv[0]), t1 = (float)(e ? sv[3] : sv[1]);
+        const float c0 = (e ? dx[2] : dx[0]) * d, c1 = (e ? dx[3] : dx[1]) * d;
+        *(float2 *)(P + 2 * pl) = make_float2(t0, t1);
+        *(float2 *)(D + 2 * pl) = make_float2(c0, c1);
+    }
+}
+
+// ---- phase 2: one lane walks one accumulator over the blocks of a slab ------------------------------------------------
+static __device__ __forceinline__ float xg_chain(const float *P, const float *D, int nblk, float acc) {
+    // nblk % 4 == 0; reads beyond nblk (up to 12 floats) stay inside the row's 128 + 4 floats and are not used
+    for (int b = 0; b < nblk; b += 16) {
+        const float4 p0 = *(const float4 *)(P + b), d0 = *(const float4 *)(D + b);
+        const float4 p1 = *(const float4 *)(P + min(b + 4, XG_NBS - 4)), d1 = *(const float4 *)(D + min(b + 4, XG_NBS - 4));
+        const float4 p2 = *(const float4 *)(P + min(b + 8, XG_NBS - 4)), d2 = *(const float4 *)(D + min(b + 8, XG_NBS - 4));
+        const float4 p3 = *(const float4 *)(P + min(b + 12, XG_NBS - 4)), d3 = *(const float4 *)(D + min(b + 12, XG_NBS - 4));
+        acc = fmaf(d0.x, p0.x, acc); acc = fmaf(d0.y, p0.y, acc); acc = fmaf(d0.z, p0.z, acc); acc = fmaf(d0.w, p0.w, acc);
+        if (b + 4 < nblk) { acc = fmaf(d1.x, p1.x, acc); acc = fmaf(d1.y, p1.y, acc); acc = fmaf(d1.z, p1.z, acc); acc = fmaf(d1.w, p1.w, acc); }
+        if (b + 8 < nblk) { acc = fmaf(d2.x, p2.x, acc); acc = fmaf(d2.y, p2.y, acc); acc = fmaf(d2.z, p2.z, acc); acc = fmaf(d2.w, p2.w, acc); }
+        if (b + 12 < nblk) { acc = fmaf(d3.x, p3.x, acc); acc = fmaf(d3.y, p3.y, acc); acc = fmaf(d3.z, p3.z, acc); acc = fmaf(d3.w, p3.w, acc); }
+    }
+    return acc;
+}
+
+// hsum_float_8 over the eight lanes of an output element: (a0+a4)+(a2+a6) + (a1+a5)+(a3+a7); the operands of each
+// addition commute, so the three exchanges leave the same bits in all eight lanes (vec_util.h:75-81)
+static __device__ __forceinline__ float xg_hsum8(float acc) {
+    acc += __shfl_xor(acc, 4, SPY_WAVE);
+    acc += __shfl_xor(acc, 2, SPY_WAVE);
+    acc += __shfl_xor(acc, 1, SPY_WAVE);
+    return acc;
+}
+
+// ---- the kernel --------------------------------------------------------------------------------------------------------
+// 1024 threads; wave w of the grid (gw) owns, per step, RPS rows:
+//   EPI_RESID / EPI_STORE : rows gw * RPS + j + k * NW * RPS                              (NSTEP steps)
+//   EPI_GATEUP            : RPS = 2: row i = gw + k * NW of W0 (gate) and of W1 (up)      (NSTEP steps)
+//   EPI_QKV               : step 0: rows 2 gw, 2 gw + 1 of [W0; W1] (a RoPE pair), step 1: row gw of W2
+// A step's rows of all 16 waves form one batch: phase 1 (all waves) -> barrier -> phase 2 (the first lanes, one per
+// accumulator) -> barrier, per slab of 4096 elements of K; the accumulators stay in their lanes from slab to slab.
+template <int WT, int NITK, int RPS, int NSTEP, int EPI, int WTV = WT>
+__global__ __launch_bounds__(XG_THREADS) void xgemv_kernel(xg_args a) {
+    constexpr bool NORM = (EPI != EPI_RESID);
+    constexpr int NCH = xg_traits<WT>::NCH, NCHV = xg_traits<WTV>::NCH;
+    constexpr int NROW = EPI == EPI_QKV ? 3 : RPS * NSTEP;                  // rows per wave
+    constexpr int SLOTF = xg_slot_floats(NCH > NCHV ? NCH : NCHV);
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    __shared__ float s_sum;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int NW = (int)gridDim.x * XG_WAVES, gw = (int)blockIdx.x * XG_WAVES + wave;
+    const int K = a.K, npair = K / 64;
+    const size_t RB = (size_t)spy_row_size(WT, K);
+
+    // row index (within its matrix) and base of the wave's row r (0 .. NROW-1); rows beyond the matrix re-read a valid row and are dropped in the epilogue
+    auto row_of = [&](int r, bool &valid) -> int {
+        if constexpr (EPI == EPI_QKV) { valid = gw < a.d; const int j = gw % a.d; return r == 2 ? j : ((2 * j) % a.d) + r; }
+        else if constexpr (EPI == EPI_GATEUP) { const int u = gw + (r >> 1) * NW; valid = u < a.M; return valid ? u : gw % a.M; }
+        else { const int u = (gw + (r / RPS) * NW) * RPS + (r % RPS); valid = u < a.M; return valid ? u : u % a.M; }
+    };
+    auto row_ptr = [&](int r) -> const uint8_t * {
+        bool v; const int i = row_of(r, v);
+        if constexpr (EPI == EPI_QKV) {
+            if (r == 2) return a.W2 + (size_t)i * spy_row_size(WTV, K);
+            return (2 * (gw % a.d) < a.d ? a.W0 : a.W1) + (size_t)i * RB;
+        } else if constexpr (EPI == EPI_GATEUP) return ((r & 1) ? a.W1 : a.W0) + (size_t)i * RB;
+        else return a.W0 + (size_t)i * RB;
+    };
+
+    // 1. the activation vector, 2. the first rows: all unconditional, in this order (the compute unit serves its requests in order)
+    float4 xv[NITK], wv[NORM ? NITK : 1];
+#pragma unroll
+    for (int j = 0; j < NITK; j++) {
+        const int i = min(tid + j * XG_THREADS, K / 4 - 1);
+        xv[j] = ((const float4 *)a.x_in)[i];
+        if constexpr (NORM) wv[j] = ((const float4 *)a.normw)[i];
+    }
+    constexpr int RING = NROW < XG_DEPTH + 1 ? NROW : XG_DEPTH + 1;
+    wtile<WT, NITK> t[RING];
+    wtile<WTV, NITK> tv;
+    auto issue = [&](int r) {
+        if (EPI == EPI_QKV && r == 2) load_tile<WTV, 64, NITK>(tv, row_ptr(r), npair, lane);
+        else load_tile<WT, 64, NITK>(t[r % RING], row_ptr(r), npair, lane);
+    };
+    __builtin_amdgcn_s_barrier();
+#pragma unroll
+    for (int r = 0; r < NROW; r++) if (r < XG_DEPTH) issue(r);
+
+    // 3. stage the activations
+    int8_t *s_q = (int8_t *)smem;
+    int2 *s_meta = (int2 *)(smem + staged_q_bytes(K));
+    float *s_part = (float *)(smem + ((staged_bytes(K) + 15) & ~(size_t)15));      // row slots; the group sums of the norm use the same bytes before
+    xg_stage<NITK, NORM>(xv, wv, K, a.eps, s_q, s_meta, s_part, &s_sum);
+    if (a.q8_dump && blockIdx.x == 0) xg_dump_q8(s_q, s_meta, K, a.q8_dump);
+    staged_act act; act.q = s_q; act.meta = s_meta;
+
+    constexpr int NSTEPS = EPI == EPI_QKV ? 2 : NSTEP;
+    static_assert(NITK == 1 || NROW == 1, "rows longer than one slab are walked one row per wave");
+#pragma unroll
+    for (int step = 0; step < NSTEPS; step++) {
+        const int r0 = EPI == EPI_QKV ? 2 * step : step * RPS;                  // first row of the step
+        const int rows = EPI == EPI_QKV ? 2 - step : RPS;
+        const bool vstep = EPI == EPI_QKV && step == 1;
+        const int nch = vstep ? NCHV : NCH;
+        const int chains = XG_WAVES * rows * nch;
+        float acc = 0.0f;
+#pragma unroll
+        for (int it = 0; it < NITK; it++) {
+            const int nblk = min(XG_NBS, K / 32 - it * XG_NBS);                // blocks of this slab
+            if (nblk > 0) {
+                const int p = it * 64 + lane;
+                // this lane's activations of the slab (the same for every row) and the -8 * sum q per dword
+                act_frag<1> af, av;
+                int n8[16];
+                if (p < npair) {
+                    load_act_frag<WT, 1>(af, act, npair, p);
+                    if constexpr (WTV != WT) { if (vstep) load_act_frag<WTV, 1>(av, act, npair, p); }
+                    if constexpr (WT == SPY_HIP_Q4_0) {
+                        const int xs[16] = {af.x[0][0].x, af.x[0][0].y, af.x[0][0].z, af.x[0][0].w, af.x[0][1].x, af.x[0][1].y, af.x[0][1].z, af.x[0][1].w,
+                                            af.x[0][2].x, af.x[0][2].y, af.x[0][2].z, af.x[0][2].w, af.x[0][3].x, af.x[0][3].y, af.x[0][3].z, af.x[0][3].w};
+#pragma unroll
+                        for (int i = 0; i < 16; i++) n8[i] = -8 * __builtin_amdgcn_sdot4(xs[i], 0x01010101, 0, false);
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < rows; j++) {
+                    const int r = r0 + j;
+                    if (it == 0 && r + XG_DEPTH < NROW) issue(r + XG_DEPTH);      // its ring slot held row r - 1, multiplied in the previous step
+                    float *slot = s_part + (size_t)(wave * rows + j) * SLOTF;
+                    if (p < npair) {
+                        if (vstep) { if constexpr (WTV != WT) xg_phase1<WTV>(tv.w[it], av, n8, p, lane, slot); else xg_phase1<WTV>(tv.w[it], af, n8, p, lane, slot); }
+                        else xg_phase1<WT>(t[r % RING].w[it], af, n8, p, lane, slot);
+                    }
+                }
+                __syncthreads();
+                if (tid < chains) {
+                    const int slot_i = tid / nch, l = tid % nch;
+                    const float *slot = s_part + (size_t)slot_i * SLOTF;
+                    acc = xg_chain(slot + l * (XG_NBS + 4), slot + nch * (XG_NBS + 4), nblk, acc);
+                }
+                __syncthreads();
+            }
+        }
+        // epilogue of the step: the lanes that walked accumulator 0 of a row hold its total after the tree
+        if (nch == 8) acc = xg_hsum8(acc);
+        const bool owner = tid < chains && (tid % nch) == 0;
+        const int slot_i = tid / nch;                                         // = wave_of_row * rows + j
+        const int ow = slot_i / rows, oj = slot_i % rows;                      // the wave that owned the row and its index in the step
+        const int ogw = (int)blockIdx.x * XG_WAVES + ow;
+        if constexpr (EPI == EPI_RESID || EPI == EPI_STORE) {
+            const int u = (ogw + step * NW) * RPS + oj;
+            if (owner && u < a.M) a.out[u] = EPI == EPI_RESID ? acc + a.resid[u] : acc;       // Add(KQV_linear, x) / Add(ffn_out, ffn_input)
+        } else if constexpr (EPI == EPI_GATEUP) {
+            const float up = __shfl_xor(acc, nch, SPY_WAVE);                   // the row after (up_i) sits nch lanes further
+            const int i = ogw + step * NW;
+            if (owner && oj == 0 && i < a.M) a.out[i] = up * a.lut[65536 + f2h(acc)];             // Mul(ffn_up, Silu(ffn_gate)) (ffn.cpp:24-35, non-linear.cpp:11-14)
+        } else {
+            const int pos = a.st ? a.st->pos : a.pos_imm;
+            const float *rt = a.rope_tab + (size_t)(pos - a.rope_row0) * a.hd;
+            if (step == 0) {
+                const float x1 = __shfl_xor(acc, nch, SPY_WAVE);
+                if (owner && oj == 0 && ogw < a.d) {
+                    const int row = (2 * ogw) % a.d, k2 = row % a.hd;
+                    const float c = rt[k2], sn = rt[k2 + 1];
+                    // (x0, x1) -> (x0*c - x1*s, x0*s + x1*c), every product rounded (non-linear.cpp:349-364)
+                    const float pa_ = acc * c, pb_ = x1 * sn, pc_ = acc * sn, pd_ = x1 * c;
+                    const uint32_t pr = (uint32_t)f2h(pa_ - pb_) | ((uint32_t)f2h(pc_ + pd_) << 16);
+                    if (2 * ogw < a.d) ((uint32_t *)a.q16)[ogw] = pr;                                  // attn_score rounds Q to fp16 (mat.cpp:37)
+                    else ((uint32_t *)(a.kc + (size_t)pos * a.d))[ogw - a.d / 2] = pr;                 // KCache_cpy: [token][head][hd]
+                }
+            } else {
+                if (owner && ogw < a.d) a.vc[(size_t)ogw * a.n_ctx + pos] = f2h(acc);                 // VCache_cpy: [d][C] column pos
+            }
+        }
+    }
+}
+
+// ---- attention scores in the order of Dot<FP16,FP16> -------------------------------------------------------------------
+// One workgroup per XS_TOK cached tokens, all heads: the keys (8 KiB per token, [head][128] fp16) are read coalesced into
+// LDS, then ONE thread per (token, head) key walks the dot exactly as vec_dot.h:124-145 does for n = 128: accumulators
+// sum[j][l] over the chunks i = 0, 32, 64 (i + 32 < n), the reduction tree of FP16::block_reduce, then the scalar tail
+// over elements 96..127 (a product of two fp16 values is exact in fp32, so `tail += a * b` is the fma it is written as
+// here), result = tail + simd.  Stored: t = dot * scale (mask 0, then * scale: non-linear.cpp:141-150).
+#define XS_TOK 8
+static inline size_t xattn_scores_lds(int n_head) { return (size_t)(XS_TOK + 1) * n_head * 16 * 16; }
+template <int DUMMY>
+__global__ __launch_bounds__(256) void xattn_scores_kernel(const dev_state *st, int pos_imm, const uint16_t *__restrict__ q16, const uint16_t *__restrict__ kc,
+                                                           float *__restrict__ scores, int n_head, int n_ctx, float scale) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const int n_kv = (st ? st->pos : pos_imm) + 1;
+    const int t0 = blockIdx.x * XS_TOK;
+    if (t0 >= n_kv) return;
+    const int d = n_head * 128, tid = threadIdx.x;
+    uint4 *s_k = (uint4 *)smem;                         // [XS_TOK][n_head][16 chunks of 16 bytes], chunk index rotated per key against bank conflicts
+    uint4 *s_qh = s_k + XS_TOK * n_head * 16;           // [n_head][16]
+    const int nchunk = XS_TOK * n_head * 16;
+    for (int c = tid; c < nchunk; c += 256) {
+        const int tt = c / (n_head * 16), rem = c % (n_head * 16), hh = rem >> 4, ch = rem & 15;
+        const int tok = min(t0 + tt, n_kv - 1);
+        s_k[(tt * n_head + hh) * 16 + ((ch + tt + 8 * (hh & 1)) & 15)] = *(const uint4 *)(kc + (size_t)tok * d + hh * 128 + ch * 8);
+    }
+    for (int c = tid; c < n_head * 16; c += 256) s_qh[c] = *(const uint4 *)(q16 + c * 8);
+    __syncthreads();
+    for (int key = tid; key < XS_TOK * n_head; key += 256) {
+        const int hh = key / XS_TOK, tt = key % XS_TOK;
+        if (t0 + tt >= n_kv) continue;
+        const uint4 *kp = s_k + (tt * n_head + hh) * 16, *qp = s_qh + hh * 16;
+        const int rot = tt + 8 * (hh & 1);
+        float sum[4][8];
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int l = 0; l < 8; l++) sum[j][l] = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 3; i++)                      // chunks of 32 elements = 4 x 16 bytes
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const uint4 kv = kp[(4 * i + j + rot) & 15], qv = qp[4 * i + j];
+                const uint32_t kw[4] = {kv.x, kv.y, kv.z, kv.w}, qw[4] = {qv.x, qv.y, qv.z, qv.w};
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    sum[j][2 * e] = fmaf(h2f((uint16_t)(kw[e] & 0xFFFFu)), h2f((uint16_t)(qw[e] & 0xFFFFu)), sum[j][2 * e]);
+                    sum[j][2 * e + 1] = fmaf(h2f((uint16_t)(kw[e] >> 16)), h2f((uint16_t)(qw[e] >> 16)), sum[j][2 * e + 1]);
+                }
+            }
+#pragma unroll
+        for (int l = 0; l < 8; l++) { sum[0][l] += sum[2][l]; sum[1][l] += sum[3][l]; }
+#pragma unroll
+        for (int l = 0; l < 8; l++) sum[0][l] += sum[1][l];
+        const float u0 = sum[0][0] + sum[0][4], u1 = sum[0][1] + sum[0][5], u2 = sum[0][2] + sum[0][6], u3 = sum[0][3] + sum[0][7];
+        const float v0 = u0 + u1, v1 = u2 + u3;
+        const float simd = v0 + v1;
+        float tail = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint4 kv = kp[(12 + j + rot) & 15], qv = qp[12 + j];
+            const uint32_t kw[4] = {kv.x, kv.y, kv.z, kv.w}, qw[4] = {qv.x, qv.y, qv.z, qv.w};
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                tail = fmaf(h2f((uint16_t)(kw[e] & 0xFFFFu)), h2f((uint16_t)(qw[e] & 0xFFFFu)), tail);
+                tail = fmaf(h2f((uint16_t)(kw[e] >> 16)), h2f((uint16_t)(qw[e] >> 16)), tail);
+            }
+        }
+        scores[(size_t)hh * n_ctx + t0 + tt] = (tail + simd) * scale;
+    }
+}
+
+// ---- softmax + P.V^T in the host order ---------------------------------------------------------------------------------
+// One 1024-thread workgroup per (head, 16 rows of V^T).  Softmax (non-linear.cpp:129-180): m = max t; e = exp_table[fp16(t - m)];
+// sum = std::reduce(e) = groups of four added to one running sum, then the last n % 4 elements; p = e * (1 / sum), rounded to
+// fp16 for the product (mat.cpp:37).  P.V^T (vec_dot.h:124-145 with n = n_kv): output row r has 4 x 8 accumulators,
+// accumulator (j, l) adds elements 32 i + 8 j + l for every chunk with 32 i + 32 < n_kv; 32 lanes hold the accumulators of one
+// row (two rows per wave, the 16 rows in waves 0..7) and read V^T and P from LDS, where the 16 waves put them slab by slab
+// (XP_SLAB tokens, coalesced 16-byte loads); tree, scalar tail (the last 1..32 elements, by the lane of accumulator 0).
+#define XP_THREADS 1024
+#define XP_SLAB 1024                       // tokens per slab: 16 rows x 2 KiB
+#define XP_VSTRIDE (XP_SLAB + 32)          // halfs between two rows of a slab in LDS: +64 bytes, the two rows of a wave use different banks
+static inline size_t xattn_pv_lds(int n_ctx) { return (size_t)n_ctx * 4 + (size_t)((n_ctx / 4 + 3) & ~3) * 4 + (size_t)((n_ctx + 32 + 7) & ~7) * 2 + (size_t)16 * XP_VSTRIDE * 2; }
+template <int DUMMY>
+__global__ __launch_bounds__(XP_THREADS) void xattn_pv_kernel(const dev_state *st, int pos_imm, const float *__restrict__ scores, const uint16_t *__restrict__ vc,
+                                                              float *__restrict__ attn_out, const float *__restrict__ lut, int n_ctx) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    __shared__ float s_red[16];
+    __shared__ float s_sum;
+    const int n_kv = (st ? st->pos : pos_imm) + 1;
+    const int head = blockIdx.x >> 3, dgrp = blockIdx.x & 7;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    float *s_e = (float *)smem;                                       // n_ctx floats: t, then e
+    float *s_grp = s_e + n_ctx;                                       // n_ctx / 4 group sums (+ pad to 16 bytes)
+    uint16_t *s_p = (uint16_t *)(s_grp + ((n_ctx / 4 + 3) & ~3));     // n_ctx + 32 halfs: the probabilities as fp16
+    uint16_t *s_v = s_p + ((n_ctx + 32 + 7) & ~7);                    // 16 x XP_VSTRIDE halfs: a slab of the 16 V^T rows
+    const float *srow = scores + (size_t)head * n_ctx;
+    // ---- softmax ----
+    float mx = -INFINITY;
+    for (int j = tid; j < n_kv; j += XP_THREADS) { const float t = srow[j]; s_e[j] = t; mx = fmaxf(mx, t); }
+    mx = wave_max(mx);
+    if (lane == 0) s_red[wave] = mx;
+    __syncthreads();
+    mx = s_red[0];
+#pragma unroll
+    for (int w = 1; w < 16; w++) mx = fmaxf(mx, s_red[w]);
+    for (int j = tid; j < n_kv; j += XP_THREADS) s_e[j] = lut[f2h(s_e[j] - mx)];
+    __syncthreads();
+    const int ngrp = n_kv / 4;
+    for (int g = tid; g < ngrp; g += XP_THREADS) {
+        const float4 v = *(const float4 *)(s_e + 4 * g);
+        const float v1 = v.x + v.y, v2 = v.z + v.w;
+        s_grp[g] = v1 + v2;
+    }
+    __syncthreads();
+    if (wave == 0) {
+        float init = 0.0f;
+        int g = 0;
+        for (; g + 4 <= ngrp; g += 4) { const float4 v = *(const float4 *)(s_grp + g); init = init + v.x; init = init + v.y; init = init + v.z; init = init + v.w; }
+        for (; g < ngrp; g++) init = init + s_grp[g];
+        for (int j = ngrp * 4; j < n_kv; j++) init = init + s_e[j];
+        if (lane == 0) s_sum = init;
+    }
+    __syncthreads();
+    const float inv = 1.0f / s_sum;
+    for (int j = tid; j < n_kv; j += XP_THREADS) s_p[j] = f2h(s_e[j] * inv);
+    // ---- P . V^T ----
+    const int nfull = (n_kv - 1) / 32;                                // chunks with 32 i + 32 < n_kv
+    const int r16 = wave * 2 + (lane >> 5), cl = lane & 31;           // row of the 16 (waves 0..7) and accumulator 8 j + l
+    const uint16_t *vbase = vc + (size_t)(head * 128 + dgrp * 16) * n_ctx;
+    float acc = 0.0f, tail = 0.0f;
+    for (int s0 = 0; s0 < n_kv; s0 += XP_SLAB) {
+        __syncthreads();                                              // the previous slab has been read (first pass: s_p is complete)
+        // 16 rows x XP_SLAB tokens = 2048 pieces of 16 bytes, two per thread; pieces beyond the cached tokens re-read the last one
+        for (int c = tid; c < 16 * (XP_SLAB / 8); c += XP_THREADS) {
+            const int rr = c / (XP_SLAB / 8), pc = c % (XP_SLAB / 8);
+            const int tok = min(s0 + pc * 8, ((n_kv - 1) >> 3) << 3);
+            *(uint4 *)(s_v + rr * XP_VSTRIDE + pc * 8) = *(const uint4 *)(vbase + (size_t)rr * n_ctx + tok);
+        }
+        __syncthreads();
+        if (wave < 8) {
+            const int i0 = s0 / 32, i1 = min(nfull, (s0 + XP_SLAB) / 32);
+            const uint16_t *vr = s_v + r16 * XP_VSTRIDE - s0;
+            for (int i = i0; i < i1; i++) acc = fmaf(h2f(vr[32 * i + cl]), h2f(s_p[32 * i + cl]), acc);
+            if (cl == 0) {                                            // the scalar tail: elements 32 nfull .. n_kv - 1, those of them in this slab
+                const int e0 = max(32 * nfull, s0), e1 = min(n_kv, s0 + XP_SLAB);
+                for (int e = e0; e < e1; e++) tail = fmaf(h2f(vr[e]), h2f(s_p[e]), tail);
+            }
+        }
+    }
+    if (wave < 8) {
+        acc += __shfl_xor(acc, 16, SPY_WAVE);         // sum[0] += sum[2], sum[1] += sum[3]
+        acc += __shfl_xor(acc, 8, SPY_WAVE);          // sum[0] += sum[1]
+        acc += __shfl_xor(acc, 4, SPY_WAVE);          // t_l = sum[0][l] + sum[0][l + 4]
+        acc += __shfl_xor(acc, 1, SPY_WAVE);          // t_0 + t_1, t_2 + t_3
+        acc += __shfl_xor(acc, 2, SPY_WAVE);          // (t_0 + t_1) + (t_2 + t_3)
+        if (cl == 0) attn_out[head * 128 + dgrp * 16 + r16] = tail + acc;
+    }
+}

@@ -536,6 +536,14 @@ __global__ __launch_bounds__(256) void exact_dots32_kernel(xdesc w, const uint8_
 
 }   // namespace
 
+// the two tables on the device: exp [65536], then silu [65536]
+int spy_exact_luts(const float **lut) {
+    const int rc = ensure_luts();
+    if (rc) return rc;
+    *lut = g_lut;
+    return 0;
+}
+
 int spy_exact_on() {
     if (g_exact < 0) {
         const char *e = getenv("SPY_HIP_EXACT");

@@ -144,7 +144,9 @@ _LAYER_FIELDS = [("attn_norm", "attn_norm"), ("ffn_norm", "ffn_norm"), ("wq", "a
 class Engine:
     """A model resident in HBM (native block layouts, uploaded once) and its token loop."""
 
-    def __init__(self, cfg, tensors, device_id=0):
+    def __init__(self, cfg, tensors, device_id=0, order=None):
+        """order: summation order of the fused single-token pass, 1 = the host backend's (bit-exact results), 0 = this
+        backend's own, None = the library's default (1 where the kernels take the model)"""
         H.init(device_id)
         self.cfg = cfg
         self.L = H.load()
@@ -166,6 +168,14 @@ class Engine:
         h = C.c_void_p()
         H.check(self.L.spy_hip_llama_create(C.byref(d), C.byref(h)), "spy_hip_llama_create")
         self.handle = h
+        if order is not None:
+            self.set_order(order)
+
+    def set_order(self, order):
+        H.check(self.L.spy_hip_llama_set_order(self.handle, int(order)), "spy_hip_llama_set_order")
+
+    def order(self):
+        return self.L.spy_hip_llama_order(self.handle)
 
     def forward(self, tokens, n_past, want_logits=True):
         tokens = np.ascontiguousarray(tokens, dtype=np.int32)

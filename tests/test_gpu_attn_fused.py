@@ -21,9 +21,9 @@ def test_fused_attention_launch_matches_split_kernels(wtype, n_layer, d, H, F, V
     cfg = M.Config(n_layer=n_layer, n_embd=d, n_head=H, n_ff=F, n_vocab=V, n_ctx=C, wtype=wtype)
     tensors = M.synth_model(cfg, seed=13)
     monkeypatch.delenv("SPY_HIP_ATTN_SPLIT", raising=False)
-    fused = M.Engine(cfg, tensors)
+    fused = M.Engine(cfg, tensors, order=0)              # the one-launch attention belongs to the backend's own summation order
     monkeypatch.setenv("SPY_HIP_ATTN_SPLIT", "1")
-    split = M.Engine(cfg, tensors)
+    split = M.Engine(cfg, tensors, order=0)
     ora = OracleModel(cfg, tensors)
     assert fused.fuses_attention() and not split.fuses_attention()
     rng = np.random.default_rng(17)
@@ -67,7 +67,7 @@ def test_bounded_wait_gives_up_with_an_error_and_the_next_pass_is_clean(monkeypa
     cfg = M.Config(n_layer=2, n_embd=1024, n_head=8, n_ff=768, n_vocab=640, n_ctx=72, wtype=O.Q4_0)
     tensors = M.synth_model(cfg, seed=21)
     monkeypatch.delenv("SPY_HIP_ATTN_SPLIT", raising=False)
-    eng, ref = M.Engine(cfg, tensors), M.Engine(cfg, tensors)
+    eng, ref = M.Engine(cfg, tensors, order=0), M.Engine(cfg, tensors, order=0)
     assert eng.fuses_attention()
     rng = np.random.default_rng(3)
     prompt = rng.integers(0, cfg.n_vocab, 9).astype(np.int32)
