@@ -140,7 +140,7 @@ extern "C" int spy_hip_llama_create(const spy_hip_llama_desc *desc, spy_hip_llam
     // the host backend's summation order: cos / sin of every position from the host's libm (theta_0 = pos, theta_{k+1} =
     // theta_k * theta_scale in fp32, non-linear.cpp:304-309), the exp / silu tables, shapes the kernels take
     if (!rc && fused_ok(m) && m->wave && m->hd == 128 && c.n_embd % 128 == 0 && c.n_ff % 128 == 0 && c.n_ff <= 16384 &&
-        xattn_pv_lds(c.n_ctx) <= 160 * 1024 && xattn_scores_lds(c.n_head) <= 160 * 1024) {
+        c.n_ctx <= 512 * XP_NP && xattn_pv_lds(c.n_ctx) <= 160 * 1024 - 256 && xattn_scores_lds(c.n_head) <= 160 * 1024) {
         std::vector<float> tab((size_t)c.n_ctx * m->hd);
         for (int pos = 0; pos < c.n_ctx; pos++) {
             float theta = (float)pos;
@@ -164,7 +164,7 @@ extern "C" int spy_hip_llama_create(const spy_hip_llama_desc *desc, spy_hip_llam
             if (env && env[0] == 'o') m->order = 0;
         }
     }
-#ifdef ATL_STAMPS
+#if defined(ATL_STAMPS) || defined(XDBG_STAMPS)
     if (!rc && getenv("SPY_HIP_STAMPS")) rc = dalloc(m, (void **)&m->stamp_dbg, (128 + 512 * 8) * sizeof(long long), true);
 #endif
     if (rc) { spy_hip_llama_destroy(m); return rc; }
@@ -227,13 +227,13 @@ static int enqueue_one(spy_hip_llama *m, hipStream_t st, int which, int il) {
     if (pass_order(m) == 1 || (m->dry && m->order == 1)) {      // the host backend's summation order: six launches per layer
         if (which == K_SCORES) {
             if (m->dry) return 0;
-            xattn_scores_kernel<0><<<dim3((unsigned)((c.n_ctx + XS_TOK - 1) / XS_TOK)), dim3(256), xattn_scores_lds(c.n_head), st>>>(
+            xattn_scores_kernel<0><<<dim3((unsigned)m->num_cu), dim3(XS_THREADS), xattn_scores_lds(c.n_head), st>>>(
                 m->st, m->pos_imm, m->q16, m->k_cache[il], m->scores, c.n_head, c.n_ctx, 1.0f / sqrtf((float)m->hd));   // SoftmaxParam::scale (attention.cpp:113)
             return SPY_LAUNCH_RC();
         }
         if (which == K_PV) {
             if (m->dry) return 0;
-            xattn_pv_kernel<0><<<dim3((unsigned)(c.n_head * 8)), dim3(XP_THREADS), xattn_pv_lds(c.n_ctx), st>>>(m->st, m->pos_imm, m->scores, m->v_cache[il], m->attn_out, m->lut, c.n_ctx);
+            xattn_pv_kernel<0><<<dim3((unsigned)(c.n_head * 8)), dim3(XP_THREADS), xattn_pv_lds(c.n_ctx), st>>>(m->st, m->pos_imm, m->scores, m->v_cache[il], m->attn_out, m->lut, c.n_ctx, m->stamp_dbg);
             return SPY_LAUNCH_RC();
         }
         const spy_hip_llama_layer &Lx = m->layers[which == K_HEAD ? 0 : il];
@@ -697,7 +697,7 @@ __global__ __launch_bounds__(1024) void stage_dump_kernel(const float *__restric
     int8_t *s_q = (int8_t *)smem;
     int2 *s_meta = (int2 *)(smem + staged_q_bytes(K));
     float *s_grp = (float *)(smem + ((staged_bytes(K) + 15) & ~(size_t)15));
-    if constexpr (ORDER == 1) xg_stage<NITK, NORM>(xv, wv, K, eps, s_q, s_meta, s_grp, &s_sum);
+    if constexpr (ORDER == 1) xg_stage<NITK, NORM>(xv, wv, K, eps, s_q, s_meta, s_grp, &s_sum, []() {});
     else wgv_stage<NITK, NORM>(xv, wv, K, eps, s_q, s_meta, s_red);
     xg_dump_q8(s_q, s_meta, K, out);
 }
@@ -809,7 +809,7 @@ extern "C" int spy_hip_attn_decode(void *stream, int32_t order, const void *q16,
     RC_TRY(f.init(order, n_head * 128, n_head, n_head * 128, 1, n_ctx, SPY_HIP_Q4_0));
     const size_t pv_lds = (size_t)n_ctx * 6 + 16;
     if (order == 1) {
-        if (xattn_pv_lds((int)n_ctx) > 160 * 1024 || xattn_scores_lds(n_head) > 160 * 1024) return SPY_HIP_EUNSUPPORTED;
+        if (n_ctx > 512 * XP_NP || xattn_pv_lds((int)n_ctx) > 160 * 1024 - 256 || xattn_scores_lds(n_head) > 160 * 1024) return SPY_HIP_EUNSUPPORTED;
         RC_TRY(spy_ensure_lds(&f.m, (const void *)xattn_pv_kernel<0>, xattn_pv_lds((int)n_ctx)));
         RC_TRY(spy_ensure_lds(&f.m, (const void *)xattn_scores_kernel<0>, xattn_scores_lds(n_head)));
     } else {

@@ -41,15 +41,54 @@ struct xg_args {
     int n_ctx, d, hd;
     uint8_t *q8_dump;                      // tests: workgroup 0 writes its staged activations here as native Q8_0 blocks
     int pos_imm, rope_row0;                // st == nullptr: the position as a number; first position of rope_tab
+    long long *dbg;                        // measurement builds (-DXDBG_STAMPS): wall-clock stamps of workgroup 0
 };
+#ifdef XDBG_STAMPS
+#define XSTAMP(dbg, i) do { if ((dbg) && blockIdx.x == 0 && threadIdx.x == 0) (dbg)[i] = wall_clock64(); } while (0)
+#else
+#define XSTAMP(dbg, i) do { } while (0)
+#endif
+
+// libstdc++'s std::reduce over the n values at s (LDS, 16-byte aligned; up to 28 floats beyond n may be read, never added): ONE
+// running sum, value after value.  Every lane of the calling wave walks the same chain (same addresses: LDS broadcasts them), so
+// the result is wave-uniform.  The additions are a chain of dependent operations (about 4 ns each); the 128-bit LDS reads of the
+// next sixteen values are requested before the current sixteen additions (two register sets), so their latency hides behind the chain.
+static __device__ __forceinline__ float xg_serial_sum(const float *s, int n, float init) {
+    float4 a[4], b[4];
+    auto ld = [&](float4 (&r)[4], int i) {
+#pragma unroll
+        for (int u = 0; u < 4; u++) r[u] = *(const float4 *)(s + i + 4 * u);
+    };
+    auto run = [&](const float4 (&r)[4]) {
+#pragma unroll
+        for (int u = 0; u < 4; u++) { init = init + r[u].x; init = init + r[u].y; init = init + r[u].z; init = init + r[u].w; }
+    };
+    const int n32 = n & ~31;
+    int i = 0;
+    if (n32) {
+        ld(a, 0);
+        for (; i < n32; i += 32) {
+            ld(b, i + 16);
+            __builtin_amdgcn_sched_barrier(0);
+            run(a);
+            __builtin_amdgcn_sched_barrier(0);
+            if (i + 32 < n32) ld(a, i + 32);
+            __builtin_amdgcn_sched_barrier(0);
+            run(b);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    for (; i < n; i++) init = init + s[i];
+    return init;
+}
 
 // ---- activations: f32 vector -> (RMSNorm * weight ->) Q8_0 in LDS, sums in the host order --------------------------
 // NormRMS (non-linear.cpp:194-223): sum = std::transform_reduce(x, x) = groups of four ((x0^2 + x1^2) + (x2^2 + x3^2))
 // added to one running sum in order; scale = 1 / sqrt(sum / n + eps); y = x * scale; then the Mul node: y * w.
 // The 1024 threads form the group sums (one float4 each per 4096 elements), lane 0 of wave 0 adds them.
-template <int NITK, bool NORM>
+template <int NITK, bool NORM, class Issue>
 static __device__ __forceinline__ void xg_stage(const float4 (&xv)[NITK], const float4 (&wv)[NORM ? NITK : 1], int K, float eps,
-                                                int8_t *s_q, int2 *s_meta, float *s_grp, float *s_sum) {
+                                                int8_t *s_q, int2 *s_meta, float *s_grp, float *s_sum, Issue issue_rows) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     float scale = 1.0f;
     if constexpr (NORM) {
@@ -64,23 +103,17 @@ static __device__ __forceinline__ void xg_stage(const float4 (&xv)[NITK], const 
             }
         }
         __syncthreads();
+        // The weight rows are requested only now: a wave that asks for several rows sits in the issue stage until the memory queue
+        // has room, and a request made earlier would hold up the barrier above for every wave.  Wave 0 walks the sum first.
         if (wave == 0) {
-            float init = 0.0f;
-            const int ng = K / 4;                          // a multiple of 4 (K % 16 == 0)
-            for (int g = 0; g < ng; g += 16) {
-                const float4 a = *(const float4 *)(s_grp + g), b = *(const float4 *)(s_grp + min(g + 4, ng - 4)),
-                             c = *(const float4 *)(s_grp + min(g + 8, ng - 4)), e = *(const float4 *)(s_grp + min(g + 12, ng - 4));
-                init = init + a.x; init = init + a.y; init = init + a.z; init = init + a.w;
-                if (g + 4 < ng) { init = init + b.x; init = init + b.y; init = init + b.z; init = init + b.w; }
-                if (g + 8 < ng) { init = init + c.x; init = init + c.y; init = init + c.z; init = init + c.w; }
-                if (g + 12 < ng) { init = init + e.x; init = init + e.y; init = init + e.z; init = init + e.w; }
-            }
+            const float init = xg_serial_sum(s_grp, K / 4, 0.0f);
             if (lane == 0) *s_sum = init;
         }
+        issue_rows();
         __syncthreads();
         const float mean = *s_sum / (float)K;
         scale = 1.0f / sqrtf(mean + eps);
-    }
+    } else issue_rows();
 #pragma unroll
     for (int j = 0; j < NITK; j++) {
         const int i = tid + j * XG_THREADS;
@@ -208,17 +241,32 @@ static __device__ __forceinline__ void xg_phase1(const uint32_t *w, const act_fr
 }
 
 // ---- phase 2: one lane walks one accumulator over the blocks of a slab ------------------------------------------------
+template <int NCH>
 static __device__ __forceinline__ float xg_chain(const float *P, const float *D, int nblk, float acc) {
-    // nblk % 4 == 0; reads beyond nblk (up to 12 floats) stay inside the row's 128 + 4 floats and are not used
+    // nblk % 4 == 0.  Eight blocks per group, the next group's 128-bit reads requested before the current group's eight dependent
+    // fmas (two register sets, no copies); reads beyond nblk stay inside the row's 128 + 4 floats and are not used.
+    // (Taking the scale products, which the eight lanes of a row share, from one lane per quad through DPP broadcasts cut the LDS
+    // traffic but measured slower: 1.25 instead of 0.8 us per 128 blocks.)
+    float4 pa[2], pb[2], da[2], db[2];
+    auto ld = [&](float4 (&p)[2], float4 (&d)[2], int b) {
+#pragma unroll
+        for (int u = 0; u < 2; u++) { p[u] = *(const float4 *)(P + min(b + 4 * u, XG_NBS - 4)); d[u] = *(const float4 *)(D + min(b + 4 * u, XG_NBS - 4)); }
+    };
+    auto run = [&](const float4 (&p)[2], const float4 (&d)[2], int b) {
+#pragma unroll
+        for (int u = 0; u < 2; u++)
+            if (b + 4 * u < nblk) { acc = fmaf(d[u].x, p[u].x, acc); acc = fmaf(d[u].y, p[u].y, acc); acc = fmaf(d[u].z, p[u].z, acc); acc = fmaf(d[u].w, p[u].w, acc); }
+    };
+    ld(pa, da, 0);
     for (int b = 0; b < nblk; b += 16) {
-        const float4 p0 = *(const float4 *)(P + b), d0 = *(const float4 *)(D + b);
-        const float4 p1 = *(const float4 *)(P + min(b + 4, XG_NBS - 4)), d1 = *(const float4 *)(D + min(b + 4, XG_NBS - 4));
-        const float4 p2 = *(const float4 *)(P + min(b + 8, XG_NBS - 4)), d2 = *(const float4 *)(D + min(b + 8, XG_NBS - 4));
-        const float4 p3 = *(const float4 *)(P + min(b + 12, XG_NBS - 4)), d3 = *(const float4 *)(D + min(b + 12, XG_NBS - 4));
-        acc = fmaf(d0.x, p0.x, acc); acc = fmaf(d0.y, p0.y, acc); acc = fmaf(d0.z, p0.z, acc); acc = fmaf(d0.w, p0.w, acc);
-        if (b + 4 < nblk) { acc = fmaf(d1.x, p1.x, acc); acc = fmaf(d1.y, p1.y, acc); acc = fmaf(d1.z, p1.z, acc); acc = fmaf(d1.w, p1.w, acc); }
-        if (b + 8 < nblk) { acc = fmaf(d2.x, p2.x, acc); acc = fmaf(d2.y, p2.y, acc); acc = fmaf(d2.z, p2.z, acc); acc = fmaf(d2.w, p2.w, acc); }
-        if (b + 12 < nblk) { acc = fmaf(d3.x, p3.x, acc); acc = fmaf(d3.y, p3.y, acc); acc = fmaf(d3.z, p3.z, acc); acc = fmaf(d3.w, p3.w, acc); }
+        ld(pb, db, b + 8);
+        __builtin_amdgcn_sched_barrier(0);
+        run(pa, da, b);
+        __builtin_amdgcn_sched_barrier(0);
+        ld(pa, da, b + 16);
+        __builtin_amdgcn_sched_barrier(0);
+        run(pb, db, b + 8);
+        __builtin_amdgcn_sched_barrier(0);
     }
     return acc;
 }
@@ -267,7 +315,7 @@ __global__ __launch_bounds__(XG_THREADS) void xgemv_kernel(xg_args a) {
         else return a.W0 + (size_t)i * RB;
     };
 
-    // 1. the activation vector, 2. the first rows: all unconditional, in this order (the compute unit serves its requests in order)
+    // 1. the activation vector, 2. the first rows (issue_first): all unconditional, in this order (the compute unit serves its requests in order)
     float4 xv[NITK], wv[NORM ? NITK : 1];
 #pragma unroll
     for (int j = 0; j < NITK; j++) {
@@ -275,22 +323,29 @@ __global__ __launch_bounds__(XG_THREADS) void xgemv_kernel(xg_args a) {
         xv[j] = ((const float4 *)a.x_in)[i];
         if constexpr (NORM) wv[j] = ((const float4 *)a.normw)[i];
     }
-    constexpr int RING = NROW < XG_DEPTH + 1 ? NROW : XG_DEPTH + 1;
+    // rows requested ahead of their use: all of the wave's rows where their registers allow (Q4_0 rows, up to 6), so
+    // that the weights stream in while the serial sum of the norm is walked; XG_DEPTH otherwise
+    constexpr int DEPTH = (NROW <= 6 && wt_traits<WT>::PAIR_DW * NITK <= 9) ? NROW : XG_DEPTH;
+    constexpr int RING = NROW < DEPTH + 1 ? NROW : DEPTH + 1;
     wtile<WT, NITK> t[RING];
     wtile<WTV, NITK> tv;
     auto issue = [&](int r) {
         if (EPI == EPI_QKV && r == 2) load_tile<WTV, 64, NITK>(tv, row_ptr(r), npair, lane);
         else load_tile<WT, 64, NITK>(t[r % RING], row_ptr(r), npair, lane);
     };
-    __builtin_amdgcn_s_barrier();
+    auto issue_first = [&]() {
+        if constexpr (!NORM) __builtin_amdgcn_s_barrier();      // x of every wave ahead of every wave's rows in the compute unit's memory queue
 #pragma unroll
-    for (int r = 0; r < NROW; r++) if (r < XG_DEPTH) issue(r);
+        for (int r = 0; r < NROW; r++) if (r < DEPTH) issue(r);
+    };
 
-    // 3. stage the activations
+    // 3. stage the activations (the first rows are requested inside: after the group sums of the norm, or at once)
     int8_t *s_q = (int8_t *)smem;
     int2 *s_meta = (int2 *)(smem + staged_q_bytes(K));
     float *s_part = (float *)(smem + ((staged_bytes(K) + 15) & ~(size_t)15));      // row slots; the group sums of the norm use the same bytes before
-    xg_stage<NITK, NORM>(xv, wv, K, a.eps, s_q, s_meta, s_part, &s_sum);
+    XSTAMP(a.dbg, 16);
+    xg_stage<NITK, NORM>(xv, wv, K, a.eps, s_q, s_meta, s_part, &s_sum, issue_first);
+    XSTAMP(a.dbg, 17);
     if (a.q8_dump && blockIdx.x == 0) xg_dump_q8(s_q, s_meta, K, a.q8_dump);
     staged_act act; act.q = s_q; act.meta = s_meta;
 
@@ -325,19 +380,23 @@ __global__ __launch_bounds__(XG_THREADS) void xgemv_kernel(xg_args a) {
 #pragma unroll
                 for (int j = 0; j < rows; j++) {
                     const int r = r0 + j;
-                    if (it == 0 && r + XG_DEPTH < NROW) issue(r + XG_DEPTH);      // its ring slot held row r - 1, multiplied in the previous step
+                    if (it == 0 && r + DEPTH < NROW) issue(r + DEPTH);            // its ring slot held row r - 1, multiplied in the previous step
                     float *slot = s_part + (size_t)(wave * rows + j) * SLOTF;
                     if (p < npair) {
                         if (vstep) { if constexpr (WTV != WT) xg_phase1<WTV>(tv.w[it], av, n8, p, lane, slot); else xg_phase1<WTV>(tv.w[it], af, n8, p, lane, slot); }
                         else xg_phase1<WT>(t[r % RING].w[it], af, n8, p, lane, slot);
                     }
                 }
+                XSTAMP(a.dbg, 18 + 3 * (step * NITK + it));
                 __syncthreads();
+                XSTAMP(a.dbg, 19 + 3 * (step * NITK + it));
                 if (tid < chains) {
                     const int slot_i = tid / nch, l = tid % nch;
                     const float *slot = s_part + (size_t)slot_i * SLOTF;
-                    acc = xg_chain(slot + l * (XG_NBS + 4), slot + nch * (XG_NBS + 4), nblk, acc);
+                    if (nch == 8) acc = xg_chain<8>(slot + l * (XG_NBS + 4), slot + nch * (XG_NBS + 4), nblk, acc);
+                    else acc = xg_chain<1>(slot + l * (XG_NBS + 4), slot + nch * (XG_NBS + 4), nblk, acc);
                 }
+                XSTAMP(a.dbg, 20 + 3 * (step * NITK + it));
                 __syncthreads();
             }
         }
@@ -376,111 +435,152 @@ __global__ __launch_bounds__(XG_THREADS) void xgemv_kernel(xg_args a) {
 }
 
 // ---- attention scores in the order of Dot<FP16,FP16> -------------------------------------------------------------------
-// One workgroup per XS_TOK cached tokens, all heads: the keys (8 KiB per token, [head][128] fp16) are read coalesced into
-// LDS, then ONE thread per (token, head) key walks the dot exactly as vec_dot.h:124-145 does for n = 128: accumulators
-// sum[j][l] over the chunks i = 0, 32, 64 (i + 32 < n), the reduction tree of FP16::block_reduce, then the scalar tail
-// over elements 96..127 (a product of two fp16 values is exact in fp32, so `tail += a * b` is the fma it is written as
-// here), result = tail + simd.  Stored: t = dot * scale (mask 0, then * scale: non-linear.cpp:141-150).
-#define XS_TOK 8
+// The cached tokens are dealt out evenly over the workgroups (one per compute unit): workgroup b takes tokens
+// b * tpw .. (b + 1) * tpw - 1, tpw = ceil(n_kv / workgroups), all heads, in rounds of XS_TOK tokens.  The keys of a round
+// (8 KiB per token, [head][128] fp16) are read coalesced, eight 16-byte pieces per thread all requested at once, and laid
+// into LDS; then ONE thread per (token, head) key walks the dot exactly as vec_dot.h:124-145 does for n = 128:
+// accumulators sum[j][l] over the chunks i = 0, 32, 64 (i + 32 < n), the reduction tree of FP16::block_reduce, then the
+// scalar tail over elements 96..127 (a product of two fp16 values is exact in fp32, so `tail += a * b` is the fma it is
+// written as here), result = tail + simd.  Stored: t = dot * scale (mask 0, then * scale: non-linear.cpp:141-150).
+#define XS_THREADS 1024
+#define XS_TOK 16
 static inline size_t xattn_scores_lds(int n_head) { return (size_t)(XS_TOK + 1) * n_head * 16 * 16; }
 template <int DUMMY>
-__global__ __launch_bounds__(256) void xattn_scores_kernel(const dev_state *st, int pos_imm, const uint16_t *__restrict__ q16, const uint16_t *__restrict__ kc,
-                                                           float *__restrict__ scores, int n_head, int n_ctx, float scale) {
+__global__ __launch_bounds__(XS_THREADS) void xattn_scores_kernel(const dev_state *st, int pos_imm, const uint16_t *__restrict__ q16, const uint16_t *__restrict__ kc,
+                                                                  float *__restrict__ scores, int n_head, int n_ctx, float scale) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int n_kv = (st ? st->pos : pos_imm) + 1;
-    const int t0 = blockIdx.x * XS_TOK;
-    if (t0 >= n_kv) return;
+    const int tpw = (n_kv + (int)gridDim.x - 1) / (int)gridDim.x;
+    const int t_begin = blockIdx.x * tpw, t_end = min(n_kv, t_begin + tpw);
+    if (t_begin >= t_end) return;
     const int d = n_head * 128, tid = threadIdx.x;
     uint4 *s_k = (uint4 *)smem;                         // [XS_TOK][n_head][16 chunks of 16 bytes], chunk index rotated per key against bank conflicts
     uint4 *s_qh = s_k + XS_TOK * n_head * 16;           // [n_head][16]
-    const int nchunk = XS_TOK * n_head * 16;
-    for (int c = tid; c < nchunk; c += 256) {
-        const int tt = c / (n_head * 16), rem = c % (n_head * 16), hh = rem >> 4, ch = rem & 15;
-        const int tok = min(t0 + tt, n_kv - 1);
-        s_k[(tt * n_head + hh) * 16 + ((ch + tt + 8 * (hh & 1)) & 15)] = *(const uint4 *)(kc + (size_t)tok * d + hh * 128 + ch * 8);
-    }
-    for (int c = tid; c < n_head * 16; c += 256) s_qh[c] = *(const uint4 *)(q16 + c * 8);
-    __syncthreads();
-    for (int key = tid; key < XS_TOK * n_head; key += 256) {
-        const int hh = key / XS_TOK, tt = key % XS_TOK;
-        if (t0 + tt >= n_kv) continue;
-        const uint4 *kp = s_k + (tt * n_head + hh) * 16, *qp = s_qh + hh * 16;
-        const int rot = tt + 8 * (hh & 1);
-        float sum[4][8];
+    const int per_tok = n_head * 16;                    // 16-byte pieces per token
+    for (int c = tid; c < per_tok; c += XS_THREADS) s_qh[c] = *(const uint4 *)(q16 + c * 8);
+    for (int t0 = t_begin; t0 < t_end; t0 += XS_TOK) {
+        const int nt = min(XS_TOK, t_end - t0), npiece = nt * per_tok;
+        if (t0 != t_begin) __syncthreads();             // the previous round's keys have been read
+        constexpr int NLD = 8;                          // pieces per thread requested together: 1024 x 8 x 16 bytes = 16 tokens of 32 heads
+        for (int c0 = 0; c0 < npiece; c0 += NLD * XS_THREADS) {
+            uint4 kreg[NLD];
 #pragma unroll
-        for (int j = 0; j < 4; j++)
+            for (int u = 0; u < NLD; u++) {
+                const int c = min(c0 + u * XS_THREADS + tid, npiece - 1);
+                const int tt = c / per_tok, rem = c - tt * per_tok;
+                kreg[u] = *(const uint4 *)(kc + (size_t)(t0 + tt) * d + rem * 8);
+            }
 #pragma unroll
-            for (int l = 0; l < 8; l++) sum[j][l] = 0.0f;
+            for (int u = 0; u < NLD; u++) {
+                const int c = c0 + u * XS_THREADS + tid;
+                if (c < npiece) {
+                    const int tt = c / per_tok, rem = c - tt * per_tok, hh = rem >> 4, ch = rem & 15;
+                    s_k[(tt * n_head + hh) * 16 + ((ch + tt + 8 * (hh & 1)) & 15)] = kreg[u];
+                }
+            }
+        }
+        __syncthreads();
+        for (int key = tid; key < nt * n_head; key += XS_THREADS) {
+            const int hh = key / nt, tt = key - hh * nt;
+            const uint4 *kp = s_k + (tt * n_head + hh) * 16, *qp = s_qh + hh * 16;
+            const int rot = tt + 8 * (hh & 1);
+            float sum[4][8];
 #pragma unroll
-        for (int i = 0; i < 3; i++)                      // chunks of 32 elements = 4 x 16 bytes
+            for (int j = 0; j < 4; j++)
+#pragma unroll
+                for (int l = 0; l < 8; l++) sum[j][l] = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 3; i++)                  // chunks of 32 elements = 4 x 16 bytes
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const uint4 kv = kp[(4 * i + j + rot) & 15], qv = qp[4 * i + j];
+                    const uint32_t kw[4] = {kv.x, kv.y, kv.z, kv.w}, qw[4] = {qv.x, qv.y, qv.z, qv.w};
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        sum[j][2 * e] = fmaf(h2f((uint16_t)(kw[e] & 0xFFFFu)), h2f((uint16_t)(qw[e] & 0xFFFFu)), sum[j][2 * e]);
+                        sum[j][2 * e + 1] = fmaf(h2f((uint16_t)(kw[e] >> 16)), h2f((uint16_t)(qw[e] >> 16)), sum[j][2 * e + 1]);
+                    }
+                }
+#pragma unroll
+            for (int l = 0; l < 8; l++) { sum[0][l] += sum[2][l]; sum[1][l] += sum[3][l]; }
+#pragma unroll
+            for (int l = 0; l < 8; l++) sum[0][l] += sum[1][l];
+            const float u0 = sum[0][0] + sum[0][4], u1 = sum[0][1] + sum[0][5], u2 = sum[0][2] + sum[0][6], u3 = sum[0][3] + sum[0][7];
+            const float v0 = u0 + u1, v1 = u2 + u3;
+            const float simd = v0 + v1;
+            float tail = 0.0f;
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                const uint4 kv = kp[(4 * i + j + rot) & 15], qv = qp[4 * i + j];
+                const uint4 kv = kp[(12 + j + rot) & 15], qv = qp[12 + j];
                 const uint32_t kw[4] = {kv.x, kv.y, kv.z, kv.w}, qw[4] = {qv.x, qv.y, qv.z, qv.w};
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    sum[j][2 * e] = fmaf(h2f((uint16_t)(kw[e] & 0xFFFFu)), h2f((uint16_t)(qw[e] & 0xFFFFu)), sum[j][2 * e]);
-                    sum[j][2 * e + 1] = fmaf(h2f((uint16_t)(kw[e] >> 16)), h2f((uint16_t)(qw[e] >> 16)), sum[j][2 * e + 1]);
+                    tail = fmaf(h2f((uint16_t)(kw[e] & 0xFFFFu)), h2f((uint16_t)(qw[e] & 0xFFFFu)), tail);
+                    tail = fmaf(h2f((uint16_t)(kw[e] >> 16)), h2f((uint16_t)(qw[e] >> 16)), tail);
                 }
             }
-#pragma unroll
-        for (int l = 0; l < 8; l++) { sum[0][l] += sum[2][l]; sum[1][l] += sum[3][l]; }
-#pragma unroll
-        for (int l = 0; l < 8; l++) sum[0][l] += sum[1][l];
-        const float u0 = sum[0][0] + sum[0][4], u1 = sum[0][1] + sum[0][5], u2 = sum[0][2] + sum[0][6], u3 = sum[0][3] + sum[0][7];
-        const float v0 = u0 + u1, v1 = u2 + u3;
-        const float simd = v0 + v1;
-        float tail = 0.0f;
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const uint4 kv = kp[(12 + j + rot) & 15], qv = qp[12 + j];
-            const uint32_t kw[4] = {kv.x, kv.y, kv.z, kv.w}, qw[4] = {qv.x, qv.y, qv.z, qv.w};
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                tail = fmaf(h2f((uint16_t)(kw[e] & 0xFFFFu)), h2f((uint16_t)(qw[e] & 0xFFFFu)), tail);
-                tail = fmaf(h2f((uint16_t)(kw[e] >> 16)), h2f((uint16_t)(qw[e] >> 16)), tail);
-            }
+            scores[(size_t)hh * n_ctx + t0 + tt] = (tail + simd) * scale;
         }
-        scores[(size_t)hh * n_ctx + t0 + tt] = (tail + simd) * scale;
     }
 }
 
 // ---- softmax + P.V^T in the host order ---------------------------------------------------------------------------------
-// One 1024-thread workgroup per (head, 16 rows of V^T).  Softmax (non-linear.cpp:129-180): m = max t; e = exp_table[fp16(t - m)];
-// sum = std::reduce(e) = groups of four added to one running sum, then the last n % 4 elements; p = e * (1 / sum), rounded to
-// fp16 for the product (mat.cpp:37).  P.V^T (vec_dot.h:124-145 with n = n_kv): output row r has 4 x 8 accumulators,
-// accumulator (j, l) adds elements 32 i + 8 j + l for every chunk with 32 i + 32 < n_kv; 32 lanes hold the accumulators of one
-// row (two rows per wave, the 16 rows in waves 0..7) and read V^T and P from LDS, where the 16 waves put them slab by slab
-// (XP_SLAB tokens, coalesced 16-byte loads); tree, scalar tail (the last 1..32 elements, by the lane of accumulator 0).
+// One 1024-thread workgroup per (head, 16 rows of V^T); wave w streams row w into registers (16-byte pieces, all requested
+// before the softmax's serial sum so that the row arrives while that sum is walked).
+// Softmax (non-linear.cpp:129-180): m = max t; e = exp_table[fp16(t - m)]; sum = std::reduce(e) = groups of four added to
+// one running sum, then the last n % 4 elements; p = e * (1 / sum), rounded to fp16 for the product (mat.cpp:37).
+// P.V^T (vec_dot.h:124-145 with n = n_kv): output row r has 4 x 8 accumulators, accumulator (j, l) adds elements
+// 32 i + 8 j + l for every chunk with 32 i + 32 < n_kv.  The 16 waves lay their rows into LDS; then 32 lanes hold the
+// accumulators of one row (two rows per wave, the 16 rows in waves 0..7) and read V^T and P from LDS; tree; scalar tail (the
+// last 1..32 elements, by the lane of accumulator 0).
 #define XP_THREADS 1024
-#define XP_SLAB 1024                       // tokens per slab: 16 rows x 2 KiB
-#define XP_VSTRIDE (XP_SLAB + 32)          // halfs between two rows of a slab in LDS: +64 bytes, the two rows of a wave use different banks
-static inline size_t xattn_pv_lds(int n_ctx) { return (size_t)n_ctx * 4 + (size_t)((n_ctx / 4 + 3) & ~3) * 4 + (size_t)((n_ctx + 32 + 7) & ~7) * 2 + (size_t)16 * XP_VSTRIDE * 2; }
+#define XP_NP 10                           // 16-byte pieces per lane of a V^T row: n_ctx <= 5120
+#define XP_NS 5                            // scores per thread: n_ctx <= 5120
+static inline int xattn_pv_vstride(int n_ctx) { return ((n_ctx + 63) / 64) * 64 + 32; }        // halfs between rows in LDS: = 64 bytes mod 128, the two rows of a wave on different banks
+static inline size_t xattn_pv_lds(int n_ctx) {
+    const size_t p_bytes = (size_t)((n_ctx + 32 + 7) & ~7) * 2, v_bytes = (size_t)16 * xattn_pv_vstride(n_ctx) * 2;
+    const size_t soft = (size_t)n_ctx * 4 + (size_t)((n_ctx / 4 + 3) & ~3) * 4;                  // t / e and the group sums live where the rows go later
+    return p_bytes + (v_bytes > soft ? v_bytes : soft);
+}
 template <int DUMMY>
-__global__ __launch_bounds__(XP_THREADS) void xattn_pv_kernel(const dev_state *st, int pos_imm, const float *__restrict__ scores, const uint16_t *__restrict__ vc,
-                                                              float *__restrict__ attn_out, const float *__restrict__ lut, int n_ctx) {
+__global__ __launch_bounds__(XP_THREADS) void xattn_pv_kernel(const dev_state *st, int pos_imm, const float *__restrict__ scores, const uint16_t *vc,
+                                                              float *attn_out, const float *__restrict__ lut, int n_ctx, long long *dbg) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     __shared__ float s_red[16];
     __shared__ float s_sum;
+    XSTAMP(dbg, 0);
     const int n_kv = (st ? st->pos : pos_imm) + 1;
-    const int head = blockIdx.x >> 3, dgrp = blockIdx.x & 7;
+    const int hd_ = blockIdx.x >> 3, dgrp = blockIdx.x & 7;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    float *s_e = (float *)smem;                                       // n_ctx floats: t, then e
-    float *s_grp = s_e + n_ctx;                                       // n_ctx / 4 group sums (+ pad to 16 bytes)
-    uint16_t *s_p = (uint16_t *)(s_grp + ((n_ctx / 4 + 3) & ~3));     // n_ctx + 32 halfs: the probabilities as fp16
-    uint16_t *s_v = s_p + ((n_ctx + 32 + 7) & ~7);                    // 16 x XP_VSTRIDE halfs: a slab of the 16 V^T rows
-    const float *srow = scores + (size_t)head * n_ctx;
-    // ---- softmax ----
+    const int VS = ((n_ctx + 63) / 64) * 64 + 32;
+    uint16_t *s_p = (uint16_t *)smem;                                 // n_ctx + 32 halfs: the probabilities as fp16
+    uint8_t *region = smem + (size_t)((n_ctx + 32 + 7) & ~7) * 2;
+    float *s_e = (float *)region;                                     // n_ctx floats: e (softmax phase)
+    float *s_grp = s_e + n_ctx;                                       // n_ctx / 4 group sums
+    uint16_t *s_v = (uint16_t *)region;                               // 16 rows x VS halfs (product phase)
+    const float *srow = scores + (size_t)hd_ * n_ctx;
+    const uint16_t *vrow = vc + (size_t)(hd_ * 128 + dgrp * 16 + wave) * n_ctx;
+    // ---- softmax: scores -> registers, maximum ----
+    float sreg[XP_NS];
+#pragma unroll
+    for (int u = 0; u < XP_NS; u++) sreg[u] = srow[min(tid + u * XP_THREADS, n_ctx - 1)];
     float mx = -INFINITY;
-    for (int j = tid; j < n_kv; j += XP_THREADS) { const float t = srow[j]; s_e[j] = t; mx = fmaxf(mx, t); }
+#pragma unroll
+    for (int u = 0; u < XP_NS; u++) if (tid + u * XP_THREADS < n_kv) mx = fmaxf(mx, sreg[u]);
     mx = wave_max(mx);
     if (lane == 0) s_red[wave] = mx;
     __syncthreads();
     mx = s_red[0];
 #pragma unroll
     for (int w = 1; w < 16; w++) mx = fmaxf(mx, s_red[w]);
-    for (int j = tid; j < n_kv; j += XP_THREADS) s_e[j] = lut[f2h(s_e[j] - mx)];
+    XSTAMP(dbg, 1);
+    // exponentials from the table
+#pragma unroll
+    for (int u = 0; u < XP_NS; u++) sreg[u] = lut[f2h(sreg[u] - mx)];
+#pragma unroll
+    for (int u = 0; u < XP_NS; u++) { const int j = tid + u * XP_THREADS; if (j < n_kv) s_e[j] = sreg[u]; }
     __syncthreads();
+    XSTAMP(dbg, 2);
     const int ngrp = n_kv / 4;
     for (int g = tid; g < ngrp; g += XP_THREADS) {
         const float4 v = *(const float4 *)(s_e + 4 * g);
@@ -488,47 +588,75 @@ __global__ __launch_bounds__(XP_THREADS) void xattn_pv_kernel(const dev_state *s
         s_grp[g] = v1 + v2;
     }
     __syncthreads();
-    if (wave == 0) {
-        float init = 0.0f;
-        int g = 0;
-        for (; g + 4 <= ngrp; g += 4) { const float4 v = *(const float4 *)(s_grp + g); init = init + v.x; init = init + v.y; init = init + v.z; init = init + v.w; }
-        for (; g < ngrp; g++) init = init + s_grp[g];
+    XSTAMP(dbg, 3);
+    // The V^T rows are requested now, by every wave but the one that walks the sum (a wave that asks for its whole row sits in the
+    // issue stage until the memory queue has room, i.e. for most of the row's transfer time): the rows arrive while the sum is walked.
+    // vc is not a restrict pointer on purpose: the loads must stay between the two barriers around them.
+    uint4 vb0, vb1, vb2, vb3, vb4, vb5, vb6, vb7, vb8, vb9;
+    const int last_piece = (n_kv - 1) >> 3;
+    auto load_row = [&]() {
+        const uint16_t *vp = vrow;
+        vb0 = *(const uint4 *)(vp + (size_t)min(0 * 64 + lane, last_piece) * 8); vb1 = *(const uint4 *)(vp + (size_t)min(1 * 64 + lane, last_piece) * 8);
+        vb2 = *(const uint4 *)(vp + (size_t)min(2 * 64 + lane, last_piece) * 8); vb3 = *(const uint4 *)(vp + (size_t)min(3 * 64 + lane, last_piece) * 8);
+        vb4 = *(const uint4 *)(vp + (size_t)min(4 * 64 + lane, last_piece) * 8); vb5 = *(const uint4 *)(vp + (size_t)min(5 * 64 + lane, last_piece) * 8);
+        vb6 = *(const uint4 *)(vp + (size_t)min(6 * 64 + lane, last_piece) * 8); vb7 = *(const uint4 *)(vp + (size_t)min(7 * 64 + lane, last_piece) * 8);
+        vb8 = *(const uint4 *)(vp + (size_t)min(8 * 64 + lane, last_piece) * 8); vb9 = *(const uint4 *)(vp + (size_t)min(9 * 64 + lane, last_piece) * 8);
+    };
+    if (wave != 0) load_row();
+    else {
+        float init = xg_serial_sum(s_grp, ngrp, 0.0f);
         for (int j = ngrp * 4; j < n_kv; j++) init = init + s_e[j];
         if (lane == 0) s_sum = init;
+        load_row();
     }
     __syncthreads();
+    XSTAMP(dbg, 4);
     const float inv = 1.0f / s_sum;
-    for (int j = tid; j < n_kv; j += XP_THREADS) s_p[j] = f2h(s_e[j] * inv);
-    // ---- P . V^T ----
-    const int nfull = (n_kv - 1) / 32;                                // chunks with 32 i + 32 < n_kv
-    const int r16 = wave * 2 + (lane >> 5), cl = lane & 31;           // row of the 16 (waves 0..7) and accumulator 8 j + l
-    const uint16_t *vbase = vc + (size_t)(head * 128 + dgrp * 16) * n_ctx;
-    float acc = 0.0f, tail = 0.0f;
-    for (int s0 = 0; s0 < n_kv; s0 += XP_SLAB) {
-        __syncthreads();                                              // the previous slab has been read (first pass: s_p is complete)
-        // 16 rows x XP_SLAB tokens = 2048 pieces of 16 bytes, two per thread; pieces beyond the cached tokens re-read the last one
-        for (int c = tid; c < 16 * (XP_SLAB / 8); c += XP_THREADS) {
-            const int rr = c / (XP_SLAB / 8), pc = c % (XP_SLAB / 8);
-            const int tok = min(s0 + pc * 8, ((n_kv - 1) >> 3) << 3);
-            *(uint4 *)(s_v + rr * XP_VSTRIDE + pc * 8) = *(const uint4 *)(vbase + (size_t)rr * n_ctx + tok);
-        }
-        __syncthreads();
-        if (wave < 8) {
-            const int i0 = s0 / 32, i1 = min(nfull, (s0 + XP_SLAB) / 32);
-            const uint16_t *vr = s_v + r16 * XP_VSTRIDE - s0;
-            for (int i = i0; i < i1; i++) acc = fmaf(h2f(vr[32 * i + cl]), h2f(s_p[32 * i + cl]), acc);
-            if (cl == 0) {                                            // the scalar tail: elements 32 nfull .. n_kv - 1, those of them in this slab
-                const int e0 = max(32 * nfull, s0), e1 = min(n_kv, s0 + XP_SLAB);
-                for (int e = e0; e < e1; e++) tail = fmaf(h2f(vr[e]), h2f(s_p[e]), tail);
-            }
-        }
+#pragma unroll
+    for (int u = 0; u < XP_NS; u++) { const int j = tid + u * XP_THREADS; if (j < n_kv) s_p[j] = f2h(sreg[u] * inv); }
+    // ---- the rows into LDS (s_e / s_grp are dead: every thread passed the barrier after the sum) ----
+    {
+        uint16_t *dst = s_v + (size_t)wave * VS + lane * 8;
+        if (0 * 64 + lane <= last_piece) *(uint4 *)(dst + 0 * 512) = vb0;
+        if (1 * 64 + lane <= last_piece) *(uint4 *)(dst + 1 * 512) = vb1;
+        if (2 * 64 + lane <= last_piece) *(uint4 *)(dst + 2 * 512) = vb2;
+        if (3 * 64 + lane <= last_piece) *(uint4 *)(dst + 3 * 512) = vb3;
+        if (4 * 64 + lane <= last_piece) *(uint4 *)(dst + 4 * 512) = vb4;
+        if (5 * 64 + lane <= last_piece) *(uint4 *)(dst + 5 * 512) = vb5;
+        if (6 * 64 + lane <= last_piece) *(uint4 *)(dst + 6 * 512) = vb6;
+        if (7 * 64 + lane <= last_piece) *(uint4 *)(dst + 7 * 512) = vb7;
+        if (8 * 64 + lane <= last_piece) *(uint4 *)(dst + 8 * 512) = vb8;
+        if (9 * 64 + lane <= last_piece) *(uint4 *)(dst + 9 * 512) = vb9;
     }
+    __syncthreads();
+    XSTAMP(dbg, 5);
+    // ---- P . V^T ----
     if (wave < 8) {
+        const int nfull = (n_kv - 1) / 32;                            // chunks with 32 i + 32 < n_kv
+        const int r16 = wave * 2 + (lane >> 5), cl = lane & 31;       // row of the 16 and accumulator 8 j + l
+        const uint16_t *vr = s_v + (size_t)r16 * VS + cl, *pr = s_p + cl;
+        float acc = 0.0f;
+        int i = 0;
+        for (; i + 8 <= nfull; i += 8) {
+            const uint16_t v0 = vr[32 * i], v1 = vr[32 * i + 32], v2 = vr[32 * i + 64], v3 = vr[32 * i + 96], v4 = vr[32 * i + 128], v5 = vr[32 * i + 160],
+                           v6 = vr[32 * i + 192], v7 = vr[32 * i + 224];
+            const uint16_t p0 = pr[32 * i], p1 = pr[32 * i + 32], p2 = pr[32 * i + 64], p3 = pr[32 * i + 96], p4 = pr[32 * i + 128], p5 = pr[32 * i + 160],
+                           p6 = pr[32 * i + 192], p7 = pr[32 * i + 224];
+            acc = fmaf(h2f(v0), h2f(p0), acc); acc = fmaf(h2f(v1), h2f(p1), acc); acc = fmaf(h2f(v2), h2f(p2), acc); acc = fmaf(h2f(v3), h2f(p3), acc);
+            acc = fmaf(h2f(v4), h2f(p4), acc); acc = fmaf(h2f(v5), h2f(p5), acc); acc = fmaf(h2f(v6), h2f(p6), acc); acc = fmaf(h2f(v7), h2f(p7), acc);
+        }
+        for (; i < nfull; i++) acc = fmaf(h2f(vr[32 * i]), h2f(pr[32 * i]), acc);
+        XSTAMP(dbg, 6);
         acc += __shfl_xor(acc, 16, SPY_WAVE);         // sum[0] += sum[2], sum[1] += sum[3]
         acc += __shfl_xor(acc, 8, SPY_WAVE);          // sum[0] += sum[1]
         acc += __shfl_xor(acc, 4, SPY_WAVE);          // t_l = sum[0][l] + sum[0][l + 4]
         acc += __shfl_xor(acc, 1, SPY_WAVE);          // t_0 + t_1, t_2 + t_3
         acc += __shfl_xor(acc, 2, SPY_WAVE);          // (t_0 + t_1) + (t_2 + t_3)
-        if (cl == 0) attn_out[head * 128 + dgrp * 16 + r16] = tail + acc;
+        if (cl == 0) {                                // the scalar tail: elements 32 nfull .. n_kv - 1
+            float tail = 0.0f;
+            for (int e = 32 * nfull; e < n_kv; e++) tail = fmaf(h2f(vr[e]), h2f(pr[e]), tail);
+            attn_out[hd_ * 128 + dgrp * 16 + r16] = tail + acc;
+        }
+        XSTAMP(dbg, 7);
     }
 }

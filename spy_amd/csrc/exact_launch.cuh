@@ -22,8 +22,11 @@ static int launch_xg(spy_hip_llama *m, hipStream_t st, const xg_args &a, int uni
 }
 
 // rows per wave of the output head and pairs per wave of gate|up, as wave_rows in decode_launch.cuh
+// Q4_0 / Q8_0: 2 rows per wave and step (32 row slots of 4.6 KB fill LDS); K-quant rows have one accumulator and small slots: 4
 template <int WT> struct xg_rows {
-    static constexpr int HEAD_STEPS = (WT == SPY_HIP_Q4_0 || WT == SPY_HIP_Q4_K) ? 4 : 2;      // x 2 rows per step
+    static constexpr bool KQ = WT == SPY_HIP_Q4_K || WT == SPY_HIP_Q6_K;
+    static constexpr int HEAD_RPS = KQ ? 4 : 2;
+    static constexpr int HEAD_STEPS = WT == SPY_HIP_Q4_0 ? 4 : 2;                               // 8 rows per wave (Q8_0: 4: its rows are twice as wide)
     static constexpr int GATEUP_STEPS = 3;
 };
 
@@ -46,10 +49,10 @@ static int enqueue_exact(spy_hip_llama *m, hipStream_t st, int which, int il) {
     xg_args a;
     memset(&a, 0, sizeof(a));
     a.st = m->st; a.rope_tab = m->rope_tab; a.q16 = m->q16; a.lut = m->lut;
-    a.n_ctx = c.n_ctx; a.d = d; a.hd = m->hd; a.eps = c.eps; a.q8_dump = m->q8_dump; a.pos_imm = m->pos_imm; a.rope_row0 = m->rope_row0;
+    a.n_ctx = c.n_ctx; a.d = d; a.hd = m->hd; a.eps = c.eps; a.q8_dump = m->q8_dump; a.pos_imm = m->pos_imm; a.rope_row0 = m->rope_row0; a.dbg = m->stamp_dbg;
     if (which == K_HEAD) {
         a.W0 = (const uint8_t *)c.w_out; a.M = c.n_vocab; a.K = d; a.x_in = m->x; a.normw = c.out_norm; a.out = m->logits;
-        return launch_xg<WT, 1, 2, xg_rows<WT>::HEAD_STEPS, EPI_STORE>(m, st, a, a.M);
+        return launch_xg<WT, 1, xg_rows<WT>::HEAD_RPS, xg_rows<WT>::HEAD_STEPS, EPI_STORE>(m, st, a, a.M);
     }
     const spy_hip_llama_layer &L = m->layers[il];
     a.kc = m->k_cache[il]; a.vc = m->v_cache[il];
