@@ -704,7 +704,7 @@ __global__ __launch_bounds__(1024) void stage_dump_kernel(const float *__restric
 
 template <int ORDER, bool NORM>
 int stage_dump(hipStream_t st, const float *x, const float *normw, float eps, int64_t K, void *yq) {
-    const size_t lds = ((staged_bytes(K) + 15) & ~(size_t)15) + (size_t)K;          // + K / 4 group sums
+    const size_t lds = ((staged_bytes(K) + 15) & ~(size_t)15) + (size_t)K + 256;    // + K / 4 group sums (+ what the serial sum reads ahead)
     switch ((K + 4095) / 4096) {
     case 1: stage_dump_kernel<ORDER, 1, NORM><<<dim3(1), dim3(1024), lds, st>>>(x, normw, eps, (int)K, (uint8_t *)yq); break;
     case 2: stage_dump_kernel<ORDER, 2, NORM><<<dim3(1), dim3(1024), lds, st>>>(x, normw, eps, (int)K, (uint8_t *)yq); break;

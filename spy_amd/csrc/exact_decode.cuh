@@ -49,32 +49,38 @@ struct xg_args {
 #define XSTAMP(dbg, i) do { } while (0)
 #endif
 
-// libstdc++'s std::reduce over the n values at s (LDS, 16-byte aligned; up to 28 floats beyond n may be read, never added): ONE
+// libstdc++'s std::reduce over the n values at s (LDS, 16-byte aligned; up to 40 floats beyond n may be read, never added): ONE
 // running sum, value after value.  Every lane of the calling wave walks the same chain (same addresses: LDS broadcasts them), so
 // the result is wave-uniform.  The additions are a chain of dependent operations (about 4 ns each); the 128-bit LDS reads of the
 // next sixteen values are requested before the current sixteen additions (two register sets), so their latency hides behind the chain.
 static __device__ __forceinline__ float xg_serial_sum(const float *s, int n, float init) {
-    float4 a[4], b[4];
-    auto ld = [&](float4 (&r)[4], int i) {
+    float4 a[2], b[2], c[2];
+    auto ld = [&](float4 (&r)[2], int i) {
 #pragma unroll
-        for (int u = 0; u < 4; u++) r[u] = *(const float4 *)(s + i + 4 * u);
+        for (int u = 0; u < 2; u++) r[u] = *(const float4 *)(s + i + 4 * u);
     };
-    auto run = [&](const float4 (&r)[4]) {
+    auto run = [&](const float4 (&r)[2]) {
 #pragma unroll
-        for (int u = 0; u < 4; u++) { init = init + r[u].x; init = init + r[u].y; init = init + r[u].z; init = init + r[u].w; }
+        for (int u = 0; u < 2; u++) { init = init + r[u].x; init = init + r[u].y; init = init + r[u].z; init = init + r[u].w; }
     };
-    const int n32 = n & ~31;
+    // groups of 8 values, each requested two groups (sixteen dependent additions) ahead of its use: three register sets in rotation
+    const int n24 = n - n % 24;
     int i = 0;
-    if (n32) {
+    if (n24) {
         ld(a, 0);
-        for (; i < n32; i += 32) {
-            ld(b, i + 16);
+        ld(b, 8);
+        for (; i < n24; i += 24) {
+            ld(c, i + 16);
             __builtin_amdgcn_sched_barrier(0);
             run(a);
             __builtin_amdgcn_sched_barrier(0);
-            if (i + 32 < n32) ld(a, i + 32);
+            ld(a, i + 24);                               // up to 28 floats beyond n: read, never added
             __builtin_amdgcn_sched_barrier(0);
             run(b);
+            __builtin_amdgcn_sched_barrier(0);
+            ld(b, i + 32);
+            __builtin_amdgcn_sched_barrier(0);
+            run(c);
             __builtin_amdgcn_sched_barrier(0);
         }
     }
@@ -243,11 +249,12 @@ static __device__ __forceinline__ void xg_phase1(const uint32_t *w, const act_fr
 // ---- phase 2: one lane walks one accumulator over the blocks of a slab ------------------------------------------------
 template <int NCH>
 static __device__ __forceinline__ float xg_chain(const float *P, const float *D, int nblk, float acc) {
-    // nblk % 4 == 0.  Eight blocks per group, the next group's 128-bit reads requested before the current group's eight dependent
-    // fmas (two register sets, no copies); reads beyond nblk stay inside the row's 128 + 4 floats and are not used.
+    // nblk % 4 == 0.  Eight blocks per group; the 128-bit reads of a group are requested two groups (sixteen dependent fmas,
+    // about the latency of an LDS read under load) before its fmas: three register sets in rotation, no copies.  Reads beyond
+    // nblk stay inside the row's 128 + 4 floats and are not used.
     // (Taking the scale products, which the eight lanes of a row share, from one lane per quad through DPP broadcasts cut the LDS
     // traffic but measured slower: 1.25 instead of 0.8 us per 128 blocks.)
-    float4 pa[2], pb[2], da[2], db[2];
+    float4 p0[2], p1[2], p2[2], d0[2], d1[2], d2[2];
     auto ld = [&](float4 (&p)[2], float4 (&d)[2], int b) {
 #pragma unroll
         for (int u = 0; u < 2; u++) { p[u] = *(const float4 *)(P + min(b + 4 * u, XG_NBS - 4)); d[u] = *(const float4 *)(D + min(b + 4 * u, XG_NBS - 4)); }
@@ -257,15 +264,20 @@ static __device__ __forceinline__ float xg_chain(const float *P, const float *D,
         for (int u = 0; u < 2; u++)
             if (b + 4 * u < nblk) { acc = fmaf(d[u].x, p[u].x, acc); acc = fmaf(d[u].y, p[u].y, acc); acc = fmaf(d[u].z, p[u].z, acc); acc = fmaf(d[u].w, p[u].w, acc); }
     };
-    ld(pa, da, 0);
-    for (int b = 0; b < nblk; b += 16) {
-        ld(pb, db, b + 8);
+    ld(p0, d0, 0);
+    ld(p1, d1, 8);
+    for (int b = 0; b < nblk; b += 24) {
+        ld(p2, d2, b + 16);
         __builtin_amdgcn_sched_barrier(0);
-        run(pa, da, b);
+        run(p0, d0, b);
         __builtin_amdgcn_sched_barrier(0);
-        ld(pa, da, b + 16);
+        ld(p0, d0, b + 24);
         __builtin_amdgcn_sched_barrier(0);
-        run(pb, db, b + 8);
+        run(p1, d1, b + 8);
+        __builtin_amdgcn_sched_barrier(0);
+        ld(p1, d1, b + 32);
+        __builtin_amdgcn_sched_barrier(0);
+        run(p2, d2, b + 16);
         __builtin_amdgcn_sched_barrier(0);
     }
     return acc;
