@@ -35,6 +35,7 @@ def main():
                     help="real: run the prompt through the model; synthetic: fill the caches with random fp16 (quick runs)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-steps", type=int, default=8)
+    ap.add_argument("--cpu-threads", type=int, default=8, help="threads of the CPU baseline (the reference's configurations name -t 8)")
     ap.add_argument("--layers", type=int, default=32, help="debug only: fewer layers (result is then not the headline config)")
     ap.add_argument("--model", choices=["q4_0", "q8_0", "q4_k_m"], default="q4_0",
                     help="q4_0: the headline workload; q8_0 / q4_k_m (Q4_K with Q6_K attn_v, ffn_down and head): the other 7B configurations")
@@ -45,7 +46,8 @@ def main():
     ap.add_argument("--no-gemm", action="store_true", help="skip the timing of the prompt's quantized GEMM")
     ap.add_argument("--no-graph", action="store_true", help="launch the kernels of every pass one by one instead of replaying a HIP graph (for profilers)")
     ap.add_argument("--order", type=int, choices=[0, 1], default=1,
-                    help="summation order of the single-token pass: 1 = the host backend's (greedy tokens identical to the CPU reference; default), 0 = this backend's own")
+                    help="with --only-order: the one summation order to time (1 = the host backend's, 0 = this backend's own); by default both are timed and 1 is the headline")
+    ap.add_argument("--only-order", action="store_true", help="time one summation order only (profiling runs)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch a plain copy kernel over 256 MiB three times (a known-size dispatch to scale profiler byte counters by)")
     args = ap.parse_args()
@@ -62,7 +64,7 @@ def main():
     info = H.device_info()
     log("device:", info)
     steps, warmup, fill = args.steps, args.warmup, args.ctx_fill
-    n_ctx = (fill + warmup + steps + 8 + 7) // 8 * 8
+    n_ctx = (fill + warmup + steps + 8 + 63) // 64 * 64
     if args.model == "q4_0":
         cfg = M.Config.llama2_7b(n_ctx=n_ctx, wtype=H.Q4_0, t_out=H.Q4_0 if args.head == "body" else H.Q6_K)
     elif args.model == "q8_0":
@@ -71,8 +73,7 @@ def main():
         cfg = M.Config.llama2_7b(n_ctx=n_ctx, wtype=H.Q4_K, t_out=H.Q6_K, tensor_types={"attn_v": H.Q6_K, "ffn_down": H.Q6_K})
     cfg.n_layer = args.layers
     t0 = time.time()
-    # K-quant matrices: random well-formed blocks (this package has no K-quant quantizer; timing only)
-    tensors = M.synth_model(cfg, seed=1234, quantizer=M.random_k_blocks)
+    tensors = M.synth_model(cfg, seed=1234, outlier_every=1000 if args.model == "q4_k_m" else 0)   # the Q4_K_M configuration: 0.1 % of the weights x 20
     log("synthetic model: %.1f s, %.2f GB of weights streamed per token" % (time.time() - t0, cfg.weight_bytes() / 1e9))
     load_info, loaded = None, None
     if args.via_gguf:
@@ -88,7 +89,6 @@ def main():
             % (load_info["file_bytes"] / 1e9, t_write, loaded.parse_ms, loaded.upload_ms, load_info["upload_GBps"], loaded.create_ms))
     else:
         eng = M.Engine(cfg, tensors)
-    eng.set_order(args.order)
     rng = np.random.default_rng(4096)
     prompt = rng.integers(0, cfg.n_vocab, fill).astype(np.int32)
     t0 = time.time()
@@ -114,68 +114,92 @@ def main():
         H.sync()
         log("calibration: dup_kernel over %d bytes read + %d bytes written, 3 launches" % (n * 4, n * 4))
 
-    # warm-up (also captures the HIP graph), then the timed region: exactly `steps` passes
-    pos = fill
-    toks = eng.decode_greedy(first, pos, warmup, use_graph=not args.no_graph)
-    pos += warmup
-    eng.timing()
-    H.sync()
-    t0 = time.perf_counter()
-    toks = eng.decode_greedy(int(toks[-1]), pos, steps, use_graph=not args.no_graph)
-    H.sync()
-    wall = time.perf_counter() - t0
-    ev_ms, n_timed = eng.timing()
-    assert n_timed == steps
-    ms_per_step = wall * 1e3 / steps
-    tok_s = steps / wall
-    n_kv_mid = pos + steps / 2.0
-    kv_bytes = 2 * cfg.n_embd * 2 * cfg.n_layer           # K and V, fp16, per cached token
-    bytes_per_token = cfg.weight_bytes() + kv_bytes * n_kv_mid
-    frac = bytes_per_token / (wall / steps) / HBM_PEAK
-    log("decode: %.3f ms/step wall, %.3f ms/step by HIP events, %.1f tok/s, %.2f GB/token -> %.1f%% of 8 TB/s"
-        % (ms_per_step, ev_ms, tok_s, bytes_per_token / 1e9, 100 * frac))
-
-    # per-kernel times: HIP events around repeated launches of each kernel of a layer, on the stream they run on
-    per_kernel = {}
-    for name in ("qkv", "scores", "pv", "wo", "gate_up", "down", "head"):
-        per_kernel[name] = eng.kernel_time_us(name, reps=4)
+    # Two summation orders of the single-token pass are timed on the same cache, from the same position:
+    #   order 1 (headline): the host backend's order -- the path whose greedy tokens and logits equal the CPU reference's bit for bit;
+    #   order 0: this backend's own lane-parallel order (per-operator results equal to ~1e-7, greedy tokens of near-tied logits may differ).
+    # Each: warm-up passes (the first also captures the HIP graphs), then exactly `steps` timed passes.
     d, F, V = cfg.n_embd, cfg.n_ff, cfg.n_vocab
-    n_kv_end = pos + steps
+    kv_bytes = 2 * cfg.n_embd * 2 * cfg.n_layer           # K and V, fp16, per cached token
     tt = lambda n: cfg.tensor_types.get(n, cfg.wtype)
     rs = H.row_size
-    alg = {"qkv": d * (rs(tt("attn_q"), d) + rs(tt("attn_k"), d) + rs(tt("attn_v"), d)), "wo": d * rs(tt("attn_output"), d),
-           "gate_up": F * (rs(tt("ffn_gate"), d) + rs(tt("ffn_up"), d)), "down": d * rs(tt("ffn_down"), F),
-           "head": V * rs(cfg.t_out, d), "scores": n_kv_end * d * 2, "pv": n_kv_end * d * 2}
-    if eng.fuses_attention():           # qkv, scores and softmax + KQV are one launch, timed under "qkv"
-        per_kernel["attention (qkv+scores+pv)"] = per_kernel.pop("qkv")
-        alg["attention (qkv+scores+pv)"] = alg["qkv"] + alg["scores"] + alg["pv"]
-        per_kernel.pop("scores"); per_kernel.pop("pv")
-    log("per-kernel (HIP events, walking the layers):")
-    for k, us in per_kernel.items():
-        log("  %-8s %8.2f us  %7.1f GB/s  (%.1f%% of 8 TB/s)" % (k, us, alg[k] / us / 1e3, alg[k] / us / 1e3 / 80))
-    # dominant kernel = largest share of the step: launches per token x time per launch
-    count = {k: (1 if k == "head" else cfg.n_layer) for k in per_kernel}
-    dom = max(per_kernel, key=lambda k: per_kernel[k] * count[k])
-    names = {"attention (qkv+scores+pv)": "attn_layer_kernel<Q4_0> (RMSNorm, Q8_0, wq|wk|wv, RoPE, cache write, q.K, softmax, P.V^T)",
-             "gate_up": "wave_gemv_kernel<gate|up + SiLU>", "down": "wave_gemv_kernel<down + residual>", "wo": "wave_gemv_kernel<wo + residual>",
-             "head": "wave_gemv_kernel<output head>", "qkv": "wave_gemv_kernel<qkv>", "scores": "attn_scores_kernel", "pv": "attn_pv_kernel"}
-    # HBM bytes per launch from profiler counters (FETCH_SIZE + WRITE_SIZE, each scaled by what the same counter reads for a
-    # copy kernel of known size; profiles/decode_7b_q4_0_ctx4096_hbm_traffic.md): measured for this model shape only.  The
-    # attention launch was counted at n_kv = 4103 (101.7 MB for 95.5 MB algorithmic); its traffic is scaled to this run's n_kv.
-    measured = {"gate_up": 51.18e6, "down": 25.83e6, "wo": 9.65e6, "head": 108.26e6,
-                "attention (qkv+scores+pv)": 101.7e6 * alg.get("attention (qkv+scores+pv)", 0) / (28311552 + 2 * 4103 * 8192)}
-    shape_ok = (cfg.n_embd, cfg.n_ff, cfg.wtype, args.model, cfg.t_out) == (4096, 11008, H.Q4_0, "q4_0", H.Q6_K) and cfg.n_layer == 32
-    def roof(k):
-        ach = alg[k] / (per_kernel[k] * 1e-6) / 1e9
-        return {"kernel": names.get(k, k), "bound": "hbm", "achieved": round(ach, 1), "peak": 8000.0, "unit": "GB/s", "frac": round(ach / 8000.0, 4),
-                "traffic": round(measured[k]) if shape_ok and k in measured else None, "bytes_per_launch": int(alg[k]),
-                "us_per_launch": round(per_kernel[k], 3), "launches_per_token": count[k], "share_of_step": round(per_kernel[k] * count[k] / (ev_ms * 1e3), 3)}
-    roofline = roof(dom)
-    roofline_others = {k: roof(k) for k in per_kernel if k != dom}
+    tn = {H.Q4_0: "Q4_0", H.Q8_0: "Q8_0", H.Q4_K: "Q4_K", H.Q6_K: "Q6_K"}
+    traffic_db = {}
+    tpath = os.path.join(ROOT, "profiles", "decode_hbm_traffic.json")      # FETCH_SIZE / WRITE_SIZE per dispatch, scaled by a copy kernel (see the file)
+    if os.path.exists(tpath):
+        with open(tpath) as f:
+            traffic_db = json.load(f)
+
+    def run_order(order):
+        eng.set_order(order)
+        pos = fill
+        toks = eng.decode_greedy(first, pos, warmup, use_graph=not args.no_graph)
+        pos += warmup
+        eng.timing()
+        H.sync()
+        t0 = time.perf_counter()
+        toks = eng.decode_greedy(int(toks[-1]), pos, steps, use_graph=not args.no_graph)
+        H.sync()
+        wall = time.perf_counter() - t0
+        ev_ms, n_timed = eng.timing()
+        assert n_timed == steps
+        n_kv_mid = pos + steps / 2.0
+        bytes_per_token = cfg.weight_bytes() + kv_bytes * n_kv_mid
+        frac = bytes_per_token / (wall / steps) / HBM_PEAK
+        log("order %d decode: %.3f ms/step wall, %.3f ms/step by HIP events, %.1f tok/s, %.2f GB/token -> %.1f%% of 8 TB/s"
+            % (order, wall * 1e3 / steps, ev_ms, steps / wall, bytes_per_token / 1e9, 100 * frac))
+        # per-kernel times: HIP events around repeated launches of each kernel of a layer, on the stream they run on, at the last position
+        per_kernel = {}
+        for name in ("qkv", "scores", "pv", "wo", "gate_up", "down", "head"):
+            per_kernel[name] = eng.kernel_time_us(name, reps=4)
+        n_kv_end = pos + steps
+        alg = {"qkv": d * (rs(tt("attn_q"), d) + rs(tt("attn_k"), d) + rs(tt("attn_v"), d)), "wo": d * rs(tt("attn_output"), d),
+               "gate_up": F * (rs(tt("ffn_gate"), d) + rs(tt("ffn_up"), d)), "down": d * rs(tt("ffn_down"), F),
+               "head": V * rs(cfg.t_out, d), "scores": n_kv_end * d * 2, "pv": n_kv_end * d * 2}
+        if eng.fuses_attention():           # qkv, scores and softmax + KQV are one launch, timed under "qkv"
+            per_kernel["attention"] = per_kernel.pop("qkv")
+            alg["attention"] = alg["qkv"] + alg["scores"] + alg["pv"]
+            per_kernel.pop("scores"); per_kernel.pop("pv")
+        log("  per-kernel (HIP events, walking the layers):")
+        for k, us in per_kernel.items():
+            log("    %-10s %8.2f us  %7.1f GB/s  (%.1f%% of 8 TB/s)" % (k, us, alg[k] / us / 1e3, alg[k] / us / 1e3 / 80))
+        count = {k: (1 if k == "head" else cfg.n_layer) for k in per_kernel}
+        if order == 1:
+            names = {"qkv": "xgemv_kernel<%s, qkv> (RMSNorm in std::reduce order, Q8_0, wq|wk|wv as 8-accumulator walks, RoPE, cache write)" % tn[tt("attn_q")],
+                     "scores": "xattn_scores_kernel (Dot<FP16,FP16> order, one thread per key)", "pv": "xattn_pv_kernel (softmax with std::reduce sum, P.V^T in Dot<FP16,FP16> order)",
+                     "wo": "xgemv_kernel<%s, wo + residual>" % tn[tt("attn_output")], "gate_up": "xgemv_kernel<%s, gate|up + SiLU table>" % tn[tt("ffn_gate")],
+                     "down": "xgemv_kernel<%s, down + residual>" % tn[tt("ffn_down")], "head": "xgemv_kernel<%s, output head>" % tn[cfg.t_out]}
+        else:
+            names = {"attention": "attn_layer_kernel<%s> (RMSNorm, Q8_0, wq|wk|wv, RoPE, cache write, q.K, softmax, P.V^T)" % tn[tt("attn_q")],
+                     "gate_up": "wave_gemv_kernel<gate|up + SiLU>", "down": "wave_gemv_kernel<down + residual>", "wo": "wave_gemv_kernel<wo + residual>",
+                     "head": "wave_gemv_kernel<output head>", "qkv": "wave_gemv_kernel<qkv>", "scores": "attn_scores_kernel", "pv": "attn_pv_kernel"}
+        model_key = "%s/head_%s/order%d" % (args.model, tn[cfg.t_out], order)
+        measured = traffic_db.get("kernels", {}).get(model_key, {}) if (cfg.n_embd, cfg.n_ff, cfg.n_layer) == (4096, 11008, 32) else {}
+
+        def roof(k):
+            ach = alg[k] / (per_kernel[k] * 1e-6) / 1e9
+            tr = measured.get(k)
+            if tr is not None and k in ("attention", "scores", "pv"):          # counted at one n_kv: scaled to this run's by the algorithmic bytes
+                tr = tr["bytes"] * alg[k] / tr["algorithmic_bytes"]
+            elif tr is not None:
+                tr = tr["bytes"]
+            return {"kernel": names.get(k, k), "bound": "hbm", "achieved": round(ach, 1), "peak": 8000.0, "unit": "GB/s", "frac": round(ach / 8000.0, 4),
+                    "traffic": round(tr) if tr is not None else None, "bytes_per_launch": int(alg[k]),
+                    "us_per_launch": round(per_kernel[k], 3), "launches_per_token": count[k], "share_of_step": round(per_kernel[k] * count[k] / (ev_ms * 1e3), 3)}
+        dom = max(per_kernel, key=lambda k: per_kernel[k] * count[k])
+        return {"order": order, "tok_s": steps / wall, "ms_per_step": wall * 1e3 / steps, "ev_ms": ev_ms, "frac": frac, "bytes_per_token": bytes_per_token, "pos": pos,
+                "per_kernel": per_kernel, "roofline": roof(dom), "others": {k: roof(k) for k in per_kernel if k != dom}}
+
+    orders = [args.order] if args.only_order else [1, 0]
+    runs = {o: run_order(o) for o in orders}
+    head_run = runs[orders[0]]
+    pos, ev_ms = head_run["pos"], head_run["ev_ms"]
+    tok_s, ms_per_step, frac, bytes_per_token = head_run["tok_s"], head_run["ms_per_step"], head_run["frac"], head_run["bytes_per_token"]
+    per_kernel, roofline, roofline_others = head_run["per_kernel"], head_run["roofline"], head_run["others"]
+    eng.set_order(orders[0])
 
     # The prompt's dominant kernels against the int8 matrix-core peak: the seven quantized GEMMs of one layer
     # (wq, wk, wv, wo: 4096 x 4096; gate, up: 11008 x 4096; down: 4096 x 11008) over the 2048 activation rows of a
-    # prompt chunk, HIP events around 4 back-to-back sets.  K-quant bodies have no quantizer in this package: random blocks.
+    # prompt chunk, HIP events around 4 back-to-back sets.  
     gemm_roofline = None
     if not args.no_gemm:
         wt_g, Tg = cfg.wtype, 2048
@@ -183,7 +207,7 @@ def main():
         L = H.load()
 
         def wdev(Mg, Kg):
-            wb = M.synth_tensor(wt_g, 7, "bench.gemm.%d.%d" % (Mg, Kg), Mg * Kg) if wt_g in (H.Q4_0, H.Q8_0) else M.random_k_blocks(np.empty(Mg * Kg, np.float32), wt_g)
+            wb = M.synth_tensor(wt_g, 7, "bench.gemm.%d.%d" % (Mg, Kg), Mg * Kg)
             return H.DeviceBuffer.from_numpy(wb)
 
         def xdev(Kg):
@@ -223,7 +247,7 @@ def main():
     if not args.no_cpu:
         from tests import oracle_lib as O            # the checker, timed as the CPU baseline
         from tests.model_util import OracleModel
-        ncpu = min(16, os.cpu_count() or 1)
+        ncpu = min(args.cpu_threads, os.cpu_count() or 1)            # the reference's configurations run with -t 8
         ora = OracleModel(cfg, tensors, nthread=ncpu)
         for il in range(cfg.n_layer):                # same cache contents as the GPU run
             ora.k_cache[il][:] = eng.read_buffer("k_cache", il, np.uint16)
@@ -235,12 +259,17 @@ def main():
             lg = ora.forward(tok, fill + i)
             tok = np.array([int(np.argmax(lg[0]))], np.int32)
         cpu_wall = time.perf_counter() - t0
-        cpu = {"value": round(args.cpu_steps / cpu_wall, 3), "unit": "tok/s", "cores": ncpu, "kind": "port",
-               "sample": "%d single-token passes of the same model at n_kv = %d.. (AVX2 port of Spy's host backend, OpenMP)" % (args.cpu_steps, fill + 1)}
-        log("cpu baseline: %.3f tok/s on %d threads" % (cpu["value"], ncpu))
+        cpu = {"value": round(args.cpu_steps / cpu_wall, 3), "unit": "tok/s", "cores": ncpu, "kind": "port", "host_cpus": os.cpu_count(),
+               "sample": "%d single-token passes of the same model at n_kv = %d.. (AVX2 port of Spy's host backend, OpenMP, %d threads as the reference's -t 8)"
+                         % (args.cpu_steps, fill + 1, ncpu)}
+        log("cpu baseline: %.3f tok/s on %d threads (%d host cpus)" % (cpu["value"], ncpu, os.cpu_count() or 0))
 
-    weights_desc = {"q4_0": "Q4_0 weights, output head Q6_K (random well-formed blocks)" if cfg.t_out == H.Q6_K else "Q4_0 weights incl. head", "q8_0": "Q8_0 weights incl. head",
-                    "q4_k_m": "Q4_K weights with Q6_K attn_v / ffn_down / head (random blocks)"}[args.model]
+    head_desc = {H.Q6_K: "output head Q6_K", H.Q4_0: "output head Q4_0", H.Q8_0: "output head Q8_0", H.Q4_K: "output head Q4_K"}[cfg.t_out]
+    weights_desc = {"q4_0": "Q4_0 weights, %s" % head_desc, "q8_0": "Q8_0 weights incl. head",
+                    "q4_k_m": "Q4_K weights with Q6_K attn_v / ffn_down / head, 0.1 %% of the weights x 20"}[args.model] + \
+                   " (seeded ~N(0, 0.02), quantized by the package's block quantizers)"
+    mode_desc = {1: "host-backend summation order: logits and greedy tokens equal to the CPU reference's bit for bit",
+                 0: "this backend's own summation order (per-operator 1e-7; not token-exact)"}
     out = {
         "metric": "decode tok/s + %% HBM roofline, LLaMA-2-7B %s ctx 4096, 1xMI355X" % {"q4_0": "Q4_0", "q8_0": "Q8_0", "q4_k_m": "Q4_K_M"}[args.model],
         "value": round(tok_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
@@ -248,12 +277,19 @@ def main():
         "dtype": "int8 dot (%s x Q8_0), fp32 accumulate, fp16 KV" % {"q4_0": "Q4_0", "q8_0": "Q8_0", "q4_k_m": "Q4_K / Q6_K"}[args.model], "data": "synthetic",
         "config": {"workload": "LLaMA-2-7B shape (32 layers, d 4096, 32 heads x 128, FFN 11008, vocab 32000), %s, " % weights_desc +
                                "f16 KV cache prefilled to %d tokens (%s), greedy single-sequence decode" % (fill, args.prefill),
+                   "mode": mode_desc[orders[0]], "summation_order": orders[0],
                    "n_layer": cfg.n_layer, "n_kv_first": pos + 1, "n_kv_last": pos + steps, "bytes_per_token": int(bytes_per_token)},
         "hbm_roofline_frac": round(frac, 4), "ms_per_step_hip_events": round(ev_ms, 4),
-        "prefill": {"tokens": fill, "seconds": round(prefill_s, 3), "tok_s": round(fill / prefill_s, 1)} if args.prefill == "real" else None,
+        "prefill": {"tokens": fill, "seconds": round(prefill_s, 3), "tok_s": round(fill / prefill_s, 1),
+                    "note": "matrix-core prompt pass in the backend's own order"} if args.prefill == "real" else None,
         "kernel_us": {k: round(v, 2) for k, v in per_kernel.items()},
         "roofline": roofline, "roofline_other_kernels": roofline_others, "prompt_gemm_roofline": gemm_roofline, "cpu_baseline": cpu,
     }
+    if len(orders) > 1:
+        o = runs[orders[1]]
+        out["other_order"] = {"summation_order": orders[1], "mode": mode_desc[orders[1]], "value": round(o["tok_s"], 2), "unit": "tok/s",
+                              "ms_per_step": round(o["ms_per_step"], 4), "hbm_roofline_frac": round(o["frac"], 4),
+                              "kernel_us": {k: round(v, 2) for k, v in o["per_kernel"].items()}, "roofline": o["roofline"]}
     if load_info:
         out["gguf_load"] = load_info
     print(json.dumps(out), flush=True)

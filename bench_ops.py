@@ -110,9 +110,7 @@ def main():
 
     def weights(wt, M_, K):
         n = M_ * K
-        if wt in (H.Q4_0, H.Q8_0):
-            return M.synth_tensor(wt, 7, "sweep.%d.%d.%d" % (wt, M_, K), n)
-        return M.random_k_blocks(np.empty(n, np.float32), wt)
+        return M.synth_tensor(wt, 7, "sweep.%d.%d.%d" % (wt, M_, K), n)
 
     def activations(T, K):
         x = np.random.default_rng(T * 131 + K).standard_normal((T, K)).astype(np.float32)

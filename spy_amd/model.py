@@ -81,40 +81,29 @@ def _name_seed(seed, name):
 
 
 def synth_tensor(ttype, seed, name, n, std=0.02, outlier_every=0, outlier_mul=20.0, quantizer=None):
-    """n elements of the named stream, stored as `ttype` blocks. Q4_K / Q6_K need `quantizer`
-    (callable(float32 array, type) -> uint8 bytes) because the block quantizers of this package
-    cover the types the reference's host backend can run (F32, Q4_0, Q8_0)."""
+    """n elements of the named stream (~N(0, std), every outlier_every-th element x outlier_mul), stored as `ttype`
+    blocks: F32, Q4_0, Q8_0 by the block rules the reference's host backend decodes, Q4_K / Q6_K by this package's own
+    one-pass rule (the reference holds their layouts only).  `quantizer` (callable(float32 array, type) -> uint8 bytes)
+    replaces the built-in rule where given."""
     S = synth_lib()
     s = _name_seed(seed, name)
-    if ttype in (H.F32, H.Q4_0, H.Q8_0):
+    if quantizer is None or ttype in (H.F32, H.Q4_0, H.Q8_0):
         out = np.empty(H.row_size(ttype, n), dtype=np.uint8)
         got = S.spy_synth_tensor(ttype, s, n, std, outlier_every, outlier_mul, out.ctypes.data)
-        assert got == out.nbytes
+        assert got == out.nbytes, (ttype, n)
         return out
-    if quantizer is None:
-        raise ValueError("no quantizer for type %d" % ttype)
     x = np.empty(n, dtype=np.float32)
     S.spy_synth_tensor(H.F32, s, n, std, outlier_every, outlier_mul, x.ctypes.data)
     return quantizer(x, ttype)
 
 
-def random_k_blocks(x, ttype):
-    """Q4_K / Q6_K blocks with random quants and small random scales for as many elements as x has:
-    well-formed weights for timing runs (the values do not approximate x)."""
-    n = len(x)
-    rng = np.random.default_rng(n * 31 + ttype)
-    nsb = n // 256
-    if ttype == H.Q4_K:
-        b = rng.integers(0, 256, (nsb, 144), dtype=np.uint8)
-        b[:, 0:2] = (rng.uniform(0.5, 1.5, nsb) * 2e-4).astype(np.float16).view(np.uint8).reshape(nsb, 2)
-        b[:, 2:4] = (rng.uniform(0.5, 1.5, nsb) * 1e-4).astype(np.float16).view(np.uint8).reshape(nsb, 2)
-    elif ttype == H.Q6_K:
-        b = rng.integers(0, 256, (nsb, 210), dtype=np.uint8)
-        b[:, 192:208] = rng.integers(1, 64, (nsb, 16), dtype=np.uint8)
-        b[:, 208:210] = (rng.uniform(0.5, 1.5, nsb) * 2e-5).astype(np.float16).view(np.uint8).reshape(nsb, 2)
-    else:
-        raise ValueError("not a K-quant type: %d" % ttype)
-    return b.reshape(-1)
+def quantize(x, ttype):
+    """float32 array -> block bytes of `ttype` (F32, Q4_0, Q8_0, Q4_K, Q6_K) by the package's own quantizers"""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty(H.row_size(ttype, x.size), dtype=np.uint8)
+    got = synth_lib().spy_synth_quantize(ttype, x.ctypes.data, x.size, out.ctypes.data)
+    assert got == out.nbytes, (ttype, x.size)
+    return out
 
 
 def synth_model(cfg, seed=1234, std=0.02, outlier_every=0, quantizer=None, norm_jitter=0.1):

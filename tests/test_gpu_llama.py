@@ -296,7 +296,7 @@ def test_llama2_7b_prompt_4096_properties(name, kw, monkeypatch):
     (c) The token loop on top: decode_greedy and one-token forward passes emit the same tokens."""
     from spy_amd import model as M
     cfg = M.Config.llama2_7b(n_ctx=4096 + 32, **kw)
-    tensors = M.synth_model(cfg, seed=1234, quantizer=M.random_k_blocks)      # K-quant matrices: random well-formed blocks
+    tensors = M.synth_model(cfg, seed=1234)
     prompt = np.random.default_rng(4096).integers(0, cfg.n_vocab, 4096).astype(np.int32)
     eng = M.Engine(cfg, tensors)
     last_2048 = eng.forward_last(prompt, 0)

@@ -212,3 +212,23 @@ def test_k_quant_roundtrip_bounds(oracle, ttype, tol):
     # zeros stay zeros
     z = O.dequantize(oracle, O.quantize(oracle, np.zeros(256, np.float32), ttype), ttype, 256)
     assert not z.any()
+
+
+@pytest.mark.parametrize("ttype", [O.Q4_0, O.Q8_0, O.Q4_K, O.Q6_K])
+def test_package_quantizers_write_the_oracles_bytes(oracle, ttype):
+    """The block quantizers of the package (spy_amd/csrc/host/synth.c: synthetic models for the bench and the full-size GPU
+    tests) against the oracle's, written independently from the same rules: identical bytes on normal weights, weights
+    with 0.1 % outliers x 20, an all-zero super-block, a constant block and a block with a single non-zero element."""
+    from spy_amd import model as M
+    rng = np.random.default_rng(ttype)
+    x = (rng.standard_normal(256 * 64) * 0.02).astype(np.float32)
+    x[::1000] *= 20.0
+    x[256:512] = 0.0
+    x[512:768] = 0.013
+    x[768:1024] = 0.0
+    x[800] = -0.4
+    assert np.array_equal(M.quantize(x, ttype), O.quantize(oracle, x, ttype))
+    # the named stream, quantized on the fly, equals quantizing its float form
+    n = 256 * 8
+    xs = np.frombuffer(M.synth_tensor(O.F32, 3, "t", n, 0.02, 100, 20.0).tobytes(), np.float32)
+    assert np.array_equal(M.synth_tensor(ttype, 3, "t", n, 0.02, 100, 20.0), O.quantize(oracle, xs, ttype))
