@@ -5,9 +5,57 @@
 
 #include <cstring>
 
+#include <rocprofiler-sdk-roctx/roctx.h>
+
 #include "../../include/spy_hip.h"
 
 namespace spy::hip {
+
+// Name of the marker range around one operator: "hip-<Op>", the counterpart of the "cpu-<Op>" ranges the host
+// backend opens around every operator (backend/host/include/operator_impl.h:57-63).
+static const char *range_name(OperatorType t) {
+    switch (t) {
+    case OperatorType::Input: return "hip-Input";
+    case OperatorType::Nop: return "hip-Nop";
+    case OperatorType::Dup: return "hip-Dup";
+    case OperatorType::Copy: return "hip-Copy";
+    case OperatorType::View: return "hip-View";
+    case OperatorType::Reshape: return "hip-Reshape";
+    case OperatorType::MaskedCopy: return "hip-MaskedCopy";
+    case OperatorType::MaskedSelect: return "hip-MaskedSelect";
+    case OperatorType::GetRow: return "hip-GetRow";
+    case OperatorType::Transpose: return "hip-Transpose";
+    case OperatorType::Permute: return "hip-Permute";
+    case OperatorType::Contiguous: return "hip-Contiguous";
+    case OperatorType::Relu: return "hip-Relu";
+    case OperatorType::Silu: return "hip-Silu";
+    case OperatorType::Gelu: return "hip-Gelu";
+    case OperatorType::Max: return "hip-Max";
+    case OperatorType::Min: return "hip-Min";
+    case OperatorType::Softmax: return "hip-Softmax";
+    case OperatorType::Add: return "hip-Add";
+    case OperatorType::Sub: return "hip-Sub";
+    case OperatorType::Mul: return "hip-Mul";
+    case OperatorType::Div: return "hip-Div";
+    case OperatorType::Mod: return "hip-Mod";
+    case OperatorType::MatMul: return "hip-MatMul";
+    case OperatorType::Sum: return "hip-Sum";
+    case OperatorType::Norm: return "hip-Norm";
+    case OperatorType::NormRMS: return "hip-NormRMS";
+    case OperatorType::Rope: return "hip-Rope";
+    case OperatorType::Quantize: return "hip-Quantize";
+    }
+    return "hip-Unknown";
+}
+
+namespace {
+struct MarkerRange {                    // closed on every return path of run()
+    explicit MarkerRange(const char *name) { roctxRangePushA(name); }
+    ~MarkerRange() { roctxRangePop(); }
+    MarkerRange(const MarkerRange &) = delete;
+    MarkerRange &operator=(const MarkerRange &) = delete;
+};
+}  // namespace
 
 static spy_hip_tensor flat(const Tensor &t, const void *data) {
     spy_hip_tensor o;
@@ -115,6 +163,7 @@ const void *HIPBackend::device_view(DataNode *node, bool is_output) {
 
 OperatorStatus HIPBackend::run(OperatorNode *op) {
     const OperatorType type = op->op_type;
+    const MarkerRange range(range_name(type));
     // zero-copy operators only move the data pointer (view.cpp:219-276): no launch
     switch (type) {
     case OperatorType::Nop: return OperatorStatus::Success;
