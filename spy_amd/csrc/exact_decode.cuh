@@ -319,7 +319,10 @@ __global__ __launch_bounds__(XG_THREADS) void xgemv_kernel(xg_args a) {
         else { const int u = (gw + (r / RPS) * NW) * RPS + (r % RPS); valid = u < a.M; return valid ? u : u % a.M; }
     };
     auto row_ptr = [&](int r) -> const uint8_t * {
-        bool v; const int i = row_of(r, v);
+        bool v; int i = row_of(r, v);
+#ifdef XDBG_SMALLROWS
+        i &= 255;                                   // measurement build: every workgroup re-reads the same cached rows
+#endif
         if constexpr (EPI == EPI_QKV) {
             if (r == 2) return a.W2 + (size_t)i * spy_row_size(WTV, K);
             return (2 * (gw % a.d) < a.d ? a.W0 : a.W1) + (size_t)i * RB;
@@ -449,16 +452,19 @@ __global__ __launch_bounds__(XG_THREADS) void xgemv_kernel(xg_args a) {
 // ---- attention scores in the order of Dot<FP16,FP16> -------------------------------------------------------------------
 // The cached tokens are dealt out evenly over the workgroups (one per compute unit): workgroup b takes tokens
 // b * tpw .. (b + 1) * tpw - 1, tpw = ceil(n_kv / workgroups), all heads, in rounds of XS_TOK tokens.  The keys of a round
-// (8 KiB per token, [head][128] fp16) are read coalesced, eight 16-byte pieces per thread all requested at once, and laid
-// into LDS; then ONE thread per (token, head) key walks the dot exactly as vec_dot.h:124-145 does for n = 128:
+// (8 KiB per token, [head][128] fp16) are read coalesced, XS_NLD 16-byte pieces per thread all requested at once and a
+// round ahead of their use, and laid into LDS; then ONE thread per (token, head) key walks the dot exactly as vec_dot.h:124-145 does for n = 128:
 // accumulators sum[j][l] over the chunks i = 0, 32, 64 (i + 32 < n), the reduction tree of FP16::block_reduce, then the
 // scalar tail over elements 96..127 (a product of two fp16 values is exact in fp32, so `tail += a * b` is the fma it is
 // written as here), result = tail + simd.  Stored: t = dot * scale (mask 0, then * scale: non-linear.cpp:141-150).
 #define XS_THREADS 1024
-#define XS_TOK 16
+#define XS_TOK 18
+#define XS_NLD 9                                        // pieces per thread requested together: 1024 x 9 x 16 bytes = 18 tokens of 32 heads
 static inline size_t xattn_scores_lds(int n_head) { return (size_t)(XS_TOK + 1) * n_head * 16 * 16; }
+// kc is not a restrict pointer on purpose: the loads of the next round must stay where they are written, ahead of the
+// barrier and the dots of the current round, so that they are in flight meanwhile.
 template <int DUMMY>
-__global__ __launch_bounds__(XS_THREADS) void xattn_scores_kernel(const dev_state *st, int pos_imm, const uint16_t *__restrict__ q16, const uint16_t *__restrict__ kc,
+__global__ __launch_bounds__(XS_THREADS) void xattn_scores_kernel(const dev_state *st, int pos_imm, const uint16_t *__restrict__ q16, const uint16_t *kc,
                                                                   float *__restrict__ scores, int n_head, int n_ctx, float scale) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int n_kv = (st ? st->pos : pos_imm) + 1;
@@ -469,28 +475,32 @@ __global__ __launch_bounds__(XS_THREADS) void xattn_scores_kernel(const dev_stat
     uint4 *s_k = (uint4 *)smem;                         // [XS_TOK][n_head][16 chunks of 16 bytes], chunk index rotated per key against bank conflicts
     uint4 *s_qh = s_k + XS_TOK * n_head * 16;           // [n_head][16]
     const int per_tok = n_head * 16;                    // 16-byte pieces per token
+    // the pieces in flight: named registers (an indexed array that lives across the rounds ends up in scratch memory)
+    uint4 k0, k1, k2, k3, k4, k5, k6, k7, k8;
+    static_assert(XS_NLD == 9, "nine named registers");
+#define XS_EACH(X) X(0, k0) X(1, k1) X(2, k2) X(3, k3) X(4, k4) X(5, k5) X(6, k6) X(7, k7) X(8, k8)
+    auto request = [&](int t0, int npiece, int c0) {
+#define XS_REQ(u, r) { const int c = min(c0 + u * XS_THREADS + tid, npiece - 1); const int tt = c / per_tok, rem = c - tt * per_tok; \
+                       r = *(const uint4 *)(kc + (size_t)(t0 + tt) * d + rem * 8); }
+        XS_EACH(XS_REQ)
+#undef XS_REQ
+    };
+    auto lay = [&](int npiece, int c0) {
+#define XS_LAY(u, r) { const int c = c0 + u * XS_THREADS + tid; \
+                       if (c < npiece) { const int tt = c / per_tok, rem = c - tt * per_tok, hh = rem >> 4, ch = rem & 15; \
+                                         s_k[(tt * n_head + hh) * 16 + ((ch + tt + 8 * (hh & 1)) & 15)] = r; } }
+        XS_EACH(XS_LAY)
+#undef XS_LAY
+    };
+#undef XS_EACH
+    request(t_begin, min(XS_TOK, t_end - t_begin) * per_tok, 0);
     for (int c = tid; c < per_tok; c += XS_THREADS) s_qh[c] = *(const uint4 *)(q16 + c * 8);
     for (int t0 = t_begin; t0 < t_end; t0 += XS_TOK) {
         const int nt = min(XS_TOK, t_end - t0), npiece = nt * per_tok;
         if (t0 != t_begin) __syncthreads();             // the previous round's keys have been read
-        constexpr int NLD = 8;                          // pieces per thread requested together: 1024 x 8 x 16 bytes = 16 tokens of 32 heads
-        for (int c0 = 0; c0 < npiece; c0 += NLD * XS_THREADS) {
-            uint4 kreg[NLD];
-#pragma unroll
-            for (int u = 0; u < NLD; u++) {
-                const int c = min(c0 + u * XS_THREADS + tid, npiece - 1);
-                const int tt = c / per_tok, rem = c - tt * per_tok;
-                kreg[u] = *(const uint4 *)(kc + (size_t)(t0 + tt) * d + rem * 8);
-            }
-#pragma unroll
-            for (int u = 0; u < NLD; u++) {
-                const int c = c0 + u * XS_THREADS + tid;
-                if (c < npiece) {
-                    const int tt = c / per_tok, rem = c - tt * per_tok, hh = rem >> 4, ch = rem & 15;
-                    s_k[(tt * n_head + hh) * 16 + ((ch + tt + 8 * (hh & 1)) & 15)] = kreg[u];
-                }
-            }
-        }
+        lay(npiece, 0);                                 // the first batch of the round was requested a round ahead
+        for (int c0 = XS_NLD * XS_THREADS; c0 < npiece; c0 += XS_NLD * XS_THREADS) { request(t0, npiece, c0); lay(npiece, c0); }
+        if (t0 + XS_TOK < t_end) request(t0 + XS_TOK, min(XS_TOK, t_end - t0 - XS_TOK) * per_tok, 0);
         __syncthreads();
         for (int key = tid; key < nt * n_head; key += XS_THREADS) {
             const int hh = key / nt, tt = key - hh * nt;
@@ -502,7 +512,8 @@ __global__ __launch_bounds__(XS_THREADS) void xattn_scores_kernel(const dev_stat
 #pragma unroll
                 for (int l = 0; l < 8; l++) sum[j][l] = 0.0f;
 #pragma unroll
-            for (int i = 0; i < 3; i++)                  // chunks of 32 elements = 4 x 16 bytes
+            for (int i = 0; i < 3; i++) {                // chunks of 32 elements = 4 x 16 bytes
+                __builtin_amdgcn_sched_barrier(0);      // one chunk's LDS reads at a time: the next round's keys occupy registers meanwhile
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
                     const uint4 kv = kp[(4 * i + j + rot) & 15], qv = qp[4 * i + j];
@@ -513,6 +524,8 @@ __global__ __launch_bounds__(XS_THREADS) void xattn_scores_kernel(const dev_stat
                         sum[j][2 * e + 1] = fmaf(h2f((uint16_t)(kw[e] >> 16)), h2f((uint16_t)(qw[e] >> 16)), sum[j][2 * e + 1]);
                     }
                 }
+            }
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int l = 0; l < 8; l++) { sum[0][l] += sum[2][l]; sum[1][l] += sum[3][l]; }
 #pragma unroll
@@ -550,7 +563,7 @@ __global__ __launch_bounds__(XS_THREADS) void xattn_scores_kernel(const dev_stat
 #define XP_NS 5                            // scores per thread: n_ctx <= 5120
 static inline int xattn_pv_vstride(int n_ctx) { return ((n_ctx + 63) / 64) * 64 + 32; }        // halfs between rows in LDS: = 64 bytes mod 128, the two rows of a wave on different banks
 static inline size_t xattn_pv_lds(int n_ctx) {
-    const size_t p_bytes = (size_t)((n_ctx + 32 + 7) & ~7) * 2, v_bytes = (size_t)16 * xattn_pv_vstride(n_ctx) * 2;
+    const size_t p_bytes = (size_t)((n_ctx + 32 + 7) & ~7) * 2, v_bytes = (size_t)16 * xattn_pv_vstride(n_ctx) * 2 + 1024;      // + the walk's read-ahead
     const size_t soft = (size_t)n_ctx * 4 + (size_t)((n_ctx / 4 + 3) & ~3) * 4;                  // t / e and the group sums live where the rows go later
     return p_bytes + (v_bytes > soft ? v_bytes : soft);
 }
@@ -643,21 +656,38 @@ __global__ __launch_bounds__(XP_THREADS) void xattn_pv_kernel(const dev_state *s
     __syncthreads();
     XSTAMP(dbg, 5);
     // ---- P . V^T ----
+    // One lane per accumulator: each step is two 16-bit LDS reads and one fma that takes the fp16 operands as they are; a
+    // wave issues an instruction every 2.6 ns or so whatever the other waves do, so the walk is spread over eight waves.
     if (wave < 8) {
         const int nfull = (n_kv - 1) / 32;                            // chunks with 32 i + 32 < n_kv
         const int r16 = wave * 2 + (lane >> 5), cl = lane & 31;       // row of the 16 and accumulator 8 j + l
-        const uint16_t *vr = s_v + (size_t)r16 * VS + cl, *pr = s_p + cl;
+        const _Float16 *vr = (const _Float16 *)s_v + (size_t)r16 * VS + cl, *pr = (const _Float16 *)s_p + cl;
         float acc = 0.0f;
+        _Float16 va[8], pa[8], vb[8], pb[8];
+        auto ld = [&](_Float16 (&v)[8], _Float16 (&q)[8], int i) {   // up to 16 chunks beyond nfull are read and not used: the next row, or the slack after the last
+#pragma unroll
+            for (int u = 0; u < 8; u++) { v[u] = vr[32 * (i + u)]; q[u] = pr[32 * (i + u)]; }
+        };
+        auto run = [&](const _Float16 (&v)[8], const _Float16 (&q)[8]) {
+#pragma unroll
+            for (int u = 0; u < 8; u++) acc = fmaf((float)v[u], (float)q[u], acc);
+        };
         int i = 0;
-        for (; i + 8 <= nfull; i += 8) {
-            const uint16_t v0 = vr[32 * i], v1 = vr[32 * i + 32], v2 = vr[32 * i + 64], v3 = vr[32 * i + 96], v4 = vr[32 * i + 128], v5 = vr[32 * i + 160],
-                           v6 = vr[32 * i + 192], v7 = vr[32 * i + 224];
-            const uint16_t p0 = pr[32 * i], p1 = pr[32 * i + 32], p2 = pr[32 * i + 64], p3 = pr[32 * i + 96], p4 = pr[32 * i + 128], p5 = pr[32 * i + 160],
-                           p6 = pr[32 * i + 192], p7 = pr[32 * i + 224];
-            acc = fmaf(h2f(v0), h2f(p0), acc); acc = fmaf(h2f(v1), h2f(p1), acc); acc = fmaf(h2f(v2), h2f(p2), acc); acc = fmaf(h2f(v3), h2f(p3), acc);
-            acc = fmaf(h2f(v4), h2f(p4), acc); acc = fmaf(h2f(v5), h2f(p5), acc); acc = fmaf(h2f(v6), h2f(p6), acc); acc = fmaf(h2f(v7), h2f(p7), acc);
+        const int n16 = nfull - nfull % 16;
+        if (n16) {
+            ld(va, pa, 0);
+            for (; i < n16; i += 16) {
+                ld(vb, pb, i + 8);
+                __builtin_amdgcn_sched_barrier(0);
+                run(va, pa);
+                __builtin_amdgcn_sched_barrier(0);
+                ld(va, pa, i + 16);
+                __builtin_amdgcn_sched_barrier(0);
+                run(vb, pb);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
-        for (; i < nfull; i++) acc = fmaf(h2f(vr[32 * i]), h2f(pr[32 * i]), acc);
+        for (; i < nfull; i++) acc = fmaf((float)vr[32 * i], (float)pr[32 * i], acc);
         XSTAMP(dbg, 6);
         acc += __shfl_xor(acc, 16, SPY_WAVE);         // sum[0] += sum[2], sum[1] += sum[3]
         acc += __shfl_xor(acc, 8, SPY_WAVE);          // sum[0] += sum[1]
@@ -666,7 +696,7 @@ __global__ __launch_bounds__(XP_THREADS) void xattn_pv_kernel(const dev_state *s
         acc += __shfl_xor(acc, 2, SPY_WAVE);          // (t_0 + t_1) + (t_2 + t_3)
         if (cl == 0) {                                // the scalar tail: elements 32 nfull .. n_kv - 1
             float tail = 0.0f;
-            for (int e = 32 * nfull; e < n_kv; e++) tail = fmaf(h2f(vr[e]), h2f(pr[e]), tail);
+            for (int e = 32 * nfull; e < n_kv; e++) tail = fmaf((float)vr[e], (float)pr[e], tail);
             attn_out[hd_ * 128 + dgrp * 16 + r16] = tail + acc;
         }
         XSTAMP(dbg, 7);
