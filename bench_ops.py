@@ -36,7 +36,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--json", action="store_true")
     ap.add_argument("--reps", type=int, default=20)
-    ap.add_argument("--skip", default="", help="comma list of: peaks, gemv, gemm, attention")
+    ap.add_argument("--skip", default="", help="comma list of: peaks, gemv, gemm, prompt_attention, attention")
     args = ap.parse_args()
     skip = set(args.skip.split(",")) if args.skip else set()
 
@@ -170,6 +170,30 @@ def main():
                 ops = 2.0 * T * M_ * K
                 print("| %s | %d x %d | %d | %.1f | %.0f | %.3f | %.2f |" % (tn, M_, K, T, us, ops / us / 1e6, ops / (us * 1e-6) / INT8_PEAK, nb / (us * 1e-6) / HBM_PEAK))
             print(flush=True)
+
+    if "prompt_attention" not in skip:
+        print("## Prompt attention, 32 heads x 128, f16 KV, one chunk of 2048 queries (`spy_hip_prompt_attention`): against the fp16 MFMA peak\n")
+        print("| cached before | queries | measured µs | useful TFLOP/s (causal q.K and P.V^T once) | of 2.5 PFLOP/s |")
+        print("|---|---|---|---|---|")
+        Hh, hd, T, n_ctx = 32, 128, 2048, 4096
+        rng = np.random.default_rng(5)
+        dq = H.DeviceBuffer.from_numpy(rng.standard_normal((Hh, T, hd)).astype(np.float16))
+        dk = H.DeviceBuffer.from_numpy(rng.standard_normal((n_ctx, Hh * hd)).astype(np.float16))
+        dv = H.DeviceBuffer.from_numpy(rng.standard_normal((Hh * hd, n_ctx)).astype(np.float16))
+        do = H.DeviceBuffer(T * Hh * hd * 4)
+        tot = 0.0
+        for past in (0, 2048):
+            def run():
+                H.check(L.spy_hip_prompt_attention(None, dq.ptr, dk.ptr, dv.ptr, do.ptr, T, Hh, hd, past, n_ctx, 1.0 / np.sqrt(hd)), "spy_hip_prompt_attention")
+            us = time_us(run, 1)
+            pairs = T * past + T * (T + 1) / 2                       # (query, visible position) pairs per head
+            flops = 2.0 * 2.0 * hd * pairs * Hh
+            tot += us
+            print("| %d | %d | %.1f | %.0f | %.3f |" % (past, T, us, flops / us / 1e6, flops / (us * 1e-6) / 2.5e15), flush=True)
+            emit({"op": "prompt_attention", "past": past, "T": T, "us": us, "tflops": flops / us / 1e6})
+        print("\nmean of the two chunks of a 4096-token prompt: %.1f µs per layer and chunk\n" % (tot / 2), flush=True)
+        for b in (dq, dk, dv, do):
+            b.free()
 
     if "attention" not in skip:
         print("## Decode attention, 32 heads x 128, f16 KV (kernels of the single-token pass, 8 layers walked in turn)\n")

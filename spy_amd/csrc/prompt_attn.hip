@@ -10,19 +10,37 @@
 // positions in ascending order.  The softmax needs the row maximum before any exponential and the row
 // sum before any probability, so the scores of a tile are computed three times (cheap on the matrix
 // cores) instead of being kept: pass 1 maximum, pass 2 sum, pass 3 probabilities and the product.
-// Only the order in which a row's exponentials are added differs from softmax_row_kernel (last-bit
-// differences of the sum).
+// (Two passes would need either the scores of a query tile against the whole cache kept somewhere,
+// 64 x n_kv floats, or probabilities rounded to fp16 before the sum is known, which is a different
+// rounding from the operators'.)  The kernel is bound by the vector instructions of the softmax, not
+// by the matrix cores: tiles below the diagonal run without mask compares, the maximum is taken over
+// the raw dot products (rounding is monotonic) and the exponential is seven instructions.
+// Only the order in which a row's exponentials are added, and the last bit of an exponential, differ
+// from softmax_row_kernel.
 //
 // 256 threads = 2 x 2 waves; a score tile is 64 cached positions x 64 queries, one 32 x 32 MFMA tile per
 // wave (positions along the accumulator registers, queries along the lanes, so a lane owns one query);
 // the output tile is 128 head dimensions x 64 queries, two 32 x 32 tiles per wave.
 #include "common.cuh"
 
+#include <type_traits>
+
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
 #define PA_KROW 272     // LDS bytes per K row: 128 halfs + 16 pad
 #define PA_VROW 144     // LDS bytes per V^T / P row: 64 halfs + 16 pad
+
+// e^x for an argument that is a value of fp16 and not above 0 (a score minus its row maximum, rounded as Softmax rounds it).
+// log2(e) = LH + LL with 13 significant bits in LH: x * LH is exact in fp32 for an 11-bit x, so is its distance f to the
+// nearest integer n; e^x = 2^n * 2^(f + x * LL), with v_exp_f32 on an argument within [-0.5, 0.5] and one rounding (an fma)
+// before it: within an ulp or so of expf.  Results below the normal range come out of ldexp as expf returns them.
+static __device__ __forceinline__ float pa_exp(_Float16 xh) {
+    const float LH = 5909.0f / 4096.0f, LL = 6.80877639634e-05f;
+    const float ph = fmaf((float)xh, LH, 0.0f), n = rintf(ph);     // the fp16 operand goes into the fma as it is
+    const float g = fmaf((float)xh, LL, ph - n);
+    return ldexpf(__builtin_amdgcn_exp2f(g), (int)n);
+}
 
 struct pattn_args {
     const uint16_t *q16;   // [H][T][128] fp16 (rotated queries)
@@ -33,10 +51,14 @@ struct pattn_args {
     float scale;
 };
 
-__global__ __launch_bounds__(256, 2) void prompt_attn_kernel(pattn_args a) {
-    __shared__ __attribute__((aligned(16))) uint8_t sK[2][64 * PA_KROW];
-    __shared__ __attribute__((aligned(16))) uint8_t sV[128 * PA_VROW];
+// LDS: K tile 0 | K tile 1 or the V^T tile | P tile = 45 KiB, three workgroups per compute unit.  Passes 1 and 2 alternate
+// between the two K tiles (one barrier per tile); pass 3 has a second barrier per tile anyway (between the scores and the
+// product), which also separates a tile's K reads from the next tile's K store: it keeps K in tile 0 and V^T in the other.
+__global__ __launch_bounds__(256, 3) void prompt_attn_kernel(pattn_args a) {
+    __shared__ __attribute__((aligned(16))) uint8_t sKV[64 * PA_KROW + 128 * PA_VROW];
     __shared__ __attribute__((aligned(16))) uint8_t sP[64 * PA_VROW];
+    static_assert(128 * PA_VROW >= 64 * PA_KROW, "the V^T tile covers the second K tile");
+    uint8_t *const sK0 = sKV, *const sK1 = sKV + 64 * PA_KROW, *const sV = sK1;
     __shared__ float s_stat[2][64];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
     const int T = a.T, H = a.H, NQ = (T + 63) / 64;
@@ -64,10 +86,20 @@ __global__ __launch_bounds__(256, 2) void prompt_attn_kernel(pattn_args a) {
     quad rk, rv;
     const uint16_t *kbase = a.kc + (size_t)h * 128 + (tid & 15) * 8;         // thread's 16-byte piece of rows (tid >> 4) + 16 i
     const uint16_t *vbase = a.vc + ((size_t)h * 128 + (tid >> 3)) * a.n_ctx;   // thread's piece (tid & 7) of rows (tid >> 3) + 32 i
-    auto krow = [&](int j, int i) { return (const uint4 *)(kbase + (size_t)min(j * 64 + (tid >> 4) + 16 * i, n_kv - 1) * d); };
-    auto gload_k = [&](int j) -> quad { return quad{*krow(j, 0), *krow(j, 1), *krow(j, 2), *krow(j, 3)}; };
+    // A tile whose 64 rows all lie inside the cache takes its addresses from the tile index alone; the last tile clamps (rows
+    // past the cache end re-read its last row: masked below).
+    const uint16_t *kthread = kbase + (size_t)(tid >> 4) * d;
+    const size_t k16 = (size_t)16 * d;
+    auto gload_k = [&](int j) -> quad {
+        if (j * 64 + 64 <= n_kv) {
+            const uint16_t *p = kthread + (size_t)j * 64 * d;
+            return quad{*(const uint4 *)p, *(const uint4 *)(p + k16), *(const uint4 *)(p + 2 * k16), *(const uint4 *)(p + 3 * k16)};
+        }
+        auto krow = [&](int i) { return (const uint4 *)(kbase + (size_t)min(j * 64 + (tid >> 4) + 16 * i, n_kv - 1) * d); };
+        return quad{*krow(0), *krow(1), *krow(2), *krow(3)};
+    };
     auto store_k = [&](int b, const quad &r) {
-        uint8_t *p = sK[b] + (tid >> 4) * PA_KROW + (tid & 15) * 16;
+        uint8_t *p = (b ? sK1 : sK0) + (tid >> 4) * PA_KROW + (tid & 15) * 16;
         *(uint4 *)p = r.a; *(uint4 *)(p + 16 * PA_KROW) = r.b; *(uint4 *)(p + 32 * PA_KROW) = r.c; *(uint4 *)(p + 48 * PA_KROW) = r.d;
     };
     auto gload_v = [&](int j) -> quad {                             // V^T tile: 128 rows x 64 positions
@@ -84,49 +116,69 @@ __global__ __launch_bounds__(256, 2) void prompt_attn_kernel(pattn_args a) {
         v16f acc = {0};
 #pragma unroll
         for (int ks = 0; ks < 8; ks++) {
-            const v8h fa = *(const v8h *)(sK[b] + (wm * 32 + (lane & 31)) * PA_KROW + ks * 32 + (lane >> 5) * 16);
+            const v8h fa = *(const v8h *)((b ? sK1 : sK0) + (wm * 32 + (lane & 31)) * PA_KROW + ks * 32 + (lane >> 5) * 16);
             acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa, fq[ks], acc, 0, 0, 0);
         }
         return acc;
     };
     // accumulator register r of tile j holds position j*64 + wm*32 + (r/4)*8 + (lane>>5)*4 + (r&3)
     const int pos0 = wm * 32 + (lane >> 5) * 4;
+    // Tiles 0 .. nfree-1 lie below the diagonal for every query of the workgroup (their last position is visible to query q0):
+    // no masking there.  The remaining one or two tiles compare positions against the lane's limit.
+    const int nfree = min(ntile, max(0, (a.past + q0 + 1) / 64));
+    using free_t = std::integral_constant<bool, false>;
+    using diag_t = std::integral_constant<bool, true>;
 
-    // pass 1: row maximum of t = s * scale
-    float m = -INFINITY;
+    // pass 1: row maximum of t = s * scale.  Rounding is monotonic, so max(s * scale) = max(s) * scale: one product per row.
+    float smax = -INFINITY;
     rk = gload_k(0);
-    for (int j = 0; j < ntile; j++) {
+    auto pass1 = [&](int j, auto masked) {
         store_k(j & 1, rk);
         rk = gload_k(min(j + 1, ntile - 1));                        // unconditional: the last tile re-reads itself
         __syncthreads();
         const v16f s = scores(j & 1);
-        const int room = limit - (j * 64 + pos0);                   // register r is visible to this lane's query iff (r/4)*8 + (r&3) <= room
+        if constexpr (decltype(masked)::value) {
+            const int room = limit - (j * 64 + pos0);               // register r is visible to this lane's query iff (r/4)*8 + (r&3) <= room
 #pragma unroll
-        for (int r = 0; r < 16; r++) m = fmaxf(m, ((r >> 2) * 8 + (r & 3) <= room) ? s[r] * scale : -INFINITY);
-    }
+            for (int r = 0; r < 16; r++) smax = fmaxf(smax, ((r >> 2) * 8 + (r & 3) <= room) ? s[r] : -INFINITY);
+        } else {
+#pragma unroll
+            for (int r = 0; r < 16; r++) smax = fmaxf(smax, s[r]);
+        }
+    };
+    for (int j = 0; j < nfree; j++) pass1(j, free_t{});
+    for (int j = nfree; j < ntile; j++) pass1(j, diag_t{});
+    float m = smax * scale;
     m = fmaxf(m, __shfl_xor(m, 32, SPY_WAVE));
     if (lane < 32) s_stat[wm][ql] = m;
     __syncthreads();
     m = fmaxf(s_stat[0][ql], s_stat[1][ql]);
     __syncthreads();
 
-    // pass 2: row sum of e = expf(fp16(t - m))
+    // pass 2: row sum of e = exp(fp16(t - m))
     float sum = 0.0f;
     rk = gload_k(0);
-    for (int j = 0; j < ntile; j++) {
+    auto pass2 = [&](int j, auto masked) {
         store_k(j & 1, rk);
         rk = gload_k(min(j + 1, ntile - 1));
         __syncthreads();
         const v16f s = scores(j & 1);
         // every exponential is evaluated (no divergent branches: the 16 evaluations interleave) and the masked ones are
         // replaced by 0 afterwards; adding those zeros changes nothing
-        const int room = limit - (j * 64 + pos0);
         float e[16];
 #pragma unroll
-        for (int r = 0; r < 16; r++) e[r] = expf(h2f(f2h(s[r] * scale - m)));
+        for (int r = 0; r < 16; r++) e[r] = pa_exp((_Float16)(s[r] * scale - m));
+        if constexpr (decltype(masked)::value) {
+            const int room = limit - (j * 64 + pos0);
 #pragma unroll
-        for (int r = 0; r < 16; r++) sum += ((r >> 2) * 8 + (r & 3) <= room) ? e[r] : 0.0f;
-    }
+            for (int r = 0; r < 16; r++) sum += ((r >> 2) * 8 + (r & 3) <= room) ? e[r] : 0.0f;
+        } else {
+#pragma unroll
+            for (int r = 0; r < 16; r++) sum += e[r];
+        }
+    };
+    for (int j = 0; j < nfree; j++) pass2(j, free_t{});
+    for (int j = nfree; j < ntile; j++) pass2(j, diag_t{});
     sum += __shfl_xor(sum, 32, SPY_WAVE);
     if (lane < 32) s_stat[wm][ql] = sum;
     __syncthreads();
@@ -135,21 +187,24 @@ __global__ __launch_bounds__(256, 2) void prompt_attn_kernel(pattn_args a) {
     // pass 3: probabilities (fp16) through LDS, times V^T
     v16f oacc[2] = {{0}, {0}};
     rk = gload_k(0);
-    for (int j = 0; j < ntile; j++) {
-        store_k(j & 1, rk);
+    auto pass3 = [&](int j, auto masked) {
+        store_k(0, rk);                                             // every wave passed the previous tile's second barrier: its K reads are done
         rk = gload_k(min(j + 1, ntile - 1));
         rv = gload_v(j);                                            // needed after the scores of this tile
         __syncthreads();                                            // K tile stored; every wave is done with the previous tile's sP / sV
-        const v16f s = scores(j & 1);
+        const v16f s = scores(0);
         const int room = limit - (j * 64 + pos0);
         float e[16];
 #pragma unroll
-        for (int r = 0; r < 16; r++) e[r] = expf(h2f(f2h(s[r] * scale - m)));
+        for (int r = 0; r < 16; r++) e[r] = pa_exp((_Float16)(s[r] * scale - m));
 #pragma unroll
         for (int g = 0; g < 4; g++) {
             uint32_t p[4];
 #pragma unroll
-            for (int k = 0; k < 4; k++) p[k] = f2h((g * 8 + k <= room) ? e[4 * g + k] * inv : 0.0f);
+            for (int k = 0; k < 4; k++) {
+                if constexpr (decltype(masked)::value) p[k] = f2h((g * 8 + k <= room) ? e[4 * g + k] * inv : 0.0f);
+                else p[k] = f2h(e[4 * g + k] * inv);
+            }
             *(uint2 *)(sP + ql * PA_VROW + (pos0 + g * 8) * 2) = make_uint2(p[0] | (p[1] << 16), p[2] | (p[3] << 16));
         }
         store_v(rv);
@@ -162,7 +217,9 @@ __global__ __launch_bounds__(256, 2) void prompt_attn_kernel(pattn_args a) {
                 const v8h fb = *(const v8h *)(sP + ql * PA_VROW + ks * 32 + (lane >> 5) * 16);
                 oacc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa, fb, oacc[i], 0, 0, 0);
             }
-    }
+    };
+    for (int j = 0; j < nfree; j++) pass3(j, free_t{});
+    for (int j = nfree; j < ntile; j++) pass3(j, diag_t{});
     if (t < T) {
         float *o = a.out + ((size_t)t * H + h) * 128;
 #pragma unroll
