@@ -96,6 +96,9 @@ def main():
     if "peaks" not in skip:
         tops, gbps = C.c_float(), C.c_float()
         H.check(L.spy_hip_measure_mfma_i8(None, 20000, C.byref(tops)), "spy_hip_measure_mfma_i8")
+        sc = [C.c_float(), C.c_float()]
+        for mode in (0, 1):
+            H.check(L.spy_hip_measure_mfma_i8_scaled(None, 20000, mode, C.byref(sc[mode])), "spy_hip_measure_mfma_i8_scaled")
         buf = H.DeviceBuffer(2 << 30)
         H.check(L.spy_hip_fill_u8(buf.ptr, 1, buf.nbytes, None), "fill")
         H.check(L.spy_hip_measure_hbm_read(None, buf.ptr, buf.nbytes, 10, C.byref(gbps)), "spy_hip_measure_hbm_read")
@@ -104,8 +107,12 @@ def main():
         print("| what | measured | published peak used as denominator | measured / published |")
         print("|---|---|---|---|")
         print("| int8 MFMA, register operands only (`v_mfma_i32_32x32x32_i8`) | %.0f TOP/s | 5000 TOP/s | %.2f |" % (tops.value, tops.value * 1e12 / INT8_PEAK))
+        print("| the same MFMA + fp16 scale outer product + conversion and fma per output (block-scaled GEMM inner loop, registers only) | %.0f TOP/s | 5000 TOP/s | %.2f |" % (sc[0].value, sc[0].value * 1e12 / INT8_PEAK))
+        print("| ... with the accumulator biased by 0x4B400000 and a subtraction in place of the conversion (what `spy_hip_gemm_q8_0act` runs) | %.0f TOP/s | 5000 TOP/s | %.2f |" % (sc[1].value, sc[1].value * 1e12 / INT8_PEAK))
         print("| HBM read, 2 GiB scan | %.0f GB/s | 8000 GB/s | %.2f |\n" % (gbps.value, gbps.value * 1e9 / HBM_PEAK), flush=True)
         emit({"op": "peak_mfma_i8", "tops": tops.value})
+        emit({"op": "peak_mfma_i8_scaled_cvt", "tops": sc[0].value})
+        emit({"op": "peak_mfma_i8_scaled_biased", "tops": sc[1].value})
         emit({"op": "peak_hbm_read", "gbps": gbps.value})
 
     def weights(wt, M_, K):

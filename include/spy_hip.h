@@ -201,6 +201,12 @@ int spy_hip_ffn_gate_up_silu(void *stream, int32_t order, int32_t wtype, const v
 /* int8 matrix-core rate in TOP/s (2 operations per multiply-accumulate): waves issuing only
  * v_mfma_i32_32x32x32_i8 on register operands, iters x 4 per wave */
 int spy_hip_measure_mfma_i8(void *stream, int32_t iters, float *tops);
+/* The same matrix instruction with what a block-scaled GEMM adds per quantization block and 32 x 32 tile, on register
+ * operands only: the fp16 outer product of the scales and the 32 vector instructions per lane that scale and
+ * accumulate the block dots (mode 0: conversion + fma; mode 1: biased integer accumulator, subtraction + fma, as
+ * spy_hip_gemm_q8_0act does it).  The ceiling that this epilogue leaves to the int8 matrix cores; TOP/s of int8
+ * operations.  No counterpart in the reference. */
+int spy_hip_measure_mfma_i8_scaled(void *stream, int32_t iters, int32_t mode, float *tops);
 /* read rate in GB/s over `bytes` of device memory (16-byte aligned, >= 1 MiB; use >= 1 GiB), reps passes */
 int spy_hip_measure_hbm_read(void *stream, const void *buf, size_t bytes, int32_t reps, float *gbps);
 

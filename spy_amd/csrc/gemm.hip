@@ -37,22 +37,38 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 #define GEMM_WGS 3                // workgroups per CU the tile kernel is compiled for (register budget 512 / GEMM_WGS per lane)
 #endif
 #ifndef GEMM_PF_Q4_0
-#define GEMM_PF_Q4_0 2           // Q4_0: two stages of global loads in flight (+2-5 % for M >= 11008, the operands come from beyond the L2); Q8_0 keeps one: two would spill
+#define GEMM_PF_Q4_0 1           // stages of global loads in flight for Q4_0; two (+2-5 % for M >= 11008) no longer fit the register budget of three workgroups per CU next to the 16 registers of the accumulator bias
 #endif
 
 // 32-bit word of 4 packed nibbles (already masked to 0..15 per byte) -> 4 int8 of (n - 8)
 static __device__ __forceinline__ uint32_t nib_m8(uint32_t lo) { return (lo + 0x78787878u) ^ 0x80808080u; }
+
+// Workgroups of the XCD-aware one-dimensional grid of gemm_q8act_kernel for gx x gy tiles: 8 XCDs x ceil(gx / 4) x ceil(gy / 2)
+// (the workgroups whose tile falls outside return at once).
+static inline int64_t gemm_xcd_grid(int64_t gx, int64_t gy) { return 8 * ((gx + 3) / 4) * ((gy + 1) / 2); }
 
 template <int WT>
 __global__ __launch_bounds__(256, GEMM_WGS) void gemm_q8act_kernel(const uint8_t *__restrict__ W1, const uint8_t *__restrict__ xq, float *__restrict__ dst1,
                                                             int M, int K, int T, int64_t dst_stride, const uint8_t *__restrict__ W2, float *__restrict__ dst2) {
     // Optionally two weight matrices of the same shape against the same activations in one grid (gate and up): the
     // workgroups of the second follow those of the first, which halves the share of the grid's tail.
-    const int tiles1 = (M + GEMM_TILE - 1) / GEMM_TILE;
-    const bool second = W2 != nullptr && (int)blockIdx.x >= tiles1;
+    // Workgroup L of the one-dimensional grid runs on XCD L % 8, each with its own L2.  The eight XCDs form a 4 x 2
+    // arrangement over (weight tiles, activation tiles): XCD (mj, ti) takes the weight tiles = mj (mod 4) against the
+    // activation tiles = ti (mod 2), so that a weight tile is fetched by two L2s and an activation tile by four (a
+    // row-major grid has every L2 fetch all the activations).  Within an XCD the weight tiles of one activation tile
+    // follow each other.
+    const int tiles1 = (M + GEMM_TILE - 1) / GEMM_TILE, gx = W2 ? 2 * tiles1 : tiles1, gy = (T + GEMM_TILE - 1) / GEMM_TILE;
+    int gbx, gby;
+    {
+        const int xcd = (int)blockIdx.x & 7, slot = (int)blockIdx.x >> 3, nm = (gx + 3) >> 2;
+        gbx = (slot % nm) * 4 + (xcd & 3);
+        gby = (slot / nm) * 2 + (xcd >> 2);
+        if (gbx >= gx || gby >= gy) return;
+    }
+    const bool second = W2 != nullptr && gbx >= tiles1;
     const uint8_t *W = second ? W2 : W1;
     float *dst = second ? dst2 : dst1;
-    const int bx = second ? (int)blockIdx.x - tiles1 : (int)blockIdx.x;
+    const int bx = second ? gbx - tiles1 : gbx;
     constexpr int PF = (WT == SPY_HIP_Q4_0) ? GEMM_PF_Q4_0 : 1; // stages of global loads in flight per thread
     constexpr int PAIR_DW = (WT == SPY_HIP_Q4_0) ? 9 : 17;       // dwords per pair of weight blocks
     constexpr int HALF_DW = (WT == SPY_HIP_Q4_0) ? 5 : 9;        // dwords that cover one block of the pair
@@ -61,7 +77,7 @@ __global__ __launch_bounds__(256, GEMM_WGS) void gemm_q8act_kernel(const uint8_t
     __shared__ uint16_t sAd[2][2][GEMM_TILE];                                // fp16 block scales [buffer][block of the pair][row]
     __shared__ uint16_t sBd[2][2][GEMM_TILE];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
-    const int m0 = bx * GEMM_TILE, t0 = blockIdx.y * GEMM_TILE;
+    const int m0 = bx * GEMM_TILE, t0 = gby * GEMM_TILE;
     const int nstage = K / 64;
     const size_t RBw = (size_t)(K / 32) * (WT == SPY_HIP_Q4_0 ? 18 : 34), RBx = (size_t)(K / 32) * 34;
 
@@ -116,8 +132,13 @@ __global__ __launch_bounds__(256, GEMM_WGS) void gemm_q8act_kernel(const uint8_t
     // Per block and 32 x 32 tile: the int32 block dots from one int8 MFMA, and the scale products
     // h2f(d_w) * h2f(d_x) of the same tile from one fp16 MFMA whose operands hold the scales at k = 0 and zeros
     // elsewhere (an outer product; fp16 x fp16 is exact in fp32, so these are the bits of the scalar product).
-    // That leaves a conversion and an fma per output on the vector units, which bound this kernel.
+    // That leaves a subtraction (below) and an fma per output on the vector units, which bound this kernel.
+    // The block dots are accumulated onto the integer 0x4B400000: as a float that is 12582912 + dot exactly (|dot| <= 32 * 127 * 127
+    // < 2^22), and subtracting 12582912 gives float(dot) with a full-rate instruction where a conversion runs at half rate.
     const int k0mask = lane < 32 ? 0xFFFF : 0;
+    v16i bias;
+#pragma unroll
+    for (int r = 0; r < 16; r++) bias[r] = 0x4B400000;
     auto multiply = [&](int b) {
 #pragma unroll 1
         for (int blk = 0; blk < 2; blk++) {
@@ -136,12 +157,11 @@ __global__ __launch_bounds__(256, GEMM_WGS) void gemm_q8act_kernel(const uint8_t
             for (int i = 0; i < 2; i++)
 #pragma unroll
                 for (int j = 0; j < 2; j++) {
-                    v16i z = {0};
                     v16f zf = {0};
-                    const v16i I = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], z, 0, 0, 0);
+                    const v16i I = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], bias, 0, 0, 0);
                     const v16f S = __builtin_amdgcn_mfma_f32_32x32x8f16(ha[i], hb[j], zf, 0, 0, 0);
 #pragma unroll
-                    for (int r = 0; r < 16; r++) acc[i][j][r] = fmaf(S[r], (float)I[r], acc[i][j][r]);
+                    for (int r = 0; r < 16; r++) acc[i][j][r] = fmaf(S[r], __int_as_float(I[r]) - 12582912.0f, acc[i][j][r]);
                 }
         }
     };
@@ -598,8 +618,10 @@ extern "C" int spy_hip_gemm_q8_0act(void *stream, int wtype, const void *w_dev, 
     // weights) beat the 128 x 128 tile, which leaves most of the part idle there (T = 16: 32 us against 130-230 us)
     if ((wtype == SPY_HIP_Q4_K || wtype == SPY_HIP_Q6_K) && T <= 32 && K <= 12288 && !force)
         return spy_hip_gemv_q8_0act(stream, wtype, w_dev, xq_dev, dst_dev, nullptr, M, K, T, dst_stride);
-    if (wtype == SPY_HIP_Q4_0) gemm_q8act_kernel<SPY_HIP_Q4_0><<<grid, dim3(256), 0, st>>>((const uint8_t *)w_dev, (const uint8_t *)xq_dev, dst_dev, (int)M, (int)K, (int)T, dst_stride, nullptr, nullptr);
-    else if (wtype == SPY_HIP_Q8_0) gemm_q8act_kernel<SPY_HIP_Q8_0><<<grid, dim3(256), 0, st>>>((const uint8_t *)w_dev, (const uint8_t *)xq_dev, dst_dev, (int)M, (int)K, (int)T, dst_stride, nullptr, nullptr);
+    const int64_t xgrid = gemm_xcd_grid(grid.x, grid.y);
+    SPY_CHECK_ARG((wtype != SPY_HIP_Q4_0 && wtype != SPY_HIP_Q8_0) || xgrid <= 0x7fffffff);
+    if (wtype == SPY_HIP_Q4_0) gemm_q8act_kernel<SPY_HIP_Q4_0><<<dim3((unsigned)xgrid), dim3(256), 0, st>>>((const uint8_t *)w_dev, (const uint8_t *)xq_dev, dst_dev, (int)M, (int)K, (int)T, dst_stride, nullptr, nullptr);
+    else if (wtype == SPY_HIP_Q8_0) gemm_q8act_kernel<SPY_HIP_Q8_0><<<dim3((unsigned)xgrid), dim3(256), 0, st>>>((const uint8_t *)w_dev, (const uint8_t *)xq_dev, dst_dev, (int)M, (int)K, (int)T, dst_stride, nullptr, nullptr);
     else if (wtype == SPY_HIP_Q4_K || wtype == SPY_HIP_Q6_K) {
         // 64 x 64 tiles where the 128 x 128 tiling gives too few workgroups to fill the part: 1.8-2.9 x faster up to 512 activation
         // rows of the 7B shapes, equal where its own workgroups stop being resident all at once, 30 % slower beyond
@@ -629,9 +651,10 @@ int spy_gemm_q8act_pair(hipStream_t st, int wtype, const void *w1, const void *w
         int rc = spy_hip_gemm_q8_0act(st, wtype, w1, xq, dst1, M, K, T, dst_stride);
         return rc ? rc : spy_hip_gemm_q8_0act(st, wtype, w2, xq, dst2, M, K, T, dst_stride);
     }
-    const dim3 grid((unsigned)(2 * tiles), (unsigned)ttiles);
-    if (wtype == SPY_HIP_Q4_0) gemm_q8act_kernel<SPY_HIP_Q4_0><<<grid, dim3(256), 0, st>>>((const uint8_t *)w1, (const uint8_t *)xq, dst1, (int)M, (int)K, (int)T, dst_stride, (const uint8_t *)w2, dst2);
-    else gemm_q8act_kernel<SPY_HIP_Q8_0><<<grid, dim3(256), 0, st>>>((const uint8_t *)w1, (const uint8_t *)xq, dst1, (int)M, (int)K, (int)T, dst_stride, (const uint8_t *)w2, dst2);
+    const int64_t xgrid = gemm_xcd_grid(2 * tiles, ttiles);
+    SPY_CHECK_ARG(xgrid <= 0x7fffffff);
+    if (wtype == SPY_HIP_Q4_0) gemm_q8act_kernel<SPY_HIP_Q4_0><<<dim3((unsigned)xgrid), dim3(256), 0, st>>>((const uint8_t *)w1, (const uint8_t *)xq, dst1, (int)M, (int)K, (int)T, dst_stride, (const uint8_t *)w2, dst2);
+    else gemm_q8act_kernel<SPY_HIP_Q8_0><<<dim3((unsigned)xgrid), dim3(256), 0, st>>>((const uint8_t *)w1, (const uint8_t *)xq, dst1, (int)M, (int)K, (int)T, dst_stride, (const uint8_t *)w2, dst2);
     return SPY_LAUNCH_RC();
 }
 
