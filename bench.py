@@ -239,7 +239,13 @@ def main():
                                    % ({H.Q4_0: "Q4_0", H.Q8_0: "Q8_0", H.Q4_K: "Q4_K", H.Q6_K: "Q6_K"}[wt_g], d_, d_, F_, d_, d_, F_, Tg),
                          "bound": "mfma", "achieved": round(tops, 1), "peak": INT8_PEAK / 1e12, "unit": "TOP/s", "frac": round(tops * 1e12 / INT8_PEAK, 4),
                          "ops_per_set": ops_set, "us_per_set": round(us_set, 1)}
-        log("prompt GEMMs of a layer, T = %d: %.1f us, %.0f TOP/s (%.1f%% of the int8 MFMA peak)" % (Tg, us_set, tops, 100 * tops * 1e12 / INT8_PEAK))
+        # what the per-block scaling leaves to the matrix cores: the kernel's inner loop on register operands only
+        ceil_tops = C.c_float()
+        H.check(L.spy_hip_measure_mfma_i8_scaled(None, 20000, 1, C.byref(ceil_tops)), "spy_hip_measure_mfma_i8_scaled")
+        gemm_roofline["inner_loop_registers_only"] = {"achieved": round(ceil_tops.value, 1), "unit": "TOP/s", "frac_of_peak": round(ceil_tops.value * 1e12 / INT8_PEAK, 4),
+                                                      "what": "one v_mfma_i32_32x32x32_i8 + the fp16 scale outer product + subtraction and fma per output, no LDS or memory"}
+        log("prompt GEMMs of a layer, T = %d: %.1f us, %.0f TOP/s (%.1f%% of the int8 MFMA peak); its inner loop on register operands only: %.0f TOP/s (%.1f%%)"
+            % (Tg, us_set, tops, 100 * tops * 1e12 / INT8_PEAK, ceil_tops.value, 100 * ceil_tops.value * 1e12 / INT8_PEAK))
         for b in (w_dd, w_Fd, w_dF, x_d, x_F, og):
             b.free()
 

@@ -209,16 +209,20 @@ def main():
         cfg = M.Config.llama2_7b(n_ctx=4352, wtype=H.Q4_0)
         cfg.n_layer = 8
         tensors = M.synth_model(cfg, seed=11)
-        for split in (True, False):
+        for mode in ("own_split", "own_fused", "host_order"):
+            split = mode == "own_split"
             if split:
                 os.environ["SPY_HIP_ATTN_SPLIT"] = "1"
             else:
                 os.environ.pop("SPY_HIP_ATTN_SPLIT", None)
-            eng = M.Engine(cfg, tensors)
+            eng = M.Engine(cfg, tensors, order=1 if mode == "host_order" else 0)
             for n_kv in (512, 4096):
                 eng.forward(np.array([1], np.int32), n_kv - 1, want_logits=False)       # leaves position n_kv - 1
                 kv = 2 * n_kv * cfg.n_embd * 2
-                if split:
+                if mode == "host_order":
+                    s_us, p_us = eng.kernel_time_us("scores", args.reps), eng.kernel_time_us("pv", args.reps)
+                    us, nb, label = s_us + p_us, kv, "host summation order: `xattn_scores_kernel` %.2f + `xattn_pv_kernel` %.2f" % (s_us, p_us)
+                elif split:
                     s_us, p_us = eng.kernel_time_us("scores", args.reps), eng.kernel_time_us("pv", args.reps)
                     us, nb, label = s_us + p_us, kv, "`attn_scores_kernel` %.2f + `attn_pv_kernel` %.2f" % (s_us, p_us)
                 elif eng.fuses_attention():
@@ -227,7 +231,7 @@ def main():
                 else:
                     continue
                 print("| %d | %s | %d | %.2f | %.2f | %.0f | %.2f |" % (n_kv, label, nb, nb / HBM_PEAK * 1e6, us, nb / us / 1e3, nb / (us * 1e-6) / HBM_PEAK), flush=True)
-                emit({"op": "attention_split" if split else "attention_layer", "n_kv": n_kv, "bytes": nb, "us": us, "hbm_frac": nb / (us * 1e-6) / HBM_PEAK})
+                emit({"op": "attention_" + mode, "n_kv": n_kv, "bytes": nb, "us": us, "hbm_frac": nb / (us * 1e-6) / HBM_PEAK})
             eng.close()
         print(flush=True)
 

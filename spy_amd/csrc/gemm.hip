@@ -46,23 +46,31 @@ static __device__ __forceinline__ uint32_t nib_m8(uint32_t lo) { return (lo + 0x
 // Workgroups of the XCD-aware one-dimensional grid of gemm_q8act_kernel for gx x gy tiles: 8 XCDs x ceil(gx / 4) x ceil(gy / 2)
 // (the workgroups whose tile falls outside return at once).
 static inline int64_t gemm_xcd_grid(int64_t gx, int64_t gy) { return 8 * ((gx + 3) / 4) * ((gy + 1) / 2); }
+// 1 where an XCD's quarter of the gx weight tiles (128 rows of K / 32 blocks each) does not fit its L2 with room to spare
+static inline int gemm_t_inner(int64_t gx, int64_t K, int wtype) {
+    return ((gx + 3) / 4) * GEMM_TILE * (K / 32) * (wtype == SPY_HIP_Q4_0 ? 18 : 34) > (3ll << 20);
+}
 
 template <int WT>
 __global__ __launch_bounds__(256, GEMM_WGS) void gemm_q8act_kernel(const uint8_t *__restrict__ W1, const uint8_t *__restrict__ xq, float *__restrict__ dst1,
-                                                            int M, int K, int T, int64_t dst_stride, const uint8_t *__restrict__ W2, float *__restrict__ dst2) {
+                                                            int M, int K, int T, int64_t dst_stride, const uint8_t *__restrict__ W2, float *__restrict__ dst2, int t_inner) {
     // Optionally two weight matrices of the same shape against the same activations in one grid (gate and up): the
     // workgroups of the second follow those of the first, which halves the share of the grid's tail.
     // Workgroup L of the one-dimensional grid runs on XCD L % 8, each with its own L2.  The eight XCDs form a 4 x 2
     // arrangement over (weight tiles, activation tiles): XCD (mj, ti) takes the weight tiles = mj (mod 4) against the
     // activation tiles = ti (mod 2), so that a weight tile is fetched by two L2s and an activation tile by four (a
-    // row-major grid has every L2 fetch all the activations).  Within an XCD the weight tiles of one activation tile
-    // follow each other.
+    // row-major grid has every L2 fetch all the activations).  Where the XCD's share of the weight matrix is larger than
+    // its 4 MB L2 (t_inner), the activation tiles of one weight tile follow each other: the hundred or so workgroups an
+    // XCD runs at a time then share a dozen weight tiles and its activation tiles, where the other order streams all its
+    // weight tiles through the L2 once per activation tile (measured: 14 times the algorithmic bytes for gate|up, and
+    // 5-9 % slower).  Where the share fits (4096 x 4096), weight tiles follow each other (that order is 9 % faster there).
     const int tiles1 = (M + GEMM_TILE - 1) / GEMM_TILE, gx = W2 ? 2 * tiles1 : tiles1, gy = (T + GEMM_TILE - 1) / GEMM_TILE;
     int gbx, gby;
     {
-        const int xcd = (int)blockIdx.x & 7, slot = (int)blockIdx.x >> 3, nm = (gx + 3) >> 2;
-        gbx = (slot % nm) * 4 + (xcd & 3);
-        gby = (slot / nm) * 2 + (xcd >> 2);
+        const int xcd = (int)blockIdx.x & 7, slot = (int)blockIdx.x >> 3, nt = (gy + 1) >> 1, nm = (gx + 3) >> 2;
+        const int sm = t_inner ? slot / nt : slot % nm, stt = t_inner ? slot % nt : slot / nm;
+        gbx = sm * 4 + (xcd & 3);
+        gby = stt * 2 + (xcd >> 2);
         if (gbx >= gx || gby >= gy) return;
     }
     const bool second = W2 != nullptr && gbx >= tiles1;
@@ -620,8 +628,9 @@ extern "C" int spy_hip_gemm_q8_0act(void *stream, int wtype, const void *w_dev, 
         return spy_hip_gemv_q8_0act(stream, wtype, w_dev, xq_dev, dst_dev, nullptr, M, K, T, dst_stride);
     const int64_t xgrid = gemm_xcd_grid(grid.x, grid.y);
     SPY_CHECK_ARG((wtype != SPY_HIP_Q4_0 && wtype != SPY_HIP_Q8_0) || xgrid <= 0x7fffffff);
-    if (wtype == SPY_HIP_Q4_0) gemm_q8act_kernel<SPY_HIP_Q4_0><<<dim3((unsigned)xgrid), dim3(256), 0, st>>>((const uint8_t *)w_dev, (const uint8_t *)xq_dev, dst_dev, (int)M, (int)K, (int)T, dst_stride, nullptr, nullptr);
-    else if (wtype == SPY_HIP_Q8_0) gemm_q8act_kernel<SPY_HIP_Q8_0><<<dim3((unsigned)xgrid), dim3(256), 0, st>>>((const uint8_t *)w_dev, (const uint8_t *)xq_dev, dst_dev, (int)M, (int)K, (int)T, dst_stride, nullptr, nullptr);
+    const int t_inner = gemm_t_inner(grid.x, K, wtype);
+    if (wtype == SPY_HIP_Q4_0) gemm_q8act_kernel<SPY_HIP_Q4_0><<<dim3((unsigned)xgrid), dim3(256), 0, st>>>((const uint8_t *)w_dev, (const uint8_t *)xq_dev, dst_dev, (int)M, (int)K, (int)T, dst_stride, nullptr, nullptr, t_inner);
+    else if (wtype == SPY_HIP_Q8_0) gemm_q8act_kernel<SPY_HIP_Q8_0><<<dim3((unsigned)xgrid), dim3(256), 0, st>>>((const uint8_t *)w_dev, (const uint8_t *)xq_dev, dst_dev, (int)M, (int)K, (int)T, dst_stride, nullptr, nullptr, t_inner);
     else if (wtype == SPY_HIP_Q4_K || wtype == SPY_HIP_Q6_K) {
         // 64 x 64 tiles where the 128 x 128 tiling gives too few workgroups to fill the part: 1.8-2.9 x faster up to 512 activation
         // rows of the 7B shapes, equal where its own workgroups stop being resident all at once, 30 % slower beyond
@@ -653,8 +662,9 @@ int spy_gemm_q8act_pair(hipStream_t st, int wtype, const void *w1, const void *w
     }
     const int64_t xgrid = gemm_xcd_grid(2 * tiles, ttiles);
     SPY_CHECK_ARG(xgrid <= 0x7fffffff);
-    if (wtype == SPY_HIP_Q4_0) gemm_q8act_kernel<SPY_HIP_Q4_0><<<dim3((unsigned)xgrid), dim3(256), 0, st>>>((const uint8_t *)w1, (const uint8_t *)xq, dst1, (int)M, (int)K, (int)T, dst_stride, (const uint8_t *)w2, dst2);
-    else gemm_q8act_kernel<SPY_HIP_Q8_0><<<dim3((unsigned)xgrid), dim3(256), 0, st>>>((const uint8_t *)w1, (const uint8_t *)xq, dst1, (int)M, (int)K, (int)T, dst_stride, (const uint8_t *)w2, dst2);
+    const int t_inner = gemm_t_inner(2 * tiles, K, wtype);
+    if (wtype == SPY_HIP_Q4_0) gemm_q8act_kernel<SPY_HIP_Q4_0><<<dim3((unsigned)xgrid), dim3(256), 0, st>>>((const uint8_t *)w1, (const uint8_t *)xq, dst1, (int)M, (int)K, (int)T, dst_stride, (const uint8_t *)w2, dst2, t_inner);
+    else gemm_q8act_kernel<SPY_HIP_Q8_0><<<dim3((unsigned)xgrid), dim3(256), 0, st>>>((const uint8_t *)w1, (const uint8_t *)xq, dst1, (int)M, (int)K, (int)T, dst_stride, (const uint8_t *)w2, dst2, t_inner);
     return SPY_LAUNCH_RC();
 }
 
