@@ -366,6 +366,8 @@ __global__ __launch_bounds__(XG_THREADS) void xgemv_kernel(xg_args a) {
 
     constexpr int NSTEPS = EPI == EPI_QKV ? 2 : NSTEP;
     static_assert(NITK == 1 || NROW == 1, "rows longer than one slab are walked one row per wave");
+    act_frag<1> af, av;
+    int n8[16];
 #pragma unroll
     for (int step = 0; step < NSTEPS; step++) {
         const int r0 = EPI == EPI_QKV ? 2 * step : step * RPS;                  // first row of the step
@@ -379,19 +381,20 @@ __global__ __launch_bounds__(XG_THREADS) void xgemv_kernel(xg_args a) {
             const int nblk = min(XG_NBS, K / 32 - it * XG_NBS);                // blocks of this slab
             if (nblk > 0) {
                 const int p = it * 64 + lane;
-                // this lane's activations of the slab (the same for every row) and the -8 * sum q per dword
-                act_frag<1> af, av;
-                int n8[16];
-                if (p < npair) {
-                    load_act_frag<WT, 1>(af, act, npair, p);
-                    if constexpr (WTV != WT) { if (vstep) load_act_frag<WTV, 1>(av, act, npair, p); }
-                    if constexpr (WT == SPY_HIP_Q4_0) {
-                        const int xs[16] = {af.x[0][0].x, af.x[0][0].y, af.x[0][0].z, af.x[0][0].w, af.x[0][1].x, af.x[0][1].y, af.x[0][1].z, af.x[0][1].w,
-                                            af.x[0][2].x, af.x[0][2].y, af.x[0][2].z, af.x[0][2].w, af.x[0][3].x, af.x[0][3].y, af.x[0][3].z, af.x[0][3].w};
+                // this lane's activations of the slab (the same for every row) and the -8 * sum q per dword: read once where the
+                // rows are one slab long (every step uses the same ones), per slab otherwise
+                if (NITK > 1 || step == 0) {
+                    if (p < npair) {
+                        load_act_frag<WT, 1>(af, act, npair, p);
+                        if constexpr (WT == SPY_HIP_Q4_0) {
+                            const int xs[16] = {af.x[0][0].x, af.x[0][0].y, af.x[0][0].z, af.x[0][0].w, af.x[0][1].x, af.x[0][1].y, af.x[0][1].z, af.x[0][1].w,
+                                                af.x[0][2].x, af.x[0][2].y, af.x[0][2].z, af.x[0][2].w, af.x[0][3].x, af.x[0][3].y, af.x[0][3].z, af.x[0][3].w};
 #pragma unroll
-                        for (int i = 0; i < 16; i++) n8[i] = -8 * __builtin_amdgcn_sdot4(xs[i], 0x01010101, 0, false);
+                            for (int i = 0; i < 16; i++) n8[i] = -8 * __builtin_amdgcn_sdot4(xs[i], 0x01010101, 0, false);
+                        }
                     }
                 }
+                if constexpr (WTV != WT) { if (vstep && p < npair) load_act_frag<WTV, 1>(av, act, npair, p); }
 #pragma unroll
                 for (int j = 0; j < rows; j++) {
                     const int r = r0 + j;
@@ -663,6 +666,8 @@ __global__ __launch_bounds__(XP_THREADS) void xattn_pv_kernel(const dev_state *s
         const int r16 = wave * 2 + (lane >> 5), cl = lane & 31;       // row of the 16 and accumulator 8 j + l
         const _Float16 *vr = (const _Float16 *)s_v + (size_t)r16 * VS + cl, *pr = (const _Float16 *)s_p + cl;
         float acc = 0.0f;
+        const int ntail = n_kv - 32 * nfull;                          // 1 .. 32
+        const float tprod = cl < ntail ? (float)vr[32 * nfull] * (float)pr[32 * nfull] : 0.0f;
         _Float16 va[8], pa[8], vb[8], pb[8];
         auto ld = [&](_Float16 (&v)[8], _Float16 (&q)[8], int i) {   // up to 16 chunks beyond nfull are read and not used: the next row, or the slack after the last
 #pragma unroll
@@ -694,11 +699,17 @@ __global__ __launch_bounds__(XP_THREADS) void xattn_pv_kernel(const dev_state *s
         acc += __shfl_xor(acc, 4, SPY_WAVE);          // t_l = sum[0][l] + sum[0][l + 4]
         acc += __shfl_xor(acc, 1, SPY_WAVE);          // t_0 + t_1, t_2 + t_3
         acc += __shfl_xor(acc, 2, SPY_WAVE);          // (t_0 + t_1) + (t_2 + t_3)
-        if (cl == 0) {                                // the scalar tail: elements 32 nfull .. n_kv - 1
-            float tail = 0.0f;
-            for (int e = 32 * nfull; e < n_kv; e++) tail = fmaf((float)vr[e], (float)pr[e], tail);
-            attn_out[hd_ * 128 + dgrp * 16 + r16] = tail + acc;
-        }
+        // the scalar tail: elements 32 nfull .. n_kv - 1, one after the other.  A product of two fp16 values is exact in fp32, so
+        // `tail = fma(v, p, tail)` is `tail + v * p` with the product formed beforehand: lane cl forms the product of element
+        // 32 nfull + cl (operands read before the walk above), the 32 products are fetched with wave permutes that do not depend
+        // on each other, and what remains serial is one addition per element.
+        float tp[32];
+#pragma unroll
+        for (int e = 0; e < 32; e++) tp[e] = __shfl(tprod, (lane & 32) + e, SPY_WAVE);
+        float tail = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 32; e++) if (e < ntail) tail = tail + tp[e];
+        if (cl == 0) attn_out[hd_ * 128 + dgrp * 16 + r16] = tail + acc;
         XSTAMP(dbg, 7);
     }
 }
