@@ -170,6 +170,12 @@ int spy_hip_block_dots(void *stream, int wtype, const void *w, const void *xq, i
  *      loop below uses for that part of a layer (same kernel, same grid), on the caller's buffers; order = 1: the host
  *      backend's summation order (results equal to the CPU backend's bit for bit), 0: this backend's own.  K (and F) must be
  *      multiples of 128 for order 1, rows at most 4096 elements wide for the norm prologue (16384 for the plain one). ------- */
+/* The running sum that NormRMS and Softmax of the host backend take over their terms: libstdc++'s std::reduce /
+ * std::transform_reduce for random-access ranges (non-linear.cpp:165-168, 205-208) adds groups of four,
+ * (t0 + t1) + (t2 + t3), to ONE running sum in order.  n non-negative floats (n % 4 == 0, n <= 8192, 16-byte aligned)
+ * -> *out, bit for bit; chunked = 0: one chain of additions, 1: the chunked form the gate|up kernel of order 1 uses
+ * (integer increments per 64-term chunk inside a binade, the chain only where the sum crosses a power of two). */
+int spy_hip_running_sum_f32(void *stream, const float *terms, int64_t n, int32_t chunked, float *out);
 /* RMSNorm * weight -> Q8_0: OperatorNormRMSImpl::execute + the Mul node + Quantizator<FP32,Q8_0>::transform
  * (non-linear.cpp:194-223, basic.cpp:15-50, vec_convert.h:178-261) as the fused kernels stage their activations;
  * normw == NULL: the quantization alone.  yq: K/32 native Q8_0 blocks. */

@@ -103,6 +103,7 @@ SIGNATURES = {
     "spy_hip_gemv_fused": (_i32, [_vp, _i32, _i32, _vp, _vp, _vp, _f32, _vp, _vp, _i64, _i64, _vp]),
     "spy_hip_ffn_gate_up_silu": (_i32, [_vp, _i32, _i32, _vp, _vp, _vp, _vp, _f32, _vp, _i64, _i64, _vp]),
     "spy_hip_measure_mfma_i8": (_i32, [_vp, _i32, C.POINTER(_f32)]),
+    "spy_hip_running_sum_f32": (_i32, [_vp, _vp, _i64, _i32, _vp]),
     "spy_hip_measure_mfma_i8_scaled": (_i32, [_vp, _i32, _i32, C.POINTER(_f32)]),
     "spy_hip_measure_hbm_read": (_i32, [_vp, _vp, _sz, _i32, C.POINTER(_f32)]),
     "spy_hip_llama_create": (_i32, [C.POINTER(LlamaDesc), C.POINTER(_vp)]),

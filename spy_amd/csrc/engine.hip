@@ -697,14 +697,14 @@ __global__ __launch_bounds__(1024) void stage_dump_kernel(const float *__restric
     int8_t *s_q = (int8_t *)smem;
     int2 *s_meta = (int2 *)(smem + staged_q_bytes(K));
     float *s_grp = (float *)(smem + ((staged_bytes(K) + 15) & ~(size_t)15));
-    if constexpr (ORDER == 1) xg_stage<NITK, NORM>(xv, wv, K, eps, s_q, s_meta, s_grp, &s_sum, []() {});
+    if constexpr (ORDER == 1) xg_stage<NITK, NORM, true>(xv, wv, K, eps, s_q, s_meta, s_grp, &s_sum, []() {});     // the chunked sum where it applies (K <= 8192): what gate|up runs
     else wgv_stage<NITK, NORM>(xv, wv, K, eps, s_q, s_meta, s_red);
     xg_dump_q8(s_q, s_meta, K, out);
 }
 
 template <int ORDER, bool NORM>
 int stage_dump(hipStream_t st, const float *x, const float *normw, float eps, int64_t K, void *yq) {
-    const size_t lds = ((staged_bytes(K) + 15) & ~(size_t)15) + (size_t)K + 256;    // + K / 4 group sums (+ what the serial sum reads ahead)
+    const size_t lds = ((staged_bytes(K) + 15) & ~(size_t)15) + (size_t)K + 1280;   // + K / 4 group sums, what the serial sum reads ahead, the records of the chunked sum
     switch ((K + 4095) / 4096) {
     case 1: stage_dump_kernel<ORDER, 1, NORM><<<dim3(1), dim3(1024), lds, st>>>(x, normw, eps, (int)K, (uint8_t *)yq); break;
     case 2: stage_dump_kernel<ORDER, 2, NORM><<<dim3(1), dim3(1024), lds, st>>>(x, normw, eps, (int)K, (uint8_t *)yq); break;
@@ -748,6 +748,38 @@ struct family_ctx {
 };
 
 }   // namespace
+
+// libstdc++'s 4-way running sum of n non-negative terms (n % 4 == 0, n <= 8192): groups (t0 + t1) + (t2 + t3) added to one
+// running sum, by one chain of additions (chunked == 0) or through xg_exact_sum (chunked == 1)
+template <int NG>
+__global__ __launch_bounds__(1024) void running_sum_kernel(const float *__restrict__ terms, int n, int chunked, float *__restrict__ out) {
+    __shared__ __attribute__((aligned(16))) float s_g[2048 + 64];
+    __shared__ xg_psum_lds s_l;
+    const int tid = threadIdx.x, ng = n / 4;
+    float grp[NG];
+#pragma unroll
+    for (int j = 0; j < NG; j++) {
+        const int i = tid + j * 1024;
+        grp[j] = 0.0f;
+        if (i < ng) {
+            const float4 v = ((const float4 *)terms)[i];
+            const float v1 = v.x + v.y, v2 = v.z + v.w;
+            grp[j] = v1 + v2;
+            s_g[i] = grp[j];
+        }
+    }
+    float tot;
+    if (chunked) tot = xg_exact_sum<NG>(grp, ng, s_g, &s_l, 0.0f, []() {});
+    else { __syncthreads(); tot = tid < 64 ? xg_serial_sum(s_g, ng, 0.0f) : 0.0f; }
+    if (tid == 0) *out = tot;
+}
+
+extern "C" int spy_hip_running_sum_f32(void *stream, const float *terms, int64_t n, int32_t chunked, float *out) {
+    SPY_CHECK_ARG(terms && out && n > 0 && n % 4 == 0 && n <= 8192 && (chunked == 0 || chunked == 1) && (((uintptr_t)terms) & 15) == 0);
+    if (n <= 4096) running_sum_kernel<1><<<dim3(1), dim3(1024), 0, (hipStream_t)stream>>>(terms, (int)n, chunked, out);
+    else running_sum_kernel<2><<<dim3(1), dim3(1024), 0, (hipStream_t)stream>>>(terms, (int)n, chunked, out);
+    return SPY_LAUNCH_RC();
+}
 
 extern "C" int spy_hip_rmsnorm_q8_0(void *stream, int32_t order, const float *x, const float *normw, float eps, int64_t K, void *yq) {
     SPY_CHECK_ARG(x && yq && K > 0 && K % 64 == 0 && (order == 0 || order == 1));

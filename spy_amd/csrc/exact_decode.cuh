@@ -23,6 +23,9 @@
 #define XG_THREADS 1024
 #define XG_WAVES 16
 #define XG_NBS 128                         // blocks per K slab (= 64 lanes x one block pair)
+#ifndef XG_PSUM
+#define XG_PSUM 1                          // gate|up: the running sum of the norm through xg_exact_sum (0: one chain, as in the other kernels)
+#endif
 #ifndef XG_DEPTH
 #define XG_DEPTH 3                         // rows per wave requested ahead of their use
 #endif
@@ -88,34 +91,155 @@ static __device__ __forceinline__ float xg_serial_sum(const float *s, int n, flo
     return init;
 }
 
+// ---- the same running sum, for NON-NEGATIVE terms, mostly in parallel and still bit for bit -----------------------------
+// While the running sum s stays inside one binade [2^e, 2^(e+1)) it is an integer multiple S of ulp = 2^(e-23), and adding a term
+// g >= 0 with round-to-nearest-even is integer arithmetic: with f = g / ulp (exact: a power-of-two scaling),
+//     RNE(S + f) = S + floor(f) + r,   r = 1 if frac(f) > 1/2, 0 if < 1/2, and for frac(f) = 1/2 the parity of S + floor(f).
+// So a term is a map from the parity of the incoming S to an increment, (inc_even, inc_odd), maps compose associatively
+// (C[p] = A[p] + B[(p + A[p]) & 1]), and 64 consecutive terms reduce to one pair in four DPP steps and three scalar ones.  The
+// sum is non-decreasing, so if the chunk's first and last value lie in binade e, every value between does.  Wave c reduces
+// chunk c (terms 64 c .. 64 c + 63) against the binade that an approximate prefix sum predicts; then one wave walks the chunks:
+// where the exact running sum has the predicted exponent and bits(s) + increment keeps it (the integer addition on the float's
+// bits IS s + increment * ulp), the chunk is one addition; otherwise (the sum crosses a power of two inside the chunk, the first
+// chunk, a wrong prediction) the chunk's 64 terms are added one by one as above.  Nothing is approximated in what is kept: the
+// prediction only selects which chunks take the short way.
+struct xg_psum_lds { float cs[32]; int t0[32], t1[32], eb[32]; };
+// g[j]: term 1024 j + tid of the n <= 1024 NG terms (0 beyond n), all of them also at s_g in LDS (written before the call,
+// 16-byte aligned, readable 40 floats beyond n).  Every thread of the 1024 calls; the sum is returned by wave 0 only (wave-uniform).
+// `others` runs in the other waves once their part is done, i.e. while wave 0 walks.
+template <int NG, class Others>
+static __device__ __forceinline__ float xg_exact_sum(const float (&g)[NG], int n, const float *s_g, xg_psum_lds *L, float init, Others others, long long *dbg = nullptr) {
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int nchunk = (n + 63) >> 6;
+    // sum over the wave through DPP only (no LDS permutes), read from lane 63; the order of these additions does not matter:
+    // they only predict binades
+    auto total = [](float v) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wave_total_lane63(v)), 63)); };
+#pragma unroll
+    for (int j = 0; j < NG; j++) {
+        const float cs = total(g[j]);
+        if (lane == 0) L->cs[wave + 16 * j] = cs;
+    }
+    XSTAMP(dbg, 8);
+    __syncthreads();                                     // chunk sums and (by the caller) the terms are in LDS
+    XSTAMP(dbg, 9);
+#pragma unroll
+    for (int j = 0; j < NG; j++) {
+        const int c = wave + 16 * j;
+        if (c < nchunk) {
+            const float before = total(lane < c ? L->cs[lane & 31] : 0.0f) + init, after = before + L->cs[c];
+            const int eb = (__float_as_int(before) >> 23) & 0xFF;
+            const float f = ldexpf(g[j], 150 - eb);      // g / ulp
+            const bool fits = f < 16777216.0f;           // false for a NaN too
+            const int fl = fits ? (int)f : 0;
+            const float frac = f - (float)fl;
+            const int up = frac > 0.5f ? 1 : 0, tie = frac == 0.5f ? 1 : 0;
+            int a0 = fl + (up | (tie & fl & 1)), a1 = fl + (up | (tie & ~fl & 1));    // incoming S even / odd: a tie rounds to the even neighbour
+            // within each row of 16 lanes: lane l takes over the terms of lane l + d (row_shl), earlier terms first; lanes
+            // that reach beyond their row compute values nobody uses
+#define XG_PS_STEP(CTRL) { const int b0 = __builtin_amdgcn_update_dpp(0, a0, CTRL, 0xF, 0xF, true), b1 = __builtin_amdgcn_update_dpp(0, a1, CTRL, 0xF, 0xF, true); \
+                           a0 = a0 + ((a0 & 1) ? b1 : b0); a1 = a1 + ((a1 & 1) ? b0 : b1); }   /* incoming odd: the parity after the first part is (1 + a1) & 1 */
+            XG_PS_STEP(0x101) XG_PS_STEP(0x102) XG_PS_STEP(0x104) XG_PS_STEP(0x108)
+#undef XG_PS_STEP
+            // the four rows in order, as scalars
+            int t0 = __builtin_amdgcn_readlane(a0, 0), t1 = __builtin_amdgcn_readlane(a1, 0);
+#pragma unroll
+            for (int r = 1; r < 4; r++) {
+                const int b0 = __builtin_amdgcn_readlane(a0, 16 * r), b1 = __builtin_amdgcn_readlane(a1, 16 * r);
+                t0 = t0 + ((t0 & 1) ? b1 : b0);
+                t1 = t1 + ((t1 & 1) ? b0 : b1);
+            }
+            const bool ok = __all(fits) && c > 0 && eb >= 1 && eb < 254 && ((__float_as_int(after) >> 23) & 0xFF) == eb;
+            if (lane == 0) { L->t0[c] = t0; L->t1[c] = t1; L->eb[c] = ok ? eb : -1; }
+        }
+    }
+    XSTAMP(dbg, 10);
+    __syncthreads();
+    XSTAMP(dbg, 11);
+    float s = init;
+    if (wave == 0) {
+        const int vt0 = L->t0[lane & 31], vt1 = L->t1[lane & 31], veb = L->eb[lane & 31];
+        // the terms of the chunks predicted to need the long way are requested ahead: the first such chunk now, the next one
+        // when the current one is taken up (a chunk that fails without having been predicted pays the LDS latency)
+        const unsigned long long slowmask = __ballot(lane < nchunk && veb < 0);
+        auto next_slow = [&](int from) -> int { const unsigned long long m = from < 64 ? (slowmask >> from) << from : 0ull; return m ? __builtin_ctzll(m) : -1; };
+        // (its first 32 terms; the other 32 are requested when the chunk is taken up and arrive behind the first 32 additions)
+        float4 v[8], w[8];
+        auto request = [&](int c) {
+#pragma unroll
+            for (int u = 0; u < 8; u++) v[u] = *(const float4 *)(s_g + 64 * c + 4 * u);
+        };
+        int pre = next_slow(0);
+        if (pre >= 0) request(pre);
+        int bits = __builtin_amdgcn_readfirstlane(__float_as_int(s));             // the running sum as a scalar
+        int nfall = 0;
+        for (int c = 0; c < nchunk; c++) {
+            const int eb = __builtin_amdgcn_readlane(veb, c), t = (bits & 1) ? __builtin_amdgcn_readlane(vt1, c) : __builtin_amdgcn_readlane(vt0, c);
+            const int nb = bits + t;
+            if (eb == (bits >> 23) && (nb >> 23) == eb && t >= 0) { bits = nb; continue; }
+            s = __int_as_float(bits);
+            nfall++;
+            if (n - 64 * c >= 64) {                      // a whole chunk one by one
+                if (c != pre) request(c);
+#pragma unroll
+                for (int u = 0; u < 8; u++) w[u] = *(const float4 *)(s_g + 64 * c + 32 + 4 * u);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int u = 0; u < 8; u++) { s = s + v[u].x; s = s + v[u].y; s = s + v[u].z; s = s + v[u].w; }
+                __builtin_amdgcn_sched_barrier(0);
+                if (c == pre) { pre = next_slow(c + 1); if (pre >= 0) request(pre); }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int u = 0; u < 8; u++) { s = s + w[u].x; s = s + w[u].y; s = s + w[u].z; s = s + w[u].w; }
+            } else s = xg_serial_sum(s_g + 64 * c, n - 64 * c, s);
+            bits = __builtin_amdgcn_readfirstlane(__float_as_int(s));
+        }
+        s = __int_as_float(bits);
+        XSTAMP(dbg, 12);
+#ifdef XDBG_STAMPS
+        if (dbg && blockIdx.x == 0 && threadIdx.x == 0) dbg[13] = nfall;
+#endif
+    } else others();
+    return s;
+}
+
 // ---- activations: f32 vector -> (RMSNorm * weight ->) Q8_0 in LDS, sums in the host order --------------------------
 // NormRMS (non-linear.cpp:194-223): sum = std::transform_reduce(x, x) = groups of four ((x0^2 + x1^2) + (x2^2 + x3^2))
 // added to one running sum in order; scale = 1 / sqrt(sum / n + eps); y = x * scale; then the Mul node: y * w.
 // The 1024 threads form the group sums (one float4 each per 4096 elements), lane 0 of wave 0 adds them.
-template <int NITK, bool NORM, class Issue>
+template <int NITK, bool NORM, bool PSUM = false, class Issue>
 static __device__ __forceinline__ void xg_stage(const float4 (&xv)[NITK], const float4 (&wv)[NORM ? NITK : 1], int K, float eps,
                                                 int8_t *s_q, int2 *s_meta, float *s_grp, float *s_sum, Issue issue_rows) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     float scale = 1.0f;
     if constexpr (NORM) {
+        float grp[NITK];
 #pragma unroll
         for (int j = 0; j < NITK; j++) {
             const int i = tid + j * XG_THREADS;
+            grp[j] = 0.0f;
             if (i < K / 4) {
                 const float4 v = xv[j];
                 const float a0 = v.x * v.x, a1 = v.y * v.y, a2 = v.z * v.z, a3 = v.w * v.w;
                 const float v1 = a0 + a1, v2 = a2 + a3;
-                s_grp[i] = v1 + v2;
+                grp[j] = v1 + v2;
+                s_grp[i] = grp[j];
             }
         }
-        __syncthreads();
-        // The weight rows are requested only now: a wave that asks for several rows sits in the issue stage until the memory queue
-        // has room, and a request made earlier would hold up the barrier above for every wave.  Wave 0 walks the sum first.
-        if (wave == 0) {
-            const float init = xg_serial_sum(s_grp, K / 4, 0.0f);
-            if (lane == 0) *s_sum = init;
+        // The weight rows are requested only after the group sums (and the scan of the sum): a wave that asks for several rows sits
+        // in the issue stage until the memory queue has room, and a request made earlier would hold up the barriers for every wave.
+        // Wave 0 walks the sum first.
+        if constexpr (NITK <= 2 && PSUM) {
+            xg_psum_lds *L = (xg_psum_lds *)(s_grp + ((K / 4 + 3) & ~3) + 64);
+            const float tot = xg_exact_sum<NITK>(grp, K / 4, s_grp, L, 0.0f, issue_rows);
+            if (wave == 0) { if (lane == 0) *s_sum = tot; issue_rows(); }
+        } else {
+            __syncthreads();
+            if (wave == 0) {
+                const float init = xg_serial_sum(s_grp, K / 4, 0.0f);
+                if (lane == 0) *s_sum = init;
+            }
+            issue_rows();
         }
-        issue_rows();
         __syncthreads();
         const float mean = *s_sum / (float)K;
         scale = 1.0f / sqrtf(mean + eps);
@@ -340,7 +464,12 @@ __global__ __launch_bounds__(XG_THREADS) void xgemv_kernel(xg_args a) {
     }
     // rows requested ahead of their use: all of the wave's rows where their registers allow (Q4_0 rows, up to 6), so
     // that the weights stream in while the serial sum of the norm is walked; XG_DEPTH otherwise
-    constexpr int DEPTH = (NROW <= 6 && wt_traits<WT>::PAIR_DW * NITK <= 9) ? NROW : XG_DEPTH;
+    // The sum of the norm in chunks (xg_exact_sum) pays where the wait that follows it is short: gate|up with three rows requested
+    // ahead (17.1 against 18.5 us; with all six requested the waves sit in the issue stage for longer than the serial walk takes, and
+    // the chunked sum gains nothing: 19.6).  It lost in the other kernels with a norm (qkv 13.2 against 12.7 at any depth, head 22.0
+    // against 20.6).
+    constexpr bool PSUM = XG_PSUM && EPI == EPI_GATEUP;
+    constexpr int DEPTH = (!PSUM && NROW <= 6 && wt_traits<WT>::PAIR_DW * NITK <= 9) ? NROW : (XG_DEPTH < NROW ? XG_DEPTH : NROW);
     constexpr int RING = NROW < DEPTH + 1 ? NROW : DEPTH + 1;
     wtile<WT, NITK> t[RING];
     wtile<WTV, NITK> tv;
@@ -359,7 +488,7 @@ __global__ __launch_bounds__(XG_THREADS) void xgemv_kernel(xg_args a) {
     int2 *s_meta = (int2 *)(smem + staged_q_bytes(K));
     float *s_part = (float *)(smem + ((staged_bytes(K) + 15) & ~(size_t)15));      // row slots; the group sums of the norm use the same bytes before
     XSTAMP(a.dbg, 16);
-    xg_stage<NITK, NORM>(xv, wv, K, a.eps, s_q, s_meta, s_part, &s_sum, issue_first);
+    xg_stage<NITK, NORM, PSUM>(xv, wv, K, a.eps, s_q, s_meta, s_part, &s_sum, issue_first);
     XSTAMP(a.dbg, 17);
     if (a.q8_dump && blockIdx.x == 0) xg_dump_q8(s_q, s_meta, K, a.q8_dump);
     staged_act act; act.q = s_q; act.meta = s_meta;
@@ -563,6 +692,9 @@ __global__ __launch_bounds__(XS_THREADS) void xattn_scores_kernel(const dev_stat
 // last 1..32 elements, by the lane of accumulator 0).
 #define XP_THREADS 1024
 #define XP_NP 10                           // 16-byte pieces per lane of a V^T row: n_ctx <= 5120
+#ifndef XP_PSUM
+#define XP_PSUM 0                          // the softmax sum through xg_exact_sum: 4.1 instead of 4.9 us for the sum, but the V^T rows are then requested later and the kernel takes 15.2 instead of 14.0 us
+#endif
 #define XP_NS 5                            // scores per thread: n_ctx <= 5120
 static inline int xattn_pv_vstride(int n_ctx) { return ((n_ctx + 63) / 64) * 64 + 32; }        // halfs between rows in LDS: = 64 bytes mod 128, the two rows of a wave on different banks
 static inline size_t xattn_pv_lds(int n_ctx) {
@@ -610,12 +742,20 @@ __global__ __launch_bounds__(XP_THREADS) void xattn_pv_kernel(const dev_state *s
     __syncthreads();
     XSTAMP(dbg, 2);
     const int ngrp = n_kv / 4;
-    for (int g = tid; g < ngrp; g += XP_THREADS) {
-        const float4 v = *(const float4 *)(s_e + 4 * g);
-        const float v1 = v.x + v.y, v2 = v.z + v.w;
-        s_grp[g] = v1 + v2;
+    float grp[2];
+    static_assert(XP_NS * XP_THREADS / 4 <= 2 * XP_THREADS, "two group sums per thread");
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+        const int g = tid + u * XP_THREADS;
+        grp[u] = 0.0f;
+        if (g < ngrp) {
+            const float4 v = *(const float4 *)(s_e + 4 * g);
+            const float v1 = v.x + v.y, v2 = v.z + v.w;
+            grp[u] = v1 + v2;
+            s_grp[g] = grp[u];
+        }
     }
-    __syncthreads();
+    if (!XP_PSUM) __syncthreads();
     XSTAMP(dbg, 3);
     // The V^T rows are requested now, by every wave but the one that walks the sum (a wave that asks for its whole row sits in the
     // issue stage until the memory queue has room, i.e. for most of the row's transfer time): the rows arrive while the sum is walked.
@@ -630,7 +770,15 @@ __global__ __launch_bounds__(XP_THREADS) void xattn_pv_kernel(const dev_state *s
         vb6 = *(const uint4 *)(vp + (size_t)min(6 * 64 + lane, last_piece) * 8); vb7 = *(const uint4 *)(vp + (size_t)min(7 * 64 + lane, last_piece) * 8);
         vb8 = *(const uint4 *)(vp + (size_t)min(8 * 64 + lane, last_piece) * 8); vb9 = *(const uint4 *)(vp + (size_t)min(9 * 64 + lane, last_piece) * 8);
     };
-    if (wave != 0) load_row();
+    if (XP_PSUM) {
+        xg_psum_lds *L = (xg_psum_lds *)(s_grp + ((n_ctx / 4 + 3) & ~3) + 64);
+        float init = xg_exact_sum<2>(grp, ngrp, s_grp, L, 0.0f, load_row, dbg);
+        if (wave == 0) {
+            for (int j = ngrp * 4; j < n_kv; j++) init = init + s_e[j];
+            if (lane == 0) s_sum = init;
+            load_row();
+        }
+    } else if (wave != 0) load_row();
     else {
         float init = xg_serial_sum(s_grp, ngrp, 0.0f);
         for (int j = ngrp * 4; j < n_kv; j++) init = init + s_e[j];

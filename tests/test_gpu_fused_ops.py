@@ -213,3 +213,64 @@ def test_attn_decode(hip, oracle, order, n_kv):
     want_t = (S[:, 0, :] * scale).astype(np.float32)
     _check(np.ascontiguousarray(got_s), np.ascontiguousarray(want_t), "scores * scale, n_kv %d" % n_kv, order)
     _check(do.download(np.float32), out.reshape(-1), "attention output, n_kv %d" % n_kv, order)
+
+
+def _running_sum_ref(t):
+    """libstdc++'s reduce for random-access ranges on floats: (t0 + t1) + (t2 + t3) per group of four, groups added to one
+    running sum in order (every operation rounded to fp32)."""
+    t = t.astype(np.float32)
+    g = ((t[0::4] + t[1::4]).astype(np.float32) + (t[2::4] + t[3::4]).astype(np.float32)).astype(np.float32)
+    s = np.float32(0.0)
+    for x in g:
+        s = np.float32(s + x)
+    return s
+
+
+def _running_sum_cases():
+    rng = np.random.default_rng(77)
+    cases = {}
+    for n in (4, 8, 252, 256, 260, 4096, 4100, 4352, 8192):
+        cases["squares of normals, n=%d" % n] = (rng.standard_normal(n) ** 2).astype(np.float32)
+    e = np.exp(-np.abs(rng.standard_normal(4352)) * 6).astype(np.float32); e[1234] = 1.0
+    cases["softmax-like exponentials"] = e
+    # ties: the running sum sits at 1 (ulp 2^-23) and every group adds exactly half an ulp; even and odd starting mantissa
+    t = np.zeros(4096, np.float32); t[0] = 1.0; t[4::4] = 2.0 ** -24
+    cases["half-ulp ties from an even sum"] = t
+    t = np.zeros(4096, np.float32); t[0] = 1.0; t[1] = 2.0 ** -23; t[4::4] = 2.0 ** -24
+    cases["half-ulp ties from an odd sum"] = t
+    t = np.zeros(4096, np.float32); t[0] = 1.0; t[4::8] = 2.0 ** -24; t[8::8] = 3 * 2.0 ** -24; t[2000] = 2.0 ** -23
+    cases["mixed half and one-and-a-half ulps"] = t
+    # sums that land exactly on powers of two, and growth by doubling (a crossing in almost every chunk)
+    cases["ones"] = np.ones(8192, np.float32)
+    cases["quarters"] = np.full(4096, 0.25, np.float32)
+    t = np.zeros(512, np.float32); t[0::4] = (2.0 ** (np.arange(128) / 2.0)).astype(np.float32)
+    cases["geometric growth"] = t
+    # a term far above the running sum, huge dynamic range, denormals, zeros
+    t = (rng.standard_normal(4096) ** 2).astype(np.float32) * 1e-20; t[1000] = 3e18; t[3000] = 7.5e30
+    cases["outliers 1e38 apart"] = t
+    t = np.zeros(4096, np.float32); t[5::7] = 1e-42; t[4000] = 1e-38
+    cases["denormals"] = t
+    cases["zeros"] = np.zeros(1024, np.float32)
+    t = (rng.standard_normal(8192) ** 2).astype(np.float32); t[::3] *= 2.0 ** -12; t = (t * 2.0 ** 12).round() / np.float32(2.0 ** 12)
+    cases["coarse grid (many exact ties)"] = t.astype(np.float32)
+    return cases
+
+
+@pytest.mark.parametrize("chunked", [0, 1])
+def test_running_sum_in_the_host_order_bit_for_bit(hip, chunked):
+    """spy_hip_running_sum_f32 against the definition, walked in numpy: the plain chain and the chunked form (integer increments
+    inside a binade, ties by the parity of the running mantissa, the chain where the sum crosses a power of two) must both give
+    the bits of the one-by-one sum.  The cases aim at what the chunked form could get wrong: exact ties from even and odd sums,
+    sums that land on powers of two, a crossing in every chunk, terms above the running sum, denormals."""
+    from tests.gpu_util import dev, dev_empty, call
+    L = hip.load()
+    bad = []
+    for name, t in _running_sum_cases().items():
+        want = _running_sum_ref(t)
+        dt, do = dev(t), dev_empty(4, 0xFF)
+        call(L.spy_hip_running_sum_f32, None, dt.ptr, t.size, chunked, do.ptr)
+        hip.sync()
+        got = do.download(np.float32)[0]
+        if got.view(np.uint32) != want.view(np.uint32):
+            bad.append("%s: got %r (0x%08x), want %r (0x%08x)" % (name, got, got.view(np.uint32), want, want.view(np.uint32)))
+    assert not bad, "\n".join(bad)

@@ -311,3 +311,26 @@ def test_prompt_attention_kernel_against_operator_sequence(hip, H_, T, past, n_c
         e = np.exp((t - t.max(axis=1, keepdims=True)).astype(np.float16).astype(np.float64))
         p = (e / e.sum(axis=1, keepdims=True)).astype(np.float16).astype(np.float64)
         assert rel_err(got[:, h * hd:(h + 1) * hd], p @ vf.T) < 1e-3
+
+
+def test_measured_ceilings_are_plausible(hip):
+    """The measurement entry points behind the denominators of the operator sweep: the bare int8 MFMA loop, the same loop with
+    the per-block scaling of the quantized GEMM in both epilogue forms, and the read scan.  Sanity bounds only: below the
+    published peaks, the scaled loops below the bare one, the biased-accumulator form not slower than the conversion form."""
+    import ctypes as C
+    L = hip.load()
+    bare, cvt, biased, gbps = C.c_float(), C.c_float(), C.c_float(), C.c_float()
+    assert L.spy_hip_measure_mfma_i8(None, 2000, C.byref(bare)) == 0
+    assert L.spy_hip_measure_mfma_i8_scaled(None, 2000, 0, C.byref(cvt)) == 0
+    assert L.spy_hip_measure_mfma_i8_scaled(None, 2000, 1, C.byref(biased)) == 0
+    assert L.spy_hip_measure_mfma_i8_scaled(None, 2000, 2, C.byref(biased)) == hip.EINVAL
+    buf = hip.DeviceBuffer(256 << 20)
+    buf.fill(1)
+    assert L.spy_hip_measure_hbm_read(None, buf.ptr, buf.nbytes, 3, C.byref(gbps)) == 0
+    buf.free()
+    print("int8 MFMA %.0f TOP/s, block-scaled inner loop %.0f (conversion) / %.0f (biased accumulator) TOP/s, read scan %.0f GB/s"
+          % (bare.value, cvt.value, biased.value, gbps.value), flush=True)
+    assert 1000 < bare.value < 5000
+    assert 300 < cvt.value < bare.value and 300 < biased.value < bare.value
+    assert biased.value > 0.95 * cvt.value
+    assert 1000 < gbps.value < 8000
