@@ -43,11 +43,12 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 // 32-bit word of 4 packed nibbles (already masked to 0..15 per byte) -> 4 int8 of (n - 8)
 static __device__ __forceinline__ uint32_t nib_m8(uint32_t lo) { return (lo + 0x78787878u) ^ 0x80808080u; }
 
-// Workgroups of the XCD-aware one-dimensional grid of gemm_q8act_kernel for gx x gy tiles: 8 XCDs x ceil(gx / 4) x ceil(gy / 2)
+// Workgroups of the XCD-aware one-dimensional grid of gemm_q8act_kernel for gx x gy tiles: 8 XCDs x ceil(gx / 4) x ceil(gy / 2), or
+// 8 x ceil(gx / 8) x gy for an odd gy
 // (the workgroups whose tile falls outside return at once).
-static inline int64_t gemm_xcd_grid(int64_t gx, int64_t gy) { return 8 * ((gx + 3) / 4) * ((gy + 1) / 2); }
+static inline int64_t gemm_xcd_grid(int64_t gx, int64_t gy) { const int64_t xt = (gy & 1) ? 1 : 2, xm = 8 / xt; return 8 * ((gx + xm - 1) / xm) * ((gy + xt - 1) / xt); }
 // 1 where an XCD's quarter of the gx weight tiles (128 rows of K / 32 blocks each) does not fit its L2 with room to spare
-static inline int gemm_t_inner(int64_t gx, int64_t K, int wtype) {
+static inline int gemm_t_inner(int64_t gx, int64_t K, int wtype) {      // (sized for the 4 x 2 arrangement)
     return ((gx + 3) / 4) * GEMM_TILE * (K / 32) * (wtype == SPY_HIP_Q4_0 ? 18 : 34) > (3ll << 20);
 }
 
@@ -57,8 +58,8 @@ __global__ __launch_bounds__(256, GEMM_WGS) void gemm_q8act_kernel(const uint8_t
     // Optionally two weight matrices of the same shape against the same activations in one grid (gate and up): the
     // workgroups of the second follow those of the first, which halves the share of the grid's tail.
     // Workgroup L of the one-dimensional grid runs on XCD L % 8, each with its own L2.  The eight XCDs form a 4 x 2
-    // arrangement over (weight tiles, activation tiles): XCD (mj, ti) takes the weight tiles = mj (mod 4) against the
-    // activation tiles = ti (mod 2), so that a weight tile is fetched by two L2s and an activation tile by four (a
+    // arrangement over (weight tiles, activation tiles) (8 x 1 for an odd number of activation tiles): XCD (mj, ti) takes the
+    // weight tiles = mj (mod 4) against the activation tiles = ti (mod 2), so that a weight tile is fetched by two L2s and an activation tile by four (a
     // row-major grid has every L2 fetch all the activations).  Where the XCD's share of the weight matrix is larger than
     // its 4 MB L2 (t_inner), the activation tiles of one weight tile follow each other: the hundred or so workgroups an
     // XCD runs at a time then share a dozen weight tiles and its activation tiles, where the other order streams all its
@@ -67,10 +68,12 @@ __global__ __launch_bounds__(256, GEMM_WGS) void gemm_q8act_kernel(const uint8_t
     const int tiles1 = (M + GEMM_TILE - 1) / GEMM_TILE, gx = W2 ? 2 * tiles1 : tiles1, gy = (T + GEMM_TILE - 1) / GEMM_TILE;
     int gbx, gby;
     {
-        const int xcd = (int)blockIdx.x & 7, slot = (int)blockIdx.x >> 3, nt = (gy + 1) >> 1, nm = (gx + 3) >> 2;
+        // an odd number of activation tiles (one, for up to 128 tokens) would leave half of the XCDs short of work: 8 x 1 then
+        const int xt = (gy & 1) ? 1 : 2, xm = 8 / xt;
+        const int xcd = (int)blockIdx.x & 7, slot = (int)blockIdx.x >> 3, nt = (gy + xt - 1) / xt, nm = (gx + xm - 1) / xm;
         const int sm = t_inner ? slot / nt : slot % nm, stt = t_inner ? slot % nt : slot / nm;
-        gbx = sm * 4 + (xcd & 3);
-        gby = stt * 2 + (xcd >> 2);
+        gbx = sm * xm + (xcd % xm);
+        gby = stt * xt + (xcd / xm);
         if (gbx >= gx || gby >= gy) return;
     }
     const bool second = W2 != nullptr && gbx >= tiles1;
@@ -144,9 +147,11 @@ __global__ __launch_bounds__(256, GEMM_WGS) void gemm_q8act_kernel(const uint8_t
     // The block dots are accumulated onto the integer 0x4B400000: as a float that is 12582912 + dot exactly (|dot| <= 32 * 127 * 127
     // < 2^22), and subtracting 12582912 gives float(dot) with a full-rate instruction where a conversion runs at half rate.
     const int k0mask = lane < 32 ? 0xFFFF : 0;
+    // (Q4_0 only: the Q8_0 kernel has no 16 registers to spare at three workgroups per CU -- it spilled and ran 15-30 % slower)
+    constexpr bool BIAS = WT == SPY_HIP_Q4_0;
     v16i bias;
 #pragma unroll
-    for (int r = 0; r < 16; r++) bias[r] = 0x4B400000;
+    for (int r = 0; r < 16; r++) bias[r] = BIAS ? 0x4B400000 : 0;
     auto multiply = [&](int b) {
 #pragma unroll 1
         for (int blk = 0; blk < 2; blk++) {
@@ -169,7 +174,7 @@ __global__ __launch_bounds__(256, GEMM_WGS) void gemm_q8act_kernel(const uint8_t
                     const v16i I = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], bias, 0, 0, 0);
                     const v16f S = __builtin_amdgcn_mfma_f32_32x32x8f16(ha[i], hb[j], zf, 0, 0, 0);
 #pragma unroll
-                    for (int r = 0; r < 16; r++) acc[i][j][r] = fmaf(S[r], __int_as_float(I[r]) - 12582912.0f, acc[i][j][r]);
+                    for (int r = 0; r < 16; r++) acc[i][j][r] = fmaf(S[r], BIAS ? __int_as_float(I[r]) - 12582912.0f : (float)I[r], acc[i][j][r]);
                 }
         }
     };
@@ -385,9 +390,14 @@ static int launch_gemm_skinny_ntw(hipStream_t st, const void *w, const void *xq,
 }
 template <int WT>
 static int launch_gemm_skinny(hipStream_t st, const void *w, const void *xq, float *dst, int64_t M, int64_t K, int64_t T, int64_t dst_stride) {
+    // Token sub-tiles per workgroup (the other waves split K): as many as still leave two workgroups per compute unit.  A wave
+    // advances one chunk of K per memory round trip, so with few workgroups (4096 rows x 128 tokens: 128) the launch is a chain
+    // of K / 256 round trips on half of the compute units; splitting K four ways instead gives 512 workgroups a quarter as long.
+    const int64_t rows = (M + 31) / 32, want = 512;
     if (T <= 32) return launch_gemm_skinny_ntw<WT, 1>(st, w, xq, dst, M, K, T, dst_stride);
-    if (T <= 64) return launch_gemm_skinny_ntw<WT, 2>(st, w, xq, dst, M, K, T, dst_stride);
-    return launch_gemm_skinny_ntw<WT, 4>(st, w, xq, dst, M, K, T, dst_stride);
+    if (T > 64 && rows * ((T + 127) / 128) >= want) return launch_gemm_skinny_ntw<WT, 4>(st, w, xq, dst, M, K, T, dst_stride);
+    if (T <= 64 || rows * ((T + 63) / 64) >= want) return launch_gemm_skinny_ntw<WT, 2>(st, w, xq, dst, M, K, T, dst_stride);
+    return launch_gemm_skinny_ntw<WT, 1>(st, w, xq, dst, M, K, T, dst_stride);
 }
 
 // ---- K-quant weights ---------------------------------------------------------------------------------
