@@ -227,7 +227,11 @@ static int enqueue_one(spy_hip_llama *m, hipStream_t st, int which, int il) {
     if (pass_order(m) == 1 || (m->dry && m->order == 1)) {      // the host backend's summation order: six launches per layer
         if (which == K_SCORES) {
             if (m->dry) return 0;
-            xattn_scores_kernel<0><<<dim3((unsigned)m->num_cu), dim3(XS_THREADS), xattn_scores_lds(c.n_head), st>>>(
+            // one workgroup per compute unit; SPY_HIP_SCORES_GRID (tests) forces fewer, so that a workgroup's share of the tokens
+            // takes several rounds of XS_TOK, as it would on a part with fewer compute units or a longer cache
+            int sgrid = m->num_cu;
+            if (const char *e = getenv("SPY_HIP_SCORES_GRID")) { const int v = atoi(e); if (v >= 1 && v <= m->num_cu) sgrid = v; }
+            xattn_scores_kernel<0><<<dim3((unsigned)sgrid), dim3(XS_THREADS), xattn_scores_lds(c.n_head), st>>>(
                 m->st, m->pos_imm, m->q16, m->k_cache[il], m->scores, c.n_head, c.n_ctx, 1.0f / sqrtf((float)m->hd));   // SoftmaxParam::scale (attention.cpp:113)
             return SPY_LAUNCH_RC();
         }

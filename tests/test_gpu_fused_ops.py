@@ -215,6 +215,34 @@ def test_attn_decode(hip, oracle, order, n_kv):
     _check(do.download(np.float32), out.reshape(-1), "attention output, n_kv %d" % n_kv, order)
 
 
+@pytest.mark.parametrize("grid,n_kv", [(64, 4351), (7, 300), (100, 1900)])
+def test_attn_scores_in_several_rounds(hip, grid, n_kv, monkeypatch):
+    """The score kernel of order 1 deals the cached tokens out over its workgroups and takes a workgroup's share in rounds of 18
+    tokens, the next round's keys requested while the current round is multiplied.  With one workgroup per compute unit of this
+    part a share never exceeds one round at the supported cache lengths; SPY_HIP_SCORES_GRID forces fewer workgroups, so that the
+    rounds (full ones, a short last one, workgroups without tokens) are exercised: same bits as the one-round launch."""
+    from tests.gpu_util import dev, dev_empty, call
+    H_, hd, n_ctx = 32, 128, 4352
+    d = H_ * hd
+    rng = np.random.default_rng(grid * 10000 + n_kv)
+    q16 = (rng.standard_normal(d) * 1.5).astype(np.float16)
+    kc = np.zeros((n_ctx, d), np.float16); kc[:n_kv] = rng.standard_normal((n_kv, d)).astype(np.float16)
+    vc = np.zeros((d, n_ctx), np.float16); vc[:, :n_kv] = rng.standard_normal((d, n_kv)).astype(np.float16)
+    dq, dk, dv = dev(q16.view(np.uint16)), dev(kc.view(np.uint16)), dev(vc.view(np.uint16))
+    res = []
+    for g in (None, grid):
+        if g is None:
+            monkeypatch.delenv("SPY_HIP_SCORES_GRID", raising=False)
+        else:
+            monkeypatch.setenv("SPY_HIP_SCORES_GRID", str(g))
+        ds, do = dev_empty(H_ * n_ctx * 4, 0xEE), dev_empty(d * 4, 0xEE)
+        call(hip.load().spy_hip_attn_decode, None, 1, dq.ptr, dk.ptr, dv.ptr, H_, n_kv, n_ctx, ds.ptr, do.ptr)
+        hip.sync()
+        res.append((ds.download(np.uint32).reshape(H_, n_ctx)[:, :n_kv].copy(), do.download(np.uint32).copy()))
+    assert np.array_equal(res[0][0], res[1][0]), "scores differ between one round and %d workgroups" % grid
+    assert np.array_equal(res[0][1], res[1][1])
+
+
 def _running_sum_ref(t):
     """libstdc++'s reduce for random-access ranges on floats: (t0 + t1) + (t2 + t3) per group of four, groups added to one
     running sum in order (every operation rounded to fp32)."""
