@@ -56,7 +56,7 @@ def _check_q8(got, want, what, order):
 
 
 @pytest.mark.parametrize("order", [1, 0])
-@pytest.mark.parametrize("K,norm", [(4096, True), (4096, False), (11008, False), (512, True), (1024, True)])
+@pytest.mark.parametrize("K,norm", [(4096, True), (4096, False), (11008, False), (512, True), (1024, True), (8192, True), (5120, True), (11008, True)])
 def test_rmsnorm_q8_0_prologue(hip, oracle, order, K, norm):
     from tests.gpu_util import dev, dev_empty, call
     rng = np.random.default_rng(K + norm)
