@@ -453,6 +453,148 @@ __global__ __launch_bounds__(256) void exact_dots8_kernel(xdesc w, const uint8_t
     if (l == 0) *(float *)xat(d, i01, i11, i02, i03) = acc;
 }
 
+// The same Q4_0 / Q8_0 dots for many activation rows at once (prompts): a workgroup computes a tile of 64 weight rows
+// by 64 activation rows, a thread 4 x 4 output elements with the eight accumulators of each in registers.  Every
+// accumulator still receives its block terms in block order, fma(d_w * d_x, float(integer sum of its four products),
+// acc), and the eight are added in hsum_float_8's tree at the end, so the results are those of exact_dots8_kernel bit
+// for bit; what changes is that a weight block and an activation block are unpacked once per tile (into LDS, as
+// words in element order: the low nibbles of a Q4_0 block first, then the high ones) instead of once per output.
+// The integer sums come from v_dot4_i32_i8 onto 0x4B400000, the bits of 1.5 * 2^23: read as a float, the sum minus
+// 12582912.0f is the exact conversion (|sum| < 2^22).  v_dot4 multiplies the signed bytes as they are, which equals
+// the host's abs / sign / saturating pair sum (vec_util.h:101-110) as long as no ACTIVATION byte is -128; the launcher
+// takes this kernel only for activations that this library quantized itself (|q| <= 127).
+#define XGB_TILE 64
+#define XGB_KB 4          // blocks per stage
+template <int WT>
+__global__ __launch_bounds__(256, 2) void exact_gemm8_kernel(const uint8_t *__restrict__ w, int64_t w_row, int64_t ne01, int64_t nb,
+                                                              const uint8_t *__restrict__ xm, int64_t x_row, int64_t ne11,
+                                                              float *__restrict__ dst, int64_t d_row) {
+    __shared__ __align__(16) uint32_t s_wq[2][XGB_KB][8][XGB_TILE];
+    __shared__ __align__(16) uint32_t s_xq[2][XGB_KB][8][XGB_TILE];
+    __shared__ __align__(16) float s_wd[2][XGB_KB][XGB_TILE];
+    __shared__ __align__(16) float s_xd[2][XGB_KB][XGB_TILE];
+    const int tid = threadIdx.x;
+    const int mg = tid & 15, tg = tid >> 4;
+    const int64_t m0 = (int64_t)blockIdx.x * XGB_TILE, t0 = (int64_t)blockIdx.y * XGB_TILE;
+
+    // loaders: waves 0 and 1 bring weight blocks, waves 2 and 3 activation blocks; a thread takes two neighbouring
+    // blocks of one row (36 bytes of Q4_0, 68 of Q8_0: whole aligned words) per stage
+    const bool ld_w = tid < 128;
+    const int ld_row = tid & 63, ld_pair = (tid >> 6) & 1;
+    constexpr int NWQ = WT == SPY_HIP_Q4_0 ? 9 : 17;
+    const uint32_t *ld_src;
+    if (ld_w) ld_src = (const uint32_t *)(w + min(m0 + ld_row, ne01 - 1) * w_row) + ld_pair * NWQ;
+    else ld_src = (const uint32_t *)(xm + min(t0 + ld_row, ne11 - 1) * x_row) + ld_pair * 17;
+    uint32_t g[17];
+    auto fetch = [&](int64_t stage) {
+        const uint32_t *p = ld_src + stage * (ld_w ? 2 * NWQ : 34);
+        if (ld_w && WT == SPY_HIP_Q4_0) {
+#pragma unroll
+            for (int i = 0; i < 9; i++) g[i] = p[i];
+        } else {
+#pragma unroll
+            for (int i = 0; i < 17; i++) g[i] = p[i];
+        }
+    };
+    auto put = [&](int buf) {
+        if (ld_w && WT == SPY_HIP_Q4_0) {
+            // block 0: scale in the low half of g[0], 16 quant bytes from byte 2; block 1: scale in the high half of g[4], quants g[5..8]
+            const int k0 = 2 * ld_pair;
+            s_wd[buf][k0][ld_row] = h2f_tab((uint16_t)(g[0] & 0xFFFFu));
+            s_wd[buf][k0 + 1][ld_row] = h2f_tab((uint16_t)(g[4] >> 16));
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const uint32_t q0 = __builtin_amdgcn_alignbit(g[k + 1], g[k], 16), q1 = g[5 + k];
+                uint32_t lo0 = q0 & 0x0F0F0F0Fu, hi0 = (q0 >> 4) & 0x0F0F0F0Fu, lo1 = q1 & 0x0F0F0F0Fu, hi1 = (q1 >> 4) & 0x0F0F0F0Fu;
+                // per byte n - 8: n + 128 - 8 never borrows across bytes, then the top bit is flipped back
+                lo0 = ((lo0 | 0x80808080u) - 0x08080808u) ^ 0x80808080u; hi0 = ((hi0 | 0x80808080u) - 0x08080808u) ^ 0x80808080u;
+                lo1 = ((lo1 | 0x80808080u) - 0x08080808u) ^ 0x80808080u; hi1 = ((hi1 | 0x80808080u) - 0x08080808u) ^ 0x80808080u;
+                s_wq[buf][k0][k][ld_row] = lo0; s_wq[buf][k0][4 + k][ld_row] = hi0;
+                s_wq[buf][k0 + 1][k][ld_row] = lo1; s_wq[buf][k0 + 1][4 + k][ld_row] = hi1;
+            }
+        } else {
+            // Q8_0 pair: block 0 = scale in the low half of g[0] and 32 quant bytes from byte 2, block 1 = scale in the high half
+            // of g[8] and quants g[9..16]
+            uint32_t (*sq)[8][XGB_TILE] = ld_w ? s_wq[buf] : s_xq[buf];
+            float (*sd)[XGB_TILE] = ld_w ? s_wd[buf] : s_xd[buf];
+            const int k0 = 2 * ld_pair;
+            sd[k0][ld_row] = h2f_tab((uint16_t)(g[0] & 0xFFFFu));
+            sd[k0 + 1][ld_row] = h2f_tab((uint16_t)(g[8] >> 16));
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                sq[k0][k][ld_row] = __builtin_amdgcn_alignbit(g[k + 1], g[k], 16);
+                sq[k0 + 1][k][ld_row] = g[9 + k];
+            }
+        }
+    };
+
+    float acc[4][4][8];
+#pragma unroll
+    for (int r = 0; r < 4; r++)
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+#pragma unroll
+            for (int a = 0; a < 8; a++) acc[r][c][a] = 0.0f;
+
+    const int64_t nstage = nb / XGB_KB;
+    fetch(0);
+    put(0);
+    __syncthreads();
+    for (int64_t s = 0; s < nstage; s++) {
+        const int buf = (int)(s & 1);
+        if (s + 1 < nstage) fetch(s + 1);
+#pragma unroll 1
+        for (int kb = 0; kb < XGB_KB; kb++) {
+            const float4 wd4 = *(const float4 *)&s_wd[buf][kb][4 * mg], xd4 = *(const float4 *)&s_xd[buf][kb][4 * tg];
+            const float wd[4] = {wd4.x, wd4.y, wd4.z, wd4.w}, xd[4] = {xd4.x, xd4.y, xd4.z, xd4.w};
+            float D[4][4];
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+#pragma unroll
+                for (int c = 0; c < 4; c++) D[r][c] = wd[r] * xd[c];
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const uint4 wq4 = *(const uint4 *)&s_wq[buf][kb][e][4 * mg], xq4 = *(const uint4 *)&s_xq[buf][kb][e][4 * tg];
+                const uint32_t wq[4] = {wq4.x, wq4.y, wq4.z, wq4.w}, xq[4] = {xq4.x, xq4.y, xq4.z, xq4.w};
+                // accumulator of element word e: Q4_0 keeps the low nibbles (elements 0..15) in 4..7 and the high ones in 0..3
+                // (vec_dot.h:42-86), Q8_0 elements 4l..4l+3 in accumulator l (vec_dot.h:88-115)
+                const int a = WT == SPY_HIP_Q4_0 ? ((e + 4) & 7) : e;
+                // The sixteen integer sums of this word in one assembly block: the three-operand form takes the constant from a
+                // scalar register (the builtin first copies it into every destination).  The compiler cannot see that these
+                // are dot instructions, whose results other vector instructions may only read a few cycles later, so the
+                // block ends with the wait itself.
+                int32_t p[16];
+#define XGB_DOT(r, c) "v_dot4_i32_i8 %[p" #r #c "], %[w" #r "], %[x" #c "], %[b]\n"
+                asm(XGB_DOT(0, 0) XGB_DOT(0, 1) XGB_DOT(0, 2) XGB_DOT(0, 3) XGB_DOT(1, 0) XGB_DOT(1, 1) XGB_DOT(1, 2) XGB_DOT(1, 3)
+                    XGB_DOT(2, 0) XGB_DOT(2, 1) XGB_DOT(2, 2) XGB_DOT(2, 3) XGB_DOT(3, 0) XGB_DOT(3, 1) XGB_DOT(3, 2) XGB_DOT(3, 3)
+                    "s_nop 4"
+                    : [p00] "=&v"(p[0]), [p01] "=&v"(p[1]), [p02] "=&v"(p[2]), [p03] "=&v"(p[3]), [p10] "=&v"(p[4]), [p11] "=&v"(p[5]),
+                      [p12] "=&v"(p[6]), [p13] "=&v"(p[7]), [p20] "=&v"(p[8]), [p21] "=&v"(p[9]), [p22] "=&v"(p[10]), [p23] "=&v"(p[11]),
+                      [p30] "=&v"(p[12]), [p31] "=&v"(p[13]), [p32] "=&v"(p[14]), [p33] "=&v"(p[15])
+                    : [w0] "v"(wq[0]), [w1] "v"(wq[1]), [w2] "v"(wq[2]), [w3] "v"(wq[3]), [x0] "v"(xq[0]), [x1] "v"(xq[1]), [x2] "v"(xq[2]),
+                      [x3] "v"(xq[3]), [b] "s"(0x4B400000));
+#undef XGB_DOT
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+#pragma unroll
+                    for (int c = 0; c < 4; c++)
+                        acc[r][c][a] = fmaf(D[r][c], __int_as_float(p[4 * r + c]) - 12582912.0f, acc[r][c][a]);
+            }
+        }
+        if (s + 1 < nstage) put(buf ^ 1);
+        __syncthreads();
+    }
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+        const int64_t tok = t0 + 4 * tg + c;
+        float o[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) o[r] = hsum8(acc[r][c]);
+        const int64_t row = m0 + 4 * mg;
+        if (tok < ne11 && row < ne01) *(float4 *)(dst + tok * d_row + row) = make_float4(o[0], o[1], o[2], o[3]);
+    }
+}
+
 // K-quant rows with the eight sub-blocks (Q4_K) or Q8_0 blocks (Q6_K) of a super-block in eight lanes: lane j forms
 // the integer sums and the fp32 term of its part, then every lane walks the ONE accumulator of the project's order
 // through the eight terms in turn (terms broadcast from their lanes), so all eight lanes hold the same sum.
@@ -641,9 +783,28 @@ int spy_exact_rope(hipStream_t st, const spy_hip_tensor *x, const spy_hip_tensor
     return (int)hipStreamSynchronize(st);      // the table is overwritten by the next call
 }
 
-int spy_exact_dots(hipStream_t st, int t0, const spy_hip_tensor *w, const uint8_t *xm, int64_t x_row, int64_t ne11, const spy_hip_tensor *dst) {
+// x_own_quants: the Q8_0 activations were quantized by this library (no byte is -128)
+int spy_exact_dots(hipStream_t st, int t0, const spy_hip_tensor *w, const uint8_t *xm, int64_t x_row, int64_t ne11, const spy_hip_tensor *dst, int x_own_quants) {
     const int64_t total = w->ne[1] * ne11 * w->ne[2] * w->ne[3];
     if (total <= 0 || (total + 7) / 8 >= (1ll << 31)) return SPY_HIP_EINVAL;
+    // many activation rows of a plain matrix: the tiled kernel (SPY_HIP_EXACT_TILED=0 keeps the row kernels, for the tests
+    // that compare the two)
+    if ((t0 == SPY_HIP_Q4_0 || t0 == SPY_HIP_Q8_0) && x_own_quants && ne11 >= 16 && w->ne[2] == 1 && w->ne[3] == 1) {
+        const char *env_tiled = getenv("SPY_HIP_EXACT_TILED");
+        const bool tiled = !(env_tiled && *env_tiled == '0');
+        const int64_t nb = w->ne[0] / 32, ne01 = w->ne[1];
+        const bool fits = nb > 0 && nb % XGB_KB == 0 && ne01 % 4 == 0 && w->nb[1] % 4 == 0 && x_row % 4 == 0 && ((uintptr_t)w->data & 3) == 0 &&
+                          ((uintptr_t)xm & 3) == 0 && dst->nb[0] == 4 && dst->nb[1] % 16 == 0 && ((uintptr_t)dst->data & 15) == 0 &&
+                          (ne11 + XGB_TILE - 1) / XGB_TILE <= 65535 && !getenv("SPY_HIP_EXACT_SERIAL");
+        if (tiled && fits) {
+            const dim3 grid((unsigned)((ne01 + XGB_TILE - 1) / XGB_TILE), (unsigned)((ne11 + XGB_TILE - 1) / XGB_TILE));
+            if (t0 == SPY_HIP_Q4_0)
+                exact_gemm8_kernel<SPY_HIP_Q4_0><<<grid, dim3(256), 0, st>>>((const uint8_t *)w->data, w->nb[1], ne01, nb, xm, x_row, ne11, (float *)dst->data, dst->nb[1] / 4);
+            else
+                exact_gemm8_kernel<SPY_HIP_Q8_0><<<grid, dim3(256), 0, st>>>((const uint8_t *)w->data, w->nb[1], ne01, nb, xm, x_row, ne11, (float *)dst->data, dst->nb[1] / 4);
+            return SPY_LAUNCH_RC();
+        }
+    }
     const dim3 grid((unsigned)((total + 63) / 64)), block(64);
     // SPY_HIP_EXACT_SERIAL=1: one thread per output element for every type (the plain restatement the lane forms are tested against)
     const bool serial = getenv("SPY_HIP_EXACT_SERIAL") != nullptr;

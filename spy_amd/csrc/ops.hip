@@ -15,7 +15,7 @@ int spy_exact_norm_rms(hipStream_t st, const spy_hip_tensor *x, const spy_hip_te
 int spy_exact_silu(hipStream_t st, const spy_hip_tensor *x, const spy_hip_tensor *dst);
 int spy_exact_softmax(hipStream_t st, const spy_hip_tensor *x, const spy_hip_tensor *mask, const spy_hip_tensor *dst, float scale);
 int spy_exact_rope(hipStream_t st, const spy_hip_tensor *x, const spy_hip_tensor *pos, const spy_hip_tensor *dst, const spy_hip_rope_param *p);
-int spy_exact_dots(hipStream_t st, int t0, const spy_hip_tensor *w, const uint8_t *xm, int64_t x_row, int64_t ne11, const spy_hip_tensor *dst);
+int spy_exact_dots(hipStream_t st, int t0, const spy_hip_tensor *w, const uint8_t *xm, int64_t x_row, int64_t ne11, const spy_hip_tensor *dst, int x_own_quants);
 
 struct tdesc {              // a tensor as the kernels see it
     uint8_t *p;
@@ -605,7 +605,7 @@ static int matmul_impl(void *stream, const spy_hip_tensor *w, const spy_hip_tens
     if (quant) {
         SPY_CHECK_ARG(w->nb[0] == spy_type_size(t0) && w->nb[1] == spy_row_size(t0, ne00));   // whole contiguous rows
         SPY_CHECK_ARG(dst->nb[1] % 4 == 0);
-        if (skip_past < 0 && klimit_past < 0 && spy_exact_on()) return spy_exact_dots(st, t0, w, xm, mid_row, ne11, dst);
+        if (skip_past < 0 && klimit_past < 0 && spy_exact_on()) return spy_exact_dots(st, t0, w, xm, mid_row, ne11, dst, t1 != tm);
         for (int64_t i3 = 0; i3 < ne03; i3++)
             for (int64_t i2 = 0; i2 < ne02; i2++) {
                 const uint8_t *wp = (const uint8_t *)w->data + i2 * w->nb[2] + i3 * w->nb[3];
@@ -620,7 +620,7 @@ static int matmul_impl(void *stream, const spy_hip_tensor *w, const spy_hip_tens
         return 0;
     }
     SPY_CHECK_ARG(w->nb[0] == 2);
-    if (skip_past < 0 && klimit_past < 0 && spy_exact_on()) return spy_exact_dots(st, t0, w, xm, mid_row, ne11, dst);
+    if (skip_past < 0 && klimit_past < 0 && spy_exact_on()) return spy_exact_dots(st, t0, w, xm, mid_row, ne11, dst, 0);
     if (ne11 >= 16 && ne01 >= 16 && ne00 % 8 == 0 && w->nb[1] % 16 == 0 && w->nb[2] % 16 == 0 && w->nb[3] % 16 == 0 &&
         ((uintptr_t)w->data & 15) == 0 && ((uintptr_t)xm & 15) == 0 && dst->nb[1] % 4 == 0 && dst->nb[2] % 4 == 0 && ne02 <= 65535) {
         for (int64_t i3 = 0; i3 < ne03; i3++) {            // prompt-sized attention products: fp16 MFMA

@@ -57,12 +57,39 @@ def test_quantized_matmul_bits(hip, oracle, wtype, M, K, T, serial, monkeypatch)
     _same_bits(dd.download(np.float32).reshape(T, M), want, "matmul type %d %dx%d T %d" % (wtype, M, K, T))
 
 
-def test_q8_0_weights_of_any_byte(hip, oracle):
+@pytest.mark.parametrize("wtype", [O.Q4_0, O.Q8_0])
+@pytest.mark.parametrize("M,K,T", [(96, 4096, 16), (200, 512, 70), (64, 128, 64), (132, 11008, 33), (4096, 4096, 130)])
+def test_tiled_matmul_bits(hip, oracle, wtype, M, K, T, monkeypatch):
+    """Sixteen activation rows and more take the tiled kernel (64 x 64 outputs per workgroup, the eight accumulators
+    of every output in registers): the oracle's bits, with whole and partial tiles along both sides, and the same
+    bits as the row kernels give (SPY_HIP_EXACT_TILED=0)."""
+    from tests.gpu_util import dev, dev_empty, call
+    rng = np.random.default_rng(7 * wtype + M + K + T)
+    w = O.quantize(oracle, (rng.standard_normal((M, K)) * 0.02).astype(np.float32), wtype)
+    x = (rng.standard_normal((T, K)) * rng.uniform(0.1, 30.0, (T, 1))).astype(np.float32)
+    want = O.matmul(oracle, w, wtype, M, K, x, nthread=8)
+    dw, dx = dev(w), dev(x)
+    tw, tx = hip.tensor(dw, wtype, [K, M]), hip.tensor(dx, hip.F32, [K, T])
+    L = hip.load()
+    need = L.spy_hip_op_matmul_scratch_size(B(tw), B(tx))
+    scratch = dev_empty(need, 0)
+    for tiled in ("1", "0"):
+        monkeypatch.setenv("SPY_HIP_EXACT_TILED", tiled)
+        dd = dev_empty(T * M * 4, 0xFF)
+        td = hip.tensor(dd, hip.F32, [M, T])
+        call(L.spy_hip_op_matmul, None, B(tw), B(tx), B(td), scratch.ptr, need)
+        _same_bits(dd.download(np.float32).reshape(T, M), want, "matmul type %d %dx%d T %d tiled %s" % (wtype, M, K, T, tiled))
+
+
+@pytest.mark.parametrize("T", [2, 40])
+def test_q8_0_weights_of_any_byte(hip, oracle, T):
     """Weight bytes a quantizer never writes (-128): the host backend's sign / maddubs sequence
-    (vec_util.h:101-110) gives 128 * -128 for (-128) * (-128); the exact mode follows it."""
+    (vec_util.h:101-110) gives 128 * -128 for (-128) * (-128); the exact mode follows it.  T = 2: the row kernel;
+    T = 40: the tiled kernel, whose plain signed products are the same numbers because the activation bytes,
+    quantized inside the call, never reach -128."""
     from tests.gpu_util import dev, dev_empty, call
     rng = np.random.default_rng(77)
-    M, K, T = 16, 512, 2
+    M, K = 16, 512
     w = O.quantize(oracle, rng.standard_normal((M, K)).astype(np.float32), O.Q8_0).copy()
     blocks = w.reshape(M * K // 32, 34)
     blocks[:, 2:] = rng.integers(0, 256, (blocks.shape[0], 32), dtype=np.uint8)
