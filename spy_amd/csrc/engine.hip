@@ -29,6 +29,7 @@ static int probe_attn(spy_hip_llama *m, int il) {
 }
 enum { PASS_LOGITS = 0, PASS_GREEDY = 1 };
 int spy_exact_on();                              // exact_order.hip
+int spy_exact_thread_scope(int on);              // exact_order.hip
 int spy_exact_luts(const float **lut);           // exact_order.hip
 // summation order of the next single-token pass: the host backend's when the engine is set to it or the library-wide
 // exact-order switch is on (and the exact kernels take the model), else this backend's own
@@ -363,6 +364,9 @@ int spy_gemm_q8act_pair(hipStream_t st, int wtype, const void *w1, const void *w
 int spy_softmax_causal_launch(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *dst, float scale, int n_past);   // ops.hip
 int spy_exact_on();                                                                                                          // exact_order.hip
 int spy_softmax_row_ok(int64_t ne0);                                                                                         // ops.hip
+int64_t spy_exact_prompt_attn_row(int64_t n_kv);                                                                             // exact_prompt.hip
+int spy_exact_prompt_attn(hipStream_t st, const float *q, const uint16_t *kc, const uint16_t *vt, float *S, uint16_t *P16, float *out, const float *lut,
+                          int T, int H, int P, int64_t C, int n_total, float scale);                                        // exact_prompt.hip
 
 // KQ mask of a pass over tokens P .. P + T - 1 (llama.cpp:248-263): row i allows the cached positions j <= P + i
 __global__ __launch_bounds__(256) void causal_mask_kernel(float *__restrict__ mask, int C, int P) {
@@ -374,7 +378,12 @@ __global__ __launch_bounds__(256) void causal_mask_kernel(float *__restrict__ ma
 #define SPY_PREFILL_CHUNK 2048        // tokens per operator-by-operator pass of a long prompt (4096-token prompt: 0.33 s with 512, 0.27 with 1024, 0.24 with 2048, 0.25 with 4096)
 #endif
 enum { HEAD_ALL = 0, HEAD_NONE = 1, HEAD_LAST = 2 };     // output head of a pass: every token's logits (the reference's graph), none, the last token's
-static int forward_ops(spy_hip_llama *m, hipStream_t st, const int32_t *tokens_host, int T, int P, float *logits_host, int head) {
+// n_total: the cached positions after the whole call this pass belongs to (= P + T unless the call is cut into chunks)
+static bool exact_attn_ok(const spy_hip_llama *m) {
+    const char *e = getenv("SPY_HIP_EXACT_PROMPT_ATTN");
+    return m->hd == 128 && m->desc.n_ctx % 32 == 0 && m->lut && !(e && e[0] == '0');
+}
+static int forward_ops(spy_hip_llama *m, hipStream_t st, const int32_t *tokens_host, int T, int P, float *logits_host, int head, int n_total) {
     const spy_hip_llama_desc &c = m->desc;
     const int64_t d = c.n_embd, F = c.n_ff, C = c.n_ctx, H = c.n_head, hd = m->hd, V = c.n_vocab, n_kv = (int64_t)P + T;
     // Passes over many tokens (every MatMul on the matrix cores): the elementwise operators between two MatMuls write the
@@ -390,10 +399,12 @@ static int forward_ops(spy_hip_llama *m, hipStream_t st, const int32_t *tokens_h
     // the logits of every row only when they were asked for
     size_t off = 0;
     auto take = [&](size_t bytes) { size_t o = off; off += (bytes + 255) & ~(size_t)255; return o; };
-    const size_t sp_bytes = fuse_attn ? 0 : (size_t)n_kv * T * H * 4;
+    // exact order with heads of 128: the three attention kernels of exact_prompt.hip (same bits as the operators, masked part left out)
+    const bool xattn = exact && exact_attn_ok(m);
+    const size_t sp_bytes = fuse_attn ? 0 : xattn ? (size_t)spy_exact_prompt_attn_row(n_kv) * T * H * 4 : (size_t)n_kv * T * H * 4;
     const size_t o_x = take(d * T * 4), o_xn = take(d * T * 4), o_q = take(d * T * 4), o_k = take(d * T * 4), o_v = take(d * T * 4),
                  o_o = take(d * T * 4), o_o2 = take(d * T * 4), o_t1 = take(d * T * 4), o_up = take(F * T * 4), o_gate = take(F * T * 4),
-                 o_par = take(F * T * 4), o_S = take(sp_bytes), o_P = take(sp_bytes), o_mask = take(fuse_attn ? 0 : C * T * 4),
+                 o_par = take(F * T * 4), o_S = take(sp_bytes), o_P = take(sp_bytes), o_mask = take(fuse_attn || xattn ? 0 : C * T * 4),
                  o_ids = take(T * 4), o_pos = take(T * 4), o_logits = take(head == HEAD_ALL ? V * T * 4 : V * 4), o_rt = take(T * hd * 4);
     const size_t act_q8 = (size_t)T * ((F > d ? F : d) / 32) * 34;
     const size_t act_f16 = sp_bytes / 2 > (size_t)d * T * 2 ? sp_bytes / 2 : (size_t)d * T * 2;
@@ -417,7 +428,7 @@ static int forward_ops(spy_hip_llama *m, hipStream_t st, const int32_t *tokens_h
         for (int i = 0; i < T; i++) hp[i] = P + i;
         HIP_TRY(hipMemcpyAsync(ids, tokens_host, (size_t)T * 4, hipMemcpyHostToDevice, st));
         HIP_TRY(hipMemcpyAsync(pos, hp.data(), (size_t)T * 4, hipMemcpyHostToDevice, st));
-        if (!fuse_attn) {
+        if (!fuse_attn && !xattn) {
             causal_mask_kernel<<<dim3((unsigned)((C + 255) / 256), (unsigned)T), dim3(256), 0, st>>>(mask, (int)C, P);   // filled on the device: 35 MB per 2048-token chunk
             HIP_TRY(hipGetLastError());
         }
@@ -475,6 +486,9 @@ static int forward_ops(spy_hip_llama *m, hipStream_t st, const int32_t *tokens_h
         if (fuse_attn) {          // scores, masked softmax and the product with V^T in one kernel: no score / probability matrix in memory
             RC_TRY(spy_prompt_attn_launch(st, (const uint16_t *)xn, (const uint16_t *)m->k_cache[il], (const uint16_t *)m->v_cache[il], o2,
                                           T, (int)H, (int)hd, P, C, scale));
+        } else if (xattn) {
+            RC_TRY(spy_exact_prompt_attn(st, q, (const uint16_t *)m->k_cache[il], (const uint16_t *)m->v_cache[il], S, (uint16_t *)Pm, o2, m->lut,
+                                         T, (int)H, P, C, n_total, scale));
         } else {
         spy_hip_tensor t_kall = T3s(SPY_HIP_F16, m->k_cache[il], hd, n_kv, H, 2, 2 * d, 2 * hd);
         spy_hip_tensor t_vall = T3s(SPY_HIP_F16, m->v_cache[il], n_kv, hd, H, 2, 2 * C, 2 * C * hd);
@@ -551,6 +565,13 @@ static int forward_any(spy_hip_llama *m, void *stream, const int32_t *tokens_hos
     SPY_CHECK_ARG((int64_t)n_past + n_token <= m->desc.n_ctx);                  // llama.cpp:249
     hipStream_t st = stream ? (hipStream_t)stream : m->own_stream;
     for (int i = 0; i < n_token; i++) SPY_CHECK_ARG(tokens_host[i] >= 0 && tokens_host[i] < m->desc.n_vocab);   // view.cpp:61
+    // A model in order 1 runs its prompt passes in the host's order as well (SPY_HIP_PROMPT_ORDER=0: prompts on the matrix cores in
+    // this backend's own order, single-token passes still in order 1)
+    struct scope_t { int prev; bool on; ~scope_t() { if (on) spy_exact_thread_scope(prev); } } scope = {-1, false};
+    if (n_token > 1 && !spy_exact_on() && pass_order(m) == 1) {
+        const char *e = getenv("SPY_HIP_PROMPT_ORDER");
+        if (!(e && e[0] == '0')) { scope.prev = spy_exact_thread_scope(1); scope.on = true; }
+    }
     const bool exact = spy_exact_on() != 0;
     // single tokens: the fused pass, in the order pass_order() names (with the library-wide exact-order switch on and a
     // model the exact kernels do not take, operator by operator instead)
@@ -568,13 +589,14 @@ static int forward_any(spy_hip_llama *m, void *stream, const int32_t *tokens_hos
     const int ch_req = ch_env ? atoi(ch_env) : 0;
     // exact order: one pass over the whole prompt, as the reference runs it (a chunk boundary moves elements between
     // the 8-lane part and the scalar tail of the KQV dots and between the groups of four of the softmax sum)
-    const int CH = exact ? n_token : ch_req >= 16 ? ch_req : SPY_PREFILL_CHUNK;
+    // ... unless the attention kernels that take the length of the whole row as a number are in use
+    const int CH = exact && !exact_attn_ok(m) ? n_token : ch_req >= 16 ? ch_req : SPY_PREFILL_CHUNK;
     for (int t0 = 0; t0 < n_token; t0 += CH) {
         const int tc = n_token - t0 < CH ? n_token - t0 : CH;
         // logits nobody asked for are not computed: no buffer -> no head; last_only -> the head runs on the last row of the last chunk
         const int head = !logits_host ? HEAD_NONE : !last_only ? HEAD_ALL : (t0 + tc == n_token ? HEAD_LAST : HEAD_NONE);
         float *dst = !logits_host ? nullptr : last_only ? logits_host : logits_host + (size_t)t0 * m->desc.n_vocab;
-        RC_TRY(forward_ops(m, st, tokens_host + t0, tc, n_past + t0, dst, head));
+        RC_TRY(forward_ops(m, st, tokens_host + t0, tc, n_past + t0, dst, head, n_past + n_token));
     }
     return 0;
 }

@@ -686,7 +686,17 @@ int spy_exact_luts(const float **lut) {
     return 0;
 }
 
+// A caller may switch the exact order on for the calls its own thread makes (a model whose passes run in the host's order
+// issues its prompt operators that way) without touching what other threads see.
+static thread_local int t_exact = -1;
+int spy_exact_thread_scope(int on) {      // on: 1, 0, or -1 for "as the library-wide switch says"; returns the previous value
+    const int prev = t_exact;
+    t_exact = on;
+    return prev;
+}
+
 int spy_exact_on() {
+    if (t_exact >= 0) return t_exact;
     if (g_exact < 0) {
         const char *e = getenv("SPY_HIP_EXACT");
         g_exact = (e && *e && *e != '0') ? 1 : 0;

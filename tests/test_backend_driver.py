@@ -42,11 +42,16 @@ def test_submit_path_matches_oracle_and_engine(wtype):
     from tests.model_util import OracleModel
     cfg = M.Config(n_layer=2, n_embd=256, n_head=2, n_ff=768, n_vocab=512, n_ctx=64, wtype=wtype)
     tensors = M.synth_model(cfg, seed=7)
-    host, eng, ora = B.HostModel(cfg, tensors), M.Engine(cfg, tensors), OracleModel(cfg, tensors)
+    host, eng, ora = B.HostModel(cfg, tensors), M.Engine(cfg, tensors, order=0), OracleModel(cfg, tensors)
     prompt = np.random.default_rng(3).integers(0, cfg.n_vocab, 6).astype(np.int32)
     lg_h, lg_e, lg_o = host.forward(prompt, 0), eng.forward(prompt, 0), ora.forward(prompt, 0)
     assert_close(lg_h, lg_o, "submit-path prefill logits vs oracle")
-    assert np.array_equal(lg_h, lg_e), "the submit path and the engine's prefill launch the same operator kernels"
+    assert np.array_equal(lg_h, lg_e), "the submit path and the engine's prefill in its own order launch the same operator kernels"
+    # the engine in the host's order (its default) issues the same operators in their exact forms: the oracle's bits
+    eng1 = M.Engine(cfg, tensors)
+    assert eng1.order() == 1
+    assert np.array_equal(eng1.forward(prompt, 0).view(np.uint32), lg_o.view(np.uint32)), "prompt pass of an engine in order 1: the oracle's bits"
+    eng1.close()
     st = host.stats()
     assert st["n_ops"] == 33 * cfg.n_layer + 4 and st["n_submit"] == st["n_ops"]      # 33 operators per layer + embedding + 3 head ops
     assert st["n_alloc"] == st["n_free"] > 0, st                                   # every Dynamic tensor went back to the pool (default_scheduler.h:186-228)
@@ -107,7 +112,7 @@ def test_engine_prompt_softmax_without_mask_tensor_matches_submit_path(monkeypat
     from spy_amd import model as M
     cfg = M.Config(n_layer=2, n_embd=256, n_head=2, n_ff=768, n_vocab=512, n_ctx=448, wtype=O.Q4_0)
     tensors = M.synth_model(cfg, seed=11)
-    host, eng = B.HostModel(cfg, tensors), M.Engine(cfg, tensors)
+    host, eng = B.HostModel(cfg, tensors), M.Engine(cfg, tensors, order=0)        # own order: the kernels the submit path launches by default
     prompt = np.random.default_rng(5).integers(0, cfg.n_vocab, 438).astype(np.int32)
     # passes of 168, 136 and 134 tokens: the attention products span several 128 x 128 tiles, some of them entirely
     # above the causal diagonal (left out by the engine); the last pass has rows of 438 positions (not a multiple of 8:
@@ -146,7 +151,7 @@ def test_engine_prompt_pass_wide_layer_matches_submit_path(monkeypatch):
         n_embd, n_head, n_ff, n_tok = dims       # the second: wq, wk, wv, wo and down wide enough for the tile kernel too
         cfg = M.Config(n_layer=1, n_embd=n_embd, n_head=n_head, n_ff=n_ff, n_vocab=512, n_ctx=n_tok + 16, wtype=wtype)
         tensors = M.synth_model(cfg, seed=3)
-        host, eng = B.HostModel(cfg, tensors), M.Engine(cfg, tensors)
+        host, eng = B.HostModel(cfg, tensors), M.Engine(cfg, tensors, order=0)
         prompt = np.random.default_rng(8).integers(0, cfg.n_vocab, n_tok).astype(np.int32)
         lg_h, lg_e = host.forward(prompt, 0), eng.forward(prompt, 0)
         assert np.isfinite(lg_e).all() and np.array_equal(lg_h, lg_e), dims

@@ -257,6 +257,48 @@ def test_engine_follows_the_switch(hip, n_prompt):
     eng.close()
 
 
+@pytest.mark.parametrize("n_prompt,n_first,chunk", [(100, 0, 0), (130, 70, 0), (97, 0, 32), (200, 33, 64), (256, 0, 0), (65, 64, 0)])
+def test_engine_prompt_attention_kernels_have_the_oracle_bits(hip, n_prompt, n_first, chunk, monkeypatch):
+    """Prompt passes of the engine in exact order with heads of 128: scores, softmax and the product with V^T come from the
+    three kernels that leave out the masked part.  One pass, a pass on top of cached tokens, and calls cut into chunks of
+    32 or 64 query rows (the row length the host's loops depend on is that of the whole call): the oracle's bits, and
+    the bits of the operator-by-operator path (SPY_HIP_EXACT_PROMPT_ATTN=0)."""
+    from spy_amd import model as M
+    from tests.model_util import OracleModel
+    cfg = M.Config(n_layer=2, n_embd=256, n_head=2, n_ff=768, n_vocab=512, n_ctx=256, wtype=O.Q4_0)
+    tensors = M.synth_model(cfg, seed=6)
+    prompt = np.random.default_rng(n_prompt).integers(0, cfg.n_vocab, n_prompt).astype(np.int32)
+    ora = OracleModel(cfg, tensors)
+    want_first = ora.forward(prompt[:n_first], 0) if n_first else None
+    want = ora.forward(prompt[n_first:], n_first)
+    if chunk:
+        monkeypatch.setenv("SPY_HIP_PREFILL_CHUNK", str(chunk))
+    for kernels in ("1", "0"):
+        monkeypatch.setenv("SPY_HIP_EXACT_PROMPT_ATTN", kernels)
+        eng = M.Engine(cfg, tensors)
+        if n_first:
+            _same_bits(eng.forward(prompt[:n_first], 0), want_first, "first %d tokens, kernels %s" % (n_first, kernels))
+        _same_bits(eng.forward(prompt[n_first:], n_first), want, "%d tokens after %d, chunk %d, kernels %s" % (n_prompt - n_first, n_first, chunk, kernels))
+        eng.close()
+
+
+def test_prompt_attention_kernels_at_the_7b_width(hip, monkeypatch):
+    """One layer of the 7B shape, 700 tokens on top of 300: the attention kernels against the operator path, bit for bit."""
+    from spy_amd import model as M
+    cfg = M.Config.llama2_7b(n_ctx=1024, wtype=O.Q4_0)
+    cfg.n_layer = 1
+    tensors = M.synth_model(cfg, seed=8)
+    prompt = np.random.default_rng(1).integers(0, cfg.n_vocab, 1000).astype(np.int32)
+    got = {}
+    for kernels in ("1", "0"):
+        monkeypatch.setenv("SPY_HIP_EXACT_PROMPT_ATTN", kernels)
+        eng = M.Engine(cfg, tensors)
+        eng.forward(prompt[:300], 0, want_logits=False)
+        got[kernels] = eng.forward_last(prompt[300:], 300)
+        eng.close()
+    _same_bits(got["1"], got["0"], "7B width, 700 tokens after 300")
+
+
 @pytest.mark.timeout(900)
 @pytest.mark.parametrize("wtype", [O.Q4_0, O.Q8_0])
 def test_llama2_7b_greedy_32_tokens_identical(wtype):
