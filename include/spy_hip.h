@@ -266,7 +266,8 @@ int spy_hip_llama_forward_last(spy_hip_llama *m, void *stream, const int32_t *to
  * receives the token sampled by step i.  use_graph: replay a captured HIP graph. */
 int spy_hip_llama_decode_greedy(spy_hip_llama *m, void *stream, int32_t first_token, int32_t n_past, int32_t n_steps,
                                 int32_t *tokens_host, int32_t use_graph);
-/* Summation order of the fused single-token pass.  1 (the default wherever the kernels take the model: 128-wide heads,
+/* Summation order of the model's passes: of the fused single-token pass, and of prompt passes (in order 1 they run
+ * operator by operator through the exact-order kernels, in order 0 on the matrix cores).  1 (the default wherever the kernels take the model: 128-wide heads,
  * n_embd and n_ff multiples of 128): the host backend's -- the eight accumulators and hsum_float_8 of its quantized dots,
  * the 4 x 8 accumulators, tree and scalar tail of its fp16 dots (vec_dot.h:42-146), libstdc++'s four-way reduce in
  * NormRMS and Softmax (non-linear.cpp:129-223), exp / silu from the fp16-indexed tables and the RoPE angles from the

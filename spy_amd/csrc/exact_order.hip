@@ -9,9 +9,9 @@
 // a model with near-tied logits can differ.  With spy_hip_set_exact_order(1) (or SPY_HIP_EXACT=1) the
 // spy_hip_op_* entry points launch the kernels below instead: every accumulator of the host loops has
 // one lane (or one thread) that walks its sum in the host backend's order, the tables and the rotation
-// angles come from the host's libm, and the outputs are the host backend's bit for bit.  This is the
-// checking mode of the operator path (7B Q4_0, short context: 70 tok/s against 118 tok/s with the default
-// operator kernels and 830 tok/s in the fused token loop, which steps aside for it while it is on).
+// angles come from the host's libm, and the outputs are the host backend's bit for bit.  The token loop
+// issues the prompt passes of a model in the host's order through these kernels as well (a thread-local
+// scope, spy_exact_thread_scope); its single-token passes have fused kernels of their own.
 #include "common.cuh"
 
 #include <math.h>
