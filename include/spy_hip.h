@@ -160,6 +160,18 @@ int spy_hip_gemm_q8_0act(void *stream, int wtype, const void *w, const void *xq,
  * hd must be 128 and n_ctx a multiple of 8 (else SPY_HIP_EUNSUPPORTED). */
 int spy_hip_prompt_attention(void *stream, const void *q16, const void *k_cache, const void *v_cache, float *out,
                              int32_t T, int32_t H, int32_t hd, int32_t past, int64_t n_ctx, float scale);
+/* The same three operators in the host backend's summation order, bit for bit (Dot<FP16,FP16> with its 32 accumulators,
+ * tree and scalar tail, vec_dot.h:117-146; Softmax with the table exp and libstdc++'s groups of four,
+ * non-linear.cpp:86-180), as three kernels that leave out what the causal mask removes.  q: rotated queries as f32
+ * [T][H*hd] (converted to fp16 inside, as MatMul does, mat.cpp:37); caches and out as above.  n_total: the cached
+ * positions after the whole pass this call is a part of (past + T when the pass is not cut into chunks): the host's
+ * dot adds the last 1..32 of them one by one and its softmax sum the last n_total % 4 terms.  scratch: device memory
+ * of spy_hip_prompt_attention_exact_scratch_size bytes, 256-byte aligned (scores and probabilities of this call).
+ * hd must be 128 and n_ctx a multiple of 32 (else SPY_HIP_EUNSUPPORTED). */
+size_t spy_hip_prompt_attention_exact_scratch_size(int32_t T, int32_t H, int32_t past);
+int spy_hip_prompt_attention_exact(void *stream, const float *q, const void *k_cache, const void *v_cache, float *out,
+                                   int32_t T, int32_t H, int32_t hd, int32_t past, int64_t n_ctx, int32_t n_total, float scale,
+                                   void *scratch, size_t scratch_bytes);
 /* the int32 dot of every 32-element block (Q4_0, Q8_0, Q4_K sub-blocks) or 16-element
  * sub-block (Q6_K) of every weight row with activation row 0: out[m*nsub + b], written by the
  * GEMV kernels themselves (same code path, dump switch on).  `out` must hold M*nsub + M int32:

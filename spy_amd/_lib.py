@@ -96,6 +96,8 @@ SIGNATURES = {
     "spy_hip_gemv_q8_0act": (_i32, [_vp, _i32, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64]),
     "spy_hip_gemm_q8_0act": (_i32, [_vp, _i32, _vp, _vp, _vp, _i64, _i64, _i64, _i64]),
     "spy_hip_prompt_attention": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i64, C.c_float]),
+    "spy_hip_prompt_attention_exact_scratch_size": (_sz, [_i32, _i32, _i32]),
+    "spy_hip_prompt_attention_exact": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i64, _i32, C.c_float, _vp, _sz]),
     "spy_hip_block_dots": (_i32, [_vp, _i32, _vp, _vp, _vp, _i64, _i64]),
     "spy_hip_rmsnorm_q8_0": (_i32, [_vp, _i32, _vp, _vp, _f32, _i64, _vp]),
     "spy_hip_rope_kvwrite": (_i32, [_vp, _i32, _i32, _i32, _vp, _vp, _vp, _vp, _vp, _f32, _i32, _i32, _i32, _i64, _vp, _vp, _vp, _vp, _vp]),

@@ -338,3 +338,25 @@ int spy_exact_prompt_attn(hipStream_t st, const float *q, const uint16_t *kc, co
     xp_pv_kernel<<<dim3((unsigned)((T + XP_PT - 1) / XP_PT), 4, (unsigned)H), dim3(256), 0, st>>>(P16, vt, out, T, H, P, s_row, C, n_total);
     return SPY_LAUNCH_RC();
 }
+
+int spy_exact_luts(const float **lut);           // exact_order.hip
+
+extern "C" size_t spy_hip_prompt_attention_exact_scratch_size(int32_t T, int32_t H, int32_t past) {
+    if (T <= 0 || H <= 0 || past < 0) return 0;
+    return (size_t)spy_exact_prompt_attn_row((int64_t)past + T) * (size_t)T * (size_t)H * 6;       // fp32 scores, then fp16 probabilities
+}
+
+extern "C" int spy_hip_prompt_attention_exact(void *stream, const float *q, const void *k_cache, const void *v_cache, float *out, int32_t T, int32_t H,
+                                              int32_t hd, int32_t past, int64_t n_ctx, int32_t n_total, float scale, void *scratch, size_t scratch_bytes) {
+    SPY_CHECK_ARG(q && k_cache && v_cache && out && scratch);
+    if (hd != 128 || n_ctx % 32) return SPY_HIP_EUNSUPPORTED;
+    const size_t need = spy_hip_prompt_attention_exact_scratch_size(T, H, past);
+    if (!need) return SPY_HIP_EINVAL;
+    if (scratch_bytes < need || ((uintptr_t)scratch & 255)) return SPY_HIP_ENOSPACE;
+    const float *lut = nullptr;
+    const int rc = spy_exact_luts(&lut);
+    if (rc) return rc;
+    float *S = (float *)scratch;
+    uint16_t *P16 = (uint16_t *)((uint8_t *)scratch + need / 6 * 4);
+    return spy_exact_prompt_attn((hipStream_t)stream, q, (const uint16_t *)k_cache, (const uint16_t *)v_cache, S, P16, out, lut, T, H, past, n_ctx, n_total, scale);
+}

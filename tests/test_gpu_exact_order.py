@@ -142,6 +142,48 @@ def test_attention_products_bits(hip, oracle, n_kv, serial, monkeypatch):
     _same_bits(dO.download(np.float32).reshape(O_want.shape), O_want, "KQV n_kv %d" % n_kv)
 
 
+@pytest.mark.parametrize("H_,past,T,n_ctx,cuts", [
+    (32, 0, 40, 64, (0, 40)),                 # all 32 heads, a pass shorter than two chunks of 32
+    (4, 168, 136, 448, (0, 136)),             # on top of cached tokens
+    (2, 57, 200, 320, (0, 37, 101, 200)),     # the same pass in three pieces: row length 257 (tail of one, remainder of one)
+    (2, 0, 230, 256, (0, 64, 230)),           # row length 230: 6 elements in the scalar tail, 2 in the softmax remainder
+    (1, 4000, 95, 4096, (0, 32, 95)),         # long rows: row length 4095, tail of 31, remainder of 3
+    (3, 31, 1, 64, (0, 1)),                   # one query row
+])
+def test_exact_prompt_attention_bits(hip, oracle, H_, past, T, n_ctx, cuts):
+    """spy_hip_prompt_attention_exact against the oracle's MatMul(K view, q) -> Softmax(causal mask, scale) ->
+    MatMul(V^T view, P) over the whole pass: equal bits, also when the pass is handed over in pieces (each piece is told
+    the row length of the whole pass)."""
+    from tests.gpu_util import dev, dev_empty, call
+    hd, n_kv = 128, past + T
+    d = H_ * hd
+    rng = np.random.default_rng(17 * T + past)
+    scale = float(1.0 / np.sqrt(hd))
+    q = (rng.standard_normal((T, H_, hd)) * 1.5).astype(np.float32)
+    kc = np.zeros((n_ctx, d), np.float16); kc[:n_kv] = rng.standard_normal((n_kv, d)).astype(np.float16)
+    vc = np.full((d, n_ctx), np.nan, np.float16); vc[:, :n_kv] = rng.standard_normal((d, n_kv)).astype(np.float16)   # NaN where nothing is cached yet
+    mask = np.where(np.arange(n_ctx)[None, :] <= (np.arange(T)[:, None] + past), 0.0, -np.inf).astype(np.float32)
+    S_o, P_o = np.zeros((H_, T, n_kv), np.float32), np.zeros((H_, T, n_kv), np.float32)
+    O_o = np.zeros((H_, T, hd), np.float32)
+    assert oracle.spy_o_matmul(B(O.tensor(kc.view(np.uint16), O.F16, [hd, n_kv, H_], nb=[2, 2 * d, 2 * hd])),
+                               B(O.tensor(q, O.F32, [hd, T, H_], nb=[4, 4 * d, 4 * hd])), B(O.tensor(S_o, O.F32, [n_kv, T, H_])), 4) == 0
+    assert oracle.spy_o_softmax(B(O.tensor(S_o, O.F32, [n_kv, T, H_])), B(O.tensor(mask, O.I32, [n_ctx, T])), B(O.tensor(P_o, O.F32, [n_kv, T, H_])), scale) == 0
+    vc_o = np.where(np.isnan(vc), np.float16(0), vc)          # the oracle multiplies the masked zeros with what the cache holds
+    assert oracle.spy_o_matmul(B(O.tensor(vc_o.view(np.uint16), O.F16, [n_kv, hd, H_], nb=[2, 2 * n_ctx, 2 * n_ctx * hd])),
+                               B(O.tensor(P_o, O.F32, [n_kv, T, H_])), B(O.tensor(O_o, O.F32, [hd, T, H_])), 4) == 0
+    want = np.ascontiguousarray(O_o.transpose(1, 0, 2)).reshape(T, d)
+    L = hip.load()
+    dq, dk, dv = dev(q), dev(kc.view(np.uint16)), dev(vc.view(np.uint16))
+    out = dev_empty(T * d * 4, 0xFF)
+    for a, b in zip(cuts[:-1], cuts[1:]):
+        need = L.spy_hip_prompt_attention_exact_scratch_size(b - a, H_, past + a)
+        sc = dev_empty(need, 0xFF)
+        call(L.spy_hip_prompt_attention_exact, None, dq.ptr + a * d * 4, dk.ptr, dv.ptr, out.ptr + a * d * 4, b - a, H_, hd, past + a, n_ctx, n_kv, scale, sc.ptr, need)
+    _same_bits(out.download(np.float32).reshape(T, d), want, "attention H %d past %d T %d in %d pieces" % (H_, past, T, len(cuts) - 1))
+    assert L.spy_hip_prompt_attention_exact(None, dq.ptr, dk.ptr, dv.ptr, out.ptr, T, H_, 64, past, n_ctx, n_kv, scale, sc.ptr, need) == hip.EUNSUPPORTED
+    assert L.spy_hip_prompt_attention_exact(None, dq.ptr, dk.ptr, dv.ptr, out.ptr, T, H_, hd, past, n_ctx, n_kv, scale, sc.ptr, 1024) == hip.ENOSPACE
+
+
 def test_norm_softmax_silu_rope_bits(hip, oracle):
     from tests.gpu_util import dev, dev_empty, call
     L = hip.load()
