@@ -459,13 +459,20 @@ __global__ __launch_bounds__(256) void exact_dots8_kernel(xdesc w, const uint8_t
 // acc), and the eight are added in hsum_float_8's tree at the end, so the results are those of exact_dots8_kernel bit
 // for bit; what changes is that a weight block and an activation block are unpacked once per tile (into LDS, as
 // words in element order: the low nibbles of a Q4_0 block first, then the high ones) instead of once per output.
-// The integer sums come from v_dot4_i32_i8 onto 0x4B400000, the bits of 1.5 * 2^23: read as a float, the sum minus
-// 12582912.0f is the exact conversion (|sum| < 2^22).  v_dot4 multiplies the signed bytes as they are, which equals
+// The integer sums are accumulated onto 0x4B400000, the bits of 1.5 * 2^23: read as a float, the sum minus
+// 12582912.0f is the exact conversion (|sum| < 2^22).  The hardware multiplies the signed bytes as they are, which equals
 // the host's abs / sign / saturating pair sum (vec_util.h:101-110) as long as no ACTIVATION byte is -128; the launcher
 // takes this kernel only for activations that this library quantized itself (|q| <= 127).
 #define XGB_TILE 64
 #define XGB_KB 4          // blocks per stage
-template <int WT>
+typedef int xgb_v4i __attribute__((ext_vector_type(4)));
+// MF = true: the integer sums come from the matrix cores instead: v_mfma_i32_4x4x4_16b_i8 multiplies, in each group of four
+// lanes, a 4 x 4 byte matrix (lane j supplies row j) by another (lane j supplies column j) and leaves column j of the 4 x 4
+// result in lane j -- sixteen four-element dot products per group, exactly one accumulator's share of a block.  A wave then
+// holds 16 weight rows x 64 activation rows (lane = activation row 4b + j; the weight words of rows 4g + j, g = 0..3, are
+// the same for all sixteen groups and come as one broadcast read), a lane again 16 outputs with 8 accumulators each, and
+// the vector units are left with the subtraction and the fma per term.
+template <int WT, bool MF>
 __global__ __launch_bounds__(256, 2) void exact_gemm8_kernel(const uint8_t *__restrict__ w, int64_t w_row, int64_t ne01, int64_t nb,
                                                               const uint8_t *__restrict__ xm, int64_t x_row, int64_t ne11,
                                                               float *__restrict__ dst, int64_t d_row) {
@@ -474,13 +481,17 @@ __global__ __launch_bounds__(256, 2) void exact_gemm8_kernel(const uint8_t *__re
     __shared__ __align__(16) float s_wd[2][XGB_KB][XGB_TILE];
     __shared__ __align__(16) float s_xd[2][XGB_KB][XGB_TILE];
     const int tid = threadIdx.x;
-    const int mg = tid & 15, tg = tid >> 4;
+    const int mg = tid & 15, tg = tid >> 4;                              // MF = false: 4 weight rows x 4 activation rows per thread
+    const int wv = tid >> 6, bj = tid & 63, jj = tid & 3;                // MF = true: wave, activation row of the tile, lane within its group of four
     const int64_t m0 = (int64_t)blockIdx.x * XGB_TILE, t0 = (int64_t)blockIdx.y * XGB_TILE;
 
     // loaders: waves 0 and 1 bring weight blocks, waves 2 and 3 activation blocks; a thread takes two neighbouring
     // blocks of one row (36 bytes of Q4_0, 68 of Q8_0: whole aligned words) per stage
     const bool ld_w = tid < 128;
     const int ld_row = tid & 63, ld_pair = (tid >> 6) & 1;
+    // where a weight row's words go in their LDS plane: in row order, or (MF) rows j, j + 4, j + 8, ... side by side so that the
+    // four words a lane feeds to its four matrix instructions are one 16-byte read
+    const int ld_slot = (MF && ld_w) ? (ld_row & 3) * 16 + (ld_row >> 2) : ld_row;
     constexpr int NWQ = WT == SPY_HIP_Q4_0 ? 9 : 17;
     const uint32_t *ld_src;
     if (ld_w) ld_src = (const uint32_t *)(w + min(m0 + ld_row, ne01 - 1) * w_row) + ld_pair * NWQ;
@@ -509,8 +520,8 @@ __global__ __launch_bounds__(256, 2) void exact_gemm8_kernel(const uint8_t *__re
                 // per byte n - 8: n + 128 - 8 never borrows across bytes, then the top bit is flipped back
                 lo0 = ((lo0 | 0x80808080u) - 0x08080808u) ^ 0x80808080u; hi0 = ((hi0 | 0x80808080u) - 0x08080808u) ^ 0x80808080u;
                 lo1 = ((lo1 | 0x80808080u) - 0x08080808u) ^ 0x80808080u; hi1 = ((hi1 | 0x80808080u) - 0x08080808u) ^ 0x80808080u;
-                s_wq[buf][k0][k][ld_row] = lo0; s_wq[buf][k0][4 + k][ld_row] = hi0;
-                s_wq[buf][k0 + 1][k][ld_row] = lo1; s_wq[buf][k0 + 1][4 + k][ld_row] = hi1;
+                s_wq[buf][k0][k][ld_slot] = lo0; s_wq[buf][k0][4 + k][ld_slot] = hi0;
+                s_wq[buf][k0 + 1][k][ld_slot] = lo1; s_wq[buf][k0 + 1][4 + k][ld_slot] = hi1;
             }
         } else {
             // Q8_0 pair: block 0 = scale in the low half of g[0] and 32 quant bytes from byte 2, block 1 = scale in the high half
@@ -522,8 +533,8 @@ __global__ __launch_bounds__(256, 2) void exact_gemm8_kernel(const uint8_t *__re
             sd[k0 + 1][ld_row] = h2f_tab((uint16_t)(g[8] >> 16));
 #pragma unroll
             for (int k = 0; k < 8; k++) {
-                sq[k0][k][ld_row] = __builtin_amdgcn_alignbit(g[k + 1], g[k], 16);
-                sq[k0 + 1][k][ld_row] = g[9 + k];
+                sq[k0][k][ld_slot] = __builtin_amdgcn_alignbit(g[k + 1], g[k], 16);
+                sq[k0 + 1][k][ld_slot] = g[9 + k];
             }
         }
     };
@@ -543,6 +554,44 @@ __global__ __launch_bounds__(256, 2) void exact_gemm8_kernel(const uint8_t *__re
     for (int64_t s = 0; s < nstage; s++) {
         const int buf = (int)(s & 1);
         if (s + 1 < nstage) fetch(s + 1);
+        if constexpr (MF) {
+            // acc[g][i]: weight row 16 * wave + 4g + i against this lane's activation row
+            const xgb_v4i bias = {0x4B400000, 0x4B400000, 0x4B400000, 0x4B400000};
+#pragma unroll 1
+            for (int kb = 0; kb < XGB_KB; kb++) {
+                const float xd = s_xd[buf][kb][bj];
+                float D[4][4];
+#pragma unroll
+                for (int gq = 0; gq < 4; gq++) {
+                    const float4 wd4 = *(const float4 *)&s_wd[buf][kb][16 * wv + 4 * gq];
+                    D[gq][0] = wd4.x * xd; D[gq][1] = wd4.y * xd; D[gq][2] = wd4.z * xd; D[gq][3] = wd4.w * xd;
+                }
+                // the four matrix instructions of word e + 1 are issued before the vector work on the results of word e
+                xgb_v4i p[2][4];
+                auto issue = [&](int e, xgb_v4i (&out)[4]) {
+                    const uint4 wq4 = *(const uint4 *)&s_wq[buf][kb][e][jj * 16 + 4 * wv];      // rows 16 * wave + 4g + j, g = 0..3
+                    const uint32_t xq = s_xq[buf][kb][e][bj];
+                    out[0] = __builtin_amdgcn_mfma_i32_4x4x4i8((int)wq4.x, (int)xq, bias, 0, 0, 0);
+                    out[1] = __builtin_amdgcn_mfma_i32_4x4x4i8((int)wq4.y, (int)xq, bias, 0, 0, 0);
+                    out[2] = __builtin_amdgcn_mfma_i32_4x4x4i8((int)wq4.z, (int)xq, bias, 0, 0, 0);
+                    out[3] = __builtin_amdgcn_mfma_i32_4x4x4i8((int)wq4.w, (int)xq, bias, 0, 0, 0);
+                };
+                issue(0, p[0]);
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    if (e + 1 < 8) issue(e + 1, p[(e + 1) & 1]);
+                    const int a = WT == SPY_HIP_Q4_0 ? ((e + 4) & 7) : e;
+#pragma unroll
+                    for (int gq = 0; gq < 4; gq++) {
+                        const xgb_v4i r = p[e & 1][gq];
+                        acc[gq][0][a] = fmaf(D[gq][0], __int_as_float(r.x) - 12582912.0f, acc[gq][0][a]);
+                        acc[gq][1][a] = fmaf(D[gq][1], __int_as_float(r.y) - 12582912.0f, acc[gq][1][a]);
+                        acc[gq][2][a] = fmaf(D[gq][2], __int_as_float(r.z) - 12582912.0f, acc[gq][2][a]);
+                        acc[gq][3][a] = fmaf(D[gq][3], __int_as_float(r.w) - 12582912.0f, acc[gq][3][a]);
+                    }
+                }
+            }
+        } else {
 #pragma unroll 1
         for (int kb = 0; kb < XGB_KB; kb++) {
             const float4 wd4 = *(const float4 *)&s_wd[buf][kb][4 * mg], xd4 = *(const float4 *)&s_xd[buf][kb][4 * tg];
@@ -581,9 +630,19 @@ __global__ __launch_bounds__(256, 2) void exact_gemm8_kernel(const uint8_t *__re
                         acc[r][c][a] = fmaf(D[r][c], __int_as_float(p[4 * r + c]) - 12582912.0f, acc[r][c][a]);
             }
         }
+        }
         if (s + 1 < nstage) put(buf ^ 1);
         __syncthreads();
     }
+    if constexpr (MF) {
+        const int64_t tok = t0 + bj;
+#pragma unroll
+        for (int gq = 0; gq < 4; gq++) {
+            const int64_t row = m0 + 16 * wv + 4 * gq;
+            if (tok < ne11 && row < ne01)
+                *(float4 *)(dst + tok * d_row + row) = make_float4(hsum8(acc[gq][0]), hsum8(acc[gq][1]), hsum8(acc[gq][2]), hsum8(acc[gq][3]));
+        }
+    } else {
 #pragma unroll
     for (int c = 0; c < 4; c++) {
         const int64_t tok = t0 + 4 * tg + c;
@@ -592,6 +651,7 @@ __global__ __launch_bounds__(256, 2) void exact_gemm8_kernel(const uint8_t *__re
         for (int r = 0; r < 4; r++) o[r] = hsum8(acc[r][c]);
         const int64_t row = m0 + 4 * mg;
         if (tok < ne11 && row < ne01) *(float4 *)(dst + tok * d_row + row) = make_float4(o[0], o[1], o[2], o[3]);
+    }
     }
 }
 
@@ -808,10 +868,12 @@ int spy_exact_dots(hipStream_t st, int t0, const spy_hip_tensor *w, const uint8_
                           (ne11 + XGB_TILE - 1) / XGB_TILE <= 65535 && !getenv("SPY_HIP_EXACT_SERIAL");
         if (tiled && fits) {
             const dim3 grid((unsigned)((ne01 + XGB_TILE - 1) / XGB_TILE), (unsigned)((ne11 + XGB_TILE - 1) / XGB_TILE));
-            if (t0 == SPY_HIP_Q4_0)
-                exact_gemm8_kernel<SPY_HIP_Q4_0><<<grid, dim3(256), 0, st>>>((const uint8_t *)w->data, w->nb[1], ne01, nb, xm, x_row, ne11, (float *)dst->data, dst->nb[1] / 4);
-            else
-                exact_gemm8_kernel<SPY_HIP_Q8_0><<<grid, dim3(256), 0, st>>>((const uint8_t *)w->data, w->nb[1], ne01, nb, xm, x_row, ne11, (float *)dst->data, dst->nb[1] / 4);
+            // SPY_HIP_EXACT_TILED=dot: the integer sums from v_dot4 on the vector units instead of the matrix cores
+            const bool mf = !(env_tiled && *env_tiled == 'd');
+#define XGB_LAUNCH(WT, MF) exact_gemm8_kernel<WT, MF><<<grid, dim3(256), 0, st>>>((const uint8_t *)w->data, w->nb[1], ne01, nb, xm, x_row, ne11, (float *)dst->data, dst->nb[1] / 4)
+            if (t0 == SPY_HIP_Q4_0) { if (mf) XGB_LAUNCH(SPY_HIP_Q4_0, true); else XGB_LAUNCH(SPY_HIP_Q4_0, false); }
+            else { if (mf) XGB_LAUNCH(SPY_HIP_Q8_0, true); else XGB_LAUNCH(SPY_HIP_Q8_0, false); }
+#undef XGB_LAUNCH
             return SPY_LAUNCH_RC();
         }
     }
