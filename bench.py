@@ -135,10 +135,11 @@ def main():
         with open(tpath) as f:
             traffic_db = json.load(f)
 
-    prefill_s = {}
+    prefill_s, firsts = {}, {}
 
     def run_order(order):
         first, prefill_s[order] = prefill(order)
+        firsts[order] = first
         pos = fill
         toks = eng.decode_greedy(first, pos, warmup, use_graph=not args.no_graph)
         pos += warmup
@@ -266,7 +267,7 @@ def main():
         for il in range(cfg.n_layer):                # same cache contents as the GPU run
             ora.k_cache[il][:] = eng.read_buffer("k_cache", il, np.uint16)
             ora.v_cache[il][:] = eng.read_buffer("v_cache", il, np.uint16)
-        tok = np.array([first], np.int32)
+        tok = np.array([firsts[orders[0]]], np.int32)
         ora.forward(tok, fill)                        # untimed warm-up pass (cli.h:78-82)
         t0 = time.perf_counter()
         for i in range(args.cpu_steps):
