@@ -167,7 +167,7 @@ int spy_hip_prompt_attention(void *stream, const void *q16, const void *k_cache,
  * positions after the whole pass this call is a part of (past + T when the pass is not cut into chunks): the host's
  * dot adds the last 1..32 of them one by one and its softmax sum the last n_total % 4 terms.  scratch: device memory
  * of spy_hip_prompt_attention_exact_scratch_size bytes, 256-byte aligned (scores and probabilities of this call).
- * hd must be 128 and n_ctx a multiple of 32 (else SPY_HIP_EUNSUPPORTED). */
+ * hd must be 128, n_ctx a multiple of 32 and past + T at most 8192 (else SPY_HIP_EUNSUPPORTED). */
 size_t spy_hip_prompt_attention_exact_scratch_size(int32_t T, int32_t H, int32_t past);
 int spy_hip_prompt_attention_exact(void *stream, const float *q, const void *k_cache, const void *v_cache, float *out,
                                    int32_t T, int32_t H, int32_t hd, int32_t past, int64_t n_ctx, int32_t n_total, float scale,

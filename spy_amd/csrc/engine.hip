@@ -381,7 +381,7 @@ enum { HEAD_ALL = 0, HEAD_NONE = 1, HEAD_LAST = 2 };     // output head of a pas
 // n_total: the cached positions after the whole call this pass belongs to (= P + T unless the call is cut into chunks)
 static bool exact_attn_ok(const spy_hip_llama *m) {
     const char *e = getenv("SPY_HIP_EXACT_PROMPT_ATTN");
-    return m->hd == 128 && m->desc.n_ctx % 32 == 0 && m->lut && !(e && e[0] == '0');
+    return m->hd == 128 && m->desc.n_ctx % 32 == 0 && m->desc.n_ctx <= 8192 && m->lut && !(e && e[0] == '0');
 }
 static int forward_ops(spy_hip_llama *m, hipStream_t st, const int32_t *tokens_host, int T, int P, float *logits_host, int head, int n_total) {
     const spy_hip_llama_desc &c = m->desc;

@@ -26,11 +26,85 @@ __device__ __forceinline__ xp_half2 xp_pack(float a, float b) {
 }
 
 // ---------------------------------------------------------------- scores
-// One workgroup per (head, 64 query rows); lane = query row, its 128 q values as 64 packed fp16 pairs in registers.
-// A tile of 64 key rows is brought into LDS by the whole workgroup (the next one travels in registers meanwhile); every
-// lane of a wave reads the same key row, which LDS delivers as a broadcast.  A wave takes 16 of the 64 cached positions
-// of a tile; the scores go through LDS as well so that the rows of S are written in whole segments.
-#define XP_QT 64
+// One workgroup per (head, 128 query rows); a lane takes query rows t0 + lane and t0 + 64 + lane, their 2 x 128 q values
+// as packed fp16 pairs in registers.  A tile of 64 key rows is brought into LDS by the whole workgroup; every lane of a
+// wave reads the same key row -- LDS delivers that as a broadcast, but
+// at the cost of a full read, which is why a key row read serves two query rows per lane: with one, the kernel ran at the
+// LDS read rate (16 ds_read_b128 per 160 vector instructions).  A wave takes 16 of the 64 cached positions of a tile; the
+// scores go through LDS as well so that the rows of S are written in whole segments.
+#define XP_QT 128
+#define XP_KSEG 512
+// fma(float(lower halves), c) and fma(float(upper halves), c) of two packed fp16 pairs, written out as instructions: left to
+// itself the compiler folds only one fp16 source into v_fma_mix_f32 and converts the loop-invariant q values to fp32 (once, which
+// doubles the registers they occupy, or inside the loop, which doubles the instructions)
+__device__ __forceinline__ float xp_fma_lo(uint32_t a, uint32_t b, float c) {
+    float r;
+    asm("v_fma_mix_f32 %0, %1, %2, %3 op_sel_hi:[1,1,0]" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+__device__ __forceinline__ float xp_fma_hi(uint32_t a, uint32_t b, float c) {
+    float r;
+    asm("v_fma_mix_f32 %0, %1, %2, %3 op_sel:[1,1,0] op_sel_hi:[1,1,0]" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
+// One key row (in LDS, 16 x 16 bytes) against the two query rows of a lane; the row is taken in its four chunks of 32 elements
+// so that only one chunk of it is in registers at a time.  A: the first query row takes part (else its score is not needed).
+template <bool A>
+__device__ __forceinline__ void xp_dot128_pair(const uint32_t (&qa)[64], const uint32_t (&qb)[64], const uint4 *kr, float &sa, float &sb) {
+    float sum_a[32], sum_b[32];
+    // chunks of 32 elements while i + 32 < 128: accumulator l takes elements l, 32 + l, 64 + l
+#pragma unroll
+    for (int c = 0; c < 3; c++) {
+        uint4 k4[4];
+#pragma unroll
+        for (int v = 0; v < 4; v++) k4[v] = kr[4 * c + v];
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            const uint32_t kw[4] = {k4[v].x, k4[v].y, k4[v].z, k4[v].w};
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int l = 8 * v + 2 * i, qi = 16 * c + 4 * v + i;
+                if (A) {
+                    sum_a[l] = xp_fma_lo(kw[i], qa[qi], c == 0 ? 0.0f : sum_a[l]);
+                    sum_a[l + 1] = xp_fma_hi(kw[i], qa[qi], c == 0 ? 0.0f : sum_a[l + 1]);
+                }
+                sum_b[l] = xp_fma_lo(kw[i], qb[qi], c == 0 ? 0.0f : sum_b[l]);
+                sum_b[l + 1] = xp_fma_hi(kw[i], qb[qi], c == 0 ? 0.0f : sum_b[l + 1]);
+            }
+        }
+    }
+    // the last 32 elements one by one (their products are exact in fp32, so each step is one fma)
+    float tail_a = 0.0f, tail_b = 0.0f;
+    {
+        uint4 k4[4];
+#pragma unroll
+        for (int v = 0; v < 4; v++) k4[v] = kr[12 + v];
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            const uint32_t kw[4] = {k4[v].x, k4[v].y, k4[v].z, k4[v].w};
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int qi = 48 + 4 * v + i;
+                if (A) { tail_a = xp_fma_lo(kw[i], qa[qi], tail_a); tail_a = xp_fma_hi(kw[i], qa[qi], tail_a); }
+                tail_b = xp_fma_lo(kw[i], qb[qi], tail_b);
+                tail_b = xp_fma_hi(kw[i], qb[qi], tail_b);
+            }
+        }
+    }
+    // FP16::block_reduce (vec_util.h:61-71), then result = tail + that sum
+    auto reduce = [](float (&sum)[32]) {
+#pragma unroll
+        for (int l = 0; l < 8; l++) { sum[l] += sum[16 + l]; sum[8 + l] += sum[24 + l]; }
+#pragma unroll
+        for (int l = 0; l < 8; l++) sum[l] += sum[8 + l];
+        const float u0 = sum[0] + sum[4], u1 = sum[1] + sum[5], u2 = sum[2] + sum[6], u3 = sum[3] + sum[7];
+        return (u0 + u1) + (u2 + u3);
+    };
+    if (A) sa = tail_a + reduce(sum_a);
+    sb = tail_b + reduce(sum_b);
+}
+
 __global__ __launch_bounds__(256, 2) void xp_scores_kernel(const float *__restrict__ q, const uint16_t *__restrict__ kc, float *__restrict__ S,
                                                            int T, int H, int P, int64_t s_row) {
     __shared__ float s_tile[XP_QT][65];
@@ -38,84 +112,57 @@ __global__ __launch_bounds__(256, 2) void xp_scores_kernel(const float *__restri
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int t0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * XP_QT, h = blockIdx.y;      // the longest rows first
     const int64_t d = (int64_t)H * 128;
-    const int tq = min(t0 + lane, T - 1);
-    xp_half2 qv[64];
+    // the cached positions are dealt out in segments of XP_KSEG over blockIdx.z, so that the workgroups are of similar length
+    // (one workgroup per 128 query rows would make the longest rows the critical path of the launch)
+    const int kv_end = min(P + min(t0 + XP_QT - 1, T - 1) + 1, ((int)blockIdx.z + 1) * XP_KSEG);       // cached positions that some row of the tile may see, within this segment
+    if ((int)blockIdx.z * XP_KSEG >= kv_end) return;
+    uint32_t qa[64], qb[64];
     {
-        const float4 *qp = (const float4 *)(q + (int64_t)tq * d + (int64_t)h * 128);
+        const float4 *qp = (const float4 *)(q + (int64_t)min(t0 + lane, T - 1) * d + (int64_t)h * 128);
+        const float4 *qp2 = (const float4 *)(q + (int64_t)min(t0 + 64 + lane, T - 1) * d + (int64_t)h * 128);
 #pragma unroll
         for (int i = 0; i < 32; i++) {
-            const float4 f = qp[i];
-            qv[2 * i] = xp_pack(f.x, f.y);
-            qv[2 * i + 1] = xp_pack(f.z, f.w);
+            const float4 f = qp[i], f2 = qp2[i];
+            qa[2 * i] = __builtin_bit_cast(uint32_t, xp_pack(f.x, f.y));
+            qa[2 * i + 1] = __builtin_bit_cast(uint32_t, xp_pack(f.z, f.w));
+            qb[2 * i] = __builtin_bit_cast(uint32_t, xp_pack(f2.x, f2.y));
+            qb[2 * i + 1] = __builtin_bit_cast(uint32_t, xp_pack(f2.z, f2.w));
         }
     }
-    const int kv_end = P + min(t0 + XP_QT - 1, T - 1) + 1;       // cached positions that some row of the tile may see
+    const int kv_end_a = P + min(t0 + 63, T - 1) + 1;            // cached positions that some row of the tile's first half may see
     // staging: thread -> key row tid / 4 of the tile, 64 of its 256 bytes
     const int st_row = threadIdx.x >> 2, st_q = (threadIdx.x & 3) * 4;
     uint4 kst0, kst1, kst2, kst3;
 #define XP_FETCH_K(kv_first) do { \
         const uint4 *src_ = (const uint4 *)(kc + (int64_t)min((kv_first) + st_row, kv_end - 1) * d + (int64_t)h * 128) + st_q; \
         kst0 = src_[0]; kst1 = src_[1]; kst2 = src_[2]; kst3 = src_[3]; } while (0)
-    XP_FETCH_K(0);
-    for (int kv0 = 0; kv0 < kv_end; kv0 += 64) {
+    for (int kv0 = (int)blockIdx.z * XP_KSEG; kv0 < kv_end; kv0 += 64) {
+        // (no key tile travelling in registers during the dots: with 2 x 64 registers of q values and 2 x 32 accumulators there is
+        // no room for it; the second workgroup of the compute unit covers the wait)
+        XP_FETCH_K(kv0);
         s_k[st_row][st_q] = kst0; s_k[st_row][st_q + 1] = kst1; s_k[st_row][st_q + 2] = kst2; s_k[st_row][st_q + 3] = kst3;
         __syncthreads();
-        if (kv0 + 64 < kv_end) XP_FETCH_K(kv0 + 64);
-#pragma unroll 2
+        const bool first_half = kv0 < kv_end_a;                   // else the whole key tile lies behind the mask of query rows t0 .. t0 + 63
+#pragma unroll 1
         for (int j = 0; j < 16; j++) {
             const int kvl = wave * 16 + j;
-            float score = 0.0f;
+            float sa = 0.0f, sb = 0.0f;
             if (kv0 + kvl < kv_end) {
-                const uint4 *kr = s_k[kvl];
-                float sum[32];
-                // chunks of 32 elements while i + 32 < 128: accumulator l takes elements l, 32 + l, 64 + l
-#pragma unroll
-                for (int c = 0; c < 3; c++)
-#pragma unroll
-                    for (int v = 0; v < 4; v++) {
-                        const uint4 k4 = kr[4 * c + v];
-                        const uint32_t kw[4] = {k4.x, k4.y, k4.z, k4.w};
-#pragma unroll
-                        for (int i = 0; i < 4; i++) {
-                            const xp_half2 k2 = __builtin_bit_cast(xp_half2, kw[i]), q2 = qv[16 * c + 4 * v + i];
-                            const int l = 8 * v + 2 * i;
-                            sum[l] = fmaf((float)k2.x, (float)q2.x, c == 0 ? 0.0f : sum[l]);
-                            sum[l + 1] = fmaf((float)k2.y, (float)q2.y, c == 0 ? 0.0f : sum[l + 1]);
-                        }
-                    }
-                // FP16::block_reduce (vec_util.h:61-71)
-#pragma unroll
-                for (int l = 0; l < 8; l++) { sum[l] += sum[16 + l]; sum[8 + l] += sum[24 + l]; }
-#pragma unroll
-                for (int l = 0; l < 8; l++) sum[l] += sum[8 + l];
-                const float u0 = sum[0] + sum[4], u1 = sum[1] + sum[5], u2 = sum[2] + sum[6], u3 = sum[3] + sum[7];
-                const float simd = (u0 + u1) + (u2 + u3);
-                // the last 32 elements one by one (their products are exact in fp32, so each step is one fma)
-                float tail = 0.0f;
-#pragma unroll
-                for (int v = 0; v < 4; v++) {
-                    const uint4 k4 = kr[12 + v];
-                    const uint32_t kw[4] = {k4.x, k4.y, k4.z, k4.w};
-#pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        const xp_half2 k2 = __builtin_bit_cast(xp_half2, kw[i]), q2 = qv[48 + 4 * v + i];
-                        tail = fmaf((float)k2.x, (float)q2.x, tail);
-                        tail = fmaf((float)k2.y, (float)q2.y, tail);
-                    }
-                }
-                score = tail + simd;
+                if (first_half) xp_dot128_pair<true>(qa, qb, s_k[kvl], sa, sb);
+                else xp_dot128_pair<false>(qa, qb, s_k[kvl], sa, sb);
             }
-            s_tile[lane][kvl] = score;
+            s_tile[lane][kvl] = sa;
+            s_tile[64 + lane][kvl] = sb;
         }
         __syncthreads();
         {
-            const int row = threadIdx.x >> 2, seg = threadIdx.x & 3;
-            if (t0 + row < T) {
-                float4 *out = (float4 *)(S + ((int64_t)h * T + t0 + row) * s_row + kv0 + seg * 16);
+            const int row = threadIdx.x >> 1, seg = threadIdx.x & 1;
+            if (t0 + row < T && (row >= 64 || first_half)) {
+                float4 *out = (float4 *)(S + ((int64_t)h * T + t0 + row) * s_row + kv0 + seg * 32);
 #pragma unroll
-                for (int i = 0; i < 4; i++)
-                    out[i] = make_float4(s_tile[row][seg * 16 + 4 * i], s_tile[row][seg * 16 + 4 * i + 1], s_tile[row][seg * 16 + 4 * i + 2],
-                                         s_tile[row][seg * 16 + 4 * i + 3]);
+                for (int i = 0; i < 8; i++)
+                    out[i] = make_float4(s_tile[row][seg * 32 + 4 * i], s_tile[row][seg * 32 + 4 * i + 1], s_tile[row][seg * 32 + 4 * i + 2],
+                                         s_tile[row][seg * 32 + 4 * i + 3]);
             }
         }
         // the next tile's key rows go into s_k at the top of the loop: every wave is past its reads of s_k once it has passed the
@@ -125,56 +172,85 @@ __global__ __launch_bounds__(256, 2) void xp_scores_kernel(const float *__restri
 }
 
 // ---------------------------------------------------------------- softmax
-// One workgroup per (head, query row).  The row is kept in S between the steps as the host keeps it in dst; L = the
-// positions the row may see.  The probabilities leave as fp16 (the first step of the KQV MatMul, mat.cpp:37), followed
-// by zeros up to the end of the 32-row tile's last chunk, which the product kernel reads.
-__global__ __launch_bounds__(256) void xp_softmax_kernel(float *__restrict__ S, uint16_t *__restrict__ P16, const float *__restrict__ lut, int T, int P,
+// One workgroup per (head, query row); L = the positions the row may see.  A thread keeps its share of the row in registers
+// (groups of four consecutive elements, the unit of the host's sum), so the row is read once and written once.  The
+// probabilities leave as fp16 (the first step of the KQV MatMul, mat.cpp:37), followed by zeros up to the end of the 32-row
+// tile's last chunk, which the product kernel reads.
+#define XP_SM_R 8          // groups per thread: rows of up to 8192 positions
+__global__ __launch_bounds__(256) void xp_softmax_kernel(const float *__restrict__ S, uint16_t *__restrict__ P16, const float *__restrict__ lut, int T, int P,
                                                          int64_t s_row, int n_total, float scale) {
-    __shared__ float s_grp[1024];
-    __shared__ float s_part[4];
+    __shared__ __align__(16) float s_grp[256 * XP_SM_R];
+    __shared__ float s_part[4], s_rem[4];
     __shared__ float s_out;
     const int t = blockIdx.x, h = blockIdx.y;
-    float *s = S + ((int64_t)h * T + t) * s_row;
+    const float4 *s4 = (const float4 *)(S + ((int64_t)h * T + t) * s_row);
     uint16_t *p = P16 + ((int64_t)h * T + t) * s_row;
-    const int L = P + t + 1;
+    const int L = P + t + 1, ng_row = (L + 3) / 4;       // groups that hold an element of the row
+    float v[XP_SM_R][4];
     float mx = -INFINITY;
-    for (int i = threadIdx.x; i < L; i += 256) {
-        float v = s[i] + 0.0f;                 // + the mask value of an allowed position
-        v = v * scale;
-        s[i] = v;
-        mx = fmaxf(mx, v);
+#pragma unroll
+    for (int r = 0; r < XP_SM_R; r++) {
+        const int g = threadIdx.x + 256 * r;
+        if (g < ng_row) {
+            const float4 f = s4[g];
+            const float e[4] = {f.x, f.y, f.z, f.w};
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                float x = e[k] + 0.0f;                   // + the mask value of an allowed position
+                x = x * scale;
+                v[r][k] = x;
+                if (4 * g + k < L) mx = fmaxf(mx, x);
+            }
+        }
     }
     mx = wave_max(mx);
     if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = mx;
     __syncthreads();
     mx = fmaxf(fmaxf(s_part[0], s_part[1]), fmaxf(s_part[2], s_part[3]));
-    const int L4 = (L + 3) & ~3;
-    for (int i = threadIdx.x; i < L4; i += 256) s[i] = i < L ? lut[f2h(s[i] - mx)] : 0.0f;
-    __syncthreads();
     // std::reduce in libstdc++: groups of four as init + ((a0 + a1) + (a2 + a3)) over the first n_total / 4 * 4 elements, the rest one
     // by one; groups and elements past L are zeros and leave the sum as it is
-    const int ngrp = min(n_total / 4, L4 / 4);
-    float init = 0.0f;
-    for (int g0 = 0; g0 < ngrp; g0 += 1024) {
-        const int cnt = min(1024, ngrp - g0);
-        for (int g = threadIdx.x; g < cnt; g += 256) {
-            const float4 a = *(const float4 *)(s + 4 * (g0 + g));
-            const float v1 = a.x + a.y, v2 = a.z + a.w;
-            s_grp[g] = v1 + v2;
+    const int ng_sum = min(n_total / 4, ng_row);
+#pragma unroll
+    for (int r = 0; r < XP_SM_R; r++) {
+        const int g = threadIdx.x + 256 * r;
+        if (g < ng_row) {
+#pragma unroll
+            for (int k = 0; k < 4; k++) v[r][k] = 4 * g + k < L ? lut[f2h(v[r][k] - mx)] : 0.0f;
+            const float v1 = v[r][0] + v[r][1], v2 = v[r][2] + v[r][3];
+            if (g < ng_sum) s_grp[g] = v1 + v2;
+            else {                                       // the group that n_total cuts short: its elements are added one by one
+#pragma unroll
+                for (int k = 0; k < 4; k++) s_rem[k] = v[r][k];
+            }
         }
-        __syncthreads();
-        if (threadIdx.x == 0)
-            for (int g = 0; g < cnt; g++) init = init + s_grp[g];
-        __syncthreads();
     }
+    __syncthreads();
     if (threadIdx.x == 0) {
-        for (int i = n_total / 4 * 4; i < min(n_total, L); i++) init = init + s[i];
+        float init = 0.0f;
+        int g = 0;
+        for (; g + 4 <= ng_sum; g += 4) {
+            const float4 a = *(const float4 *)&s_grp[g];
+            init = init + a.x; init = init + a.y; init = init + a.z; init = init + a.w;
+        }
+        for (; g < ng_sum; g++) init = init + s_grp[g];
+        for (int i = n_total / 4 * 4; i < min(n_total, L); i++) init = init + s_rem[i & 3];
         s_out = init;
     }
     __syncthreads();
     const float inv = 1.0f / s_out;
-    const int zend = (int)min((int64_t)((P + (t | 31) + 1 + 31) & ~31), s_row);
-    for (int i = threadIdx.x; i < zend; i += 256) p[i] = i < L ? f2h(s[i] * inv) : (uint16_t)0;
+    const int zend = (int)min((int64_t)((P + (t | 31) + 1 + 31) & ~31), s_row);       // a multiple of 32
+    uint2 *p4 = (uint2 *)p;
+#pragma unroll
+    for (int r = 0; r < XP_SM_R; r++) {
+        const int g = threadIdx.x + 256 * r;
+        if (g < ng_row) {
+            uint16_t o[4];
+#pragma unroll
+            for (int k = 0; k < 4; k++) o[k] = 4 * g + k < L ? f2h(v[r][k] * inv) : (uint16_t)0;
+            p4[g] = make_uint2((uint32_t)o[0] | ((uint32_t)o[1] << 16), (uint32_t)o[2] | ((uint32_t)o[3] << 16));
+        }
+    }
+    for (int g = ng_row + threadIdx.x; g < zend / 4; g += 256) p4[g] = make_uint2(0, 0);
 }
 
 // ---------------------------------------------------------------- product with V^T
@@ -198,8 +274,9 @@ __global__ __launch_bounds__(256, 2) void xp_pv_kernel(const uint16_t *__restric
     const uint16_t *vrow[4];
 #pragma unroll
     for (int j = 0; j < 4; j++) vrow[j] = vt + ((int64_t)h * 128 + dd0 + j) * C + l;
-    // staging of the probabilities: thread -> query row tid / 8, sixteen positions
-    const int st_t = threadIdx.x >> 3, st_k = (threadIdx.x & 7) * 16;
+    // staging of the probabilities: thread -> query row tid % 32, sixteen positions; neighbouring lanes write neighbouring
+    // query rows of one position, i.e. neighbouring LDS words (the other way round, 64 lanes would meet in four banks)
+    const int st_t = threadIdx.x & 31, st_k = (threadIdx.x >> 5) * 16;
     const uint16_t *prow = P16 + ((int64_t)h * T + min(t0 + st_t, T - 1)) * p_row + st_k;
     float acc[4][32];
 #pragma unroll
@@ -329,9 +406,10 @@ int64_t spy_exact_prompt_attn_row(int64_t n_kv) { return (n_kv + 127) & ~(int64_
 int spy_exact_prompt_attn(hipStream_t st, const float *q, const uint16_t *kc, const uint16_t *vt, float *S, uint16_t *P16, float *out, const float *lut,
                           int T, int H, int P, int64_t C, int n_total, float scale) {
     if (T <= 0 || H <= 0 || H > 65535 || P < 0 || (int64_t)P + T > C || n_total < P + T || n_total > C || C % 32) return SPY_HIP_EINVAL;
+    if ((int64_t)P + T > 1024 * XP_SM_R) return SPY_HIP_EUNSUPPORTED;      // the softmax kernel keeps a row in the registers of 256 threads
     if (((uintptr_t)q & 15) || ((uintptr_t)kc & 15) || ((uintptr_t)S & 15) || ((uintptr_t)P16 & 7) || ((uintptr_t)out & 15)) return SPY_HIP_EINVAL;
     const int64_t s_row = spy_exact_prompt_attn_row((int64_t)P + T);
-    xp_scores_kernel<<<dim3((unsigned)((T + XP_QT - 1) / XP_QT), (unsigned)H), dim3(256), 0, st>>>(q, kc, S, T, H, P, s_row);
+    xp_scores_kernel<<<dim3((unsigned)((T + XP_QT - 1) / XP_QT), (unsigned)H, (unsigned)((P + T + XP_KSEG - 1) / XP_KSEG)), dim3(256), 0, st>>>(q, kc, S, T, H, P, s_row);
     if (hipGetLastError() != hipSuccess) return SPY_HIP_EINVAL;
     xp_softmax_kernel<<<dim3((unsigned)T, (unsigned)H), dim3(256), 0, st>>>(S, P16, lut, T, P, s_row, n_total, scale);
     if (hipGetLastError() != hipSuccess) return SPY_HIP_EINVAL;
