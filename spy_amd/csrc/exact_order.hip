@@ -466,6 +466,28 @@ __global__ __launch_bounds__(256) void exact_dots8_kernel(xdesc w, const uint8_t
 #define XGB_TILE 64
 #define XGB_KB 4          // blocks per stage
 typedef int xgb_v4i __attribute__((ext_vector_type(4)));
+typedef float xgb_v4f __attribute__((ext_vector_type(4)));
+// The four matrix instructions of one element word: the A operand (weight words of rows 4g + j) is taken from lane group `abid`
+// for all sixteen groups.  abid has to be an immediate, hence the switch over constants (the callers' loops are unrolled).
+__device__ __forceinline__ void xgb_mfma_word(xgb_v4i (&out)[4], const uint4 &wq4, uint32_t xq, const xgb_v4i &bias, int abid) {
+#define XGB_CASE(n) case n: \
+        out[0] = __builtin_amdgcn_mfma_i32_4x4x4i8((int)wq4.x, (int)xq, bias, 4, n, 0); out[1] = __builtin_amdgcn_mfma_i32_4x4x4i8((int)wq4.y, (int)xq, bias, 4, n, 0); \
+        out[2] = __builtin_amdgcn_mfma_i32_4x4x4i8((int)wq4.z, (int)xq, bias, 4, n, 0); out[3] = __builtin_amdgcn_mfma_i32_4x4x4i8((int)wq4.w, (int)xq, bias, 4, n, 0); break;
+    switch (abid) {
+        XGB_CASE(0) XGB_CASE(1) XGB_CASE(2) XGB_CASE(3) XGB_CASE(4) XGB_CASE(5) XGB_CASE(6) XGB_CASE(7)
+        XGB_CASE(8) XGB_CASE(9) XGB_CASE(10) XGB_CASE(11) XGB_CASE(12) XGB_CASE(13) XGB_CASE(14) XGB_CASE(15)
+    }
+#undef XGB_CASE
+}
+// D[g][i] = d_w(row 4g + i) * d_x(this lane's activation row) for block kb of a pair: lane group 4 * kb + g supplies the four d_w
+template <int>
+__device__ __forceinline__ void xgb_mfma_scale(xgb_v4f (&D)[4], float wd, float xd, const xgb_v4f &zero4, int kb) {
+#define XGB_CASE(n) case n: \
+        D[0] = __builtin_amdgcn_mfma_f32_4x4x1f32(wd, xd, zero4, 4, 4 * n, 0); D[1] = __builtin_amdgcn_mfma_f32_4x4x1f32(wd, xd, zero4, 4, 4 * n + 1, 0); \
+        D[2] = __builtin_amdgcn_mfma_f32_4x4x1f32(wd, xd, zero4, 4, 4 * n + 2, 0); D[3] = __builtin_amdgcn_mfma_f32_4x4x1f32(wd, xd, zero4, 4, 4 * n + 3, 0); break;
+    switch (kb) { XGB_CASE(0) XGB_CASE(1) }
+#undef XGB_CASE
+}
 // MF = true: the integer sums come from the matrix cores instead: v_mfma_i32_4x4x4_16b_i8 multiplies, in each group of four
 // lanes, a 4 x 4 byte matrix (lane j supplies row j) by another (lane j supplies column j) and leaves column j of the 4 x 4
 // result in lane j -- sixteen four-element dot products per group, exactly one accumulator's share of a block.  A wave then
@@ -476,7 +498,8 @@ template <int WT, bool MF>
 __global__ __launch_bounds__(256, 2) void exact_gemm8_kernel(const uint8_t *__restrict__ w, int64_t w_row, int64_t ne01, int64_t nb,
                                                               const uint8_t *__restrict__ xm, int64_t x_row, int64_t ne11,
                                                               float *__restrict__ dst, int64_t d_row) {
-    __shared__ __align__(16) uint32_t s_wq[2][XGB_KB][8][XGB_TILE];
+    constexpr int WPL = MF ? XGB_TILE + 4 : XGB_TILE;              // words per weight plane: MF reads 16 planes at once, the padding spreads them over the banks
+    __shared__ __align__(16) uint32_t s_wq[2][XGB_KB][8][WPL];
     __shared__ __align__(16) uint32_t s_xq[2][XGB_KB][8][XGB_TILE];
     __shared__ __align__(16) float s_wd[2][XGB_KB][XGB_TILE];
     __shared__ __align__(16) float s_xd[2][XGB_KB][XGB_TILE];
@@ -526,15 +549,15 @@ __global__ __launch_bounds__(256, 2) void exact_gemm8_kernel(const uint8_t *__re
         } else {
             // Q8_0 pair: block 0 = scale in the low half of g[0] and 32 quant bytes from byte 2, block 1 = scale in the high half
             // of g[8] and quants g[9..16]
-            uint32_t (*sq)[8][XGB_TILE] = ld_w ? s_wq[buf] : s_xq[buf];
             float (*sd)[XGB_TILE] = ld_w ? s_wd[buf] : s_xd[buf];
             const int k0 = 2 * ld_pair;
             sd[k0][ld_row] = h2f_tab((uint16_t)(g[0] & 0xFFFFu));
             sd[k0 + 1][ld_row] = h2f_tab((uint16_t)(g[8] >> 16));
 #pragma unroll
             for (int k = 0; k < 8; k++) {
-                sq[k0][k][ld_slot] = __builtin_amdgcn_alignbit(g[k + 1], g[k], 16);
-                sq[k0 + 1][k][ld_slot] = g[9 + k];
+                const uint32_t q0 = __builtin_amdgcn_alignbit(g[k + 1], g[k], 16), q1 = g[9 + k];
+                if (ld_w) { s_wq[buf][k0][k][ld_slot] = q0; s_wq[buf][k0 + 1][k][ld_slot] = q1; }
+                else { s_xq[buf][k0][k][ld_slot] = q0; s_xq[buf][k0 + 1][k][ld_slot] = q1; }
             }
         }
     };
@@ -555,39 +578,42 @@ __global__ __launch_bounds__(256, 2) void exact_gemm8_kernel(const uint8_t *__re
         const int buf = (int)(s & 1);
         if (s + 1 < nstage) fetch(s + 1);
         if constexpr (MF) {
-            // acc[g][i]: weight row 16 * wave + 4g + i against this lane's activation row
+            // acc[g][i]: weight row 16 * wave + 4g + i against this lane's activation row.  Every group of four lanes would feed the
+            // same weight words to its matrix instructions; instead each group reads the words of ANOTHER (block, element word) pair
+            // -- one 16-byte read per lane covers two blocks -- and the instruction is told which group's words to use for all sixteen
+            // (cbsz = 4, abid = the group).  The scale products d_w * d_x come the same way from v_mfma_f32_4x4x1_16b_f32 (one product
+            // per output, rounded once: the bits of the vector multiply).
             const xgb_v4i bias = {0x4B400000, 0x4B400000, 0x4B400000, 0x4B400000};
+            const xgb_v4f zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
+            const int grp = bj >> 2;                                                  // this lane's group of four, 0..15
 #pragma unroll 1
-            for (int kb = 0; kb < XGB_KB; kb++) {
-                const float xd = s_xd[buf][kb][bj];
-                float D[4][4];
+            for (int half = 0; half < XGB_KB / 2; half++) {
+                const float wdreg = s_wd[buf][2 * half + ((grp >> 2) & 1)][16 * wv + 4 * (grp & 3) + jj];    // group 4 * (block & 1) + g holds the scales of rows 4g + j
+                const uint4 wq4 = *(const uint4 *)&s_wq[buf][2 * half + (grp >> 3)][grp & 7][jj * 16 + 4 * wv];      // group 8 * (block & 1) + e: rows 4g + j, g = 0..3
 #pragma unroll
-                for (int gq = 0; gq < 4; gq++) {
-                    const float4 wd4 = *(const float4 *)&s_wd[buf][kb][16 * wv + 4 * gq];
-                    D[gq][0] = wd4.x * xd; D[gq][1] = wd4.y * xd; D[gq][2] = wd4.z * xd; D[gq][3] = wd4.w * xd;
-                }
-                // the four matrix instructions of word e + 1 are issued before the vector work on the results of word e
-                xgb_v4i p[2][4];
-                auto issue = [&](int e, xgb_v4i (&out)[4]) {
-                    const uint4 wq4 = *(const uint4 *)&s_wq[buf][kb][e][jj * 16 + 4 * wv];      // rows 16 * wave + 4g + j, g = 0..3
-                    const uint32_t xq = s_xq[buf][kb][e][bj];
-                    out[0] = __builtin_amdgcn_mfma_i32_4x4x4i8((int)wq4.x, (int)xq, bias, 0, 0, 0);
-                    out[1] = __builtin_amdgcn_mfma_i32_4x4x4i8((int)wq4.y, (int)xq, bias, 0, 0, 0);
-                    out[2] = __builtin_amdgcn_mfma_i32_4x4x4i8((int)wq4.z, (int)xq, bias, 0, 0, 0);
-                    out[3] = __builtin_amdgcn_mfma_i32_4x4x4i8((int)wq4.w, (int)xq, bias, 0, 0, 0);
-                };
-                issue(0, p[0]);
+                for (int kb2 = 0; kb2 < 2; kb2++) {
+                    const int kb = 2 * half + kb2;
+                    const float xd = s_xd[buf][kb][bj];
+                    xgb_v4f D[4];
+                    xgb_mfma_scale<0>(D, wdreg, xd, zero4, kb2);
+                    uint32_t xq[8];
 #pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    if (e + 1 < 8) issue(e + 1, p[(e + 1) & 1]);
-                    const int a = WT == SPY_HIP_Q4_0 ? ((e + 4) & 7) : e;
+                    for (int e = 0; e < 8; e++) xq[e] = s_xq[buf][kb][e][bj];
+                    // the four matrix instructions of word e + 1 are issued before the vector work on the results of word e
+                    xgb_v4i p[2][4];
+                    xgb_mfma_word(p[0], wq4, xq[0], bias, kb2 * 8 + 0);
 #pragma unroll
-                    for (int gq = 0; gq < 4; gq++) {
-                        const xgb_v4i r = p[e & 1][gq];
-                        acc[gq][0][a] = fmaf(D[gq][0], __int_as_float(r.x) - 12582912.0f, acc[gq][0][a]);
-                        acc[gq][1][a] = fmaf(D[gq][1], __int_as_float(r.y) - 12582912.0f, acc[gq][1][a]);
-                        acc[gq][2][a] = fmaf(D[gq][2], __int_as_float(r.z) - 12582912.0f, acc[gq][2][a]);
-                        acc[gq][3][a] = fmaf(D[gq][3], __int_as_float(r.w) - 12582912.0f, acc[gq][3][a]);
+                    for (int e = 0; e < 8; e++) {
+                        if (e + 1 < 8) xgb_mfma_word(p[(e + 1) & 1], wq4, xq[e + 1], bias, kb2 * 8 + e + 1);
+                        const int a = WT == SPY_HIP_Q4_0 ? ((e + 4) & 7) : e;
+#pragma unroll
+                        for (int gq = 0; gq < 4; gq++) {
+                            const xgb_v4i r = p[e & 1][gq];
+                            acc[gq][0][a] = fmaf(D[gq].x, __int_as_float(r.x) - 12582912.0f, acc[gq][0][a]);
+                            acc[gq][1][a] = fmaf(D[gq].y, __int_as_float(r.y) - 12582912.0f, acc[gq][1][a]);
+                            acc[gq][2][a] = fmaf(D[gq].z, __int_as_float(r.z) - 12582912.0f, acc[gq][2][a]);
+                            acc[gq][3][a] = fmaf(D[gq].w, __int_as_float(r.w) - 12582912.0f, acc[gq][3][a]);
+                        }
                     }
                 }
             }
