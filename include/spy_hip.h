@@ -100,8 +100,10 @@ int spy_hip_op_silu(void *stream, const spy_hip_tensor *x, const spy_hip_tensor 
  * product can take them without a conversion pass */
 int spy_hip_op_softmax(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *mask, const spy_hip_tensor *dst, float scale);
 /* Rope -- OperatorRopeImpl::execute (non-linear.cpp:270-371); fields of RopeParam
- * (orchestration/include/operator/non-linear.h:191-207).  Supported: mode None/Norm (-1/0) with
- * extend_factor == 0 and xpos_base == 0 (the LLaMA defaults); anything else -> EUNSUPPORTED. */
+ * (orchestration/include/operator/non-linear.h:191-207).  Supported: mode None/Norm (-1/0), including
+ * extend_factor != 0 (rope_yarn, :242-260: as written its ramp is 0, so the angle stays the interpolated one and the
+ * magnitude is multiplied by 1 + 0.1 ln(1 / freq_scale)) and xpos_base != 0 (zeta, :353-354).  GLM and Neox (the
+ * latter aborts in the reference) -> EUNSUPPORTED. */
 typedef struct spy_hip_rope_param {
     int32_t mode, num_past, num_dim, num_context, num_origin_context;
     float   freq_base, freq_scale, extend_factor, attention_factor, beta_fast, beta_slow, xpos_base;

@@ -168,22 +168,28 @@ __global__ __launch_bounds__(256) void exact_softmax_kernel(xdesc x, xdesc mask,
 }
 
 // Rope (non-linear.cpp:270-371), default branch; tab = cos, sin per pair, from the host: one row per token of
-// this call (pos == nullptr) or one row per position 0 .. npos-1, the token's position read here
+// this call (pos == nullptr) or one row per position 0 .. npos-1, the token's position read here.  zeta: the xpos
+// factors of the call's tokens (one per pair, after the cos / sin of a row: rows of ne0 + ne0 / 2 floats), or none.
 __global__ __launch_bounds__(64) void exact_rope_kernel(xdesc x, xdesc y, const float *__restrict__ tab, const uint8_t *__restrict__ pos, int64_t pos_stride,
-                                                        int64_t npos, int *err) {
+                                                        int64_t npos, int *err, int zeta) {
     const int64_t i1 = blockIdx.x, i2 = blockIdx.y, i3 = blockIdx.z;
     const int64_t ne0 = y.ne[0];
+    const int64_t tab_row = zeta ? ne0 + ne0 / 2 : ne0;
     int64_t row = i2;
     if (pos) {
         row = *(const int32_t *)(pos + i2 * pos_stride);
         if (row < 0 || row >= npos) { if (threadIdx.x == 0) *err = 1; return; }      // beyond the context the table was built for
     }
     for (int64_t i0 = 2 * threadIdx.x; i0 < ne0; i0 += 128) {
-        const float c = tab[row * ne0 + i0], s = tab[row * ne0 + i0 + 1];
+        const float c = tab[row * tab_row + i0], s = tab[row * tab_row + i0 + 1];
         const float *sp = (const float *)xat(x, i0, i1, i2, i3);
         float *dp = (float *)xat(y, i0, i1, i2, i3);
         const float x0 = sp[0], x1 = sp[1];
-        const float a = x0 * c, b = x1 * s, e = x0 * s, f = x1 * c;
+        float a = x0 * c, b = x1 * s, e = x0 * s, f = x1 * c;
+        if (zeta) {
+            const float z = tab[row * tab_row + ne0 + i0 / 2];
+            a = a * z; b = b * z; e = e * z; f = f * z;
+        }
         dp[0] = a - b;
         dp[1] = e + f;
     }
@@ -819,14 +825,27 @@ int spy_exact_softmax(hipStream_t st, const spy_hip_tensor *x, const spy_hip_ten
 }
 
 // cos / sin of one token: theta starts at the position and is multiplied by theta_scale once per pair
-// (non-linear.cpp:304-309), cosf / sinf from the host's libm as in the reference
-static void rope_row(float *row, int32_t position, int64_t ne0, float theta_scale, const spy_hip_rope_param *p) {
+// (non-linear.cpp:304-309), cosf / sinf from the host's libm as in the reference.  extend_factor != 0 (rope_yarn,
+// :247-260): the ramp is 1 - std::clamp(0.0F, 1.0F, y), which clamps the VALUE 0 into [1, y] and is therefore 0; the mix
+// and the magnitude correction are evaluated as written.  zeta (xpos, :353-354), when asked for, follows the pairs.
+static void rope_row(float *row, int32_t position, int64_t ne0, float theta_scale, const spy_hip_rope_param *p, bool zeta) {
     float theta = (float)position;
     for (int64_t i0 = 0; i0 < ne0; i0 += 2) {
-        const float ang = p->freq_scale * theta;
-        row[i0] = cosf(ang) * p->attention_factor;
-        row[i0 + 1] = sinf(ang) * p->attention_factor;
+        const float theta_interp = p->freq_scale * theta;
+        float ang = theta_interp, mscale = p->attention_factor;
+        if (p->extend_factor != 0.0f) {
+            const float ramp_mix = (1.0f - 1.0f) * p->extend_factor;
+            ang = theta_interp * (1 - ramp_mix) + theta * ramp_mix;
+            mscale *= 1.0f + 0.1f * logf(1.0f / p->freq_scale);
+        }
+        row[i0] = cosf(ang) * mscale;
+        row[i0 + 1] = sinf(ang) * mscale;
         theta *= theta_scale;
+        if (zeta) {
+            float z = powf(((float)i0 + 0.4f * (float)ne0) / (1.4f * (float)ne0), (float)position / p->xpos_base);
+            if (p->xpos_down) z = 1.0f / z;
+            row[ne0 + i0 / 2] = z;
+        }
     }
 }
 
@@ -840,11 +859,12 @@ int spy_exact_rope(hipStream_t st, const spy_hip_tensor *x, const spy_hip_tensor
     // then looks its token's position up itself and the call needs no copy and no wait.
     static struct { int64_t npos, ne0; float freq_base, freq_scale, factor; int32_t num_dim; float *dev; } cache = {0, 0, 0, 0, 0, 0, nullptr};
     const int64_t npos = p->num_context;
-    if (npos > 0 && npos * ne0 * 4 <= (64ll << 20) && spy_hip_err_flag_ptr()) {
+    const bool zeta = p->xpos_base != 0.0f;
+    if (npos > 0 && npos * ne0 * 4 <= (64ll << 20) && spy_hip_err_flag_ptr() && !zeta && p->extend_factor == 0.0f) {
         if (!cache.dev || cache.npos != npos || cache.ne0 != ne0 || cache.freq_base != p->freq_base || cache.freq_scale != p->freq_scale ||
             cache.factor != p->attention_factor || cache.num_dim != p->num_dim) {
             std::vector<float> tab((size_t)(npos * ne0));
-            for (int64_t q = 0; q < npos; q++) rope_row(&tab[(size_t)(q * ne0)], (int32_t)q, ne0, theta_scale, p);
+            for (int64_t q = 0; q < npos; q++) rope_row(&tab[(size_t)(q * ne0)], (int32_t)q, ne0, theta_scale, p, false);
             if (cache.dev) { (void)hipDeviceSynchronize(); (void)hipFree(cache.dev); cache.dev = nullptr; }
             hipError_t e = hipMalloc((void **)&cache.dev, tab.size() * sizeof(float));
             if (e != hipSuccess) { cache.dev = nullptr; return (int)e; }
@@ -853,7 +873,7 @@ int spy_exact_rope(hipStream_t st, const spy_hip_tensor *x, const spy_hip_tensor
             cache.npos = npos; cache.ne0 = ne0; cache.freq_base = p->freq_base; cache.freq_scale = p->freq_scale;
             cache.factor = p->attention_factor; cache.num_dim = p->num_dim;
         }
-        exact_rope_kernel<<<grid, dim3(64), 0, st>>>(mkx(x), mkx(dst), cache.dev, (const uint8_t *)pos->data, pos->nb[0], npos, spy_hip_err_flag_ptr());
+        exact_rope_kernel<<<grid, dim3(64), 0, st>>>(mkx(x), mkx(dst), cache.dev, (const uint8_t *)pos->data, pos->nb[0], npos, spy_hip_err_flag_ptr(), 0);
         return SPY_LAUNCH_RC();
     }
     // No context length given: wait for the stream, read the positions back and upload the rows of this call's tokens.
@@ -863,8 +883,9 @@ int spy_exact_rope(hipStream_t st, const spy_hip_tensor *x, const spy_hip_tensor
     if (pos->nb[0] == 4) e = hipMemcpy(hp.data(), pos->data, (size_t)ne2 * 4, hipMemcpyDeviceToHost);
     else e = hipMemcpy2D(hp.data(), 4, pos->data, (size_t)pos->nb[0], 4, (size_t)ne2, hipMemcpyDeviceToHost);
     if (e != hipSuccess) return (int)e;
-    std::vector<float> tab((size_t)(ne2 * ne0));
-    for (int64_t i2 = 0; i2 < ne2; i2++) rope_row(&tab[(size_t)(i2 * ne0)], hp[(size_t)i2], ne0, theta_scale, p);
+    const int64_t tab_row = zeta ? ne0 + ne0 / 2 : ne0;
+    std::vector<float> tab((size_t)(ne2 * tab_row));
+    for (int64_t i2 = 0; i2 < ne2; i2++) rope_row(&tab[(size_t)(i2 * tab_row)], hp[(size_t)i2], ne0, theta_scale, p, zeta);
     const size_t need = tab.size() * sizeof(float);
     if (need > g_rope_cap) {
         if (g_rope) { (void)hipDeviceSynchronize(); (void)hipFree(g_rope); g_rope = nullptr; g_rope_cap = 0; }
@@ -874,7 +895,7 @@ int spy_exact_rope(hipStream_t st, const spy_hip_tensor *x, const spy_hip_tensor
     }
     e = hipMemcpy(g_rope, tab.data(), need, hipMemcpyHostToDevice);
     if (e != hipSuccess) return (int)e;
-    exact_rope_kernel<<<grid, dim3(64), 0, st>>>(mkx(x), mkx(dst), g_rope, nullptr, 0, 0, nullptr);
+    exact_rope_kernel<<<grid, dim3(64), 0, st>>>(mkx(x), mkx(dst), g_rope, nullptr, 0, 0, nullptr, zeta ? 1 : 0);
     if (hipGetLastError() != hipSuccess) return SPY_HIP_EINVAL;
     return (int)hipStreamSynchronize(st);      // the table is overwritten by the next call
 }

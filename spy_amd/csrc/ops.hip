@@ -312,21 +312,35 @@ static int softmax_launch(void *stream, const spy_hip_tensor *x, const spy_hip_t
 // theta_k = pos[i2] * theta_scale^k where the power is built by k successive fp32
 // multiplications (:304-309); cos/sin of theta*freq_scale, times attention_factor.
 // ---------------------------------------------------------------------------------------------
+// ramp_on: extend_factor != 0 (YaRN, rope_yarn :247-260).  As written, rope_yarn_ramp (:242-245) clamps the VALUE 0 into
+// [1, y] -- std::clamp(0.0F, 1.0F, y) -- and so returns 1 - 1 = 0: ramp_mix = 0 * extend_factor, the angle stays the
+// interpolated one (the mix is still evaluated as written) and only the magnitude changes (mscale, folded in by the caller).
+// xpos (:353-354): zeta = pow((i0 + 0.4 ne0) / (1.4 ne0), position / xpos_base), inverted for xpos_down, times every product.
 __global__ __launch_bounds__(64) void rope_kernel(tdesc x, const int32_t *pos, int64_t pos_stride, tdesc y, float theta_scale,
-                                                  float freq_scale, float mscale) {
+                                                  float freq_scale, float mscale, int ramp_on, float ramp_mix, float xpos_base, int xpos_down) {
     const int64_t i1 = blockIdx.x, i2 = blockIdx.y, i3 = blockIdx.z;
-    const float p = (float)*(const int32_t *)((const uint8_t *)pos + i2 * pos_stride);
+    const int32_t pi = *(const int32_t *)((const uint8_t *)pos + i2 * pos_stride);
+    const float p = (float)pi;
     const int64_t npair = y.ne[0] / 2;
+    const float ne0f = (float)y.ne[0];
     for (int64_t k = threadIdx.x; k < npair; k += 64) {
         float theta = p;
         for (int64_t j = 0; j < k; j++) theta *= theta_scale;
-        const float ang = freq_scale * theta;
+        float ang = freq_scale * theta;
+        if (ramp_on) ang = ang * (1 - ramp_mix) + theta * ramp_mix;
         const float c = cosf(ang) * mscale, s = sinf(ang) * mscale;
         const float *sp = (const float *)at(x, 2 * k, i1, i2, i3);
         float *dp = (float *)at(y, 2 * k, i1, i2, i3);
         const float x0 = sp[0], x1 = sp[1];
-        dp[0] = x0 * c - x1 * s;
-        dp[1] = x0 * s + x1 * c;
+        if (xpos_base != 0.0f) {
+            float zeta = powf(((float)(2 * k) + 0.4f * ne0f) / (1.4f * ne0f), p / xpos_base);
+            if (xpos_down) zeta = 1.0f / zeta;
+            dp[0] = x0 * c * zeta - x1 * s * zeta;
+            dp[1] = x0 * s * zeta + x1 * c * zeta;
+        } else {
+            dp[0] = x0 * c - x1 * s;
+            dp[1] = x0 * s + x1 * c;
+        }
     }
 }
 
@@ -334,7 +348,6 @@ extern "C" int spy_hip_op_rope(void *stream, const spy_hip_tensor *x, const spy_
     SPY_CHECK_ARG(x && pos && dst && p && x->data && pos->data && dst->data);
     if (x->type != SPY_HIP_F32 || dst->type != SPY_HIP_F32 || pos->type != SPY_HIP_I32) return SPY_HIP_EUNSUPPORTED;
     if (p->mode != 0 && p->mode != -1) return SPY_HIP_EUNSUPPORTED;          // GLM / Neox (Neox aborts in the reference too)
-    if (p->extend_factor != 0.0f || p->xpos_base != 0.0f) return SPY_HIP_EUNSUPPORTED;
     SPY_CHECK_ARG(same_ne(x, dst) && x->nb[0] == 4 && dst->nb[0] == 4 && dst->ne[0] % 2 == 0 && p->num_dim > 0);
     SPY_CHECK_ARG(pos->ne[0] >= dst->ne[2] && dst->ne[1] < 65536 && dst->ne[2] < (1ll << 31) && dst->ne[3] < 65536);
     SPY_CHECK_ARG(dst->ne[1] > 0 && dst->ne[2] > 0 && dst->ne[3] > 0);
@@ -343,8 +356,11 @@ extern "C" int spy_hip_op_rope(void *stream, const spy_hip_tensor *x, const spy_
     const dim3 grid((unsigned)dst->ne[1], (unsigned)dst->ne[2], (unsigned)dst->ne[3]);
     SPY_CHECK_ARG(dst->ne[2] < 65536);
     if (spy_exact_on()) return spy_exact_rope((hipStream_t)stream, x, pos, dst, p);
+    float mscale = p->attention_factor;
+    const int ramp_on = p->extend_factor != 0.0f;
+    if (ramp_on) mscale *= 1.0f + 0.1f * logf(1.0f / p->freq_scale);          // :257, host libm as the reference
     rope_kernel<<<grid, dim3(64), 0, (hipStream_t)stream>>>(mk(x), (const int32_t *)pos->data, pos->nb[0], mk(dst), theta_scale,
-                                                           p->freq_scale, p->attention_factor);
+                                                           p->freq_scale, mscale, ramp_on, (1.0f - 1.0f) * p->extend_factor, p->xpos_base, p->xpos_down);
     return SPY_LAUNCH_RC();
 }
 

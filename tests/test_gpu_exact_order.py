@@ -232,6 +232,18 @@ def test_norm_softmax_silu_rope_bits(hip, oracle):
         dy = dev_empty(x.nbytes, 0xFF)
         call(L.spy_hip_op_rope, None, B(hip.tensor(dx, hip.F32, [hd, H_, T])), B(hip.tensor(dp, hip.I32, [T])), B(hip.tensor(dy, hip.F32, [hd, H_, T])), B(hp))
         _same_bits(dy.download(np.float32).reshape(x.shape), want, "rope, context %d" % n_ctx)
+    # YaRN magnitude and xpos: tables of this call's tokens from the host, zeta beside cos / sin
+    for kw in (dict(freq_scale=0.25, extend_factor=1.0, attention_factor=1.1), dict(xpos_base=512.0, xpos_down=0),
+               dict(freq_scale=0.5, extend_factor=0.7, xpos_base=300.0, xpos_down=1)):
+        rp2 = O.default_rope(hd, 4352)
+        hp = hip.RopeParam(0, 0, hd, 4352, 4352, 10000.0, 1.0, 0.0, 1.0, 32.0, 1.0, 0.0, 0)
+        for k, v in kw.items():
+            setattr(rp2, k, v); setattr(hp, k, v)
+        want2 = np.zeros_like(x)
+        assert oracle.spy_o_rope(B(O.tensor(x, O.F32, [hd, H_, T])), B(O.tensor(pos, O.I32, [T])), B(O.tensor(want2, O.F32, [hd, H_, T])), B(rp2)) == 0
+        dy = dev_empty(x.nbytes, 0xFF)
+        call(L.spy_hip_op_rope, None, B(hip.tensor(dx, hip.F32, [hd, H_, T])), B(hip.tensor(dp, hip.I32, [T])), B(hip.tensor(dy, hip.F32, [hd, H_, T])), B(hp))
+        _same_bits(dy.download(np.float32).reshape(x.shape), want2, "rope %s" % kw)
     flag = C.c_int32(-1)
     call(L.spy_hip_take_error, C.byref(flag)); assert flag.value == 0
     hp = hip.RopeParam(0, 0, hd, 4096, 4096, 10000.0, 1.0, 0.0, 1.0, 32.0, 1.0, 0.0, 0)       # position 4351 lies beyond this context

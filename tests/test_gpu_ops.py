@@ -147,6 +147,32 @@ def test_rope(hip, oracle):
                                       B(hip.tensor(dy, hip.F32, [hd, H_, T])), B(hp)) == hip.EUNSUPPORTED
 
 
+@pytest.mark.parametrize("name,kw", [
+    ("YaRN magnitude (extend_factor 1, freq_scale 0.25)", dict(freq_scale=0.25, extend_factor=1.0, attention_factor=1.1)),
+    ("xpos up", dict(xpos_base=512.0, xpos_down=0)),
+    ("xpos down with YaRN", dict(freq_scale=0.5, extend_factor=0.7, xpos_base=300.0, xpos_down=1)),
+])
+def test_rope_yarn_and_xpos(hip, oracle, name, kw):
+    """The two Rope extensions the reference plumbs through its default branch (non-linear.cpp:242-260, 349-364):
+    extend_factor != 0 changes the magnitude only (the ramp is 1 - std::clamp(0.0F, 1.0F, y) = 0 as written), xpos
+    multiplies every product by zeta.  Against the oracle to 1e-5 here, to the bit in exact order (test_gpu_exact_order.py)."""
+    from tests.gpu_util import dev, dev_empty, call, assert_close
+    rng = np.random.default_rng(51)
+    hd, H_, T = 128, 4, 5
+    pos = np.array([0, 3, 100, 2047, 4351], dtype=np.int32)
+    x = rng.standard_normal((T, H_, hd)).astype(np.float32)
+    want = np.zeros_like(x)
+    rp = O.default_rope(hd, 4352)
+    hp = hip.RopeParam(0, 0, hd, 4352, 4352, 10000.0, 1.0, 0.0, 1.0, 32.0, 1.0, 0.0, 0)
+    for k, v in kw.items():
+        setattr(rp, k, v); setattr(hp, k, v)
+    assert oracle.spy_o_rope(B(O.tensor(x, O.F32, [hd, H_, T])), B(O.tensor(pos, O.I32, [T])), B(O.tensor(want, O.F32, [hd, H_, T])), B(rp)) == 0
+    dx, dp, dy = dev(x), dev(pos), dev_empty(x.nbytes, 0xFF)
+    call(hip.load().spy_hip_op_rope, None, B(hip.tensor(dx, hip.F32, [hd, H_, T])), B(hip.tensor(dp, hip.I32, [T])),
+         B(hip.tensor(dy, hip.F32, [hd, H_, T])), B(hp))
+    assert_close(dy.download(np.float32).reshape(x.shape), want, "rope, " + name, tol=1e-5)
+
+
 def test_kv_cache_copy_bit_exact(hip, oracle):
     """KCache_cpy / VCache_cpy (attention.cpp:188-246 in the Spy tree) through the Copy operator."""
     from tests.gpu_util import dev, call

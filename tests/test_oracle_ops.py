@@ -179,6 +179,51 @@ def test_rope(oracle):
                              C.byref(O.tensor(y, O.F32, [hd, H, T])), C.byref(O.RopeParam(2, 0, hd, 64, 64, 1e4, 1, 0, 1, 32, 1, 0, 0))) == 1
 
 
+def test_rope_yarn_and_xpos_reduce_to_known_forms(oracle):
+    """Pins for the two extensions of the default Rope branch.  (1) extend_factor != 0 (rope_yarn, non-linear.cpp:247-260): the
+    ramp is 1 - std::clamp(0.0F, 1.0F, y), which clamps the value 0 into [1, y] and so is 0, leaving only
+    mscale *= 1 + 0.1 ln(1 / freq_scale): the result must equal, bit for bit, a plain Rope whose attention_factor is
+    that product -- for any extend_factor and any beta_fast / beta_slow.  (2) xpos (:353-354): every product is
+    multiplied by zeta = ((i0 + 0.4 ne0) / (1.4 ne0)) ^ (pos / xpos_base), or its inverse: out / zeta must be the plain
+    rotation, pair norms scale by zeta^2, position 0 has zeta = 1, and up * down restores the plain rotation's norm."""
+    rng = np.random.default_rng(16)
+    hd, H, T = 64, 3, 5
+    pos = np.array([0, 2, 31, 500, 3000], dtype=np.int32)
+    x = rng.standard_normal((T, H, hd)).astype(np.float32)
+
+    def run(rp):
+        y = np.zeros_like(x)
+        assert oracle.spy_o_rope(C.byref(O.tensor(x, O.F32, [hd, H, T])), C.byref(O.tensor(pos, O.I32, [T])),
+                                 C.byref(O.tensor(y, O.F32, [hd, H, T])), C.byref(rp)) == 0
+        return y
+
+    # (1)
+    for ext, fs, af, bf, bs in ((1.0, 0.25, 1.0, 32.0, 1.0), (0.3, 0.5, 1.3, 8.0, 2.0), (-2.0, 2.0, 0.7, 32.0, 1.0)):
+        yarn = O.RopeParam(0, 0, hd, 4096, 2048, 1e4, fs, ext, af, bf, bs, 0, 0)
+        m = np.float32(af) * (np.float32(1.0) + np.float32(0.1) * np.log(np.float32(1.0) / np.float32(fs)).astype(np.float32))
+        plain = O.RopeParam(0, 0, hd, 4096, 2048, 1e4, fs, 0.0, float(np.float32(m)), bf, bs, 0, 0)
+        a, b = run(yarn), run(plain)
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), (ext, fs)
+    # (2)
+    plain = run(O.default_rope(hd, 4096))
+    i0 = np.arange(0, hd, 2, dtype=np.float64)
+    for base in (512.0, 77.0):
+        # base and exponent rounded to fp32 as the reference forms them (a rounding of the base grows with the exponent), the power in fp64
+        f = np.float32
+        b32 = ((i0.astype(f) + f(0.4) * f(hd)) / (f(1.4) * f(hd))).astype(np.float64)
+        e32 = (pos.astype(f) / f(base)).astype(np.float64)
+        zeta = b32[None, :] ** e32[:, None]                                                       # [T, hd / 2]
+        up = run(O.RopeParam(0, 0, hd, 4096, 4096, 1e4, 1, 0, 1, 32, 1, base, 0))
+        down = run(O.RopeParam(0, 0, hd, 4096, 4096, 1e4, 1, 0, 1, 32, 1, base, 1))
+        z = np.repeat(zeta, 2, axis=1)[:, None, :]
+        # the two products of an output cancel, so the bound is relative to their size: a few fp32 roundings of (|x0| + |x1|) * zeta
+        mag = np.repeat(np.abs(x[..., 0::2]) + np.abs(x[..., 1::2]), 2, axis=-1).astype(np.float64)
+        assert (np.abs(up - plain * z) <= 8 * 2.0 ** -24 * mag * z).all()
+        assert (np.abs(down - plain / z) <= 8 * 2.0 ** -24 * mag / z).all()
+        assert np.array_equal(up[0], plain[0]) and np.array_equal(down[0], plain[0])         # position 0: zeta = 1
+        assert (np.abs(up.astype(np.float64) * down - plain.astype(np.float64) ** 2) <= 32 * 2.0 ** -24 * mag ** 2).all()
+
+
 def test_kv_cache_writes(oracle):
     """KCache_cpy / VCache_cpy (attention.cpp:188-246): K lands at [token][head][hd], V lands
     transposed at [d][C] column P+t; every other cache byte is untouched."""
