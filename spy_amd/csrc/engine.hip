@@ -569,16 +569,8 @@ static int forward_any(spy_hip_llama *m, void *stream, const int32_t *tokens_hos
     // this backend's own order, single-token passes still in order 1)
     struct scope_t { int prev; bool on; ~scope_t() { if (on) spy_exact_thread_scope(prev); } } scope = {-1, false};
     if (n_token > 1 && !spy_exact_on() && pass_order(m) == 1) {
-        // ... where the tiled exact MatMul takes every matrix of the layers (Q4_0, Q8_0).  K-quant layers would go through the
-        // row kernels (30 x slower on a long prompt); the reference has no K-quant arithmetic whose order could be followed,
-        // so their prompts stay in order 0 unless SPY_HIP_PROMPT_ORDER=1 asks for the host order.
-        bool tiled = true;
-        for (int il = 0; il < m->desc.n_layer && tiled; il++) {
-            const spy_hip_llama_layer &L = m->layers[il];
-            for (int t : {L.t_wq, L.t_wk, L.t_wv, L.t_wo, L.t_gate, L.t_up, L.t_down}) tiled = tiled && (t == SPY_HIP_Q4_0 || t == SPY_HIP_Q8_0);
-        }
         const char *e = getenv("SPY_HIP_PROMPT_ORDER");
-        if (e && (e[0] == '0' || e[0] == '1') ? e[0] == '1' : tiled) { scope.prev = spy_exact_thread_scope(1); scope.on = true; }
+        if (!(e && e[0] == '0')) { scope.prev = spy_exact_thread_scope(1); scope.on = true; }
     }
     const bool exact = spy_exact_on() != 0;
     // single tokens: the fused pass, in the order pass_order() names (with the library-wide exact-order switch on and a

@@ -485,6 +485,17 @@ __device__ __forceinline__ void xgb_mfma_word(xgb_v4i (&out)[4], const uint4 &wq
     }
 #undef XGB_CASE
 }
+// the same four instructions accumulating onto their previous results (integer sums over several element words)
+__device__ __forceinline__ void xgb_mfma_word_acc(xgb_v4i (&io)[4], const uint4 &wq4, uint32_t xq, int abid) {
+#define XGB_CASE(n) case n: \
+        io[0] = __builtin_amdgcn_mfma_i32_4x4x4i8((int)wq4.x, (int)xq, io[0], 4, n, 0); io[1] = __builtin_amdgcn_mfma_i32_4x4x4i8((int)wq4.y, (int)xq, io[1], 4, n, 0); \
+        io[2] = __builtin_amdgcn_mfma_i32_4x4x4i8((int)wq4.z, (int)xq, io[2], 4, n, 0); io[3] = __builtin_amdgcn_mfma_i32_4x4x4i8((int)wq4.w, (int)xq, io[3], 4, n, 0); break;
+    switch (abid) {
+        XGB_CASE(0) XGB_CASE(1) XGB_CASE(2) XGB_CASE(3) XGB_CASE(4) XGB_CASE(5) XGB_CASE(6) XGB_CASE(7)
+        XGB_CASE(8) XGB_CASE(9) XGB_CASE(10) XGB_CASE(11) XGB_CASE(12) XGB_CASE(13) XGB_CASE(14) XGB_CASE(15)
+    }
+#undef XGB_CASE
+}
 // D[g][i] = d_w(row 4g + i) * d_x(this lane's activation row) for block kb of a pair: lane group 4 * kb + g supplies the four d_w
 template <int>
 __device__ __forceinline__ void xgb_mfma_scale(xgb_v4f (&D)[4], float wd, float xd, const xgb_v4f &zero4, int kb) {
@@ -684,6 +695,193 @@ __global__ __launch_bounds__(256, 2) void exact_gemm8_kernel(const uint8_t *__re
         const int64_t row = m0 + 4 * mg;
         if (tok < ne11 && row < ne01) *(float4 *)(dst + tok * d_row + row) = make_float4(o[0], o[1], o[2], o[3]);
     }
+    }
+}
+
+// The K-quant dots for many activation rows at once, tiled like exact_gemm8_kernel<., true> (64 x 64 outputs per workgroup, a
+// wave 16 weight rows x 64 activation rows, lane = activation row, weight words through the A-matrix broadcast of the 4 x 4 x 4
+// matrix instruction).  These dots keep ONE accumulator per output and add a term per sub-block of 32 elements, in order:
+//   Q4_K:  acc = fma(d_x, d * float(sc * isum) - dmin * float(m * bsum), acc)       isum = sum q * x, bsum = sum x over the sub-block
+//   Q6_K:  acc = fma(d_x * d, float(sc0 * isum0 + sc1 * isum1), acc)                 isum0 / isum1 over the two halves of 16 elements
+// The integer sums are chains of matrix instructions over the element words of a sub-block (exact: integers); a stage is half a
+// super-block (four sub-blocks).  The bits are those of exact_dotsk_kernel and of the oracle.
+template <int WT>
+__global__ __launch_bounds__(256, 2) void exact_gemmk_kernel(const uint8_t *__restrict__ w, int64_t w_row, int64_t ne01, int64_t nsb,
+                                                              const uint8_t *__restrict__ xm, int64_t x_row, int64_t ne11,
+                                                              float *__restrict__ dst, int64_t d_row) {
+    constexpr bool K4 = WT == SPY_HIP_Q4_K;
+    constexpr int WPL = XGB_TILE + 4;
+    __shared__ __align__(16) uint32_t s_wq[2][XGB_KB][8][WPL];     // element words of the weights, rows j, j + 4, ... side by side
+    __shared__ __align__(16) uint32_t s_xq[2][XGB_KB][8][XGB_TILE];
+    __shared__ __align__(16) int32_t s_ws0[2][XGB_KB][XGB_TILE];   // Q4_K: sc          Q6_K: scale of elements 0..15
+    __shared__ __align__(16) int32_t s_ws1[2][XGB_KB][XGB_TILE];   // Q4_K: m           Q6_K: scale of elements 16..31
+    __shared__ __align__(16) float s_wd[2][2][XGB_TILE];           // d, dmin of the super-block (Q6_K: d)
+    __shared__ __align__(16) float s_xd[2][XGB_KB][XGB_TILE];
+    __shared__ __align__(16) int32_t s_xb[2][XGB_KB][XGB_TILE];    // Q4_K: sum of the activation quants of the block
+    const int tid = threadIdx.x;
+    const int wv = tid >> 6, bj = tid & 63, jj = tid & 3, grp = bj >> 2;
+    const int64_t m0 = (int64_t)blockIdx.x * XGB_TILE, t0 = (int64_t)blockIdx.y * XGB_TILE;
+
+    // loaders: waves 0 and 1 bring weights (a thread: one row, two of the stage's four sub-blocks), waves 2 and 3 activation blocks
+    const bool ld_w = tid < 128;
+    const int ld_row = tid & 63, ld_pair = (tid >> 6) & 1;
+    const int ld_slot = (ld_row & 3) * 16 + (ld_row >> 2);
+    const uint8_t *ld_wrow = w + min(m0 + ld_row, ne01 - 1) * w_row;
+    const uint32_t *ld_xsrc = (const uint32_t *)(xm + min(t0 + ld_row, ne11 - 1) * x_row) + ld_pair * 17;
+    uint32_t g[17];                                                // activations: two Q8_0 blocks; weights: quant words and scale bytes
+    auto fetch = [&](int64_t stage) {
+        if (!ld_w) {
+            const uint32_t *p = ld_xsrc + stage * 34;
+#pragma unroll
+            for (int i = 0; i < 17; i++) g[i] = p[i];
+        } else if (K4) {
+            // super-block of 144 bytes: d, dmin, scales[12], qs[128]; sub-blocks 2k and 2k + 1 are the low and high nibbles of qs[32k .. 32k + 31]
+            const uint8_t *sb = ld_wrow + (stage >> 1) * 144;
+            const uint4 *q = (const uint4 *)(sb + 16 + 64 * (stage & 1) + 32 * ld_pair);
+            const uint4 a = q[0], b = q[1];
+            g[0] = a.x; g[1] = a.y; g[2] = a.z; g[3] = a.w; g[4] = b.x; g[5] = b.y; g[6] = b.z; g[7] = b.w;
+            const uint32_t *h = (const uint32_t *)sb;
+            g[8] = h[0]; g[9] = h[1]; g[10] = h[2]; g[11] = h[3];
+        } else {
+            // super-block of 210 bytes (2-byte aligned): ql[128], qh[64], scales[16], d.  Half h of it = sub-blocks 4h .. 4h + 3; this thread
+            // takes sub-blocks 4h + p and 4h + p + 2: the low and high nibbles of ql[64h + 32p ..], with bits 2(p), 2(p + 2) of qh[32h ..]
+            const uint8_t *sb = ld_wrow + (stage >> 1) * 210;
+            const int h = (int)(stage & 1);
+#pragma unroll
+            for (int i = 0; i < 8; i++) g[i] = ld_u32_a2(sb + 64 * h + 32 * ld_pair + 4 * i);
+#pragma unroll
+            for (int i = 0; i < 8; i++) g[8 + i] = ld_u32_a2(sb + 128 + 32 * h + 4 * i);
+            g[16] = (uint32_t)*(const uint16_t *)(sb + 192 + 2 * (4 * h + ld_pair)) | ((uint32_t)*(const uint16_t *)(sb + 192 + 2 * (4 * h + ld_pair + 2)) << 16);
+        }
+    };
+    auto put = [&](int buf, int64_t stage) {
+        if (!ld_w) {
+            const int k0 = 2 * ld_pair;
+            s_xd[buf][k0][ld_row] = h2f_tab((uint16_t)(g[0] & 0xFFFFu));
+            s_xd[buf][k0 + 1][ld_row] = h2f_tab((uint16_t)(g[8] >> 16));
+            int32_t b0 = 0, b1 = 0;
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                const uint32_t q0 = __builtin_amdgcn_alignbit(g[k + 1], g[k], 16), q1 = g[9 + k];
+                s_xq[buf][k0][k][ld_row] = q0; s_xq[buf][k0 + 1][k][ld_row] = q1;
+                if (K4) { b0 = __builtin_amdgcn_sdot4((int)q0, 0x01010101, b0, false); b1 = __builtin_amdgcn_sdot4((int)q1, 0x01010101, b1, false); }
+            }
+            if (K4) { s_xb[buf][k0][ld_row] = b0; s_xb[buf][k0 + 1][ld_row] = b1; }
+        } else if (K4) {
+            const int k0 = 2 * ld_pair;                            // sub-blocks k0 (low nibbles) and k0 + 1 (high nibbles) of the stage
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                s_wq[buf][k0][k][ld_slot] = g[k] & 0x0F0F0F0Fu;
+                s_wq[buf][k0 + 1][k][ld_slot] = (g[k] >> 4) & 0x0F0F0F0Fu;
+            }
+            // get_scale_min_k4 for sub-blocks j and j + 1 of the super-block, j = 4 * (stage & 1) + k0
+            const uint8_t sbytes[12] = {(uint8_t)(g[9]), (uint8_t)(g[9] >> 8), (uint8_t)(g[9] >> 16), (uint8_t)(g[9] >> 24), (uint8_t)(g[10]), (uint8_t)(g[10] >> 8),
+                                        (uint8_t)(g[10] >> 16), (uint8_t)(g[10] >> 24), (uint8_t)(g[11]), (uint8_t)(g[11] >> 8), (uint8_t)(g[11] >> 16), (uint8_t)(g[11] >> 24)};
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                int32_t sc, m;
+                if ((stage & 1) == 0) { const int j = k0 + u; sc = sbytes[j] & 63; m = sbytes[j + 4] & 63; }
+                else { const int j = 4 + k0 + u; sc = (sbytes[j + 4] & 0x0F) | ((sbytes[j - 4] >> 6) << 4); m = (sbytes[j + 4] >> 4) | ((sbytes[j] >> 6) << 4); }
+                s_ws0[buf][k0 + u][ld_slot] = sc;
+                s_ws1[buf][k0 + u][ld_slot] = m;
+            }
+            if (ld_pair == 0) {
+                s_wd[buf][0][ld_slot] = h2f_tab((uint16_t)(g[8] & 0xFFFFu));
+                s_wd[buf][1][ld_slot] = h2f_tab((uint16_t)(g[8] >> 16));
+            }
+        } else {
+            const uint8_t *sb = ld_wrow + (stage >> 1) * 210;
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                const int gq = ld_pair + 2 * u;                    // sub-block of the stage: 0 / 2 for pair 0, 1 / 3 for pair 1
+#pragma unroll
+                for (int k = 0; k < 8; k++) {
+                    const uint32_t lo = (u ? (g[k] >> 4) : g[k]) & 0x0F0F0F0Fu, hi = (g[8 + k] >> (2 * gq)) & 0x03030303u;
+                    const uint32_t q = lo | (hi << 4);
+                    s_wq[buf][gq][k][ld_slot] = ((q | 0x80808080u) - 0x20202020u) ^ 0x80808080u;      // per byte q - 32
+                }
+                const uint32_t sc2 = u ? (g[16] >> 16) : (g[16] & 0xFFFFu);
+                s_ws0[buf][gq][ld_slot] = (int32_t)(int8_t)(sc2 & 0xFFu);
+                s_ws1[buf][gq][ld_slot] = (int32_t)(int8_t)(sc2 >> 8);
+            }
+            if (ld_pair == 0) s_wd[buf][0][ld_slot] = h2f_tab(*(const uint16_t *)(sb + 208));
+        }
+    };
+
+    float acc[4][4];
+#pragma unroll
+    for (int r = 0; r < 4; r++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) acc[r][c] = 0.0f;
+    const xgb_v4i zero4i = {0, 0, 0, 0};
+
+    const int64_t nstage = 2 * nsb;
+    fetch(0);
+    put(0, 0);
+    __syncthreads();
+    for (int64_t s = 0; s < nstage; s++) {
+        const int buf = (int)(s & 1);
+        if (s + 1 < nstage) fetch(s + 1);
+        // rows 16 * wave + 4g + i sit at slot i * 16 + 4 * wave + g of their planes: one 16-byte read per i brings g = 0..3
+        xgb_v4f dw[4], dmn[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            dw[i] = *(const xgb_v4f *)&s_wd[buf][0][i * 16 + 4 * wv];
+            if (K4) dmn[i] = *(const xgb_v4f *)&s_wd[buf][1][i * 16 + 4 * wv];
+        }
+#pragma unroll 1
+        for (int half = 0; half < XGB_KB / 2; half++) {
+            const uint4 wq4 = *(const uint4 *)&s_wq[buf][2 * half + (grp >> 3)][grp & 7][jj * 16 + 4 * wv];      // lane group 8 * (block & 1) + e: rows 4g + j, g = 0..3
+#pragma unroll
+            for (int kb2 = 0; kb2 < 2; kb2++) {
+                const int kb = 2 * half + kb2;
+                const float xd = s_xd[buf][kb][bj];
+                uint32_t xq[8];
+#pragma unroll
+                for (int e = 0; e < 8; e++) xq[e] = s_xq[buf][kb][e][bj];
+                xgb_v4i s0[4], s1[4];                              // [i][g]: scale integers of row 4g + i
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    s0[i] = *(const xgb_v4i *)&s_ws0[buf][kb][i * 16 + 4 * wv];
+                    s1[i] = *(const xgb_v4i *)&s_ws1[buf][kb][i * 16 + 4 * wv];
+                }
+                // integer sums of the sub-block: isum[g] (Q4_K) or the two halves lo[g], hi[g] (Q6_K), component i = row 4g + i
+                xgb_v4i lo[4] = {zero4i, zero4i, zero4i, zero4i}, hi[4] = {zero4i, zero4i, zero4i, zero4i};
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    if (K4 || e < 4) xgb_mfma_word_acc(lo, wq4, xq[e], kb2 * 8 + e);
+                    else xgb_mfma_word_acc(hi, wq4, xq[e], kb2 * 8 + e);
+                }
+                if (K4) {
+                    const int32_t xb = s_xb[buf][kb][bj];
+#pragma unroll
+                    for (int gq = 0; gq < 4; gq++)
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            const float pos = dw[i][gq] * (float)__mul24(s0[i][gq], lo[gq][i]);
+                            const float neg = dmn[i][gq] * (float)__mul24(s1[i][gq], xb);
+                            acc[gq][i] = fmaf(xd, pos - neg, acc[gq][i]);
+                        }
+                } else {
+#pragma unroll
+                    for (int gq = 0; gq < 4; gq++)
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            const int32_t sv = __mul24(s0[i][gq], lo[gq][i]) + __mul24(s1[i][gq], hi[gq][i]);
+                            const float dd = xd * dw[i][gq];
+                            acc[gq][i] = fmaf(dd, (float)sv, acc[gq][i]);
+                        }
+                }
+            }
+        }
+        if (s + 1 < nstage) put(buf ^ 1, s + 1);
+        __syncthreads();
+    }
+    const int64_t tok = t0 + bj;
+#pragma unroll
+    for (int gq = 0; gq < 4; gq++) {
+        const int64_t row = m0 + 16 * wv + 4 * gq;
+        if (tok < ne11 && row < ne01) *(float4 *)(dst + tok * d_row + row) = make_float4(acc[gq][0], acc[gq][1], acc[gq][2], acc[gq][3]);
     }
 }
 
@@ -926,6 +1124,21 @@ int spy_exact_dots(hipStream_t st, int t0, const spy_hip_tensor *w, const uint8_
     }
     const dim3 grid((unsigned)((total + 63) / 64)), block(64);
     // SPY_HIP_EXACT_SERIAL=1: one thread per output element for every type (the plain restatement the lane forms are tested against)
+    if ((t0 == SPY_HIP_Q4_K || t0 == SPY_HIP_Q6_K) && ne11 >= 16 && w->ne[2] == 1 && w->ne[3] == 1) {
+        const char *env_tiled = getenv("SPY_HIP_EXACT_TILED");
+        const int64_t nsb = w->ne[0] / 256, ne01 = w->ne[1];
+        const bool fits = nsb > 0 && w->ne[0] % 256 == 0 && ne01 % 4 == 0 && x_row % 4 == 0 && ((uintptr_t)xm & 3) == 0 && dst->nb[0] == 4 && dst->nb[1] % 16 == 0 &&
+                          ((uintptr_t)dst->data & 15) == 0 && (ne11 + XGB_TILE - 1) / XGB_TILE <= 65535 && !getenv("SPY_HIP_EXACT_SERIAL") &&
+                          (t0 == SPY_HIP_Q4_K ? (((uintptr_t)w->data & 15) == 0 && w->nb[1] % 16 == 0) : (((uintptr_t)w->data & 1) == 0 && w->nb[1] % 2 == 0));
+        if (fits && !(env_tiled && *env_tiled == '0')) {
+            const dim3 grid((unsigned)((ne01 + XGB_TILE - 1) / XGB_TILE), (unsigned)((ne11 + XGB_TILE - 1) / XGB_TILE));
+            if (t0 == SPY_HIP_Q4_K)
+                exact_gemmk_kernel<SPY_HIP_Q4_K><<<grid, dim3(256), 0, st>>>((const uint8_t *)w->data, w->nb[1], ne01, nsb, xm, x_row, ne11, (float *)dst->data, dst->nb[1] / 4);
+            else
+                exact_gemmk_kernel<SPY_HIP_Q6_K><<<grid, dim3(256), 0, st>>>((const uint8_t *)w->data, w->nb[1], ne01, nsb, xm, x_row, ne11, (float *)dst->data, dst->nb[1] / 4);
+            return SPY_LAUNCH_RC();
+        }
+    }
     const bool serial = getenv("SPY_HIP_EXACT_SERIAL") != nullptr;
     const dim3 grid8((unsigned)((total + 31) / 32)), grid32((unsigned)((total + 7) / 8));
     if (!serial && t0 == SPY_HIP_Q4_0) { exact_dots8_kernel<SPY_HIP_Q4_0><<<grid8, dim3(256), 0, st>>>(mkx(w), xm, x_row, mkx(dst), ne11, total); return SPY_LAUNCH_RC(); }

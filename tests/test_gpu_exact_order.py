@@ -57,13 +57,15 @@ def test_quantized_matmul_bits(hip, oracle, wtype, M, K, T, serial, monkeypatch)
     _same_bits(dd.download(np.float32).reshape(T, M), want, "matmul type %d %dx%d T %d" % (wtype, M, K, T))
 
 
-@pytest.mark.parametrize("wtype", [O.Q4_0, O.Q8_0])
-@pytest.mark.parametrize("M,K,T", [(96, 4096, 16), (200, 512, 70), (64, 128, 64), (132, 11008, 33), (4096, 4096, 130)])
+@pytest.mark.parametrize("wtype", [O.Q4_0, O.Q8_0, O.Q4_K, O.Q6_K])
+@pytest.mark.parametrize("M,K,T", [(96, 4096, 16), (200, 512, 70), (64, 128, 64), (64, 256, 64), (132, 11008, 33), (4096, 4096, 130)])
 def test_tiled_matmul_bits(hip, oracle, wtype, M, K, T, monkeypatch):
     """Sixteen activation rows and more take the tiled kernel (64 x 64 outputs per workgroup, the eight accumulators
     of every output in registers): the oracle's bits, with whole and partial tiles along both sides, and the same
     bits as the row kernels give (SPY_HIP_EXACT_TILED=0)."""
     from tests.gpu_util import dev, dev_empty, call
+    if K % 256 and wtype in (O.Q4_K, O.Q6_K):
+        pytest.skip("K-quant rows are whole super-blocks")
     rng = np.random.default_rng(7 * wtype + M + K + T)
     w = O.quantize(oracle, (rng.standard_normal((M, K)) * 0.02).astype(np.float32), wtype)
     x = (rng.standard_normal((T, K)) * rng.uniform(0.1, 30.0, (T, 1))).astype(np.float32)
