@@ -473,65 +473,39 @@ __global__ __launch_bounds__(256) void exact_dots8_kernel(xdesc w, const uint8_t
 #define XGB_KB 4          // blocks per stage
 typedef int xgb_v4i __attribute__((ext_vector_type(4)));
 typedef float xgb_v4f __attribute__((ext_vector_type(4)));
-// The four matrix instructions of one element word: the A operand (weight words of rows 4g + j) is taken from lane group `abid`
-// for all sixteen groups.  abid has to be an immediate, hence the switch over constants (the callers' loops are unrolled).
-__device__ __forceinline__ void xgb_mfma_word(xgb_v4i (&out)[4], const uint4 &wq4, uint32_t xq, const xgb_v4i &bias, int abid) {
-#define XGB_CASE(n) case n: \
-        out[0] = __builtin_amdgcn_mfma_i32_4x4x4i8((int)wq4.x, (int)xq, bias, 4, n, 0); out[1] = __builtin_amdgcn_mfma_i32_4x4x4i8((int)wq4.y, (int)xq, bias, 4, n, 0); \
-        out[2] = __builtin_amdgcn_mfma_i32_4x4x4i8((int)wq4.z, (int)xq, bias, 4, n, 0); out[3] = __builtin_amdgcn_mfma_i32_4x4x4i8((int)wq4.w, (int)xq, bias, 4, n, 0); break;
+typedef int xgb_v16i __attribute__((ext_vector_type(16)));
+typedef float xgb_v16f __attribute__((ext_vector_type(16)));
+// v_mfma_i32_16x16x4_4b_i8 with the A operand of lane block abid for all four products (abid has to be an immediate)
+__device__ __forceinline__ xgb_v16i xgb_mfma16(uint32_t w, uint32_t x, const xgb_v16i &c, int abid) {
     switch (abid) {
-        XGB_CASE(0) XGB_CASE(1) XGB_CASE(2) XGB_CASE(3) XGB_CASE(4) XGB_CASE(5) XGB_CASE(6) XGB_CASE(7)
-        XGB_CASE(8) XGB_CASE(9) XGB_CASE(10) XGB_CASE(11) XGB_CASE(12) XGB_CASE(13) XGB_CASE(14) XGB_CASE(15)
+    case 0: return __builtin_amdgcn_mfma_i32_16x16x4i8((int)w, (int)x, c, 2, 0, 0);
+    case 1: return __builtin_amdgcn_mfma_i32_16x16x4i8((int)w, (int)x, c, 2, 1, 0);
+    case 2: return __builtin_amdgcn_mfma_i32_16x16x4i8((int)w, (int)x, c, 2, 2, 0);
+    default: return __builtin_amdgcn_mfma_i32_16x16x4i8((int)w, (int)x, c, 2, 3, 0);
     }
-#undef XGB_CASE
 }
-// the same four instructions accumulating onto their previous results (integer sums over several element words)
-__device__ __forceinline__ void xgb_mfma_word_acc(xgb_v4i (&io)[4], const uint4 &wq4, uint32_t xq, int abid) {
-#define XGB_CASE(n) case n: \
-        io[0] = __builtin_amdgcn_mfma_i32_4x4x4i8((int)wq4.x, (int)xq, io[0], 4, n, 0); io[1] = __builtin_amdgcn_mfma_i32_4x4x4i8((int)wq4.y, (int)xq, io[1], 4, n, 0); \
-        io[2] = __builtin_amdgcn_mfma_i32_4x4x4i8((int)wq4.z, (int)xq, io[2], 4, n, 0); io[3] = __builtin_amdgcn_mfma_i32_4x4x4i8((int)wq4.w, (int)xq, io[3], 4, n, 0); break;
-    switch (abid) {
-        XGB_CASE(0) XGB_CASE(1) XGB_CASE(2) XGB_CASE(3) XGB_CASE(4) XGB_CASE(5) XGB_CASE(6) XGB_CASE(7)
-        XGB_CASE(8) XGB_CASE(9) XGB_CASE(10) XGB_CASE(11) XGB_CASE(12) XGB_CASE(13) XGB_CASE(14) XGB_CASE(15)
-    }
-#undef XGB_CASE
-}
-// D[g][i] = d_w(row 4g + i) * d_x(this lane's activation row) for block kb of a pair: lane group 4 * kb + g supplies the four d_w
-template <int>
-__device__ __forceinline__ void xgb_mfma_scale(xgb_v4f (&D)[4], float wd, float xd, const xgb_v4f &zero4, int kb) {
-#define XGB_CASE(n) case n: \
-        D[0] = __builtin_amdgcn_mfma_f32_4x4x1f32(wd, xd, zero4, 4, 4 * n, 0); D[1] = __builtin_amdgcn_mfma_f32_4x4x1f32(wd, xd, zero4, 4, 4 * n + 1, 0); \
-        D[2] = __builtin_amdgcn_mfma_f32_4x4x1f32(wd, xd, zero4, 4, 4 * n + 2, 0); D[3] = __builtin_amdgcn_mfma_f32_4x4x1f32(wd, xd, zero4, 4, 4 * n + 3, 0); break;
-    switch (kb) { XGB_CASE(0) XGB_CASE(1) }
-#undef XGB_CASE
-}
-// MF = true: the integer sums come from the matrix cores instead: v_mfma_i32_4x4x4_16b_i8 multiplies, in each group of four
-// lanes, a 4 x 4 byte matrix (lane j supplies row j) by another (lane j supplies column j) and leaves column j of the 4 x 4
-// result in lane j -- sixteen four-element dot products per group, exactly one accumulator's share of a block.  A wave then
-// holds 16 weight rows x 64 activation rows (lane = activation row 4b + j; the weight words of rows 4g + j, g = 0..3, are
-// the same for all sixteen groups and come as one broadcast read), a lane again 16 outputs with 8 accumulators each, and
-// the vector units are left with the subtraction and the fma per term.
+// MF = true: the integer sums come from the matrix cores instead.  v_mfma_i32_16x16x4_4b_i8 computes four 16 x 16 products over
+// four elements each, exactly one accumulator's share of a block for 16 weight rows x 64 activation rows.  A wave holds such a
+// tile, a lane again 16 outputs with 8 accumulators each, and the vector units are left with the subtraction and the fma per term.
 template <int WT, bool MF>
 __global__ __launch_bounds__(256, 2) void exact_gemm8_kernel(const uint8_t *__restrict__ w, int64_t w_row, int64_t ne01, int64_t nb,
                                                               const uint8_t *__restrict__ xm, int64_t x_row, int64_t ne11,
                                                               float *__restrict__ dst, int64_t d_row) {
-    constexpr int WPL = MF ? XGB_TILE + 4 : XGB_TILE;              // words per weight plane: MF reads 16 planes at once, the padding spreads them over the banks
+    constexpr int WPL = MF ? XGB_TILE + 16 : XGB_TILE;             // words per weight plane: MF reads four planes at once, the padding puts them on different banks
     __shared__ __align__(16) uint32_t s_wq[2][XGB_KB][8][WPL];
     __shared__ __align__(16) uint32_t s_xq[2][XGB_KB][8][XGB_TILE];
     __shared__ __align__(16) float s_wd[2][XGB_KB][XGB_TILE];
     __shared__ __align__(16) float s_xd[2][XGB_KB][XGB_TILE];
     const int tid = threadIdx.x;
     const int mg = tid & 15, tg = tid >> 4;                              // MF = false: 4 weight rows x 4 activation rows per thread
-    const int wv = tid >> 6, bj = tid & 63, jj = tid & 3;                // MF = true: wave, activation row of the tile, lane within its group of four
+    const int wv = tid >> 6, bj = tid & 63;                              // MF = true: wave, activation row of the tile
     const int64_t m0 = (int64_t)blockIdx.x * XGB_TILE, t0 = (int64_t)blockIdx.y * XGB_TILE;
 
     // loaders: waves 0 and 1 bring weight blocks, waves 2 and 3 activation blocks; a thread takes two neighbouring
     // blocks of one row (36 bytes of Q4_0, 68 of Q8_0: whole aligned words) per stage
     const bool ld_w = tid < 128;
     const int ld_row = tid & 63, ld_pair = (tid >> 6) & 1;
-    // where a weight row's words go in their LDS plane: in row order, or (MF) rows j, j + 4, j + 8, ... side by side so that the
-    // four words a lane feeds to its four matrix instructions are one 16-byte read
-    const int ld_slot = (MF && ld_w) ? (ld_row & 3) * 16 + (ld_row >> 2) : ld_row;
+    const int ld_slot = ld_row;
     constexpr int NWQ = WT == SPY_HIP_Q4_0 ? 9 : 17;
     const uint32_t *ld_src;
     if (ld_w) ld_src = (const uint32_t *)(w + min(m0 + ld_row, ne01 - 1) * w_row) + ld_pair * NWQ;
@@ -587,6 +561,10 @@ __global__ __launch_bounds__(256, 2) void exact_gemm8_kernel(const uint8_t *__re
 #pragma unroll
             for (int a = 0; a < 8; a++) acc[r][c][a] = 0.0f;
 
+    xgb_v16i bias16;
+    xgb_v16f zero16;
+#pragma unroll
+    for (int n = 0; n < 16; n++) { bias16[n] = 0x4B400000; zero16[n] = 0.0f; }
     const int64_t nstage = nb / XGB_KB;
     fetch(0);
     put(0);
@@ -595,42 +573,39 @@ __global__ __launch_bounds__(256, 2) void exact_gemm8_kernel(const uint8_t *__re
         const int buf = (int)(s & 1);
         if (s + 1 < nstage) fetch(s + 1);
         if constexpr (MF) {
-            // acc[g][i]: weight row 16 * wave + 4g + i against this lane's activation row.  Every group of four lanes would feed the
-            // same weight words to its matrix instructions; instead each group reads the words of ANOTHER (block, element word) pair
-            // -- one 16-byte read per lane covers two blocks -- and the instruction is told which group's words to use for all sixteen
-            // (cbsz = 4, abid = the group).  The scale products d_w * d_x come the same way from v_mfma_f32_4x4x1_16b_f32 (one product
-            // per output, rounded once: the bits of the vector multiply).
-            const xgb_v4i bias = {0x4B400000, 0x4B400000, 0x4B400000, 0x4B400000};
-            const xgb_v4f zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
-            const int grp = bj >> 2;                                                  // this lane's group of four, 0..15
+            // v_mfma_i32_16x16x4_4b_i8: four 16 x 16 x 4 products at once, lane l supplying row l % 16 of A and column l % 16 of B for
+            // product l / 16.  With the A-matrix broadcast (cbsz:2 abid:q) all four use the weight words held by lane block q, so
+            // one instruction multiplies the wave's 16 weight rows by its 64 activation rows over one element word, and the four lane
+            // blocks can hold the words of four different (block, element word) pairs: a 4-byte LDS read per lane covers four
+            // instructions.  Output register 4b + v of lane (blk, r): weight row 16 * wave + 4 * blk + v, activation row 16b + r.
+            // The scale products d_w * d_x come the same way from v_mfma_f32_16x16x1_4b_f32 (one product per output, rounded once:
+            // the bits of the vector multiply).
+            const int blk = bj >> 4, r = bj & 15;
 #pragma unroll 1
             for (int half = 0; half < XGB_KB / 2; half++) {
-                const float wdreg = s_wd[buf][2 * half + ((grp >> 2) & 1)][16 * wv + 4 * (grp & 3) + jj];    // group 4 * (block & 1) + g holds the scales of rows 4g + j
-                const uint4 wq4 = *(const uint4 *)&s_wq[buf][2 * half + (grp >> 3)][grp & 7][jj * 16 + 4 * wv];      // group 8 * (block & 1) + e: rows 4g + j, g = 0..3
+                const float wdreg = s_wd[buf][2 * half + (blk & 1)][16 * wv + r];       // lane block q: scales of block 2 * half + (q & 1)
+                uint32_t wreg[4];                                                          // lane block q, read i: word (4i + q) & 7 of block 2 * half + (4i + q) / 8
+#pragma unroll
+                for (int i = 0; i < 4; i++) wreg[i] = s_wq[buf][2 * half + (i >> 1)][4 * (i & 1) + blk][16 * wv + r];
 #pragma unroll
                 for (int kb2 = 0; kb2 < 2; kb2++) {
                     const int kb = 2 * half + kb2;
-                    const float xd = s_xd[buf][kb][bj];
-                    xgb_v4f D[4];
-                    xgb_mfma_scale<0>(D, wdreg, xd, zero4, kb2);
-                    uint32_t xq[8];
+                    const float xdl = s_xd[buf][kb][bj];                    // the B operands are the lane's own activation row bj = 16 * blk + r
+                    uint32_t xql[8];
 #pragma unroll
-                    for (int e = 0; e < 8; e++) xq[e] = s_xq[buf][kb][e][bj];
-                    // the four matrix instructions of word e + 1 are issued before the vector work on the results of word e
-                    xgb_v4i p[2][4];
-                    xgb_mfma_word(p[0], wq4, xq[0], bias, kb2 * 8 + 0);
+                    for (int e = 0; e < 8; e++) xql[e] = s_xq[buf][kb][e][bj];
+                    const xgb_v16f D = kb2 == 0 ? __builtin_amdgcn_mfma_f32_16x16x1f32(wdreg, xdl, zero16, 2, 0, 0)
+                                                : __builtin_amdgcn_mfma_f32_16x16x1f32(wdreg, xdl, zero16, 2, 1, 0);
+                    // the matrix instruction of word e + 1 is issued before the vector work on the results of word e
+                    xgb_v16i p[2];
+                    p[0] = xgb_mfma16(wreg[2 * kb2], xql[0], bias16, 0);
 #pragma unroll
                     for (int e = 0; e < 8; e++) {
-                        if (e + 1 < 8) xgb_mfma_word(p[(e + 1) & 1], wq4, xq[e + 1], bias, kb2 * 8 + e + 1);
+                        if (e + 1 < 8) p[(e + 1) & 1] = xgb_mfma16(wreg[2 * kb2 + ((e + 1) >> 2)], xql[e + 1], bias16, (e + 1) & 3);
                         const int a = WT == SPY_HIP_Q4_0 ? ((e + 4) & 7) : e;
 #pragma unroll
-                        for (int gq = 0; gq < 4; gq++) {
-                            const xgb_v4i r = p[e & 1][gq];
-                            acc[gq][0][a] = fmaf(D[gq].x, __int_as_float(r.x) - 12582912.0f, acc[gq][0][a]);
-                            acc[gq][1][a] = fmaf(D[gq].y, __int_as_float(r.y) - 12582912.0f, acc[gq][1][a]);
-                            acc[gq][2][a] = fmaf(D[gq].z, __int_as_float(r.z) - 12582912.0f, acc[gq][2][a]);
-                            acc[gq][3][a] = fmaf(D[gq].w, __int_as_float(r.w) - 12582912.0f, acc[gq][3][a]);
-                        }
+                        for (int n = 0; n < 16; n++)
+                            acc[n >> 2][n & 3][a] = fmaf(D[n], __int_as_float(p[e & 1][n]) - 12582912.0f, acc[n >> 2][n & 3][a]);
                     }
                 }
             }
@@ -678,12 +653,13 @@ __global__ __launch_bounds__(256, 2) void exact_gemm8_kernel(const uint8_t *__re
         __syncthreads();
     }
     if constexpr (MF) {
-        const int64_t tok = t0 + bj;
+        const int blk = bj >> 4, r = bj & 15;
+        const int64_t row = m0 + 16 * wv + 4 * blk;
 #pragma unroll
-        for (int gq = 0; gq < 4; gq++) {
-            const int64_t row = m0 + 16 * wv + 4 * gq;
+        for (int b = 0; b < 4; b++) {
+            const int64_t tok = t0 + 16 * b + r;
             if (tok < ne11 && row < ne01)
-                *(float4 *)(dst + tok * d_row + row) = make_float4(hsum8(acc[gq][0]), hsum8(acc[gq][1]), hsum8(acc[gq][2]), hsum8(acc[gq][3]));
+                *(float4 *)(dst + tok * d_row + row) = make_float4(hsum8(acc[b][0]), hsum8(acc[b][1]), hsum8(acc[b][2]), hsum8(acc[b][3]));
         }
     } else {
 #pragma unroll
@@ -699,19 +675,18 @@ __global__ __launch_bounds__(256, 2) void exact_gemm8_kernel(const uint8_t *__re
 }
 
 // The K-quant dots for many activation rows at once, tiled like exact_gemm8_kernel<., true> (64 x 64 outputs per workgroup, a
-// wave 16 weight rows x 64 activation rows, lane = activation row, weight words through the A-matrix broadcast of the 4 x 4 x 4
-// matrix instruction).  These dots keep ONE accumulator per output and add a term per sub-block of 32 elements, in order:
+// wave 16 weight rows x 64 activation rows per v_mfma_i32_16x16x4_4b_i8, weight words through its A-matrix broadcast).  These dots keep ONE accumulator per output and add a term per sub-block of 32 elements, in order:
 //   Q4_K:  acc = fma(d_x, d * float(sc * isum) - dmin * float(m * bsum), acc)       isum = sum q * x, bsum = sum x over the sub-block
 //   Q6_K:  acc = fma(d_x * d, float(sc0 * isum0 + sc1 * isum1), acc)                 isum0 / isum1 over the two halves of 16 elements
 // The integer sums are chains of matrix instructions over the element words of a sub-block (exact: integers); a stage is half a
 // super-block (four sub-blocks).  The bits are those of exact_dotsk_kernel and of the oracle.
 template <int WT>
-__global__ __launch_bounds__(256, 2) void exact_gemmk_kernel(const uint8_t *__restrict__ w, int64_t w_row, int64_t ne01, int64_t nsb,
+__global__ __launch_bounds__(256, 3) void exact_gemmk_kernel(const uint8_t *__restrict__ w, int64_t w_row, int64_t ne01, int64_t nsb,
                                                               const uint8_t *__restrict__ xm, int64_t x_row, int64_t ne11,
                                                               float *__restrict__ dst, int64_t d_row) {
     constexpr bool K4 = WT == SPY_HIP_Q4_K;
-    constexpr int WPL = XGB_TILE + 4;
-    __shared__ __align__(16) uint32_t s_wq[2][XGB_KB][8][WPL];     // element words of the weights, rows j, j + 4, ... side by side
+    constexpr int WPL = XGB_TILE + 16;                             // four weight planes are read at once: the padding puts them on different banks
+    __shared__ __align__(16) uint32_t s_wq[2][XGB_KB][8][WPL];     // element words of the weights
     __shared__ __align__(16) uint32_t s_xq[2][XGB_KB][8][XGB_TILE];
     __shared__ __align__(16) int32_t s_ws0[2][XGB_KB][XGB_TILE];   // Q4_K: sc          Q6_K: scale of elements 0..15
     __shared__ __align__(16) int32_t s_ws1[2][XGB_KB][XGB_TILE];   // Q4_K: m           Q6_K: scale of elements 16..31
@@ -719,13 +694,13 @@ __global__ __launch_bounds__(256, 2) void exact_gemmk_kernel(const uint8_t *__re
     __shared__ __align__(16) float s_xd[2][XGB_KB][XGB_TILE];
     __shared__ __align__(16) int32_t s_xb[2][XGB_KB][XGB_TILE];    // Q4_K: sum of the activation quants of the block
     const int tid = threadIdx.x;
-    const int wv = tid >> 6, bj = tid & 63, jj = tid & 3, grp = bj >> 2;
+    const int wv = tid >> 6, bj = tid & 63, blk = bj >> 4, r = bj & 15;
     const int64_t m0 = (int64_t)blockIdx.x * XGB_TILE, t0 = (int64_t)blockIdx.y * XGB_TILE;
 
     // loaders: waves 0 and 1 bring weights (a thread: one row, two of the stage's four sub-blocks), waves 2 and 3 activation blocks
     const bool ld_w = tid < 128;
     const int ld_row = tid & 63, ld_pair = (tid >> 6) & 1;
-    const int ld_slot = (ld_row & 3) * 16 + (ld_row >> 2);
+    const int ld_slot = ld_row;
     const uint8_t *ld_wrow = w + min(m0 + ld_row, ne01 - 1) * w_row;
     const uint32_t *ld_xsrc = (const uint32_t *)(xm + min(t0 + ld_row, ne11 - 1) * x_row) + ld_pair * 17;
     uint32_t g[17];                                                // activations: two Q8_0 blocks; weights: quant words and scale bytes
@@ -808,12 +783,14 @@ __global__ __launch_bounds__(256, 2) void exact_gemmk_kernel(const uint8_t *__re
         }
     };
 
-    float acc[4][4];
+    float acc[4][4];                                               // [b][v]: activation row 16b + r, weight row 16 * wave + 4 * blk + v
 #pragma unroll
-    for (int r = 0; r < 4; r++)
+    for (int b = 0; b < 4; b++)
 #pragma unroll
-        for (int c = 0; c < 4; c++) acc[r][c] = 0.0f;
-    const xgb_v4i zero4i = {0, 0, 0, 0};
+        for (int c = 0; c < 4; c++) acc[b][c] = 0.0f;
+    xgb_v16i zero16i;
+#pragma unroll
+    for (int n = 0; n < 16; n++) zero16i[n] = 0;
 
     const int64_t nstage = 2 * nsb;
     fetch(0);
@@ -822,66 +799,59 @@ __global__ __launch_bounds__(256, 2) void exact_gemmk_kernel(const uint8_t *__re
     for (int64_t s = 0; s < nstage; s++) {
         const int buf = (int)(s & 1);
         if (s + 1 < nstage) fetch(s + 1);
-        // rows 16 * wave + 4g + i sit at slot i * 16 + 4 * wave + g of their planes: one 16-byte read per i brings g = 0..3
-        xgb_v4f dw[4], dmn[4];
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            dw[i] = *(const xgb_v4f *)&s_wd[buf][0][i * 16 + 4 * wv];
-            if (K4) dmn[i] = *(const xgb_v4f *)&s_wd[buf][1][i * 16 + 4 * wv];
-        }
+        // this lane's four weight rows 16 * wave + 4 * blk + v: d, dmin of the super-block
+        const xgb_v4f dw = *(const xgb_v4f *)&s_wd[buf][0][16 * wv + 4 * blk];
+        xgb_v4f dmn = dw;
+        if (K4) dmn = *(const xgb_v4f *)&s_wd[buf][1][16 * wv + 4 * blk];
 #pragma unroll 1
         for (int half = 0; half < XGB_KB / 2; half++) {
-            const uint4 wq4 = *(const uint4 *)&s_wq[buf][2 * half + (grp >> 3)][grp & 7][jj * 16 + 4 * wv];      // lane group 8 * (block & 1) + e: rows 4g + j, g = 0..3
+            uint32_t wreg[4];                                      // lane block q, read i: word (4i + q) & 7 of sub-block 2 * half + (4i + q) / 8, row 16 * wave + r
+#pragma unroll
+            for (int i = 0; i < 4; i++) wreg[i] = s_wq[buf][2 * half + (i >> 1)][4 * (i & 1) + blk][16 * wv + r];
 #pragma unroll
             for (int kb2 = 0; kb2 < 2; kb2++) {
                 const int kb = 2 * half + kb2;
-                const float xd = s_xd[buf][kb][bj];
                 uint32_t xq[8];
 #pragma unroll
                 for (int e = 0; e < 8; e++) xq[e] = s_xq[buf][kb][e][bj];
-                xgb_v4i s0[4], s1[4];                              // [i][g]: scale integers of row 4g + i
-#pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    s0[i] = *(const xgb_v4i *)&s_ws0[buf][kb][i * 16 + 4 * wv];
-                    s1[i] = *(const xgb_v4i *)&s_ws1[buf][kb][i * 16 + 4 * wv];
-                }
-                // integer sums of the sub-block: isum[g] (Q4_K) or the two halves lo[g], hi[g] (Q6_K), component i = row 4g + i
-                xgb_v4i lo[4] = {zero4i, zero4i, zero4i, zero4i}, hi[4] = {zero4i, zero4i, zero4i, zero4i};
+                const xgb_v4i s0 = *(const xgb_v4i *)&s_ws0[buf][kb][16 * wv + 4 * blk], s1 = *(const xgb_v4i *)&s_ws1[buf][kb][16 * wv + 4 * blk];
+                // integer sums of the sub-block, register 4b + v: isum (Q4_K) or the two halves lo, hi (Q6_K)
+                xgb_v16i lo = zero16i, hi = zero16i;
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
-                    if (K4 || e < 4) xgb_mfma_word_acc(lo, wq4, xq[e], kb2 * 8 + e);
-                    else xgb_mfma_word_acc(hi, wq4, xq[e], kb2 * 8 + e);
+                    if (K4 || e < 4) lo = xgb_mfma16(wreg[2 * kb2 + (e >> 2)], xq[e], lo, e & 3);
+                    else hi = xgb_mfma16(wreg[2 * kb2 + (e >> 2)], xq[e], hi, e & 3);
                 }
-                if (K4) {
-                    const int32_t xb = s_xb[buf][kb][bj];
 #pragma unroll
-                    for (int gq = 0; gq < 4; gq++)
+                for (int b = 0; b < 4; b++) {
+                    const float xd = s_xd[buf][kb][16 * b + r];
+                    if (K4) {
+                        const int32_t xb = s_xb[buf][kb][16 * b + r];
 #pragma unroll
-                        for (int i = 0; i < 4; i++) {
-                            const float pos = dw[i][gq] * (float)__mul24(s0[i][gq], lo[gq][i]);
-                            const float neg = dmn[i][gq] * (float)__mul24(s1[i][gq], xb);
-                            acc[gq][i] = fmaf(xd, pos - neg, acc[gq][i]);
+                        for (int v = 0; v < 4; v++) {
+                            const float pos = dw[v] * (float)__mul24(s0[v], lo[4 * b + v]);
+                            const float neg = dmn[v] * (float)__mul24(s1[v], xb);
+                            acc[b][v] = fmaf(xd, pos - neg, acc[b][v]);
                         }
-                } else {
+                    } else {
 #pragma unroll
-                    for (int gq = 0; gq < 4; gq++)
-#pragma unroll
-                        for (int i = 0; i < 4; i++) {
-                            const int32_t sv = __mul24(s0[i][gq], lo[gq][i]) + __mul24(s1[i][gq], hi[gq][i]);
-                            const float dd = xd * dw[i][gq];
-                            acc[gq][i] = fmaf(dd, (float)sv, acc[gq][i]);
+                        for (int v = 0; v < 4; v++) {
+                            const int32_t sv = __mul24(s0[v], lo[4 * b + v]) + __mul24(s1[v], hi[4 * b + v]);
+                            const float dd = xd * dw[v];
+                            acc[b][v] = fmaf(dd, (float)sv, acc[b][v]);
                         }
+                    }
                 }
             }
         }
         if (s + 1 < nstage) put(buf ^ 1, s + 1);
         __syncthreads();
     }
-    const int64_t tok = t0 + bj;
+    const int64_t row = m0 + 16 * wv + 4 * blk;
 #pragma unroll
-    for (int gq = 0; gq < 4; gq++) {
-        const int64_t row = m0 + 16 * wv + 4 * gq;
-        if (tok < ne11 && row < ne01) *(float4 *)(dst + tok * d_row + row) = make_float4(acc[gq][0], acc[gq][1], acc[gq][2], acc[gq][3]);
+    for (int b = 0; b < 4; b++) {
+        const int64_t tok = t0 + 16 * b + r;
+        if (tok < ne11 && row < ne01) *(float4 *)(dst + tok * d_row + row) = make_float4(acc[b][0], acc[b][1], acc[b][2], acc[b][3]);
     }
 }
 
