@@ -355,6 +355,39 @@ def test_prompt_attention_kernels_at_the_7b_width(hip, monkeypatch):
     _same_bits(got["1"], got["0"], "7B width, 700 tokens after 300")
 
 
+@pytest.mark.timeout(600)
+@pytest.mark.parametrize("name,kw", [
+    ("Q4_0 body, Q6_K head", dict(wtype=O.Q4_0, t_out=O.Q6_K)),
+    ("Q8_0", dict(wtype=O.Q8_0)),
+    ("Q4_K_M mix", dict(wtype=O.Q4_K, t_out=O.Q6_K, tensor_types={"attn_v": O.Q6_K, "ffn_down": O.Q6_K})),
+])
+def test_default_engine_at_7b_width_prompt_and_tokens_have_the_oracle_bits(name, kw):
+    """The engine as it comes (order 1, no switch set), two layers of the 7B width: a 70-token prompt (tiled exact MatMul of the
+    layer's weight types, the three causal attention kernels), a second prompt pass of 33 tokens on top of it, then 6 greedy
+    steps through the fused single-token kernels.  Logits of both prompt passes and every generated token equal the CPU
+    oracle's, bit for bit."""
+    from spy_amd import _lib as H
+    from spy_amd import model as M
+    from tests.model_util import OracleModel, k_quant_quantizer
+    H.init(0)
+    cfg = M.Config.llama2_7b(n_ctx=128, **kw)
+    cfg.n_layer = 2
+    tensors = M.synth_model(cfg, seed=77, quantizer=k_quant_quantizer)
+    eng, ora = M.Engine(cfg, tensors), OracleModel(cfg, tensors, nthread=min(16, os.cpu_count() or 8))
+    assert eng.order() == 1
+    prompt = np.random.default_rng(12).integers(0, cfg.n_vocab, 103).astype(np.int32)
+    _same_bits(eng.forward_last(prompt[:70], 0), ora.forward(prompt[:70], 0)[-1], name + ": last row of a 70-token prompt")
+    lg = ora.forward(prompt[70:], 70)
+    _same_bits(eng.forward(prompt[70:], 70), lg, name + ": 33 tokens on top of 70")
+    first = int(np.argmax(lg[-1]))
+    want = [first]
+    for i in range(6):
+        want.append(int(np.argmax(ora.forward(np.array([want[-1]], np.int32), 103 + i)[0])))
+    got = eng.decode_greedy(first, 103, 6)
+    assert [int(t) for t in got] == want[1:], (name, got, want)
+    eng.close()
+
+
 @pytest.mark.timeout(900)
 @pytest.mark.parametrize("wtype", [O.Q4_0, O.Q8_0])
 def test_llama2_7b_greedy_32_tokens_identical(wtype):
