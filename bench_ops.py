@@ -36,7 +36,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--json", action="store_true")
     ap.add_argument("--reps", type=int, default=20)
-    ap.add_argument("--skip", default="", help="comma list of: peaks, gemv, gemm, prompt_attention, attention")
+    ap.add_argument("--skip", default="", help="comma list of: peaks, gemv, gemm, prompt_attention, exact_prompt, attention")
     args = ap.parse_args()
     skip = set(args.skip.split(",")) if args.skip else set()
 
@@ -199,6 +199,57 @@ def main():
             print("| %d | %d | %.1f | %.0f | %.3f |" % (past, T, us, flops / us / 1e6, flops / (us * 1e-6) / 2.5e15), flush=True)
             emit({"op": "prompt_attention", "past": past, "T": T, "us": us, "tflops": flops / us / 1e6})
         print("\nmean of the two chunks of a 4096-token prompt: %.1f µs per layer and chunk\n" % (tot / 2), flush=True)
+        for b in (dq, dk, dv, do):
+            b.free()
+
+    if "exact_prompt" not in skip:
+        # the prompt kernels of summation order 1: tiled exact MatMul (`spy_hip_op_matmul` with the exact-order switch on, activations
+        # quantized inside the call) and the three causal attention kernels behind `spy_hip_prompt_attention_exact`
+        print("## Prompt kernels in the host backend's summation order (order 1): tiled exact MatMul and causal exact attention, 2048 activation rows\n")
+        print("| weights | M x K | T | measured µs (Q8_0 quantization of the activations included) | TMAC/s |")
+        print("|---|---|---|---|---|")
+        prev = L.spy_hip_set_exact_order(1)
+        T = 2048
+        for wt in (H.Q4_0, H.Q8_0, H.Q4_K, H.Q6_K):
+            for (M_, K) in ((4096, 4096), (11008, 4096), (4096, 11008)):
+                w = weights(wt, M_, K)
+                dw = H.DeviceBuffer.from_numpy(w)
+                dx = H.DeviceBuffer.from_numpy(np.random.default_rng(M_ + K).standard_normal((T, K)).astype(np.float32))
+                dd = H.DeviceBuffer(T * M_ * 4)
+                tw, tx, td = H.tensor(dw, wt, [K, M_]), H.tensor(dx, H.F32, [K, T]), H.tensor(dd, H.F32, [M_, T])
+                need = L.spy_hip_op_matmul_scratch_size(C.byref(tw), C.byref(tx))
+                scr = H.DeviceBuffer(need)
+
+                def run():
+                    H.check(L.spy_hip_op_matmul(None, C.byref(tw), C.byref(tx), C.byref(td), scr.ptr, need), "spy_hip_op_matmul")
+                us = time_us(run, 1)
+                print("| %s | %d x %d | %d | %.1f | %.1f |" % (TYPE_NAMES[wt], M_, K, T, us, T * M_ * K / us / 1e6), flush=True)
+                emit({"op": "exact_matmul", "wtype": TYPE_NAMES[wt], "M": M_, "K": K, "T": T, "us": us, "tmacs": T * M_ * K / us / 1e6})
+                for b in (dw, dx, dd, scr):
+                    b.free()
+        L.spy_hip_set_exact_order(prev)
+        print()
+        print("| cached before | queries | measured µs (scores + softmax + product with V^T) | fp32 fmas per second, T (256 per pair of a query and a visible position) |")
+        print("|---|---|---|---|")
+        Hh, hd, n_ctx = 32, 128, 4096
+        rng = np.random.default_rng(6)
+        dq = H.DeviceBuffer.from_numpy(rng.standard_normal((T, Hh * hd)).astype(np.float32))
+        dk = H.DeviceBuffer.from_numpy(rng.standard_normal((n_ctx, Hh * hd)).astype(np.float16))
+        dv = H.DeviceBuffer.from_numpy(rng.standard_normal((Hh * hd, n_ctx)).astype(np.float16))
+        do = H.DeviceBuffer(T * Hh * hd * 4)
+        for past in (0, 2048):
+            need = L.spy_hip_prompt_attention_exact_scratch_size(T, Hh, past)
+            scr = H.DeviceBuffer(need)
+
+            def run():
+                H.check(L.spy_hip_prompt_attention_exact(None, dq.ptr, dk.ptr, dv.ptr, do.ptr, T, Hh, hd, past, n_ctx, past + T, 1.0 / np.sqrt(hd), scr.ptr, need),
+                        "spy_hip_prompt_attention_exact")
+            us = time_us(run, 3)
+            pairs = (T * past + T * (T + 1) / 2) * Hh
+            print("| %d | %d | %.1f | %.1f |" % (past, T, us * 3, pairs * 256 / (us * 3) / 1e6), flush=True)
+            emit({"op": "prompt_attention_exact", "past": past, "T": T, "us": us * 3})
+            scr.free()
+        print(flush=True)
         for b in (dq, dk, dv, do):
             b.free()
 
