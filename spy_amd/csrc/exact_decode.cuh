@@ -171,7 +171,7 @@ static __device__ __forceinline__ float xg_exact_sum(const float (&g)[NG], int n
         int pre = next_slow(0);
         if (pre >= 0) request(pre);
         int bits = __builtin_amdgcn_readfirstlane(__float_as_int(s));             // the running sum as a scalar
-        int nfall = 0;
+        [[maybe_unused]] int nfall = 0;
         for (int c = 0; c < nchunk; c++) {
             const int eb = __builtin_amdgcn_readlane(veb, c), t = (bits & 1) ? __builtin_amdgcn_readlane(vt1, c) : __builtin_amdgcn_readlane(vt0, c);
             const int nb = bits + t;
