@@ -459,18 +459,24 @@ __global__ __launch_bounds__(256) void exact_dots8_kernel(xdesc w, const uint8_t
     if (l == 0) *(float *)xat(d, i01, i11, i02, i03) = acc;
 }
 
-// The same Q4_0 / Q8_0 dots for many activation rows at once (prompts): a workgroup computes a tile of 64 weight rows
-// by 64 activation rows, a thread 4 x 4 output elements with the eight accumulators of each in registers.  Every
-// accumulator still receives its block terms in block order, fma(d_w * d_x, float(integer sum of its four products),
-// acc), and the eight are added in hsum_float_8's tree at the end, so the results are those of exact_dots8_kernel bit
-// for bit; what changes is that a weight block and an activation block are unpacked once per tile (into LDS, as
-// words in element order: the low nibbles of a Q4_0 block first, then the high ones) instead of once per output.
-// The integer sums are accumulated onto 0x4B400000, the bits of 1.5 * 2^23: read as a float, the sum minus
-// 12582912.0f is the exact conversion (|sum| < 2^22).  The hardware multiplies the signed bytes as they are, which equals
-// the host's abs / sign / saturating pair sum (vec_util.h:101-110) as long as no ACTIVATION byte is -128; the launcher
-// takes this kernel only for activations that this library quantized itself (|q| <= 127).
+// The Q4_0 / Q8_0 dots for many activation rows at once (prompts): a workgroup computes a tile of 64 weight rows by 64 activation
+// rows, a wave 16 x 64 of it, a lane 16 output elements with the eight accumulators of each in registers.  Every accumulator still
+// receives its block terms in block order, fma(d_w * d_x, float(integer sum of its four products), acc), and the eight are added in
+// hsum_float_8's tree at the end, so the results are those of exact_dots8_kernel bit for bit; what changes is that a weight block
+// and an activation block are unpacked once per tile (into LDS, as words in element order: the low nibbles of a Q4_0 block first,
+// then the high ones) instead of once per output, and that the integer sums come from the matrix cores.
+// v_mfma_*_16x16x4_4b_* computes four 16 x 16 products over four elements each, lane l supplying row l % 16 of A and column l % 16 of
+// B for product l / 16: with the A-matrix broadcast (cbsz:2 abid:q: all four products take the A operand of lane block q) one
+// instruction multiplies a wave's 16 weight rows by its 64 activation rows over one element word -- exactly one accumulator's share
+// of a block, nothing wasted -- and the four lane blocks can hold the words of four different element words: one LDS read per lane
+// feeds four instructions.  Output register 4b + v of lane (blk, r): weight row 16 * wave + 4 * blk + v, activation row 16b + r.
+// The scale products d_w * d_x of a block come the same way from v_mfma_f32_16x16x1_4b_f32 (one product per output, rounded once:
+// the bits of the vector multiply).
+// The hardware multiplies the signed values as they are, which equals the host's abs / sign / saturating pair sum
+// (vec_util.h:101-110) as long as no ACTIVATION byte is -128; the launcher takes this kernel only for activations that this
+// library quantized itself (|q| <= 127).
 #define XGB_TILE 64
-#define XGB_KB 4          // blocks per stage
+#define XGB_KB 4          // blocks per stage of the K-quant kernel
 typedef int xgb_v4i __attribute__((ext_vector_type(4)));
 typedef float xgb_v4f __attribute__((ext_vector_type(4)));
 typedef int xgb_v16i __attribute__((ext_vector_type(16)));
@@ -484,197 +490,139 @@ __device__ __forceinline__ xgb_v16i xgb_mfma16(uint32_t w, uint32_t x, const xgb
     default: return __builtin_amdgcn_mfma_i32_16x16x4i8((int)w, (int)x, c, 2, 3, 0);
     }
 }
-// MF = true: the integer sums come from the matrix cores instead.  v_mfma_i32_16x16x4_4b_i8 computes four 16 x 16 products over
-// four elements each, exactly one accumulator's share of a block for 16 weight rows x 64 activation rows.  A wave holds such a
-// tile, a lane again 16 outputs with 8 accumulators each, and the vector units are left with the subtraction and the fma per term.
-template <int WT, bool MF>
-__global__ __launch_bounds__(256, 2) void exact_gemm8_kernel(const uint8_t *__restrict__ w, int64_t w_row, int64_t ne01, int64_t nb,
-                                                              const uint8_t *__restrict__ xm, int64_t x_row, int64_t ne11,
-                                                              float *__restrict__ dst, int64_t d_row) {
-    constexpr int WPL = MF ? XGB_TILE + 16 : XGB_TILE;             // words per weight plane: MF reads four planes at once, the padding puts them on different banks
-    __shared__ __align__(16) uint32_t s_wq[2][XGB_KB][8][WPL];
-    __shared__ __align__(16) uint32_t s_xq[2][XGB_KB][8][XGB_TILE];
-    __shared__ __align__(16) float s_wd[2][XGB_KB][XGB_TILE];
-    __shared__ __align__(16) float s_xd[2][XGB_KB][XGB_TILE];
+// The integer sums are delivered as floats: the quants are converted to fp16 once, when a tile is staged (every int8 is an fp16
+// exactly), and v_mfma_f32_16x16x4_4b_f16 adds the four products of an accumulator's share in fp32 -- integers below 2^16, so the
+// sum is exact whatever order the hardware adds them in.  The vector units are left with ONE instruction per term, the fma onto
+// the accumulator (with the int8 form of the instruction and a biased accumulator they need a subtraction as well: 0.88 ms per
+// GEMM of a 2048-row chunk against 0.75).  A stage is two blocks (the fp16 operands take twice the LDS).
+typedef _Float16 xgf_h2 __attribute__((ext_vector_type(2)));
+typedef _Float16 xgf_h4 __attribute__((ext_vector_type(4)));
+// bytes v0..v3 (already biased to 0..255 resp. 0..15) -> fp16 pairs (v0 - sub, v1 - sub), (v2 - sub, v3 - sub): 0x6400 | v is the fp16
+// 1024 + v, and the subtraction of 1024 + bias is exact
+__device__ __forceinline__ uint2 xgf_bytes_to_h4(uint32_t v, float sub) {
+    const uint32_t lo = __builtin_amdgcn_perm(0x64646464u, v, 0x04010400u), hi = __builtin_amdgcn_perm(0x64646464u, v, 0x04030402u);
+    const xgf_h2 c = {(_Float16)sub, (_Float16)sub};
+    const xgf_h2 l2 = __builtin_bit_cast(xgf_h2, lo) - c, h2 = __builtin_bit_cast(xgf_h2, hi) - c;
+    return make_uint2(__builtin_bit_cast(uint32_t, l2), __builtin_bit_cast(uint32_t, h2));
+}
+__device__ __forceinline__ xgb_v16f xgf_mfma16(const uint2 &w, const uint2 &x, int abid) {
+    const xgf_h4 a = __builtin_bit_cast(xgf_h4, w), b = __builtin_bit_cast(xgf_h4, x);
+    const xgb_v16f c = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    switch (abid) {
+    case 0: return __builtin_amdgcn_mfma_f32_16x16x4f16(a, b, c, 2, 0, 0);
+    case 1: return __builtin_amdgcn_mfma_f32_16x16x4f16(a, b, c, 2, 1, 0);
+    case 2: return __builtin_amdgcn_mfma_f32_16x16x4f16(a, b, c, 2, 2, 0);
+    default: return __builtin_amdgcn_mfma_f32_16x16x4f16(a, b, c, 2, 3, 0);
+    }
+}
+#define XGF_KB 2
+template <int WT>
+__global__ __launch_bounds__(256, 2) void exact_gemm8f_kernel(const uint8_t *__restrict__ w, int64_t w_row, int64_t ne01, int64_t nb,
+                                                               const uint8_t *__restrict__ xm, int64_t x_row, int64_t ne11,
+                                                               float *__restrict__ dst, int64_t d_row) {
+    constexpr int WPL = XGB_TILE + 8;
+    __shared__ __align__(16) uint2 s_wq[2][XGF_KB][8][WPL];        // [buffer][block][element word][weight row]: four fp16
+    __shared__ __align__(16) uint2 s_xq[2][XGF_KB][8][XGB_TILE];
+    __shared__ __align__(16) float s_wd[2][XGF_KB][XGB_TILE];
+    __shared__ __align__(16) float s_xd[2][XGF_KB][XGB_TILE];
     const int tid = threadIdx.x;
-    const int mg = tid & 15, tg = tid >> 4;                              // MF = false: 4 weight rows x 4 activation rows per thread
-    const int wv = tid >> 6, bj = tid & 63;                              // MF = true: wave, activation row of the tile
+    const int wv = tid >> 6, bj = tid & 63, blk = bj >> 4, r = bj & 15;
     const int64_t m0 = (int64_t)blockIdx.x * XGB_TILE, t0 = (int64_t)blockIdx.y * XGB_TILE;
 
-    // loaders: waves 0 and 1 bring weight blocks, waves 2 and 3 activation blocks; a thread takes two neighbouring
-    // blocks of one row (36 bytes of Q4_0, 68 of Q8_0: whole aligned words) per stage
+    // loaders: a thread takes ONE block of one row per stage -- waves 0, 1: weight rows, blocks 0 / 1 of the stage; waves 2, 3: activation
+    // rows.  Two neighbouring blocks are 36 (Q4_0) or 68 bytes (Q8_0), whole aligned words; the second block starts in the middle of a word.
     const bool ld_w = tid < 128;
-    const int ld_row = tid & 63, ld_pair = (tid >> 6) & 1;
-    const int ld_slot = ld_row;
-    constexpr int NWQ = WT == SPY_HIP_Q4_0 ? 9 : 17;
+    const int ld_row = tid & 63, ld_blk = (tid >> 6) & 1;
+    constexpr int NWQ = WT == SPY_HIP_Q4_0 ? 9 : 17;               // words per pair of weight blocks
     const uint32_t *ld_src;
-    if (ld_w) ld_src = (const uint32_t *)(w + min(m0 + ld_row, ne01 - 1) * w_row) + ld_pair * NWQ;
-    else ld_src = (const uint32_t *)(xm + min(t0 + ld_row, ne11 - 1) * x_row) + ld_pair * 17;
-    uint32_t g[17];
+    if (ld_w) ld_src = (const uint32_t *)(w + min(m0 + ld_row, ne01 - 1) * w_row) + (WT == SPY_HIP_Q4_0 ? 4 : 8) * ld_blk;
+    else ld_src = (const uint32_t *)(xm + min(t0 + ld_row, ne11 - 1) * x_row) + 8 * ld_blk;
+    uint32_t g[9];
     auto fetch = [&](int64_t stage) {
-        const uint32_t *p = ld_src + stage * (ld_w ? 2 * NWQ : 34);
+        const uint32_t *p = ld_src + stage * (ld_w ? NWQ : 17);
         if (ld_w && WT == SPY_HIP_Q4_0) {
 #pragma unroll
-            for (int i = 0; i < 9; i++) g[i] = p[i];
+            for (int i = 0; i < 5; i++) g[i] = p[i];
         } else {
 #pragma unroll
-            for (int i = 0; i < 17; i++) g[i] = p[i];
+            for (int i = 0; i < 9; i++) g[i] = p[i];
         }
     };
     auto put = [&](int buf) {
         if (ld_w && WT == SPY_HIP_Q4_0) {
-            // block 0: scale in the low half of g[0], 16 quant bytes from byte 2; block 1: scale in the high half of g[4], quants g[5..8]
-            const int k0 = 2 * ld_pair;
-            s_wd[buf][k0][ld_row] = h2f_tab((uint16_t)(g[0] & 0xFFFFu));
-            s_wd[buf][k0 + 1][ld_row] = h2f_tab((uint16_t)(g[4] >> 16));
+            // block 0 of the pair: scale in the low half of g[0], quant bytes from byte 2; block 1: scale in the high half of g[0] (= word 4
+            // of the pair), quants g[1..4]
+            s_wd[buf][ld_blk][ld_row] = h2f_tab((uint16_t)(ld_blk ? g[0] >> 16 : g[0] & 0xFFFFu));
 #pragma unroll
             for (int k = 0; k < 4; k++) {
-                const uint32_t q0 = __builtin_amdgcn_alignbit(g[k + 1], g[k], 16), q1 = g[5 + k];
-                uint32_t lo0 = q0 & 0x0F0F0F0Fu, hi0 = (q0 >> 4) & 0x0F0F0F0Fu, lo1 = q1 & 0x0F0F0F0Fu, hi1 = (q1 >> 4) & 0x0F0F0F0Fu;
-                // per byte n - 8: n + 128 - 8 never borrows across bytes, then the top bit is flipped back
-                lo0 = ((lo0 | 0x80808080u) - 0x08080808u) ^ 0x80808080u; hi0 = ((hi0 | 0x80808080u) - 0x08080808u) ^ 0x80808080u;
-                lo1 = ((lo1 | 0x80808080u) - 0x08080808u) ^ 0x80808080u; hi1 = ((hi1 | 0x80808080u) - 0x08080808u) ^ 0x80808080u;
-                s_wq[buf][k0][k][ld_slot] = lo0; s_wq[buf][k0][4 + k][ld_slot] = hi0;
-                s_wq[buf][k0 + 1][k][ld_slot] = lo1; s_wq[buf][k0 + 1][4 + k][ld_slot] = hi1;
+                const uint32_t q = ld_blk ? g[1 + k] : __builtin_amdgcn_alignbit(g[k + 1], g[k], 16);
+                s_wq[buf][ld_blk][k][ld_row] = xgf_bytes_to_h4(q & 0x0F0F0F0Fu, 1032.0f);              // low nibbles: elements 4k .. 4k + 3, n - 8
+                s_wq[buf][ld_blk][4 + k][ld_row] = xgf_bytes_to_h4((q >> 4) & 0x0F0F0F0Fu, 1032.0f);   // high nibbles: elements 16 + 4k ..
             }
         } else {
-            // Q8_0 pair: block 0 = scale in the low half of g[0] and 32 quant bytes from byte 2, block 1 = scale in the high half
-            // of g[8] and quants g[9..16]
-            float (*sd)[XGB_TILE] = ld_w ? s_wd[buf] : s_xd[buf];
-            const int k0 = 2 * ld_pair;
-            sd[k0][ld_row] = h2f_tab((uint16_t)(g[0] & 0xFFFFu));
-            sd[k0 + 1][ld_row] = h2f_tab((uint16_t)(g[8] >> 16));
+            // Q8_0: block 0 = scale in the low half of g[0], quants from byte 2; block 1 = scale in the high half of g[0] (word 8 of the pair), quants g[1..8]
+            const float d = h2f_tab((uint16_t)(ld_blk ? g[0] >> 16 : g[0] & 0xFFFFu));
+            if (ld_w) s_wd[buf][ld_blk][ld_row] = d; else s_xd[buf][ld_blk][ld_row] = d;
 #pragma unroll
             for (int k = 0; k < 8; k++) {
-                const uint32_t q0 = __builtin_amdgcn_alignbit(g[k + 1], g[k], 16), q1 = g[9 + k];
-                if (ld_w) { s_wq[buf][k0][k][ld_slot] = q0; s_wq[buf][k0 + 1][k][ld_slot] = q1; }
-                else { s_xq[buf][k0][k][ld_slot] = q0; s_xq[buf][k0 + 1][k][ld_slot] = q1; }
+                const uint32_t q = ld_blk ? g[1 + k] : __builtin_amdgcn_alignbit(g[k + 1], g[k], 16);
+                const uint2 h = xgf_bytes_to_h4(q ^ 0x80808080u, 1152.0f);                               // signed bytes: b + 128, then - 128
+                if (ld_w) s_wq[buf][ld_blk][k][ld_row] = h; else s_xq[buf][ld_blk][k][ld_row] = h;
             }
         }
     };
 
     float acc[4][4][8];
 #pragma unroll
-    for (int r = 0; r < 4; r++)
+    for (int b = 0; b < 4; b++)
 #pragma unroll
         for (int c = 0; c < 4; c++)
 #pragma unroll
-            for (int a = 0; a < 8; a++) acc[r][c][a] = 0.0f;
+            for (int a = 0; a < 8; a++) acc[b][c][a] = 0.0f;
+    const xgb_v16f zero16 = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
 
-    xgb_v16i bias16;
-    xgb_v16f zero16;
-#pragma unroll
-    for (int n = 0; n < 16; n++) { bias16[n] = 0x4B400000; zero16[n] = 0.0f; }
-    const int64_t nstage = nb / XGB_KB;
+    const int64_t nstage = nb / XGF_KB;
     fetch(0);
     put(0);
     __syncthreads();
     for (int64_t s = 0; s < nstage; s++) {
         const int buf = (int)(s & 1);
         if (s + 1 < nstage) fetch(s + 1);
-        if constexpr (MF) {
-            // v_mfma_i32_16x16x4_4b_i8: four 16 x 16 x 4 products at once, lane l supplying row l % 16 of A and column l % 16 of B for
-            // product l / 16.  With the A-matrix broadcast (cbsz:2 abid:q) all four use the weight words held by lane block q, so
-            // one instruction multiplies the wave's 16 weight rows by its 64 activation rows over one element word, and the four lane
-            // blocks can hold the words of four different (block, element word) pairs: a 4-byte LDS read per lane covers four
-            // instructions.  Output register 4b + v of lane (blk, r): weight row 16 * wave + 4 * blk + v, activation row 16b + r.
-            // The scale products d_w * d_x come the same way from v_mfma_f32_16x16x1_4b_f32 (one product per output, rounded once:
-            // the bits of the vector multiply).
-            const int blk = bj >> 4, r = bj & 15;
+        // output register 4b + v of lane (blk, r): weight row 16 * wave + 4 * blk + v, activation row 16b + r
 #pragma unroll 1
-            for (int half = 0; half < XGB_KB / 2; half++) {
-                const float wdreg = s_wd[buf][2 * half + (blk & 1)][16 * wv + r];       // lane block q: scales of block 2 * half + (q & 1)
-                uint32_t wreg[4];                                                          // lane block q, read i: word (4i + q) & 7 of block 2 * half + (4i + q) / 8
+        for (int kb = 0; kb < XGF_KB; kb++) {
+            const float wdreg = s_wd[buf][kb][16 * wv + r], xdl = s_xd[buf][kb][bj];
+            const uint2 w0 = s_wq[buf][kb][blk][16 * wv + r], w1 = s_wq[buf][kb][4 + blk][16 * wv + r];      // lane block q holds words q and 4 + q
+            uint2 xql[8];
 #pragma unroll
-                for (int i = 0; i < 4; i++) wreg[i] = s_wq[buf][2 * half + (i >> 1)][4 * (i & 1) + blk][16 * wv + r];
-#pragma unroll
-                for (int kb2 = 0; kb2 < 2; kb2++) {
-                    const int kb = 2 * half + kb2;
-                    const float xdl = s_xd[buf][kb][bj];                    // the B operands are the lane's own activation row bj = 16 * blk + r
-                    uint32_t xql[8];
-#pragma unroll
-                    for (int e = 0; e < 8; e++) xql[e] = s_xq[buf][kb][e][bj];
-                    const xgb_v16f D = kb2 == 0 ? __builtin_amdgcn_mfma_f32_16x16x1f32(wdreg, xdl, zero16, 2, 0, 0)
-                                                : __builtin_amdgcn_mfma_f32_16x16x1f32(wdreg, xdl, zero16, 2, 1, 0);
-                    // the matrix instruction of word e + 1 is issued before the vector work on the results of word e
-                    xgb_v16i p[2];
-                    p[0] = xgb_mfma16(wreg[2 * kb2], xql[0], bias16, 0);
-#pragma unroll
-                    for (int e = 0; e < 8; e++) {
-                        if (e + 1 < 8) p[(e + 1) & 1] = xgb_mfma16(wreg[2 * kb2 + ((e + 1) >> 2)], xql[e + 1], bias16, (e + 1) & 3);
-                        const int a = WT == SPY_HIP_Q4_0 ? ((e + 4) & 7) : e;
-#pragma unroll
-                        for (int n = 0; n < 16; n++)
-                            acc[n >> 2][n & 3][a] = fmaf(D[n], __int_as_float(p[e & 1][n]) - 12582912.0f, acc[n >> 2][n & 3][a]);
-                    }
-                }
-            }
-        } else {
-#pragma unroll 1
-        for (int kb = 0; kb < XGB_KB; kb++) {
-            const float4 wd4 = *(const float4 *)&s_wd[buf][kb][4 * mg], xd4 = *(const float4 *)&s_xd[buf][kb][4 * tg];
-            const float wd[4] = {wd4.x, wd4.y, wd4.z, wd4.w}, xd[4] = {xd4.x, xd4.y, xd4.z, xd4.w};
-            float D[4][4];
-#pragma unroll
-            for (int r = 0; r < 4; r++)
-#pragma unroll
-                for (int c = 0; c < 4; c++) D[r][c] = wd[r] * xd[c];
+            for (int e = 0; e < 8; e++) xql[e] = s_xq[buf][kb][e][bj];
+            const xgb_v16f D = __builtin_amdgcn_mfma_f32_16x16x1f32(wdreg, xdl, zero16, 2, 0, 0);
+            // the matrix instruction of word e + 1 is issued before the vector work on the results of word e
+            xgb_v16f p[2];
+            p[0] = xgf_mfma16(w0, xql[0], 0);
 #pragma unroll
             for (int e = 0; e < 8; e++) {
-                const uint4 wq4 = *(const uint4 *)&s_wq[buf][kb][e][4 * mg], xq4 = *(const uint4 *)&s_xq[buf][kb][e][4 * tg];
-                const uint32_t wq[4] = {wq4.x, wq4.y, wq4.z, wq4.w}, xq[4] = {xq4.x, xq4.y, xq4.z, xq4.w};
-                // accumulator of element word e: Q4_0 keeps the low nibbles (elements 0..15) in 4..7 and the high ones in 0..3
-                // (vec_dot.h:42-86), Q8_0 elements 4l..4l+3 in accumulator l (vec_dot.h:88-115)
+                if (e + 1 < 8) p[(e + 1) & 1] = xgf_mfma16(e + 1 < 4 ? w0 : w1, xql[e + 1], (e + 1) & 3);
+                __builtin_amdgcn_sched_barrier(0);      // keeps the matrix instruction ahead of the fmas below (else the compiler issues it after them and waits for it)
                 const int a = WT == SPY_HIP_Q4_0 ? ((e + 4) & 7) : e;
-                // The sixteen integer sums of this word in one assembly block: the three-operand form takes the constant from a
-                // scalar register (the builtin first copies it into every destination).  The compiler cannot see that these
-                // are dot instructions, whose results other vector instructions may only read a few cycles later, so the
-                // block ends with the wait itself.
-                int32_t p[16];
-#define XGB_DOT(r, c) "v_dot4_i32_i8 %[p" #r #c "], %[w" #r "], %[x" #c "], %[b]\n"
-                asm(XGB_DOT(0, 0) XGB_DOT(0, 1) XGB_DOT(0, 2) XGB_DOT(0, 3) XGB_DOT(1, 0) XGB_DOT(1, 1) XGB_DOT(1, 2) XGB_DOT(1, 3)
-                    XGB_DOT(2, 0) XGB_DOT(2, 1) XGB_DOT(2, 2) XGB_DOT(2, 3) XGB_DOT(3, 0) XGB_DOT(3, 1) XGB_DOT(3, 2) XGB_DOT(3, 3)
-                    "s_nop 4"
-                    : [p00] "=&v"(p[0]), [p01] "=&v"(p[1]), [p02] "=&v"(p[2]), [p03] "=&v"(p[3]), [p10] "=&v"(p[4]), [p11] "=&v"(p[5]),
-                      [p12] "=&v"(p[6]), [p13] "=&v"(p[7]), [p20] "=&v"(p[8]), [p21] "=&v"(p[9]), [p22] "=&v"(p[10]), [p23] "=&v"(p[11]),
-                      [p30] "=&v"(p[12]), [p31] "=&v"(p[13]), [p32] "=&v"(p[14]), [p33] "=&v"(p[15])
-                    : [w0] "v"(wq[0]), [w1] "v"(wq[1]), [w2] "v"(wq[2]), [w3] "v"(wq[3]), [x0] "v"(xq[0]), [x1] "v"(xq[1]), [x2] "v"(xq[2]),
-                      [x3] "v"(xq[3]), [b] "s"(0x4B400000));
-#undef XGB_DOT
 #pragma unroll
-                for (int r = 0; r < 4; r++)
-#pragma unroll
-                    for (int c = 0; c < 4; c++)
-                        acc[r][c][a] = fmaf(D[r][c], __int_as_float(p[4 * r + c]) - 12582912.0f, acc[r][c][a]);
+                for (int n = 0; n < 16; n++) acc[n >> 2][n & 3][a] = fmaf(D[n], p[e & 1][n], acc[n >> 2][n & 3][a]);
+                __builtin_amdgcn_sched_barrier(0);
             }
-        }
         }
         if (s + 1 < nstage) put(buf ^ 1);
         __syncthreads();
     }
-    if constexpr (MF) {
-        const int blk = bj >> 4, r = bj & 15;
-        const int64_t row = m0 + 16 * wv + 4 * blk;
+    const int64_t row = m0 + 16 * wv + 4 * blk;
 #pragma unroll
-        for (int b = 0; b < 4; b++) {
-            const int64_t tok = t0 + 16 * b + r;
-            if (tok < ne11 && row < ne01)
-                *(float4 *)(dst + tok * d_row + row) = make_float4(hsum8(acc[b][0]), hsum8(acc[b][1]), hsum8(acc[b][2]), hsum8(acc[b][3]));
-        }
-    } else {
-#pragma unroll
-    for (int c = 0; c < 4; c++) {
-        const int64_t tok = t0 + 4 * tg + c;
-        float o[4];
-#pragma unroll
-        for (int r = 0; r < 4; r++) o[r] = hsum8(acc[r][c]);
-        const int64_t row = m0 + 4 * mg;
-        if (tok < ne11 && row < ne01) *(float4 *)(dst + tok * d_row + row) = make_float4(o[0], o[1], o[2], o[3]);
-    }
+    for (int b = 0; b < 4; b++) {
+        const int64_t tok = t0 + 16 * b + r;
+        if (tok < ne11 && row < ne01)
+            *(float4 *)(dst + tok * d_row + row) = make_float4(hsum8(acc[b][0]), hsum8(acc[b][1]), hsum8(acc[b][2]), hsum8(acc[b][3]));
     }
 }
 
-// The K-quant dots for many activation rows at once, tiled like exact_gemm8_kernel<., true> (64 x 64 outputs per workgroup, a
+// The K-quant dots for many activation rows at once, tiled like exact_gemm8f_kernel (64 x 64 outputs per workgroup, a
 // wave 16 weight rows x 64 activation rows per v_mfma_i32_16x16x4_4b_i8, weight words through its A-matrix broadcast).  These dots keep ONE accumulator per output and add a term per sub-block of 32 elements, in order:
 //   Q4_K:  acc = fma(d_x, d * float(sc * isum) - dmin * float(m * bsum), acc)       isum = sum q * x, bsum = sum x over the sub-block
 //   Q6_K:  acc = fma(d_x * d, float(sc0 * isum0 + sc1 * isum1), acc)                 isum0 / isum1 over the two halves of 16 elements
@@ -1078,17 +1026,15 @@ int spy_exact_dots(hipStream_t st, int t0, const spy_hip_tensor *w, const uint8_
         const char *env_tiled = getenv("SPY_HIP_EXACT_TILED");
         const bool tiled = !(env_tiled && *env_tiled == '0');
         const int64_t nb = w->ne[0] / 32, ne01 = w->ne[1];
-        const bool fits = nb > 0 && nb % XGB_KB == 0 && ne01 % 4 == 0 && w->nb[1] % 4 == 0 && x_row % 4 == 0 && ((uintptr_t)w->data & 3) == 0 &&
+        const bool fits = nb > 0 && nb % XGF_KB == 0 && ne01 % 4 == 0 && w->nb[1] % 4 == 0 && x_row % 4 == 0 && ((uintptr_t)w->data & 3) == 0 &&
                           ((uintptr_t)xm & 3) == 0 && dst->nb[0] == 4 && dst->nb[1] % 16 == 0 && ((uintptr_t)dst->data & 15) == 0 &&
                           (ne11 + XGB_TILE - 1) / XGB_TILE <= 65535 && !getenv("SPY_HIP_EXACT_SERIAL");
         if (tiled && fits) {
             const dim3 grid((unsigned)((ne01 + XGB_TILE - 1) / XGB_TILE), (unsigned)((ne11 + XGB_TILE - 1) / XGB_TILE));
-            // SPY_HIP_EXACT_TILED=dot: the integer sums from v_dot4 on the vector units instead of the matrix cores
-            const bool mf = !(env_tiled && *env_tiled == 'd');
-#define XGB_LAUNCH(WT, MF) exact_gemm8_kernel<WT, MF><<<grid, dim3(256), 0, st>>>((const uint8_t *)w->data, w->nb[1], ne01, nb, xm, x_row, ne11, (float *)dst->data, dst->nb[1] / 4)
-            if (t0 == SPY_HIP_Q4_0) { if (mf) XGB_LAUNCH(SPY_HIP_Q4_0, true); else XGB_LAUNCH(SPY_HIP_Q4_0, false); }
-            else { if (mf) XGB_LAUNCH(SPY_HIP_Q8_0, true); else XGB_LAUNCH(SPY_HIP_Q8_0, false); }
-#undef XGB_LAUNCH
+            if (t0 == SPY_HIP_Q4_0)
+                exact_gemm8f_kernel<SPY_HIP_Q4_0><<<grid, dim3(256), 0, st>>>((const uint8_t *)w->data, w->nb[1], ne01, nb, xm, x_row, ne11, (float *)dst->data, dst->nb[1] / 4);
+            else
+                exact_gemm8f_kernel<SPY_HIP_Q8_0><<<grid, dim3(256), 0, st>>>((const uint8_t *)w->data, w->nb[1], ne01, nb, xm, x_row, ne11, (float *)dst->data, dst->nb[1] / 4);
             return SPY_LAUNCH_RC();
         }
     }
