@@ -75,7 +75,10 @@ const char *spy_hip_error_string(int code);
  * target_buffer_type (mat.cpp:32-42): (Q4_0|Q8_0, F32) quantizes x to Q8_0, (F16, F32) rounds x
  * to fp16; additionally (Q4_K|Q6_K, F32) -> Q8_0 activations, which the reference lacks.
  * `scratch` holds the converted activations (the reference allocates it in get_control_header,
- * mat.cpp:61-68); query its size with spy_hip_op_matmul_scratch_size. */
+ * mat.cpp:61-68); query its size with spy_hip_op_matmul_scratch_size.  While the host's summation
+ * order is on (spy_hip_set_exact_order) that size also covers fp16 copies of both operands, from which
+ * the prompt-sized Q4_0 / Q8_0 MatMul of that order runs fastest; a buffer that holds only the
+ * activations (rows * row size of the converted type) is accepted too and gives the same results. */
 size_t spy_hip_op_matmul_scratch_size(const spy_hip_tensor *w, const spy_hip_tensor *x);
 int spy_hip_op_matmul(void *stream, const spy_hip_tensor *w, const spy_hip_tensor *x, const spy_hip_tensor *dst,
                       void *scratch, size_t scratch_bytes);
@@ -83,8 +86,8 @@ int spy_hip_op_matmul(void *stream, const spy_hip_tensor *w, const spy_hip_tenso
  * per node (mat.cpp:61-68).  For callers that cannot allocate: code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc.  Same operator and same results as spy_hip_op_matmul; the converted activations go
  * to a fixed array in device memory (spy_hip_op_matmul_noalloc_max_scratch() bytes, 8 MiB, held by every device the
- * library runs on until the process ends) instead of a caller buffer.  Returns SPY_HIP_ENOSPACE when
- * spy_hip_op_matmul_scratch_size(w, x) exceeds that.  All calls on a device share the array: calls that overlap on one
+ * library runs on until the process ends) instead of a caller buffer.  Returns SPY_HIP_ENOSPACE when the converted
+ * activations (rows * row size of the converted type) exceed that.  All calls on a device share the array: calls that overlap on one
  * device (different streams or threads) race. */
 size_t spy_hip_op_matmul_noalloc_max_scratch(void);
 int spy_hip_op_matmul_noalloc(void *stream, const spy_hip_tensor *w, const spy_hip_tensor *x, const spy_hip_tensor *dst);

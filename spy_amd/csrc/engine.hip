@@ -365,6 +365,7 @@ int spy_softmax_causal_launch(void *stream, const spy_hip_tensor *x, const spy_h
 int spy_exact_on();                                                                                                          // exact_order.hip
 int spy_softmax_row_ok(int64_t ne0);                                                                                         // ops.hip
 int64_t spy_exact_prompt_attn_row(int64_t n_kv);                                                                             // exact_prompt.hip
+size_t spy_exact_pack_bytes(int64_t ne01, int64_t ne00, int64_t ne11);                                                           // exact_order.hip
 int spy_exact_prompt_attn(hipStream_t st, const float *q, const uint16_t *kc, const uint16_t *vt, float *S, uint16_t *P16, float *out, const float *lut,
                           int T, int H, int P, int64_t C, int n_total, float scale);                                        // exact_prompt.hip
 
@@ -408,7 +409,13 @@ static int forward_ops(spy_hip_llama *m, hipStream_t st, const int32_t *tokens_h
                  o_ids = take(T * 4), o_pos = take(T * 4), o_logits = take(head == HEAD_ALL ? V * T * 4 : V * 4), o_rt = take(T * hd * 4);
     const size_t act_q8 = (size_t)T * ((F > d ? F : d) / 32) * 34;
     const size_t act_f16 = sp_bytes / 2 > (size_t)d * T * 2 ? sp_bytes / 2 : (size_t)d * T * 2;
-    const size_t o_scr = take(act_q8 > act_f16 ? act_q8 : act_f16);
+    // exact order: room behind the activations for the packed fp16 operands of the largest MatMul (spy_exact_pack_bytes)
+    size_t pack = 0;
+    if (exact && T >= 16) {
+        const int64_t shapes[3][2] = {{d, d}, {F, d}, {d, F}};
+        for (auto &sh : shapes) { const size_t b = spy_exact_pack_bytes(sh[0], sh[1], T); pack = b > pack ? b : pack; }
+    }
+    const size_t o_scr = take((act_q8 > act_f16 ? act_q8 : act_f16) + 256 + pack);
     const size_t scr_bytes = off - o_scr;
     if (off > m->ops_bytes) {
         if (m->ops_buf) { HIP_TRY(hipStreamSynchronize(st)); HIP_TRY(hipFree(m->ops_buf)); m->ops_buf = nullptr; m->ops_bytes = 0; }

@@ -622,6 +622,120 @@ __global__ __launch_bounds__(256, 2) void exact_gemm8f_kernel(const uint8_t *__r
     }
 }
 
+// The same tile from operands that were staged as fp16 ONCE per MatMul instead of once per tile (a weight tile is used by every
+// tile of activation rows and the other way round: 32 and 64 to 172 times for a 2048-row chunk of a 7B prompt).  The packing kernel
+// writes the words in the order the tile kernel's LDS holds them -- [tile of 64 rows][block][element word][row], four fp16 per
+// entry, and the block scales as floats, [tile][block][row] -- so staging is a plain copy of 16-byte pieces, and the vector units
+// of the tile kernel issue little but the fma per term.  Rows past the end of the matrix are packed as zeros (never stored).
+// Weight words are rotated by 16 rows in the odd element words, which spreads the four lane blocks of a wave's read (four
+// different element words, the same 16 rows) over all LDS banks.
+#define XGP_KB 2
+#define XGP_WPOS(row, e) (((row) + 16 * ((e) & 1)) & 63)
+template <int WT>        // type of the source blocks: Q4_0 (weights) or Q8_0 (weights, activations)
+__global__ __launch_bounds__(256) void xgp_pack_kernel(const uint8_t *__restrict__ src, int64_t row_bytes, int64_t nrows, int64_t nb,
+                                                       uint2 *__restrict__ q, float *__restrict__ d, int rotate) {
+    const int row_in = threadIdx.x & 63;
+    const int64_t tile = blockIdx.y, ib = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6), row = tile * XGB_TILE + row_in;
+    if (ib >= nb) return;
+    uint2 *qo = q + (tile * nb + ib) * (8 * XGB_TILE);
+    float *dout = d + (tile * nb + ib) * XGB_TILE + row_in;
+    if (row >= nrows) {
+#pragma unroll
+        for (int e = 0; e < 8; e++) qo[e * XGB_TILE + (rotate ? XGP_WPOS(row_in, e) : row_in)] = make_uint2(0u, 0u);
+        *dout = 0.0f;
+        return;
+    }
+    // blocks are 2-byte aligned: scale, then 16 (Q4_0) or 32 (Q8_0) quant bytes
+    const uint16_t *p = (const uint16_t *)(src + row * row_bytes + ib * (WT == SPY_HIP_Q4_0 ? 18 : 34));
+    *dout = h2f_tab(p[0]);
+    if (WT == SPY_HIP_Q4_0) {
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const uint32_t v = (uint32_t)p[1 + 2 * k] | ((uint32_t)p[2 + 2 * k] << 16);
+            qo[k * XGB_TILE + (rotate ? XGP_WPOS(row_in, k) : row_in)] = xgf_bytes_to_h4(v & 0x0F0F0F0Fu, 1032.0f);                  // elements 4k .. 4k + 3
+            qo[(4 + k) * XGB_TILE + (rotate ? XGP_WPOS(row_in, 4 + k) : row_in)] = xgf_bytes_to_h4((v >> 4) & 0x0F0F0F0Fu, 1032.0f); // elements 16 + 4k ..
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const uint32_t v = (uint32_t)p[1 + 2 * k] | ((uint32_t)p[2 + 2 * k] << 16);
+            qo[k * XGB_TILE + (rotate ? XGP_WPOS(row_in, k) : row_in)] = xgf_bytes_to_h4(v ^ 0x80808080u, 1152.0f);
+        }
+    }
+}
+template <int WT>        // weight type: decides which accumulator a word belongs to
+__global__ __launch_bounds__(256, 2) void exact_gemm8p_kernel(const uint2 *__restrict__ wq, const float *__restrict__ wd, const uint2 *__restrict__ xq,
+                                                               const float *__restrict__ xd, int64_t nb, int64_t ne01, int64_t ne11,
+                                                               float *__restrict__ dst, int64_t d_row) {
+    __shared__ __align__(16) uint2 s_wq[2][XGP_KB][8][XGB_TILE];
+    __shared__ __align__(16) uint2 s_xq[2][XGP_KB][8][XGB_TILE];
+    __shared__ __align__(16) float s_wd[2][XGP_KB * XGB_TILE];
+    __shared__ __align__(16) float s_xd[2][XGP_KB * XGB_TILE];
+    static_assert(XGP_KB == 2, "the copy below moves two 16-byte pieces per operand and one scale per thread and stage");
+    const int tid = threadIdx.x;
+    const int wv = tid >> 6, bj = tid & 63, blk = bj >> 4, r = bj & 15;
+    const int64_t m0 = (int64_t)blockIdx.x * XGB_TILE, t0 = (int64_t)blockIdx.y * XGB_TILE;
+    // a stage of an operand: XGP_KB blocks x 8 words x 64 rows x 8 bytes = 512 pieces of 16 bytes, two per thread
+    const uint4 *gw = (const uint4 *)(wq + (int64_t)blockIdx.x * nb * (8 * XGB_TILE)) + tid;
+    const uint4 *gx = (const uint4 *)(xq + (int64_t)blockIdx.y * nb * (8 * XGB_TILE)) + tid;
+    const float *gd = tid < 128 ? wd + (int64_t)blockIdx.x * nb * XGB_TILE + tid : xd + (int64_t)blockIdx.y * nb * XGB_TILE + (tid - 128);
+    uint4 g0, g1, g2, g3;
+    float gs;
+#define XGP_FETCH(stage) { g0 = gw[(stage) * 512]; g1 = gw[(stage) * 512 + 256]; g2 = gx[(stage) * 512]; g3 = gx[(stage) * 512 + 256]; \
+                           gs = gd[(stage) * (XGP_KB * XGB_TILE)]; }
+#define XGP_PUT(buf) { uint4 *lw = (uint4 *)&s_wq[buf][0][0][0] + tid, *lx = (uint4 *)&s_xq[buf][0][0][0] + tid; \
+                       lw[0] = g0; lw[256] = g1; lx[0] = g2; lx[256] = g3; \
+                       if (tid < 128) s_wd[buf][tid] = gs; else s_xd[buf][tid - 128] = gs; }
+
+    float acc[4][4][8];
+#pragma unroll
+    for (int b = 0; b < 4; b++)
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+#pragma unroll
+            for (int a = 0; a < 8; a++) acc[b][c][a] = 0.0f;
+    const xgb_v16f zero16 = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    const int wpos = XGP_WPOS(16 * wv + r, blk);      // words blk and 4 + blk have the same parity
+
+    const int64_t nstage = nb / XGP_KB;
+    XGP_FETCH(0)
+    XGP_PUT(0)
+    __syncthreads();
+    for (int64_t s = 0; s < nstage; s++) {
+        const int buf = (int)(s & 1);
+        if (s + 1 < nstage) XGP_FETCH(s + 1)
+#pragma unroll 1
+        for (int kb = 0; kb < XGP_KB; kb++) {
+            const float wdreg = s_wd[buf][kb * XGB_TILE + 16 * wv + r], xdl = s_xd[buf][kb * XGB_TILE + bj];
+            const uint2 w0 = s_wq[buf][kb][blk][wpos], w1 = s_wq[buf][kb][4 + blk][wpos];
+            uint2 xql[8];
+#pragma unroll
+            for (int e = 0; e < 8; e++) xql[e] = s_xq[buf][kb][e][bj];
+            const xgb_v16f D = __builtin_amdgcn_mfma_f32_16x16x1f32(wdreg, xdl, zero16, 2, 0, 0);
+            xgb_v16f p[2];
+            p[0] = xgf_mfma16(w0, xql[0], 0);
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                if (e + 1 < 8) p[(e + 1) & 1] = xgf_mfma16(e + 1 < 4 ? w0 : w1, xql[e + 1], (e + 1) & 3);
+                __builtin_amdgcn_sched_barrier(0);      // the matrix instruction of word e + 1 stays ahead of the fmas on word e
+                const int a = WT == SPY_HIP_Q4_0 ? ((e + 4) & 7) : e;
+#pragma unroll
+                for (int n = 0; n < 16; n++) acc[n >> 2][n & 3][a] = fmaf(D[n], p[e & 1][n], acc[n >> 2][n & 3][a]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        if (s + 1 < nstage) XGP_PUT(buf ^ 1)
+        __syncthreads();
+    }
+    const int64_t row = m0 + 16 * wv + 4 * blk;
+#pragma unroll
+    for (int b = 0; b < 4; b++) {
+        const int64_t tok = t0 + 16 * b + r;
+        if (tok < ne11 && row < ne01)
+            *(float4 *)(dst + tok * d_row + row) = make_float4(hsum8(acc[b][0]), hsum8(acc[b][1]), hsum8(acc[b][2]), hsum8(acc[b][3]));
+    }
+}
+
 // The K-quant dots for many activation rows at once, tiled like exact_gemm8f_kernel (64 x 64 outputs per workgroup, a
 // wave 16 weight rows x 64 activation rows per v_mfma_i32_16x16x4_4b_i8, weight words through its A-matrix broadcast).  These dots keep ONE accumulator per output and add a term per sub-block of 32 elements, in order:
 //   Q4_K:  acc = fma(d_x, d * float(sc * isum) - dmin * float(m * bsum), acc)       isum = sum q * x, bsum = sum x over the sub-block
@@ -1017,7 +1131,17 @@ int spy_exact_rope(hipStream_t st, const spy_hip_tensor *x, const spy_hip_tensor
 }
 
 // x_own_quants: the Q8_0 activations were quantized by this library (no byte is -128)
-int spy_exact_dots(hipStream_t st, int t0, const spy_hip_tensor *w, const uint8_t *xm, int64_t x_row, int64_t ne11, const spy_hip_tensor *dst, int x_own_quants) {
+// bytes of workspace with which a MatMul of ne01 weight rows of ne00 elements by ne11 activation rows runs from packed fp16 operands
+// (0: that kernel does not apply to the shape)
+size_t spy_exact_pack_bytes(int64_t ne01, int64_t ne00, int64_t ne11) {
+    const int64_t nb = ne00 / 32;
+    if (ne11 < 16 || ne00 % 32 != 0 || nb <= 0 || nb % XGP_KB != 0) return 0;
+    const int64_t tiles = (ne01 + XGB_TILE - 1) / XGB_TILE + (ne11 + XGB_TILE - 1) / XGB_TILE;
+    return (size_t)(tiles * nb * (8 * XGB_TILE * 8 + XGB_TILE * 4));       // quants and scales: multiples of 256 bytes each
+}
+// pack, pack_bytes: workspace for the packed operands (may be null / short: the tile kernel then unpacks per tile)
+int spy_exact_dots(hipStream_t st, int t0, const spy_hip_tensor *w, const uint8_t *xm, int64_t x_row, int64_t ne11, const spy_hip_tensor *dst, int x_own_quants,
+                   void *pack, size_t pack_bytes) {
     const int64_t total = w->ne[1] * ne11 * w->ne[2] * w->ne[3];
     if (total <= 0 || (total + 7) / 8 >= (1ll << 31)) return SPY_HIP_EINVAL;
     // many activation rows of a plain matrix: the tiled kernel (SPY_HIP_EXACT_TILED=0 keeps the row kernels, for the tests
@@ -1031,6 +1155,23 @@ int spy_exact_dots(hipStream_t st, int t0, const spy_hip_tensor *w, const uint8_
                           (ne11 + XGB_TILE - 1) / XGB_TILE <= 65535 && !getenv("SPY_HIP_EXACT_SERIAL");
         if (tiled && fits) {
             const dim3 grid((unsigned)((ne01 + XGB_TILE - 1) / XGB_TILE), (unsigned)((ne11 + XGB_TILE - 1) / XGB_TILE));
+            const size_t pk = spy_exact_pack_bytes(ne01, w->ne[0], ne11);
+            // SPY_HIP_EXACT_TILED=u: operands unpacked per tile even where the workspace would do
+            if (pk && pack && pack_bytes >= pk && ((uintptr_t)pack & 15) == 0 && grid.x <= 65535 && !(env_tiled && *env_tiled == 'u')) {
+                const int64_t mt = grid.x, tt = grid.y;
+                uint2 *wq = (uint2 *)pack, *xq = wq + mt * nb * (8 * XGB_TILE);
+                float *wd = (float *)(xq + tt * nb * (8 * XGB_TILE)), *xd = wd + mt * nb * XGB_TILE;
+                const dim3 gw((unsigned)((nb + 3) / 4), (unsigned)mt), gx((unsigned)((nb + 3) / 4), (unsigned)tt);
+                if (t0 == SPY_HIP_Q4_0) xgp_pack_kernel<SPY_HIP_Q4_0><<<gw, dim3(256), 0, st>>>((const uint8_t *)w->data, w->nb[1], ne01, nb, wq, wd, 1);
+                else xgp_pack_kernel<SPY_HIP_Q8_0><<<gw, dim3(256), 0, st>>>((const uint8_t *)w->data, w->nb[1], ne01, nb, wq, wd, 1);
+                xgp_pack_kernel<SPY_HIP_Q8_0><<<gx, dim3(256), 0, st>>>(xm, x_row, ne11, nb, xq, xd, 0);
+                if (hipGetLastError() != hipSuccess) return SPY_HIP_EINVAL;
+                if (t0 == SPY_HIP_Q4_0)
+                    exact_gemm8p_kernel<SPY_HIP_Q4_0><<<grid, dim3(256), 0, st>>>(wq, wd, xq, xd, nb, ne01, ne11, (float *)dst->data, dst->nb[1] / 4);
+                else
+                    exact_gemm8p_kernel<SPY_HIP_Q8_0><<<grid, dim3(256), 0, st>>>(wq, wd, xq, xd, nb, ne01, ne11, (float *)dst->data, dst->nb[1] / 4);
+                return SPY_LAUNCH_RC();
+            }
             if (t0 == SPY_HIP_Q4_0)
                 exact_gemm8f_kernel<SPY_HIP_Q4_0><<<grid, dim3(256), 0, st>>>((const uint8_t *)w->data, w->nb[1], ne01, nb, xm, x_row, ne11, (float *)dst->data, dst->nb[1] / 4);
             else

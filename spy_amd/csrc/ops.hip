@@ -15,7 +15,9 @@ int spy_exact_norm_rms(hipStream_t st, const spy_hip_tensor *x, const spy_hip_te
 int spy_exact_silu(hipStream_t st, const spy_hip_tensor *x, const spy_hip_tensor *dst);
 int spy_exact_softmax(hipStream_t st, const spy_hip_tensor *x, const spy_hip_tensor *mask, const spy_hip_tensor *dst, float scale);
 int spy_exact_rope(hipStream_t st, const spy_hip_tensor *x, const spy_hip_tensor *pos, const spy_hip_tensor *dst, const spy_hip_rope_param *p);
-int spy_exact_dots(hipStream_t st, int t0, const spy_hip_tensor *w, const uint8_t *xm, int64_t x_row, int64_t ne11, const spy_hip_tensor *dst, int x_own_quants);
+int spy_exact_dots(hipStream_t st, int t0, const spy_hip_tensor *w, const uint8_t *xm, int64_t x_row, int64_t ne11, const spy_hip_tensor *dst, int x_own_quants,
+                   void *pack, size_t pack_bytes);
+size_t spy_exact_pack_bytes(int64_t ne01, int64_t ne00, int64_t ne11);
 
 struct tdesc {              // a tensor as the kernels see it
     uint8_t *p;
@@ -550,13 +552,22 @@ __global__ __launch_bounds__(256) void to_f16_batched_kernel(const uint8_t *__re
     *(uint2 *)(y + (b * ne11 + row) * ne10 + c * 4) = o;
 }
 
-extern "C" size_t spy_hip_op_matmul_scratch_size(const spy_hip_tensor *w, const spy_hip_tensor *x) {
+// bytes of the converted activations: the part of the scratch buffer that MatMul cannot do without
+static size_t matmul_act_bytes(const spy_hip_tensor *w, const spy_hip_tensor *x) {
     if (!w || !x) return 0;
     const int tm = mid_type(w->type, x->type);
     if (tm == x->type) return 0;
     if (tm != SPY_HIP_Q8_0 && tm != SPY_HIP_F16) return 0;
     if (x->ne[0] % spy_block_size(tm) != 0) return 0;
     return (size_t)(spy_t_nrow(x) * spy_row_size(tm, x->ne[0]));
+}
+// ... plus, while the exact summation order is on, room for the fp16 copies of both operands that its prompt-sized Q4_0 / Q8_0
+// MatMul runs from (a call with less than this, but the activations' part, runs the kernel that unpacks per tile: same results)
+extern "C" size_t spy_hip_op_matmul_scratch_size(const spy_hip_tensor *w, const spy_hip_tensor *x) {
+    const size_t act = matmul_act_bytes(w, x);
+    if (!act || !spy_exact_on() || x->type != SPY_HIP_F32 || (w->type != SPY_HIP_Q4_0 && w->type != SPY_HIP_Q8_0) || w->ne[2] != 1 || w->ne[3] != 1) return act;
+    const size_t pk = spy_exact_pack_bytes(w->ne[1], w->ne[0], x->ne[1]);
+    return pk ? ((act + 255) & ~(size_t)255) + pk : act;
 }
 
 static int matmul_impl(void *stream, const spy_hip_tensor *w, const spy_hip_tensor *x, const spy_hip_tensor *dst, void *scratch, size_t scratch_bytes,
@@ -621,7 +632,12 @@ static int matmul_impl(void *stream, const spy_hip_tensor *w, const spy_hip_tens
     if (quant) {
         SPY_CHECK_ARG(w->nb[0] == spy_type_size(t0) && w->nb[1] == spy_row_size(t0, ne00));   // whole contiguous rows
         SPY_CHECK_ARG(dst->nb[1] % 4 == 0);
-        if (skip_past < 0 && klimit_past < 0 && spy_exact_on()) return spy_exact_dots(st, t0, w, xm, mid_row, ne11, dst, t1 != tm);
+        if (skip_past < 0 && klimit_past < 0 && spy_exact_on()) {
+            // what the activations leave of the scratch buffer: workspace for packed operands
+            const size_t used = t1 != tm ? ((size_t)(spy_t_nrow(x) * mid_row) + 255) & ~(size_t)255 : 0;
+            const bool room = scratch && scratch_bytes > used && ((uintptr_t)scratch & 15) == 0;
+            return spy_exact_dots(st, t0, w, xm, mid_row, ne11, dst, t1 != tm, room ? (uint8_t *)scratch + used : nullptr, room ? scratch_bytes - used : 0);
+        }
         for (int64_t i3 = 0; i3 < ne03; i3++)
             for (int64_t i2 = 0; i2 < ne02; i2++) {
                 const uint8_t *wp = (const uint8_t *)w->data + i2 * w->nb[2] + i3 * w->nb[3];
@@ -636,7 +652,7 @@ static int matmul_impl(void *stream, const spy_hip_tensor *w, const spy_hip_tens
         return 0;
     }
     SPY_CHECK_ARG(w->nb[0] == 2);
-    if (skip_past < 0 && klimit_past < 0 && spy_exact_on()) return spy_exact_dots(st, t0, w, xm, mid_row, ne11, dst, 0);
+    if (skip_past < 0 && klimit_past < 0 && spy_exact_on()) return spy_exact_dots(st, t0, w, xm, mid_row, ne11, dst, 0, nullptr, 0);
     if (ne11 >= 16 && ne01 >= 16 && ne00 % 8 == 0 && w->nb[1] % 16 == 0 && w->nb[2] % 16 == 0 && w->nb[3] % 16 == 0 &&
         ((uintptr_t)w->data & 15) == 0 && ((uintptr_t)xm & 15) == 0 && dst->nb[1] % 4 == 0 && dst->nb[2] % 4 == 0 && ne02 <= 65535) {
         for (int64_t i3 = 0; i3 < ne03; i3++) {            // prompt-sized attention products: fp16 MFMA
@@ -685,7 +701,7 @@ extern "C" int spy_hip_op_matmul_noalloc(void *stream, const spy_hip_tensor *w, 
     if (e != hipSuccess) return (int)e;
     const int rc = spy_static_scratch_setup(dev);
     if (rc) return rc;
-    const size_t need = spy_hip_op_matmul_scratch_size(w, x);
+    const size_t need = matmul_act_bytes(w, x);
     if (need > SPY_STATIC_SCRATCH_BYTES) return SPY_HIP_ENOSPACE;     // the converted activations do not fit the fixed array
     return matmul_impl(stream, w, x, dst, g_scratch_ptr[dev], SPY_STATIC_SCRATCH_BYTES, -1, -1);
 }

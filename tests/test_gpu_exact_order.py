@@ -75,7 +75,7 @@ def test_tiled_matmul_bits(hip, oracle, wtype, M, K, T, monkeypatch):
     L = hip.load()
     need = L.spy_hip_op_matmul_scratch_size(B(tw), B(tx))
     scratch = dev_empty(need, 0)
-    for tiled in ("1", "0"):          # tiled kernel, row kernels
+    for tiled in ("1", "u", "0"):          # tiled kernel from packed operands, unpacking per tile, row kernels
         monkeypatch.setenv("SPY_HIP_EXACT_TILED", tiled)
         dd = dev_empty(T * M * 4, 0xFF)
         td = hip.tensor(dd, hip.F32, [M, T])
