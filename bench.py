@@ -283,7 +283,7 @@ def main():
     weights_desc = {"q4_0": "Q4_0 weights, %s" % head_desc, "q8_0": "Q8_0 weights incl. head",
                     "q4_k_m": "Q4_K weights with Q6_K attn_v / ffn_down / head, 0.1 %% of the weights x 20"}[args.model] + \
                    " (seeded ~N(0, 0.02), quantized by the package's block quantizers)"
-    prefill_note = {1: "prompt pass in the host backend's summation order (tiled exact kernels: integer sums on the matrix cores, every accumulator of the host loops kept apart on the vector units): same logits and caches as the CPU reference's",
+    prefill_note = {1: "prompt pass in the host backend's summation order (tiled exact kernels: integer sums from the matrix cores as floats, every accumulator of the host loops kept apart on the vector units): same logits and caches as the CPU reference's",
                     0: "matrix-core prompt pass in the backend's own order"}
     mode_desc = {1: "host-backend summation order: logits and greedy tokens equal to the CPU reference's bit for bit",
                  0: "this backend's own summation order (per-operator 1e-7; not token-exact)"}
