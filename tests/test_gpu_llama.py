@@ -248,6 +248,84 @@ def test_llama2_7b_q4_0_greedy_32_tokens():
     eng.close()
 
 
+def _full_size_case(cfg, seed, n_prompt, n_steps, n_forced, outlier_every=0):
+    """A named configuration at its full size on the engine as it comes (summation order 1): the prompt in one call (tiled exact
+    MatMul from packed operands, causal exact attention kernels, chunks of 2048 rows), n_steps greedy single-token passes (graph
+    replay), n_forced teacher-forced passes.  Logits of every prompt row, every token and the logits of the forced passes must be
+    the CPU oracle's bit for bit."""
+    import os
+    from spy_amd import model as M
+    from tests.model_util import OracleModel
+    tensors = M.synth_model(cfg, seed=seed, outlier_every=outlier_every)       # the package's own block quantizers, as in bench.py
+    eng, ora = M.Engine(cfg, tensors), OracleModel(cfg, tensors, nthread=min(16, os.cpu_count() or 8))
+    assert eng.order() == 1
+    prompt = np.random.default_rng(seed + 1).integers(0, cfg.n_vocab, n_prompt).astype(np.int32)
+    print("oracle prompt pass of %d tokens ..." % n_prompt, flush=True)
+    import threading, time
+    done = threading.Event()
+
+    def heartbeat():                                 # a long CPU pass prints nothing by itself
+        t0 = time.time()
+        while not done.wait(60.0):
+            print("  ... %d s" % (time.time() - t0), flush=True)
+    threading.Thread(target=heartbeat, daemon=True).start()
+    try:
+        lg_o = ora.forward(prompt, 0)
+    finally:
+        done.set()
+    lg_g = eng.forward(prompt, 0)
+    _bits(lg_g, lg_o, "prompt pass of %d tokens, every row" % n_prompt)
+    want, logits, pos = [], lg_o[-1], n_prompt
+    del lg_o, lg_g
+    for step in range(n_steps):
+        want.append(int(np.argmax(logits)))
+        if step + 1 < n_steps:
+            logits = ora.forward(np.array([want[-1]], np.int32), pos)[0]
+            pos += 1
+        if step % 32 == 31:
+            print("oracle step", step + 1, flush=True)
+    got = [want[0]] + eng.decode_greedy(want[0], n_prompt, n_steps - 1, use_graph=True).tolist()
+    print("oracle tokens:", want, "\nhip tokens:   ", got, flush=True)
+    assert got == want
+    same = 0
+    for step in range(n_forced):
+        lo = ora.forward(np.array([want[step]], np.int32), n_prompt + step)[0]
+        lg = eng.forward(np.array([want[step]], np.int32), n_prompt + step)[0]
+        same += int(np.array_equal(lo.view(np.uint32), lg.view(np.uint32)))
+    print("%d of %d single-token passes with bit-identical logits" % (same, n_forced), flush=True)
+    assert same == n_forced
+    eng.close()
+
+
+@pytest.mark.timeout(600)
+def test_llama2_7b_q8_0_prompt_512_then_64_tokens():
+    """The third named configuration: 7B shape in Q8_0 (32 layers), 512-token prompt, 64 greedy steps (n_kv 513 ... 576)."""
+    from spy_amd import model as M
+    _full_size_case(M.Config.llama2_7b(n_ctx=576, wtype=O.Q8_0), 4321, 512, 64, 16)
+
+
+_slow = pytest.mark.skipif(not __import__("os").environ.get("SPY_FULL_SIZE_TESTS"), reason="many minutes of CPU oracle at the 7B size: set SPY_FULL_SIZE_TESTS=1")
+
+
+@_slow
+@pytest.mark.timeout(1150)
+def test_llama2_7b_q4_k_m_prompt_2048_then_96_tokens():
+    """The fourth named configuration: the Q4_K / Q6_K mix, 2048-token prompt; 96 of its 512 greedy steps (the oracle's K-quant
+    prompt pass alone takes 16 minutes on 16 threads)."""
+    from spy_amd import model as M
+    cfg = M.Config.llama2_7b(n_ctx=2560, wtype=O.Q4_K, t_out=O.Q6_K, tensor_types={"attn_v": O.Q6_K, "ffn_down": O.Q6_K})
+    _full_size_case(cfg, 4322, 2048, 96, 4, outlier_every=1000)            # 0.1 % of the weights x 20
+
+
+@_slow
+@pytest.mark.timeout(1150)
+def test_llama2_7b_q4_0_prompt_4096_then_256_tokens():
+    """The second named configuration (the one the bench times): Q4_0 with the Q6_K head, 4096-token prompt in two chunks, 256 greedy
+    steps at n_kv 4097 ... 4352."""
+    from spy_amd import model as M
+    _full_size_case(M.Config.llama2_7b(n_ctx=4352, wtype=O.Q4_0, t_out=O.Q6_K), 4323, 4096, 256, 4)
+
+
 @pytest.mark.timeout(900)
 def test_llama2_7b_q4_0_own_order_stays_within_the_noise_bound():
     """The same configuration on the engine's own summation order (order 0), which is NOT the parity path.  Every MatMul of
