@@ -716,10 +716,7 @@ __global__ __launch_bounds__(256, 2) void exact_gemm8p_kernel(const uint2 *__res
             p[0] = xgf_mfma16(w0, xql[0], 0);
 #pragma unroll
             for (int e = 0; e < 8; e++) {
-                // the matrix instruction goes out at raised wave priority: it takes one issue slot and then runs beside the other wave's fmas (1.5 %)
-                __builtin_amdgcn_s_setprio(1);
                 if (e + 1 < 8) p[(e + 1) & 1] = xgf_mfma16(e + 1 < 4 ? w0 : w1, xql[e + 1], (e + 1) & 3);
-                __builtin_amdgcn_s_setprio(0);
                 __builtin_amdgcn_sched_barrier(0);      // the matrix instruction of word e + 1 stays ahead of the fmas on word e
                 const int a = WT == SPY_HIP_Q4_0 ? ((e + 4) & 7) : e;
 #pragma unroll
