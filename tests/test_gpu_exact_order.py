@@ -81,6 +81,16 @@ def test_tiled_matmul_bits(hip, oracle, wtype, M, K, T, monkeypatch):
         td = hip.tensor(dd, hip.F32, [M, T])
         call(L.spy_hip_op_matmul, None, B(tw), B(tx), B(td), scratch.ptr, need)
         _same_bits(dd.download(np.float32).reshape(T, M), want, "matmul type %d %dx%d T %d tiled %s" % (wtype, M, K, T, tiled))
+    # a scratch buffer that holds the converted activations and nothing else: no room for packed operands, same bits
+    monkeypatch.setenv("SPY_HIP_EXACT_TILED", "1")
+    act = T * (K // 32) * 34
+    assert act <= need
+    small = dev_empty(act, 0)
+    dd = dev_empty(T * M * 4, 0xFF)
+    call(L.spy_hip_op_matmul, None, B(tw), B(tx), B(hip.tensor(dd, hip.F32, [M, T])), small.ptr, act)
+    _same_bits(dd.download(np.float32).reshape(T, M), want, "matmul type %d %dx%d T %d, activations-only scratch" % (wtype, M, K, T))
+    if wtype in (O.Q4_0, O.Q8_0) and T >= 16 and (K // 32) % 2 == 0:
+        assert need > act + 2 * (M + T) * K, "the scratch size of the exact order covers the packed operands"
 
 
 @pytest.mark.parametrize("T", [2, 40])
