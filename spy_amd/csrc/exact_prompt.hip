@@ -110,7 +110,10 @@ __global__ __launch_bounds__(256, 2) void xp_scores_kernel(const float *__restri
     __shared__ float s_tile[XP_QT][65];
     __shared__ __align__(16) uint4 s_k[64][16];                  // 64 key rows of 256 bytes
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int t0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * XP_QT, h = blockIdx.y;      // the longest rows first
+    // The head is the fastest-running index of the grid: consecutive workgroups go to the eight XCDs in turn, and with the query tile
+    // there an XCD would get tiles k and k + 8 of 16 only -- under the causal mask 24 to 10 units of work (68 % of the compute units
+    // busy over the launch).  With the head there every XCD gets the same mix of tiles, and the key rows of its heads stay in its L2.
+    const int t0 = ((int)gridDim.y - 1 - (int)blockIdx.y) * XP_QT, h = blockIdx.x;      // the longest rows first
     const int64_t d = (int64_t)H * 128;
     // the cached positions are dealt out in segments of XP_KSEG over blockIdx.z, so that the workgroups are of similar length
     // (one workgroup per 128 query rows would make the longest rows the critical path of the launch)
@@ -265,7 +268,7 @@ __global__ __launch_bounds__(256, 2) void xp_pv_kernel(const uint16_t *__restric
                                                        int T, int H, int P, int64_t p_row, int64_t C, int n_total) {
     __shared__ __align__(16) uint16_t s_p[2][32 * XP_SC][40];  // [buffer][position in the stage][query row], rows of 80 bytes
     const int g = threadIdx.x >> 5, l = threadIdx.x & 31;
-    const int t0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * XP_PT, h = blockIdx.z;
+    const int t0 = ((int)gridDim.z - 1 - (int)blockIdx.z) * XP_PT, h = blockIdx.x;      // head fastest: see xp_scores_kernel
     const int dd0 = blockIdx.y * 32 + g * 4;
     const int Lmax = P + min(t0 + XP_PT - 1, T - 1) + 1;
     const int tail_start = (n_total - 1) / 32 * 32;
@@ -409,11 +412,11 @@ int spy_exact_prompt_attn(hipStream_t st, const float *q, const uint16_t *kc, co
     if ((int64_t)P + T > 1024 * XP_SM_R) return SPY_HIP_EUNSUPPORTED;      // the softmax kernel keeps a row in the registers of 256 threads
     if (((uintptr_t)q & 15) || ((uintptr_t)kc & 15) || ((uintptr_t)S & 15) || ((uintptr_t)P16 & 7) || ((uintptr_t)out & 15)) return SPY_HIP_EINVAL;
     const int64_t s_row = spy_exact_prompt_attn_row((int64_t)P + T);
-    xp_scores_kernel<<<dim3((unsigned)((T + XP_QT - 1) / XP_QT), (unsigned)H, (unsigned)((P + T + XP_KSEG - 1) / XP_KSEG)), dim3(256), 0, st>>>(q, kc, S, T, H, P, s_row);
+    xp_scores_kernel<<<dim3((unsigned)H, (unsigned)((T + XP_QT - 1) / XP_QT), (unsigned)((P + T + XP_KSEG - 1) / XP_KSEG)), dim3(256), 0, st>>>(q, kc, S, T, H, P, s_row);
     if (hipGetLastError() != hipSuccess) return SPY_HIP_EINVAL;
     xp_softmax_kernel<<<dim3((unsigned)T, (unsigned)H), dim3(256), 0, st>>>(S, P16, lut, T, P, s_row, n_total, scale);
     if (hipGetLastError() != hipSuccess) return SPY_HIP_EINVAL;
-    xp_pv_kernel<<<dim3((unsigned)((T + XP_PT - 1) / XP_PT), 4, (unsigned)H), dim3(256), 0, st>>>(P16, vt, out, T, H, P, s_row, C, n_total);
+    xp_pv_kernel<<<dim3((unsigned)H, 4, (unsigned)((T + XP_PT - 1) / XP_PT)), dim3(256), 0, st>>>(P16, vt, out, T, H, P, s_row, C, n_total);
     return SPY_LAUNCH_RC();
 }
 
