@@ -15,7 +15,12 @@
  *     backend/host/include/default_backend.h:72-78);
  *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); launches are
  *     asynchronous, the caller synchronises;
- *   - all tensor memory is device memory owned by the caller; kernels never allocate;
+ *   - all tensor memory is device memory owned by the caller; the spy_hip_op_* entry points never allocate, free or
+ *     synchronise once spy_hip_init has run on the device (it builds the tables the exact-order operators look values
+ *     up in), so they can be recorded under HIP stream capture.  The one exception is exact-order Rope, whose table of
+ *     host-libm angles depends on the call's parameters: spy_hip_rope_prepare builds it ahead of time; without that the
+ *     first call with a new parameter set builds it (allocating) where it may, and under capture returns
+ *     SPY_HIP_EUNSUPPORTED instead;
  *   - shapes use Spy's order: ne[0] is the contiguous dimension, nb[] are BYTE strides and nb[0]
  *     is the size of one block (tensor.h:50-57).
  */
@@ -66,6 +71,14 @@ int spy_hip_event_create(void **event);
 int spy_hip_event_record(void *event, void *stream);
 int spy_hip_event_elapsed_ms(void *start, void *stop, float *ms);   /* synchronises on `stop` */
 int spy_hip_event_destroy(void *event);
+/* Stream capture for callers without the HIP headers: every call made on `stream` between begin and end is recorded
+ * instead of run; end instantiates the recording as an executable graph (*graph_exec), which graph_launch replays on a
+ * stream.  No counterpart in the reference (its scheduler re-dispatches every operator every pass,
+ * default_scheduler.h:46-111). */
+int spy_hip_capture_begin(void *stream);
+int spy_hip_capture_end(void *stream, void **graph_exec);
+int spy_hip_graph_launch(void *graph_exec, void *stream);
+int spy_hip_graph_destroy(void *graph_exec);
 const char *spy_hip_error_string(int code);
 
 /* ---- operators: one per OperatorImpl<Op>::execute of the host backend ---------------------- */
@@ -88,7 +101,9 @@ int spy_hip_op_matmul(void *stream, const spy_hip_tensor *w, const spy_hip_tenso
  * to a fixed array in device memory (spy_hip_op_matmul_noalloc_max_scratch() bytes, 8 MiB, held by every device the
  * library runs on until the process ends) instead of a caller buffer.  Returns SPY_HIP_ENOSPACE when the converted
  * activations (rows * row size of the converted type) exceed that.  All calls on a device share the array: calls that overlap on one
- * device (different streams or threads) race. */
+ * device (different streams or threads) race, and a replay of a graph that recorded such a call counts as a call.  While
+ * the host's summation order is on, the fp16 operand copies of spy_hip_op_matmul_scratch_size go into the array as well
+ * when they fit behind the activations, and are left out (same results) when they do not. */
 size_t spy_hip_op_matmul_noalloc_max_scratch(void);
 int spy_hip_op_matmul_noalloc(void *stream, const spy_hip_tensor *w, const spy_hip_tensor *x, const spy_hip_tensor *dst);
 /* NormRMS -- OperatorNormRMSImpl::execute (non-linear.cpp:194-223); eps = NormRMSParam::eps */
@@ -113,6 +128,13 @@ typedef struct spy_hip_rope_param {
     int32_t xpos_down;
 } spy_hip_rope_param;
 int spy_hip_op_rope(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *pos, const spy_hip_tensor *dst, const spy_hip_rope_param *p);
+/* Exact-order Rope takes cosf / sinf of every position's angles from the host's libm, as the reference does
+ * (non-linear.cpp:304-309): a table per parameter set {num_context, ne0, freq_base, freq_scale, attention_factor, num_dim},
+ * kept on the device until the process ends (at most 16 per device).  This call builds it ahead of time (ne0 = the rotated
+ * row length, dst->ne[0] of the calls to come), after which exact-order spy_hip_op_rope with these parameters neither
+ * allocates nor synchronises.  SPY_HIP_EUNSUPPORTED where no table applies (no context length, xpos, YaRN extension:
+ * those calls read the positions back and synchronise). */
+int spy_hip_rope_prepare(const spy_hip_rope_param *p, int64_t ne0);
 /* Dup / Copy -- dup_execute (view.cpp:83-195): F32->F32, F32->F16, F16->F32 through strides */
 int spy_hip_op_dup(void *stream, const spy_hip_tensor *src, const spy_hip_tensor *dst);
 /* Contiguous -- OperatorContiguousImpl::execute (view.cpp:285-321) */

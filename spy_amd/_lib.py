@@ -75,6 +75,10 @@ SIGNATURES = {
     "spy_hip_event_record": (_i32, [_vp, _vp]),
     "spy_hip_event_elapsed_ms": (_i32, [_vp, _vp, C.POINTER(_f32)]),
     "spy_hip_event_destroy": (_i32, [_vp]),
+    "spy_hip_capture_begin": (_i32, [_vp]),
+    "spy_hip_capture_end": (_i32, [_vp, C.POINTER(_vp)]),
+    "spy_hip_graph_launch": (_i32, [_vp, _vp]),
+    "spy_hip_graph_destroy": (_i32, [_vp]),
     "spy_hip_error_string": (C.c_char_p, [_i32]),
     "spy_hip_op_matmul_scratch_size": (_sz, [_TP, _TP]),
     "spy_hip_op_matmul": (_i32, [_vp, _TP, _TP, _TP, _vp, _sz]),
@@ -85,6 +89,7 @@ SIGNATURES = {
     "spy_hip_op_silu": (_i32, [_vp, _TP, _TP]),
     "spy_hip_op_softmax": (_i32, [_vp, _TP, _TP, _TP, _f32]),
     "spy_hip_op_rope": (_i32, [_vp, _TP, _TP, _TP, C.POINTER(RopeParam)]),
+    "spy_hip_rope_prepare": (_i32, [C.POINTER(RopeParam), _i64]),
     "spy_hip_op_dup": (_i32, [_vp, _TP, _TP]),
     "spy_hip_op_contiguous": (_i32, [_vp, _TP, _TP]),
     "spy_hip_op_get_row": (_i32, [_vp, _TP, _TP, _TP]),

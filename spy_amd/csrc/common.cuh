@@ -61,6 +61,10 @@ static __device__ __forceinline__ int wave_sum_i32(int v) {
     return v;
 }
 
+// raises the dynamic-LDS limit of `kern` on the current device to at least `lds` bytes (runtime.hip: one record per device and
+// kernel for the whole process, only ever raised)
+int spy_raise_lds_limit(const void *kern, size_t lds);
+
 #define SPY_CHECK_ARG(cond) do { if (!(cond)) return SPY_HIP_EINVAL; } while (0)
 #define SPY_LAUNCH_RC() ((int)hipGetLastError())
 

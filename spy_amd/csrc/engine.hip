@@ -125,7 +125,7 @@ extern "C" int spy_hip_llama_create(const spy_hip_llama_desc *desc, spy_hip_llam
     {   // softmax + P.V keeps one head's scores (f32) and probabilities (f16) in LDS
         const size_t pv_lds = C * 4 + C * 2 + 16;
         if (!rc && pv_lds > 160 * 1024) rc = SPY_HIP_EUNSUPPORTED;
-        if (!rc && pv_lds > 48 * 1024) rc = (int)hipFuncSetAttribute((const void *)attn_pv_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)pv_lds);
+        if (!rc) rc = spy_raise_lds_limit((const void *)attn_pv_kernel, pv_lds);
     }
     if (!rc && fused_ok(m) && m->wave) {   // one launch for the attention part of a layer where its workgroups are all resident (SPY_HIP_ATTN_SPLIT=1: three launches)
         const char *env = getenv("SPY_HIP_ATTN_SPLIT");

@@ -47,18 +47,20 @@ struct spy_hip_llama {
     int pos_imm = 0, rope_row0 = 0;             // kernel-family entry points (no device state): the position; first position of rope_tab
     long long *stamp_dbg = nullptr;             // measurement builds (-DATL_STAMPS) only
     uint32_t spin_limit = 400000;               // polls of a bounded inter-workgroup wait before a pass gives up (~0.5 s)
-    // per engine (= per device) launcher state: dynamic-LDS limit already set for a kernel, resident workgroups of a persistent grid
+    // per engine launcher state: the largest dynamic-LDS size this engine has asked for per kernel (the limit itself is kept
+    // per device and kernel for the whole process and only ever raised: spy_raise_lds_limit), resident workgroups of a persistent grid
     std::unordered_map<const void *, size_t> lds_set;
     std::unordered_map<const void *, int> grid_cap;
     std::vector<void *> owned;
 };
 
 
-// raise a kernel's dynamic-LDS limit once per engine and size
+// a kernel's dynamic-LDS limit covers this engine's launches: the limit belongs to the kernel function for the whole process,
+// so it is raised through the process-wide record and never lowered by an engine with a smaller context
 static inline int spy_ensure_lds(spy_hip_llama *m, const void *kern, size_t lds) {
     size_t &have = m->lds_set[kern];
     if (lds > have) {
-        if (lds > 48 * 1024) HIP_TRY(hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        RC_TRY(spy_raise_lds_limit(kern, lds));
         have = lds;
     }
     return 0;

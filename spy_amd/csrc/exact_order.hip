@@ -18,6 +18,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <mutex>
 #include <vector>
 
 namespace {
@@ -37,9 +38,19 @@ __device__ __forceinline__ uint8_t *xat(const xdesc &t, int64_t i0, int64_t i1, 
 }
 
 int g_exact = -1;          // -1: not decided yet (environment), 0 / 1
-float *g_lut = nullptr;    // device: exp table [65536], then silu table [65536]
-float *g_rope = nullptr;   // device: cos / sin pairs per token of the current Rope call
-size_t g_rope_cap = 0;
+// Per-device state, set up once per device and kept until the process ends (never freed, never replaced: a stream of
+// another thread may still read it), guarded by one mutex:
+//   lut    exp table [65536], then silu table [65536]; built by spy_exact_device_setup, which spy_hip_init calls
+//   rope   the Rope tables (cos / sin of every position of a context) by parameter set; built by spy_hip_rope_prepare, or by
+//          the first exact-order Rope call with a new parameter set where that call is allowed to allocate (not under capture)
+#define XO_MAX_DEVICES 64
+#define XO_MAX_ROPE_TABLES 16
+struct rope_key { int64_t npos, ne0; float freq_base, freq_scale, factor; int32_t num_dim; };
+struct rope_entry { rope_key k; float *dev; };
+struct device_state { float *lut = nullptr; std::vector<rope_entry> rope; };
+device_state g_dev[XO_MAX_DEVICES];
+std::mutex g_mu;
+int current_device() { int dev = -1; return (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < XO_MAX_DEVICES) ? dev : -1; }
 
 // IEEE binary16 -> binary32 on the host
 float host_h2f(uint16_t h) {
@@ -61,8 +72,11 @@ float host_h2f(uint16_t h) {
 
 // The reference's tables (lookup_table_impl/non-linear.h:39-47,131-139): entry k holds the function of
 // float(half k), evaluated by the host's libm in fp32; the loop stops before k = 0xFFFF, which stays 0.
-int ensure_luts() {
-    if (g_lut) return 0;
+int device_luts(const float **lut) {
+    const int dev = current_device();
+    if (dev < 0) return SPY_HIP_EINVAL;
+    std::lock_guard<std::mutex> lock(g_mu);
+    if (g_dev[dev].lut) { *lut = g_dev[dev].lut; return 0; }
     std::vector<float> h(2 * 65536, 0.0f);
     for (uint32_t k = 0; k < 0xFFFFu; k++) {
         const float v = host_h2f((uint16_t)k);
@@ -74,7 +88,8 @@ int ensure_luts() {
     if (e != hipSuccess) return (int)e;
     e = hipMemcpy(d, h.data(), h.size() * sizeof(float), hipMemcpyHostToDevice);
     if (e != hipSuccess) { (void)hipFree(d); return (int)e; }
-    g_lut = d;
+    g_dev[dev].lut = d;
+    *lut = d;
     return 0;
 }
 
@@ -1000,13 +1015,10 @@ __global__ __launch_bounds__(256) void exact_dots32_kernel(xdesc w, const uint8_
 
 }   // namespace
 
-// the two tables on the device: exp [65536], then silu [65536]
-int spy_exact_luts(const float **lut) {
-    const int rc = ensure_luts();
-    if (rc) return rc;
-    *lut = g_lut;
-    return 0;
-}
+// the two tables on the current device: exp [65536], then silu [65536]
+int spy_exact_luts(const float **lut) { return device_luts(lut); }
+// spy_hip_init: the tables exist before the first operator call, which then has nothing to allocate
+int spy_exact_device_setup() { const float *lut = nullptr; return device_luts(&lut); }
 
 // A caller may switch the exact order on for the calls its own thread makes (a model whose passes run in the host's order
 // issues its prompt operators that way) without touching what other threads see.
@@ -1039,18 +1051,20 @@ int spy_exact_norm_rms(hipStream_t st, const spy_hip_tensor *x, const spy_hip_te
 }
 
 int spy_exact_silu(hipStream_t st, const spy_hip_tensor *x, const spy_hip_tensor *dst) {
-    int rc = ensure_luts();
+    const float *lut = nullptr;
+    int rc = device_luts(&lut);
     if (rc) return rc;
     const int64_t total = spy_t_nelem(x);
-    exact_silu_kernel<<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st>>>(mkx(x), mkx(dst), g_lut, total);
+    exact_silu_kernel<<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st>>>(mkx(x), mkx(dst), lut, total);
     return SPY_LAUNCH_RC();
 }
 
 int spy_exact_softmax(hipStream_t st, const spy_hip_tensor *x, const spy_hip_tensor *mask, const spy_hip_tensor *dst, float scale) {
     if (dst->type != SPY_HIP_F32) return SPY_HIP_EUNSUPPORTED;      // the fp16 output is a shortcut of the fast path
-    int rc = ensure_luts();
+    const float *lut = nullptr;
+    int rc = device_luts(&lut);
     if (rc) return rc;
-    exact_softmax_kernel<<<dim3((unsigned)spy_t_nrow(dst)), dim3(256), 0, st>>>(mkx(x), mkx(mask ? mask : x), mask != nullptr, mkx(dst), scale, g_lut);
+    exact_softmax_kernel<<<dim3((unsigned)spy_t_nrow(dst)), dim3(256), 0, st>>>(mkx(x), mkx(mask ? mask : x), mask != nullptr, mkx(dst), scale, lut);
     return SPY_LAUNCH_RC();
 }
 
@@ -1081,32 +1095,70 @@ static void rope_row(float *row, int32_t position, int64_t ne0, float theta_scal
 
 int *spy_hip_err_flag_ptr();      // runtime.hip
 
+// The table of a parameter set on the current device: cos / sin of every position of the context, from the host's libm.
+// build: make it if it is missing (allocates and copies: not under stream capture).  *tab stays nullptr when it is missing and
+// was not built.
+static bool rope_table_applies(const spy_hip_rope_param *p, int64_t ne0) {
+    return p->num_context > 0 && (int64_t)p->num_context * ne0 * 4 <= (64ll << 20) && p->xpos_base == 0.0f && p->extend_factor == 0.0f;
+}
+static int rope_table(const spy_hip_rope_param *p, int64_t ne0, bool build, const float **tab) {
+    *tab = nullptr;
+    const int dev = current_device();
+    if (dev < 0) return SPY_HIP_EINVAL;
+    const rope_key k = {p->num_context, ne0, p->freq_base, p->freq_scale, p->attention_factor, p->num_dim};
+    std::lock_guard<std::mutex> lock(g_mu);
+    for (const rope_entry &e : g_dev[dev].rope)
+        if (e.k.npos == k.npos && e.k.ne0 == k.ne0 && e.k.freq_base == k.freq_base && e.k.freq_scale == k.freq_scale && e.k.factor == k.factor && e.k.num_dim == k.num_dim) {
+            *tab = e.dev;
+            return 0;
+        }
+    if (!build || g_dev[dev].rope.size() >= XO_MAX_ROPE_TABLES) return 0;
+    const float theta_scale = powf(p->freq_base, -2.0f / (float)p->num_dim);
+    std::vector<float> h((size_t)(k.npos * ne0));
+    for (int64_t q = 0; q < k.npos; q++) rope_row(&h[(size_t)(q * ne0)], (int32_t)q, ne0, theta_scale, p, false);
+    float *d = nullptr;
+    hipError_t e = hipMalloc((void **)&d, h.size() * sizeof(float));
+    if (e != hipSuccess) return (int)e;
+    e = hipMemcpy(d, h.data(), h.size() * sizeof(float), hipMemcpyHostToDevice);
+    if (e != hipSuccess) { (void)hipFree(d); return (int)e; }
+    g_dev[dev].rope.push_back({k, d});
+    *tab = d;
+    return 0;
+}
+
+// Builds the exact-order Rope table of a parameter set ahead of time (ne0: the rotated row length, dst->ne[0] of the Rope
+// calls to come), so that those calls neither allocate nor synchronise and can be captured into a HIP graph.
+extern "C" int spy_hip_rope_prepare(const spy_hip_rope_param *p, int64_t ne0) {
+    SPY_CHECK_ARG(p && ne0 > 0 && ne0 % 2 == 0 && p->num_dim > 0);
+    if (!rope_table_applies(p, ne0)) return SPY_HIP_EUNSUPPORTED;
+    const float *tab = nullptr;
+    const int rc = rope_table(p, ne0, true, &tab);
+    if (rc) return rc;
+    return tab ? 0 : SPY_HIP_ENOSPACE;                     // XO_MAX_ROPE_TABLES parameter sets per device
+}
+
 int spy_exact_rope(hipStream_t st, const spy_hip_tensor *x, const spy_hip_tensor *pos, const spy_hip_tensor *dst, const spy_hip_rope_param *p) {
     const int64_t ne0 = dst->ne[0], ne2 = dst->ne[2];
     const float theta_scale = powf(p->freq_base, -2.0f / (float)p->num_dim);
     const dim3 grid((unsigned)dst->ne[1], (unsigned)dst->ne[2], (unsigned)dst->ne[3]);
-    // The rotations of every position of the context, built once per parameter set and kept on the device: the kernel
-    // then looks its token's position up itself and the call needs no copy and no wait.
-    static struct { int64_t npos, ne0; float freq_base, freq_scale, factor; int32_t num_dim; float *dev; } cache = {0, 0, 0, 0, 0, 0, nullptr};
-    const int64_t npos = p->num_context;
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (st && hipStreamIsCapturing(st, &cap) != hipSuccess) cap = hipStreamCaptureStatusNone;
+    const bool capturing = cap != hipStreamCaptureStatusNone;
     const bool zeta = p->xpos_base != 0.0f;
-    if (npos > 0 && npos * ne0 * 4 <= (64ll << 20) && spy_hip_err_flag_ptr() && !zeta && p->extend_factor == 0.0f) {
-        if (!cache.dev || cache.npos != npos || cache.ne0 != ne0 || cache.freq_base != p->freq_base || cache.freq_scale != p->freq_scale ||
-            cache.factor != p->attention_factor || cache.num_dim != p->num_dim) {
-            std::vector<float> tab((size_t)(npos * ne0));
-            for (int64_t q = 0; q < npos; q++) rope_row(&tab[(size_t)(q * ne0)], (int32_t)q, ne0, theta_scale, p, false);
-            if (cache.dev) { (void)hipDeviceSynchronize(); (void)hipFree(cache.dev); cache.dev = nullptr; }
-            hipError_t e = hipMalloc((void **)&cache.dev, tab.size() * sizeof(float));
-            if (e != hipSuccess) { cache.dev = nullptr; return (int)e; }
-            e = hipMemcpy(cache.dev, tab.data(), tab.size() * sizeof(float), hipMemcpyHostToDevice);
-            if (e != hipSuccess) return (int)e;
-            cache.npos = npos; cache.ne0 = ne0; cache.freq_base = p->freq_base; cache.freq_scale = p->freq_scale;
-            cache.factor = p->attention_factor; cache.num_dim = p->num_dim;
+    // The rotations of every position of the context, built once per parameter set and kept on the device: the kernel
+    // then looks its token's position up itself and the call needs no allocation, no copy and no wait.
+    if (rope_table_applies(p, ne0) && spy_hip_err_flag_ptr()) {
+        const float *tab = nullptr;
+        const int rc = rope_table(p, ne0, !capturing, &tab);
+        if (rc) return rc;
+        if (tab) {
+            exact_rope_kernel<<<grid, dim3(64), 0, st>>>(mkx(x), mkx(dst), tab, (const uint8_t *)pos->data, pos->nb[0], p->num_context, spy_hip_err_flag_ptr(), 0);
+            return SPY_LAUNCH_RC();
         }
-        exact_rope_kernel<<<grid, dim3(64), 0, st>>>(mkx(x), mkx(dst), cache.dev, (const uint8_t *)pos->data, pos->nb[0], npos, spy_hip_err_flag_ptr(), 0);
-        return SPY_LAUNCH_RC();
     }
-    // No context length given: wait for the stream, read the positions back and upload the rows of this call's tokens.
+    // No table (no context length, xpos or the YaRN extension, more parameter sets than are kept): wait for the stream, read the
+    // positions back and upload the rows of this call's tokens.  Allocates and synchronises: not available under capture.
+    if (capturing) return SPY_HIP_EUNSUPPORTED;
     hipError_t e = hipStreamSynchronize(st);
     if (e != hipSuccess) return (int)e;
     std::vector<int32_t> hp((size_t)ne2);
@@ -1117,17 +1169,17 @@ int spy_exact_rope(hipStream_t st, const spy_hip_tensor *x, const spy_hip_tensor
     std::vector<float> tab((size_t)(ne2 * tab_row));
     for (int64_t i2 = 0; i2 < ne2; i2++) rope_row(&tab[(size_t)(i2 * tab_row)], hp[(size_t)i2], ne0, theta_scale, p, zeta);
     const size_t need = tab.size() * sizeof(float);
-    if (need > g_rope_cap) {
-        if (g_rope) { (void)hipDeviceSynchronize(); (void)hipFree(g_rope); g_rope = nullptr; g_rope_cap = 0; }
-        e = hipMalloc((void **)&g_rope, need);
-        if (e != hipSuccess) return (int)e;
-        g_rope_cap = need;
-    }
-    e = hipMemcpy(g_rope, tab.data(), need, hipMemcpyHostToDevice);
+    float *d = nullptr;                                     // this call's own rows: nothing shared with other threads
+    e = hipMalloc((void **)&d, need);
     if (e != hipSuccess) return (int)e;
-    exact_rope_kernel<<<grid, dim3(64), 0, st>>>(mkx(x), mkx(dst), g_rope, nullptr, 0, 0, nullptr, zeta ? 1 : 0);
-    if (hipGetLastError() != hipSuccess) return SPY_HIP_EINVAL;
-    return (int)hipStreamSynchronize(st);      // the table is overwritten by the next call
+    e = hipMemcpy(d, tab.data(), need, hipMemcpyHostToDevice);
+    if (e == hipSuccess) {
+        exact_rope_kernel<<<grid, dim3(64), 0, st>>>(mkx(x), mkx(dst), d, nullptr, 0, 0, nullptr, zeta ? 1 : 0);
+        e = hipGetLastError();
+        if (e == hipSuccess) e = hipStreamSynchronize(st);
+    }
+    (void)hipFree(d);
+    return e == hipSuccess ? 0 : (int)e;
 }
 
 // x_own_quants: the Q8_0 activations were quantized by this library (no byte is -128)

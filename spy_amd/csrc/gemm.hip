@@ -378,12 +378,7 @@ template <int WT, int NTW>
 static int launch_gemm_skinny_ntw(hipStream_t st, const void *w, const void *xq, float *dst, int64_t M, int64_t K, int64_t T, int64_t dst_stride) {
     auto kern = gemm_skinny_kernel<WT, NTW>;
     constexpr size_t lds = 4 * (size_t)gsk_traits<WT>::WAVE_LDS;
-    static bool attr_set = false;
-    if (!attr_set) {
-        hipError_t e_ = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e_ != hipSuccess) return (int)e_;
-        attr_set = true;
-    }
+    { const int rc_ = spy_raise_lds_limit((const void *)kern, lds); if (rc_) return rc_; }
     kern<<<dim3((unsigned)((M + 31) / 32), (unsigned)((T + 32 * NTW - 1) / (32 * NTW))), dim3(256), lds, st>>>(
         (const uint8_t *)w, (const uint8_t *)xq, dst, (int)M, (int)K, (int)T, dst_stride);
     return SPY_LAUNCH_RC();

@@ -138,12 +138,7 @@ __global__ __launch_bounds__(WROW_THREADS) void wave_row_kernel(gemv_args a, int
 template <int WT, int NITK, int NR>
 static int launch_wave_row_nr(hipStream_t st, const gemv_args &a, int T, size_t lds, int grid) {
     auto kern = wave_row_kernel<WT, NITK, NR>;
-    static size_t lds_set = 0;
-    if (lds > 48 * 1024 && lds > lds_set) {
-        hipError_t e_ = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e_ != hipSuccess) return (int)e_;
-        lds_set = lds;
-    }
+    { const int rc_ = spy_raise_lds_limit((const void *)kern, lds); if (rc_) return rc_; }
     kern<<<dim3((unsigned)grid), dim3(WROW_THREADS), lds, st>>>(a, T);
     return SPY_LAUNCH_RC();
 }
@@ -301,10 +296,7 @@ static int launch_fast(hipStream_t st, const gemv_args &a) {
     const size_t lds = (size_t)NT * staged_bytes(a.K);
     if (lds > 160 * 1024) return SPY_HIP_EUNSUPPORTED;
     auto kern = gemv_kernel<WT, LPR, NIT, NT, DUMP>;
-    if (lds > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return (int)e;
-    }
+    { const int rc_ = spy_raise_lds_limit((const void *)kern, lds); if (rc_) return rc_; }
     const int ntiles = (a.M + RPT - 1) / RPT;
     const int cap = resident_blocks(kern, lds);
     kern<<<dim3((unsigned)(ntiles < cap ? ntiles : cap)), dim3(GEMV_THREADS), lds, st>>>(a);

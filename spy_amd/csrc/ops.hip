@@ -293,12 +293,10 @@ static int softmax_launch(void *stream, const spy_hip_tensor *x, const spy_hip_t
     if (dst->type == SPY_HIP_F16 && !row_ok) return SPY_HIP_EUNSUPPORTED;
     if (row_ok) {
         const size_t lds = (size_t)dst->ne[0] * 4;
-        static size_t lds_set = 0;
-        if (lds > 48 * 1024 && lds > lds_set) {
-            hipError_t e1_ = hipFuncSetAttribute((const void *)softmax_row_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, SOFTMAX_LDS_ROW * 4);
-            hipError_t e2_ = hipFuncSetAttribute((const void *)softmax_row_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, SOFTMAX_LDS_ROW * 4);
-            if (e1_ != hipSuccess || e2_ != hipSuccess) return (int)(e1_ != hipSuccess ? e1_ : e2_);
-            lds_set = SOFTMAX_LDS_ROW * 4;
+        if (lds > 48 * 1024) {
+            int rc_ = spy_raise_lds_limit((const void *)softmax_row_kernel<false>, SOFTMAX_LDS_ROW * 4);
+            if (!rc_) rc_ = spy_raise_lds_limit((const void *)softmax_row_kernel<true>, SOFTMAX_LDS_ROW * 4);
+            if (rc_) return rc_;
         }
         if (dst->type == SPY_HIP_F16) softmax_row_kernel<true><<<dim3((unsigned)nrow), dim3(256), lds, (hipStream_t)stream>>>(mk(x), m, mask != nullptr, mk(dst), scale, causal_past);
         else softmax_row_kernel<false><<<dim3((unsigned)nrow), dim3(256), lds, (hipStream_t)stream>>>(mk(x), m, mask != nullptr, mk(dst), scale, causal_past);

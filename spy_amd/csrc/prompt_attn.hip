@@ -35,8 +35,11 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 // log2(e) = LH + LL with 13 significant bits in LH: x * LH is exact in fp32 for an 11-bit x, so is its distance f to the
 // nearest integer n; e^x = 2^n * 2^(f + x * LL), with v_exp_f32 on an argument within [-0.5, 0.5] and one rounding (an fma)
 // before it: within an ulp or so of expf.  Results below the normal range come out of ldexp as expf returns them.
+// A score more than 65504 below its row maximum rounds to -inf in fp16 (expf gives 0 there, the decomposition inf - inf): the
+// argument is held at the lowest finite fp16 value, whose exponential is 0 as well.
 static __device__ __forceinline__ float pa_exp(_Float16 xh) {
     const float LH = 5909.0f / 4096.0f, LL = 6.80877639634e-05f;
+    xh = xh > (_Float16)(-65504.0f) ? xh : (_Float16)(-65504.0f);
     const float ph = fmaf((float)xh, LH, 0.0f), n = rintf(ph);     // the fp16 operand goes into the fma as it is
     const float g = fmaf((float)xh, LL, ph - n);
     return ldexpf(__builtin_amdgcn_exp2f(g), (int)n);
@@ -238,6 +241,7 @@ int spy_prompt_attn_launch(hipStream_t st, const uint16_t *q16, const uint16_t *
                            int T, int H, int hd, int past, int64_t n_ctx, float scale) {
     SPY_CHECK_ARG(q16 && k_cache && v_cache && out && T > 0 && H > 0 && H < 65536 && past >= 0 && (int64_t)((T + 63) / 64) * H < (1ll << 31));
     if (hd != 128 || n_ctx % 8 != 0 || n_ctx < 64 || n_ctx >= (1ll << 31)) return SPY_HIP_EUNSUPPORTED;
+    SPY_CHECK_ARG(scale > 0.0f);          // the row maximum is taken over the raw dot products and scaled afterwards
     SPY_CHECK_ARG((int64_t)past + T <= n_ctx && ((uintptr_t)q16 % 16) == 0 && ((uintptr_t)k_cache % 16) == 0 && ((uintptr_t)v_cache % 16) == 0 && ((uintptr_t)out % 16) == 0);
     pattn_args a;
     a.q16 = q16; a.kc = k_cache; a.vc = v_cache; a.out = out; a.T = T; a.H = H; a.past = past; a.n_ctx = (int)n_ctx; a.scale = scale;

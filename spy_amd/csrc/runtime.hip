@@ -6,27 +6,67 @@
 #include <stdio.h>
 #include <string.h>
 
-static int g_device = -1;
-static int *g_err_flag = nullptr;   // device int, raised by kernels that detect bad operands
+#include <map>
+#include <mutex>
+#include <utility>
 
-int *spy_hip_err_flag_ptr() { return g_err_flag; }
+// Per-device state of the library.  Everything an operator call needs beyond its operands is set up by spy_hip_init, once per
+// device and kept until the process ends, so that the spy_hip_op_* entry points neither allocate nor synchronise:
+//   err_flag   device int raised by kernels that detect bad operands
+//   (the exp / silu tables of the exact-order operators and their Rope tables live in exact_order.hip, same discipline)
+#define SPY_MAX_DEVICES 64
+static int g_device = -1;
+static int *g_err_flag[SPY_MAX_DEVICES];
+static std::mutex g_runtime_mu;
+
+int *spy_hip_err_flag_ptr() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= SPY_MAX_DEVICES) return nullptr;
+    return g_err_flag[dev];
+}
 int spy_static_scratch_setup(int device);    // ops.hip: address of the fixed scratch array on the current device
+int spy_exact_device_setup();                // exact_order.hip: the exp / silu tables of the current device
+
+// A kernel's dynamic-LDS limit (hipFuncAttributeMaxDynamicSharedMemorySize) belongs to the kernel function on a device for the
+// whole process, whoever launches it: it is kept here per (device, kernel) and only ever raised, so that an engine or operator
+// call with a smaller need never lowers it under a launch that was sized for more.
+int spy_raise_lds_limit(const void *kern, size_t lds) {
+    if (lds <= 48 * 1024) return 0;
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    static std::map<std::pair<int, const void *>, size_t> limit;
+    std::lock_guard<std::mutex> lock(g_runtime_mu);
+    size_t &have = limit[std::make_pair(dev, kern)];
+    if (lds > have) {
+        e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int)e;
+        have = lds;
+    }
+    return 0;
+}
 
 extern "C" int spy_hip_init(int device_id) {
     int n = 0;
     hipError_t e = hipGetDeviceCount(&n);
     if (e != hipSuccess) return (int)e;
-    if (device_id < 0 || device_id >= n) return SPY_HIP_EINVAL;
+    if (device_id < 0 || device_id >= n || device_id >= SPY_MAX_DEVICES) return SPY_HIP_EINVAL;
     e = hipSetDevice(device_id);
     if (e != hipSuccess) return (int)e;
-    if (g_device != device_id || !g_err_flag) {
-        if (g_err_flag) { (void)hipFree(g_err_flag); g_err_flag = nullptr; }
-        e = hipMalloc((void **)&g_err_flag, sizeof(int));
-        if (e != hipSuccess) return (int)e;
-        e = hipMemset(g_err_flag, 0, sizeof(int));
-        if (e != hipSuccess) return (int)e;
+    {
+        std::lock_guard<std::mutex> lock(g_runtime_mu);
+        if (!g_err_flag[device_id]) {
+            int *p = nullptr;
+            e = hipMalloc((void **)&p, sizeof(int));
+            if (e != hipSuccess) return (int)e;
+            e = hipMemset(p, 0, sizeof(int));
+            if (e != hipSuccess) { (void)hipFree(p); return (int)e; }
+            g_err_flag[device_id] = p;
+        }
+        g_device = device_id;
     }
-    g_device = device_id;
+    const int rc = spy_exact_device_setup();
+    if (rc) return rc;
     return spy_static_scratch_setup(device_id);
 }
 
@@ -115,13 +155,41 @@ extern "C" int spy_hip_event_elapsed_ms(void *start, void *stop, float *ms) {
 extern "C" int spy_hip_event_destroy(void *event) { return event ? (int)hipEventDestroy((hipEvent_t)event) : 0; }
 
 extern "C" int spy_hip_take_error(int *flag) {
-    if (!flag || !g_err_flag) return SPY_HIP_EINVAL;
+    int *dflag = spy_hip_err_flag_ptr();
+    if (!flag || !dflag) return SPY_HIP_EINVAL;
     hipError_t e = hipDeviceSynchronize();
     if (e != hipSuccess) return (int)e;
-    e = hipMemcpy(flag, g_err_flag, sizeof(int), hipMemcpyDeviceToHost);
+    e = hipMemcpy(flag, dflag, sizeof(int), hipMemcpyDeviceToHost);
     if (e != hipSuccess) return (int)e;
-    return (int)hipMemset(g_err_flag, 0, sizeof(int));
+    return (int)hipMemset(dflag, 0, sizeof(int));
 }
+
+// ---- stream capture: a sequence of calls on `stream` recorded once and replayed --------------------------------------------
+// Thin wrappers so that a caller without the HIP headers (a binding in another language, the tests) can put operator calls
+// under capture.  Between begin and end every call on the stream is recorded instead of run; calls that would allocate or
+// synchronise fail there, which is what the operator entry points are built to avoid.
+extern "C" int spy_hip_capture_begin(void *stream) {
+    if (!stream) return SPY_HIP_EINVAL;                         // the null stream cannot be captured
+    return (int)hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeThreadLocal);
+}
+extern "C" int spy_hip_capture_end(void *stream, void **graph_exec) {
+    if (!stream || !graph_exec) return SPY_HIP_EINVAL;
+    *graph_exec = nullptr;
+    hipGraph_t g = nullptr;
+    hipError_t e = hipStreamEndCapture((hipStream_t)stream, &g);
+    if (e != hipSuccess) return (int)e;
+    hipGraphExec_t x = nullptr;
+    e = hipGraphInstantiate(&x, g, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(g);
+    if (e != hipSuccess) return (int)e;
+    *graph_exec = (void *)x;
+    return 0;
+}
+extern "C" int spy_hip_graph_launch(void *graph_exec, void *stream) {
+    if (!graph_exec) return SPY_HIP_EINVAL;
+    return (int)hipGraphLaunch((hipGraphExec_t)graph_exec, (hipStream_t)stream);
+}
+extern "C" int spy_hip_graph_destroy(void *graph_exec) { return graph_exec ? (int)hipGraphExecDestroy((hipGraphExec_t)graph_exec) : 0; }
 
 extern "C" const char *spy_hip_error_string(int code) {
     switch (code) {

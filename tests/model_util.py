@@ -13,8 +13,8 @@ _FIELDS = [("attn_norm", "attn_norm", None), ("ffn_norm", "ffn_norm", None), ("w
 class OracleModel:
     """The reference's token loop (cli.h:60-129 in the Spy tree) on the CPU oracle."""
 
-    def __init__(self, cfg, tensors, nthread=8):
-        self.cfg, self.tensors, self.L = cfg, tensors, O.load()
+    def __init__(self, cfg, tensors, nthread=8, lib=None):
+        self.cfg, self.tensors, self.L = cfg, tensors, lib if lib is not None else O.load()
         self.layers = (O.LlamaLayer * cfg.n_layer)()
         for i in range(cfg.n_layer):
             for field, gname, tfield in _FIELDS:

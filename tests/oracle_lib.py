@@ -89,7 +89,26 @@ def load():
         return _lib
     if not os.path.exists(LIB):
         build()
-    L = C.CDLL(LIB)
+    _lib = _bind(C.CDLL(LIB))
+    return _lib
+
+
+LIB_FPFAST = os.path.join(ROOT, "oracle", "libspy_oracle_fpfast.so")
+_lib_fpfast = None
+
+
+def load_fpfast():
+    """The same source compiled with -ffp-contract=fast -mfma (make -C oracle FPCONTRACT=fast): gcc may then fuse the scalar
+    a * b + c expressions too, as a default GCC build of the reference would.  Only for the test that reports the difference."""
+    global _lib_fpfast
+    if _lib_fpfast is None:
+        if not os.path.exists(LIB_FPFAST):
+            subprocess.check_call(["make", "-s", "-C", os.path.join(ROOT, "oracle"), "FPCONTRACT=fast"])
+        _lib_fpfast = _bind(C.CDLL(LIB_FPFAST))
+    return _lib_fpfast
+
+
+def _bind(L):
     vp, i64, i32, f32 = C.c_void_p, C.c_int64, C.c_int32, C.c_float
     TP = C.POINTER(Tensor)
     sig = {
@@ -119,7 +138,6 @@ def load():
     for name, (res, args) in sig.items():
         fn = getattr(L, name)
         fn.restype, fn.argtypes = res, args
-    _lib = L
     return L
 
 

@@ -263,6 +263,67 @@ def test_norm_softmax_silu_rope_bits(hip, oracle):
     call(L.spy_hip_take_error, C.byref(flag)); assert flag.value == 1
 
 
+def test_exact_order_operators_under_stream_capture(hip, oracle):
+    """The exact-order Silu, Softmax and Rope recorded under HIP stream capture and replayed: the operator entry points
+    allocate nothing and wait for nothing once spy_hip_init has built the device's tables (and spy_hip_rope_prepare the
+    table of the Rope parameters), so the recording succeeds, and every replay -- with eager calls of the same operators on
+    other data in between -- leaves the oracle's bits.  An exact-order Rope whose table was not prepared is refused under
+    capture (it would have to allocate) and the capture survives the refusal."""
+    from tests.gpu_util import dev, dev_empty, call
+    L = hip.load()
+    rng = np.random.default_rng(33)
+    hd, H_, T, n_kv, Cx = 128, 4, 3, 700, 768
+    scale = float(1.0 / np.sqrt(128.0))
+    g = (rng.standard_normal(2048) * 3).astype(np.float32)
+    s = (rng.standard_normal((H_, T, n_kv)) * 9).astype(np.float32)
+    mask = np.where(np.arange(Cx)[None, :] <= (np.arange(T)[:, None] + n_kv - T), 0.0, -np.inf).astype(np.float32)
+    xr = rng.standard_normal((T, H_, hd)).astype(np.float32)
+    pos = np.array([5, 400, 767], np.int32)
+    w_silu, w_soft, w_rope = np.zeros_like(g), np.zeros_like(s), np.zeros_like(xr)
+    assert oracle.spy_o_silu(B(O.tensor(g, O.F32, [g.size])), B(O.tensor(w_silu, O.F32, [g.size]))) == 0
+    assert oracle.spy_o_softmax(B(O.tensor(s, O.F32, [n_kv, T, H_])), B(O.tensor(mask, O.I32, [Cx, T])), B(O.tensor(w_soft, O.F32, [n_kv, T, H_])), scale) == 0
+    rp = O.default_rope(hd, Cx)
+    assert oracle.spy_o_rope(B(O.tensor(xr, O.F32, [hd, H_, T])), B(O.tensor(pos, O.I32, [T])), B(O.tensor(w_rope, O.F32, [hd, H_, T])), B(rp)) == 0
+    dg, ds, dm, dx, dp = dev(g), dev(s), dev(mask), dev(xr), dev(pos)
+    o_silu, o_soft, o_rope = dev_empty(g.nbytes, 0xFF), dev_empty(s.nbytes, 0xFF), dev_empty(xr.nbytes, 0xFF)
+    hp = hip.RopeParam(0, 0, hd, Cx, Cx, 10000.0, 1.0, 0.0, 1.0, 32.0, 1.0, 0.0, 0)
+    hp_new = hip.RopeParam(0, 0, hd, Cx, Cx, 5000.0, 1.0, 0.0, 1.0, 32.0, 1.0, 0.0, 0)       # a parameter set nobody prepared
+    call(L.spy_hip_rope_prepare, B(hp), hd)
+    st = C.c_void_p()
+    call(L.spy_hip_stream_create, C.byref(st))
+    t_g, t_os = hip.tensor(dg, hip.F32, [g.size]), hip.tensor(o_silu, hip.F32, [g.size])
+    t_s, t_m, t_o = hip.tensor(ds, hip.F32, [n_kv, T, H_]), hip.tensor(dm, hip.I32, [Cx, T]), hip.tensor(o_soft, hip.F32, [n_kv, T, H_])
+    t_x, t_p, t_r = hip.tensor(dx, hip.F32, [hd, H_, T]), hip.tensor(dp, hip.I32, [T]), hip.tensor(o_rope, hip.F32, [hd, H_, T])
+    print("capture: exact-order silu, softmax, rope", flush=True)
+    call(L.spy_hip_capture_begin, st)
+    rcs = [L.spy_hip_op_silu(st, B(t_g), B(t_os)), L.spy_hip_op_softmax(st, B(t_s), B(t_m), B(t_o), scale), L.spy_hip_op_rope(st, B(t_x), B(t_p), B(t_r), B(hp))]
+    rc_unprepared = L.spy_hip_op_rope(st, B(t_x), B(t_p), B(t_r), B(hp_new))
+    gexec = C.c_void_p()
+    rc_end = L.spy_hip_capture_end(st, C.byref(gexec))
+    assert rcs == [0, 0, 0] and rc_end == 0 and gexec.value, (rcs, rc_end)
+    assert rc_unprepared == hip.EUNSUPPORTED
+    # other data for the eager calls between the replays
+    g2, s2 = dev((rng.standard_normal(2048) * 3).astype(np.float32)), dev((rng.standard_normal((H_, T, n_kv)) * 9).astype(np.float32))
+    e_silu, e_soft = dev_empty(g.nbytes, 0), dev_empty(s.nbytes, 0)
+    for replay in range(3):
+        for b in (o_silu, o_soft, o_rope):
+            b.fill(0xFF)
+        hip.sync()                                       # the fills ran on the null stream; the graph's stream does not wait for them by itself
+        call(L.spy_hip_graph_launch, gexec, st)
+        hip.sync(st)
+        _same_bits(o_silu.download(np.float32), w_silu, "silu, replay %d" % replay)
+        _same_bits(o_soft.download(np.float32).reshape(s.shape), w_soft, "softmax, replay %d" % replay)
+        _same_bits(o_rope.download(np.float32).reshape(xr.shape), w_rope, "rope, replay %d" % replay)
+        call(L.spy_hip_op_silu, None, B(hip.tensor(g2, hip.F32, [g.size])), B(hip.tensor(e_silu, hip.F32, [g.size])))
+        call(L.spy_hip_op_softmax, None, B(hip.tensor(s2, hip.F32, [n_kv, T, H_])), B(t_m), B(hip.tensor(e_soft, hip.F32, [n_kv, T, H_])), scale)
+        hip.sync()
+    call(L.spy_hip_graph_destroy, gexec)
+    # outside capture the unprepared parameter set builds its table on first use
+    call(L.spy_hip_op_rope, None, B(t_x), B(t_p), B(t_r), B(hp_new))
+    hip.sync()
+    call(L.spy_hip_stream_destroy, st)
+
+
 def test_switch_returns_previous_setting_and_default_is_off():
     from spy_amd import _lib as H
     L = H.load()

@@ -210,23 +210,47 @@ def test_fused_decode_real_widths_long_cache(order, n_ctx, positions):
     eng.close()
 
 
+@pytest.mark.parametrize("order", [1, 0])
+def test_engine_with_a_smaller_context_does_not_lower_the_lds_limit_of_a_larger_one(order):
+    """A kernel's dynamic-LDS limit belongs to the kernel for the whole process.  An engine with a long context raises it
+    (softmax + P.V^T keeps a head's scores and V^T rows in LDS: about 140 KB at 4352 positions); an engine with a short
+    context created afterwards, and the kernel-family entry points, must not lower it under the first engine's launches."""
+    from spy_amd import model as M
+    big = M.Config(n_layer=1, n_embd=4096, n_head=32, n_ff=11008, n_vocab=1024, n_ctx=4352, wtype=O.Q4_0)
+    small = M.Config(n_layer=1, n_embd=4096, n_head=32, n_ff=11008, n_vocab=1024, n_ctx=64, wtype=O.Q4_0)
+    tensors = M.synth_model(big, seed=3)
+    a = M.Engine(big, tensors, order=order)
+    rng = np.random.default_rng(2)
+    a.write_buffer("k_cache", 0, (rng.standard_normal(big.n_ctx * big.n_embd) * 0.5).astype(np.float16).view(np.uint16))
+    a.write_buffer("v_cache", 0, (rng.standard_normal(big.n_ctx * big.n_embd) * 0.5).astype(np.float16).view(np.uint16))
+    tok = np.array([7], np.int32)
+    first = a.forward(tok, 4300)[0]
+    b = M.Engine(small, tensors, order=order)
+    assert np.isfinite(b.forward(tok, 3)[0]).all()
+    again = a.forward(tok, 4300)[0]                      # the same slot is rewritten with the same values
+    assert np.array_equal(first.view(np.uint32), again.view(np.uint32))
+    toks = a.decode_greedy(7, 4300, 4, use_graph=True)
+    assert len(toks) == 4
+    a.close(); b.close()
+
+
 @pytest.mark.timeout(900)
 def test_llama2_7b_q4_0_greedy_32_tokens():
-    """The first named configuration on the engine the bench times: the 7B shape, Q4_0, 8 random prompt tokens, 32 greedy
-    steps, ctx 48.  The prompt goes through the exact-order operator kernels (library-wide switch on for that call only),
+    """The first named configuration on the engine the bench times: the 7B shape, Q4_0 body with the Q6_K output head, 8 random
+    prompt tokens, 32 greedy steps, ctx 48.  The prompt goes through the exact-order operator kernels (library-wide switch on for that call only),
     the 32 steps through the engine's default single-token pass -- the fused launches in the host backend's summation
     order, replayed as a HIP graph.  All 32 tokens must be the CPU oracle's, and so must the bits of every pass's
     logits (teacher-forced single-token passes), no filter on near-ties."""
     import os
     from spy_amd import _lib as H
     from spy_amd import model as M
-    cfg = M.Config.llama2_7b(n_ctx=48, wtype=O.Q4_0)
+    cfg = M.Config.llama2_7b(n_ctx=48, wtype=O.Q4_0, t_out=O.Q6_K)
     eng, ora, _ = _mk(cfg, seed=1234, nthread=min(16, os.cpu_count() or 8))
     assert eng.order() == 1
     prompt = np.random.default_rng(5).integers(0, cfg.n_vocab, 8).astype(np.int32)
     margins = []
     want = ora.generate(prompt, 32, margins)
-    print("7B Q4_0: prompt", prompt.tolist(), "\noracle tokens:", want.tolist(), "\nsmallest top-1/top-2 gap %.3e" % min(margins), flush=True)
+    print("7B Q4_0 + Q6_K head: prompt", prompt.tolist(), "\noracle tokens:", want.tolist(), "\nsmallest top-1/top-2 gap %.3e" % min(margins), flush=True)
     prev = H.load().spy_hip_set_exact_order(1)
     try:
         first = eng.forward_last(prompt, 0)
@@ -304,6 +328,27 @@ def test_llama2_7b_q8_0_prompt_512_then_64_tokens():
     _full_size_case(M.Config.llama2_7b(n_ctx=576, wtype=O.Q8_0), 4321, 512, 64, 16)
 
 
+@pytest.mark.timeout(600)
+def test_llama2_7b_width_4_layers_q4_0_prompt_4096_then_32_tokens():
+    """The second named configuration (the one the bench times) with 4 of its 32 layers, so that the CPU oracle's pass fits the
+    regular suite: Q4_0 body, Q6_K head, 4096-token prompt in two chunks of 2048 rows (the long-row grids of the exact prompt
+    attention: 64 query tiles, key segments beyond one), 32 greedy steps at n_kv 4097 ... 4128 in a context of 4352, 4 forced passes."""
+    from spy_amd import model as M
+    cfg = M.Config.llama2_7b(n_ctx=4352, wtype=O.Q4_0, t_out=O.Q6_K)
+    cfg.n_layer = 4
+    _full_size_case(cfg, 4323, 4096, 32, 4)
+
+
+@pytest.mark.timeout(600)
+def test_llama2_7b_width_4_layers_q4_k_m_prompt_2048_then_32_tokens():
+    """The fourth named configuration with 4 of its 32 layers: the Q4_K / Q6_K mix with 0.1 % of the weights x 20, 2048-token
+    prompt, 32 greedy steps, 4 forced passes."""
+    from spy_amd import model as M
+    cfg = M.Config.llama2_7b(n_ctx=2560, wtype=O.Q4_K, t_out=O.Q6_K, tensor_types={"attn_v": O.Q6_K, "ffn_down": O.Q6_K})
+    cfg.n_layer = 4
+    _full_size_case(cfg, 4322, 2048, 32, 4, outlier_every=1000)
+
+
 _slow = pytest.mark.skipif(not __import__("os").environ.get("SPY_FULL_SIZE_TESTS"), reason="many minutes of CPU oracle at the 7B size: set SPY_FULL_SIZE_TESTS=1")
 
 
@@ -379,7 +424,7 @@ def test_llama2_7b_prompt_4096_properties(name, kw, order, monkeypatch):
     (c) The token loop on top: decode_greedy and one-token forward passes emit the same tokens."""
     from spy_amd import model as M
     cfg = M.Config.llama2_7b(n_ctx=4096 + 32, **kw)
-    tensors = M.synth_model(cfg, seed=1234)
+    tensors = M.synth_model(cfg, seed=1234, outlier_every=1000 if kw["wtype"] == O.Q4_K else 0)     # the mix as named: 0.1 % of the weights x 20
     prompt = np.random.default_rng(4096).integers(0, cfg.n_vocab, 4096).astype(np.int32)
     eng = M.Engine(cfg, tensors, order=order)
     assert eng.order() == order

@@ -339,6 +339,41 @@ def test_prompt_attention_kernel_against_operator_sequence(hip, H_, T, past, n_c
         assert rel_err(got[:, h * hd:(h + 1) * hd], p @ vf.T) < 1e-3
 
 
+def test_prompt_attention_score_far_below_the_row_maximum(hip):
+    """A key whose score lies more than 65504 below its row's maximum: the softmax argument rounds to -inf in fp16, its
+    exponential is 0 (as expf gives in the operator sequence) and the row stays finite.  Also: a scale that is not positive
+    is refused (the kernel takes the row maximum over the raw dot products)."""
+    from tests.gpu_util import dev, dev_empty, call, rel_err
+    H_, T, past, n_ctx, hd = 2, 72, 9, 128, 128
+    d, n_kv = H_ * hd, past + T
+    rng = np.random.default_rng(5)
+    scale = 1.0 / np.sqrt(hd)
+    q = rng.standard_normal((H_, T, hd)).astype(np.float16)
+    q[:, 5::7, :] = np.float16(200.0)                                 # some queries point one way ...
+    kc = np.zeros((n_ctx, d), np.float16); kc[:n_kv] = rng.standard_normal((n_kv, d)).astype(np.float16)
+    kc[3] = np.float16(-200.0)                                        # ... and one visible key the opposite way: q.k = -5.1e6
+    vc = np.zeros((d, n_ctx), np.float16); vc[:, :n_kv] = rng.standard_normal((d, n_kv)).astype(np.float16)
+    dq, dk, dv = dev(q), dev(kc), dev(vc)
+    L = hip.load()
+    fused = dev_empty(T * d * 4, 0xFF)
+    call(L.spy_hip_prompt_attention, None, dq.ptr, dk.ptr, dv.ptr, fused.ptr, T, H_, hd, past, n_ctx, scale)
+    hip.sync()
+    got = fused.download(np.float32).reshape(T, d)
+    assert np.isfinite(got).all()
+    for h in range(H_):
+        qf, kf, vf = q[h].astype(np.float64), kc[:n_kv, h * hd:(h + 1) * hd].astype(np.float64), vc[h * hd:(h + 1) * hd, :n_kv].astype(np.float64)
+        t = ((qf @ kf.T).astype(np.float32) * np.float32(scale)).astype(np.float64)
+        t[np.arange(n_kv)[None, :] > (np.arange(T)[:, None] + past)] = -np.inf
+        with np.errstate(over="ignore"):
+            arg = (t - t.max(axis=1, keepdims=True)).astype(np.float32).astype(np.float16)
+        assert np.isneginf(arg[5, 3])                                  # the case is there: a visible key at -inf
+        e = np.exp(arg.astype(np.float64))
+        p = (e / e.sum(axis=1, keepdims=True)).astype(np.float16).astype(np.float64)
+        assert rel_err(got[:, h * hd:(h + 1) * hd], p @ vf.T) < 1e-3
+    assert L.spy_hip_prompt_attention(None, dq.ptr, dk.ptr, dv.ptr, fused.ptr, T, H_, hd, past, n_ctx, 0.0) == hip.EINVAL
+    assert L.spy_hip_prompt_attention(None, dq.ptr, dk.ptr, dv.ptr, fused.ptr, T, H_, hd, past, n_ctx, -scale) == hip.EINVAL
+
+
 def test_measured_ceilings_are_plausible(hip):
     """The measurement entry points behind the denominators of the operator sweep: the bare int8 MFMA loop, the same loop with
     the per-block scaling of the quantized GEMM in both epilogue forms, and the read scan.  Sanity bounds only: below the

@@ -1,7 +1,7 @@
 """The isolated operator sweep (configuration C5) as assertions: every kernel family at the full 7B shapes against the
 CPU oracle, through the C ABI.  GEMV: all four weight types x all four matrix shapes at batch 1, every output row for the
-three layer shapes and 2048 sampled rows for the 32000-row head; GEMM: batches 16, 128, 512 on 4096 x 4096 and
-11008 x 4096, sampled (row, token) pairs; decode attention at KV length 512 and 4096 is in test_gpu_fused_ops.py.
+three layer shapes and 2048 sampled rows for the 32000-row head; GEMM: batches 16, 128, 512 on all four shapes,
+sampled (row, token) pairs; decode attention at KV length 512 and 4096 is in test_gpu_fused_ops.py.
 Weights ~N(0, 0.02) quantized by the oracle's quantizers, activations ~N(0, 1) quantized by Quantizator<FP32,Q8_0>."""
 import numpy as np
 import pytest
@@ -43,11 +43,13 @@ def test_gemv_batch_1_all_shapes_all_types(hip, oracle, wtype, M, K):
     assert np.all(np.isfinite(got))
 
 
+@pytest.mark.parametrize("T", [16, 128, 512])            # the top decorator varies fastest: one weight matrix serves its three batches
 @pytest.mark.parametrize("wtype", TYPES)
-@pytest.mark.parametrize("M,K", [(4096, 4096), (11008, 4096)])
-@pytest.mark.parametrize("T", [16, 128, 512])
+@pytest.mark.parametrize("M,K", [(4096, 4096), (11008, 4096), (4096, 11008), (32000, 4096)])
 def test_gemm_batches_all_types(hip, oracle, wtype, M, K, T):
     from tests.gpu_util import dev, dev_empty, call, assert_close
+    if wtype in (O.Q4_K, O.Q6_K) and K % 256:
+        pytest.skip("K-quant rows are whole super-blocks of 256 elements")
     w = _weights(oracle, wtype, M, K)
     x = np.random.default_rng(T * 131 + K).standard_normal((T, K)).astype(np.float32)
     xq = O.quantize(oracle, x, O.Q8_0).reshape(T, -1)
