@@ -121,7 +121,7 @@ def main():
         log("calibration: dup_kernel over %d bytes read + %d bytes written, 3 launches" % (n * 4, n * 4))
 
     # Two summation orders of the single-token pass are timed on the same cache, from the same position:
-    #   order 1 (headline): the host backend's order -- the path whose greedy tokens and logits equal the CPU reference's bit for bit;
+    #   order 1 (headline): the host backend's order -- the path whose greedy tokens and logits equal the CPU oracle's bit for bit;
     #   order 0: this backend's own lane-parallel order (per-operator results equal to ~1e-7, greedy tokens of near-tied logits may differ).
     # Each: warm-up passes (the first also captures the HIP graphs), then exactly `steps` timed passes.
     d, F, V = cfg.n_embd, cfg.n_ff, cfg.n_vocab
@@ -209,7 +209,7 @@ def main():
     # The prompt's dominant kernels against the int8 matrix-core peak: the seven quantized GEMMs of one layer
     # (wq, wk, wv, wo: 4096 x 4096; gate, up: 11008 x 4096; down: 4096 x 11008) over the 2048 activation rows of a
     # prompt chunk, HIP events around 4 back-to-back sets.  
-    gemm_roofline = None
+    gemm_roofline, gemm_roofline_o1 = None, None
     if not args.no_gemm:
         wt_g, Tg = cfg.wtype, 2048
         d_, F_ = cfg.n_embd, cfg.n_ff
@@ -244,7 +244,8 @@ def main():
         us_set = ms.value * 1000.0 / n_set
         ops_set = 2.0 * Tg * (4 * d_ * d_ + 3 * d_ * F_)
         tops = ops_set / us_set / 1e6
-        gemm_roofline = {"kernel": "quantized GEMMs of one layer (%s weights x Q8_0 activations, int8 MFMA, per-block scales): 4 x %dx%d, 2 x %dx%d, 1 x %dx%d, %d activation rows"
+        gemm_roofline = {"summation_order": 0,
+                         "kernel": "gemm_q8act_kernel, the prompt GEMM of summation order 0 (NOT what the headline order's prompt runs: see prompt_gemm_roofline_order1): quantized GEMMs of one layer (%s weights x Q8_0 activations, int8 MFMA, per-block scales): 4 x %dx%d, 2 x %dx%d, 1 x %dx%d, %d activation rows"
                                    % ({H.Q4_0: "Q4_0", H.Q8_0: "Q8_0", H.Q4_K: "Q4_K", H.Q6_K: "Q6_K"}[wt_g], d_, d_, F_, d_, d_, F_, Tg),
                          "bound": "mfma", "achieved": round(tops, 1), "peak": INT8_PEAK / 1e12, "unit": "TOP/s", "frac": round(tops * 1e12 / INT8_PEAK, 4),
                          "ops_per_set": ops_set, "us_per_set": round(us_set, 1)}
@@ -255,6 +256,42 @@ def main():
                                                       "what": "one v_mfma_i32_32x32x32_i8 + the fp16 scale outer product + subtraction and fma per output, no LDS or memory"}
         log("prompt GEMMs of a layer, T = %d: %.1f us, %.0f TOP/s (%.1f%% of the int8 MFMA peak); its inner loop on register operands only: %.0f TOP/s (%.1f%%)"
             % (Tg, us_set, tops, 100 * tops * 1e12 / INT8_PEAK, ceil_tops.value, 100 * ceil_tops.value * 1e12 / INT8_PEAK))
+        # The same seven products the way the prompt pass of summation order 1 runs them: spy_hip_op_matmul in the host backend's
+        # order = Q8_0 quantization of the f32 activations, both operands packed as fp16, exact_gemm8p_kernel (integer sums of
+        # four products from v_mfma_f32_16x16x4_4b_f16, one fma per accumulator and block on the vector units).
+        gemm_roofline_o1 = None
+        if cfg.wtype in (H.Q4_0, H.Q8_0):
+            prev = L.spy_hip_set_exact_order(1)
+            try:
+                xf_d = H.DeviceBuffer.from_numpy(np.random.default_rng(d_).standard_normal((Tg, d_)).astype(np.float32))
+                xf_F = H.DeviceBuffer.from_numpy(np.random.default_rng(F_).standard_normal((Tg, F_)).astype(np.float32))
+                sets = [(w_dd, xf_d, d_, d_)] * 4 + [(w_Fd, xf_d, F_, d_)] * 2 + [(w_dF, xf_F, d_, F_)]
+                tens = [(H.tensor(wb_, wt_g, [Kg, Mg]), H.tensor(xb_, H.F32, [Kg, Tg]), H.tensor(og, H.F32, [Mg, Tg])) for (wb_, xb_, Mg, Kg) in sets]
+                need = max(L.spy_hip_op_matmul_scratch_size(C.byref(tw), C.byref(tx)) for tw, tx, _ in tens)
+                scr = H.DeviceBuffer(need)
+                n_set1 = 2
+                for timed in (False, True):
+                    H.check(L.spy_hip_event_record(e0, None), "record")
+                    for i in range(n_set1):
+                        for tw, tx, to in tens:
+                            H.check(L.spy_hip_op_matmul(None, C.byref(tw), C.byref(tx), C.byref(to), scr.ptr, need), "spy_hip_op_matmul")
+                    H.check(L.spy_hip_event_record(e1, None), "record")
+                    H.sync()
+                H.check(L.spy_hip_event_elapsed_ms(e0, e1, C.byref(ms)), "elapsed")
+                us1 = ms.value * 1000.0 / n_set1
+                tops1 = ops_set / us1 / 1e6
+                gemm_roofline_o1 = {"summation_order": 1,
+                                    "kernel": "exact_gemm8p_kernel + xgp_pack_kernel x 2 + Q8_0 quantization, the prompt MatMul of summation order 1 (the headline's): the same seven products "
+                                              "through spy_hip_op_matmul in the host backend's order; integer sums of four products from v_mfma_f32_16x16x4_4b_f16 (fp16 matrix instructions), "
+                                              "one fp32 fma per accumulator and block on the vector units",
+                                    "bound": "mfma", "achieved": round(tops1, 1), "peak": INT8_PEAK / 1e12, "unit": "TOP/s", "frac": round(tops1 * 1e12 / INT8_PEAK, 4),
+                                    "frac_of_fp16_mfma_peak": round(tops1 * 1e12 / 2.5e15, 4), "ops_per_set": ops_set, "us_per_set": round(us1, 1)}
+                log("prompt MatMuls of a layer in summation order 1, T = %d: %.1f us, %.0f TOP/s (%.1f%% of the int8 MFMA peak, %.1f%% of the fp16 MFMA peak its matrix instructions have)"
+                    % (Tg, us1, tops1, 100 * tops1 * 1e12 / INT8_PEAK, 100 * tops1 * 1e12 / 2.5e15))
+                for b in (xf_d, xf_F, scr):
+                    b.free()
+            finally:
+                L.spy_hip_set_exact_order(prev)
         for b in (w_dd, w_Fd, w_dF, x_d, x_F, og):
             b.free()
 
@@ -283,9 +320,10 @@ def main():
     weights_desc = {"q4_0": "Q4_0 weights, %s" % head_desc, "q8_0": "Q8_0 weights incl. head",
                     "q4_k_m": "Q4_K weights with Q6_K attn_v / ffn_down / head, 0.1 %% of the weights x 20"}[args.model] + \
                    " (seeded ~N(0, 0.02), quantized by the package's block quantizers)"
-    prefill_note = {1: "prompt pass in the host backend's summation order (tiled exact kernels: integer sums from the matrix cores as floats, every accumulator of the host loops kept apart on the vector units): same logits and caches as the CPU reference's",
+    prefill_note = {1: "prompt pass in the host backend's summation order (tiled exact kernels: integer sums from the matrix cores as floats, every accumulator of the host loops kept apart on the vector units): same logits and caches as the CPU oracle's",
                     0: "matrix-core prompt pass in the backend's own order"}
-    mode_desc = {1: "host-backend summation order: logits and greedy tokens equal to the CPU reference's bit for bit",
+    mode_desc = {1: "host-backend summation order: logits and greedy tokens equal, bit for bit, to the CPU oracle's (Spy's host backend restated, fp contraction off; "
+                    "a GCC build of Spy with its default -ffp-contract=fast fuses x * x + y in NormRMS and differs from both in the last bits)",
                  0: "this backend's own summation order (per-operator 1e-7; not token-exact)"}
     out = {
         "metric": "decode tok/s + %% HBM roofline, LLaMA-2-7B %s ctx 4096, 1xMI355X" % {"q4_0": "Q4_0", "q8_0": "Q8_0", "q4_k_m": "Q4_K_M"}[args.model],
@@ -300,7 +338,8 @@ def main():
         "prefill": {"tokens": fill, "seconds": round(prefill_s[orders[0]], 3), "tok_s": round(fill / prefill_s[orders[0]], 1), "summation_order": orders[0],
                     "note": prefill_note[orders[0]]} if args.prefill == "real" else None,
         "kernel_us": {k: round(v, 2) for k, v in per_kernel.items()},
-        "roofline": roofline, "roofline_other_kernels": roofline_others, "prompt_gemm_roofline": gemm_roofline, "cpu_baseline": cpu,
+        "roofline": roofline, "roofline_other_kernels": roofline_others, "prompt_gemm_roofline": gemm_roofline_o1 if (orders[0] == 1 and gemm_roofline_o1) else gemm_roofline,
+        "prompt_gemm_roofline_other_order": gemm_roofline if (orders[0] == 1 and gemm_roofline_o1) else gemm_roofline_o1, "cpu_baseline": cpu,
     }
     if len(orders) > 1:
         o = runs[orders[1]]

@@ -39,6 +39,11 @@ int spy_host_model_stats(spy_host_model *m, int64_t *n_ops, int64_t *n_submit, i
 int spy_host_model_cache(spy_host_model *m, int layer, int which, void *dst_host);
 int spy_host_model_destroy(spy_host_model *m);
 
+/* One unary operator node through Backend::submit: x = f32 [ne1][ne0] in host memory (an IO node), the result in host memory
+ * too.  op: 0 Relu, 1 Silu, 2 Quantize to target_type (NumberType code; out_bytes = the result's size in that type).
+ * Returns 0, -1 if the backend does not take the operator or conversion, -2 on bad arguments, else the backend's error. */
+int spy_host_unary_through_submit(const char *backend_name, int op, const float *x, int64_t ne0, int64_t ne1, int target_type, void *out, int64_t out_bytes);
+
 #ifdef __cplusplus
 }
 #endif

@@ -112,6 +112,12 @@ int spy_hip_op_norm_rms(void *stream, const spy_hip_tensor *x, const spy_hip_ten
 int spy_hip_op_binary(void *stream, int op, const spy_hip_tensor *a, const spy_hip_tensor *b, const spy_hip_tensor *dst);
 /* Silu -- OperatorSiluImpl::execute (non-linear.cpp:57-77) */
 int spy_hip_op_silu(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *dst);
+/* Relu -- OperatorReluImpl::execute (non-linear.cpp:16-50): max(x, 0), f32 */
+int spy_hip_op_relu(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *dst);
+/* Quantize -- OperatorQuantizeImpl::execute (backend/host/operator/quantize.cpp:18-41): rows of x converted to dst's type by
+ * auto_quantize_inner (vec_convert.h:463-468).  F32 -> Q8_0 and F32 -> F16; dst rows back to back.  F32 -> Q4_0 is
+ * SPY_HIP_EUNSUPPORTED: the reference's own (vec_convert.h:83-117) fills half of every block and inverts the scale. */
+int spy_hip_op_quantize(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *dst);
 /* Softmax -- OperatorSoftmaxImpl::execute (non-linear.cpp:86-185); mask may be NULL;
  * scale = SoftmaxParam::scale.  dst may also be FP16 (rows of up to 16384 elements, scale > 0): the
  * probabilities rounded the way the KQV MatMul rounds its right operand first (mat.cpp:37), so that the
@@ -120,8 +126,11 @@ int spy_hip_op_softmax(void *stream, const spy_hip_tensor *x, const spy_hip_tens
 /* Rope -- OperatorRopeImpl::execute (non-linear.cpp:270-371); fields of RopeParam
  * (orchestration/include/operator/non-linear.h:191-207).  Supported: mode None/Norm (-1/0), including
  * extend_factor != 0 (rope_yarn, :242-260: as written its ramp is 0, so the angle stays the interpolated one and the
- * magnitude is multiplied by 1 + 0.1 ln(1 / freq_scale)) and xpos_base != 0 (zeta, :353-354).  GLM and Neox (the
- * latter aborts in the reference) -> EUNSUPPORTED. */
+ * magnitude is multiplied by 1 + 0.1 ln(1 / freq_scale)) and xpos_base != 0 (zeta, :353-354), and mode GLM (4; :315-343,
+ * as written: elements i0, i0 + num_dim / 2 rotated by min(p, num_context - 2) * theta_scale^i0 and elements i0 + num_dim,
+ * i0 + 3 num_dim / 2 by max(p - (num_context - 2), 0) * theta_scale^i0 for i0 < ne0 / 4; rows in which those indices would
+ * leave the row are refused with EINVAL where the reference reads past it; not in the exact-order mode).  Neox (2) aborts in
+ * the reference and is EUNSUPPORTED here. */
 typedef struct spy_hip_rope_param {
     int32_t mode, num_past, num_dim, num_context, num_origin_context;
     float   freq_base, freq_scale, extend_factor, attention_factor, beta_fast, beta_slow, xpos_base;

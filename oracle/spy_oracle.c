@@ -834,6 +834,32 @@ int spy_o_silu(const spy_o_tensor *x, spy_o_tensor *dst) {
     return 0;
 }
 
+/* OperatorReluImpl::execute (non-linear.cpp:28-50) with Relu<T> (:16-19): std::max(val, 0) */
+int spy_o_relu(const spy_o_tensor *x, spy_o_tensor *dst) {
+    const int64_t ne00 = x->ne[0], ne01 = x->ne[1], ne02 = x->ne[2], nrow = t_nrow(x);
+    for (int64_t r = 0; r < nrow; r++) {
+        const int64_t i03 = r / (ne01 * ne02), i02 = r % (ne01 * ne02) / ne01, i01 = r % ne01;
+        const float *s = (const float *)tget(x, 0, i01, i02, i03);
+        float *d = (float *)tget(dst, 0, i01, i02, i03);
+        for (int64_t i = 0; i < ne00; i++) d[i] = (s[i] < 0.0f) ? 0.0f : s[i];      /* std::max(a, b) = (a < b) ? b : a */
+    }
+    return 0;
+}
+
+/* OperatorQuantizeImpl::execute (backend/host/operator/quantize.cpp:18-41): rows through auto_quantize_inner
+ * (vec_convert.h:463-468); F32 -> Q8_0 and F32 -> F16 (the reference's F32 -> Q4_0 is the known-bad *_as_written) */
+int spy_o_quantize(const spy_o_tensor *x, spy_o_tensor *dst) {
+    if (x->type != SPY_O_F32 || (dst->type != SPY_O_Q8_0 && dst->type != SPY_O_F16)) return 1;
+    const int64_t ne00 = x->ne[0], ne01 = x->ne[1], ne02 = x->ne[2], nrow = t_nrow(x);
+    for (int64_t r = 0; r < nrow; r++) {
+        const int64_t i03 = r / (ne01 * ne02), i02 = r % (ne01 * ne02) / ne01, i01 = r % ne01;
+        const float *s = (const float *)tget(x, 0, i01, i02, i03);
+        void *d = tget(dst, 0, i01, i02, i03);
+        if (dst->type == SPY_O_Q8_0) spy_o_quantize_q8_0(s, d, ne00); else spy_o_quantize_f16(s, (uint16_t *)d, ne00);
+    }
+    return 0;
+}
+
 /* operator_softmax_execute (non-linear.cpp:86-127) when mask == NULL, else
  * operator_masked_softmax_execute (:129-180): t = (s + mask) * scale; m = max t; t -= m;
  * e = mask == -inf ? 0 : exp_lut(fp16(t)); sum = std::reduce(e); e *= 1/sum. */
@@ -894,8 +920,34 @@ static void rope_yarn(float theta_extrap, float freq_scale, const float corr[2],
  * per pair (:304-309); adjacent pairs are rotated (:349-364).  GLM / Neox: unsupported here
  * (Neox aborts in the reference too, :344-346). */
 int spy_o_rope(const spy_o_tensor *x, const spy_o_tensor *pos, spy_o_tensor *dst, const spy_o_rope_param *p) {
-    if (p->mode == 2 || p->mode == 4) return 1;
+    if (p->mode == 2) return 1;
     const float theta_scale = powf(p->freq_base, -2.0f / (float)p->num_dim);
+    if (p->mode == 4) {
+        /* GLM (non-linear.cpp:315-343), as written; the caller keeps the four indices of every i0 inside the row */
+        const int64_t ne0 = dst->ne[0], ne1 = dst->ne[1], ne2 = dst->ne[2], ne3 = dst->ne[3];
+        const int nd = p->num_dim;
+        for (int64_t mi = 0; mi < ne2 * ne3; mi++) {
+            const int64_t i3 = mi / ne2, i2 = mi % ne2;
+            const int32_t pp = ((const int32_t *)pos->data)[i2];
+            for (int64_t i1 = 0; i1 < ne1; i1++) {
+                float theta_base = (float)(pp < p->num_context - 2 ? pp : p->num_context - 2);
+                float block_theta = (float)(pp - (p->num_context - 2) > 0 ? pp - (p->num_context - 2) : 0);
+                for (int64_t i0 = 0; i0 < ne0 / 4; i0++) {
+                    const float c = cosf(theta_base), s = sinf(theta_base), cb = cosf(block_theta), sb = sinf(block_theta);
+                    theta_base *= theta_scale;
+                    block_theta *= theta_scale;
+                    const float *sp = (const float *)tget(x, i0, i1, i2, i3);
+                    float *dp = (float *)tget(dst, i0, i1, i2, i3);
+                    const float x0 = sp[0], x1 = sp[nd / 2], x2 = sp[nd], x3 = sp[nd / 2 + nd];
+                    dp[0] = x0 * c - x1 * s;
+                    dp[nd / 2] = x0 * s + x1 * c;
+                    dp[nd] = x2 * cb - x3 * sb;
+                    dp[nd / 2 + nd] = x2 * sb + x3 * cb;
+                }
+            }
+        }
+        return 0;
+    }
     float corr[2];
     {
         const float start = floorf(yarn_corr_dim(p->num_dim, p->num_origin_context, p->beta_fast, p->freq_base));

@@ -91,6 +91,8 @@ int spy_o_matmul(const spy_o_tensor *w, const spy_o_tensor *x, spy_o_tensor *dst
 int spy_o_norm_rms(const spy_o_tensor *x, spy_o_tensor *dst, float eps);                              /* non-linear.cpp:194-223 */
 int spy_o_binary(int op, const spy_o_tensor *a, const spy_o_tensor *b, spy_o_tensor *dst);            /* basic.cpp:15-50; op 0 add 1 sub 2 mul 3 div */
 int spy_o_silu(const spy_o_tensor *x, spy_o_tensor *dst);                                             /* non-linear.cpp:57-77 */
+int spy_o_relu(const spy_o_tensor *x, spy_o_tensor *dst);                                             /* non-linear.cpp:16-50 */
+int spy_o_quantize(const spy_o_tensor *x, spy_o_tensor *dst);                                         /* quantize.cpp:18-41; F32 -> Q8_0 / F16 */
 int spy_o_softmax(const spy_o_tensor *x, const spy_o_tensor *mask, spy_o_tensor *dst, float scale);   /* non-linear.cpp:86-180 */
 typedef struct spy_o_rope_param {  /* operator/non-linear.h:191-207 */
     int32_t mode, num_past, num_dim, num_context, num_origin_context;

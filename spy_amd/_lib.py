@@ -87,6 +87,8 @@ SIGNATURES = {
     "spy_hip_op_norm_rms": (_i32, [_vp, _TP, _TP, _f32]),
     "spy_hip_op_binary": (_i32, [_vp, _i32, _TP, _TP, _TP]),
     "spy_hip_op_silu": (_i32, [_vp, _TP, _TP]),
+    "spy_hip_op_relu": (_i32, [_vp, _TP, _TP]),
+    "spy_hip_op_quantize": (_i32, [_vp, _TP, _TP]),
     "spy_hip_op_softmax": (_i32, [_vp, _TP, _TP, _TP, _f32]),
     "spy_hip_op_rope": (_i32, [_vp, _TP, _TP, _TP, C.POINTER(RopeParam)]),
     "spy_hip_rope_prepare": (_i32, [C.POINTER(RopeParam), _i64]),

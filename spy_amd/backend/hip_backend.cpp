@@ -124,6 +124,7 @@ bool HIPBackend::is_support(OperatorType t) const {
     case OperatorType::GetRow: case OperatorType::Transpose: case OperatorType::Permute: case OperatorType::Contiguous:
     case OperatorType::Silu: case OperatorType::Softmax: case OperatorType::Add: case OperatorType::Sub: case OperatorType::Mul:
     case OperatorType::Div: case OperatorType::MatMul: case OperatorType::NormRMS: case OperatorType::Rope:
+    case OperatorType::Relu: case OperatorType::Quantize:
         return true;
     default:
         return false;
@@ -216,6 +217,8 @@ OperatorStatus HIPBackend::run(OperatorNode *op) {
     case OperatorType::Mul: rc = spy_hip_op_binary(stream_, 2, &in[0], &in[1], &out); break;
     case OperatorType::Div: rc = spy_hip_op_binary(stream_, 3, &in[0], &in[1], &out); break;
     case OperatorType::Silu: rc = spy_hip_op_silu(stream_, &in[0], &out); break;
+    case OperatorType::Relu: rc = spy_hip_op_relu(stream_, &in[0], &out); break;
+    case OperatorType::Quantize: rc = spy_hip_op_quantize(stream_, &in[0], &out); break;
     case OperatorType::Softmax:
         rc = spy_hip_op_softmax(stream_, &in[0], nin > 1 ? &in[1] : nullptr, &out,
                                 static_cast<OperatorDefinition<OperatorType::Softmax> *>(op)->params.get_val().scale);

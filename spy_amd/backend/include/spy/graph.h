@@ -92,7 +92,7 @@ template <OperatorType T_op_type> struct OperatorDefinition {};
         void propagate() override;                                             \
     };
 SPY_SIMPLE_OP(Input) SPY_SIMPLE_OP(Nop) SPY_SIMPLE_OP(Dup) SPY_SIMPLE_OP(Copy) SPY_SIMPLE_OP(GetRow) SPY_SIMPLE_OP(Transpose)
-SPY_SIMPLE_OP(Contiguous) SPY_SIMPLE_OP(Silu) SPY_SIMPLE_OP(Add) SPY_SIMPLE_OP(Sub) SPY_SIMPLE_OP(Mul) SPY_SIMPLE_OP(Div) SPY_SIMPLE_OP(MatMul)
+SPY_SIMPLE_OP(Contiguous) SPY_SIMPLE_OP(Silu) SPY_SIMPLE_OP(Relu) SPY_SIMPLE_OP(Add) SPY_SIMPLE_OP(Sub) SPY_SIMPLE_OP(Mul) SPY_SIMPLE_OP(Div) SPY_SIMPLE_OP(MatMul)
 #undef SPY_SIMPLE_OP
 
 #define SPY_PARAM_OP(OP, ...)                                                  \
@@ -108,6 +108,7 @@ SPY_PARAM_OP(NormRMS, struct Param { float eps; };)                             
 SPY_PARAM_OP(Reshape, struct Param { Shape new_shape; };)                           // view.h (Reshape)
 SPY_PARAM_OP(View, struct Param { int64_t offset; Shape new_shape; };)              // view.h (View)
 SPY_PARAM_OP(Permute, struct Param { std::array<int64_t, MAX_DIM> axis; };)         // view.h (Permute)
+SPY_PARAM_OP(Quantize, struct Param { NumberType target_type; };)                   // operator/quantize.h:19
 enum class RopeType : int { None = -1, Norm = 0, Neox = 2, GLM = 4 };              // non-linear.h:184-189
 SPY_PARAM_OP(Rope, struct Param {                                                   // non-linear.h:191-207
     RopeType mode; int32_t num_past, num_dim, num_context, num_origin_context;
@@ -120,5 +121,6 @@ using ReshapeParam = OperatorDefinition<OperatorType::Reshape>::Param;
 using ViewParam    = OperatorDefinition<OperatorType::View>::Param;
 using PermuteParam = OperatorDefinition<OperatorType::Permute>::Param;
 using RopeParam    = OperatorDefinition<OperatorType::Rope>::Param;
+using QuantizeParam = OperatorDefinition<OperatorType::Quantize>::Param;
 
 }  // namespace spy

@@ -29,6 +29,14 @@ void OperatorDefinition<OperatorType::Input>::propagate() {}
 void OperatorDefinition<OperatorType::Nop>::propagate() { same_as_input(this); output_data(0)->view_src = input_data(0); }
 void OperatorDefinition<OperatorType::Dup>::propagate() { same_as_input(this); }
 void OperatorDefinition<OperatorType::Silu>::propagate() { same_as_input(this); }
+void OperatorDefinition<OperatorType::Relu>::propagate() { same_as_input(this); }
+void OperatorDefinition<OperatorType::Quantize>::propagate() {                      // operator/quantize.h: the operand's elements in the target type
+    const Shape &s = input_data(0)->tensor.shape;
+    DataNode *o = output_data(0);
+    o->view_src = nullptr;
+    o->tensor.shape = Shape({s.elements[0], s.elements[1], s.elements[2], s.elements[3]}, params.get_val().target_type);
+    o->tensor.shape.dim = s.dim;
+}
 void OperatorDefinition<OperatorType::Softmax>::propagate() { same_as_input(this); }
 void OperatorDefinition<OperatorType::NormRMS>::propagate() { same_as_input(this); }
 void OperatorDefinition<OperatorType::Rope>::propagate() { same_as_input(this); }
@@ -307,5 +315,41 @@ int spy_host_model_cache(spy_host_model *h, int layer, int which, void *dst_host
 }
 
 int spy_host_model_destroy(spy_host_model *h) { delete h; return 0; }
+
+// One unary operator node through Backend::submit on host data: x = f32 [ne1][ne0] (IO node, uploaded by the backend), the
+// result an IO node as well (host-visible when submit's callback has run).  op: 0 Relu, 1 Silu, 2 Quantize to target_type
+// (NumberType code).  Returns 0, -1 unsupported by the backend, -2 bad arguments, else the backend's error.
+int spy_host_unary_through_submit(const char *backend_name, int op, const float *x, int64_t ne0, int64_t ne1, int target_type, void *out, int64_t out_bytes) {
+    if (!backend_name || !x || !out || ne0 <= 0 || ne1 <= 0) return -2;
+    BackendFactory factory;
+    ConfigTable config;
+    config.set("device_id", "0");
+    std::unique_ptr<Backend> be = factory.init_backend(backend_name, config);
+    if (!be) return -1;
+    DataNode in, res;
+    in.name = "x"; in.node_prop.node_type = DataNodeType::IO; in.id = 0;
+    in.tensor = Tensor(Shape({ne0, ne1}, NumberType::FP32), const_cast<float *>(x));
+    res.name = "y"; res.node_prop.node_type = DataNodeType::IO; res.id = 1;
+    std::unique_ptr<OperatorNode> node;
+    if (op == 0) node = std::make_unique<OperatorDefinition<OperatorType::Relu>>();
+    else if (op == 1) node = std::make_unique<OperatorDefinition<OperatorType::Silu>>();
+    else if (op == 2) node = std::make_unique<OperatorDefinition<OperatorType::Quantize>>(QuantizeParam{static_cast<NumberType>(target_type)});
+    else return -2;
+    node->add_input(&in);
+    node->add_output(&res);
+    node->propagate();
+    if ((int64_t)res.tensor.total_size() != out_bytes) return -2;
+    res.tensor.set_data_ptr(out);
+    if (!be->is_support(node->op_type)) return -1;
+    bool called = false;
+    be->submit(node.get(), [&called]() { called = true; });
+    if (!called) return 1;
+    auto *hb = dynamic_cast<spy::hip::HIPBackend *>(be.get());
+    if (hb) {
+        hb->sync();
+        if (hb->last_status() != OperatorStatus::Success) return hb->last_status() == OperatorStatus::Unsupport ? -1 : (hb->last_error() ? hb->last_error() : 1);
+    }
+    return 0;
+}
 
 }  // extern "C"

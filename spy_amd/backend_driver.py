@@ -22,6 +22,7 @@ SIGNATURES = {
     "spy_host_model_stats": [C.c_void_p, C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.POINTER(C.c_int64)],
     "spy_host_model_cache": [C.c_void_p, C.c_int, C.c_int, C.c_void_p],
     "spy_host_model_destroy": [C.c_void_p],
+    "spy_host_unary_through_submit": [C.c_char_p, C.c_int, C.c_void_p, C.c_int64, C.c_int64, C.c_int, C.c_void_p, C.c_int64],
 }
 
 
@@ -85,3 +86,17 @@ class HostModel:
             self.close()
         except Exception:
             pass
+
+
+def unary_through_submit(op, x, target_type=H.F32, backend="hip:default"):
+    """One unary operator node (op: "relu", "silu", "quantize") on the rows of x (float32 [rows, cols]) through Backend::submit.
+    Returns the result bytes as uint8 (quantize) or float32."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    rows, cols = x.shape
+    code = {"relu": 0, "silu": 1, "quantize": 2}[op]
+    ttype = target_type if op == "quantize" else H.F32
+    out = np.zeros(rows * H.row_size(ttype, cols), dtype=np.uint8)
+    rc = load().spy_host_unary_through_submit(backend.encode(), code, x.ctypes.data, cols, rows, ttype, out.ctypes.data, out.nbytes)
+    if rc != 0:
+        raise H.SpyHipError(rc, "spy_host_unary_through_submit") if rc > 0 else RuntimeError("spy_host_unary_through_submit: %d" % rc)
+    return out if op == "quantize" else out.view(np.float32).reshape(rows, cols)

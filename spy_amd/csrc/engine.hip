@@ -91,10 +91,7 @@ extern "C" int spy_hip_llama_create(const spy_hip_llama_desc *desc, spy_hip_llam
     }
     m->cfg_d  = pick_cfg(c.n_embd, 32);
     m->cfg_ff = pick_cfg(c.n_ff);
-    {   // SPY_HIP_TILED=1 keeps the 256-thread tiled kernels (the only ones for n_embd > 4096)
-        const char *env = getenv("SPY_HIP_TILED");
-        m->wave = wave_ok(m) && !(env && env[0] == '1' && m->uniform);
-    }
+    m->wave = wave_ok(m);                   // n_embd > 4096 (uniform Q4_0 / Q8_0 models): the 256-thread tiled kernels
     {
         int dev = 0; hipDeviceProp_t prop;
         if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0) m->num_cu = prop.multiProcessorCount;
@@ -391,7 +388,7 @@ static int forward_ops(spy_hip_llama *m, hipStream_t st, const int32_t *tokens_h
     // next MatMul's Q8_0 activations directly (same bytes as the separate operators: prompt_fused.hip)
     // exact-order mode (spy_hip_set_exact_order): the plain operators only, each in its exact form
     const bool exact = spy_exact_on() != 0;
-    const bool fuse_act = !exact && T >= 16 && d % 64 == 0 && F % 64 == 0 && !getenv("SPY_HIP_PROMPT_UNFUSED");
+    const bool fuse_act = !exact && T >= 16 && d % 64 == 0 && F % 64 == 0;
     // ... and the attention of a layer is one kernel (prompt_attn.hip) where its shape conditions hold;
     // SPY_HIP_PROMPT_ATTN=0: attention as MatMul -> Softmax -> MatMul (bit-identical to the operator path)
     const char *pa_env = getenv("SPY_HIP_PROMPT_ATTN");
@@ -582,7 +579,7 @@ static int forward_any(spy_hip_llama *m, void *stream, const int32_t *tokens_hos
     const bool exact = spy_exact_on() != 0;
     // single tokens: the fused pass, in the order pass_order() names (with the library-wide exact-order switch on and a
     // model the exact kernels do not take, operator by operator instead)
-    if (n_token == 1 && fused_ok(m) && (!exact || m->exact_ok) && !getenv("SPY_HIP_FORCE_OPS")) {
+    if (n_token == 1 && fused_ok(m) && (!exact || m->exact_ok)) {
         dev_state h = {tokens_host[0], n_past, 0, 0};
         HIP_TRY(hipMemcpyAsync(m->st, &h, sizeof(h), hipMemcpyHostToDevice, st));
         RC_TRY(enqueue_pass_any(m, st, PASS_LOGITS));
@@ -625,7 +622,7 @@ extern "C" int spy_hip_llama_decode_greedy(spy_hip_llama *m, void *stream, int32
                                            int32_t *tokens_host, int32_t use_graph) {
     SPY_CHECK_ARG(m && n_steps > 0 && n_past >= 0 && first_token >= 0 && first_token < m->desc.n_vocab);
     SPY_CHECK_ARG((int64_t)n_past + n_steps <= m->desc.n_ctx && n_steps <= m->max_out);
-    if (spy_exact_on() && (!m->exact_ok || getenv("SPY_HIP_FORCE_OPS"))) {
+    if (spy_exact_on() && !m->exact_ok) {
         // exact order for a model the fused exact kernels do not take: the reference's loop as it stands (cli.h:88-128) -- one operator-by-operator pass per token,
         // the first maximum of its logits (greedy.h:20-25) taken on the host
         std::vector<float> lg((size_t)m->desc.n_vocab);

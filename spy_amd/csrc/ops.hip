@@ -174,6 +174,55 @@ extern "C" int spy_hip_op_silu(void *stream, const spy_hip_tensor *x, const spy_
 }
 
 // ---------------------------------------------------------------------------------------------
+// Relu (non-linear.cpp:16-19,28-50): std::max(x, 0) element by element (a NaN stays a NaN: std::max returns its first
+// argument unless it is smaller than the second).
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void relu_kernel(tdesc x, tdesc d, int64_t total) {
+    const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (g >= total) return;
+    const int64_t i0 = g % x.ne[0], r = g / x.ne[0];
+    const int64_t i1 = r % x.ne[1], i2 = r / x.ne[1] % x.ne[2], i3 = r / (x.ne[1] * x.ne[2]);
+    const float v = *(const float *)at(x, i0, i1, i2, i3);
+    *(float *)at(d, i0, i1, i2, i3) = v < 0.0f ? 0.0f : v;
+}
+
+extern "C" int spy_hip_op_relu(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *dst) {
+    SPY_CHECK_ARG(x && dst && x->data && dst->data);
+    if (x->type != SPY_HIP_F32 || dst->type != SPY_HIP_F32) return SPY_HIP_EUNSUPPORTED;
+    SPY_CHECK_ARG(same_ne(x, dst) && x->nb[0] == 4 && dst->nb[0] == 4);
+    const int64_t total = spy_t_nelem(x);
+    CHECK_GRID(total, 256);
+    relu_kernel<<<dim3(grid_for(total, 256)), dim3(256), 0, (hipStream_t)stream>>>(mk(x), mk(dst), total);
+    return SPY_LAUNCH_RC();
+}
+
+// ---------------------------------------------------------------------------------------------
+// Quantize (backend/host/operator/quantize.cpp:18-41): row by row through auto_quantize_inner (vec_convert.h:463-468).
+// F32 -> Q8_0 (Quantizator<FP32,Q8_0>, :178-261) and F32 -> F16 (:39-65) are the conversions of the reference that work;
+// its F32 -> Q4_0 fills half of every block and inverts the scale (:83-117) and is refused here, like the K-quants
+// (no quantizer in the reference at all).
+// ---------------------------------------------------------------------------------------------
+extern "C" int spy_hip_op_quantize(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *dst) {
+    SPY_CHECK_ARG(x && dst && x->data && dst->data);
+    if (x->type != SPY_HIP_F32 || (dst->type != SPY_HIP_Q8_0 && dst->type != SPY_HIP_F16)) return SPY_HIP_EUNSUPPORTED;
+    SPY_CHECK_ARG(same_ne(x, dst) && x->nb[0] == 4 && dst->nb[0] == spy_type_size(dst->type) && x->ne[0] > 0 && spy_t_nrow(x) > 0);
+    if (dst->type == SPY_HIP_Q8_0) SPY_CHECK_ARG(x->ne[0] % 32 == 0);
+    // rows of a matrix in one launch where both sides step evenly from row to row; otherwise one launch per matrix
+    const int64_t K = x->ne[0], drow = spy_row_size(dst->type, K);
+    const bool dst_rows_packed = dst->nb[1] == drow && dst->nb[2] == drow * dst->ne[1] && dst->nb[3] == dst->nb[2] * dst->ne[2];
+    SPY_CHECK_ARG(dst_rows_packed);                                     // the quantizing kernels write rows back to back
+    for (int64_t i3 = 0; i3 < x->ne[3]; i3++)
+        for (int64_t i2 = 0; i2 < x->ne[2]; i2++) {
+            const float *src = (const float *)((const uint8_t *)x->data + i2 * x->nb[2] + i3 * x->nb[3]);
+            uint8_t *out = (uint8_t *)dst->data + i2 * dst->nb[2] + i3 * dst->nb[3];
+            const int rc = dst->type == SPY_HIP_Q8_0 ? spy_hip_quantize_q8_0(stream, src, x->nb[1], out, x->ne[1], K)
+                                                     : spy_hip_quantize_f16(stream, src, x->nb[1], out, x->ne[1], K);
+            if (rc) return rc;
+        }
+    return 0;
+}
+
+// ---------------------------------------------------------------------------------------------
 // Softmax (non-linear.cpp:86-180): t = (s + mask) * scale; m = max t; e = mask == -inf ? 0 :
 // expf(float(fp16(t - m))); p = e * (1 / sum e).  One workgroup per row; dst doubles as the
 // row scratch exactly as in the reference.
@@ -264,7 +313,7 @@ __global__ __launch_bounds__(256) void softmax_row_kernel(tdesc x, tdesc mask, b
 static int softmax_launch(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *mask, const spy_hip_tensor *dst, float scale, int causal_past);
 // Softmax under the causal mask of a pass that starts at position n_past, without reading a mask tensor (the token
 // loop fills its masks itself and knows their shape).  Same bits as spy_hip_op_softmax with that mask.
-int spy_softmax_row_ok(int64_t ne0) { return ne0 <= SOFTMAX_LDS_ROW && !getenv("SPY_HIP_SOFTMAX_GENERIC"); }   // rows of ne0 elements take the row kernel
+int spy_softmax_row_ok(int64_t ne0) { return ne0 <= SOFTMAX_LDS_ROW; }   // rows of ne0 elements take the row kernel
 int spy_softmax_causal_launch(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *dst, float scale, int n_past) {
     SPY_CHECK_ARG(n_past >= 0 && dst && scale > 0.0f && spy_softmax_row_ok(dst->ne[0]));
     return softmax_launch(stream, x, nullptr, dst, scale, n_past);
@@ -344,10 +393,44 @@ __global__ __launch_bounds__(64) void rope_kernel(tdesc x, const int32_t *pos, i
     }
 }
 
+// Mode GLM (non-linear.cpp:315-343), as written: per row (i1, i2, i3) and i0 < ne0 / 4, with p = pos[i2]:
+// theta_base = min(p, num_context - 2), block_theta = max(p - (num_context - 2), 0), both multiplied by theta_scale once per
+// i0; elements i0 and i0 + num_dim / 2 are rotated by theta_base, elements i0 + num_dim and i0 + num_dim / 2 + num_dim by
+// block_theta.  cosf / sinf on the device (within the per-operator tolerance of the host's).
+__global__ __launch_bounds__(64) void rope_glm_kernel(tdesc x, const int32_t *pos, int64_t pos_stride, tdesc y, float theta_scale, int num_context, int num_dim) {
+    const int64_t i1 = blockIdx.x, i2 = blockIdx.y, i3 = blockIdx.z;
+    const int32_t p = *(const int32_t *)((const uint8_t *)pos + i2 * pos_stride);
+    const int nd = num_dim;
+    for (int64_t i0 = threadIdx.x; i0 < y.ne[0] / 4; i0 += 64) {
+        float theta_base = (float)min(p, num_context - 2), block_theta = (float)max(p - (num_context - 2), 0);
+        for (int64_t j = 0; j < i0; j++) { theta_base *= theta_scale; block_theta *= theta_scale; }
+        const float c = cosf(theta_base), s = sinf(theta_base), cb = cosf(block_theta), sb = sinf(block_theta);
+        const float *sp = (const float *)at(x, i0, i1, i2, i3);
+        float *dp = (float *)at(y, i0, i1, i2, i3);
+        const float x0 = sp[0], x1 = sp[nd / 2], x2 = sp[nd], x3 = sp[nd / 2 + nd];
+        dp[0] = x0 * c - x1 * s;
+        dp[nd / 2] = x0 * s + x1 * c;
+        dp[nd] = x2 * cb - x3 * sb;
+        dp[nd / 2 + nd] = x2 * sb + x3 * cb;
+    }
+}
+
 extern "C" int spy_hip_op_rope(void *stream, const spy_hip_tensor *x, const spy_hip_tensor *pos, const spy_hip_tensor *dst, const spy_hip_rope_param *p) {
     SPY_CHECK_ARG(x && pos && dst && p && x->data && pos->data && dst->data);
     if (x->type != SPY_HIP_F32 || dst->type != SPY_HIP_F32 || pos->type != SPY_HIP_I32) return SPY_HIP_EUNSUPPORTED;
-    if (p->mode != 0 && p->mode != -1) return SPY_HIP_EUNSUPPORTED;          // GLM / Neox (Neox aborts in the reference too)
+    if (p->mode == 4) {                                                       // GLM
+        if (spy_exact_on()) return SPY_HIP_EUNSUPPORTED;                      // no host-libm table for this mode
+        SPY_CHECK_ARG(same_ne(x, dst) && x->nb[0] == 4 && dst->nb[0] == 4 && p->num_dim > 0 && p->num_dim % 2 == 0 && dst->ne[0] >= 4);
+        SPY_CHECK_ARG(pos->ne[0] >= dst->ne[2] && dst->ne[1] < 65536 && dst->ne[2] < 65536 && dst->ne[3] < 65536 && dst->ne[1] > 0 && dst->ne[2] > 0 && dst->ne[3] > 0);
+        // the four elements of the last i0 must lie inside the row (the reference does not check: it would read the next row); and an
+        // in-place call must not have one i0 write what another reads: true when the four index ranges do not overlap
+        SPY_CHECK_ARG(dst->ne[0] / 4 - 1 + p->num_dim / 2 + p->num_dim < dst->ne[0] && p->num_dim / 2 >= dst->ne[0] / 4);
+        const float ts = powf(p->freq_base, -2.0f / (float)p->num_dim);
+        rope_glm_kernel<<<dim3((unsigned)dst->ne[1], (unsigned)dst->ne[2], (unsigned)dst->ne[3]), dim3(64), 0, (hipStream_t)stream>>>(
+            mk(x), (const int32_t *)pos->data, pos->nb[0], mk(dst), ts, p->num_context, p->num_dim);
+        return SPY_LAUNCH_RC();
+    }
+    if (p->mode != 0 && p->mode != -1) return SPY_HIP_EUNSUPPORTED;          // Neox (aborts in the reference too)
     SPY_CHECK_ARG(same_ne(x, dst) && x->nb[0] == 4 && dst->nb[0] == 4 && dst->ne[0] % 2 == 0 && p->num_dim > 0);
     SPY_CHECK_ARG(pos->ne[0] >= dst->ne[2] && dst->ne[1] < 65536 && dst->ne[2] < (1ll << 31) && dst->ne[3] < 65536);
     SPY_CHECK_ARG(dst->ne[1] > 0 && dst->ne[2] > 0 && dst->ne[3] > 0);

@@ -128,7 +128,7 @@ def _bind(L):
         "spy_o_dot_q4_k_q8_0": (f32, [vp, vp, i64]), "spy_o_dot_q6_k_q8_0": (f32, [vp, vp, i64]),
         "spy_o_block_dots": (i32, [i32, vp, vp, i64, vp]), "spy_o_have_avx2": (i32, []),
         "spy_o_matmul": (i32, [TP, TP, TP, i32]), "spy_o_norm_rms": (i32, [TP, TP, f32]),
-        "spy_o_binary": (i32, [i32, TP, TP, TP]), "spy_o_silu": (i32, [TP, TP]),
+        "spy_o_binary": (i32, [i32, TP, TP, TP]), "spy_o_silu": (i32, [TP, TP]), "spy_o_relu": (i32, [TP, TP]), "spy_o_quantize": (i32, [TP, TP]),
         "spy_o_softmax": (i32, [TP, TP, TP, f32]), "spy_o_rope": (i32, [TP, TP, TP, C.POINTER(RopeParam)]),
         "spy_o_dup": (i32, [TP, TP]), "spy_o_contiguous": (i32, [TP, TP]), "spy_o_get_row": (i32, [TP, TP, TP]),
         "spy_o_argmax": (i32, [vp, i64]),

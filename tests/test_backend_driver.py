@@ -15,7 +15,7 @@ def test_driver_library_exports_header_symbols():
     from spy_amd import backend_driver as B
     text = open(os.path.join(ROOT, "include", "spy_backend_driver.h")).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    names = sorted(set(re.findall(r"\b(spy_host_model_[a-z0-9_]+)\s*\(", text)))
+    names = sorted(set(re.findall(r"\b(spy_host_[a-z0-9_]+)\s*\(", text)))
     L = B.load()
     assert names == sorted(B.SIGNATURES)
     for n in names:
@@ -181,3 +181,22 @@ def test_submit_path_k_quant_mix_with_outliers():
         assert_close(lh, l1, "K-quant mix decode step %d" % step, 3e-3)
         tok = int(np.argmax(l1))
     host.close()
+
+
+@pytest.mark.gpu
+def test_relu_silu_quantize_nodes_through_submit(oracle):
+    """The operators of the host backend's set that the LLaMA graph does not emit (Relu, Quantize; operator_impl.h:73,89 in
+    the Spy tree), each as one node through Backend::submit with IO operands, against the oracle."""
+    import ctypes as C
+    from spy_amd import backend_driver as BD
+    rng = np.random.default_rng(14)
+    x = (rng.standard_normal((7, 128)) * 2).astype(np.float32)
+    want = np.zeros_like(x)
+    assert oracle.spy_o_relu(C.byref(O.tensor(x, O.F32, [128, 7])), C.byref(O.tensor(want, O.F32, [128, 7]))) == 0
+    assert np.array_equal(BD.unary_through_submit("relu", x).view(np.uint32), want.view(np.uint32))
+    for ttype in (O.Q8_0, O.F16):
+        wq = np.zeros(7 * O.row_size(ttype, 128), np.uint8)
+        assert oracle.spy_o_quantize(C.byref(O.tensor(x, O.F32, [128, 7])), C.byref(O.tensor(wq, ttype, [128, 7]))) == 0
+        assert np.array_equal(BD.unary_through_submit("quantize", x, ttype), wq)
+    with pytest.raises(RuntimeError):                                       # F32 -> Q4_0: OperatorStatus::Unsupport
+        BD.unary_through_submit("quantize", x, O.Q4_0)

@@ -210,6 +210,31 @@ def test_fused_decode_real_widths_long_cache(order, n_ctx, positions):
     eng.close()
 
 
+def test_model_wider_than_4096_takes_the_tiled_kernels():
+    """n_embd = 5120 (the 13B width): the one-row-per-wave kernels stage 4096 activations per workgroup at most, so the fused
+    single-token pass of such a model runs the 256-thread tiled kernels, in this backend's own summation order (the kernels of
+    the host's order take n_embd <= 4096).  One layer against the oracle: per-pass bound, same greedy tokens both ways of
+    running the loop."""
+    from spy_amd import model as M
+    from tests.gpu_util import E2E_TOL
+    cfg = M.Config(n_layer=1, n_embd=5120, n_head=40, n_ff=13824, n_vocab=2048, n_ctx=64, wtype=O.Q4_0)
+    eng, ora, _ = _mk(cfg, seed=41)
+    assert eng.order() == 0
+    prompt = np.random.default_rng(3).integers(0, cfg.n_vocab, 6).astype(np.int32)
+    lg_g, lg_o = eng.forward(prompt, 0), ora.forward(prompt, 0)
+    _close(lg_g, lg_o, "prompt logits, n_embd 5120", E2E_TOL)
+    tok = int(np.argmax(lg_o[-1]))
+    for step in range(3):
+        t = np.array([tok], np.int32)
+        lg, lo = eng.forward(t, 6 + step)[0], ora.forward(t, 6 + step)[0]
+        _close(lg, lo, "single-token logits, n_embd 5120, step %d" % step, E2E_TOL)
+        tok = int(np.argmax(lo))
+    a = eng.decode_greedy(tok, 9, 4, use_graph=False)
+    b = eng.decode_greedy(tok, 9, 4, use_graph=True)
+    assert a.tolist() == b.tolist()
+    eng.close()
+
+
 @pytest.mark.parametrize("order", [1, 0])
 def test_engine_with_a_smaller_context_does_not_lower_the_lds_limit_of_a_larger_one(order):
     """A kernel's dynamic-LDS limit belongs to the kernel for the whole process.  An engine with a long context raises it

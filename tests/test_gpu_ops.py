@@ -92,38 +92,34 @@ def test_masked_softmax(hip, oracle):
 
 
 def test_softmax_row_kernel_and_fp16_output(hip, oracle):
-    """The kernel that keeps a row in LDS gives the bits of the three-pass kernel (same additions in the same
-    order), with and without a causal mask; the fp16 output is the fp32 output rounded to nearest even, which is
-    what the KQV product does to it first (mat.cpp:37 in the Spy tree)."""
-    import os
+    """Rows of up to 16384 elements take the kernel that keeps a row in LDS, longer rows the three-pass kernel; both against
+    the oracle, with and without a causal mask.  The fp16 output of the row kernel is its fp32 output rounded to nearest even,
+    which is what the KQV product does to it first (mat.cpp:37 in the Spy tree)."""
     from tests.gpu_util import dev, dev_empty, call
     rng = np.random.default_rng(12)
     scale = 0.0883883461356163
     L = hip.load()
-    for (H_, T, n_kv, Cx, P) in [(4, 24, 40, 64, 16), (2, 5, 1000, 1024, 995), (1, 3, 4104, 4352, 4101)]:
+    for (H_, T, n_kv, Cx, P) in [(4, 24, 40, 64, 16), (2, 5, 1000, 1024, 995), (1, 3, 4104, 4352, 4101), (1, 2, 16500, 16512, 16498)]:
         s = (rng.standard_normal((H_, T, n_kv)) * 4).astype(np.float32)
         mask = np.where(np.arange(Cx)[None, :] <= (np.arange(T)[:, None] + P), 0.0, -np.inf).astype(np.float32)
         ds, dm = dev(s), dev(mask.view(np.int32))
-        outs = {}
         for name, use_mask in (("masked", True), ("plain", False)):
             tm = B(hip.tensor(dm, hip.I32, [Cx, T])) if use_mask else None
-            os.environ["SPY_HIP_SOFTMAX_GENERIC"] = "1"
-            try:
-                dg = dev_empty(s.nbytes, 0xFF)
-                call(L.spy_hip_op_softmax, None, B(hip.tensor(ds, hip.F32, [n_kv, T, H_])), tm, B(hip.tensor(dg, hip.F32, [n_kv, T, H_])), scale)
-                hip.sync()
-            finally:
-                del os.environ["SPY_HIP_SOFTMAX_GENERIC"]
-            dr, dh = dev_empty(s.nbytes, 0xFF), dev_empty(s.nbytes // 2, 0xFF)
+            dr = dev_empty(s.nbytes, 0xFF)
             call(L.spy_hip_op_softmax, None, B(hip.tensor(ds, hip.F32, [n_kv, T, H_])), tm, B(hip.tensor(dr, hip.F32, [n_kv, T, H_])), scale)
-            call(L.spy_hip_op_softmax, None, B(hip.tensor(ds, hip.F32, [n_kv, T, H_])), tm, B(hip.tensor(dh, hip.F16, [n_kv, T, H_])), scale)
-            generic, row, half = dg.download(np.float32), dr.download(np.float32), dh.download(np.float16)
-            assert np.array_equal(generic.view(np.uint32), row.view(np.uint32)), (name, H_, T, n_kv)
-            assert np.array_equal(half.view(np.uint16), row.astype(np.float16).view(np.uint16)), (name, H_, T, n_kv)
-            outs[name] = row
-        want = np.zeros_like(s)
-        assert oracle.spy_o_softmax(B(O.tensor(s, O.F32, [n_kv, T, H_])), B(O.tensor(mask.view(np.int32), O.I32, [Cx, T])), B(O.tensor(want, O.F32, [n_kv, T, H_])), scale) == 0
-        assert float(np.abs(outs["masked"].reshape(want.shape) - want).max()) < 1e-5
+            row = dr.download(np.float32)
+            if n_kv <= 16384:
+                dh = dev_empty(s.nbytes // 2, 0xFF)
+                call(L.spy_hip_op_softmax, None, B(hip.tensor(ds, hip.F32, [n_kv, T, H_])), tm, B(hip.tensor(dh, hip.F16, [n_kv, T, H_])), scale)
+                assert np.array_equal(dh.download(np.float16).view(np.uint16), row.astype(np.float16).view(np.uint16)), (name, H_, T, n_kv)
+            else:       # the fp16 output is the row kernel's alone
+                dh = dev_empty(s.nbytes // 2, 0xFF)
+                assert L.spy_hip_op_softmax(None, B(hip.tensor(ds, hip.F32, [n_kv, T, H_])), tm, B(hip.tensor(dh, hip.F16, [n_kv, T, H_])), scale) == hip.EUNSUPPORTED
+            want = np.zeros_like(s)
+            om = B(O.tensor(mask.view(np.int32), O.I32, [Cx, T])) if use_mask else None
+            assert oracle.spy_o_softmax(B(O.tensor(s, O.F32, [n_kv, T, H_])), om, B(O.tensor(want, O.F32, [n_kv, T, H_])), scale) == 0
+            assert float(np.abs(row.reshape(want.shape) - want).max()) < 1e-5, (name, H_, T, n_kv)
+            assert np.array_equal(row.reshape(want.shape) == 0, want == 0)
 
 
 def test_rope(hip, oracle):
@@ -145,6 +141,58 @@ def test_rope(hip, oracle):
     hp.mode = 2
     assert hip.load().spy_hip_op_rope(None, B(hip.tensor(dx, hip.F32, [hd, H_, T])), B(hip.tensor(dp, hip.I32, [T])),
                                       B(hip.tensor(dy, hip.F32, [hd, H_, T])), B(hp)) == hip.EUNSUPPORTED
+
+
+def test_rope_glm(hip, oracle):
+    """Mode GLM (non-linear.cpp:315-343 in the Spy tree) as written: rows of 2 * num_dim elements, positions on both sides of
+    num_context - 2 (the second angle is 0 before it); in place as well; rows the four indices would leave are refused."""
+    from tests.gpu_util import dev, dev_empty, call, assert_close
+    rng = np.random.default_rng(6)
+    nd, H_, T, C_ = 64, 8, 6, 100
+    ne0 = 2 * nd
+    pos = np.array([0, 1, 50, 98, 99, 140], dtype=np.int32)
+    x = rng.standard_normal((T, H_, ne0)).astype(np.float32)
+    want = np.zeros_like(x)
+    rp = O.default_rope(nd, C_); rp.mode = 4
+    assert oracle.spy_o_rope(B(O.tensor(x, O.F32, [ne0, H_, T])), B(O.tensor(pos, O.I32, [T])), B(O.tensor(want, O.F32, [ne0, H_, T])), B(rp)) == 0
+    dx, dp, dy = dev(x), dev(pos), dev_empty(x.nbytes, 0xFF)
+    hp = hip.RopeParam(4, 0, nd, C_, C_, 10000.0, 1.0, 0.0, 1.0, 32.0, 1.0, 0.0, 0)
+    L = hip.load()
+    call(L.spy_hip_op_rope, None, B(hip.tensor(dx, hip.F32, [ne0, H_, T])), B(hip.tensor(dp, hip.I32, [T])), B(hip.tensor(dy, hip.F32, [ne0, H_, T])), B(hp))
+    got = dy.download(np.float32).reshape(x.shape)
+    assert_close(got, want, "rope GLM", tol=1e-5)
+    assert np.array_equal(got[0], x[0])                                     # position 0: both angles 0
+    call(L.spy_hip_op_rope, None, B(hip.tensor(dx, hip.F32, [ne0, H_, T])), B(hip.tensor(dp, hip.I32, [T])), B(hip.tensor(dx, hip.F32, [ne0, H_, T])), B(hp))   # in place
+    assert np.array_equal(dx.download(np.float32).reshape(x.shape).view(np.uint32), got.view(np.uint32))
+    hp.num_dim = ne0                                                        # i0 + 3 num_dim / 2 would leave the row
+    assert L.spy_hip_op_rope(None, B(hip.tensor(dx, hip.F32, [ne0, H_, T])), B(hip.tensor(dp, hip.I32, [T])), B(hip.tensor(dy, hip.F32, [ne0, H_, T])), B(hp)) == hip.EINVAL
+
+
+def test_relu_and_quantize_operators(hip, oracle):
+    """Relu (non-linear.cpp:16-50) and Quantize (backend/host/operator/quantize.cpp:18-41) of the host backend's operator
+    set: exact results; the conversions the reference cannot do right are refused."""
+    from tests.gpu_util import dev, dev_empty, call
+    rng = np.random.default_rng(8)
+    L = hip.load()
+    x = (rng.standard_normal((3, 5, 256)) * 3).astype(np.float32)
+    x[0, 0, :4] = [0.0, -0.0, np.inf, -np.inf]
+    dx, dy = dev(x), dev_empty(x.nbytes, 0xFF)
+    call(L.spy_hip_op_relu, None, B(hip.tensor(dx, hip.F32, [256, 5, 3])), B(hip.tensor(dy, hip.F32, [256, 5, 3])))
+    want = np.zeros_like(x)
+    assert oracle.spy_o_relu(B(O.tensor(x, O.F32, [256, 5, 3])), B(O.tensor(want, O.F32, [256, 5, 3]))) == 0
+    assert np.array_equal(dy.download(np.float32).view(np.uint32), want.reshape(-1).view(np.uint32))
+    assert np.array_equal(want, np.where(x < 0, np.float32(0), x))
+    x[0, 0, 2:4] = [7.5, -7.5]                                              # finite values for the quantizers (an infinite block scale has no defined quants)
+    dx = dev(x)
+    for ttype in (O.Q8_0, O.F16):
+        nbytes = 15 * O.row_size(ttype, 256)
+        dq = dev_empty(nbytes, 0xFF)
+        call(L.spy_hip_op_quantize, None, B(hip.tensor(dx, hip.F32, [256, 5, 3])), B(hip.tensor(dq, ttype, [256, 5, 3])))
+        wq = np.zeros(nbytes, np.uint8)
+        assert oracle.spy_o_quantize(B(O.tensor(x, O.F32, [256, 5, 3])), B(O.tensor(wq, ttype, [256, 5, 3]))) == 0
+        assert np.array_equal(dq.download(np.uint8), wq), ttype
+    dq = dev_empty(15 * O.row_size(O.Q4_0, 256), 0)
+    assert L.spy_hip_op_quantize(None, B(hip.tensor(dx, hip.F32, [256, 5, 3])), B(hip.tensor(dq, hip.Q4_0, [256, 5, 3]))) == hip.EUNSUPPORTED
 
 
 @pytest.mark.parametrize("name,kw", [

@@ -179,6 +179,55 @@ def test_rope(oracle):
                              C.byref(O.tensor(y, O.F32, [hd, H, T])), C.byref(O.RopeParam(2, 0, hd, 64, 64, 1e4, 1, 0, 1, 32, 1, 0, 0))) == 1
 
 
+def test_rope_glm_closed_form(oracle):
+    """Mode GLM (non-linear.cpp:315-343 in the Spy tree) against its definition in float64: for i0 < ne0 / 4 the elements
+    (i0, i0 + nd / 2) turn by min(p, C - 2) * base^(-2 i0 / nd) and the elements (i0 + nd, i0 + 3 nd / 2) by
+    max(p - (C - 2), 0) * base^(-2 i0 / nd); pair norms are kept, position 0 is the identity, and below C - 2 the second
+    pair does not move."""
+    rng = np.random.default_rng(26)
+    nd, H, T, Cx = 64, 3, 6, 100
+    ne0 = 2 * nd
+    pos = np.array([0, 1, 50, 98, 99, 140], dtype=np.int32)
+    x = rng.standard_normal((T, H, ne0)).astype(np.float32)
+    y = np.zeros_like(x)
+    rp = O.default_rope(nd, Cx); rp.mode = 4
+    assert oracle.spy_o_rope(C.byref(O.tensor(x, O.F32, [ne0, H, T])), C.byref(O.tensor(pos, O.I32, [T])),
+                             C.byref(O.tensor(y, O.F32, [ne0, H, T])), C.byref(rp)) == 0
+    i0 = np.arange(ne0 // 4, dtype=np.float64)
+    sc = 10000.0 ** (-2.0 * i0 / nd)
+    ta = np.minimum(pos, Cx - 2)[:, None].astype(np.float64) * sc[None, :]
+    tb = np.maximum(pos - (Cx - 2), 0)[:, None].astype(np.float64) * sc[None, :]
+    xd = x.astype(np.float64)
+    want = xd.copy()
+    q = ne0 // 4
+    for (a, b, th) in ((0, nd // 2, ta), (nd, nd // 2 + nd, tb)):
+        c, s_ = np.cos(th)[:, None, :], np.sin(th)[:, None, :]
+        xa, xb = xd[..., a:a + q], xd[..., b:b + q]
+        want[..., a:a + q] = xa * c - xb * s_
+        want[..., b:b + q] = xa * s_ + xb * c
+    assert np.abs(y - want).max() < 140 * 64 * 2.0 ** -24 * np.abs(x).max() * 2 + 1e-6
+    assert np.array_equal(y[0], x[0])
+    assert np.array_equal(y[2][:, nd:], x[2][:, nd:])                        # p = 50 < C - 2: the second angle is 0
+    n_in = xd[..., :q] ** 2 + xd[..., nd // 2:nd // 2 + q] ** 2
+    n_out = y[..., :q].astype(np.float64) ** 2 + y[..., nd // 2:nd // 2 + q].astype(np.float64) ** 2
+    assert np.allclose(n_in, n_out, rtol=1e-5)
+
+
+def test_relu_and_quantize_operators(oracle):
+    rng = np.random.default_rng(27)
+    x = (rng.standard_normal((2, 3, 64)) * 2).astype(np.float32)
+    y = np.zeros_like(x)
+    assert oracle.spy_o_relu(C.byref(O.tensor(x, O.F32, [64, 3, 2])), C.byref(O.tensor(y, O.F32, [64, 3, 2]))) == 0
+    assert np.array_equal(y, np.maximum(x, 0))
+    q = np.zeros(6 * 68, np.uint8)
+    assert oracle.spy_o_quantize(C.byref(O.tensor(x, O.F32, [64, 3, 2])), C.byref(O.tensor(q, O.Q8_0, [64, 3, 2]))) == 0
+    assert np.array_equal(q, O.quantize(oracle, x, O.Q8_0))                   # the operator = the row quantizer, row after row
+    h = np.zeros(6 * 128, np.uint8)
+    assert oracle.spy_o_quantize(C.byref(O.tensor(x, O.F32, [64, 3, 2])), C.byref(O.tensor(h, O.F16, [64, 3, 2]))) == 0
+    assert np.array_equal(h.view(np.float16), x.astype(np.float16).reshape(-1))
+    assert oracle.spy_o_quantize(C.byref(O.tensor(x, O.F32, [64, 3, 2])), C.byref(O.tensor(q, O.Q4_0, [64, 3, 2]))) == 1
+
+
 def test_rope_yarn_and_xpos_reduce_to_known_forms(oracle):
     """Pins for the two extensions of the default Rope branch.  (1) extend_factor != 0 (rope_yarn, non-linear.cpp:247-260): the
     ramp is 1 - std::clamp(0.0F, 1.0F, y), which clamps the value 0 into [1, y] and so is 0, leaving only
