@@ -245,7 +245,7 @@ def main():
         ops_set = 2.0 * Tg * (4 * d_ * d_ + 3 * d_ * F_)
         tops = ops_set / us_set / 1e6
         gemm_roofline = {"summation_order": 0,
-                         "kernel": "gemm_q8act_kernel, the prompt GEMM of summation order 0 (NOT what the headline order's prompt runs: see prompt_gemm_roofline_order1): quantized GEMMs of one layer (%s weights x Q8_0 activations, int8 MFMA, per-block scales): 4 x %dx%d, 2 x %dx%d, 1 x %dx%d, %d activation rows"
+                         "kernel": "gemm_q8act_kernel, the prompt GEMM of summation order 0 (NOT what the headline order's prompt runs: that is prompt_gemm_roofline): quantized GEMMs of one layer (%s weights x Q8_0 activations, int8 MFMA, per-block scales): 4 x %dx%d, 2 x %dx%d, 1 x %dx%d, %d activation rows"
                                    % ({H.Q4_0: "Q4_0", H.Q8_0: "Q8_0", H.Q4_K: "Q4_K", H.Q6_K: "Q6_K"}[wt_g], d_, d_, F_, d_, d_, F_, Tg),
                          "bound": "mfma", "achieved": round(tops, 1), "peak": INT8_PEAK / 1e12, "unit": "TOP/s", "frac": round(tops * 1e12 / INT8_PEAK, 4),
                          "ops_per_set": ops_set, "us_per_set": round(us_set, 1)}

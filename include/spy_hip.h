@@ -216,7 +216,7 @@ int spy_hip_block_dots(void *stream, int wtype, const void *w, const void *xq, i
 
 /* ---- the kernel families of the fused single-token pass, one launch at a time.  Each runs exactly the launch the token
  *      loop below uses for that part of a layer (same kernel, same grid), on the caller's buffers; order = 1: the host
- *      backend's summation order (results equal to the CPU backend's bit for bit), 0: this backend's own.  K (and F) must be
+ *      backend's summation order (results equal, bit for bit, to the host backend's compiled without fp contraction), 0: this backend's own.  K (and F) must be
  *      multiples of 128 for order 1, rows at most 4096 elements wide for the norm prologue (16384 for the plain one). ------- */
 /* The running sum that NormRMS and Softmax of the host backend take over their terms: libstdc++'s std::reduce /
  * std::transform_reduce for random-access ranges (non-linear.cpp:165-168, 205-208) adds groups of four,
@@ -319,7 +319,8 @@ int spy_hip_llama_decode_greedy(spy_hip_llama *m, void *stream, int32_t first_to
  * n_embd and n_ff multiples of 128): the host backend's -- the eight accumulators and hsum_float_8 of its quantized dots,
  * the 4 x 8 accumulators, tree and scalar tail of its fp16 dots (vec_dot.h:42-146), libstdc++'s four-way reduce in
  * NormRMS and Softmax (non-linear.cpp:129-223), exp / silu from the fp16-indexed tables and the RoPE angles from the
- * host's libm -- so that logits and greedy tokens equal the CPU backend's bit for bit.  0: this backend's own order
+ * host's libm -- so that logits and greedy tokens equal, bit for bit, those of the host backend compiled without fp contraction (a
+ * build with -ffp-contract=fast fuses x * x + y in NormRMS and differs in last bits).  0: this backend's own order
  * (lane-parallel sums; per-operator results equal to about 1e-7, greedy tokens of a model with near-tied logits may
  * differ).  The environment variable SPY_HIP_ORDER=own at creation selects 0.  spy_hip_set_exact_order(1) forces 1 for
  * every engine while it is on.  spy_hip_llama_order returns the order the next single-token pass will use. */
