@@ -1,8 +1,8 @@
 // SentencePiece tokenizer over the vocabulary of a GGUF file (see include/spy_vocab.h for what it follows).
 #include "../../include/spy_vocab.h"
 
+#include <algorithm>
 #include <cstring>
-#include <queue>
 #include <string>
 #include <string_view>
 #include <unordered_map>
@@ -43,71 +43,87 @@ struct spy_vocab {
 
 namespace {
 
-struct Symbol { int prev, next; const char *text; size_t n; };
-struct Bigram { int left, right; float score; size_t size; };
-struct BigramLess {                                       // priority: higher score first, then the leftmost pair (:27-30)
-    bool operator()(const Bigram &a, const Bigram &b) const { return a.score < b.score || (a.score == b.score && a.left > b.left); }
-};
+// Greedy pair merging over the characters of one text (the SentencePiece scheme of sentence_piece_vocab.h:120-211): the text is
+// a chain of pieces, at first one per UTF-8 character; the best-scoring adjacent pair that is a vocabulary entry is joined, and
+// so on until no adjacent pair is an entry.  Pieces are kept as parallel arrays indexed by their position in the first chain;
+// a piece of length 0 has been absorbed by its left neighbour.
+struct Candidate { float score; int lhs, rhs; size_t joined; };   // joined: byte length of the pair when it was proposed
+// heap order: the higher score wins, among equal scores the pair further left (:27-30)
+inline bool worse(const Candidate &a, const Candidate &b) { return a.score < b.score || (a.score == b.score && a.lhs > b.lhs); }
 
-struct Session {
-    const spy_vocab &v;
-    std::vector<Symbol> symbols;
-    std::priority_queue<Bigram, std::vector<Bigram>, BigramLess> queue;
-    std::unordered_map<std::string, std::pair<int, int>> rev_merge;
-    bool failed = false;
+class Merger {
+public:
+    explicit Merger(const spy_vocab &vocab) : v_(vocab) {}
+    bool failed() const { return failed_; }
 
-    void try_add_bigram(int left, int right) {
-        if (left == -1 || right == -1) return;
-        const std::string_view text(symbols[left].text, symbols[left].n + symbols[right].n);
-        const int32_t id = v.find(text);
-        if (id < 0) return;
-        queue.push(Bigram{left, right, v.tokens[id].score, text.size()});
-        rev_merge[std::string(text)] = {left, right};
+    void tokenize(const std::string &text, std::vector<int32_t> &out) {
+        split_characters(text);
+        const int n = (int)len_.size();
+        if (n == 0) return;
+        for (int i = 0; i + 1 < n; i++) propose(i, i + 1);
+        while (!heap_.empty()) {
+            std::pop_heap(heap_.begin(), heap_.end(), worse);
+            const Candidate c = heap_.back();
+            heap_.pop_back();
+            // stale when either side was absorbed or grew since the proposal
+            if (len_[c.lhs] == 0 || len_[c.rhs] == 0 || len_[c.lhs] + len_[c.rhs] != c.joined) continue;
+            len_[c.lhs] = c.joined;
+            len_[c.rhs] = 0;
+            const int after = after_[c.rhs];
+            after_[c.lhs] = after;
+            if (after >= 0) before_[after] = c.lhs;
+            propose(before_[c.lhs], c.lhs);
+            propose(c.lhs, after);
+        }
+        for (int i = 0; i >= 0; i = after_[i]) emit(i, out);
     }
-    void resegment(const Symbol &s, std::vector<int32_t> &out) {
-        const std::string_view text(s.text, s.n);
-        const int32_t id = v.find(text);
-        if (id >= 0) { out.push_back(id); return; }
-        const auto p = rev_merge.find(std::string(text));
-        if (p == rev_merge.end()) {                       // no token and no merge: spell the bytes
-            for (size_t j = 0; j < s.n; j++) {
-                const int32_t b = v.byte_token((uint8_t)s.text[j]);
-                if (b < 0) { failed = true; return; }
+
+private:
+    const spy_vocab &v_;
+    std::vector<const char *> at_;
+    std::vector<size_t> len_;
+    std::vector<int> before_, after_;
+    std::vector<Candidate> heap_;
+    // every pair ever proposed, by its joined text: how a piece that is no entry itself is taken apart again (:181-211)
+    std::unordered_map<std::string, std::pair<int, int>> halves_;
+    bool failed_ = false;
+
+    void split_characters(const std::string &text) {
+        for (size_t o = 0; o < text.size();) {
+            const size_t n = std::min(utf8_len(text[o]), text.size() - o);
+            at_.push_back(text.data() + o);
+            len_.push_back(n);
+            before_.push_back((int)len_.size() - 2);
+            o += n;
+            after_.push_back(o < text.size() ? (int)len_.size() : -1);
+        }
+    }
+    void propose(int lhs, int rhs) {
+        if (lhs < 0 || rhs < 0) return;
+        const std::string_view joined(at_[lhs], len_[lhs] + len_[rhs]);
+        const int32_t id = v_.find(joined);
+        if (id < 0) return;
+        heap_.push_back(Candidate{v_.tokens[id].score, lhs, rhs, joined.size()});
+        std::push_heap(heap_.begin(), heap_.end(), worse);
+        halves_[std::string(joined)] = {lhs, rhs};
+    }
+    // a piece's ids: its own entry, else the ids of the two pieces it was joined from, else its bytes (explicit stack, right half pushed first)
+    void emit(int piece, std::vector<int32_t> &out) {
+        std::vector<int> todo(1, piece);
+        while (!todo.empty()) {
+            const int p = todo.back();
+            todo.pop_back();
+            const std::string_view text(at_[p], len_[p]);
+            const int32_t id = v_.find(text);
+            if (id >= 0) { out.push_back(id); continue; }
+            const auto h = halves_.find(std::string(text));
+            if (h != halves_.end()) { todo.push_back(h->second.second); todo.push_back(h->second.first); continue; }
+            for (const char ch : text) {
+                const int32_t b = v_.byte_token((uint8_t)ch);
+                if (b < 0) { failed_ = true; return; }
                 out.push_back(b);
             }
-            return;
         }
-        resegment(symbols[p->second.first], out);
-        resegment(symbols[p->second.second], out);
-    }
-    void run(const std::string &text, std::vector<int32_t> &out) {
-        int index = 0;
-        size_t offs = 0;
-        while (offs < text.size()) {                      // one symbol per UTF-8 character
-            Symbol s;
-            s.text = text.data() + offs;
-            s.n = std::min(utf8_len(text[offs]), text.size() - offs);
-            offs += s.n;
-            s.prev = index - 1;
-            s.next = offs == text.size() ? -1 : index + 1;
-            index++;
-            symbols.push_back(s);
-        }
-        for (size_t i = 1; i < symbols.size(); i++) try_add_bigram((int)i - 1, (int)i);
-        while (!queue.empty()) {
-            const Bigram b = queue.top();
-            queue.pop();
-            Symbol &l = symbols[b.left], &r = symbols[b.right];
-            if (l.n == 0 || r.n == 0 || l.n + r.n != b.size) continue;     // one of them was merged meanwhile
-            l.n += r.n;
-            r.n = 0;
-            l.next = r.next;
-            if (r.next >= 0) symbols[r.next].prev = b.left;
-            try_add_bigram(l.prev, b.left);
-            try_add_bigram(b.left, l.next);
-        }
-        if (symbols.empty()) return;
-        for (int i = 0; i != -1; i = symbols[i].next) resegment(symbols[i], out);
     }
 };
 
@@ -194,9 +210,9 @@ extern "C" int64_t spy_vocab_tokenize(const spy_vocab *v, const char *text, uint
         s.reserve(len * 3 + 3);
         if (v->add_space_prefix) s += ESC;
         for (uint64_t i = 0; i < len; i++) { if (text[i] == ' ') s += ESC; else s += text[i]; }
-        Session session{*v, {}, {}, {}, false};
-        session.run(s, out);
-        if (session.failed) return spy_gguf_fail(SPY_GGUF_EKEY, "a character of the text has neither a token nor a byte token in this vocabulary");
+        Merger merger(*v);
+        merger.tokenize(s, out);
+        if (merger.failed()) return spy_gguf_fail(SPY_GGUF_EKEY, "a character of the text has neither a token nor a byte token in this vocabulary");
     }
     for (uint64_t i = 0; i < out.size() && i < cap; i++) ids[i] = out[i];
     return (int64_t)out.size();
