@@ -85,6 +85,12 @@ int spy_enqueue_exact_q4_0(spy_hip_llama *m, hipStream_t st, int which, int il);
 int spy_enqueue_exact_q8_0(spy_hip_llama *m, hipStream_t st, int which, int il);
 int spy_enqueue_exact_q4_k(spy_hip_llama *m, hipStream_t st, int which, int il);
 int spy_enqueue_exact_q6_k(spy_hip_llama *m, hipStream_t st, int which, int il);
+// out[0..M) = rows of w (M x K, type of the name) . x (K floats, 16-byte aligned) in the host backend's order, one launch, no engine:
+// SPY_HIP_EUNSUPPORTED for lengths the kernel does not take (K % 128, K-quants K % 256; K <= 16384, K-quants 12288)
+int spy_exact_matvec_q4_0(hipStream_t st, const void *w, const float *x, float *out, int M, int K);
+int spy_exact_matvec_q8_0(hipStream_t st, const void *w, const float *x, float *out, int M, int K);
+int spy_exact_matvec_q4_k(hipStream_t st, const void *w, const float *x, float *out, int M, int K);
+int spy_exact_matvec_q6_k(hipStream_t st, const void *w, const float *x, float *out, int M, int K);
 // probe: only check that the fused attention launch for this layer's types exists and that all its workgroups are resident
 int spy_probe_attn_layer_q4_0(spy_hip_llama *m, int il);
 int spy_probe_attn_layer_q8_0(spy_hip_llama *m, int il);

@@ -555,7 +555,7 @@ __global__ __launch_bounds__(XG_THREADS) void xgemv_kernel(xg_args a) {
         const int ogw = (int)blockIdx.x * XG_WAVES + ow;
         if constexpr (EPI == EPI_RESID || EPI == EPI_STORE) {
             const int u = (ogw + step * NW) * RPS + oj;
-            if (owner && u < a.M) a.out[u] = EPI == EPI_RESID ? acc + a.resid[u] : acc;       // Add(KQV_linear, x) / Add(ffn_out, ffn_input)
+            if (owner && u < a.M) a.out[u] = (EPI == EPI_RESID && a.resid) ? acc + a.resid[u] : acc;       // Add(KQV_linear, x) / Add(ffn_out, ffn_input); no resid: the MatMul alone
         } else if constexpr (EPI == EPI_GATEUP) {
             const float up = __shfl_xor(acc, nch, SPY_WAVE);                   // the row after (up_i) sits nch lanes further
             const int i = ogw + step * NW;

@@ -41,6 +41,35 @@ static int xg_resid(spy_hip_llama *m, hipStream_t st, const xg_args &a) {
     }
 }
 
+// MatMul of ONE f32 activation row (the operator path's single-token products) through the same two-phase kernel: the row is
+// quantized to Q8_0 in LDS as Quantizator<FP32,Q8_0> does, the dots are Dot<W,Q8_0>::exec per row, nothing is added to them.
+// No engine behind the call: the LDS limit goes straight to the process-wide record.
+template <int WT, int NITK>
+static int launch_xg_plain(hipStream_t st, const xg_args &a) {
+    constexpr int NCH = xg_traits<WT>::NCH;
+    const size_t lds = ((staged_bytes(a.K) + 15) & ~(size_t)15) + (size_t)XG_WAVES * xg_slot_floats(NCH) * 4;
+    if (lds > 160 * 1024) return SPY_HIP_EUNSUPPORTED;
+    auto kern = xgemv_kernel<WT, NITK, 1, 1, EPI_RESID, WT>;
+    RC_TRY(spy_raise_lds_limit((const void *)kern, lds));
+    kern<<<dim3((unsigned)((a.M + XG_WAVES - 1) / XG_WAVES)), dim3(XG_THREADS), lds, st>>>(a);
+    return SPY_LAUNCH_RC();
+}
+template <int WT>
+static int xg_plain(hipStream_t st, const void *w, const float *x, float *out, int M, int K) {
+    constexpr bool KQ = WT == SPY_HIP_Q4_K || WT == SPY_HIP_Q6_K;
+    if (M <= 0 || K <= 0 || K % (KQ ? 256 : 128) != 0) return SPY_HIP_EUNSUPPORTED;
+    xg_args a;
+    memset(&a, 0, sizeof(a));
+    a.W0 = (const uint8_t *)w; a.M = M; a.K = K; a.x_in = x; a.out = out;
+    switch ((K + 4095) / 4096) {
+    case 1: return launch_xg_plain<WT, 1>(st, a);
+    case 2: return launch_xg_plain<WT, 2>(st, a);
+    case 3: return launch_xg_plain<WT, 3>(st, a);
+    case 4: if constexpr (!KQ) return launch_xg_plain<WT, 4>(st, a); else return SPY_HIP_EUNSUPPORTED;
+    default: return SPY_HIP_EUNSUPPORTED;
+    }
+}
+
 // one exact-order kernel of layer il (which: K_QKV, K_WO, K_GATEUP, K_DOWN) or the head (K_HEAD); WT = type of the kernel's (first) matrix
 template <int WT>
 static int enqueue_exact(spy_hip_llama *m, hipStream_t st, int which, int il) {

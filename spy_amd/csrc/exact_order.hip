@@ -1191,6 +1191,27 @@ size_t spy_exact_pack_bytes(int64_t ne01, int64_t ne00, int64_t ne11) {
     const int64_t tiles = (ne01 + XGB_TILE - 1) / XGB_TILE + (ne11 + XGB_TILE - 1) / XGB_TILE;
     return (size_t)(tiles * nb * (8 * XGB_TILE * 8 + XGB_TILE * 4));       // quants and scales: multiples of 256 bytes each
 }
+// MatMul of one f32 activation row with a quantized matrix: the two-phase kernel of the fused single-token pass (exact_decode.cuh),
+// which quantizes the row in LDS and walks every row's accumulators in the host's order -- one launch instead of a quantization
+// and one of the lane kernels below, at the bandwidth of the fused pass.  SPY_HIP_EUNSUPPORTED where it does not apply (lengths,
+// alignment, or the test switches that select the lane / serial kernels): the caller then takes the general way.
+int spy_exact_matvec_q4_0(hipStream_t st, const void *w, const float *x, float *out, int M, int K);
+int spy_exact_matvec_q8_0(hipStream_t st, const void *w, const float *x, float *out, int M, int K);
+int spy_exact_matvec_q4_k(hipStream_t st, const void *w, const float *x, float *out, int M, int K);
+int spy_exact_matvec_q6_k(hipStream_t st, const void *w, const float *x, float *out, int M, int K);
+int spy_exact_matvec(hipStream_t st, int t0, const void *w, const float *x, float *out, int64_t M, int64_t K) {
+    if (getenv("SPY_HIP_EXACT_SERIAL")) return SPY_HIP_EUNSUPPORTED;
+    const char *env_tiled = getenv("SPY_HIP_EXACT_TILED");
+    if (env_tiled && *env_tiled == '0') return SPY_HIP_EUNSUPPORTED;
+    if (M <= 0 || M >= (1ll << 30) || K <= 0 || K > 16384 || ((uintptr_t)w & 3) != 0 || ((uintptr_t)x & 15) != 0 || ((uintptr_t)out & 3) != 0) return SPY_HIP_EUNSUPPORTED;
+    switch (t0) {
+    case SPY_HIP_Q4_0: return spy_exact_matvec_q4_0(st, w, x, out, (int)M, (int)K);
+    case SPY_HIP_Q8_0: return spy_exact_matvec_q8_0(st, w, x, out, (int)M, (int)K);
+    case SPY_HIP_Q4_K: return ((uintptr_t)w & 15) == 0 ? spy_exact_matvec_q4_k(st, w, x, out, (int)M, (int)K) : SPY_HIP_EUNSUPPORTED;
+    case SPY_HIP_Q6_K: return spy_exact_matvec_q6_k(st, w, x, out, (int)M, (int)K);
+    default: return SPY_HIP_EUNSUPPORTED;
+    }
+}
 // pack, pack_bytes: workspace for the packed operands (may be null / short: the tile kernel then unpacks per tile)
 int spy_exact_dots(hipStream_t st, int t0, const spy_hip_tensor *w, const uint8_t *xm, int64_t x_row, int64_t ne11, const spy_hip_tensor *dst, int x_own_quants,
                    void *pack, size_t pack_bytes) {

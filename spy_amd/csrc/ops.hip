@@ -15,6 +15,7 @@ int spy_exact_norm_rms(hipStream_t st, const spy_hip_tensor *x, const spy_hip_te
 int spy_exact_silu(hipStream_t st, const spy_hip_tensor *x, const spy_hip_tensor *dst);
 int spy_exact_softmax(hipStream_t st, const spy_hip_tensor *x, const spy_hip_tensor *mask, const spy_hip_tensor *dst, float scale);
 int spy_exact_rope(hipStream_t st, const spy_hip_tensor *x, const spy_hip_tensor *pos, const spy_hip_tensor *dst, const spy_hip_rope_param *p);
+int spy_exact_matvec(hipStream_t st, int t0, const void *w, const float *x, float *out, int64_t M, int64_t K);
 int spy_exact_dots(hipStream_t st, int t0, const spy_hip_tensor *w, const uint8_t *xm, int64_t x_row, int64_t ne11, const spy_hip_tensor *dst, int x_own_quants,
                    void *pack, size_t pack_bytes);
 size_t spy_exact_pack_bytes(int64_t ne01, int64_t ne00, int64_t ne11);
@@ -633,6 +634,15 @@ __global__ __launch_bounds__(256) void to_f16_batched_kernel(const uint8_t *__re
     *(uint2 *)(y + (b * ne11 + row) * ne10 + c * 4) = o;
 }
 
+// the same for any row length and alignment (4-byte aligned floats): one element per thread
+__global__ __launch_bounds__(256) void to_f16_batched_scalar_kernel(const uint8_t *__restrict__ x, int64_t nb1, int64_t nb2, int64_t nb3,
+                                                                     uint16_t *__restrict__ y, int64_t ne10, int64_t ne11, int64_t ne12) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= ne10 * ne11) return;
+    const int64_t row = i / ne10, c = i - row * ne10, b = blockIdx.y, i12 = b % ne12, i13 = b / ne12;
+    y[(b * ne11 + row) * ne10 + c] = f2h(*(const float *)(x + i13 * nb3 + i12 * nb2 + row * nb1 + c * 4));
+}
+
 // bytes of the converted activations: the part of the scratch buffer that MatMul cannot do without
 static size_t matmul_act_bytes(const spy_hip_tensor *w, const spy_hip_tensor *x) {
     if (!w || !x) return 0;
@@ -682,6 +692,13 @@ static int matmul_impl(void *stream, const spy_hip_tensor *w, const spy_hip_tens
     SPY_CHECK_ARG(ne00 % spy_block_size(t0) == 0 && ne00 % spy_block_size(tm) == 0);
     hipStream_t st = (hipStream_t)stream;
 
+    // a single f32 row against a quantized matrix in the host's summation order: one launch that quantizes the row itself
+    if (quant && t1 == SPY_HIP_F32 && ne11 == 1 && ne12 == 1 && ne13 == 1 && skip_past < 0 && klimit_past < 0 && spy_exact_on() && x->nb[0] == 4 &&
+        w->nb[0] == spy_type_size(t0) && w->nb[1] == spy_row_size(t0, ne00)) {
+        const int rc = spy_exact_matvec(st, t0, w->data, (const float *)x->data, (float *)dst->data, ne01, ne00);
+        if (rc != SPY_HIP_EUNSUPPORTED) return rc;
+    }
+
     // 1. activations -> mid type, contiguous [ne10, ne11, ne12, ne13] in scratch (mat.cpp:95-128)
     const uint8_t *xm = (const uint8_t *)x->data;
     const int64_t mid_row = spy_row_size(tm, ne10);
@@ -693,6 +710,12 @@ static int matmul_impl(void *stream, const spy_hip_tensor *w, const spy_hip_tens
             x->nb[3] % 16 == 0 && ((uintptr_t)x->data & 15) == 0 && ne10 * ne11 / 4 < (1ll << 31) * 256) {
             // all batches (heads) in one launch
             to_f16_batched_kernel<<<dim3((unsigned)((ne10 / 4 * ne11 + 255) / 256), (unsigned)(ne12 * ne13)), dim3(256), 0, st>>>(
+                (const uint8_t *)x->data, x->nb[1], x->nb[2], x->nb[3], (uint16_t *)scratch, ne10, ne11, ne12);
+            if (hipGetLastError() != hipSuccess) return SPY_HIP_EINVAL;
+        } else if (tm == SPY_HIP_F16 && ne12 * ne13 > 1 && ne12 * ne13 <= 65535 && x->nb[1] % 4 == 0 && x->nb[2] % 4 == 0 && x->nb[3] % 4 == 0 &&
+                   ((uintptr_t)x->data & 3) == 0 && (ne10 * ne11 + 255) / 256 < (1ll << 31)) {
+            // all batches in one launch, element by element (a single token's probabilities: n_kv is a multiple of 4 one time in four)
+            to_f16_batched_scalar_kernel<<<dim3((unsigned)((ne10 * ne11 + 255) / 256), (unsigned)(ne12 * ne13)), dim3(256), 0, st>>>(
                 (const uint8_t *)x->data, x->nb[1], x->nb[2], x->nb[3], (uint16_t *)scratch, ne10, ne11, ne12);
             if (hipGetLastError() != hipSuccess) return SPY_HIP_EINVAL;
         } else

@@ -58,6 +58,40 @@ def test_quantized_matmul_bits(hip, oracle, wtype, M, K, T, serial, monkeypatch)
 
 
 @pytest.mark.parametrize("wtype", [O.Q4_0, O.Q8_0, O.Q4_K, O.Q6_K])
+@pytest.mark.parametrize("M,K", [(100, 4096), (4096, 4096), (37, 128), (33, 256), (50, 8192), (21, 11008), (19, 16384)])
+def test_single_row_matmul_takes_the_two_phase_kernel(hip, oracle, wtype, M, K, monkeypatch):
+    """One f32 activation row against a quantized matrix (every MatMul of a single-token pass through Backend::submit) runs as ONE
+    launch of the fused pass's two-phase kernel, which quantizes the row itself: the oracle's bits, and the bits of the lane
+    kernels behind SPY_HIP_EXACT_TILED=0, for row counts that are no multiple of the 16 rows of a workgroup and for one to
+    four slabs of K."""
+    from tests.gpu_util import dev, dev_empty, call
+    kq = wtype in (O.Q4_K, O.Q6_K)
+    if kq and (K % 256 or K > 12288):
+        pytest.skip("K-quant rows: whole super-blocks, at most three slabs")
+    rng = np.random.default_rng(31 * wtype + M + K)
+    w = O.quantize(oracle, (rng.standard_normal((M, K)) * 0.02).astype(np.float32), wtype)
+    x = (rng.standard_normal((1, K)) * 3.0).astype(np.float32)
+    x[0, 5] = 0.0
+    x[0, 64:96] = 0.0                                                   # a block of zeros: scale 0
+    want = O.matmul(oracle, w, wtype, M, K, x, nthread=4)
+    dw, dx = dev(w), dev(x)
+    tw, tx = hip.tensor(dw, wtype, [K, M]), hip.tensor(dx, hip.F32, [K, 1])
+    L = hip.load()
+    need = L.spy_hip_op_matmul_scratch_size(B(tw), B(tx))
+    scratch = dev_empty(need, 0xEE)
+    for tiled in ("1", "0"):
+        monkeypatch.setenv("SPY_HIP_EXACT_TILED", tiled)
+        dd = dev_empty(M * 4 + 64, 0xFF)
+        call(L.spy_hip_op_matmul, None, B(tw), B(tx), B(hip.tensor(dd, hip.F32, [M, 1])), scratch.ptr, need)
+        got = dd.download(np.float32)
+        _same_bits(got[:M].reshape(1, M), want, "single-row matmul type %d %dx%d, SPY_HIP_EXACT_TILED=%s" % (wtype, M, K, tiled))
+        assert (got[M:].view(np.uint32) == 0xFFFFFFFF).all(), "nothing is written beyond the M outputs"
+        if tiled == "1":
+            # the one-launch route leaves the scratch buffer alone (the row is quantized in LDS)
+            assert (scratch.download(np.uint8) == 0xEE).all(), "the single-row route does not use the scratch buffer"
+
+
+@pytest.mark.parametrize("wtype", [O.Q4_0, O.Q8_0, O.Q4_K, O.Q6_K])
 @pytest.mark.parametrize("M,K,T", [(96, 4096, 16), (200, 512, 70), (64, 128, 64), (64, 256, 64), (132, 11008, 33), (4096, 4096, 130)])
 def test_tiled_matmul_bits(hip, oracle, wtype, M, K, T, monkeypatch):
     """Sixteen activation rows and more take the tiled kernel (64 x 64 outputs per workgroup, the eight accumulators
@@ -93,7 +127,7 @@ def test_tiled_matmul_bits(hip, oracle, wtype, M, K, T, monkeypatch):
         assert need > act + 2 * (M + T) * K, "the scratch size of the exact order covers the packed operands"
 
 
-@pytest.mark.parametrize("T", [2, 40])
+@pytest.mark.parametrize("T", [1, 2, 40])
 def test_q8_0_weights_of_any_byte(hip, oracle, T):
     """Weight bytes a quantizer never writes (-128): the host backend's sign / maddubs sequence
     (vec_util.h:101-110) gives 128 * -128 for (-128) * (-128); the exact mode follows it.  T = 2: the row kernel;
