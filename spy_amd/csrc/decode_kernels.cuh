@@ -244,7 +244,7 @@ __global__ __launch_bounds__(WGV_THREADS) void wave_gemv_kernel(fused_args a) {
         } else {
             const int u = gw + k * NW, r = u < a.M ? u : gw % a.M;
             load_tile<WT, 64, NITK>(t[k % RING], a.W0 + (size_t)r * RB, npair, lane);
-            if constexpr (EPI == EPI_RESID) side[k] = a.resid[r];
+            if constexpr (EPI == EPI_RESID) side[k] = a.resid ? a.resid[r] : 0.0f;
         }
     };
     // The compute unit serves its memory requests in order: every wave's activation request goes into the queue before any
@@ -310,7 +310,7 @@ __global__ __launch_bounds__(WGV_THREADS) void wave_gemv_kernel(fused_args a) {
 #pragma unroll
         for (int k = 0; k < NR; k++) {
             const int r = gw + k * NW;
-            if (lane == 63 && r < a.M) { if constexpr (EPI == EPI_RESID) a.out[r] = s[k] + side[k]; else a.out[r] = s[k]; }
+            if (lane == 63 && r < a.M) { if constexpr (EPI == EPI_RESID) a.out[r] = a.resid ? s[k] + side[k] : s[k]; else a.out[r] = s[k]; }     // no resid: the MatMul alone
         }
     }
 }

@@ -89,6 +89,39 @@ static int launch_wave_resid(spy_hip_llama *m, hipStream_t st, const fused_args 
     }
 }
 
+// MatMul of ONE f32 activation row (the operator path's single-token products) through the one-row-per-wave kernel: the row is
+// quantized to Q8_0 in LDS by the launch itself, nothing is added to the dots.  No engine behind the call.  One row per wave
+// up to about one workgroup per compute unit (4096 rows), three rows per wave above (11008 rows: 230 workgroups); matrices
+// with more rows than that are left to the caller's two-launch way (SPY_HIP_EUNSUPPORTED).
+template <int WT, int NITK, int NR>
+static int launch_wave_plain(hipStream_t st, const fused_args &a) {
+    const size_t lds = staged_bytes(a.K);
+    auto kern = wave_gemv_kernel<WT, NITK, NR, EPI_RESID, WT>;
+    RC_TRY(spy_raise_lds_limit((const void *)kern, lds));
+    kern<<<dim3((unsigned)((a.M + WGV_WAVES * NR - 1) / (WGV_WAVES * NR))), dim3(WGV_THREADS), lds, st>>>(a);
+    return SPY_LAUNCH_RC();
+}
+template <int WT>
+static int wave_plain(hipStream_t st, const void *w, const float *x, float *out, int M, int K) {
+    constexpr bool KQ = WT == SPY_HIP_Q4_K || WT == SPY_HIP_Q6_K;
+    if (M <= 0 || K <= 0 || K % (KQ ? 256 : 64) != 0) return SPY_HIP_EUNSUPPORTED;
+    fused_args a;
+    memset(&a, 0, sizeof(a));
+    a.W0 = (const uint8_t *)w; a.M = M; a.K = K; a.x_in = x; a.out = out;
+    const int nitk = (K + 4095) / 4096;
+    if (M <= 320 * WGV_WAVES) {
+        switch (nitk) {
+        case 1: return launch_wave_plain<WT, 1, 1>(st, a);
+        case 2: return launch_wave_plain<WT, 2, 1>(st, a);
+        case 3: return launch_wave_plain<WT, 3, 1>(st, a);
+        case 4: if constexpr (!KQ) return launch_wave_plain<WT, 4, 1>(st, a); else return SPY_HIP_EUNSUPPORTED;
+        default: return SPY_HIP_EUNSUPPORTED;
+        }
+    }
+    if (nitk == 1 && M <= 320 * WGV_WAVES * 3) return launch_wave_plain<WT, 1, 3>(st, a);
+    return SPY_HIP_EUNSUPPORTED;
+}
+
 // qkv + scores + softmax/KQV of one layer in one launch (head-local barriers)
 template <int WT, int WTV>
 static int launch_attn_layer_tv(spy_hip_llama *m, hipStream_t st, int il, bool probe) {

@@ -91,6 +91,11 @@ int spy_exact_matvec_q4_0(hipStream_t st, const void *w, const float *x, float *
 int spy_exact_matvec_q8_0(hipStream_t st, const void *w, const float *x, float *out, int M, int K);
 int spy_exact_matvec_q4_k(hipStream_t st, const void *w, const float *x, float *out, int M, int K);
 int spy_exact_matvec_q6_k(hipStream_t st, const void *w, const float *x, float *out, int M, int K);
+// the same in this backend's own summation order (one-row-per-wave kernel; K % 64, K-quants K % 256; matrices of up to 15360 rows)
+int spy_own_matvec_q4_0(hipStream_t st, const void *w, const float *x, float *out, int M, int K);
+int spy_own_matvec_q8_0(hipStream_t st, const void *w, const float *x, float *out, int M, int K);
+int spy_own_matvec_q4_k(hipStream_t st, const void *w, const float *x, float *out, int M, int K);
+int spy_own_matvec_q6_k(hipStream_t st, const void *w, const float *x, float *out, int M, int K);
 // probe: only check that the fused attention launch for this layer's types exists and that all its workgroups are resident
 int spy_probe_attn_layer_q4_0(spy_hip_llama *m, int il);
 int spy_probe_attn_layer_q8_0(spy_hip_llama *m, int il);

@@ -661,6 +661,20 @@ extern "C" size_t spy_hip_op_matmul_scratch_size(const spy_hip_tensor *w, const 
     return pk ? ((act + 255) & ~(size_t)255) + pk : act;
 }
 
+int spy_own_matvec_q4_0(hipStream_t st, const void *w, const float *x, float *out, int M, int K);      // engine_q*.hip: the one-row-per-wave kernel without a residual
+int spy_own_matvec_q8_0(hipStream_t st, const void *w, const float *x, float *out, int M, int K);
+int spy_own_matvec_q4_k(hipStream_t st, const void *w, const float *x, float *out, int M, int K);
+int spy_own_matvec_q6_k(hipStream_t st, const void *w, const float *x, float *out, int M, int K);
+static int own_matvec(hipStream_t st, int t0, const void *w, const float *x, float *out, int64_t M, int64_t K) {
+    if (M <= 0 || M >= (1ll << 30) || K <= 0 || K > 16384 || ((uintptr_t)w & 3) != 0 || ((uintptr_t)x & 15) != 0 || ((uintptr_t)out & 3) != 0) return SPY_HIP_EUNSUPPORTED;
+    switch (t0) {
+    case SPY_HIP_Q4_0: return spy_own_matvec_q4_0(st, w, x, out, (int)M, (int)K);
+    case SPY_HIP_Q8_0: return spy_own_matvec_q8_0(st, w, x, out, (int)M, (int)K);
+    case SPY_HIP_Q4_K: return ((uintptr_t)w & 15) == 0 ? spy_own_matvec_q4_k(st, w, x, out, (int)M, (int)K) : SPY_HIP_EUNSUPPORTED;
+    case SPY_HIP_Q6_K: return spy_own_matvec_q6_k(st, w, x, out, (int)M, (int)K);
+    default: return SPY_HIP_EUNSUPPORTED;
+    }
+}
 static int matmul_impl(void *stream, const spy_hip_tensor *w, const spy_hip_tensor *x, const spy_hip_tensor *dst, void *scratch, size_t scratch_bytes,
                        int skip_past, int klimit_past);
 extern "C" int spy_hip_op_matmul(void *stream, const spy_hip_tensor *w, const spy_hip_tensor *x, const spy_hip_tensor *dst,
@@ -692,10 +706,12 @@ static int matmul_impl(void *stream, const spy_hip_tensor *w, const spy_hip_tens
     SPY_CHECK_ARG(ne00 % spy_block_size(t0) == 0 && ne00 % spy_block_size(tm) == 0);
     hipStream_t st = (hipStream_t)stream;
 
-    // a single f32 row against a quantized matrix in the host's summation order: one launch that quantizes the row itself
-    if (quant && t1 == SPY_HIP_F32 && ne11 == 1 && ne12 == 1 && ne13 == 1 && skip_past < 0 && klimit_past < 0 && spy_exact_on() && x->nb[0] == 4 &&
+    // a single f32 row against a quantized matrix (every weight product of a single-token pass): one launch that quantizes the row
+    // itself in LDS, in the host's summation order or this backend's own
+    if (quant && t1 == SPY_HIP_F32 && ne11 == 1 && ne12 == 1 && ne13 == 1 && skip_past < 0 && klimit_past < 0 && x->nb[0] == 4 &&
         w->nb[0] == spy_type_size(t0) && w->nb[1] == spy_row_size(t0, ne00)) {
-        const int rc = spy_exact_matvec(st, t0, w->data, (const float *)x->data, (float *)dst->data, ne01, ne00);
+        const int rc = spy_exact_on() ? spy_exact_matvec(st, t0, w->data, (const float *)x->data, (float *)dst->data, ne01, ne00)
+                                      : own_matvec(st, t0, w->data, (const float *)x->data, (float *)dst->data, ne01, ne00);
         if (rc != SPY_HIP_EUNSUPPORTED) return rc;
     }
 

@@ -300,6 +300,34 @@ def test_op_matmul_quantized(hip, oracle, wtype):
     assert np.array_equal(scratch.download(np.uint8), O.quantize(oracle, x, O.Q8_0))
 
 
+@pytest.mark.parametrize("wtype", [O.Q4_0, O.Q8_0, O.Q4_K, O.Q6_K])
+@pytest.mark.parametrize("M,K", [(100, 4096), (4096, 4096), (37, 64), (33, 256), (21, 11008), (6000, 4096), (50, 16384), (16000, 512)])
+def test_op_matmul_single_row(hip, oracle, wtype, M, K):
+    """One f32 activation row (the weight products of a single-token pass through Backend::submit): one launch of the
+    one-row-per-wave kernel, which quantizes the row in LDS and leaves the scratch buffer alone; one row per wave up to 5120
+    rows, three above, the two-launch way beyond 15360 rows or where the row length does not fit."""
+    from tests.gpu_util import dev, dev_empty, call, assert_close
+    kq = wtype in (O.Q4_K, O.Q6_K)
+    if kq and K % 256:
+        pytest.skip("K-quant rows are whole super-blocks")
+    rng = np.random.default_rng(5 * wtype + M + K)
+    w = O.quantize(oracle, (rng.standard_normal((M, K)) * 0.02).astype(np.float32), wtype)
+    x = rng.standard_normal((1, K)).astype(np.float32)
+    x[0, :32] = 0.0
+    want = O.matmul(oracle, w, wtype, M, K, x, nthread=8)
+    dw, dx, dd = dev(w), dev(x), dev_empty(M * 4 + 64, 0xFF)
+    tw, tx, td = hip.tensor(dw, wtype, [K, M]), hip.tensor(dx, hip.F32, [K, 1]), hip.tensor(dd, hip.F32, [M, 1])
+    L = hip.load()
+    need = L.spy_hip_op_matmul_scratch_size(B(tw), B(tx))
+    scratch = dev_empty(need, 0xEE)
+    call(L.spy_hip_op_matmul, None, B(tw), B(tx), B(td), scratch.ptr, need)
+    got = dd.download(np.float32)
+    assert_close(got[:M].reshape(1, M), want, "single-row op_matmul type %d %dx%d" % (wtype, M, K))
+    assert (got[M:].view(np.uint32) == 0xFFFFFFFF).all(), "nothing is written beyond the M outputs"
+    one_launch = M <= 15360 and not (kq and K > 12288) and (M <= 5120 or K <= 4096)
+    assert (scratch.download(np.uint8) == 0xEE).all() == one_launch, "which route ran (the one-launch route does not touch the scratch buffer)"
+
+
 def test_op_matmul_attention_views(hip, oracle):
     """attn_score and KQV through the strided K / V^T cache views and the permuted Q."""
     from tests.gpu_util import dev, dev_empty, call, assert_close
