@@ -91,7 +91,9 @@ const char *spy_hip_error_string(int code);
  * mat.cpp:61-68); query its size with spy_hip_op_matmul_scratch_size.  While the host's summation
  * order is on (spy_hip_set_exact_order) that size also covers fp16 copies of both operands, from which
  * the prompt-sized Q4_0 / Q8_0 MatMul of that order runs fastest; a buffer that holds only the
- * activations (rows * row size of the converted type) is accepted too and gives the same results. */
+ * activations (rows * row size of the converted type) is accepted too and gives the same results.
+ * One contiguous f32 row against a plain quantized matrix (the weight products of a single-token pass) is
+ * quantized inside the launch that multiplies it and leaves `scratch` untouched, in either summation order. */
 size_t spy_hip_op_matmul_scratch_size(const spy_hip_tensor *w, const spy_hip_tensor *x);
 int spy_hip_op_matmul(void *stream, const spy_hip_tensor *w, const spy_hip_tensor *x, const spy_hip_tensor *dst,
                       void *scratch, size_t scratch_bytes);
