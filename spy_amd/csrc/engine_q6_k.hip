@@ -7,3 +7,4 @@ int spy_probe_attn_layer_q6_k(spy_hip_llama *m, int il) { return launch_attn_lay
 int spy_enqueue_exact_q6_k(spy_hip_llama *m, hipStream_t st, int which, int il) { return enqueue_exact<SPY_HIP_Q6_K>(m, st, which, il); }
 int spy_exact_matvec_q6_k(hipStream_t st, const void *w, const float *x, float *out, int M, int K) { return xg_plain<SPY_HIP_Q6_K>(st, w, x, out, M, K); }
 int spy_own_matvec_q6_k(hipStream_t st, const void *w, const float *x, float *out, int M, int K) { return wave_plain<SPY_HIP_Q6_K>(st, w, x, out, M, K); }
+int spy_exact_matvec_prepare_q6_k() { return xg_plain_prepare<SPY_HIP_Q6_K>(); }

@@ -54,6 +54,22 @@ static int launch_xg_plain(hipStream_t st, const xg_args &a) {
     kern<<<dim3((unsigned)((a.M + XG_WAVES - 1) / XG_WAVES)), dim3(XG_THREADS), lds, st>>>(a);
     return SPY_LAUNCH_RC();
 }
+// the LDS limits of these launches for every row length they take, raised ahead (spy_hip_init): an operator call then finds them
+// in the process-wide record and sets no kernel attribute, whatever it runs under
+template <int WT, int NITK>
+static int xg_plain_prepare_one() {
+    constexpr int NCH = xg_traits<WT>::NCH;
+    const size_t lds = ((staged_bytes(4096 * NITK) + 15) & ~(size_t)15) + (size_t)XG_WAVES * xg_slot_floats(NCH) * 4;
+    return lds > 160 * 1024 ? 0 : spy_raise_lds_limit((const void *)xgemv_kernel<WT, NITK, 1, 1, EPI_RESID, WT>, lds);
+}
+template <int WT>
+static int xg_plain_prepare() {
+    RC_TRY((xg_plain_prepare_one<WT, 1>()));
+    RC_TRY((xg_plain_prepare_one<WT, 2>()));
+    RC_TRY((xg_plain_prepare_one<WT, 3>()));
+    if constexpr (WT == SPY_HIP_Q4_0 || WT == SPY_HIP_Q8_0) RC_TRY((xg_plain_prepare_one<WT, 4>()));
+    return 0;
+}
 template <int WT>
 static int xg_plain(hipStream_t st, const void *w, const float *x, float *out, int M, int K) {
     constexpr bool KQ = WT == SPY_HIP_Q4_K || WT == SPY_HIP_Q6_K;

@@ -1018,7 +1018,19 @@ __global__ __launch_bounds__(256) void exact_dots32_kernel(xdesc w, const uint8_
 // the two tables on the current device: exp [65536], then silu [65536]
 int spy_exact_luts(const float **lut) { return device_luts(lut); }
 // spy_hip_init: the tables exist before the first operator call, which then has nothing to allocate
-int spy_exact_device_setup() { const float *lut = nullptr; return device_luts(&lut); }
+int spy_exact_matvec_prepare_q4_0();      // engine_q*.hip: LDS limits of the single-row MatMul launches
+int spy_exact_matvec_prepare_q8_0();
+int spy_exact_matvec_prepare_q4_k();
+int spy_exact_matvec_prepare_q6_k();
+int spy_exact_device_setup() {
+    const float *lut = nullptr;
+    int rc = device_luts(&lut);
+    if (!rc) rc = spy_exact_matvec_prepare_q4_0();
+    if (!rc) rc = spy_exact_matvec_prepare_q8_0();
+    if (!rc) rc = spy_exact_matvec_prepare_q4_k();
+    if (!rc) rc = spy_exact_matvec_prepare_q6_k();
+    return rc;
+}
 
 // A caller may switch the exact order on for the calls its own thread makes (a model whose passes run in the host's order
 // issues its prompt operators that way) without touching what other threads see.

@@ -328,19 +328,29 @@ def test_exact_order_operators_under_stream_capture(hip, oracle):
     t_g, t_os = hip.tensor(dg, hip.F32, [g.size]), hip.tensor(o_silu, hip.F32, [g.size])
     t_s, t_m, t_o = hip.tensor(ds, hip.F32, [n_kv, T, H_]), hip.tensor(dm, hip.I32, [Cx, T]), hip.tensor(o_soft, hip.F32, [n_kv, T, H_])
     t_x, t_p, t_r = hip.tensor(dx, hip.F32, [hd, H_, T]), hip.tensor(dp, hip.I32, [T]), hip.tensor(o_rope, hip.F32, [hd, H_, T])
-    print("capture: exact-order silu, softmax, rope", flush=True)
+    # a single-row MatMul with 8192-wide Q8_0 rows: its launch needs 86 KB of LDS, a limit that spy_hip_init has raised already
+    Mm, Km = 64, 8192
+    wm = O.quantize(oracle, (rng.standard_normal((Mm, Km)) * 0.02).astype(np.float32), O.Q8_0)
+    xm = rng.standard_normal((1, Km)).astype(np.float32)
+    w_mm = O.matmul(oracle, wm, O.Q8_0, Mm, Km, xm, nthread=2)
+    dwm, dxm, o_mm = dev(wm), dev(xm), dev_empty(Mm * 4, 0xFF)
+    t_wm, t_xm, t_om = hip.tensor(dwm, hip.Q8_0, [Km, Mm]), hip.tensor(dxm, hip.F32, [Km, 1]), hip.tensor(o_mm, hip.F32, [Mm, 1])
+    mm_need = L.spy_hip_op_matmul_scratch_size(B(t_wm), B(t_xm))
+    mm_scratch = dev_empty(mm_need, 0)
+    print("capture: exact-order silu, softmax, rope, single-row matmul", flush=True)
     call(L.spy_hip_capture_begin, st)
     rcs = [L.spy_hip_op_silu(st, B(t_g), B(t_os)), L.spy_hip_op_softmax(st, B(t_s), B(t_m), B(t_o), scale), L.spy_hip_op_rope(st, B(t_x), B(t_p), B(t_r), B(hp))]
+    rc_mm = L.spy_hip_op_matmul(st, B(t_wm), B(t_xm), B(t_om), mm_scratch.ptr, mm_need)
     rc_unprepared = L.spy_hip_op_rope(st, B(t_x), B(t_p), B(t_r), B(hp_new))
     gexec = C.c_void_p()
     rc_end = L.spy_hip_capture_end(st, C.byref(gexec))
-    assert rcs == [0, 0, 0] and rc_end == 0 and gexec.value, (rcs, rc_end)
+    assert rcs == [0, 0, 0] and rc_mm == 0 and rc_end == 0 and gexec.value, (rcs, rc_mm, rc_end)
     assert rc_unprepared == hip.EUNSUPPORTED
     # other data for the eager calls between the replays
     g2, s2 = dev((rng.standard_normal(2048) * 3).astype(np.float32)), dev((rng.standard_normal((H_, T, n_kv)) * 9).astype(np.float32))
     e_silu, e_soft = dev_empty(g.nbytes, 0), dev_empty(s.nbytes, 0)
     for replay in range(3):
-        for b in (o_silu, o_soft, o_rope):
+        for b in (o_silu, o_soft, o_rope, o_mm):
             b.fill(0xFF)
         hip.sync()                                       # the fills ran on the null stream; the graph's stream does not wait for them by itself
         call(L.spy_hip_graph_launch, gexec, st)
@@ -348,6 +358,7 @@ def test_exact_order_operators_under_stream_capture(hip, oracle):
         _same_bits(o_silu.download(np.float32), w_silu, "silu, replay %d" % replay)
         _same_bits(o_soft.download(np.float32).reshape(s.shape), w_soft, "softmax, replay %d" % replay)
         _same_bits(o_rope.download(np.float32).reshape(xr.shape), w_rope, "rope, replay %d" % replay)
+        _same_bits(o_mm.download(np.float32).reshape(1, Mm), w_mm, "single-row matmul, replay %d" % replay)
         call(L.spy_hip_op_silu, None, B(hip.tensor(g2, hip.F32, [g.size])), B(hip.tensor(e_silu, hip.F32, [g.size])))
         call(L.spy_hip_op_softmax, None, B(hip.tensor(s2, hip.F32, [n_kv, T, H_])), B(t_m), B(hip.tensor(e_soft, hip.F32, [n_kv, T, H_])), scale)
         hip.sync()
