@@ -157,8 +157,8 @@ const void *HIPBackend::device_view(DataNode *node, bool is_output) {
             s.bytes = bytes;
         }
         if (is_output) { s.uploaded_valid = false; return s.dev; }                                   // the device copy is about to change
-        // host vectors change from pass to pass, not within one: a small tensor whose bytes are those of the last upload stays
-        constexpr size_t kCompareLimit = 64 * 1024;
+        // host vectors change from pass to pass, not within one: a tensor of up to 8 MiB whose bytes are those of the last upload stays
+        constexpr size_t kCompareLimit = 8u << 20;                                                   // the mask of a 1024-token prompt is 4 MiB: comparing costs a third of uploading
         if (bytes <= kCompareLimit && s.uploaded_valid && s.uploaded.size() == bytes && std::memcmp(s.uploaded.data(), t.data_ptr, bytes) == 0) return s.dev;
         if (spy_hip_upload(s.dev, t.data_ptr, bytes, stream_) != 0) return nullptr;
         s.uploaded_valid = bytes <= kCompareLimit;

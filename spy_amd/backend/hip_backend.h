@@ -51,7 +51,7 @@ private:
     std::map<size_t, std::vector<void *>> pool_;                  // bucket size -> free blocks
     std::unordered_map<void *, size_t> bucket_of_;
     std::unordered_map<const void *, void *> constants_;          // host pointer -> device copy
-    // device copy of an IO tensor, and (small tensors) the host bytes it was last uploaded from: the positions and the mask of a
+    // device copy of an IO tensor, and (up to 8 MiB) the host bytes it was last uploaded from: the positions and the mask of a
     // pass are read by one operator per layer, and uploading them again for each costs more than comparing them
     struct Staged { void *dev = nullptr; size_t bytes = 0; std::vector<uint8_t> uploaded; bool uploaded_valid = false; };
     std::unordered_map<const DataNode *, Staged> io_;             // IO node -> staging buffer
