@@ -714,6 +714,17 @@ static int matmul_impl(void *stream, const spy_hip_tensor *w, const spy_hip_tens
                                       : own_matvec(st, t0, w->data, (const float *)x->data, (float *)dst->data, ne01, ne00);
         if (rc != SPY_HIP_EUNSUPPORTED) return rc;
     }
+    // the host's order with 2 .. 15 rows (a short prompt): the same launch once per row -- the lane kernels below take 44 us per row
+    // of a 4096 x 4096 matrix, this one 5; from 16 rows on the tiled kernel
+    if (quant && t1 == SPY_HIP_F32 && ne11 >= 2 && ne11 <= 15 && ne12 == 1 && ne13 == 1 && skip_past < 0 && klimit_past < 0 && spy_exact_on() &&
+        x->nb[0] == 4 && x->nb[1] % 16 == 0 && dst->nb[1] % 4 == 0 && w->nb[0] == spy_type_size(t0) && w->nb[1] == spy_row_size(t0, ne00)) {
+        int rc = 0;
+        for (int64_t i = 0; i < ne11 && rc == 0; i++) {
+            rc = spy_exact_matvec(st, t0, w->data, (const float *)((const uint8_t *)x->data + i * x->nb[1]), (float *)((uint8_t *)dst->data + i * dst->nb[1]), ne01, ne00);
+            if (rc == SPY_HIP_EUNSUPPORTED && i == 0) break;             // nothing launched yet: the general way
+        }
+        if (rc != SPY_HIP_EUNSUPPORTED) return rc;
+    }
 
     // 1. activations -> mid type, contiguous [ne10, ne11, ne12, ne13] in scratch (mat.cpp:95-128)
     const uint8_t *xm = (const uint8_t *)x->data;
